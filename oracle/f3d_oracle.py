@@ -1,0 +1,332 @@
+"""CPU oracle for the Flash3D forward hot path.  TEST INFRASTRUCTURE ONLY.
+
+Python face of ``oracle/f3d_oracle.c`` (integer / byte arithmetic, loaded through ctypes) plus fp32
+torch restatements of the floating-point ops (bucketed attention, linear, LayerNorm, MLP).  Only
+tests, the smoke test and the benchmark's CPU-baseline leg import this module; the product package
+never does.
+
+Arrays are numpy: fp16 coordinates as ``np.float16``, bf16 features as raw ``np.uint16`` bit
+patterns, counters as ``np.uint32`` / ``np.uint16`` (the reference's CounterT / HashT).
+"""
+import ctypes
+import math
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "libf3d_oracle.so")
+
+
+def build(force: bool = False) -> str:
+    """Compile the C oracle with gcc (seconds).  Returns the library path."""
+    src = os.path.join(_HERE, "f3d_oracle.c")
+    stale = (not os.path.exists(_LIB_PATH)) or os.path.getmtime(_LIB_PATH) < os.path.getmtime(src)
+    if force or stale:
+        subprocess.check_call(["make", "-C", _HERE, "-B", "libf3d_oracle.so"], stdout=subprocess.DEVNULL)
+    return _LIB_PATH
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        build()
+        _lib = ctypes.CDLL(_LIB_PATH)
+        _lib.f3d_or_half_to_float.restype = ctypes.c_float
+        _lib.f3d_or_half_to_float.argtypes = [ctypes.c_uint16]
+        _lib.f3d_or_float_to_half.restype = ctypes.c_uint16
+        _lib.f3d_or_float_to_half.argtypes = [ctypes.c_float]
+        _lib.f3d_or_bf16_to_float.restype = ctypes.c_float
+        _lib.f3d_or_bf16_to_float.argtypes = [ctypes.c_uint16]
+        _lib.f3d_or_float_to_bf16.restype = ctypes.c_uint16
+        _lib.f3d_or_float_to_bf16.argtypes = [ctypes.c_float]
+        _lib.f3d_or_vox1.restype = ctypes.c_uint16
+        _lib.f3d_or_vox1.argtypes = [ctypes.c_float, ctypes.c_float, ctypes.c_float, ctypes.c_uint32]
+        _lib.f3d_or_space_out_bit_3d.restype = ctypes.c_uint64
+        _lib.f3d_or_space_out_bit_3d.argtypes = [ctypes.c_uint64]
+        _lib.f3d_or_zorder16.restype = ctypes.c_uint16
+        _lib.f3d_or_zorder16.argtypes = [ctypes.c_uint16] * 3
+        _lib.f3d_or_hash.restype = ctypes.c_uint16
+        _lib.f3d_or_hash.argtypes = [ctypes.c_uint16] * 3 + [ctypes.c_uint32] * 3
+        _lib.f3d_or_rng_u32.restype = ctypes.c_uint32
+        _lib.f3d_or_rng_u32.argtypes = [ctypes.c_uint32] * 4
+        _lib.f3d_or_rng_u01.restype = ctypes.c_float
+        _lib.f3d_or_rng_u01.argtypes = [ctypes.c_uint32] * 4
+    return _lib
+
+
+def _p(a: np.ndarray):
+    assert a.flags["C_CONTIGUOUS"], "oracle arrays must be C-contiguous"
+    return ctypes.c_void_p(a.ctypes.data)
+
+
+def _u16(a):
+    """fp16 / bf16-bits / u16 array -> uint16 view"""
+    a = np.ascontiguousarray(a)
+    return a.view(np.uint16) if a.dtype == np.float16 else a.astype(np.uint16, copy=False)
+
+
+# ---------------------------------------------------------------------------------------------
+# helpers restated from flash3dxfmr/psh/{arithmatic,batching,subbuck,bucket_scope}.py
+# ---------------------------------------------------------------------------------------------
+
+def round_next_two_power(v: int) -> int:
+    """flash3dxfmr/psh/arithmatic.py:12-19"""
+    v -= 1
+    for s in (1, 2, 4, 8, 16):
+        v |= v >> s
+    return v + 1
+
+
+def psh_params(seps, bucket_size: int, num_vox: int = 0xFFFF):
+    """num_bucket / divisor heuristics of flash3dxfmr/psh/psh_main.py:100-104: mean cloud size (fp32
+    mean), floor-divided by the bucket size, next power of two; divisor = ceil(num_vox / NB)."""
+    seps = np.asarray(seps, dtype=np.int64)
+    sizes = np.diff(np.concatenate([[0], seps]))
+    mean_n = float(np.float32(sizes.astype(np.float32).mean()))
+    nb = round_next_two_power(int(mean_n / bucket_size))
+    div = int(math.ceil(num_vox / nb)) if nb > 0 else 0
+    return nb, div, int(sizes.max())
+
+
+def calc_red_sep_sizes(seps, subbuck_size: int):
+    """flash3dxfmr/psh/subbuck.py:40-53"""
+    seps = np.asarray(seps, dtype=np.int64)
+    sizes = np.diff(np.concatenate([[0], seps]))
+    red_sizes = (sizes + subbuck_size - 1) // subbuck_size
+    return int(red_sizes.sum()), red_sizes.astype(np.uint32), np.cumsum(red_sizes).astype(np.uint32)
+
+
+def gen_scopes(total_n: int, buck_size: int, scope_size: int, plan: str = "swin"):
+    """flash3dxfmr/psh/bucket_scope.py:58-140 — consecutive groups of ``scope_size`` buckets when the
+    length is aligned (swin: buck*scope; stride: buck*scope*6), one global scope otherwise."""
+    assert plan in ("swin", "stride")
+    assert total_n % buck_size == 0
+    nbuck = total_n // buck_size
+    align = buck_size * scope_size * (6 if plan == "stride" else 1)
+    if total_n % align == 0:
+        return np.arange(nbuck, dtype=np.uint32).reshape(nbuck // scope_size, scope_size)
+    return np.arange(nbuck, dtype=np.uint32).reshape(1, nbuck)
+
+
+# ---------------------------------------------------------------------------------------------
+# A1 / A2
+# ---------------------------------------------------------------------------------------------
+
+def vox_coord(coord_h, bbox_min_h, bbox_max_h, num_vox: int = 0xFFFF):
+    c = _u16(coord_h).reshape(-1, 3)
+    out = np.empty_like(c)
+    lib().f3d_or_vox_coord(_p(c), ctypes.c_uint32(c.shape[0]), _p(_u16(bbox_min_h)), _p(_u16(bbox_max_h)),
+                           ctypes.c_uint32(num_vox), _p(out))
+    return out
+
+
+def hash_ids(vox, hash_type: int, divisor: int, num_bucket: int):
+    """vectorised numpy restatement of f3d_or_hash (kept separate from the C code on purpose: the
+    two are checked against each other in the oracle tests)"""
+    v = vox.astype(np.uint64)
+
+    def spread(x):
+        x = (x | x << np.uint64(32)) & np.uint64(0x1f00000000ffff)
+        x = (x | x << np.uint64(16)) & np.uint64(0x1f0000ff0000ff)
+        x = (x | x << np.uint64(8)) & np.uint64(0x100f00f00f00f00f)
+        x = (x | x << np.uint64(4)) & np.uint64(0x10c30c30c30c30c3)
+        x = (x | x << np.uint64(2)) & np.uint64(0x1249249249249249)
+        return x
+
+    if hash_type in (1, 3):
+        m = spread(v[:, 0]) | spread(v[:, 1]) << np.uint64(1) | spread(v[:, 2]) << np.uint64(2)
+        h = ((m >> np.uint64(31)) & np.uint64(0xFFFF)).astype(np.uint32)
+    else:
+        h = (vox[:, 0] ^ vox[:, 1] ^ vox[:, 2]).astype(np.uint32)
+    if hash_type in (1, 2):
+        return (h // np.uint32(divisor & 0xFFFF)).astype(np.uint16)
+    return (h % np.uint32(num_bucket & 0xFFFF)).astype(np.uint16)
+
+
+# ---------------------------------------------------------------------------------------------
+# A3 / A5 / scoreboard
+# ---------------------------------------------------------------------------------------------
+
+def psh_claim(coord_h, seps, bbox_min_h, bbox_max_h, num_vox, divisor, num_bucket, hash_type):
+    c = _u16(coord_h).reshape(-1, 3)
+    seps = np.ascontiguousarray(seps, dtype=np.uint32)
+    n, b = c.shape[0], seps.shape[0]
+    bucket_id = np.ones(n, dtype=np.uint16)
+    counter = np.zeros((b, num_bucket), dtype=np.uint32)
+    offset = np.zeros(n, dtype=np.uint32)
+    rc = lib().f3d_or_psh_claim(_p(c), ctypes.c_uint32(n), _p(seps), ctypes.c_uint32(b), _p(_u16(bbox_min_h)),
+                                _p(_u16(bbox_max_h)), ctypes.c_uint32(num_vox), ctypes.c_uint32(divisor),
+                                ctypes.c_uint32(num_bucket), ctypes.c_uint32(hash_type), _p(bucket_id),
+                                _p(counter), _p(offset))
+    if rc != 0:
+        raise RuntimeError(f"oracle psh_claim failed rc={rc}")
+    return bucket_id, counter, offset
+
+
+def cumsum_scatter_pad(coord_h, seps, num_bucket, bucket_id, counter, offset, pad_to, pad_num=0.0,
+                       prefill_nan=True):
+    c = _u16(coord_h).reshape(-1, 3)
+    seps = np.ascontiguousarray(seps, dtype=np.uint32)
+    n, b = c.shape[0], seps.shape[0]
+    cumsum = np.zeros((b, num_bucket), dtype=np.uint32)
+    scattered = np.full((pad_to, 3), 0x7E00 if prefill_nan else 0, dtype=np.uint16)
+    rc = lib().f3d_or_cumsum_scatter_pad(_p(c), ctypes.c_uint32(n), _p(seps), ctypes.c_uint32(b),
+                                         ctypes.c_uint32(num_bucket), _p(bucket_id), _p(counter), _p(offset),
+                                         _p(cumsum), _p(scattered), ctypes.c_uint32(pad_to),
+                                         ctypes.c_float(pad_num))
+    if rc != 0:
+        raise RuntimeError(f"oracle cumsum_scatter_pad failed rc={rc}")
+    return cumsum, scattered.view(np.float16)
+
+
+def scoreboard(bucket_id, counter, offset, seps):
+    """0 when every (cloud, bucket, slot < count) is claimed exactly once (bucket_sanitizer_cpu.cpp:92-176)"""
+    seps = np.ascontiguousarray(seps, dtype=np.uint32)
+    counter = np.ascontiguousarray(counter, dtype=np.uint32)
+    bad = ctypes.c_int64(-1)
+    rc = lib().f3d_or_scoreboard(_p(np.ascontiguousarray(bucket_id, dtype=np.uint16)), _p(counter),
+                                 _p(np.ascontiguousarray(offset, dtype=np.uint32)), _p(seps),
+                                 ctypes.c_uint32(seps.shape[0]), ctypes.c_uint32(counter.shape[1]),
+                                 ctypes.byref(bad))
+    return rc, bad.value
+
+
+# ---------------------------------------------------------------------------------------------
+# A6 / A7 / A8
+# ---------------------------------------------------------------------------------------------
+
+def subbuck_build(coord_h, seps, subbuck_size, num_vox=0xFFFF, seed=3407, out_align=1):
+    c = _u16(coord_h).reshape(-1, 3)
+    seps = np.ascontiguousarray(seps, dtype=np.uint32)
+    n = c.shape[0]
+    red_len, _, red_sep = calc_red_sep_sizes(seps, subbuck_size)
+    r_aligned = -(-red_len // out_align) * out_align
+    sub_id = np.zeros(n, dtype=np.uint32)
+    sub_off = np.zeros(n, dtype=np.uint16)
+    unpool = np.full((red_len, subbuck_size), n + 3, dtype=np.uint32)
+    red_coord = np.zeros((r_aligned, 3), dtype=np.uint16)
+    rc = lib().f3d_or_subbuck_build(_p(c), ctypes.c_uint32(n), _p(seps), _p(red_sep),
+                                    ctypes.c_uint32(seps.shape[0]), ctypes.c_uint32(subbuck_size),
+                                    ctypes.c_uint32(num_vox), ctypes.c_uint32(seed), _p(sub_id), _p(sub_off),
+                                    _p(unpool), _p(red_coord), ctypes.c_uint32(r_aligned))
+    if rc != 0:
+        raise RuntimeError(f"oracle subbuck_build failed rc={rc}")
+    return sub_id, sub_off, unpool, red_coord.view(np.float16), red_sep
+
+
+def reduce_feat(feat_bf, unpool_ind, red_op, r_aligned=None):
+    f = np.ascontiguousarray(feat_bf, dtype=np.uint16)
+    u = np.ascontiguousarray(unpool_ind, dtype=np.uint32)
+    n, c = f.shape
+    r, s = u.shape
+    ra = r if r_aligned is None else r_aligned
+    out = np.zeros((ra, c), dtype=np.uint16)
+    rc = lib().f3d_or_reduce_feat(_p(f), ctypes.c_uint32(n), ctypes.c_uint32(c), _p(u), ctypes.c_uint32(r),
+                                  ctypes.c_uint32(s), ctypes.c_uint32(red_op), _p(out), ctypes.c_uint32(ra))
+    if rc != 0:
+        raise RuntimeError(f"oracle reduce_feat failed rc={rc}")
+    return out
+
+
+def additive_unpool(res_bf, down_bf, unpool_ind, up_init=None):
+    res = np.ascontiguousarray(res_bf, dtype=np.uint16)
+    down = np.ascontiguousarray(down_bf, dtype=np.uint16)
+    u = np.ascontiguousarray(unpool_ind, dtype=np.uint32)
+    up = np.zeros_like(res) if up_init is None else np.ascontiguousarray(up_init, dtype=np.uint16).copy()
+    rc = lib().f3d_or_additive_unpool(_p(res), _p(down), _p(up), _p(u), ctypes.c_uint32(res.shape[0]),
+                                      ctypes.c_uint32(u.shape[0]), ctypes.c_uint32(res.shape[1]),
+                                      ctypes.c_uint32(u.shape[1]))
+    assert rc == 0
+    return up
+
+
+# ---------------------------------------------------------------------------------------------
+# bf16 bit helpers (numpy)
+# ---------------------------------------------------------------------------------------------
+
+def bf16_bits_to_f32(bits):
+    return (np.asarray(bits, dtype=np.uint16).astype(np.uint32) << np.uint32(16)).view(np.float32)
+
+
+def f32_to_bf16_bits(x):
+    u = np.ascontiguousarray(x, dtype=np.float32).view(np.uint32)
+    nan = (u & np.uint32(0x7FFFFFFF)) > np.uint32(0x7F800000)
+    r = ((u + np.uint32(0x7FFF) + ((u >> np.uint32(16)) & np.uint32(1))) >> np.uint32(16)).astype(np.uint16)
+    return np.where(nan, ((u >> np.uint32(16)) | np.uint32(0x40)).astype(np.uint16), r)
+
+
+# ---------------------------------------------------------------------------------------------
+# A9 / A9m bucketed attention, A11 / A12 dense layers — fp32 torch on bf16-rounded inputs
+# ---------------------------------------------------------------------------------------------
+
+def buck_swin_fwd(Q, K, V, scope_buckets, bucket_size, kv_len=None, O_init=None, LSE_init=None):
+    """Definition of pshattn.buck_swin_fwd (declared src/f3d_frontend.cu:90-92; semantics pinned by
+    tests/test_attn_fwd.py:167-190, 404-452): for every batch row and every scope (row of
+    ``scope_buckets``), full softmax attention among the rows of the scope's buckets, per head,
+    scale 1/sqrt(D); LSE is the natural-log sum of exponentials.  Rows no scope covers keep
+    ``O_init`` / ``LSE_init``.
+
+    ``kv_len`` (extension, int per bucket): keys at in-bucket position >= kv_len are masked out;
+    query rows at such positions produce O = 0, LSE = 0.
+
+    Q, K, V: torch tensors [B, L, H, D] (any float dtype; computed in fp32).  Returns (O, LSE) fp32.
+    """
+    import torch
+
+    B, L, H, D = Q.shape
+    scopes = torch.as_tensor(np.asarray(scope_buckets).astype(np.int64))
+    Qf, Kf, Vf = Q.float(), K.float(), V.float()
+    O = torch.zeros(B, L, H, D, dtype=torch.float32) if O_init is None else O_init.float().clone()
+    LSE = torch.zeros(B, L, H, dtype=torch.float32) if LSE_init is None else LSE_init.float().clone()
+    ar = torch.arange(bucket_size)
+    scale = 1.0 / math.sqrt(D)
+    for s in range(scopes.shape[0]):
+        rows = (scopes[s][:, None] * bucket_size + ar[None, :]).reshape(-1)
+        if kv_len is not None:
+            kl = torch.as_tensor(np.asarray(kv_len).astype(np.int64))[scopes[s]]
+            valid = (ar[None, :] < kl[:, None]).reshape(-1)
+        else:
+            valid = torch.ones(rows.shape[0], dtype=torch.bool)
+        q = Qf[:, rows].permute(0, 2, 1, 3)  # [B,H,T,D]
+        k = Kf[:, rows].permute(0, 2, 1, 3)
+        v = Vf[:, rows].permute(0, 2, 1, 3)
+        logits = torch.matmul(q, k.transpose(-1, -2)) * scale
+        logits = logits.masked_fill(~valid[None, None, None, :], float("-inf"))
+        lse = torch.logsumexp(logits, dim=-1)  # [B,H,T]
+        p = torch.exp(logits - lse[..., None])
+        o = torch.matmul(p, v)  # [B,H,T,D]
+        o = torch.where(valid[None, None, :, None], o, torch.zeros_like(o))
+        lse = torch.where(valid[None, None, :], lse, torch.zeros_like(lse))
+        O[:, rows] = o.permute(0, 2, 1, 3)
+        LSE[:, rows] = lse.permute(0, 2, 1)
+    return O, LSE
+
+
+def linear(x, w, b=None):
+    """y = x @ w.T + b in fp32 (torch.nn.Linear semantics; layers/buck_swin.py:159,163)"""
+    import torch
+    y = x.float() @ w.float().t()
+    return y + b.float() if b is not None else y
+
+
+def layernorm(x, g, b, eps=1e-5):
+    import torch
+    return torch.nn.functional.layer_norm(x.float(), (x.shape[-1],), g.float(), b.float(), eps)
+
+
+def gelu(x):
+    import torch
+    return torch.nn.functional.gelu(x.float())
+
+
+def swiglu(h):
+    """silu(h[:, :hid]) * h[:, hid:] — the definition this build gives te.LayerNormMLP(activation="swiglu")
+    (layers/elem_wise.py:22-26); TransformerEngine itself is absent, so this ordering is parity-unpinned."""
+    import torch
+    hid = h.shape[-1] // 2
+    return torch.nn.functional.silu(h[..., :hid].float()) * h[..., hid:].float()
