@@ -1,0 +1,138 @@
+// Device-side building blocks shared by the gfx950 kernels: 16-bit float conversions, the voxel
+// quantiser and first-hash family, the stateless RNG, and wave64 helpers.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace f3d {
+
+constexpr int kWave = 64;
+
+// ---- 16-bit float bit patterns <-> fp32 -------------------------------------------------------
+
+__device__ __forceinline__ float half_bits_to_float(uint16_t h) {
+  return (float)__builtin_bit_cast(_Float16, h);
+}
+
+__device__ __forceinline__ uint16_t float_to_half_bits(float f) {
+  return __builtin_bit_cast(uint16_t, (_Float16)f);  // v_cvt_f16_f32: round to nearest even
+}
+
+__device__ __forceinline__ float bf16_bits_to_float(uint16_t b) {
+  return __builtin_bit_cast(float, (uint32_t)b << 16);
+}
+
+// round to nearest even; NaN stays NaN
+__device__ __forceinline__ uint16_t float_to_bf16_bits(float f) {
+  uint32_t u = __builtin_bit_cast(uint32_t, f);
+  if ((u & 0x7FFFFFFFu) > 0x7F800000u) return (uint16_t)((u >> 16) | 0x40u);
+  u += 0x7FFFu + ((u >> 16) & 1u);
+  return (uint16_t)(u >> 16);
+}
+
+// ---- voxel quantiser (reference: src/psh/hash_fns.cuh:23-33) ----------------------------------
+// q = ((c - min) * num_vox) * inv with inv = 1 / (max - min) rounded once; floor; clamp to
+// [0, num_vox - 1] with NaN -> num_vox - 1.  All steps are separate IEEE fp32 operations: the
+// translation units that use this are built with -ffp-contract=off.
+struct VoxAxis {
+  float mn, inv, nv, hi;
+};
+
+__device__ __forceinline__ VoxAxis make_vox_axis(uint16_t min_h, uint16_t max_h, uint32_t num_vox) {
+  VoxAxis a;
+  a.mn = half_bits_to_float(min_h);
+  float den = half_bits_to_float(max_h) - a.mn;
+  a.inv = __fdiv_rn(1.0f, den);
+  a.nv = (float)num_vox;
+  a.hi = (float)(num_vox - 1u);
+  return a;
+}
+
+__device__ __forceinline__ VoxAxis make_vox_axis_f(float mn, float mx, uint32_t num_vox) {
+  VoxAxis a;
+  a.mn = mn;
+  a.inv = __fdiv_rn(1.0f, mx - mn);
+  a.nv = (float)num_vox;
+  a.hi = (float)(num_vox - 1u);
+  return a;
+}
+
+__device__ __forceinline__ uint32_t vox1(float c, const VoxAxis& a) {
+  float q = __fmul_rn(__fmul_rn(__fsub_rn(c, a.mn), a.nv), a.inv);
+  float v = floorf(q);
+  float m = (v < a.hi) ? v : a.hi;  // NaN -> hi
+  float r = (m > 0.f) ? m : 0.f;
+  return (uint32_t)r;
+}
+
+// ---- first-hash family (reference: src/psh/hash_fns.cuh:48-135) --------------------------------
+
+// spread the low 6 bits of x to bit positions 0,3,6,9,12,15
+__device__ __forceinline__ uint32_t spread3_6(uint32_t x) {
+  x = (x | (x << 8)) & 0x0000300Fu;
+  x = (x | (x << 4)) & 0x000030C3u;
+  x = (x | (x << 2)) & 0x00009249u;
+  return x;
+}
+
+// low 16 bits of (morton48(x,y,z) >> 31): bits, from bit 0 up, y10 z10 x11 y11 z11 ... x15 y15
+__device__ __forceinline__ uint32_t zorder16(uint32_t vx, uint32_t vy, uint32_t vz) {
+  uint32_t xs = spread3_6((vx >> 11) & 0x1Fu);
+  uint32_t ys = spread3_6((vy >> 10) & 0x3Fu);
+  uint32_t zs = spread3_6((vz >> 10) & 0x1Fu);
+  return (ys | (zs << 1) | (xs << 2)) & 0xFFFFu;
+}
+
+// divisor16 / num_bucket16 are the 16-bit truncations the reference's HashT parameters apply
+__device__ __forceinline__ uint32_t first_hash(uint32_t vx, uint32_t vy, uint32_t vz, uint32_t hash_type,
+                                               uint32_t divisor16, uint32_t num_bucket16) {
+  uint32_t h = (hash_type & 1u) ? zorder16(vx, vy, vz) : ((vx ^ vy ^ vz) & 0xFFFFu);
+  return (hash_type <= 2u) ? h / divisor16 : h % num_bucket16;
+}
+
+// ---- stateless RNG: 32-bit finaliser chained over (seed, a, b, c) -------------------------------
+
+__device__ __forceinline__ uint32_t mix32(uint32_t x) {
+  x ^= x >> 16; x *= 0x7feb352dU;
+  x ^= x >> 15; x *= 0x846ca68bU;
+  x ^= x >> 16;
+  return x;
+}
+
+__device__ __forceinline__ uint32_t rng_u32(uint32_t seed, uint32_t a, uint32_t b, uint32_t c) {
+  uint32_t h = mix32(seed + 0x9E3779B9u);
+  h = mix32(h ^ (a + 0x85EBCA6Bu));
+  h = mix32(h ^ (b + 0xC2B2AE35u));
+  h = mix32(h ^ (c + 0x27D4EB2Fu));
+  return h;
+}
+
+__device__ __forceinline__ float rng_u01(uint32_t seed, uint32_t a, uint32_t b, uint32_t c) {
+  return (float)(rng_u32(seed, a, b, c) >> 8) * (1.0f / 16777216.0f);
+}
+
+// ---- wave64 helpers -----------------------------------------------------------------------------
+
+__device__ __forceinline__ uint32_t lane_id() {
+  return __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+}
+
+// number of set bits of `mask` strictly below this lane
+__device__ __forceinline__ uint32_t mask_rank(uint64_t mask) {
+  return __builtin_amdgcn_mbcnt_hi((uint32_t)(mask >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0u));
+}
+
+// Lanes of the wave whose `key` (low `nbits` bits significant) equals this lane's, restricted to
+// lanes with `valid` set.  One ballot per key bit.
+__device__ __forceinline__ uint64_t match_any(uint32_t key, uint32_t nbits, bool valid) {
+  uint64_t mask = __ballot(valid);
+  for (uint32_t k = 0; k < nbits; ++k) {
+    bool bit = (key >> k) & 1u;
+    uint64_t b = __ballot(bit);
+    mask &= bit ? b : ~b;
+  }
+  return mask;
+}
+
+}  // namespace f3d

@@ -1,0 +1,72 @@
+// Shared host-side plumbing of the gfx950 library: error reporting, per-device workspace,
+// stream synchronisation flag.  Device helpers live in f3d_device.h.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#include "../../include/f3d_hip.h"
+
+namespace f3d {
+
+// Message of the last failing call on this thread (returned by f3d_last_error()).
+void set_error(const char* fmt, ...) __attribute__((format(printf, 1, 2)));
+
+// Grow-only scratch buffer owned by the library, one per device.  Work that uses it is ordered on
+// the caller's stream; calls that overlap on different streams of one device must not share it, so
+// every entry point that needs scratch documents that it is not re-entrant per device.
+// Returns nullptr (and sets the error) on allocation failure.
+void* workspace(int device, size_t bytes);
+
+bool sync_stream_enabled();
+uint32_t global_seed();
+int rebalance_mode();
+
+#define F3D_CHECK_ARG(cond, ...)            \
+  do {                                      \
+    if (!(cond)) {                          \
+      ::f3d::set_error(__VA_ARGS__);        \
+      return F3D_ERR_INVALID;               \
+    }                                       \
+  } while (0)
+
+#define F3D_CHECK_HIP(expr)                                                              \
+  do {                                                                                   \
+    hipError_t _e = (expr);                                                              \
+    if (_e != hipSuccess) {                                                              \
+      ::f3d::set_error("HIP error %d (%s) at %s:%d", (int)_e, hipGetErrorString(_e),    \
+                       __FILE__, __LINE__);                                              \
+      return F3D_ERR_RUNTIME;                                                            \
+    }                                                                                    \
+  } while (0)
+
+// RAII bracket reproducing the reference's optional stream synchronisation around an op
+// (src/psh/batch_psh_bucket_dispatcher.cu:278-280, 323-325).
+struct SyncBracket {
+  hipStream_t s;
+  explicit SyncBracket(hipStream_t stream) : s(stream) {
+    if (sync_stream_enabled()) (void)hipStreamSynchronize(s);
+  }
+  ~SyncBracket() {
+    if (sync_stream_enabled()) (void)hipStreamSynchronize(s);
+  }
+};
+
+// Makes `device` current for the lifetime of the object and restores the previous one.
+struct DeviceGuard {
+  int prev = -1;
+  bool ok = true;
+  explicit DeviceGuard(int device) {
+    if (hipGetDevice(&prev) != hipSuccess) prev = -1;
+    if (prev != device) ok = hipSetDevice(device) == hipSuccess;
+  }
+  ~DeviceGuard() {
+    int cur = -1;
+    if (prev >= 0 && hipGetDevice(&cur) == hipSuccess && cur != prev) (void)hipSetDevice(prev);
+  }
+};
+
+static inline uint32_t cdiv_u32(uint32_t a, uint32_t b) { return (a + b - 1) / b; }
+
+}  // namespace f3d

@@ -1,0 +1,379 @@
+// PSH bucketing for gfx950: voxel quantise -> first hash -> per-bucket slot claim -> cumsum ->
+// scatter (+ tail padding).  Counterpart of the reference's three launches in
+// src/psh/batch_psh_bucket_dispatcher.cu:287-320 (kernels in src/psh/batch_psh_bucket.cuh).
+//
+// Design (not a translation): the reference claims slots with shared->global atomics, so slot
+// order depends on arbitration.  Here slots are a stable counting sort:
+//   K1  hash_hist   one workgroup per tile of a cloud: quantise + hash, write bucket_id, LDS
+//                   histogram of the tile -> tile_hist[cloud][tile][bucket]
+//   K2  scan        per cloud: exclusive scan of tile_hist over tiles (in place -> tile base),
+//                   bucket totals -> bucket_counter, inclusive scan over buckets -> cumsum_counter
+//   K3  rank_scatter per tile: stable rank of every point among the tile's points of the same
+//                   bucket (wave64 ballot matching + per-wave LDS counters), slot = tile base + rank,
+//                   write bucket_offset and scatter the coordinate row; extra workgroups fill the pad rows
+// No global atomics, no dependence on workgroup scheduling: bucket ids, counts AND slots are a pure
+// function of the input.  HBM traffic per point: K1 6 B read + 2 B write, K3 8 B read + 10 B write.
+#include "f3d_device.h"
+#include "f3d_internal.h"
+
+namespace f3d {
+
+constexpr int kPshThreads = 256;
+constexpr int kPshWaves = kPshThreads / kWave;
+
+// Position inside a tile of the point handled by (wave w, round j, lane l): each wave owns a
+// contiguous run of 64*ITEMS points and walks it 64 at a time, so (j, l) order is input order.
+template <int ITEMS>
+__device__ __forceinline__ uint32_t tile_pos(uint32_t w, uint32_t j, uint32_t l) {
+  return w * (kWave * ITEMS) + j * kWave + l;
+}
+
+template <int ITEMS>
+__global__ __launch_bounds__(kPshThreads) void psh_hash_hist_kernel(
+    const uint16_t* __restrict__ coord, uint16_t* __restrict__ bucket_id, const uint32_t* __restrict__ batch_sep,
+    const uint16_t* __restrict__ bbox_min, const uint16_t* __restrict__ bbox_max, uint32_t num_vox,
+    uint32_t divisor16, uint32_t num_bucket, uint32_t hash_type, uint32_t* __restrict__ tile_hist,
+    uint32_t max_tiles) {
+  extern __shared__ uint32_t lds_hist[];
+  const uint32_t cloud = blockIdx.y, tile = blockIdx.x, tid = threadIdx.x;
+  const uint32_t start = cloud ? batch_sep[cloud - 1] : 0u;
+  const uint32_t n = batch_sep[cloud] - start;
+  const uint32_t tile0 = tile * (kPshThreads * ITEMS);
+  if (tile0 >= n) return;  // uniform for the workgroup
+
+  for (uint32_t b = tid; b < num_bucket; b += kPshThreads) lds_hist[b] = 0u;
+  VoxAxis ax[3];
+#pragma unroll
+  for (int d = 0; d < 3; ++d) ax[d] = make_vox_axis(bbox_min[d], bbox_max[d], num_vox);
+  __syncthreads();
+
+  const uint32_t w = tid / kWave, l = tid % kWave;
+  const uint32_t nb16 = num_bucket & 0xFFFFu;
+#pragma unroll
+  for (int j = 0; j < ITEMS; ++j) {
+    const uint32_t local = tile0 + tile_pos<ITEMS>(w, j, l);
+    if (local < n) {
+      const size_t g = (size_t)start + local;
+      const uint16_t* p = coord + 3 * g;
+      uint32_t v[3];
+#pragma unroll
+      for (int d = 0; d < 3; ++d) v[d] = vox1(half_bits_to_float(p[d]), ax[d]);
+      const uint32_t id = first_hash(v[0], v[1], v[2], hash_type, divisor16, nb16);
+      bucket_id[g] = (uint16_t)id;
+      atomicAdd(&lds_hist[id], 1u);
+    }
+  }
+  __syncthreads();
+  uint32_t* out = tile_hist + ((size_t)cloud * max_tiles + tile) * num_bucket;
+  for (uint32_t b = tid; b < num_bucket; b += kPshThreads) out[b] = lds_hist[b];
+}
+
+// One workgroup per cloud.  tile_hist -> exclusive prefix over tiles (plus the counter value the
+// caller passed in, which the reference's atomicAdd commit also builds on), totals -> bucket_counter,
+// inclusive scan over buckets -> cumsum_counter.
+__global__ __launch_bounds__(kPshThreads) void psh_scan_kernel(
+    uint32_t* __restrict__ tile_hist, uint32_t* __restrict__ bucket_counter, uint32_t* __restrict__ cumsum_counter,
+    const uint32_t* __restrict__ batch_sep, uint32_t num_bucket, uint32_t tile_pts, uint32_t max_tiles) {
+  extern __shared__ uint32_t lds_cnt[];  // num_bucket totals, then wave partials
+  const uint32_t cloud = blockIdx.x, tid = threadIdx.x;
+  const uint32_t start = cloud ? batch_sep[cloud - 1] : 0u;
+  const uint32_t n = batch_sep[cloud] - start;
+  const uint32_t ntile = (n + tile_pts - 1) / tile_pts;
+  uint32_t* counter = bucket_counter + (size_t)cloud * num_bucket;
+  for (uint32_t b = tid; b < num_bucket; b += kPshThreads) {
+    uint32_t run = counter[b];
+    uint32_t* h = tile_hist + (size_t)cloud * max_tiles * num_bucket + b;
+    for (uint32_t t = 0; t < ntile; ++t) {
+      const uint32_t c = h[(size_t)t * num_bucket];
+      h[(size_t)t * num_bucket] = run;
+      run += c;
+    }
+    counter[b] = run;
+    lds_cnt[b] = run;
+  }
+  __syncthreads();
+  // inclusive scan over buckets by the first wave: lane owns a contiguous chunk
+  if (tid < kWave) {
+    const uint32_t chunk = (num_bucket + kWave - 1) / kWave;
+    const uint32_t b0 = tid * chunk;
+    uint32_t sum = 0;
+    for (uint32_t i = 0; i < chunk; ++i)
+      if (b0 + i < num_bucket) sum += lds_cnt[b0 + i];
+    uint32_t incl = sum;
+#pragma unroll
+    for (int off = 1; off < kWave; off <<= 1) {
+      const uint32_t up = __shfl_up(incl, off, kWave);
+      if ((int)tid >= off) incl += up;
+    }
+    uint32_t run = incl - sum;
+    uint32_t* cs = cumsum_counter + (size_t)cloud * num_bucket;
+    for (uint32_t i = 0; i < chunk; ++i)
+      if (b0 + i < num_bucket) {
+        run += lds_cnt[b0 + i];
+        cs[b0 + i] = run;
+      }
+  }
+}
+
+template <int ITEMS>
+__global__ __launch_bounds__(kPshThreads) void psh_rank_scatter_kernel(
+    const uint16_t* __restrict__ coord, const uint16_t* __restrict__ bucket_id,
+    uint32_t* __restrict__ bucket_offset, const uint32_t* __restrict__ batch_sep, uint32_t batch_size,
+    const uint32_t* __restrict__ tile_base, const uint32_t* __restrict__ bucket_counter,
+    const uint32_t* __restrict__ cumsum_counter, uint32_t num_bucket, uint32_t nbits, uint32_t max_tiles,
+    uint16_t* __restrict__ scatter_coord, uint32_t total_n, uint32_t pad_to_n, uint16_t pad_bits) {
+  extern __shared__ uint32_t lds[];
+  const uint32_t cloud = blockIdx.y, tile = blockIdx.x, tid = threadIdx.x;
+
+  if (cloud == batch_size) {  // tail padding rows [total_n, pad_to_n)
+    const uint32_t row0 = total_n + tile * (kPshThreads * ITEMS);
+#pragma unroll
+    for (int j = 0; j < ITEMS; ++j) {
+      const uint32_t r = row0 + j * kPshThreads + tid;
+      if (r < pad_to_n) {
+        uint16_t* q = scatter_coord + 3 * (size_t)r;
+        q[0] = pad_bits; q[1] = pad_bits; q[2] = pad_bits;
+      }
+    }
+    return;
+  }
+
+  const uint32_t start = cloud ? batch_sep[cloud - 1] : 0u;
+  const uint32_t n = batch_sep[cloud] - start;
+  const uint32_t tile0 = tile * (kPshThreads * ITEMS);
+  if (tile0 >= n) return;
+
+  uint32_t* whist = lds;                             // [kPshWaves][num_bucket] per-wave counts
+  uint32_t* dst_base = lds + kPshWaves * num_bucket; // [num_bucket] bucket start row + tile base
+  uint32_t* slot_base = dst_base + num_bucket;       // [num_bucket] tile base inside the bucket
+  const uint32_t* tb = tile_base + ((size_t)cloud * max_tiles + tile) * num_bucket;
+  const uint32_t* cs = cumsum_counter + (size_t)cloud * num_bucket;
+  const uint32_t* cnt = bucket_counter + (size_t)cloud * num_bucket;
+  for (uint32_t b = tid; b < num_bucket; b += kPshThreads) {
+#pragma unroll
+    for (int w = 0; w < kPshWaves; ++w) whist[w * num_bucket + b] = 0u;
+    const uint32_t base = tb[b];
+    slot_base[b] = base;
+    dst_base[b] = start + (cs[b] - cnt[b]) + base;  // exclusive cumsum + tile base
+  }
+  __syncthreads();
+
+  const uint32_t w = tid / kWave, l = tid % kWave;
+  uint32_t* mine = whist + w * num_bucket;
+  uint32_t id[ITEMS], rank[ITEMS];
+#pragma unroll
+  for (int j = 0; j < ITEMS; ++j) {
+    const uint32_t local = tile0 + tile_pos<ITEMS>(w, j, l);
+    id[j] = (local < n) ? (uint32_t)bucket_id[(size_t)start + local] : 0xFFFFFFFFu;
+  }
+#pragma unroll
+  for (int j = 0; j < ITEMS; ++j) {
+    const bool valid = id[j] != 0xFFFFFFFFu;
+    const uint64_t peers = match_any(id[j], nbits, valid);
+    const uint32_t r = mask_rank(peers);
+    // the lowest peer claims the group's run of slots in the wave's counter and hands the old
+    // value to the others
+    uint32_t before = 0;
+    if (valid && r == 0) before = atomicAdd(&mine[id[j]], (uint32_t)__popcll(peers));
+    before = __shfl(before, __ffsll((unsigned long long)peers) - 1, kWave);
+    rank[j] = before + r;
+  }
+  __syncthreads();
+  // per-wave counts -> exclusive prefix over waves
+  for (uint32_t b = tid; b < num_bucket; b += kPshThreads) {
+    uint32_t run = 0;
+#pragma unroll
+    for (int ww = 0; ww < kPshWaves; ++ww) {
+      const uint32_t c = whist[ww * num_bucket + b];
+      whist[ww * num_bucket + b] = run;
+      run += c;
+    }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int j = 0; j < ITEMS; ++j) {
+    if (id[j] == 0xFFFFFFFFu) continue;
+    const uint32_t local = tile0 + tile_pos<ITEMS>(w, j, l);
+    const size_t g = (size_t)start + local;
+    const uint32_t in_tile = mine[id[j]] + rank[j];
+    bucket_offset[g] = slot_base[id[j]] + in_tile;
+    const size_t dst = (size_t)dst_base[id[j]] + in_tile;
+    const uint16_t* p = coord + 3 * g;
+    uint16_t* q = scatter_coord + 3 * dst;
+    q[0] = p[0]; q[1] = p[1]; q[2] = p[2];
+  }
+}
+
+// min / max of every axis over all points; two-level: per-workgroup partials then one finishing wave.
+__global__ __launch_bounds__(256) void bbox_partial_kernel(const uint16_t* __restrict__ coord, uint32_t total_n,
+                                                          float* __restrict__ partial) {
+  __shared__ float red[6][4];
+  float mn[3] = {INFINITY, INFINITY, INFINITY}, mx[3] = {-INFINITY, -INFINITY, -INFINITY};
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total_n; i += (size_t)gridDim.x * blockDim.x) {
+#pragma unroll
+    for (int d = 0; d < 3; ++d) {
+      const float v = half_bits_to_float(coord[3 * i + d]);
+      mn[d] = fminf(mn[d], v);
+      mx[d] = fmaxf(mx[d], v);
+    }
+  }
+#pragma unroll
+  for (int d = 0; d < 3; ++d)
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+      mn[d] = fminf(mn[d], __shfl_xor(mn[d], off, kWave));
+      mx[d] = fmaxf(mx[d], __shfl_xor(mx[d], off, kWave));
+    }
+  const uint32_t w = threadIdx.x / kWave;
+  if (threadIdx.x % kWave == 0)
+    for (int d = 0; d < 3; ++d) { red[d][w] = mn[d]; red[3 + d][w] = mx[d]; }
+  __syncthreads();
+  if (threadIdx.x < 6) {
+    float a = red[threadIdx.x][0];
+    for (int i = 1; i < 4; ++i) a = threadIdx.x < 3 ? fminf(a, red[threadIdx.x][i]) : fmaxf(a, red[threadIdx.x][i]);
+    partial[blockIdx.x * 6 + threadIdx.x] = a;
+  }
+}
+
+__global__ void bbox_final_kernel(const float* __restrict__ partial, uint32_t nblock, uint16_t* __restrict__ bbox_min,
+                                  uint16_t* __restrict__ bbox_max) {
+  const uint32_t d = threadIdx.x / kWave, l = threadIdx.x % kWave;  // 6 waves: one per output
+  float a = d < 3 ? INFINITY : -INFINITY;
+  for (uint32_t i = l; i < nblock; i += kWave) a = d < 3 ? fminf(a, partial[i * 6 + d]) : fmaxf(a, partial[i * 6 + d]);
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    const float o = __shfl_xor(a, off, kWave);
+    a = d < 3 ? fminf(a, o) : fmaxf(a, o);
+  }
+  if (l == 0) {
+    if (d < 3) bbox_min[d] = float_to_half_bits(a);
+    else bbox_max[d - 3] = float_to_half_bits(a);
+  }
+}
+
+static uint32_t pick_items(uint32_t instance_max_n, uint32_t batch_size) {
+  // Larger tiles amortise the per-tile histogram traffic; smaller tiles give small inputs enough
+  // workgroups to cover 256 CUs.
+  const uint64_t pts = (uint64_t)instance_max_n * batch_size;
+  if (pts >= (uint64_t)4 << 20) return 8;
+  if (pts >= (uint64_t)1 << 20) return 4;
+  if (pts >= (uint64_t)256 << 10) return 2;
+  return 1;
+}
+
+template <int ITEMS>
+static void launch_psh(const uint16_t* coord, uint16_t* bucket_id, uint32_t* bucket_counter, uint32_t* bucket_offset,
+                       const uint32_t* batch_sep, uint32_t batch_size, uint32_t total_n, uint32_t instance_max_n,
+                       uint32_t num_bucket, uint32_t divisor16, uint32_t num_vox, const uint16_t* bbox_min,
+                       const uint16_t* bbox_max, uint32_t* cumsum_counter, uint16_t* scatter_coord, uint32_t pad_to_n,
+                       uint16_t pad_bits, uint32_t hash_type, uint32_t* tile_hist, uint32_t max_tiles, uint32_t nbits,
+                       hipStream_t stream) {
+  const uint32_t tile_pts = kPshThreads * ITEMS;
+  if (max_tiles > 0 && batch_size > 0) {
+    hipLaunchKernelGGL(psh_hash_hist_kernel<ITEMS>, dim3(max_tiles, batch_size), dim3(kPshThreads),
+                       num_bucket * sizeof(uint32_t), stream, coord, bucket_id, batch_sep, bbox_min, bbox_max, num_vox,
+                       divisor16, num_bucket, hash_type, tile_hist, max_tiles);
+    hipLaunchKernelGGL(psh_scan_kernel, dim3(batch_size), dim3(kPshThreads), num_bucket * sizeof(uint32_t), stream,
+                       tile_hist, bucket_counter, cumsum_counter, batch_sep, num_bucket, tile_pts, max_tiles);
+  }
+  const uint32_t pad_tiles = cdiv_u32(pad_to_n - total_n, tile_pts);
+  const uint32_t gx = max_tiles > pad_tiles ? max_tiles : pad_tiles;
+  if (gx > 0) {
+    hipLaunchKernelGGL(psh_rank_scatter_kernel<ITEMS>, dim3(gx, batch_size + (pad_tiles ? 1 : 0)), dim3(kPshThreads),
+                       (kPshWaves + 2) * num_bucket * sizeof(uint32_t), stream, coord, bucket_id, bucket_offset,
+                       batch_sep, batch_size, tile_hist, bucket_counter, cumsum_counter, num_bucket, nbits, max_tiles,
+                       scatter_coord, total_n, pad_to_n, pad_bits);
+  }
+}
+
+}  // namespace f3d
+
+extern "C" {
+
+int f3d_batch_psh_scatter_pad_hash(const f3d_half_t* coord, uint16_t* bucket_id, uint32_t* bucket_counter,
+                                   uint32_t* bucket_offset, const uint32_t* batch_sep, uint32_t batch_size,
+                                   uint32_t total_n, uint32_t instance_max_n, uint32_t num_bucket,
+                                   uint32_t bucket_divisor, uint32_t bucket_size, uint32_t num_vox,
+                                   const f3d_half_t* bbox_min, const f3d_half_t* bbox_max,
+                                   const int16_t* probe_offsets, uint32_t* cumsum_counter,
+                                   f3d_half_t* scatter_coord, uint32_t pad_to_n, float pad_num,
+                                   uint32_t hash_type, int device, void* stream) {
+  using namespace f3d;
+  (void)bucket_size;
+  (void)probe_offsets;
+  // argument checks of src/psh/batch_psh_bucket_dispatcher.cu:239-250
+  F3D_CHECK_ARG(bucket_divisor != 0 && num_bucket != 0 && num_vox / bucket_divisor <= num_bucket,
+                "bucket divisor too small");
+  F3D_CHECK_ARG(pad_to_n >= total_n, "Output coord buffer length(%u) is smaller than the input length(%u).",
+                pad_to_n, total_n);
+  F3D_CHECK_ARG(hash_type >= 1 && hash_type <= 4,
+                "Currently only four types of hash modes are supported. Requested hash_type=%u is unsupported.",
+                hash_type);
+  if (!(num_bucket == 32 || num_bucket == 64 || num_bucket == 128 || num_bucket == 256 || num_bucket == 512 ||
+        num_bucket == 1024)) {
+    set_error("No kernel found for num_bucket=%u hash_type=%u", num_bucket, hash_type);
+    return F3D_ERR_UNSUPPORTED;
+  }
+  const uint32_t div16 = bucket_divisor & 0xFFFFu;
+  F3D_CHECK_ARG(div16 != 0 && (hash_type > 2 || 0xFFFFu / div16 < num_bucket), "bucket divisor too small");
+  F3D_CHECK_ARG(num_vox >= 2 && num_vox <= 0x10000u, "num_vox=%u does not fit the 16-bit voxel type", num_vox);
+  F3D_CHECK_ARG(coord && bucket_id && bucket_counter && bucket_offset && batch_sep && bbox_min && bbox_max &&
+                    cumsum_counter && scatter_coord,
+                "null tensor pointer");
+  if (pad_to_n == 0) return F3D_OK;
+
+  DeviceGuard guard(device);
+  F3D_CHECK_ARG(guard.ok, "cannot select device %d", device);
+  hipStream_t s = (hipStream_t)stream;
+  const uint32_t items = pick_items(instance_max_n, batch_size);
+  const uint32_t tile_pts = kPshThreads * items;
+  const uint32_t max_tiles = cdiv_u32(instance_max_n, tile_pts);
+  const size_t hist_bytes = (size_t)batch_size * max_tiles * num_bucket * sizeof(uint32_t);
+  uint32_t* tile_hist = (uint32_t*)workspace(device, hist_bytes ? hist_bytes : 4);
+  if (!tile_hist) return F3D_ERR_RUNTIME;
+  uint32_t nbits = 0;
+  while ((1u << nbits) < num_bucket) ++nbits;
+  _Float16 pad_h = (_Float16)pad_num;
+  uint16_t pad_bits;
+  __builtin_memcpy(&pad_bits, &pad_h, 2);
+
+  SyncBracket sync(s);
+#define F3D_PSH_CASE(I)                                                                                          \
+  case I:                                                                                                        \
+    launch_psh<I>(coord, bucket_id, bucket_counter, bucket_offset, batch_sep, batch_size, total_n, instance_max_n, \
+                  num_bucket, div16, num_vox, bbox_min, bbox_max, cumsum_counter, scatter_coord, pad_to_n, pad_bits, \
+                  hash_type, tile_hist, max_tiles, nbits, s);                                                   \
+    break;
+  switch (items) {
+    F3D_PSH_CASE(1)
+    F3D_PSH_CASE(2)
+    F3D_PSH_CASE(4)
+    F3D_PSH_CASE(8)
+  }
+#undef F3D_PSH_CASE
+  F3D_CHECK_HIP(hipGetLastError());
+  return F3D_OK;
+}
+
+int f3d_coord_bbox(const f3d_half_t* coord, uint32_t total_n, f3d_half_t* bbox_min, f3d_half_t* bbox_max, int device,
+                   void* stream) {
+  using namespace f3d;
+  F3D_CHECK_ARG(coord && bbox_min && bbox_max, "null tensor pointer");
+  F3D_CHECK_ARG(total_n > 0, "bounding box of an empty point set");
+  DeviceGuard guard(device);
+  F3D_CHECK_ARG(guard.ok, "cannot select device %d", device);
+  hipStream_t s = (hipStream_t)stream;
+  uint32_t nblock = cdiv_u32(total_n, 256 * 8);
+  if (nblock > 1024) nblock = 1024;
+  // partials live after the PSH histogram area would; a private slice at the workspace start is
+  // enough because the op is ordered on the same stream as its consumers
+  float* partial = (float*)workspace(device, (size_t)1024 * 6 * sizeof(float));
+  if (!partial) return F3D_ERR_RUNTIME;
+  SyncBracket sync(s);
+  hipLaunchKernelGGL(bbox_partial_kernel, dim3(nblock), dim3(256), 0, s, coord, total_n, partial);
+  hipLaunchKernelGGL(bbox_final_kernel, dim3(1), dim3(6 * kWave), 0, s, partial, nblock, bbox_min, bbox_max);
+  F3D_CHECK_HIP(hipGetLastError());
+  return F3D_OK;
+}
+
+}  // extern "C"

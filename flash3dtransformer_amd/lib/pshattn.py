@@ -1,0 +1,383 @@
+"""`pshattn` — the custom-op surface of the reference (pybind module built from
+src/f3d_frontend.cu:112-138), re-created over the C ABI of ``libf3d_hip.so``.
+
+Same function names and positional argument order as the reference module, so the layer code and
+tests that call ``pshattn.<op>(tensors..., scalars...)`` read the same.  Every function mutates
+caller-allocated output tensors in place and returns ``None``.  Tensor-level checks (contiguity,
+device, dtype) live here because the C ABI only sees pointers; value checks live in the library and
+come back as ``RuntimeError`` with the library's message — the reference's
+``throw std::runtime_error`` behaviour (src/common/runtime.h:36-86).
+
+There is no CPU fallback: if the HIP library is missing this module raises on import of the first op.
+"""
+import ctypes
+import os
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "libf3d_hip.so")
+_lib = None
+
+_u32, _i32, _f32, _vp = ctypes.c_uint32, ctypes.c_int, ctypes.c_float, ctypes.c_void_p
+
+
+def _load():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB_PATH):
+            raise RuntimeError(
+                f"{_LIB_PATH} is missing: build it with `python -m flash3dtransformer_amd.csrc.build` "
+                "(hipcc, gfx950). There is no CPU fallback for the Flash3D ops.")
+        _lib = ctypes.CDLL(_LIB_PATH)
+        _lib.f3d_last_error.restype = ctypes.c_char_p
+        _lib.f3d_get_seed.restype = ctypes.c_uint32
+    return _lib
+
+
+def library_path() -> str:
+    return _LIB_PATH
+
+
+def _check(rc: int):
+    if rc != 0:
+        raise RuntimeError(_load().f3d_last_error().decode("utf-8", "replace"))
+
+
+def _ptr(t):
+    return _vp(t.data_ptr()) if t is not None else _vp(0)
+
+
+def _stream(dev_index: int):
+    return _vp(torch.cuda.current_stream(dev_index).cuda_stream)
+
+
+def assert_contiguous(tensors):
+    """src/common/runtime.h assert_contiguous"""
+    for i, t in enumerate(tensors):
+        if not t.is_contiguous():
+            raise RuntimeError(f"Tensor #{i} is not contiguous.")
+
+
+def assert_same_device(tensors):
+    dev = tensors[0].device
+    for i, t in enumerate(tensors):
+        if t.device != dev:
+            raise RuntimeError(f"Tensor #{i} is on {t.device}, expected {dev}.")
+    if dev.type != "cuda":
+        raise RuntimeError(f"Flash3D ops need tensors on a GPU device, got {dev}.")
+    return dev.index if dev.index is not None else torch.cuda.current_device()
+
+
+def assert_dtype(tensors, dtype):
+    for i, t in enumerate(tensors):
+        if t.dtype != dtype:
+            raise RuntimeError(f"Tensor #{i} has dtype {t.dtype}, expected {dtype}.")
+
+
+class DeviceManagerSingleton:
+    """src/common/device_manager.{cuh,cu}; bound at src/f3d_frontend.cu:115-120"""
+    _inst = None
+
+    @staticmethod
+    def instance():
+        if DeviceManagerSingleton._inst is None:
+            DeviceManagerSingleton._inst = DeviceManagerSingleton()
+        return DeviceManagerSingleton._inst
+
+    def init_dev_info(self, dev_id: int):
+        _check(_load().f3d_init_dev_info(_i32(dev_id)))
+
+    def init_dispatchers(self):
+        _load()  # kernels are selected at call time; loading the library is all there is to do
+
+    def set_sync_stream(self, is_syncing: bool) -> bool:
+        return bool(_load().f3d_set_sync_stream(_i32(1 if is_syncing else 0)))
+
+    def get_sync_stream(self) -> bool:
+        return bool(_load().f3d_get_sync_stream())
+
+    # extensions -----------------------------------------------------------------------------
+    def set_seed(self, seed: int):
+        _check(_load().f3d_set_seed(_u32(seed)))
+
+    def get_seed(self) -> int:
+        return int(_load().f3d_get_seed())
+
+    def set_psh_rebalance(self, mode: int):
+        _check(_load().f3d_set_psh_rebalance(_i32(mode)))
+
+    def get_psh_rebalance(self) -> int:
+        return int(_load().f3d_get_psh_rebalance())
+
+
+# ---------------------------------------------------------------------------------------------
+# PSH bucketing
+# ---------------------------------------------------------------------------------------------
+
+def batch_psh_scatter_pad_hash(coord, bucket_id, bucket_counter, bucket_offset, batch_sep, instance_max_N,
+                               num_bucket, bucket_divisor, bucket_size, num_vox, bbox_min, bbox_max,
+                               probe_offsets, cumsum_counter, scatter_coord, pad_num, hash_type):
+    """src/f3d_frontend.cu:52-58 -> src/psh/batch_psh_bucket_dispatcher.cu:221-326"""
+    ts = [coord, bucket_id, bucket_counter, bucket_offset, batch_sep, probe_offsets, cumsum_counter, scatter_coord]
+    assert_contiguous(ts)
+    dev = assert_same_device(ts + [bbox_min, bbox_max])
+    assert_dtype([coord, bbox_min, bbox_max, scatter_coord], torch.float16)
+    assert_dtype([bucket_counter, bucket_offset, batch_sep, cumsum_counter], torch.uint32)
+    assert_dtype([bucket_id], torch.uint16)
+    bbox_min, bbox_max = bbox_min.contiguous(), bbox_max.contiguous()
+    _check(_load().f3d_batch_psh_scatter_pad_hash(
+        _ptr(coord), _ptr(bucket_id), _ptr(bucket_counter), _ptr(bucket_offset), _ptr(batch_sep),
+        _u32(batch_sep.shape[0]), _u32(coord.shape[0]), _u32(instance_max_N), _u32(num_bucket),
+        _u32(bucket_divisor), _u32(bucket_size), _u32(num_vox), _ptr(bbox_min), _ptr(bbox_max),
+        _ptr(probe_offsets), _ptr(cumsum_counter), _ptr(scatter_coord), _u32(scatter_coord.shape[0]),
+        _f32(pad_num), _u32(hash_type), _i32(dev), _stream(dev)))
+
+
+def batch_psh_scatter_pad(coord, bucket_id, bucket_counter, bucket_offset, batch_sep, instance_max_N,
+                          num_bucket, bucket_divisor, bucket_size, num_vox, bbox_min, bbox_max,
+                          probe_offsets, cumsum_counter, scatter_coord, pad_num):
+    """src/f3d_frontend.cu:45-50; hash fixed to H_ZORDER_MOD (batch_psh_bucket_dispatcher.cu:161-163)"""
+    batch_psh_scatter_pad_hash(coord, bucket_id, bucket_counter, bucket_offset, batch_sep, instance_max_N,
+                               num_bucket, bucket_divisor, bucket_size, num_vox, bbox_min, bbox_max,
+                               probe_offsets, cumsum_counter, scatter_coord, pad_num, 3)
+
+
+def batch_psh_scatter(coord, bucket_id, bucket_counter, bucket_offset, batch_sep, instance_max_N, num_bucket,
+                      bucket_divisor, bucket_size, num_vox, bbox_min, bbox_max, probe_offsets, cumsum_counter,
+                      scatter_coord, hash_dtype=None, coord_dtype=None, block_size_N=1024):
+    """src/f3d_frontend.cu:38-43: no tail padding (scatter_coord has exactly N rows); the dtype objects
+    and block size of the reference signature are accepted and unused (types are fixed on the wire)."""
+    if scatter_coord.shape[0] != coord.shape[0]:
+        raise RuntimeError(
+            f"Output coord buffer length({scatter_coord.shape[0]}) must equal the input length({coord.shape[0]}).")
+    batch_psh_scatter_pad_hash(coord, bucket_id, bucket_counter, bucket_offset, batch_sep, instance_max_N,
+                               num_bucket, bucket_divisor, bucket_size, num_vox, bbox_min, bbox_max,
+                               probe_offsets, cumsum_counter, scatter_coord, 0.0, 3)
+
+
+def coord_bbox(coord, bbox_min, bbox_max):
+    """extension: one-pass whole-batch bounding box (replaces torch.min/max of psh_main.py:117-118)"""
+    assert_contiguous([coord, bbox_min, bbox_max])
+    dev = assert_same_device([coord, bbox_min, bbox_max])
+    assert_dtype([coord, bbox_min, bbox_max], torch.float16)
+    _check(_load().f3d_coord_bbox(_ptr(coord), _u32(coord.shape[0]), _ptr(bbox_min), _ptr(bbox_max), _i32(dev),
+                                  _stream(dev)))
+
+
+def batch_bucket_sanitizer_cpu(bucket_id, bucket_counter, bucket_offset, offset_check_table, bucket_residual,
+                               batch_sep, offset_maxcnt, batch_size, num_bucket):
+    """src/psh/bucket_sanitizer_cpu.cpp:92-176 — host-side scoreboard: every (cloud, bucket,
+    slot < count) must be claimed exactly once.  Raises RuntimeError on the first violation and
+    writes the residual counts / hit table back, like the reference."""
+    ids = bucket_id.cpu().to(torch.int64)
+    cnt = bucket_counter.cpu().to(torch.int64)
+    off = bucket_offset.cpu().to(torch.int64)
+    seps = batch_sep.cpu().to(torch.int64)
+    maxcnt = offset_maxcnt.cpu().to(torch.int64)
+    table = offset_check_table.cpu().to(torch.int64)
+    res = bucket_residual.cpu().to(torch.int64)
+    start = 0
+    for b in range(batch_size):
+        end = int(seps[b])
+        i, o = ids[start:end], off[start:end]
+        bad = (i >= num_bucket) | (o >= maxcnt[b])
+        if bool(bad.any()):
+            c = int(torch.nonzero(bad)[0]) + start
+            raise RuntimeError(f"col={c}: buckid={int(ids[c])}|num_bucket={num_bucket}, "
+                               f"buckoff={int(off[c])}|offset_maxcnt={int(maxcnt[b])}, overflow ")
+        res[b] -= torch.bincount(i, minlength=num_bucket)[:num_bucket]
+        flat = table[b].reshape(-1)
+        flat += torch.bincount(i * table.shape[2] + o, minlength=flat.numel())
+        start = end
+    for b in range(batch_size):
+        slot = torch.arange(table.shape[2])[None, :]
+        wrong = (slot < cnt[b][:, None]) & (table[b] != 1)
+        if bool(wrong.any()):
+            k, s = [int(x) for x in torch.nonzero(wrong)[0]]
+            raise RuntimeError(f"Wrong scoreboard, batchid={b} buck={k},[Slot={s}|MaxCnt={int(cnt[b, k])}],"
+                               f"Score={int(table[b, k, s])}")
+    bucket_residual.copy_(res.to(bucket_residual.dtype))
+    offset_check_table.copy_(table.to(offset_check_table.dtype))
+
+
+# ---------------------------------------------------------------------------------------------
+# sub-bucket pooling / additive unpool
+# ---------------------------------------------------------------------------------------------
+
+def batch_subbuck_reduce(scattered_coord, scattered_feat, batch_sep, instance_max_N, subbuck_size, num_vox,
+                         bbox_min, bbox_max, subbuck_id, subbuck_off, reduced_batch_sep, reduced_coord,
+                         reduced_feat, unpool_ind, hash_type, red_op):
+    """src/f3d_frontend.cu:60-66 -> src/psh/batch_subbuck_pooling_dispatcher.cu:35-144"""
+    ts = [scattered_coord, scattered_feat, batch_sep, subbuck_id, subbuck_off, reduced_batch_sep, reduced_coord,
+          reduced_feat]
+    assert_contiguous(ts + [unpool_ind])
+    dev = assert_same_device(ts + [unpool_ind])
+    assert_dtype([scattered_feat, reduced_feat], torch.bfloat16)
+    assert_dtype([scattered_coord, reduced_coord, bbox_min, bbox_max], torch.float16)
+    assert_dtype([batch_sep, subbuck_id, reduced_batch_sep, unpool_ind], torch.uint32)
+    assert_dtype([subbuck_off], torch.uint16)
+    if scattered_feat.shape[1] != reduced_feat.shape[1]:
+        raise RuntimeError(f"Input feature dim({scattered_feat.shape[1]}) != output feature dim({reduced_feat.shape[1]}).")
+    if reduced_coord.shape[0] != reduced_feat.shape[0]:
+        raise RuntimeError(f"Reduced coordinate length({reduced_coord.shape[0]}) != reduced feature length({reduced_feat.shape[0]}).")
+    if scattered_coord.shape[1] != 3 or reduced_coord.shape[1] != 3:
+        raise RuntimeError(f"Input coordinates dim({scattered_coord.shape[1]}) or reduced coordinates "
+                           f"dim({reduced_coord.shape[1]}) are NOT 3D.")
+    if unpool_ind.shape[1] != subbuck_size:
+        raise RuntimeError(f"Unpool_ind last dimension({unpool_ind.shape[1]}) != subbucket_size({subbuck_size})")
+    # Rows of the feature tensor beyond the coordinate count are ignored, as in the reference
+    # (total_N is taken from the coordinates, dispatcher :43).
+    _check(_load().f3d_batch_subbuck_reduce(
+        _ptr(scattered_coord), _ptr(scattered_feat), _ptr(batch_sep), _u32(batch_sep.shape[0]),
+        _u32(scattered_coord.shape[0]), _u32(instance_max_N), _u32(scattered_feat.shape[1]), _u32(subbuck_size),
+        _u32(num_vox), _ptr(bbox_min.contiguous()), _ptr(bbox_max.contiguous()), _ptr(subbuck_id), _ptr(subbuck_off),
+        _ptr(reduced_batch_sep), _ptr(reduced_coord), _ptr(reduced_feat), _u32(reduced_feat.shape[0]),
+        _ptr(unpool_ind), _u32(unpool_ind.shape[0]), _u32(hash_type), _u32(red_op), _i32(dev), _stream(dev)))
+
+
+def batch_subbuck_reduce_backward(grad_red_feat, input_feat, unpool_ind, grad_input_feat, subbuck_size, red_op):
+    """src/f3d_frontend.cu:68-71 — backward is outside the forward hot path this library implements"""
+    raise NotImplementedError("batch_subbuck_reduce_backward: the gfx950 library implements the forward path only")
+
+
+def additive_unpool_fwd(res_feat, down_feat, up_add_feat, unpool_ind, subbuck_size):
+    """src/f3d_frontend.cu:99-101 -> src/psh/additive_unpool_dispatcher.cu:26-79"""
+    ts = [res_feat, down_feat, up_add_feat, unpool_ind]
+    assert_contiguous(ts)
+    dev = assert_same_device(ts)
+    assert_dtype([res_feat, down_feat, up_add_feat], torch.bfloat16)
+    assert_dtype([unpool_ind], torch.uint32)
+    if res_feat.shape != up_add_feat.shape:
+        raise RuntimeError(f"res_feat shape {tuple(res_feat.shape)} != up_add_feat shape {tuple(up_add_feat.shape)}")
+    if res_feat.shape[1] != down_feat.shape[1]:
+        raise RuntimeError(f"Feature dim mismatch: res({res_feat.shape[1]}) vs down({down_feat.shape[1]})")
+    if unpool_ind.shape[1] != subbuck_size:
+        raise RuntimeError(f"Unpool_ind last dimension({unpool_ind.shape[1]}) != subbucket_size({subbuck_size})")
+    if down_feat.shape[0] < unpool_ind.shape[0]:
+        raise RuntimeError(f"down_feat has {down_feat.shape[0]} rows, unpool_ind needs {unpool_ind.shape[0]}")
+    _check(_load().f3d_additive_unpool_fwd(
+        _ptr(res_feat), _ptr(down_feat), _ptr(up_add_feat), _ptr(unpool_ind), _u32(res_feat.shape[0]),
+        _u32(unpool_ind.shape[0]), _u32(res_feat.shape[1]), _u32(subbuck_size), _i32(dev), _stream(dev)))
+
+
+def additive_unpool_bwd(grad_res, grad_down, grad_up_added, unpool_ind, subbuck_size):
+    """src/f3d_frontend.cu:103-105 — backward, not part of the forward hot path"""
+    raise NotImplementedError("additive_unpool_bwd: the gfx950 library implements the forward path only")
+
+
+# ---------------------------------------------------------------------------------------------
+# bucketed attention
+# ---------------------------------------------------------------------------------------------
+
+def buck_swin_fwd(Q, K, V, O, L, Scope_buckets, bucket_size, kv_len=None):
+    """declared src/f3d_frontend.cu:90-92, called at flash3dxfmr/layers/buck_swin.py:57.
+    Q,K,V,O [B,L,H,D] bf16; L (LSE) [B,L,H] fp32; Scope_buckets [n_scope, scope_size] uint32.
+    Q/K/V may be column slices of one [B,L,3*H*D] projection output (equal row strides, dense last
+    two axes); O and L must be contiguous.  ``kv_len`` (extension) int32 [L/bucket_size]."""
+    dev = assert_same_device([Q, K, V, O, L, Scope_buckets])
+    assert_dtype([Q, K, V, O], torch.bfloat16)
+    assert_dtype([L], torch.float32)
+    assert_dtype([Scope_buckets], torch.uint32)
+    assert_contiguous([O, L, Scope_buckets])
+    if Q.dim() != 4 or Q.shape != K.shape or Q.shape != V.shape or Q.shape != O.shape:
+        raise RuntimeError(f"Q/K/V/O must share one [B,L,H,D] shape, got {tuple(Q.shape)} {tuple(K.shape)} "
+                           f"{tuple(V.shape)} {tuple(O.shape)}")
+    B, Ls, H, D = Q.shape
+    if tuple(L.shape) != (B, Ls, H):
+        raise RuntimeError(f"LSE shape {tuple(L.shape)} != {(B, Ls, H)}")
+    if Scope_buckets.dim() != 2:
+        raise RuntimeError("Scope_buckets must be [num_scopes, scope_size]")
+    for t in (Q, K, V):
+        if t.stride(3) != 1 or t.stride(2) != D or t.stride(0) != t.stride(1) * Ls or t.stride() != Q.stride():
+            raise RuntimeError("Q/K/V must be dense over (H, D) with identical strides")
+    if kv_len is not None:
+        assert_dtype([kv_len], torch.int32)
+        assert_contiguous([kv_len])
+    _check(_load().f3d_buck_swin_fwd_strided(
+        _ptr(Q), _ptr(K), _ptr(V), _u32(Q.stride(1)), _ptr(O), _ptr(L), _ptr(Scope_buckets),
+        _u32(Scope_buckets.shape[0]), _u32(Scope_buckets.shape[1]), _u32(bucket_size), _u32(B), _u32(Ls), _u32(H),
+        _u32(D), _ptr(kv_len), _i32(dev), _stream(dev)))
+
+
+def buck_swin_bwd(Q, K, V, O, dO, LSE, Delta, dQ, dK, dV, Scope_buckets, bucket_size):
+    """declared src/f3d_frontend.cu:94-97 — backward, not part of the forward hot path"""
+    raise NotImplementedError("buck_swin_bwd: the gfx950 library implements the forward path only")
+
+
+# ---------------------------------------------------------------------------------------------
+# dense layers
+# ---------------------------------------------------------------------------------------------
+
+def gemm_sm_bf16(A, B, O):
+    """src/f3d_frontend.cu:87-88: O[M,N] = A[M,K] @ B[K,N], bf16 in/out, fp32 accumulate"""
+    assert_contiguous([A, B, O])
+    dev = assert_same_device([A, B, O])
+    assert_dtype([A, B, O], torch.bfloat16)
+    M, K = A.shape
+    K2, N = B.shape
+    if K != K2 or tuple(O.shape) != (M, N):
+        raise RuntimeError(f"gemm shape mismatch: A{tuple(A.shape)} B{tuple(B.shape)} O{tuple(O.shape)}")
+    _check(_load().f3d_gemm_sm_bf16(_ptr(A), _ptr(B), _ptr(O), _u32(M), _u32(N), _u32(K), _i32(dev), _stream(dev)))
+    torch.cuda.current_stream(dev).synchronize()  # the reference op always synchronises (gemm_dispatcher.cu:77)
+
+
+ACT = {None: 0, "none": 0, "gelu": 1, "swiglu": 2, "silu": 3, "relu": 4}
+
+
+def linear_bf16(x, w, bias, residual, y, act=None):
+    """extension: y = act(x @ w.T + bias) + residual on MFMA (the nn.Linear / te.Linear sites)"""
+    dev = assert_same_device([x, w, y])
+    assert_dtype([x, w, y], torch.bfloat16)
+    assert_contiguous([w])
+    if x.dim() != 2 or y.dim() != 2 or x.stride(1) != 1 or y.stride(1) != 1:
+        raise RuntimeError("linear_bf16 expects 2-D row-major x and y")
+    m, k = x.shape
+    n = w.shape[0]
+    a = ACT[act] if not isinstance(act, int) else act
+    n_out = n // 2 if a == 2 else n
+    if w.shape[1] != k or tuple(y.shape) != (m, n_out):
+        raise RuntimeError(f"linear shape mismatch: x{tuple(x.shape)} w{tuple(w.shape)} y{tuple(y.shape)}")
+    if bias is not None:
+        assert_dtype([bias], torch.bfloat16)
+        assert_contiguous([bias])
+    ldr = 0
+    if residual is not None:
+        assert_dtype([residual], torch.bfloat16)
+        if tuple(residual.shape) != (m, n_out) or residual.stride(1) != 1:
+            raise RuntimeError("residual must be [m, n_out] row-major")
+        ldr = residual.stride(0)
+    _check(_load().f3d_linear_bf16(_ptr(x), _u32(x.stride(0)), _ptr(w), _ptr(bias), _ptr(residual), _u32(ldr),
+                                   _ptr(y), _u32(y.stride(0)), _u32(m), _u32(n), _u32(k), _u32(a), _i32(dev),
+                                   _stream(dev)))
+
+
+def layernorm_bf16(x, gamma, beta, y, eps=1e-5):
+    """extension: LayerNorm over the last axis, fp32 statistics"""
+    assert_contiguous([x, gamma, y])
+    dev = assert_same_device([x, gamma, y])
+    assert_dtype([x, gamma, y], torch.bfloat16)
+    m, c = x.shape
+    _check(_load().f3d_layernorm_bf16(_ptr(x), _ptr(gamma), _ptr(beta), _ptr(y), _u32(m), _u32(c), _f32(eps),
+                                      _i32(dev), _stream(dev)))
+
+
+def coord_embed_bf16(coord, w, bias, y):
+    """extension: y = bf16(coord) @ w.T + bias for w [C,3] (PSH3DCoordEmbedding, psh_ops.py:64-67)"""
+    assert_contiguous([coord, w, y])
+    dev = assert_same_device([coord, w, y])
+    assert_dtype([coord], torch.float16)
+    assert_dtype([w, y], torch.bfloat16)
+    _check(_load().f3d_coord_embed_bf16(_ptr(coord), _ptr(w), _ptr(bias), _ptr(y), _u32(coord.shape[0]),
+                                        _u32(w.shape[0]), _i32(dev), _stream(dev)))
+
+
+def affine_act_bf16(x, scale, shift, y, act=None):
+    """extension: y = act(x * scale + shift) per channel (eval BatchNorm1d folded + GELU/ReLU)"""
+    assert_contiguous([x, scale, shift, y])
+    dev = assert_same_device([x, scale, shift, y])
+    assert_dtype([x, y], torch.bfloat16)
+    assert_dtype([scale, shift], torch.float32)
+    a = ACT[act] if not isinstance(act, int) else act
+    _check(_load().f3d_affine_act_bf16(_ptr(x), _ptr(scale), _ptr(shift), _ptr(y), _u32(x.shape[0]),
+                                       _u32(x.shape[1]), _u32(a), _i32(dev), _stream(dev)))

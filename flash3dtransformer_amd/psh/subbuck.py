@@ -1,0 +1,67 @@
+"""Sub-bucket pooling buffers (reference: flash3dxfmr/psh/subbuck.py:40-132)."""
+import dataclasses as dcls
+
+import torch
+
+from .arithmatic import cdiv
+from . import batching as f3dbatch
+
+
+def calc_red_sep_sizes(seps: torch.Tensor, subbuck_size: int):
+    """Every cloud of n points pools to ceil(n / subbuck_size) rows: (total rows, per-cloud rows,
+    cumulative rows) with the dtype of `seps` (subbuck.py:40-53)."""
+    assert seps.dim() == 1, f"Seps dimension is expected to be 1, got {seps.dim()} instead"
+    sizes = f3dbatch.sep2sizes(seps.to(torch.int64))
+    red_sizes = torch.div(sizes + (subbuck_size - 1), subbuck_size, rounding_mode="floor")
+    return int(red_sizes.sum()), red_sizes.to(seps.dtype), torch.cumsum(red_sizes, dim=0).to(seps.dtype)
+
+
+@dcls.dataclass(slots=True)
+class SubbuckBuffers:
+    bbox_min: torch.Tensor
+    bbox_max: torch.Tensor
+    expect_sep: torch.Tensor
+    subbuck_id: torch.Tensor
+    subbuck_off: torch.Tensor
+    reduced_sep: torch.Tensor
+    reduced_coord: torch.Tensor
+    reduced_feat: torch.Tensor
+    unpool_ind: torch.Tensor
+
+    @staticmethod
+    def create_subbuck_buff(coords: torch.Tensor, input_feat: torch.Tensor, seps: torch.Tensor,
+                            subbuck_size=2, out_alignment=1):
+        """Allocation contract of batch_subbuck_reduce (subbuck.py:68-102).  `unpool_ind` MUST be
+        prefilled with an index >= N: that marks a slot no point was mapped to.  The reduced length is
+        rounded up to `out_alignment` so the next level's attention buckets divide it; the op
+        zero-fills the extra rows (the reference leaves them uninitialised)."""
+        total_n, d = coords.shape
+        dev = coords.device
+        # The op quantises inside each tile's own box; the whole-batch box is part of the reference
+        # signature only.  It is kept cheap: no reduction pass, just the representable range.
+        bbox_min = torch.full((d,), -65504.0, dtype=torch.float16, device=dev)
+        bbox_max = torch.full((d,), 65504.0, dtype=torch.float16, device=dev)
+        red_len, _, red_sep = calc_red_sep_sizes(seps, subbuck_size)
+        aligned = cdiv(red_len, out_alignment) * out_alignment
+        return SubbuckBuffers(
+            bbox_min, bbox_max, red_sep,
+            torch.zeros(total_n, dtype=torch.uint32, device=dev),
+            torch.empty(total_n, dtype=torch.uint16, device=dev),
+            red_sep,
+            torch.empty(aligned, d, dtype=torch.float16, device=dev),
+            torch.empty(aligned, input_feat.shape[1], dtype=input_feat.dtype, device=dev),
+            torch.full((red_len, subbuck_size), total_n + 3, dtype=torch.int32, device=dev).view(torch.uint32),
+        )
+
+    def remove_unused_buffers(self):
+        del self.subbuck_id
+        del self.subbuck_off
+
+
+@dcls.dataclass(slots=True)
+class UnpoolBuffers:
+    up_add_feat: torch.Tensor
+
+    @staticmethod
+    def create_unpool_buff(residual_feat: torch.Tensor):
+        return UnpoolBuffers(torch.empty_like(residual_feat))

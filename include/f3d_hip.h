@@ -1,0 +1,185 @@
+/*
+ * C ABI of libf3d_hip.so — the gfx950 (MI355X) implementation of the Flash3D forward hot path.
+ *
+ * Every entry point is what a host binding for this path binds: plain pointers to DEVICE memory
+ * (unless a parameter says "host"), sizes, and the HIP stream to launch on (`stream` is a
+ * hipStream_t passed as void*, nullptr = the default stream).  Outputs are caller-allocated and
+ * written in place, exactly as the reference's pybind functions do with at::Tensor& arguments
+ * (src/f3d_frontend.cu:38-105).  All calls are asynchronous on `stream` unless
+ * f3d_set_sync_stream(1) is in force.
+ *
+ * Return value: F3D_OK, or an error code with a message available from f3d_last_error().  Argument
+ * violations mirror the reference's `throw std::runtime_error` sites; the host binding turns a
+ * non-zero return into its language's exception.
+ *
+ * Types on the wire (reference: CoordT=fp16, CounterT=uint32, HashT=uint16, FeatT=bf16,
+ * src/psh/batch_psh_bucket_dispatcher.cu:252-254, src/psh/batch_subbuck_pooling_dispatcher.cu:45-48):
+ *   f3d_half_t  IEEE binary16 bit pattern          f3d_bf16_t  bfloat16 bit pattern
+ */
+#ifndef F3D_HIP_H
+#define F3D_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef uint16_t f3d_half_t;
+typedef uint16_t f3d_bf16_t;
+
+#define F3D_OK 0
+#define F3D_ERR_INVALID 1     /* bad argument (reference: std::runtime_error from a dispatcher) */
+#define F3D_ERR_UNSUPPORTED 2 /* no kernel for this configuration (reference: "No kernel found") */
+#define F3D_ERR_RUNTIME 3     /* HIP runtime failure */
+
+/* hash_type values, src/psh/hash_fns.cuh:151-158 */
+#define F3D_H_ZORDER_DIV 1
+#define F3D_H_XORSUM_DIV 2
+#define F3D_H_ZORDER_MOD 3
+#define F3D_H_XORSUM_MOD 4
+
+/* reduction ops, src/psh/batch_psh_subbuck_reduce.cuh:47-52 */
+#define F3D_O_MEAN 0
+#define F3D_O_SUM 1
+#define F3D_O_MIN 2
+#define F3D_O_MAX 3
+
+/* activation / epilogue selectors of f3d_linear_bf16 */
+#define F3D_ACT_NONE 0
+#define F3D_ACT_GELU 1   /* exact erf GELU */
+#define F3D_ACT_SWIGLU 2 /* out[:, j] = silu(acc[:, j]) * acc[:, j + N/2]; output has N/2 columns */
+#define F3D_ACT_SILU 3
+#define F3D_ACT_RELU 4
+
+/* ---- module state: DeviceManagerSingleton, src/common/device_manager.cu:58-119,
+ *      src/f3d_frontend.cu:115-120 ------------------------------------------------------------ */
+
+const char* f3d_last_error(void);      /* message of the last failing call on this thread */
+int f3d_init_dev_info(int device);     /* init_dev_info: per-device one-time setup (idempotent) */
+int f3d_set_sync_stream(int enable);   /* set_sync_stream: returns the new value */
+int f3d_get_sync_stream(void);         /* get_sync_stream */
+/* Seed of the stateless generator behind the sub-bucket rotation and the overflow probes.  The
+ * reference seeds cuRAND with 3407 (device_manager.cu:66); same default here. */
+int f3d_set_seed(uint32_t seed);
+uint32_t f3d_get_seed(void);
+
+/* ---- PSH bucketing: batch_psh_scatter_pad_hash, src/f3d_frontend.cu:52-58,
+ *      src/psh/batch_psh_bucket_dispatcher.cu:221-326 ------------------------------------------
+ * coord [total_n,3] fp16; bucket_id [total_n] u16; bucket_counter, cumsum_counter
+ * [batch_size,num_bucket] u32 (bucket_counter is accumulated into: zero it first);
+ * bucket_offset [total_n] u32; batch_sep [batch_size] u32 inclusive cumulative sizes;
+ * bbox_min/max [3] fp16; probe_offsets [128,3] i16 (may be NULL when rebalancing is off);
+ * scatter_coord [pad_to_n,3] fp16; rows [total_n,pad_to_n) receive pad_num.
+ * Slots inside a bucket follow input order (the reference's order is arbitration-dependent).
+ * Uses the per-device workspace: not re-entrant per device. */
+int f3d_batch_psh_scatter_pad_hash(const f3d_half_t* coord, uint16_t* bucket_id, uint32_t* bucket_counter,
+                                   uint32_t* bucket_offset, const uint32_t* batch_sep, uint32_t batch_size,
+                                   uint32_t total_n, uint32_t instance_max_n, uint32_t num_bucket,
+                                   uint32_t bucket_divisor, uint32_t bucket_size, uint32_t num_vox,
+                                   const f3d_half_t* bbox_min, const f3d_half_t* bbox_max,
+                                   const int16_t* probe_offsets, uint32_t* cumsum_counter,
+                                   f3d_half_t* scatter_coord, uint32_t pad_to_n, float pad_num,
+                                   uint32_t hash_type, int device, void* stream);
+
+/* Overflow handling of the bucketing op (src/psh/batch_psh_bucket.cuh:154-246, 259-382).
+ * 0 = hash + claim only (every point stays in its first-hash bucket);
+ * 1 = deterministic probe rebalance + recycle (default). */
+int f3d_set_psh_rebalance(int mode);
+int f3d_get_psh_rebalance(void);
+
+/* Whole-batch bounding box of fp16 coordinates (replaces the two torch.min/max passes of
+ * flash3dxfmr/psh/psh_main.py:117-118).  bbox_min/max [3] fp16, written in place. */
+int f3d_coord_bbox(const f3d_half_t* coord, uint32_t total_n, f3d_half_t* bbox_min, f3d_half_t* bbox_max,
+                   int device, void* stream);
+
+/* ---- sub-bucket pooling: batch_subbuck_reduce, src/f3d_frontend.cu:60-66,
+ *      src/psh/batch_subbuck_pooling_dispatcher.cu:35-144 ---------------------------------------
+ * scattered_coord [total_n,3] fp16; scattered_feat [total_n,feat_dim] bf16; subbuck_id [total_n] u32;
+ * subbuck_off [total_n] u16; reduced_batch_sep [batch_size] u32 (input: cumsum of ceil(n_b/S));
+ * reduced_coord [reduced_aligned_n,3] fp16; reduced_feat [reduced_aligned_n,feat_dim] bf16;
+ * unpool_ind [reduced_n,subbuck_size] u32 prefilled with a value >= total_n ("empty slot").
+ * hash_type is accepted and ignored, as in the reference (dispatcher :108-109).
+ * Rows [reduced_n, reduced_aligned_n) of reduced_coord / reduced_feat are zero-filled. */
+int f3d_batch_subbuck_reduce(const f3d_half_t* scattered_coord, const f3d_bf16_t* scattered_feat,
+                             const uint32_t* batch_sep, uint32_t batch_size, uint32_t total_n,
+                             uint32_t instance_max_n, uint32_t feat_dim, uint32_t subbuck_size,
+                             uint32_t num_vox, const f3d_half_t* bbox_min, const f3d_half_t* bbox_max,
+                             uint32_t* subbuck_id, uint16_t* subbuck_off, const uint32_t* reduced_batch_sep,
+                             f3d_half_t* reduced_coord, f3d_bf16_t* reduced_feat, uint32_t reduced_aligned_n,
+                             uint32_t* unpool_ind, uint32_t reduced_n, uint32_t hash_type, uint32_t red_op,
+                             int device, void* stream);
+
+/* The two halves of the op above, separately callable (kernels local_subbuck_ker and
+ * reduce_feat_ker, src/psh/batch_psh_subbuck_reduce.cuh:104-298 and :300-359). */
+int f3d_subbuck_build(const f3d_half_t* coord, const uint32_t* batch_sep, uint32_t batch_size,
+                      uint32_t total_n, uint32_t instance_max_n, uint32_t subbuck_size, uint32_t num_vox,
+                      uint32_t* subbuck_id, uint16_t* subbuck_off, const uint32_t* reduced_batch_sep,
+                      f3d_half_t* reduced_coord, uint32_t reduced_aligned_n, uint32_t* unpool_ind,
+                      uint32_t reduced_n, int device, void* stream);
+int f3d_reduce_feat(const f3d_bf16_t* feat, uint32_t total_n, uint32_t feat_dim, const uint32_t* unpool_ind,
+                    uint32_t reduced_n, uint32_t subbuck_size, uint32_t red_op, f3d_bf16_t* reduced_feat,
+                    uint32_t reduced_aligned_n, int device, void* stream);
+
+/* ---- additive unpool: additive_unpool_fwd, src/f3d_frontend.cu:99-101,
+ *      src/psh/additive_unpool_dispatcher.cu:26-79 ----------------------------------------------
+ * up[r,:] = bf16(float(down[i,:]) + float(res[r,:])) for r = unpool_ind[i,s] < up_n. */
+int f3d_additive_unpool_fwd(const f3d_bf16_t* res_feat, const f3d_bf16_t* down_feat, f3d_bf16_t* up_add_feat,
+                            const uint32_t* unpool_ind, uint32_t up_n, uint32_t down_n, uint32_t feat_dim,
+                            uint32_t subbuck_size, int device, void* stream);
+
+/* ---- bucketed attention forward: buck_swin_fwd, declared src/f3d_frontend.cu:90-92, called from
+ *      flash3dxfmr/layers/buck_swin.py:57 (kernel source absent from the reference) --------------
+ * q,k,v,o [batch,seq_len,num_head,head_dim] bf16 contiguous; lse [batch,seq_len,num_head] fp32;
+ * scope_buckets [num_scope,scope_size] u32; every scope attends within the union of its buckets
+ * (rows [k*bucket_size,(k+1)*bucket_size)).  kv_len (may be NULL) [seq_len/bucket_size] i32 is an
+ * extension: valid rows per bucket; masked query rows get o = 0, lse = 0. */
+int f3d_buck_swin_fwd(const f3d_bf16_t* q, const f3d_bf16_t* k, const f3d_bf16_t* v, f3d_bf16_t* o, float* lse,
+                      const uint32_t* scope_buckets, uint32_t num_scope, uint32_t scope_size,
+                      uint32_t bucket_size, uint32_t batch, uint32_t seq_len, uint32_t num_head,
+                      uint32_t head_dim, const int32_t* kv_len, int device, void* stream);
+
+/* Strided variant: q/k/v rows are `qkv_row_stride` elements apart (e.g. the three thirds of one
+ * [seq, 3*C] projection output), which removes the three .contiguous() copies of
+ * flash3dxfmr/layers/buck_swin.py:187-190.  o is dense [batch,seq_len,num_head,head_dim]. */
+int f3d_buck_swin_fwd_strided(const f3d_bf16_t* q, const f3d_bf16_t* k, const f3d_bf16_t* v,
+                              uint32_t qkv_row_stride, f3d_bf16_t* o, float* lse,
+                              const uint32_t* scope_buckets, uint32_t num_scope, uint32_t scope_size,
+                              uint32_t bucket_size, uint32_t batch, uint32_t seq_len, uint32_t num_head,
+                              uint32_t head_dim, const int32_t* kv_len, int device, void* stream);
+
+/* ---- dense layers --------------------------------------------------------------------------
+ * gemm_sm_bf16(A[M,K], B[K,N], O[M,N]) — src/f3d_frontend.cu:87-88, src/psh/gemm_dispatcher.cu;
+ * the reference only accepts M == 128, this one any shape with K % 8 == 0 and N % 8 == 0. */
+int f3d_gemm_sm_bf16(const f3d_bf16_t* a, const f3d_bf16_t* b, f3d_bf16_t* o, uint32_t m, uint32_t n,
+                     uint32_t k, int device, void* stream);
+
+/* y = act(x · wᵀ + bias) + residual — the nn.Linear / te.Linear sites of the layer API
+ * (flash3dxfmr/layers/buck_swin.py:159,163; hourglass.py:65,148,150; flash3d.py:32).
+ * x [m,k] bf16 (row stride ldx), w [n,k] bf16, bias [n] bf16 or NULL, residual [m,n_out] bf16 or
+ * NULL (row stride ldr), y [m,n_out] bf16 (row stride ldy); n_out = n/2 for F3D_ACT_SWIGLU else n.
+ * fp32 accumulate; k % 8 == 0. */
+int f3d_linear_bf16(const f3d_bf16_t* x, uint32_t ldx, const f3d_bf16_t* w, const f3d_bf16_t* bias,
+                    const f3d_bf16_t* residual, uint32_t ldr, f3d_bf16_t* y, uint32_t ldy, uint32_t m,
+                    uint32_t n, uint32_t k, uint32_t act, int device, void* stream);
+
+/* LayerNorm over the last axis, fp32 statistics (norm callables of flash3dxfmr/layers/stage.py:67).
+ * x,y [m,c] bf16; gamma,beta [c] bf16 (beta may be NULL). */
+int f3d_layernorm_bf16(const f3d_bf16_t* x, const f3d_bf16_t* gamma, const f3d_bf16_t* beta, f3d_bf16_t* y,
+                       uint32_t m, uint32_t c, float eps, int device, void* stream);
+
+/* Coordinate embedding input cast + K=3 linear of PSH3DCoordEmbedding
+ * (flash3dxfmr/layers/psh_ops.py:64-67): y[r,:] = bf16(coord[r,:]) · wᵀ + bias; w [c,3] bf16. */
+int f3d_coord_embed_bf16(const f3d_half_t* coord, const f3d_bf16_t* w, const f3d_bf16_t* bias, f3d_bf16_t* y,
+                         uint32_t m, uint32_t c, int device, void* stream);
+
+/* Per-channel affine + optional activation: eval-mode BatchNorm1d folded to scale/shift followed
+ * by GELU/ReLU (pool / unpool norm+act callables, tests/test_psh_hourglass.py:103-106).
+ * y = act(x * scale + shift); x,y [m,c] bf16; scale,shift [c] fp32. */
+int f3d_affine_act_bf16(const f3d_bf16_t* x, const float* scale, const float* shift, f3d_bf16_t* y, uint32_t m,
+                        uint32_t c, uint32_t act, int device, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* F3D_HIP_H */

@@ -1,0 +1,147 @@
+"""GPU parity of PSH bucketing (rows A1-A3, A5) against the CPU oracle, through the C ABI
+(pshattn -> libf3d_hip.so).  Bit-exact: bucket ids, histograms, slots (stable order), cumsum and
+every scattered coordinate row.  Also the reference's own invariants (tests/test_psh.py:117-129 of
+the reference): no NaN left, cumsum identity, scoreboard."""
+import numpy as np
+import pytest
+import torch
+
+from tests.gpu_util import DEV, n_f16, n_u16, n_u32, t_f16, t_u32
+
+pytestmark = pytest.mark.gpu
+
+
+def _run_psh(coords, seps, bucket_size, hash_op, pad_align, oracle, rebalance=0):
+    from flash3dtransformer_amd.lib import pshattn
+    from flash3dtransformer_amd.psh import bucket as f3dbuck
+    nb, div, max_n = oracle.psh_params(seps, bucket_size)
+    n = coords.shape[0]
+    pad_to = -(-n // pad_align) * pad_align
+    c, s = t_f16(coords), t_u32(seps)
+    bucket_id = torch.ones(n, dtype=torch.uint16, device=DEV)
+    cntr = torch.zeros(len(seps), nb, dtype=torch.uint32, device=DEV)
+    offs = torch.empty(n, dtype=torch.uint32, device=DEV)
+    cumsum = torch.zeros_like(cntr)
+    probes = f3dbuck.generate_probe_offsets(DEV, shuffle_seed=0)
+    scat = torch.full((pad_to, 3), float("nan"), dtype=torch.float16, device=DEV)
+    bmin, bmax = torch.min(c, dim=0)[0], torch.max(c, dim=0)[0]
+    mgr = pshattn.DeviceManagerSingleton.instance()
+    mgr.init_dev_info(0)
+    mgr.set_sync_stream(True)
+    mgr.set_psh_rebalance(rebalance)
+    pshattn.batch_psh_scatter_pad_hash(c, bucket_id, cntr, offs, s, max_n, nb, div, bucket_size, 0xFFFF, bmin, bmax,
+                                       probes, cumsum, scat, 0.0, hash_op)
+    torch.cuda.synchronize()
+    return dict(nb=nb, div=div, pad_to=pad_to, ids=n_u16(bucket_id), cnt=n_u32(cntr), off=n_u32(offs),
+                cumsum=n_u32(cumsum), scat=n_f16(scat), bmin=n_f16(bmin), bmax=n_f16(bmax),
+                t=(bucket_id, cntr, offs, s))
+
+
+def _check_against_oracle(coords, seps, out, hash_op, oracle):
+    ids, cnt, off = oracle.psh_claim(coords, seps, out["bmin"], out["bmax"], 0xFFFF, out["div"], out["nb"], hash_op)
+    cumsum, scat = oracle.cumsum_scatter_pad(coords, seps, out["nb"], ids, cnt, off, out["pad_to"], 0.0)
+    assert np.array_equal(out["ids"], ids), "bucket ids differ"
+    assert np.array_equal(out["cnt"], cnt), "bucket histograms differ"
+    assert np.array_equal(out["off"], off), "slots differ (stable order expected)"
+    assert np.array_equal(out["cumsum"], cumsum)
+    assert np.array_equal(out["scat"].view(np.uint16), scat.view(np.uint16)), "scattered rows differ"
+
+
+@pytest.mark.parametrize("hash_op", [1, 2, 3, 4])
+def test_c1_uniform_cube_bit_exact(oracle, hash_op):
+    """BASELINE config 1: 1 x 32,768 points uniform in a 51.2 m cube, bucket 512 -> 64 buckets"""
+    from flash3dtransformer_amd import synth
+    coords, seps = synth.batch_of([synth.uniform_cube(32768, 51.2, 1001)])
+    out = _run_psh(coords, seps, 512, hash_op, 512, oracle)
+    assert out["nb"] == 64 and out["div"] == 1024
+    _check_against_oracle(coords, seps, out, hash_op, oracle)
+    assert not np.isnan(out["scat"]).any()
+    rc, _ = oracle.scoreboard(out["ids"], out["cnt"], out["off"], seps)
+    assert rc == 0
+
+
+@pytest.mark.parametrize("sizes,bucket_size", [
+    ([20000, 17001, 23456], 512),          # ragged batch, partial tail tiles
+    ([70000, 300, 65000, 1], 512),         # tiny and single-point clouds next to large ones
+    ([9000, 0, 8000], 256),                # an empty cloud in the middle
+    ([300000, 280000], 512),               # 512 buckets, multi-item tiles
+])
+def test_ragged_batches_bit_exact(oracle, sizes, bucket_size):
+    rng = np.random.default_rng(sum(sizes))
+    pts = np.concatenate([rng.normal(0, 20, (n, 3)) + rng.uniform(-5, 5, 3) for n in sizes]).astype(np.float16)
+    seps = np.cumsum(sizes).astype(np.uint32)
+    for hash_op in (1, 4):
+        out = _run_psh(pts, seps, bucket_size, hash_op, bucket_size * 6, oracle)
+        _check_against_oracle(pts, seps, out, hash_op, oracle)
+        n = pts.shape[0]
+        assert (out["scat"][n:] == 0).all() and not np.isnan(out["scat"]).any()
+
+
+def test_lidar_batch_reference_invariants(oracle):
+    """4 synthetic sweeps (heavily clustered): the reference's three checks, through its own
+    sanitizer entry point"""
+    from flash3dtransformer_amd import synth
+    from flash3dtransformer_amd.lib import pshattn
+    clouds = [synth.lidar_sweep(30000, 1004 + i, oversample=2) for i in range(4)]
+    coords, seps = synth.batch_of(clouds)
+    for hash_op in (1, 2, 3, 4):
+        out = _run_psh(coords, seps, 512, hash_op, 512, oracle)
+        _check_against_oracle(coords, seps, out, hash_op, oracle)
+        bucket_id, cntr, offs, s = out["t"]
+        assert not np.isnan(out["scat"]).any()
+        assert np.array_equal(np.cumsum(out["cnt"], axis=1), out["cumsum"])
+        maxc = int(out["cnt"].max())
+        table = torch.zeros((4, out["nb"], maxc), dtype=torch.int8, device=DEV)
+        res = cntr.clone()
+        maxcnt = torch.from_numpy(out["cnt"].max(1).astype(np.int32)).to(DEV).view(torch.uint32)
+        pshattn.batch_bucket_sanitizer_cpu(bucket_id, cntr, offs, table, res, s, maxcnt, 4, out["nb"])
+        assert int(res.view(torch.int32).abs().sum()) == 0
+
+
+def test_degenerate_axis_and_special_values(oracle):
+    """flat cloud (z constant -> 0/0 in the quantiser) and points outside the given box"""
+    rng = np.random.default_rng(1)
+    pts = rng.uniform(-10, 10, (20000, 3)).astype(np.float16)
+    pts[:, 2] = np.float16(1.5)
+    seps = np.array([20000], np.uint32)
+    out = _run_psh(pts, seps, 512, 1, 512, oracle)
+    _check_against_oracle(pts, seps, out, 1, oracle)
+
+
+def test_bbox_kernel_matches_torch():
+    from flash3dtransformer_amd.lib import pshattn
+    g = torch.Generator().manual_seed(3)
+    for n in (1, 63, 4097, 500001):
+        c = (torch.randn(n, 3, generator=g) * 30).to(torch.float16).to(DEV)
+        bb = torch.empty(2, 3, dtype=torch.float16, device=DEV)
+        pshattn.coord_bbox(c, bb[0], bb[1])
+        assert torch.equal(bb[0], c.min(0)[0]) and torch.equal(bb[1], c.max(0)[0])
+
+
+def test_python_wrapper_and_saturating_size_properties(oracle):
+    """psh_main.batch_bucket_scatter on 16 x 262,144 points: size-independent properties only
+    (multiset of rows preserved, rows sorted by bucket id inside each cloud, pads zero)"""
+    from flash3dtransformer_amd.psh import psh_main
+    n_c, b = 262144, 16
+    g = torch.Generator().manual_seed(5)
+    coords = (torch.rand(n_c * b, 3, generator=g) * 51.2).to(torch.float16).to(DEV)
+    seps = (torch.arange(1, b + 1, dtype=torch.int32) * n_c).to(DEV).view(torch.uint32)
+    pad_to = -(-coords.shape[0] // 3072) * 3072
+    scat, buf = psh_main.batch_bucket_scatter(coords, seps, 512, pad_to, 2)
+    torch.cuda.synchronize()
+    assert not torch.isnan(scat).any()
+    cnt = buf.bucket_cntr.view(torch.int32).long()
+    assert torch.equal(torch.cumsum(cnt, 1), buf.bucket_cumsum.view(torch.int32).long())
+    assert int(cnt.sum()) == n_c * b
+    # checksum of rows is permutation invariant per cloud
+    key = lambda t: (t.view(torch.int16).long() & 0xFFFF).mul(torch.tensor([1, 65536, 65536 ** 2], device=DEV)).sum(1)
+    kin, kout = key(coords).view(b, n_c), key(scat[:n_c * b]).view(b, n_c)
+    assert torch.equal(kin.sort(1)[0], kout.sort(1)[0])
+    # recompute bucket ids of the scattered rows: must be non-decreasing inside each cloud
+    ids = buf.bucket_id.view(torch.int16).long() & 0xFFFF
+    excl = torch.cumsum(cnt, 1) - cnt
+    dst = (torch.arange(b, device=DEV).repeat_interleave(n_c) * n_c
+           + excl.view(-1)[torch.arange(b, device=DEV).repeat_interleave(n_c) * cnt.shape[1] + ids]
+           + buf.bucket_offs.view(torch.int32).long())
+    assert torch.equal(scat[dst], coords)
+    assert dst.unique().numel() == n_c * b

@@ -69,7 +69,13 @@ def test_vox_bruteforce_all_fp16(oracle):
     got = oracle.vox_coord(coords, np.array([mn] * 3, np.float16), np.array([mx] * 3, np.float16))
     c32 = c.astype(np.float32)
     with np.errstate(all="ignore"):
-        q = ((c32 - np.float32(mn)) * np.float32(65535.0)) / (np.float32(mx) - np.float32(mn))
+        inv = np.float32(1.0) / (np.float32(mx) - np.float32(mn))
+        q = ((c32 - np.float32(mn)) * np.float32(65535.0)) * inv
+        q_div = ((c32 - np.float32(mn)) * np.float32(65535.0)) / (np.float32(mx) - np.float32(mn))
+    # the reciprocal form may differ from true division only by landing on the other side of an
+    # integer boundary, i.e. by one cell, and only rarely
+    d = np.abs(np.clip(np.floor(q), 0, 65534) - np.clip(np.floor(q_div), 0, 65534))
+    assert d.max() <= 1 and (d > 0).mean() < 0.01
     want = np.clip(np.floor(q), 0, 65534).astype(np.uint16)
     assert np.array_equal(got[:, 0], want)
     assert np.array_equal(got[:, 2], want)
