@@ -27,7 +27,6 @@ struct alignas(16) U16x8 {
 };
 
 constexpr int kAttnThreads = 256;
-constexpr int kAttnWaves = 4;
 constexpr int kQBlock = 128;  // query rows per workgroup
 constexpr int kNumXcd = 8;
 

@@ -1,0 +1,69 @@
+"""Bucketed (scoped) multi-head self-attention (reference: flash3dxfmr/layers/buck_swin.py)."""
+from typing import Tuple
+
+import torch
+import torch.cuda.nvtx as nvtx
+from torch import nn
+from torch.autograd import Function
+
+from ..lib import pshattn
+from ..psh import dev_context as f3ddev
+from ..psh import swin_attn as sa
+from .nn_ops import Linear
+
+
+class BuckSwinFwdFunction(Function):
+    """O = attention(Q, K, V) inside every scope of buckets; keeps (Q, K, V, O, LSE) for a backward
+    pass that this library does not provide (buck_swin.py:20-95 of the reference)."""
+
+    @staticmethod
+    def forward(ctx, Q, K, V, scope_buckets, buck_size: int) -> torch.Tensor:
+        buff = sa.BuckSwinFwdBuffers.create_buckswin_fwd_buff(Q)
+        pshattn.buck_swin_fwd(Q, K, V, buff.O, buff.LSE, scope_buckets, buck_size)
+        ctx.save_for_backward(Q, K, V, buff.O, buff.LSE)
+        ctx.scope_buckets, ctx.buck_size = scope_buckets, buck_size
+        return buff.O
+
+    @staticmethod
+    def backward(ctx, grad_output) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, None, None]:
+        raise NotImplementedError("buck_swin_bwd: the gfx950 library implements the forward pass only")
+
+
+class BucketSwinAttention(nn.Module):
+    def __init__(self, buck_size: int) -> None:
+        super().__init__()
+        self.buck_size = buck_size
+
+    def forward(self, Q, K, V, scope_buckets) -> torch.Tensor:
+        assert Q.dim() == 4, f"Expect Q with four axes [B, L, H, D], but got shape={Q.shape}"
+        return BuckSwinFwdFunction.apply(Q, K, V, scope_buckets, self.buck_size)
+
+
+class BucketSwinAttentionModule(nn.Module):
+    NVTX_SCOPE = "BucketSwinAttention"
+
+    def __init__(self, channels: int, num_heads: int, buck_size: int, qkv_bias: bool = True):
+        super().__init__()
+        assert channels % num_heads == 0, f"Channels={channels} NOT divisible by num_heads={num_heads}"
+        self.num_heads = num_heads
+        self.head_dim = channels // num_heads
+        self.qkv = Linear(channels, channels * 3, bias=qkv_bias)
+        self.attn = BucketSwinAttention(buck_size)
+        self.proj = Linear(channels, channels)
+
+    def forward(self, x: torch.Tensor, scope_buckets: torch.Tensor, residual: torch.Tensor = None) -> torch.Tensor:
+        """x [B, L, C] -> [B, L, C].  Q, K and V are read by the attention kernel straight out of the
+        [B, L, 3C] projection output (the reference makes three contiguous copies, :187-190); the
+        residual, when given, is added in the out-projection's epilogue."""
+        assert x.dim() == 3, f"Expect input features with three axes [B, L, C], but got shape={x.shape}"
+        B, L, C = x.shape
+        assert C == self.num_heads * self.head_dim, f"Expect input channels are {self.num_heads * self.head_dim}, but got {C}"
+        if f3ddev.get_nvtx():
+            nvtx.range_push(self.NVTX_SCOPE)
+        qkv = self.qkv(x)
+        q, k, v = (t.view(B, L, self.num_heads, self.head_dim) for t in torch.chunk(qkv, 3, dim=-1))
+        attn_out = self.attn(q, k, v, scope_buckets)
+        out = self.proj(attn_out.view(B, L, C), residual=residual)
+        if f3ddev.get_nvtx():
+            nvtx.range_pop()
+        return out

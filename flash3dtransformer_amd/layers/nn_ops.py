@@ -1,0 +1,188 @@
+"""HIP-backed building blocks of the layer API: Linear, LayerNorm, LayerNormMLP and the fused
+norm + activation used around pooling.  Parameters are ordinary nn.Parameters (fp32 by default, so
+a checkpoint of the reference's torch / TransformerEngine modules loads by name); the kernels run on
+bf16 copies that are refreshed whenever a parameter changes.
+
+The library implements the forward pass only: every op is wrapped in an autograd.Function whose
+backward raises, so a training loop fails loudly instead of silently dropping gradients.
+"""
+import math
+
+import torch
+from torch import nn
+
+from ..lib import pshattn
+
+
+class _ForwardOnly(torch.autograd.Function):
+    """Marks the output of a forward-only kernel: asking for its gradient raises."""
+
+    @staticmethod
+    def forward(ctx, out, name, *deps):
+        ctx.name = name
+        return out.view_as(out)
+
+    @staticmethod
+    def backward(ctx, grad):
+        raise NotImplementedError(f"{ctx.name}: the gfx950 library implements the forward pass only")
+
+
+def forward_only(out: torch.Tensor, name: str, *deps) -> torch.Tensor:
+    if torch.is_grad_enabled() and any(isinstance(d, torch.Tensor) and d.requires_grad for d in deps):
+        return _ForwardOnly.apply(out, name, *deps)
+    return out
+
+
+class _Bf16Cache:
+    """bf16 device copy of a parameter, rebuilt when the parameter is modified or moved"""
+
+    def __init__(self):
+        self._key = None
+        self._val = None
+
+    def get(self, p: torch.Tensor) -> torch.Tensor:
+        if p is None:
+            return None
+        key = (p.data_ptr(), p._version, p.dtype, p.device)
+        if key != self._key:
+            self._val = p.detach().to(torch.bfloat16).contiguous()
+            self._key = key
+        return self._val
+
+
+def as_bf16_2d(x: torch.Tensor) -> torch.Tensor:
+    if x.dtype != torch.bfloat16:
+        x = x.to(torch.bfloat16)
+    if x.stride(-1) != 1:
+        x = x.contiguous()
+    return x
+
+
+class Linear(nn.Module):
+    """y = act(x W^T + b) (+ residual) on MFMA; parameter names match torch.nn.Linear / te.Linear"""
+
+    def __init__(self, in_features: int, out_features: int, bias: bool = True):
+        super().__init__()
+        self.in_features, self.out_features = in_features, out_features
+        self.weight = nn.Parameter(torch.empty(out_features, in_features))
+        self.bias = nn.Parameter(torch.empty(out_features)) if bias else None
+        self._w, self._b = _Bf16Cache(), _Bf16Cache()
+        self.reset_parameters()
+
+    def reset_parameters(self):
+        nn.init.kaiming_uniform_(self.weight, a=math.sqrt(5))
+        if self.bias is not None:
+            bound = 1.0 / math.sqrt(self.in_features)
+            nn.init.uniform_(self.bias, -bound, bound)
+
+    def forward(self, x: torch.Tensor, residual: torch.Tensor = None, act=None, out: torch.Tensor = None):
+        lead = x.shape[:-1]
+        x2 = as_bf16_2d(x.reshape(-1, x.shape[-1]))
+        n_out = self.out_features // 2 if act == "swiglu" else self.out_features
+        y = out if out is not None else torch.empty(x2.shape[0], n_out, dtype=torch.bfloat16, device=x.device)
+        r2 = None if residual is None else as_bf16_2d(residual.reshape(-1, n_out))
+        pshattn.linear_bf16(x2, self._w.get(self.weight), self._b.get(self.bias), r2, y, act)
+        return forward_only(y.view(*lead, n_out), "Linear", x, self.weight)
+
+    def extra_repr(self):
+        return f"in_features={self.in_features}, out_features={self.out_features}, bias={self.bias is not None}"
+
+
+class LayerNorm(nn.Module):
+    """LayerNorm over the last axis with fp32 statistics; parameter names match nn.LayerNorm / te.LayerNorm"""
+
+    def __init__(self, normalized_shape: int, eps: float = 1e-5):
+        super().__init__()
+        self.normalized_shape, self.eps = int(normalized_shape), eps
+        self.weight = nn.Parameter(torch.ones(self.normalized_shape))
+        self.bias = nn.Parameter(torch.zeros(self.normalized_shape))
+        self._w, self._b = _Bf16Cache(), _Bf16Cache()
+
+    def forward(self, x: torch.Tensor):
+        x2 = as_bf16_2d(x.reshape(-1, x.shape[-1])).contiguous()
+        y = torch.empty_like(x2)
+        pshattn.layernorm_bf16(x2, self._w.get(self.weight), self._b.get(self.bias), y, self.eps)
+        return forward_only(y.view(x.shape), "LayerNorm", x, self.weight)
+
+
+def apply_norm(norm: nn.Module, x: torch.Tensor) -> torch.Tensor:
+    """Runs a norm module the user passed as a callable: LayerNorm flavours go to the HIP kernel,
+    eval-mode BatchNorm1d folds into one affine kernel, anything else runs as given."""
+    if isinstance(norm, LayerNorm):
+        return norm(x)
+    if isinstance(norm, nn.LayerNorm) and norm.elementwise_affine and len(norm.normalized_shape) == 1 \
+            and x.is_cuda and x.shape[-1] % 8 == 0:
+        x2 = as_bf16_2d(x.reshape(-1, x.shape[-1])).contiguous()
+        y = torch.empty_like(x2)
+        b = None if norm.bias is None else norm.bias.detach().to(torch.bfloat16)
+        pshattn.layernorm_bf16(x2, norm.weight.detach().to(torch.bfloat16), b, y, norm.eps)
+        return forward_only(y.view(x.shape), "LayerNorm", x, norm.weight)
+    return norm(x)
+
+
+def _bn_affine(bn: nn.BatchNorm1d):
+    rstd = torch.rsqrt(bn.running_var.float() + bn.eps)
+    g = bn.weight.detach().float() if bn.affine else torch.ones_like(rstd)
+    b = bn.bias.detach().float() if bn.affine else torch.zeros_like(rstd)
+    return (g * rstd).contiguous(), (b - bn.running_mean.float() * g * rstd).contiguous()
+
+
+_ACT_NAMES = {nn.GELU: "gelu", nn.ReLU: "relu", nn.SiLU: "silu"}
+
+
+def apply_norm_act(norm, act, x: torch.Tensor) -> torch.Tensor:
+    """norm followed by activation as used around pooling / unpooling (hourglass.py:104-109, 152-159
+    of the reference).  Eval-mode BatchNorm1d + GELU/ReLU/SiLU is one fused kernel."""
+    act_name = None
+    if act is not None:
+        act_name = _ACT_NAMES.get(type(act))
+        if isinstance(act, nn.GELU) and act.approximate != "none":
+            act_name = None
+    fusable_act = act is None or act_name is not None
+    if isinstance(norm, nn.BatchNorm1d) and not norm.training and norm.track_running_stats and fusable_act \
+            and x.is_cuda and x.shape[-1] % 8 == 0:
+        scale, shift = _bn_affine(norm)
+        x2 = as_bf16_2d(x).contiguous()
+        y = torch.empty_like(x2)
+        pshattn.affine_act_bf16(x2, scale, shift, y, act_name)
+        return forward_only(y, "BatchNorm1d+act", x)
+    if norm is not None:
+        x = apply_norm(norm, x)
+    if act is not None:
+        x = act(x)
+    return x
+
+
+class LayerNormMLP(nn.Module):
+    """LayerNorm -> fc1 -> activation -> fc2, the role te.LayerNormMLP plays in the reference
+    (flash3dxfmr/layers/elem_wise.py:22-26).  Parameter names follow TransformerEngine
+    (layer_norm_weight/bias, fc1_weight/bias, fc2_weight/bias).  activation "swiglu": fc1 has
+    2 * ffn_hidden_size outputs and the hidden state is silu(h[:, :ffn]) * h[:, ffn:]; "gelu": plain
+    fc1 -> GELU -> fc2."""
+
+    def __init__(self, hidden_size: int, ffn_hidden_size: int, activation: str = "swiglu", eps: float = 1e-5):
+        super().__init__()
+        assert activation in ("swiglu", "gelu")
+        self.hidden_size, self.ffn_hidden_size, self.activation, self.eps = hidden_size, ffn_hidden_size, activation, eps
+        fc1_out = 2 * ffn_hidden_size if activation == "swiglu" else ffn_hidden_size
+        self.layer_norm_weight = nn.Parameter(torch.ones(hidden_size))
+        self.layer_norm_bias = nn.Parameter(torch.zeros(hidden_size))
+        self.fc1_weight = nn.Parameter(torch.empty(fc1_out, hidden_size))
+        self.fc1_bias = nn.Parameter(torch.zeros(fc1_out))
+        self.fc2_weight = nn.Parameter(torch.empty(hidden_size, ffn_hidden_size))
+        self.fc2_bias = nn.Parameter(torch.zeros(hidden_size))
+        nn.init.normal_(self.fc1_weight, std=0.023)
+        nn.init.normal_(self.fc2_weight, std=0.023)
+        self._c = [_Bf16Cache() for _ in range(6)]
+
+    def forward(self, x: torch.Tensor, residual: torch.Tensor = None):
+        x2 = as_bf16_2d(x.reshape(-1, self.hidden_size)).contiguous()
+        c = self._c
+        ln = torch.empty_like(x2)
+        pshattn.layernorm_bf16(x2, c[0].get(self.layer_norm_weight), c[1].get(self.layer_norm_bias), ln, self.eps)
+        h = torch.empty(x2.shape[0], self.ffn_hidden_size, dtype=torch.bfloat16, device=x.device)
+        pshattn.linear_bf16(ln, c[2].get(self.fc1_weight), c[3].get(self.fc1_bias), None, h, self.activation)
+        y = torch.empty_like(x2)
+        r2 = None if residual is None else as_bf16_2d(residual.reshape(-1, self.hidden_size))
+        pshattn.linear_bf16(h, c[4].get(self.fc2_weight), c[5].get(self.fc2_bias), r2, y, None)
+        return forward_only(y.view(x.shape), "LayerNormMLP", x, self.fc1_weight)
