@@ -1,0 +1,274 @@
+#!/usr/bin/env python3
+"""Benchmark of the Flash3D forward hot path on one MI355X.
+
+A step = one encoder-stage forward on 4 synthetic LiDAR sweeps x 120,000 points (BASELINE config
+"encoder stage"): PSH bucketing (bbox + hash + claim + scatter) -> coordinate embedding ->
+LayerNorm -> QKV GEMM -> bucketed attention -> out-projection + residual -> LayerNorm + MLP
+(256 -> 1024 -> 256) + residual.  C = 256, 8 heads x 32, bucket 512, scope of 1 bucket, hash 2.
+
+Prints ONE JSON line: whole-job throughput in Mpts/s, the roofline of the dominant kernel measured
+live with stream events, per-op sub-metrics (attention TFLOP/s on config 2, PSH / pooling GB/s), and
+a CPU baseline (the oracle pipeline on a bounded sample, host cores stated).
+"""
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+import numpy as np
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+MFMA_BF16_PEAK_TFLOPS = 2500.0
+
+
+def ev_time(fn, iters, warmup=3):
+    """average milliseconds of fn() over `iters` launches, timed with events on the current stream"""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record()
+    for _ in range(iters):
+        fn()
+    b.record()
+    torch.cuda.synchronize()
+    return a.elapsed_time(b) / iters
+
+
+def make_block(C, hid, H, bs, scope, activation, seed):
+    from flash3dtransformer_amd import layers as L
+    from flash3dtransformer_amd.psh.bucket_scope import SwinPlan
+    torch.manual_seed(seed)
+    emb = L.PSH3DCoordEmbedding(C, bs, bs * scope * 6)
+    blk = L.XFMR(C, hid, H, bs, True, SwinPlan("swin", bs, scope, 0), lambda ch: L.LayerNorm(ch), activation)
+    g = torch.Generator().manual_seed(seed)
+    for m in list(emb.modules()) + list(blk.modules()):
+        for name, p in m.named_parameters(recurse=False):
+            if p.dim() == 2:   # Xavier-uniform, bf16-rounded
+                bound = math.sqrt(6.0 / (p.shape[0] + p.shape[1]))
+                p.data = ((torch.rand(p.shape, generator=g) * 2 - 1) * bound).to(torch.bfloat16).float()
+    return emb.to("cuda:0"), blk.to("cuda:0")
+
+
+def cpu_baseline(clouds, emb, blk, C, H, bs, scope, hash_op, activation):
+    """the oracle pipeline on the first sweep only, all host cores for the torch part"""
+    from oracle import f3d_oracle as orc
+    from flash3dtransformer_amd import synth
+    cores = os.cpu_count() or 1
+    torch.set_num_threads(cores)
+    coords, seps = synth.batch_of(clouds[:1])
+    n = coords.shape[0]
+    align = bs * scope * 6
+    pad_to = -(-n // align) * align
+    f = lambda p: p.detach().float().cpu().to(torch.bfloat16).float()
+    w = {"norm.weight": f(blk.norm.weight), "norm.bias": f(blk.norm.bias), "qkv.weight": f(blk.bwa.qkv.weight),
+         "qkv.bias": f(blk.bwa.qkv.bias), "proj.weight": f(blk.bwa.proj.weight), "proj.bias": f(blk.bwa.proj.bias),
+         "ln.weight": f(blk.mlp.mlp.layer_norm_weight), "ln.bias": f(blk.mlp.mlp.layer_norm_bias),
+         "fc1.weight": f(blk.mlp.mlp.fc1_weight), "fc1.bias": f(blk.mlp.mlp.fc1_bias),
+         "fc2.weight": f(blk.mlp.mlp.fc2_weight), "fc2.bias": f(blk.mlp.mlp.fc2_bias)}
+    ew, eb = f(emb.lin.weight), f(emb.lin.bias)
+    t0 = time.perf_counter()
+    scat = orc.psh_scatter_coords(coords, seps, bs, pad_to, hash_op)
+    x = orc._r(orc.linear(torch.from_numpy(scat.astype(np.float32)).to(torch.bfloat16), ew, eb))
+    scopes = orc.gen_scopes(pad_to, bs, scope)
+    out = orc.xfmr_block(x, w, scopes, bs, H, activation)
+    dt = time.perf_counter() - t0
+    return {"value": n / dt / 1e6, "unit": "Mpts/s", "cores": cores, "kind": "port",
+            "sample": f"first of 4 sweeps ({n} points), one pass of the same stage through the oracle "
+                      f"(C PSH single-threaded + torch fp32 on {cores} threads), {dt:.2f} s"}, out
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--mlp", default="swiglu", choices=["swiglu", "gelu"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-sub-metrics", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU; the path shards by cloud without any exchange "
+              "(see DESIGN.md), and no multi-GPU figure is produced. Re-run with --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+
+    from flash3dtransformer_amd import synth
+    from flash3dtransformer_amd.lib import pshattn
+    from flash3dtransformer_amd.psh import psh_main
+    dev = "cuda:0"
+    C, HID, H, BS, SCOPE, HASH = 256, 1024, 8, 512, 1, 2
+    clouds = [synth.lidar_sweep(120_000, 1004 + i) for i in range(4)]
+    coords_np, seps_np = synth.batch_of(clouds)
+    coords = torch.from_numpy(coords_np).to(dev)
+    seps = torch.from_numpy(seps_np.view(np.int32)).to(dev).view(torch.uint32)
+    n_pts = coords.shape[0]
+    emb, blk = make_block(C, HID, H, BS, SCOPE, args.mlp, 1004)
+
+    @torch.no_grad()
+    def step():
+        feat = emb(coords, seps, HASH)
+        return blk(None, feat, None)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        out = step()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    ms_per_step = dt / args.steps * 1e3
+    value = n_pts / (dt / args.steps) / 1e6
+
+    # ---- per-op breakdown on the same tensors, events on the launch stream ----
+    with torch.no_grad():
+        feat = emb(coords, seps, HASH)
+        n_pad = feat.shape[0]
+        mlp = blk.mlp.mlp
+        scopes = blk.swin_plan.gen_scopes_from_plan(n_pad, feat.device)
+        ln_out, qkv = torch.empty_like(feat), torch.empty(n_pad, 3 * C, dtype=torch.bfloat16, device=dev)
+        o = torch.empty(1, n_pad, H, C // H, dtype=torch.bfloat16, device=dev)
+        lse = torch.zeros(1, n_pad, H, dtype=torch.float32, device=dev)
+        mid, hid, y = torch.empty_like(feat), torch.empty(n_pad, HID, dtype=torch.bfloat16, device=dev), torch.empty_like(feat)
+        bw = lambda p: p.detach().to(torch.bfloat16).contiguous()
+        Wn, Bn, Wq, Bq, Wp, Bp = bw(blk.norm.weight), bw(blk.norm.bias), bw(blk.bwa.qkv.weight), bw(blk.bwa.qkv.bias), bw(blk.bwa.proj.weight), bw(blk.bwa.proj.bias)
+        W1, B1, W2, B2 = bw(mlp.fc1_weight), bw(mlp.fc1_bias), bw(mlp.fc2_weight), bw(mlp.fc2_bias)
+        q, k, v = (t.view(1, n_pad, H, C // H) for t in qkv.chunk(3, dim=-1))
+        ops = {
+            "psh_scatter": lambda: psh_main.batch_bucket_scatter(coords, seps, BS, n_pad, HASH),
+            "layernorm": lambda: pshattn.layernorm_bf16(feat, Wn, Bn, ln_out, 1e-5),
+            "qkv_gemm": lambda: pshattn.linear_bf16(ln_out, Wq, Bq, None, qkv, None),
+            "attention": lambda: pshattn.buck_swin_fwd(q, k, v, o, lse, scopes, BS),
+            "proj_gemm": lambda: pshattn.linear_bf16(o.view(n_pad, C), Wp, Bp, feat, mid, None),
+            "fc1_gemm": lambda: pshattn.linear_bf16(ln_out, W1, B1, None, hid, args.mlp),
+            "fc2_gemm": lambda: pshattn.linear_bf16(hid, W2, B2, mid, y, None),
+        }
+        breakdown = {name: ev_time(fn, 20) for name, fn in ops.items()}
+    fc1_n = 2 * HID if args.mlp == "swiglu" else HID
+    flops = {"qkv_gemm": 2.0 * n_pad * C * 3 * C, "proj_gemm": 2.0 * n_pad * C * C,
+             "fc1_gemm": 2.0 * n_pad * C * fc1_n, "fc2_gemm": 2.0 * n_pad * HID * C,
+             "attention": 4.0 * n_pad * BS * SCOPE * C}
+    dominant = max(("attention", "qkv_gemm", "proj_gemm", "fc1_gemm", "fc2_gemm"), key=lambda kname: breakdown[kname])
+    ach = flops[dominant] / (breakdown[dominant] * 1e-3) / 1e12
+    roofline = {"kernel": {"attention": "buck_swin_fwd_kernel<32,128>"}.get(dominant, "gemm_bf16_kernel"),
+                "op": dominant, "bound": "mfma", "achieved": round(ach, 2), "peak": MFMA_BF16_PEAK_TFLOPS,
+                "unit": "TFLOP/s", "frac": round(ach / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None,
+                "avg_launch_ms": round(breakdown[dominant], 4), "algorithmic_flop_per_launch": flops[dominant]}
+
+    sub = {}
+    if not args.no_sub_metrics:
+        sub = sub_metrics(dev)
+
+    result = {
+        "metric": "Flash3D encoder-stage forward throughput @ 4x120k-point LiDAR sweeps",
+        "value": round(value, 3), "unit": "Mpts/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "encoder stage fwd: PSH -> embed -> LN -> QKV -> bucketed attention -> proj -> MLP "
+                               f"({args.mlp}) on 4 synthetic LiDAR sweeps x 120k points",
+                   "points": n_pts, "padded_rows": int(n_pad), "channels": C, "heads": H, "head_dim": C // H,
+                   "mlp_hidden": HID, "bucket_size": BS, "scope_size": SCOPE, "hash_type": HASH},
+        "roofline": roofline,
+        "breakdown_ms": {kname: round(vv, 4) for kname, vv in breakdown.items()},
+        "sub_metrics": sub,
+    }
+    if not args.no_cpu_baseline:
+        cb, ref_out = cpu_baseline(clouds, emb, blk, C, H, BS, SCOPE, HASH, args.mlp)
+        result["cpu_baseline"] = cb
+    print(json.dumps(result))
+
+
+def sub_metrics(dev):
+    """attention TFLOP/s on config 2, PSH GB/s (config 1 latency + saturating size), pooling and
+    unpooling GB/s on config 3 — each against its roofline"""
+    from flash3dtransformer_amd.lib import pshattn
+    from flash3dtransformer_amd.psh import psh_main, subbuck
+    out = {}
+    # ---- attention, config 2: L = 131,072, H = 8, D = 32, bucket 512, scope 1 ----
+    L, H, D, BS = 131072, 8, 32, 512
+    g = torch.Generator().manual_seed(1002)
+    qkv = (torch.randn(1, L, 3 * H * D, generator=g) / math.sqrt(32)).to(torch.bfloat16).to(dev)
+    q, k, v = [t.view(1, L, H, D) for t in qkv.chunk(3, dim=-1)]
+    o = torch.empty(1, L, H, D, dtype=torch.bfloat16, device=dev)
+    lse = torch.zeros(1, L, H, dtype=torch.float32, device=dev)
+    sc = torch.arange(L // BS, dtype=torch.int32, device=dev).view(-1, 1).view(torch.uint32)
+    ms = ev_time(lambda: pshattn.buck_swin_fwd(q, k, v, o, lse, sc, BS), 30)
+    fl = 4.0 * L * BS * H * D
+    out["attention_c2_unmasked"] = {"ms": round(ms, 4), "tflops": round(fl / ms / 1e9, 2),
+                                    "frac_of_bf16_mfma_peak": round(fl / ms / 1e9 / MFMA_BF16_PEAK_TFLOPS, 4),
+                                    "algorithmic_gflop": round(fl / 1e9, 2)}
+    kl = torch.from_numpy(np.random.default_rng(1002).integers(384, 513, L // BS).astype(np.int32)).to(dev)
+    ms = ev_time(lambda: pshattn.buck_swin_fwd(q, k, v, o, lse, sc, BS, kl), 30)
+    flm = 4.0 * float((kl.double() ** 2).sum()) * H * D
+    out["attention_c2_masked"] = {"ms": round(ms, 4), "tflops": round(flm / ms / 1e9, 2),
+                                  "algorithmic_gflop": round(flm / 1e9, 2)}
+    del qkv, q, k, v, o, lse
+    # ---- PSH: config 1 (latency bound) and a saturating batch, 30 B/pt three-kernel accounting ----
+    for name, n_c, b in (("psh_c1_32768", 32768, 1), ("psh_saturating_64x262144", 262144, 64)):
+        gg = torch.Generator().manual_seed(1001)
+        coords = (torch.rand(n_c * b, 3, generator=gg) * 51.2).to(torch.float16).to(dev)
+        seps = (torch.arange(1, b + 1, dtype=torch.int32) * n_c).to(dev).view(torch.uint32)
+        nb, div, mx = psh_main.bucket_geometry(seps, 512)
+        buf = psh_main.BucketScatterBuffers.create_buffers(coords, seps, 512, n_c * b, nb)
+        bb = torch.stack([coords.min(0)[0], coords.max(0)[0]])
+
+        def run():
+            buf.bucket_cntr.zero_()
+            pshattn.batch_psh_scatter_pad_hash(coords, buf.bucket_id, buf.bucket_cntr, buf.bucket_offs, seps, mx, nb,
+                                               div, 512, 0xFFFF, bb[0], bb[1], buf.probe_offs, buf.bucket_cumsum,
+                                               buf.scattered_coord, 0.0, 1)
+        ms = ev_time(run, 30)
+        byts = 26.0 * n_c * b      # K1: 6 B read + 2 B write; K3: 8 B read + 10 B write
+        out[name] = {"ms": round(ms, 4), "gbs_26B_per_pt": round(byts / ms / 1e6, 1),
+                     "frac_of_hbm_peak": round(byts / ms / 1e6 / HBM_PEAK_GBS, 4),
+                     "mpts_per_s": round(n_c * b / ms / 1e3, 1)}
+        del coords, buf
+    # ---- pooling / unpooling, config 3: 262,144 points x 128 channels, S = 8 ----
+    n, C, S = 262144, 128, 8
+    gg = torch.Generator().manual_seed(1003)
+    coords = (torch.rand(n, 3, generator=gg) * 51.2).to(torch.float16).to(dev)
+    seps = (torch.arange(1, 5, dtype=torch.int32) * (n // 4)).to(dev).view(torch.uint32)
+    feat = torch.randn(n, C, generator=gg).to(torch.bfloat16).to(dev)
+    res = torch.randn(n, C, generator=gg).to(torch.bfloat16).to(dev)
+    sb = subbuck.SubbuckBuffers.create_subbuck_buff(coords, feat, seps, S)
+    L_ = pshattn._load()
+    import ctypes
+    u32, vp, ci = ctypes.c_uint32, ctypes.c_void_p, ctypes.c_int
+    st = vp(torch.cuda.current_stream(0).cuda_stream)
+
+    def build():
+        L_.f3d_subbuck_build(vp(coords.data_ptr()), vp(seps.data_ptr()), u32(4), u32(n), u32(n // 4), u32(S),
+                             u32(0xFFFF), vp(sb.subbuck_id.data_ptr()), vp(sb.subbuck_off.data_ptr()),
+                             vp(sb.reduced_sep.data_ptr()), vp(sb.reduced_coord.data_ptr()),
+                             u32(sb.reduced_coord.shape[0]), vp(sb.unpool_ind.data_ptr()),
+                             u32(sb.unpool_ind.shape[0]), ci(0), st)
+
+    def reduce(op):
+        L_.f3d_reduce_feat(vp(feat.data_ptr()), u32(n), u32(C), vp(sb.unpool_ind.data_ptr()),
+                           u32(sb.unpool_ind.shape[0]), u32(S), u32(op), vp(sb.reduced_feat.data_ptr()),
+                           u32(sb.reduced_feat.shape[0]), ci(0), st)
+    up = torch.empty_like(res)
+    ms_b = ev_time(build, 30)
+    ms_mean = ev_time(lambda: reduce(0), 30)
+    ms_max = ev_time(lambda: reduce(3), 30)
+    ms_up = ev_time(lambda: pshattn.additive_unpool_fwd(res, sb.reduced_feat, up, sb.unpool_ind, S), 30)
+    r = n // S
+    red_bytes = n * C * 2 + r * S * 4 + r * C * 2
+    up_bytes = n * C * 2 + r * C * 2 + r * S * 4 + n * C * 2
+    bld_bytes = n * 6 + n * 4 + n * 2 + r * S * 4 + r * 6
+    gb = lambda b_, ms_: round(b_ / ms_ / 1e6, 1)
+    out["pool_c3_builder"] = {"ms": round(ms_b, 4), "gbs": gb(bld_bytes, ms_b), "frac_of_hbm_peak": round(gb(bld_bytes, ms_b) / HBM_PEAK_GBS, 4)}
+    out["pool_c3_reduce_mean"] = {"ms": round(ms_mean, 4), "gbs": gb(red_bytes, ms_mean), "frac_of_hbm_peak": round(gb(red_bytes, ms_mean) / HBM_PEAK_GBS, 4)}
+    out["pool_c3_reduce_max"] = {"ms": round(ms_max, 4), "gbs": gb(red_bytes, ms_max), "frac_of_hbm_peak": round(gb(red_bytes, ms_max) / HBM_PEAK_GBS, 4)}
+    out["unpool_c3"] = {"ms": round(ms_up, 4), "gbs": gb(up_bytes, ms_up), "frac_of_hbm_peak": round(gb(up_bytes, ms_up) / HBM_PEAK_GBS, 4)}
+    return out
+
+
+if __name__ == "__main__":
+    main()

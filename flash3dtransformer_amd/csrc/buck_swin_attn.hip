@@ -22,21 +22,9 @@ namespace f3d {
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16_t;
 
-struct alignas(16) U16x8 {
-  uint16_t v[8];
-};
-
 constexpr int kAttnThreads = 256;
 constexpr int kQBlock = 128;  // query rows per workgroup
 constexpr int kNumXcd = 8;
-
-__device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
-  // round-to-nearest-even of two finite, non-negative probabilities
-  uint32_t ua = __builtin_bit_cast(uint32_t, a), ub = __builtin_bit_cast(uint32_t, b);
-  ua += 0x7FFFu + ((ua >> 16) & 1u);
-  ub += 0x7FFFu + ((ub >> 16) & 1u);
-  return (ua >> 16) | (ub & 0xFFFF0000u);
-}
 
 // position of key (kk = key % 16) inside its group of 16 in the transposed V tile:
 // storage order 0..3, 8..11, 4..7, 12..15
@@ -120,7 +108,7 @@ __global__ __launch_bounds__(kAttnThreads) void buck_swin_fwd_kernel(
     return false;
   };
 
-  U16x8 rk[C::NCH], rv[C::NCH];
+  u32x4_t rk[C::NCH], rv[C::NCH];
   auto fetch = [&](uint32_t j, uint32_t t) {
     const size_t row0 = tok0 + (size_t)my_scope[j] * bs + t * KT;
 #pragma unroll
@@ -129,8 +117,8 @@ __global__ __launch_bounds__(kAttnThreads) void buck_swin_fwd_kernel(
       if (C::CHUNKS % kAttnThreads == 0 || c < (uint32_t)C::CHUNKS) {
         const uint32_t key = c / (D / 8), dc = c % (D / 8);
         const size_t off = (row0 + key) * ld + head * D + dc * 8;
-        rk[i] = *reinterpret_cast<const U16x8*>(k + off);
-        rv[i] = *reinterpret_cast<const U16x8*>(v + off);
+        rk[i] = *reinterpret_cast<const u32x4_t*>(k + off);
+        rv[i] = *reinterpret_cast<const u32x4_t*>(v + off);
       }
     }
   };
@@ -140,10 +128,14 @@ __global__ __launch_bounds__(kAttnThreads) void buck_swin_fwd_kernel(
       const uint32_t c = tid + i * kAttnThreads;
       if (C::CHUNKS % kAttnThreads == 0 || c < (uint32_t)C::CHUNKS) {
         const uint32_t key = c / (D / 8), dc = c % (D / 8);
-        *reinterpret_cast<U16x8*>(sK + key * C::KROW + dc * 8) = rk[i];
+        *reinterpret_cast<u32x4_t*>(sK + key * C::KROW + dc * 8) = rk[i];
         const uint32_t pos = (key & ~15u) | vperm16(key & 15u);
+        uint16_t* col = sVt + (dc * 8) * C::VROW + pos;
 #pragma unroll
-        for (int e = 0; e < 8; ++e) sVt[(dc * 8 + e) * C::VROW + pos] = rv[i].v[e];
+        for (int e = 0; e < 4; ++e) {
+          col[(2 * e) * C::VROW] = (uint16_t)(rv[i][e] & 0xFFFFu);
+          col[(2 * e + 1) * C::VROW] = (uint16_t)(rv[i][e] >> 16);
+        }
       }
     }
   };
@@ -206,16 +198,19 @@ __global__ __launch_bounds__(kAttnThreads) void buck_swin_fwd_kernel(
       pb[i / 2] = pack_bf16x2(p0, p1);
     }
     l_run = l_run * alpha + psum;
+    // the running maximum settles after the first tiles: rescale the accumulators only when some
+    // query of this wave actually moved (wave-uniform branch)
+    if (__ballot(alpha != 1.0f)) {
 #pragma unroll
-    for (int dt = 0; dt < C::DT; ++dt)
+      for (int dt = 0; dt < C::DT; ++dt)
 #pragma unroll
-      for (int i = 0; i < 16; ++i) acc[dt][i] *= alpha;
+        for (int i = 0; i < 16; ++i) acc[dt][i] *= alpha;
+    }
     // ---- Ot += Vt Pt ----
 #pragma unroll
     for (int j = 0; j < C::NSUB; ++j)
 #pragma unroll
       for (int kk = 0; kk < 2; ++kk) {
-        typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t u32x4_t;
         u32x4_t praw = {pb[j * 8 + kk * 4 + 0], pb[j * 8 + kk * 4 + 1], pb[j * 8 + kk * 4 + 2], pb[j * 8 + kk * 4 + 3]};
         const bf16x8_t pf = __builtin_bit_cast(bf16x8_t, praw);
 #pragma unroll
@@ -244,10 +239,8 @@ __global__ __launch_bounds__(kAttnThreads) void buck_swin_fwd_kernel(
       const uint32_t d0 = dt * 32 + g * 8 + half * 4;
       if (D >= 32 || d0 < (uint32_t)D) {
         uint2 w;
-        w.x = (uint32_t)float_to_bf16_bits(acc[dt][g * 4 + 0] * inv) |
-              ((uint32_t)float_to_bf16_bits(acc[dt][g * 4 + 1] * inv) << 16);
-        w.y = (uint32_t)float_to_bf16_bits(acc[dt][g * 4 + 2] * inv) |
-              ((uint32_t)float_to_bf16_bits(acc[dt][g * 4 + 3] * inv) << 16);
+        w.x = pack_bf16x2(acc[dt][g * 4 + 0] * inv, acc[dt][g * 4 + 1] * inv);
+        w.y = pack_bf16x2(acc[dt][g * 4 + 2] * inv, acc[dt][g * 4 + 3] * inv);
         *reinterpret_cast<uint2*>(op + d0) = w;
       }
     }
@@ -308,7 +301,7 @@ int f3d_buck_swin_fwd_strided(const f3d_bf16_t* q, const f3d_bf16_t* k, const f3
                            seq_len, num_head, kv_len, s)
   switch (head_dim) {
     case 16: F3D_ATTN(16, 128); break;
-    case 32: F3D_ATTN(32, 128); break;
+    case 32: F3D_ATTN(32, 64); break;
     case 64: F3D_ATTN(64, 64); break;
     default: F3D_ATTN(128, 64); break;
   }

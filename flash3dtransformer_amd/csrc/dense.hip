@@ -86,26 +86,28 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_kernel(
       for (int i = 0; i < 16; ++i) acc[a][b][i] = 0.f;
 
   // each thread moves 4 x-chunks and 4 w-chunks (16 bytes each) per K step
-  U16x8 rx[4], rw[4];
+  u32x4_t rx[4], rw[4];
   auto fetch = [&](uint32_t k0) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const uint32_t c = tid + i * kGemmThreads;
       const uint32_t row = c >> 3, kc = (c & 7u) * 8;
       const bool kin = k0 + kc < K;
-      U16x8 z;
-#pragma unroll
-      for (int e = 0; e < 8; ++e) z.v[e] = 0;
-      rx[i] = (kin && m0 + row < M) ? *reinterpret_cast<const U16x8*>(x + (size_t)(m0 + row) * ldx + k0 + kc) : z;
+      const u32x4_t z = {0u, 0u, 0u, 0u};
+      rx[i] = (kin && m0 + row < M) ? *reinterpret_cast<const u32x4_t*>(x + (size_t)(m0 + row) * ldx + k0 + kc) : z;
       if (!B_TRANS) {
-        rw[i] = (kin && wrow_ok(row)) ? *reinterpret_cast<const U16x8*>(w + (size_t)wrow(row) * ldw + k0 + kc) : z;
+        rw[i] = (kin && wrow_ok(row)) ? *reinterpret_cast<const u32x4_t*>(w + (size_t)wrow(row) * ldw + k0 + kc) : z;
       } else {
         // b[K][N]: gather 8 k-values of column n0+row (only the demo op uses this path)
-        U16x8 t = z;
+        u32x4_t t = z;
         if (n0 + row < N) {
 #pragma unroll
-          for (int e = 0; e < 8; ++e)
-            if (k0 + kc + e < K) t.v[e] = w[(size_t)(k0 + kc + e) * ldw + n0 + row];
+          for (int e = 0; e < 4; ++e) {
+            const uint32_t ka = k0 + kc + 2 * e;
+            const uint32_t lo = ka < K ? w[(size_t)ka * ldw + n0 + row] : 0u;
+            const uint32_t hi = ka + 1 < K ? w[(size_t)(ka + 1) * ldw + n0 + row] : 0u;
+            t[e] = lo | (hi << 16);
+          }
         }
         rw[i] = t;
       }
@@ -116,8 +118,8 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_kernel(
     for (int i = 0; i < 4; ++i) {
       const uint32_t c = tid + i * kGemmThreads;
       const uint32_t row = c >> 3, kc = (c & 7u) * 8;
-      *reinterpret_cast<U16x8*>(sX + row * LDK + kc) = rx[i];
-      *reinterpret_cast<U16x8*>(sW + row * LDK + kc) = rw[i];
+      *reinterpret_cast<u32x4_t*>(sX + row * LDK + kc) = rx[i];
+      *reinterpret_cast<u32x4_t*>(sW + row * LDK + kc) = rw[i];
     }
   };
 
@@ -154,10 +156,8 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_kernel(
         const uint32_t col = wn * 64 + a * 32 + g * 8 + half * 4;
         const uint32_t row = wm * 64 + b * 32 + lq;
         uint2 pk;
-        pk.x = (uint32_t)float_to_bf16_bits(acc[a][b][g * 4 + 0] + s_bias[col + 0]) |
-               ((uint32_t)float_to_bf16_bits(acc[a][b][g * 4 + 1] + s_bias[col + 1]) << 16);
-        pk.y = (uint32_t)float_to_bf16_bits(acc[a][b][g * 4 + 2] + s_bias[col + 2]) |
-               ((uint32_t)float_to_bf16_bits(acc[a][b][g * 4 + 3] + s_bias[col + 3]) << 16);
+        pk.x = pack_bf16x2(acc[a][b][g * 4 + 0] + s_bias[col + 0], acc[a][b][g * 4 + 1] + s_bias[col + 1]);
+        pk.y = pack_bf16x2(acc[a][b][g * 4 + 2] + s_bias[col + 2], acc[a][b][g * 4 + 3] + s_bias[col + 3]);
         *reinterpret_cast<uint2*>(sC + row * LDC + col) = pk;
       }
   __syncthreads();
@@ -169,19 +169,22 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_kernel(
       const uint32_t c = tid + i * kGemmThreads;
       const uint32_t row = c >> 4, cc = (c & 15u) * 8;
       if (m0 + row >= M || n0 + cc >= N) continue;
-      U16x8 t = *reinterpret_cast<const U16x8*>(sC + row * LDC + cc);
+      u32x4_t t = *reinterpret_cast<const u32x4_t*>(sC + row * LDC + cc);
       if (act != F3D_ACT_NONE || residual) {
-        U16x8 r;
-        if (residual) r = *reinterpret_cast<const U16x8*>(residual + (size_t)(m0 + row) * ldr + n0 + cc);
+        u32x4_t r = {0u, 0u, 0u, 0u};
+        if (residual) r = *reinterpret_cast<const u32x4_t*>(residual + (size_t)(m0 + row) * ldr + n0 + cc);
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          float f = bf16_bits_to_float(t.v[e]);
-          if (act != F3D_ACT_NONE) f = bf16_bits_to_float(float_to_bf16_bits(apply_act(f, act)));
-          if (residual) f += bf16_bits_to_float(r.v[e]);
-          t.v[e] = float_to_bf16_bits(f);
+        for (int e = 0; e < 4; ++e) {
+          float f0 = bf16_lo(t[e]), f1 = bf16_hi(t[e]);
+          if (act != F3D_ACT_NONE) {
+            const uint32_t a2 = pack_bf16x2(apply_act(f0, act), apply_act(f1, act));  // activation output is bf16
+            f0 = bf16_lo(a2); f1 = bf16_hi(a2);
+          }
+          if (residual) { f0 += bf16_lo(r[e]); f1 += bf16_hi(r[e]); }
+          t[e] = pack_bf16x2(f0, f1);
         }
       }
-      *reinterpret_cast<U16x8*>(y + (size_t)(m0 + row) * ldy + n0 + cc) = t;
+      *reinterpret_cast<u32x4_t*>(y + (size_t)(m0 + row) * ldy + n0 + cc) = t;
     }
   } else {
     // out[:, n0 + j] = silu(value_j) * gate_j, 64 output columns per tile
@@ -190,18 +193,23 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_kernel(
       const uint32_t c = tid + i * kGemmThreads;
       const uint32_t row = c >> 3, cc = (c & 7u) * 8;
       if (m0 + row >= M || n0 + cc >= half_n) continue;
-      const U16x8 a = *reinterpret_cast<const U16x8*>(sC + row * LDC + cc);
-      const U16x8 gt = *reinterpret_cast<const U16x8*>(sC + row * LDC + BN / 2 + cc);
-      U16x8 r, t;
-      if (residual) r = *reinterpret_cast<const U16x8*>(residual + (size_t)(m0 + row) * ldr + n0 + cc);
+      const u32x4_t a = *reinterpret_cast<const u32x4_t*>(sC + row * LDC + cc);
+      const u32x4_t gt = *reinterpret_cast<const u32x4_t*>(sC + row * LDC + BN / 2 + cc);
+      u32x4_t r = {0u, 0u, 0u, 0u}, t;
+      if (residual) r = *reinterpret_cast<const u32x4_t*>(residual + (size_t)(m0 + row) * ldr + n0 + cc);
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        const float av = bf16_bits_to_float(a.v[e]);
-        float f = (av / (1.0f + __expf(-av))) * bf16_bits_to_float(gt.v[e]);
-        if (residual) f = bf16_bits_to_float(float_to_bf16_bits(f)) + bf16_bits_to_float(r.v[e]);
-        t.v[e] = float_to_bf16_bits(f);
+      for (int e = 0; e < 4; ++e) {
+        const float a0 = bf16_lo(a[e]), a1 = bf16_hi(a[e]);
+        float f0 = (a0 / (1.0f + __expf(-a0))) * bf16_lo(gt[e]);
+        float f1 = (a1 / (1.0f + __expf(-a1))) * bf16_hi(gt[e]);
+        if (residual) {
+          const uint32_t h2 = pack_bf16x2(f0, f1);
+          f0 = bf16_lo(h2) + bf16_lo(r[e]);
+          f1 = bf16_hi(h2) + bf16_hi(r[e]);
+        }
+        t[e] = pack_bf16x2(f0, f1);
       }
-      *reinterpret_cast<U16x8*>(y + (size_t)(m0 + row) * ldy + n0 + cc) = t;
+      *reinterpret_cast<u32x4_t*>(y + (size_t)(m0 + row) * ldy + n0 + cc) = t;
     }
   }
 }

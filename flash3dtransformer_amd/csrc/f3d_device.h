@@ -23,13 +23,23 @@ __device__ __forceinline__ float bf16_bits_to_float(uint16_t b) {
   return __builtin_bit_cast(float, (uint32_t)b << 16);
 }
 
-// round to nearest even; NaN stays NaN
+// round to nearest even (v_cvt_pk_bf16_f32)
 __device__ __forceinline__ uint16_t float_to_bf16_bits(float f) {
-  uint32_t u = __builtin_bit_cast(uint32_t, f);
-  if ((u & 0x7FFFFFFFu) > 0x7F800000u) return (uint16_t)((u >> 16) | 0x40u);
-  u += 0x7FFFu + ((u >> 16) & 1u);
-  return (uint16_t)(u >> 16);
+  return __builtin_bit_cast(uint16_t, (__bf16)f);
 }
+
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));  // one 16-byte chunk = 8 bf16 / fp16 values
+
+// two fp32 -> packed bf16 pair (low half = a), one instruction
+__device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
+  f32x2_t v = {a, b};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
+}
+
+__device__ __forceinline__ float bf16_lo(uint32_t w) { return __builtin_bit_cast(float, w << 16); }
+__device__ __forceinline__ float bf16_hi(uint32_t w) { return __builtin_bit_cast(float, w & 0xFFFF0000u); }
 
 // ---- voxel quantiser (reference: src/psh/hash_fns.cuh:23-33) ----------------------------------
 // q = ((c - min) * num_vox) * inv with inv = 1 / (max - min) rounded once; floor; clamp to

@@ -1,0 +1,55 @@
+"""In-bucket pooling layer (reference: flash3dxfmr/layers/pooling.py)."""
+import torch
+from torch import nn
+from torch.autograd import Function
+
+from ..lib import pshattn
+from ..psh import batching as f3dbatch
+from ..psh import subbuck as f3dsubbuck
+
+NUM_VOX = 0xFFFF
+
+
+class SubbuckReduceFunction(Function):
+    """(coords, feat, seps) -> (reduced_feat, SubbuckBuffers): groups of `subbuck_size` spatially
+    close points of every cloud are reduced to one row (0 mean, 1 sum, 2 min, 3 max).  The buffers
+    carry reduced_coord, reduced_sep and unpool_ind for the next level and for unpooling."""
+
+    @staticmethod
+    def forward(ctx, coords, input_feat, seps, subbuck_size, reduction_op, out_alignment=1):
+        max_n = f3dbatch.max_inslen_from_seps(seps)
+        sb = f3dsubbuck.SubbuckBuffers.create_subbuck_buff(coords, input_feat, seps, subbuck_size,
+                                                           out_alignment=out_alignment)
+        pshattn.batch_subbuck_reduce(coords, input_feat, seps, max_n, subbuck_size, NUM_VOX, sb.bbox_min, sb.bbox_max,
+                                     sb.subbuck_id, sb.subbuck_off, sb.reduced_sep, sb.reduced_coord, sb.reduced_feat,
+                                     sb.unpool_ind, 1, reduction_op)
+        ctx.save_for_backward(input_feat, sb.unpool_ind)
+        ctx.subbuck_size, ctx.reduction_op = subbuck_size, reduction_op
+        sb.remove_unused_buffers()
+        ctx.mark_non_differentiable(sb.reduced_coord)
+        return sb.reduced_feat, sb
+
+    @staticmethod
+    def backward(ctx, grad_reduced_feat, grad_buffers):
+        raise NotImplementedError("batch_subbuck_reduce_backward: the gfx950 library implements the forward pass only")
+
+
+class InbucketPoolingLayer(nn.Module):
+    REDOP_MAP = {"mean": 0, "sum": 1, "min": 2, "max": 3}
+
+    def __init__(self, reduction_op, out_alignment=1024, subbuck_size=2):
+        """The reference restricts subbuck_size to 2 (pooling.py:159); the kernels here take any size
+        from 1 to 1024, e.g. 8 for a 2x2x2-like reduction."""
+        super().__init__()
+        assert 1 <= subbuck_size <= 1024, f"subbuck_size must be in [1, 1024], input is {subbuck_size}"
+        if isinstance(reduction_op, str):
+            assert reduction_op in self.REDOP_MAP, f"Unsupported reduction op name:{reduction_op}"
+            reduction_op = self.REDOP_MAP[reduction_op]
+        self.reduction_op = int(reduction_op)
+        self.out_align = out_alignment
+        self.subbuck_size = subbuck_size
+
+    def forward(self, coords, input_feat, seps):
+        feat = input_feat if input_feat.dtype == torch.bfloat16 else input_feat.to(torch.bfloat16)
+        return SubbuckReduceFunction.apply(coords, feat.contiguous(), seps, self.subbuck_size, self.reduction_op,
+                                           self.out_align)

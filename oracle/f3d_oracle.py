@@ -330,3 +330,53 @@ def swiglu(h):
     import torch
     hid = h.shape[-1] // 2
     return torch.nn.functional.silu(h[..., :hid].float()) * h[..., hid:].float()
+
+
+# ---------------------------------------------------------------------------------------------
+# model-level restatement: the op sequence of flash3dxfmr/layers (flash3d.py:148-166,
+# stage.py:71-102, hourglass.py:79-112, 165-188, 268-293), every layer output rounded to bf16 as
+# the bf16 modules of the reference do
+# ---------------------------------------------------------------------------------------------
+
+def _r(t):
+    """round an fp32 torch tensor to bf16 and back"""
+    import torch
+    return t.to(torch.bfloat16).float()
+
+
+def psh_scatter_coords(coord_h, seps, bucket_size, pad_to, hash_op, num_vox=0xFFFF):
+    """psh_main.batch_bucket_scatter: whole-batch bbox, geometry heuristics, claim, scatter, pad"""
+    nb, div, _ = psh_params(seps, bucket_size, num_vox)
+    c = np.ascontiguousarray(coord_h, dtype=np.float16)
+    ids, cnt, off = psh_claim(c, seps, c.min(0), c.max(0), num_vox, div, nb, hash_op)
+    _, scat = cumsum_scatter_pad(c, seps, nb, ids, cnt, off, pad_to, 0.0)
+    return scat
+
+
+def xfmr_block(x, w, scopes, bucket_size, num_heads, activation="swiglu"):
+    """x [N,C] fp32 holding bf16 values; w: dict of fp32 tensors (bf16-rounded weights) with keys
+    norm.weight/bias, qkv.weight/bias, proj.weight/bias, ln.weight/bias, fc1.weight/bias, fc2.weight/bias"""
+    import torch
+    n, c = x.shape
+    h = _r(layernorm(x, w["norm.weight"], w["norm.bias"]))
+    qkv = _r(linear(h, w["qkv.weight"], w.get("qkv.bias")))
+    q, k, v = [t.reshape(1, n, num_heads, c // num_heads) for t in qkv.chunk(3, dim=-1)]
+    o, _ = buck_swin_fwd(q, k, v, scopes, bucket_size)
+    o = _r(o).reshape(n, c)
+    mid = _r(_r(linear(o, w["proj.weight"], w["proj.bias"])) + x)
+    h2 = _r(layernorm(mid, w["ln.weight"], w["ln.bias"]))
+    f1 = _r(linear(h2, w["fc1.weight"], w["fc1.bias"]))
+    hid = _r(swiglu(f1)) if activation == "swiglu" else _r(gelu(f1))
+    return _r(_r(linear(hid, w["fc2.weight"], w["fc2.bias"])) + mid)
+
+
+def bn_act(x, bn, act):
+    """eval-mode BatchNorm1d (dict weight, bias, mean, var, eps) then activation name"""
+    import torch
+    if bn is not None:
+        x = _r((x - bn["mean"]) * torch.rsqrt(bn["var"] + bn["eps"]) * bn["weight"] + bn["bias"])
+    if act == "gelu":
+        x = _r(gelu(x))
+    elif act == "relu":
+        x = _r(torch.relu(x))
+    return x
