@@ -6,8 +6,9 @@
 // order depends on arbitration.  Here slots are a stable counting sort:
 //   K1  hash_hist   one workgroup per tile of a cloud: quantise + hash, write bucket_id, LDS
 //                   histogram of the tile -> tile_hist[cloud][tile][bucket]
-//   K2  scan        per cloud: exclusive scan of tile_hist over tiles (in place -> tile base),
-//                   bucket totals -> bucket_counter, inclusive scan over buckets -> cumsum_counter
+//   K2a tile_scan   exclusive scan of tile_hist over the tiles of a cloud (in place -> tile base), totals
+//   K2b bucket_plan per cloud: (optional) deterministic overflow rebalance plan, final bucket counts ->
+//                   bucket_counter, inclusive scan over buckets -> cumsum_counter
 //   K3  rank_scatter per tile: stable rank of every point among the tile's points of the same
 //                   bucket (wave64 ballot matching + per-wave LDS counters), slot = tile base + rank,
 //                   write bucket_offset and scatter the coordinate row; extra workgroups fill the pad rows
@@ -68,60 +69,146 @@ __global__ __launch_bounds__(kPshThreads) void psh_hash_hist_kernel(
   for (uint32_t b = tid; b < num_bucket; b += kPshThreads) out[b] = lds_hist[b];
 }
 
-// One workgroup per cloud.  tile_hist -> exclusive prefix over tiles (plus the counter value the
-// caller passed in, which the reference's atomicAdd commit also builds on), totals -> bucket_counter,
-// inclusive scan over buckets -> cumsum_counter.
-__global__ __launch_bounds__(kPshThreads) void psh_scan_kernel(
-    uint32_t* __restrict__ tile_hist, uint32_t* __restrict__ bucket_counter, uint32_t* __restrict__ cumsum_counter,
+// ---- K2a: exclusive prefix of tile_hist over the tiles of a cloud -------------------------------
+// grid (ceil(NB / 64), clouds) x 1024 threads.  Lane = bucket (64 neighbouring buckets per
+// workgroup, so every access is a coalesced 256-byte row segment), wave = a contiguous range of tiles.
+// Each wave first sums its range, the 16 partial sums are combined through LDS, then each wave
+// rewrites its range with the running prefix.  All loads of a phase are independent of each other.
+constexpr int kScanWaves = 16;
+
+__global__ __launch_bounds__(kScanWaves * kWave) void psh_tile_scan_kernel(
+    uint32_t* __restrict__ tile_hist, const uint32_t* __restrict__ bucket_counter_in, uint32_t* __restrict__ cnt_out,
     const uint32_t* __restrict__ batch_sep, uint32_t num_bucket, uint32_t tile_pts, uint32_t max_tiles) {
-  extern __shared__ uint32_t lds_cnt[];  // num_bucket totals, then wave partials
-  const uint32_t cloud = blockIdx.x, tid = threadIdx.x;
+  __shared__ uint32_t part[kScanWaves][kWave];
+  const uint32_t cloud = blockIdx.y, tid = threadIdx.x, w = tid / kWave, l = tid % kWave;
+  const uint32_t b = blockIdx.x * kWave + l;
   const uint32_t start = cloud ? batch_sep[cloud - 1] : 0u;
   const uint32_t n = batch_sep[cloud] - start;
   const uint32_t ntile = (n + tile_pts - 1) / tile_pts;
-  uint32_t* counter = bucket_counter + (size_t)cloud * num_bucket;
-  for (uint32_t b = tid; b < num_bucket; b += kPshThreads) {
-    uint32_t run = counter[b];
-    uint32_t* h = tile_hist + (size_t)cloud * max_tiles * num_bucket + b;
-    for (uint32_t t = 0; t < ntile; ++t) {
+  const uint32_t per = (ntile + kScanWaves - 1) / kScanWaves;
+  const uint32_t t0 = min(w * per, ntile), t1 = min(t0 + per, ntile);
+  const bool ok = b < num_bucket;
+  uint32_t* h = tile_hist + (size_t)cloud * max_tiles * num_bucket + b;
+  uint32_t sum = 0;
+  if (ok)
+    for (uint32_t t = t0; t < t1; ++t) sum += h[(size_t)t * num_bucket];
+  part[w][l] = sum;
+  __syncthreads();
+  // slots continue from whatever the caller left in bucket_counter (zero by contract)
+  uint32_t run = ok ? bucket_counter_in[(size_t)cloud * num_bucket + b] : 0u;
+  for (uint32_t ww = 0; ww < w; ++ww) run += part[ww][l];
+  if (ok) {
+    for (uint32_t t = t0; t < t1; ++t) {
       const uint32_t c = h[(size_t)t * num_bucket];
       h[(size_t)t * num_bucket] = run;
       run += c;
     }
-    counter[b] = run;
-    lds_cnt[b] = run;
-  }
-  __syncthreads();
-  // inclusive scan over buckets by the first wave: lane owns a contiguous chunk
-  if (tid < kWave) {
-    const uint32_t chunk = (num_bucket + kWave - 1) / kWave;
-    const uint32_t b0 = tid * chunk;
-    uint32_t sum = 0;
-    for (uint32_t i = 0; i < chunk; ++i)
-      if (b0 + i < num_bucket) sum += lds_cnt[b0 + i];
-    uint32_t incl = sum;
-#pragma unroll
-    for (int off = 1; off < kWave; off <<= 1) {
-      const uint32_t up = __shfl_up(incl, off, kWave);
-      if ((int)tid >= off) incl += up;
-    }
-    uint32_t run = incl - sum;
-    uint32_t* cs = cumsum_counter + (size_t)cloud * num_bucket;
-    for (uint32_t i = 0; i < chunk; ++i)
-      if (b0 + i < num_bucket) {
-        run += lds_cnt[b0 + i];
-        cs[b0 + i] = run;
-      }
+    if (w == kScanWaves - 1) cnt_out[(size_t)cloud * num_bucket + b] = run;
   }
 }
 
-template <int ITEMS>
+// inclusive scan of lds_in[0..n) into lds_out[0..n) by the first wave (lane owns a contiguous chunk)
+__device__ __forceinline__ uint32_t wave0_inclusive_scan(const uint32_t* lds_in, uint32_t* lds_out, uint32_t n,
+                                                        uint32_t tid) {
+  const uint32_t chunk = (n + kWave - 1) / kWave;
+  const uint32_t b0 = tid * chunk;
+  uint32_t sum = 0;
+  for (uint32_t i = 0; i < chunk; ++i)
+    if (b0 + i < n) sum += lds_in[b0 + i];
+  uint32_t incl = sum;
+#pragma unroll
+  for (int off = 1; off < kWave; off <<= 1) {
+    const uint32_t up = __shfl_up(incl, off, kWave);
+    if ((int)tid >= off) incl += up;
+  }
+  uint32_t run = incl - sum;
+  for (uint32_t i = 0; i < chunk; ++i)
+    if (b0 + i < n) {
+      run += lds_in[b0 + i];
+      lds_out[b0 + i] = run;
+    }
+  return __shfl(incl, kWave - 1, kWave);  // grand total
+}
+
+// ---- K2b: per-cloud bucket plan ---------------------------------------------------------------------
+// One workgroup per cloud.  From the first-hash counts cnt[b]:
+//   rebalance off: final counts = cnt.
+//   rebalance on : points with slot >= bucket_size in a bucket other than 0 ("overflow units", ordered
+//     by (bucket, slot)) are matched one to one, in order, with the free slots of the buckets other
+//     than 0 that hold fewer than bucket_size points ("free units", ordered by (bucket, slot)); overflow
+//     units beyond the total free capacity are appended to bucket 0, the recycle bucket.  For a z-order
+//     hash this is the order-preserving (nearest in Morton order) transport of the excess.
+// Outputs: bucket_counter = final counts, cumsum_counter = their inclusive scan, and for K3
+// plan[cloud] = { cnt[NB], over_excl[NB], free_incl[NB], total_free }.
+template <bool REBAL>
+__global__ __launch_bounds__(kPshThreads) void psh_bucket_plan_kernel(
+    const uint32_t* __restrict__ cnt_in, uint32_t* __restrict__ bucket_counter, uint32_t* __restrict__ cumsum_counter,
+    uint32_t* __restrict__ plan, uint32_t num_bucket, uint32_t bucket_size) {
+  extern __shared__ uint32_t lds_plan[];
+  uint32_t* s_cnt = lds_plan;                 // first-hash counts
+  uint32_t* s_a = lds_plan + num_bucket;      // overflow per bucket -> inclusive scan
+  uint32_t* s_b = lds_plan + 2 * num_bucket;  // free per bucket -> inclusive scan
+  uint32_t* s_fin = lds_plan + 3 * num_bucket;
+  __shared__ uint32_t s_tot[2];
+  const uint32_t cloud = blockIdx.x, tid = threadIdx.x;
+  const uint32_t* cnt = cnt_in + (size_t)cloud * num_bucket;
+  uint32_t* pl = plan + (size_t)cloud * (3 * num_bucket + 4);
+  for (uint32_t b = tid; b < num_bucket; b += kPshThreads) {
+    const uint32_t c = cnt[b];
+    s_cnt[b] = c;
+    if (REBAL) {
+      s_a[b] = (b != 0 && c > bucket_size) ? c - bucket_size : 0u;
+      s_b[b] = (b != 0 && c < bucket_size) ? bucket_size - c : 0u;
+    }
+  }
+  __syncthreads();
+  if (REBAL) {
+    if (tid < kWave) {
+      const uint32_t tot_over = wave0_inclusive_scan(s_a, s_a, num_bucket, tid);
+      const uint32_t tot_free = wave0_inclusive_scan(s_b, s_b, num_bucket, tid);
+      if (tid == 0) { s_tot[0] = tot_over; s_tot[1] = tot_free; }
+    }
+    __syncthreads();
+    const uint32_t tot_over = s_tot[0], tot_free = s_tot[1];
+    for (uint32_t b = tid; b < num_bucket; b += kPshThreads) {
+      const uint32_t c = s_cnt[b];
+      const uint32_t free_excl = b ? s_b[b - 1] : 0u, free_b = s_b[b] - free_excl;
+      const uint32_t over_excl = b ? s_a[b - 1] : 0u;
+      uint32_t fin;
+      if (b == 0) {
+        fin = c + (tot_over > tot_free ? tot_over - tot_free : 0u);
+      } else {
+        const uint32_t kept = c < bucket_size ? c : bucket_size;
+        const uint32_t filled = tot_over > free_excl ? min(free_b, tot_over - free_excl) : 0u;
+        fin = kept + filled;
+      }
+      s_fin[b] = fin;
+      bucket_counter[(size_t)cloud * num_bucket + b] = fin;
+      pl[b] = c;
+      pl[num_bucket + b] = over_excl;
+      pl[2 * num_bucket + b] = s_b[b];
+    }
+    if (tid == 0) pl[3 * num_bucket] = tot_free;
+  } else {
+    for (uint32_t b = tid; b < num_bucket; b += kPshThreads) {
+      s_fin[b] = s_cnt[b];
+      bucket_counter[(size_t)cloud * num_bucket + b] = s_cnt[b];
+    }
+  }
+  __syncthreads();
+  if (tid < kWave) wave0_inclusive_scan(s_fin, s_fin, num_bucket, tid);
+  __syncthreads();
+  for (uint32_t b = tid; b < num_bucket; b += kPshThreads) cumsum_counter[(size_t)cloud * num_bucket + b] = s_fin[b];
+}
+
+template <int ITEMS, bool REBAL>
 __global__ __launch_bounds__(kPshThreads) void psh_rank_scatter_kernel(
-    const uint16_t* __restrict__ coord, const uint16_t* __restrict__ bucket_id,
+    const uint16_t* __restrict__ coord, uint16_t* __restrict__ bucket_id,
     uint32_t* __restrict__ bucket_offset, const uint32_t* __restrict__ batch_sep, uint32_t batch_size,
     const uint32_t* __restrict__ tile_base, const uint32_t* __restrict__ bucket_counter,
-    const uint32_t* __restrict__ cumsum_counter, uint32_t num_bucket, uint32_t nbits, uint32_t max_tiles,
-    uint16_t* __restrict__ scatter_coord, uint32_t total_n, uint32_t pad_to_n, uint16_t pad_bits) {
+    const uint32_t* __restrict__ cumsum_counter, const uint32_t* __restrict__ plan, uint32_t num_bucket,
+    uint32_t nbits, uint32_t max_tiles, uint32_t bucket_size, uint16_t* __restrict__ scatter_coord, uint32_t total_n,
+    uint32_t pad_to_n, uint16_t pad_bits) {
   extern __shared__ uint32_t lds[];
   const uint32_t cloud = blockIdx.y, tile = blockIdx.x, tid = threadIdx.x;
 
@@ -143,19 +230,28 @@ __global__ __launch_bounds__(kPshThreads) void psh_rank_scatter_kernel(
   const uint32_t tile0 = tile * (kPshThreads * ITEMS);
   if (tile0 >= n) return;
 
-  uint32_t* whist = lds;                             // [kPshWaves][num_bucket] per-wave counts
-  uint32_t* dst_base = lds + kPshWaves * num_bucket; // [num_bucket] bucket start row + tile base
-  uint32_t* slot_base = dst_base + num_bucket;       // [num_bucket] tile base inside the bucket
+  uint32_t* whist = lds;                               // [kPshWaves][NB] per-wave counts
+  uint32_t* row_base = lds + kPshWaves * num_bucket;   // [NB] first output row of the bucket (final layout)
+  uint32_t* slot_base = row_base + num_bucket;         // [NB] tile base inside the first-hash bucket
+  uint32_t* s_cnt = slot_base + num_bucket;            // REBAL: [NB] first-hash counts
+  uint32_t* s_over = s_cnt + num_bucket;               // REBAL: [NB] exclusive scan of the overflow
+  uint32_t* s_free = s_over + num_bucket;              // REBAL: [NB] inclusive scan of the free capacity
   const uint32_t* tb = tile_base + ((size_t)cloud * max_tiles + tile) * num_bucket;
   const uint32_t* cs = cumsum_counter + (size_t)cloud * num_bucket;
-  const uint32_t* cnt = bucket_counter + (size_t)cloud * num_bucket;
+  const uint32_t* fin = bucket_counter + (size_t)cloud * num_bucket;
+  const uint32_t* pl = plan + (size_t)cloud * (3 * num_bucket + 4);
   for (uint32_t b = tid; b < num_bucket; b += kPshThreads) {
 #pragma unroll
     for (int w = 0; w < kPshWaves; ++w) whist[w * num_bucket + b] = 0u;
-    const uint32_t base = tb[b];
-    slot_base[b] = base;
-    dst_base[b] = start + (cs[b] - cnt[b]) + base;  // exclusive cumsum + tile base
+    slot_base[b] = tb[b];
+    row_base[b] = start + (cs[b] - fin[b]);  // exclusive cumsum of the final counts
+    if (REBAL) {
+      s_cnt[b] = pl[b];
+      s_over[b] = pl[num_bucket + b];
+      s_free[b] = pl[2 * num_bucket + b];
+    }
   }
+  const uint32_t tot_free = REBAL ? pl[3 * num_bucket] : 0u;
   __syncthreads();
 
   const uint32_t w = tid / kWave, l = tid % kWave;
@@ -195,9 +291,27 @@ __global__ __launch_bounds__(kPshThreads) void psh_rank_scatter_kernel(
     if (id[j] == 0xFFFFFFFFu) continue;
     const uint32_t local = tile0 + tile_pos<ITEMS>(w, j, l);
     const size_t g = (size_t)start + local;
-    const uint32_t in_tile = mine[id[j]] + rank[j];
-    bucket_offset[g] = slot_base[id[j]] + in_tile;
-    const size_t dst = (size_t)dst_base[id[j]] + in_tile;
+    uint32_t bucket = id[j];
+    uint32_t slot = slot_base[bucket] + mine[bucket] + rank[j];  // stable slot in the first-hash bucket
+    if (REBAL && bucket != 0 && slot >= bucket_size) {
+      // k-th overflow unit of the cloud takes the k-th free unit; none left -> recycle bucket 0
+      const uint32_t k = s_over[bucket] + (slot - bucket_size);
+      if (k < tot_free) {
+        uint32_t lo = 1, hi = num_bucket - 1;  // first bucket whose inclusive free count exceeds k
+        while (lo < hi) {
+          const uint32_t mid = (lo + hi) >> 1;
+          if (s_free[mid] > k) hi = mid; else lo = mid + 1;
+        }
+        bucket = lo;
+        slot = s_cnt[lo] + (k - s_free[lo - 1]);
+      } else {
+        bucket = 0;
+        slot = s_cnt[0] + (k - tot_free);
+      }
+      bucket_id[g] = (uint16_t)bucket;
+    }
+    bucket_offset[g] = slot;
+    const size_t dst = (size_t)row_base[bucket] + slot;
     const uint16_t* p = coord + 3 * g;
     uint16_t* q = scatter_coord + 3 * dst;
     q[0] = p[0]; q[1] = p[1]; q[2] = p[2];
@@ -261,28 +375,31 @@ static uint32_t pick_items(uint32_t instance_max_n, uint32_t batch_size) {
   return 1;
 }
 
-template <int ITEMS>
+template <int ITEMS, bool REBAL>
 static void launch_psh(const uint16_t* coord, uint16_t* bucket_id, uint32_t* bucket_counter, uint32_t* bucket_offset,
-                       const uint32_t* batch_sep, uint32_t batch_size, uint32_t total_n, uint32_t instance_max_n,
-                       uint32_t num_bucket, uint32_t divisor16, uint32_t num_vox, const uint16_t* bbox_min,
+                       const uint32_t* batch_sep, uint32_t batch_size, uint32_t total_n, uint32_t num_bucket,
+                       uint32_t divisor16, uint32_t bucket_size, uint32_t num_vox, const uint16_t* bbox_min,
                        const uint16_t* bbox_max, uint32_t* cumsum_counter, uint16_t* scatter_coord, uint32_t pad_to_n,
-                       uint16_t pad_bits, uint32_t hash_type, uint32_t* tile_hist, uint32_t max_tiles, uint32_t nbits,
-                       hipStream_t stream) {
+                       uint16_t pad_bits, uint32_t hash_type, uint32_t* tile_hist, uint32_t* cnt_ws, uint32_t* plan_ws,
+                       uint32_t max_tiles, uint32_t nbits, hipStream_t stream) {
   const uint32_t tile_pts = kPshThreads * ITEMS;
   if (max_tiles > 0 && batch_size > 0) {
     hipLaunchKernelGGL(psh_hash_hist_kernel<ITEMS>, dim3(max_tiles, batch_size), dim3(kPshThreads),
                        num_bucket * sizeof(uint32_t), stream, coord, bucket_id, batch_sep, bbox_min, bbox_max, num_vox,
                        divisor16, num_bucket, hash_type, tile_hist, max_tiles);
-    hipLaunchKernelGGL(psh_scan_kernel, dim3(batch_size), dim3(kPshThreads), num_bucket * sizeof(uint32_t), stream,
-                       tile_hist, bucket_counter, cumsum_counter, batch_sep, num_bucket, tile_pts, max_tiles);
+    hipLaunchKernelGGL(psh_tile_scan_kernel, dim3(cdiv_u32(num_bucket, kWave), batch_size), dim3(kScanWaves * kWave), 0,
+                       stream, tile_hist, bucket_counter, cnt_ws, batch_sep, num_bucket, tile_pts, max_tiles);
+    hipLaunchKernelGGL(psh_bucket_plan_kernel<REBAL>, dim3(batch_size), dim3(kPshThreads),
+                       4 * num_bucket * sizeof(uint32_t), stream, cnt_ws, bucket_counter, cumsum_counter, plan_ws,
+                       num_bucket, bucket_size);
   }
   const uint32_t pad_tiles = cdiv_u32(pad_to_n - total_n, tile_pts);
   const uint32_t gx = max_tiles > pad_tiles ? max_tiles : pad_tiles;
   if (gx > 0) {
-    hipLaunchKernelGGL(psh_rank_scatter_kernel<ITEMS>, dim3(gx, batch_size + (pad_tiles ? 1 : 0)), dim3(kPshThreads),
-                       (kPshWaves + 2) * num_bucket * sizeof(uint32_t), stream, coord, bucket_id, bucket_offset,
-                       batch_sep, batch_size, tile_hist, bucket_counter, cumsum_counter, num_bucket, nbits, max_tiles,
-                       scatter_coord, total_n, pad_to_n, pad_bits);
+    hipLaunchKernelGGL((psh_rank_scatter_kernel<ITEMS, REBAL>), dim3(gx, batch_size + (pad_tiles ? 1 : 0)),
+                       dim3(kPshThreads), (kPshWaves + 5) * num_bucket * sizeof(uint32_t), stream, coord, bucket_id,
+                       bucket_offset, batch_sep, batch_size, tile_hist, bucket_counter, cumsum_counter, plan_ws,
+                       num_bucket, nbits, max_tiles, bucket_size, scatter_coord, total_n, pad_to_n, pad_bits);
   }
 }
 
@@ -299,7 +416,8 @@ int f3d_batch_psh_scatter_pad_hash(const f3d_half_t* coord, uint16_t* bucket_id,
                                    f3d_half_t* scatter_coord, uint32_t pad_to_n, float pad_num,
                                    uint32_t hash_type, int device, void* stream) {
   using namespace f3d;
-  (void)bucket_size;
+  // The probe table is part of the reference signature; the deterministic rebalance below does not
+  // probe (see psh_bucket_plan_kernel) and never reads it.
   (void)probe_offsets;
   // argument checks of src/psh/batch_psh_bucket_dispatcher.cu:239-250
   F3D_CHECK_ARG(bucket_divisor != 0 && num_bucket != 0 && num_vox / bucket_divisor <= num_bucket,
@@ -328,9 +446,14 @@ int f3d_batch_psh_scatter_pad_hash(const f3d_half_t* coord, uint16_t* bucket_id,
   const uint32_t items = pick_items(instance_max_n, batch_size);
   const uint32_t tile_pts = kPshThreads * items;
   const uint32_t max_tiles = cdiv_u32(instance_max_n, tile_pts);
-  const size_t hist_bytes = (size_t)batch_size * max_tiles * num_bucket * sizeof(uint32_t);
-  uint32_t* tile_hist = (uint32_t*)workspace(device, hist_bytes ? hist_bytes : 4);
+  const size_t hist_words = (size_t)batch_size * max_tiles * num_bucket;
+  const size_t cnt_words = (size_t)batch_size * num_bucket;
+  const size_t plan_words = (size_t)batch_size * (3 * num_bucket + 4);
+  uint32_t* tile_hist = (uint32_t*)workspace(device, (hist_words + cnt_words + plan_words + 4) * sizeof(uint32_t));
   if (!tile_hist) return F3D_ERR_RUNTIME;
+  uint32_t* cnt_ws = tile_hist + hist_words;
+  uint32_t* plan_ws = cnt_ws + cnt_words;
+  const bool rebal = rebalance_mode() != 0 && bucket_size > 0;
   uint32_t nbits = 0;
   while ((1u << nbits) < num_bucket) ++nbits;
   _Float16 pad_h = (_Float16)pad_num;
@@ -340,9 +463,14 @@ int f3d_batch_psh_scatter_pad_hash(const f3d_half_t* coord, uint16_t* bucket_id,
   SyncBracket sync(s);
 #define F3D_PSH_CASE(I)                                                                                          \
   case I:                                                                                                        \
-    launch_psh<I>(coord, bucket_id, bucket_counter, bucket_offset, batch_sep, batch_size, total_n, instance_max_n, \
-                  num_bucket, div16, num_vox, bbox_min, bbox_max, cumsum_counter, scatter_coord, pad_to_n, pad_bits, \
-                  hash_type, tile_hist, max_tiles, nbits, s);                                                   \
+    if (rebal)                                                                                                   \
+      launch_psh<I, true>(coord, bucket_id, bucket_counter, bucket_offset, batch_sep, batch_size, total_n, num_bucket, \
+                          div16, bucket_size, num_vox, bbox_min, bbox_max, cumsum_counter, scatter_coord, pad_to_n,    \
+                          pad_bits, hash_type, tile_hist, cnt_ws, plan_ws, max_tiles, nbits, s);                 \
+    else                                                                                                         \
+      launch_psh<I, false>(coord, bucket_id, bucket_counter, bucket_offset, batch_sep, batch_size, total_n, num_bucket, \
+                           div16, bucket_size, num_vox, bbox_min, bbox_max, cumsum_counter, scatter_coord, pad_to_n,   \
+                           pad_bits, hash_type, tile_hist, cnt_ws, plan_ws, max_tiles, nbits, s);                \
     break;
   switch (items) {
     F3D_PSH_CASE(1)

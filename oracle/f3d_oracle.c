@@ -203,6 +203,53 @@ int f3d_or_psh_claim(const uint16_t *coord_h, uint32_t total_n, const uint32_t *
 }
 
 /* ------------------------------------------------------------------------------------------ */
+/* A4: overflow rebalance + recycle — src/psh/batch_psh_bucket.cuh:154-246 (probe rebalance),   */
+/* :259-382 (recycle).  The reference moves a point whose slot is >= bucket_size (bucket != 0)   */
+/* to the first probed neighbour bucket that still has room, racing on global counters with a   */
+/* shared cuRAND state, and drops the losers into bucket 0; its result is not reproducible.      */
+/* Deterministic restatement used by this build: overflow units, ordered by (bucket, slot), are  */
+/* matched one to one, in order, with the free slots (ordered by (bucket, slot)) of the buckets   */
+/* != 0 holding fewer than bucket_size points; units beyond the total free capacity are appended  */
+/* to bucket 0 (the recycle bucket, which may exceed bucket_size exactly as in the reference).     */
+/* Same invariants as the reference's: every point keeps exactly one (bucket, slot), slots are     */
+/* dense per bucket, points of a bucket that neither overflows nor receives anything stay put.     */
+/* In: first-hash ids / counts / stable slots.  Out (in place): final ids, counts, slots.          */
+/* ------------------------------------------------------------------------------------------ */
+
+int f3d_or_psh_rebalance(uint16_t *bucket_id, uint32_t *bucket_counter, uint32_t *bucket_offset,
+                         const uint32_t *batch_sep, uint32_t batch_size, uint32_t num_bucket,
+                         uint32_t bucket_size) {
+  uint32_t start = 0;
+  for (uint32_t b = 0; b < batch_size; ++b) {
+    uint32_t end = batch_sep[b];
+    uint32_t *cnt = bucket_counter + (size_t)b * num_bucket;
+    /* point index of every (bucket, slot) */
+    size_t *base = (size_t *)malloc(sizeof(size_t) * (num_bucket + 1));
+    base[0] = 0;
+    for (uint32_t k = 0; k < num_bucket; ++k) base[k + 1] = base[k] + cnt[k];
+    uint32_t *who = (uint32_t *)malloc(sizeof(uint32_t) * (base[num_bucket] ? base[num_bucket] : 1));
+    for (uint32_t i = start; i < end; ++i) who[base[bucket_id[i]] + bucket_offset[i]] = i;
+    uint32_t *fin = (uint32_t *)malloc(sizeof(uint32_t) * num_bucket);
+    for (uint32_t k = 0; k < num_bucket; ++k) fin[k] = (k != 0 && cnt[k] > bucket_size) ? bucket_size : cnt[k];
+    uint32_t fb = 1; /* next bucket that may have room */
+    for (uint32_t k = 1; k < num_bucket; ++k) {
+      for (uint32_t slot = bucket_size; slot < cnt[k]; ++slot) {
+        uint32_t p = who[base[k] + slot];
+        /* a bucket that overflowed itself (cnt > bucket_size) never takes immigrants */
+        while (fb < num_bucket && (cnt[fb] >= bucket_size || fin[fb] >= bucket_size)) ++fb;
+        uint32_t dst = (fb < num_bucket) ? fb : 0u;
+        bucket_id[p] = (uint16_t)dst;
+        bucket_offset[p] = fin[dst]++;
+      }
+    }
+    for (uint32_t k = 0; k < num_bucket; ++k) cnt[k] = fin[k];
+    free(base); free(who); free(fin);
+    start = end;
+  }
+  return 0;
+}
+
+/* ------------------------------------------------------------------------------------------ */
 /* A5: cumsum + scatter + tail pad — src/psh/batch_psh_bucket.cuh:493-614                      */
 /* ------------------------------------------------------------------------------------------ */
 

@@ -168,6 +168,18 @@ def psh_claim(coord_h, seps, bbox_min_h, bbox_max_h, num_vox, divisor, num_bucke
     return bucket_id, counter, offset
 
 
+def psh_rebalance(bucket_id, counter, offset, seps, bucket_size):
+    """deterministic overflow rebalance + recycle (A4); returns new (ids, counts, slots)"""
+    ids = np.ascontiguousarray(bucket_id, dtype=np.uint16).copy()
+    cnt = np.ascontiguousarray(counter, dtype=np.uint32).copy()
+    off = np.ascontiguousarray(offset, dtype=np.uint32).copy()
+    seps = np.ascontiguousarray(seps, dtype=np.uint32)
+    rc = lib().f3d_or_psh_rebalance(_p(ids), _p(cnt), _p(off), _p(seps), ctypes.c_uint32(seps.shape[0]),
+                                    ctypes.c_uint32(cnt.shape[1]), ctypes.c_uint32(bucket_size))
+    assert rc == 0
+    return ids, cnt, off
+
+
 def cumsum_scatter_pad(coord_h, seps, num_bucket, bucket_id, counter, offset, pad_to, pad_num=0.0,
                        prefill_nan=True):
     c = _u16(coord_h).reshape(-1, 3)
@@ -344,11 +356,13 @@ def _r(t):
     return t.to(torch.bfloat16).float()
 
 
-def psh_scatter_coords(coord_h, seps, bucket_size, pad_to, hash_op, num_vox=0xFFFF):
-    """psh_main.batch_bucket_scatter: whole-batch bbox, geometry heuristics, claim, scatter, pad"""
+def psh_scatter_coords(coord_h, seps, bucket_size, pad_to, hash_op, num_vox=0xFFFF, rebalance=True):
+    """psh_main.batch_bucket_scatter: whole-batch bbox, geometry heuristics, claim, rebalance, scatter, pad"""
     nb, div, _ = psh_params(seps, bucket_size, num_vox)
     c = np.ascontiguousarray(coord_h, dtype=np.float16)
     ids, cnt, off = psh_claim(c, seps, c.min(0), c.max(0), num_vox, div, nb, hash_op)
+    if rebalance:
+        ids, cnt, off = psh_rebalance(ids, cnt, off, seps, bucket_size)
     _, scat = cumsum_scatter_pad(c, seps, nb, ids, cnt, off, pad_to, 0.0)
     return scat
 

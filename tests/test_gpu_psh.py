@@ -37,8 +37,10 @@ def _run_psh(coords, seps, bucket_size, hash_op, pad_align, oracle, rebalance=0)
                 t=(bucket_id, cntr, offs, s))
 
 
-def _check_against_oracle(coords, seps, out, hash_op, oracle):
+def _check_against_oracle(coords, seps, out, hash_op, oracle, rebalance=0, bucket_size=512):
     ids, cnt, off = oracle.psh_claim(coords, seps, out["bmin"], out["bmax"], 0xFFFF, out["div"], out["nb"], hash_op)
+    if rebalance:
+        ids, cnt, off = oracle.psh_rebalance(ids, cnt, off, seps, bucket_size)
     cumsum, scat = oracle.cumsum_scatter_pad(coords, seps, out["nb"], ids, cnt, off, out["pad_to"], 0.0)
     assert np.array_equal(out["ids"], ids), "bucket ids differ"
     assert np.array_equal(out["cnt"], cnt), "bucket histograms differ"
@@ -145,3 +147,32 @@ def test_python_wrapper_and_saturating_size_properties(oracle):
            + buf.bucket_offs.view(torch.int32).long())
     assert torch.equal(scat[dst], coords)
     assert dst.unique().numel() == n_c * b
+
+
+@pytest.mark.parametrize("case", ["lidar", "uniform_exact_capacity", "ragged"])
+def test_rebalance_bit_exact_and_reference_invariants(oracle, case):
+    """A4 (deterministic overflow rebalance + recycle): final ids, counts, slots and scattered rows
+    bit-exact vs the oracle, and the reference's three checks on the result"""
+    from flash3dtransformer_amd import synth
+    from flash3dtransformer_amd.lib import pshattn
+    if case == "lidar":
+        clouds = [synth.lidar_sweep(40000, 1004 + i, oversample=2) for i in range(3)]
+    elif case == "uniform_exact_capacity":
+        clouds = [synth.uniform_cube(65536, 51.2, 1002), synth.uniform_cube(65536, 51.2, 1003)]
+    else:
+        rng = np.random.default_rng(5)
+        clouds = [rng.normal(0, s, (n, 3)).astype(np.float32) for n, s in ((50000, 3.0), (700, 30.0), (90001, 12.0))]
+    coords, seps = synth.batch_of(clouds)
+    for hash_op in (1, 2):
+        out = _run_psh(coords, seps, 512, hash_op, 3072, oracle, rebalance=1)
+        _check_against_oracle(coords, seps, out, hash_op, oracle, rebalance=1)
+        assert not np.isnan(out["scat"]).any()
+        assert np.array_equal(np.cumsum(out["cnt"], axis=1), out["cumsum"])
+        assert (out["cnt"][:, 1:] <= 512).all()
+        bucket_id, cntr, offs, s = out["t"]
+        b = len(seps)
+        table = torch.zeros((b, out["nb"], int(out["cnt"].max())), dtype=torch.int8, device=DEV)
+        res = cntr.clone()
+        maxcnt = torch.from_numpy(out["cnt"].max(1).astype(np.int32)).to(DEV).view(torch.uint32)
+        pshattn.batch_bucket_sanitizer_cpu(bucket_id, cntr, offs, table, res, s, maxcnt, b, out["nb"])
+    pshattn.DeviceManagerSingleton.instance().set_psh_rebalance(1)

@@ -201,3 +201,46 @@ def test_helpers_closed_forms(oracle):
     assert oracle.gen_scopes(512 * 7, 512, 2, "swin").tolist() == [list(range(7))]
     assert oracle.gen_scopes(512 * 8, 512, 2, "stride").tolist() == [list(range(8))]   # 8 % 12 != 0
     assert oracle.gen_scopes(512 * 12, 512, 2, "stride").shape == (6, 2)
+
+
+@pytest.mark.parametrize("case", ["lidar", "uniform_exact_capacity", "uniform_spare"])
+def test_rebalance_invariants(oracle, case):
+    """A4: the invariants the reference's own checks rest on (tests/test_psh.py:117-129) plus the
+    properties that define a rebalance: conservation, dense unique slots, bounded occupancy wherever
+    capacity exists, untouched buckets stay put, leftovers go to bucket 0 only."""
+    from flash3dtransformer_amd import synth
+    bs = 512
+    if case == "lidar":
+        clouds = [synth.lidar_sweep(30000, 7 + i, oversample=2) for i in range(2)]
+    elif case == "uniform_exact_capacity":
+        clouds = [synth.uniform_cube(65536, 51.2, 3)]          # 128 buckets x 512 == N
+    else:
+        clouds = [synth.uniform_cube(60000, 51.2, 4), synth.uniform_cube(50000, 20.0, 5)]
+    coords, seps = synth.batch_of(clouds)
+    nb, div, _ = oracle.psh_params(seps, bs)
+    ids0, cnt0, off0 = oracle.psh_claim(coords, seps, coords.min(0), coords.max(0), 0xFFFF, div, nb, 1)
+    ids, cnt, off = oracle.psh_rebalance(ids0, cnt0, off0, seps, bs)
+    assert oracle.scoreboard(ids, cnt, off, seps)[0] == 0
+    assert ids.max() < nb
+    start = 0
+    for b, end in enumerate(seps):
+        end = int(end)
+        n = end - start
+        assert cnt[b].sum() == n
+        assert np.array_equal(cnt[b], np.bincount(ids[start:end], minlength=nb))
+        over = np.maximum(cnt0[b][1:].astype(np.int64) - bs, 0).sum()
+        free = np.maximum(bs - cnt0[b][1:].astype(np.int64), 0).sum()
+        assert (cnt[b][1:] <= bs).all()                                   # buckets != 0 are bounded
+        assert cnt[b][0] == cnt0[b][0] + max(0, over - free)              # leftovers land in bucket 0 only
+        moved = ids[start:end] != ids0[start:end]
+        assert moved.sum() == over
+        # only points that overflowed move; everyone else keeps id and slot
+        was_over = (off0[start:end] >= bs) & (ids0[start:end] != 0)
+        assert np.array_equal(moved, was_over)
+        assert np.array_equal(off[start:end][~moved], off0[start:end][~moved])
+        # order-preserving transport: destinations are non-decreasing in (source bucket, slot) order
+        src_order = np.lexsort((off0[start:end][moved], ids0[start:end][moved]))
+        dst = ids[start:end][moved][src_order].astype(np.int64)
+        dst[dst == 0] = nb                                                # recycle bucket comes last
+        assert (np.diff(dst) >= 0).all()
+        start = end
