@@ -1,0 +1,138 @@
+"""End-to-end forward of the layer API on the GPU (Flash3D: PSH embed -> encoder XFMR -> pooling ->
+inner stage -> unpooling -> decoder XFMR) against the same op sequence restated with the CPU oracle.
+
+The reference's own end-to-end test is a smoke test without numeric assertions
+(tests/test_psh_hourglass.py:159-163 of the reference); this one checks numbers: every integer
+structure (scatter order, sub-bucket map) is bit-exact in the per-op tests, so the only differences
+left here are bf16 roundings of the floating-point layers, which stay within a small band."""
+import numpy as np
+import pytest
+import torch
+
+from tests.gpu_util import DEV, bf16_bits
+
+pytestmark = pytest.mark.gpu
+
+
+def _w(sd, prefix, names):
+    f = lambda t: t.detach().float().cpu().to(torch.bfloat16).float()
+    return {k: f(sd[prefix + v]) for k, v in names.items()}
+
+
+XFMR_KEYS = {"norm.weight": "norm.weight", "norm.bias": "norm.bias", "qkv.weight": "bwa.qkv.weight",
+             "qkv.bias": "bwa.qkv.bias", "proj.weight": "bwa.proj.weight", "proj.bias": "bwa.proj.bias",
+             "ln.weight": "mlp.mlp.layer_norm_weight", "ln.bias": "mlp.mlp.layer_norm_bias",
+             "fc1.weight": "mlp.mlp.fc1_weight", "fc1.bias": "mlp.mlp.fc1_bias",
+             "fc2.weight": "mlp.mlp.fc2_weight", "fc2.bias": "mlp.mlp.fc2_bias"}
+
+
+def _bn(sd, prefix):
+    f = lambda k: sd[prefix + k].detach().float().cpu()
+    return {"weight": f("weight"), "bias": f("bias"), "mean": f("running_mean"), "var": f("running_var"), "eps": 1e-3}
+
+
+def test_two_level_hourglass_matches_oracle_pipeline(oracle):
+    from flash3dtransformer_amd import layers as L, synth
+    from flash3dtransformer_amd.psh.bucket_scope import SwinPlan
+    bs, scope, S, hash_op, align1 = 128, 2, 2, 1, 256
+    torch.manual_seed(0)
+    ln = lambda ch: L.LayerNorm(ch)
+    bn = lambda ch: torch.nn.BatchNorm1d(ch, eps=1e-3, momentum=0.01)
+    spec = lambda c, h: L.XFMRSpecs(c, 2 * c, h, True, SwinPlan("swin", bs, scope, 0), ln)
+    levels = [L.F3DLevelSpecs([spec(32, 1)], [spec(32, 1)], "mean", align1, bn, torch.nn.GELU, bn, torch.nn.GELU),
+              L.F3DLevelSpecs([spec(64, 2)], [spec(64, 2)], "mean", align1, None, None, None, None)]
+    model = L.Flash3D(levels, bs, scope, hash_op, subbuck_size=S)
+    # non-trivial norm statistics / affine parameters
+    g = torch.Generator().manual_seed(1)
+    for m in model.modules():
+        if isinstance(m, torch.nn.BatchNorm1d):
+            m.running_mean.copy_(torch.randn(m.num_features, generator=g) * 0.1)
+            m.running_var.copy_(torch.rand(m.num_features, generator=g) + 0.5)
+            m.weight.data.copy_(torch.rand(m.num_features, generator=g) + 0.5)
+            m.bias.data.copy_(torch.randn(m.num_features, generator=g) * 0.1)
+    for n_, p in model.named_parameters():
+        if p.dim() == 2:
+            p.data.mul_(3.0)       # make attention logits and MLP outputs matter
+    model = model.to(DEV).eval()
+
+    rng = np.random.default_rng(3)
+    clouds = [rng.normal(0, 10, (n, 3)).astype(np.float32) for n in (2500, 1800, 2304)]
+    coords, seps = synth.batch_of(clouds)
+    c = torch.from_numpy(coords).to(DEV)
+    s = torch.from_numpy(seps.view(np.int32)).to(DEV).view(torch.uint32)
+    with torch.no_grad():
+        out = model(c, None, s)
+    torch.cuda.synchronize()
+    got = out.float().cpu()
+
+    # ---- the same forward through the oracle ----
+    sd = model.state_dict()
+    n = coords.shape[0]
+    pad_to = -(-n // (bs * scope * 6)) * (bs * scope * 6)
+    assert got.shape == (pad_to, 32)
+    scat = oracle.psh_scatter_coords(coords, seps, bs, pad_to, hash_op)
+    assert np.array_equal(model.psh_scatter.last_scattered_coord.cpu().numpy().view(np.uint16), scat.view(np.uint16))
+    r = oracle._r
+    emb = _w(sd, "psh_scatter.lin.", {"w": "weight", "b": "bias"})
+    x = r(oracle.linear(torch.from_numpy(scat.astype(np.float32)).to(torch.bfloat16), emb["w"], emb["b"]))
+    tree_seps = seps.copy()
+    tree_seps[-1] = pad_to
+    x = oracle.xfmr_block(x, _w(sd, "module_tree.encoder_blocks.0.", XFMR_KEYS), oracle.gen_scopes(pad_to, bs, scope), bs, 1)
+    pw = _w(sd, "module_tree.middle.pooling.proj.", {"w": "weight", "b": "bias"})
+    proj = r(oracle.linear(x, pw["w"], pw["b"]))
+    _, _, unpool, red_coord, red_sep = oracle.subbuck_build(scat, tree_seps, S, out_align=align1)
+    red_len = unpool.shape[0]
+    r_al = -(-red_len // align1) * align1
+    red = torch.from_numpy(oracle.bf16_bits_to_f32(oracle.reduce_feat(bf16_bits(proj.numpy()), unpool, 0, r_aligned=r_al)))
+    red = oracle.bn_act(red, _bn(sd, "module_tree.middle.pooling.norm."), "gelu")
+    sub = "module_tree.middle.submodule."
+    x1 = oracle.xfmr_block(red, _w(sd, sub + "encoder_blocks.0.", XFMR_KEYS), oracle.gen_scopes(r_al, bs, scope), bs, 2)
+    lw = _w(sd, sub + "middle.proj.", {"w": "weight", "b": "bias"})
+    x1 = r(oracle.linear(x1, lw["w"], lw["b"]))
+    x1 = oracle.xfmr_block(x1, _w(sd, sub + "decoder_blocks.0.", XFMR_KEYS), oracle.gen_scopes(r_al, bs, scope), bs, 2)
+    uw = _w(sd, "module_tree.middle.unpooling.proj.0.", {"w": "weight", "b": "bias"})
+    sw = _w(sd, "module_tree.middle.unpooling.proj_skip.0.", {"w": "weight", "b": "bias"})
+    pd = oracle.bn_act(r(oracle.linear(x1, uw["w"], uw["b"])), _bn(sd, "module_tree.middle.unpooling.proj.norm."), "gelu")
+    ps = oracle.bn_act(r(oracle.linear(proj, sw["w"], sw["b"])), _bn(sd, "module_tree.middle.unpooling.proj_skip.norm."), "gelu")
+    up = oracle.additive_unpool(bf16_bits(ps.numpy()), bf16_bits(pd.numpy()), unpool)
+    up = torch.from_numpy(oracle.bf16_bits_to_f32(up))
+    want = oracle.xfmr_block(up, _w(sd, "module_tree.decoder_blocks.0.", XFMR_KEYS), oracle.gen_scopes(pad_to, bs, scope), bs, 1)
+
+    err = (got - want).abs()
+    scale = want.abs().mean().item()
+    assert scale > 0.05, "degenerate test: output too small to be meaningful"
+    assert err.mean().item() <= 0.02 * max(1.0, scale), f"mean err {err.mean().item()} at scale {scale}"
+    assert err.max().item() <= 0.25 * max(1.0, want.abs().max().item()), f"max err {err.max().item()}"
+    # the bulk of the entries agree to bf16 precision
+    assert (err <= 0.05 * max(1.0, scale)).float().mean().item() >= 0.99
+
+
+def test_forward_only_ops_refuse_backward():
+    from flash3dtransformer_amd import layers as L
+    lin = L.Linear(16, 16).to(DEV)
+    x = torch.randn(8, 16, device=DEV, dtype=torch.bfloat16, requires_grad=True)
+    y = lin(x)
+    with pytest.raises(NotImplementedError):
+        y.float().sum().backward()
+    from flash3dtransformer_amd.lib import pshattn
+    with pytest.raises(NotImplementedError):
+        pshattn.buck_swin_bwd(*([None] * 12))
+
+
+def test_state_dict_names_match_reference_module_tree():
+    """parameter names a reference checkpoint would carry (flash3dxfmr/layers/*.py module attributes;
+    TransformerEngine's LayerNormMLP / Linear parameter names)"""
+    from flash3dtransformer_amd import layers as L
+    from flash3dtransformer_amd.psh.bucket_scope import SwinPlan
+    spec = lambda c, h: L.XFMRSpecs(c, 2 * c, h, True, SwinPlan("swin", 128, 1, 0), lambda ch: torch.nn.LayerNorm(ch))
+    bn = lambda ch: torch.nn.BatchNorm1d(ch)
+    levels = [L.F3DLevelSpecs([spec(32, 1)], [spec(32, 1)], "mean", 128, bn, torch.nn.GELU, bn, torch.nn.GELU),
+              L.F3DLevelSpecs([spec(64, 2)], [spec(64, 2)], "mean", 128, None, None, None, None)]
+    keys = set(L.Flash3D(levels, 128, 1, 2).state_dict().keys())
+    for k in ["psh_scatter.lin.weight", "module_tree.encoder_blocks.0.norm.weight",
+              "module_tree.encoder_blocks.0.bwa.qkv.weight", "module_tree.encoder_blocks.0.bwa.proj.bias",
+              "module_tree.encoder_blocks.0.mlp.mlp.fc1_weight", "module_tree.encoder_blocks.0.mlp.mlp.layer_norm_weight",
+              "module_tree.middle.pooling.proj.weight", "module_tree.middle.pooling.norm.running_mean",
+              "module_tree.middle.unpooling.proj.0.weight", "module_tree.middle.unpooling.proj_skip.0.bias",
+              "module_tree.middle.submodule.middle.proj.weight", "module_tree.decoder_blocks.0.mlp.mlp.fc2_bias"]:
+        assert k in keys, k
