@@ -35,7 +35,7 @@ constexpr int kNumXcdG = 8;
 __device__ __forceinline__ float apply_act(float x, uint32_t act) {
   switch (act) {
     case F3D_ACT_GELU: return 0.5f * x * (1.0f + erff(x * 0.70710678118654752440f));
-    case F3D_ACT_SILU: return x / (1.0f + __expf(-x));
+    case F3D_ACT_SILU: return x * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * x));
     case F3D_ACT_RELU: return x > 0.f ? x : 0.f;
     default: return x;
   }
@@ -200,8 +200,8 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_kernel(
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         const float a0 = bf16_lo(a[e]), a1 = bf16_hi(a[e]);
-        float f0 = (a0 / (1.0f + __expf(-a0))) * bf16_lo(gt[e]);
-        float f1 = (a1 / (1.0f + __expf(-a1))) * bf16_hi(gt[e]);
+        float f0 = apply_act(a0, F3D_ACT_SILU) * bf16_lo(gt[e]);
+        float f1 = apply_act(a1, F3D_ACT_SILU) * bf16_hi(gt[e]);
         if (residual) {
           const uint32_t h2 = pack_bf16x2(f0, f1);
           f0 = bf16_lo(h2) + bf16_lo(r[e]);
@@ -317,6 +317,10 @@ __global__ __launch_bounds__(256) void affine_act_kernel(const uint16_t* __restr
   *reinterpret_cast<U16x8*>(y + (size_t)row * C + ch) = o;
 }
 
+bool launch_xstat_linear(const uint16_t* x, uint32_t ldx, const uint16_t* gamma, const uint16_t* beta, float eps,
+                         const uint16_t* w, const uint16_t* bias, const uint16_t* residual, uint32_t ldr, uint16_t* y,
+                         uint32_t ldy, uint32_t M, uint32_t N, uint32_t K, uint32_t act, hipStream_t s);
+
 static int launch_gemm(bool b_trans, const uint16_t* x, uint32_t ldx, const uint16_t* w, uint32_t ldw,
                        const uint16_t* bias, const uint16_t* residual, uint32_t ldr, uint16_t* y, uint32_t ldy,
                        uint32_t M, uint32_t N, uint32_t K, uint32_t act, hipStream_t s) {
@@ -363,8 +367,45 @@ int f3d_linear_bf16(const f3d_bf16_t* x, uint32_t ldx, const f3d_bf16_t* w, cons
   F3D_CHECK_ARG(guard.ok, "cannot select device %d", device);
   hipStream_t s = (hipStream_t)stream;
   SyncBracket sync(s);
-  int rc = launch_gemm(false, x, ldx, w, k, bias, residual, ldr, y, ldy, m, n, k, act, s);
-  if (rc != F3D_OK) return rc;
+  // small inner dimensions: row-panel kernel (x read once, w streamed); otherwise the tiled GEMM
+  if (!launch_xstat_linear(x, ldx, nullptr, nullptr, 0.f, w, bias, residual, ldr, y, ldy, m, n, k, act, s)) {
+    int rc = launch_gemm(false, x, ldx, w, k, bias, residual, ldr, y, ldy, m, n, k, act, s);
+    if (rc != F3D_OK) return rc;
+  }
+  F3D_CHECK_HIP(hipGetLastError());
+  return F3D_OK;
+}
+
+int f3d_ln_linear_bf16(const f3d_bf16_t* x, uint32_t ldx, const f3d_bf16_t* gamma, const f3d_bf16_t* beta, float eps,
+                       const f3d_bf16_t* w, const f3d_bf16_t* bias, const f3d_bf16_t* residual, uint32_t ldr,
+                       f3d_bf16_t* y, uint32_t ldy, uint32_t m, uint32_t n, uint32_t k, uint32_t act, int device,
+                       void* stream) {
+  using namespace f3d;
+  F3D_CHECK_ARG(x && gamma && w && y, "null tensor pointer");
+  F3D_CHECK_ARG(act <= F3D_ACT_RELU, "unknown activation id %u", act);
+  const uint32_t n_out = act == F3D_ACT_SWIGLU ? n / 2 : n;
+  F3D_CHECK_ARG(k == 32 || k == 64 || k == 128 || k == 256,
+                "No kernel found for LayerNorm+Linear with inner dimension K=%u (supported: 32, 64, 128, 256)", k);
+  F3D_CHECK_ARG(n_out % 8 == 0 && (act != F3D_ACT_SWIGLU || n % 64 == 0), "output width %u must be a multiple of 8", n_out);
+  F3D_CHECK_ARG(ldx >= k && ldx % 8 == 0 && ldy >= n_out && ldy % 4 == 0 && (!residual || (ldr >= n_out && ldr % 4 == 0)),
+                "row strides must be aligned and cover a row (ldx=%u ldy=%u ldr=%u)", ldx, ldy, ldr);
+  F3D_CHECK_ARG((((uintptr_t)x | (uintptr_t)w | (uintptr_t)y | (uintptr_t)residual | (uintptr_t)gamma | (uintptr_t)beta) & 15u) == 0,
+                "x/w/y/residual/gamma/beta must be 16-byte aligned");
+  if (m == 0) return F3D_OK;
+  DeviceGuard guard(device);
+  F3D_CHECK_ARG(guard.ok, "cannot select device %d", device);
+  hipStream_t s = (hipStream_t)stream;
+  SyncBracket sync(s);
+  if (!launch_xstat_linear(x, ldx, gamma, beta, eps, w, bias, residual, ldr, y, ldy, m, n, k, act, s)) {
+    // shape outside the fused kernel: normalise into the per-device workspace, then the tiled GEMM
+    uint16_t* tmp = (uint16_t*)workspace(device, (size_t)m * k * sizeof(uint16_t));
+    if (!tmp) return F3D_ERR_RUNTIME;
+    F3D_CHECK_ARG(ldx == k, "LayerNorm+Linear on a strided input needs an output width that is a multiple of 64");
+    const dim3 grid(cdiv_u32(m, 4)), block(256);
+    hipLaunchKernelGGL(layernorm_kernel<1>, grid, block, 0, s, x, gamma, beta, tmp, m, k, eps);
+    int rc = launch_gemm(false, tmp, k, w, k, bias, residual, ldr, y, ldy, m, n, k, act, s);
+    if (rc != F3D_OK) return rc;
+  }
   F3D_CHECK_HIP(hipGetLastError());
   return F3D_OK;
 }

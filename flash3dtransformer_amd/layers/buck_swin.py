@@ -51,7 +51,8 @@ class BucketSwinAttentionModule(nn.Module):
         self.attn = BucketSwinAttention(buck_size)
         self.proj = Linear(channels, channels)
 
-    def forward(self, x: torch.Tensor, scope_buckets: torch.Tensor, residual: torch.Tensor = None) -> torch.Tensor:
+    def forward(self, x: torch.Tensor, scope_buckets: torch.Tensor, residual: torch.Tensor = None,
+                pre_norm=None) -> torch.Tensor:
         """x [B, L, C] -> [B, L, C].  Q, K and V are read by the attention kernel straight out of the
         [B, L, 3C] projection output (the reference makes three contiguous copies, :187-190); the
         residual, when given, is added in the out-projection's epilogue."""
@@ -60,7 +61,7 @@ class BucketSwinAttentionModule(nn.Module):
         assert C == self.num_heads * self.head_dim, f"Expect input channels are {self.num_heads * self.head_dim}, but got {C}"
         if f3ddev.get_nvtx():
             nvtx.range_push(self.NVTX_SCOPE)
-        qkv = self.qkv(x)
+        qkv = self.qkv(x, pre_norm=pre_norm)   # pre_norm: LayerNorm applied inside the projection kernel
         q, k, v = (t.view(B, L, self.num_heads, self.head_dim) for t in torch.chunk(qkv, 3, dim=-1))
         attn_out = self.attn(q, k, v, scope_buckets)
         out = self.proj(attn_out.view(B, L, C), residual=residual)

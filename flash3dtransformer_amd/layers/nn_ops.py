@@ -75,13 +75,19 @@ class Linear(nn.Module):
             bound = 1.0 / math.sqrt(self.in_features)
             nn.init.uniform_(self.bias, -bound, bound)
 
-    def forward(self, x: torch.Tensor, residual: torch.Tensor = None, act=None, out: torch.Tensor = None):
+    def forward(self, x: torch.Tensor, residual: torch.Tensor = None, act=None, out: torch.Tensor = None,
+                pre_norm=None):
+        """`pre_norm`: a LayerNorm-like module (weight, bias, eps) applied to x inside the same kernel"""
         lead = x.shape[:-1]
         x2 = as_bf16_2d(x.reshape(-1, x.shape[-1]))
         n_out = self.out_features // 2 if act == "swiglu" else self.out_features
         y = out if out is not None else torch.empty(x2.shape[0], n_out, dtype=torch.bfloat16, device=x.device)
         r2 = None if residual is None else as_bf16_2d(residual.reshape(-1, n_out))
-        pshattn.linear_bf16(x2, self._w.get(self.weight), self._b.get(self.bias), r2, y, act)
+        if pre_norm is not None:
+            g, b = norm_params_bf16(pre_norm)
+            pshattn.ln_linear_bf16(x2, g, b, pre_norm.eps, self._w.get(self.weight), self._b.get(self.bias), r2, y, act)
+        else:
+            pshattn.linear_bf16(x2, self._w.get(self.weight), self._b.get(self.bias), r2, y, act)
         return forward_only(y.view(*lead, n_out), "Linear", x, self.weight)
 
     def extra_repr(self):
@@ -103,6 +109,25 @@ class LayerNorm(nn.Module):
         y = torch.empty_like(x2)
         pshattn.layernorm_bf16(x2, self._w.get(self.weight), self._b.get(self.bias), y, self.eps)
         return forward_only(y.view(x.shape), "LayerNorm", x, self.weight)
+
+
+FUSABLE_LN_WIDTHS = (32, 64, 128, 256)
+
+
+def is_fusable_layernorm(norm, width: int) -> bool:
+    """LayerNorm over one axis with affine weights, at a width the fused LayerNorm+Linear kernel covers"""
+    if width not in FUSABLE_LN_WIDTHS:
+        return False
+    if isinstance(norm, LayerNorm):
+        return True
+    return isinstance(norm, nn.LayerNorm) and norm.elementwise_affine and len(norm.normalized_shape) == 1
+
+
+def norm_params_bf16(norm):
+    if isinstance(norm, LayerNorm):
+        return norm._w.get(norm.weight), norm._b.get(norm.bias)
+    b = None if norm.bias is None else norm.bias.detach().to(torch.bfloat16).contiguous()
+    return norm.weight.detach().to(torch.bfloat16).contiguous(), b
 
 
 def apply_norm(norm: nn.Module, x: torch.Tensor) -> torch.Tensor:
@@ -178,10 +203,14 @@ class LayerNormMLP(nn.Module):
     def forward(self, x: torch.Tensor, residual: torch.Tensor = None):
         x2 = as_bf16_2d(x.reshape(-1, self.hidden_size)).contiguous()
         c = self._c
-        ln = torch.empty_like(x2)
-        pshattn.layernorm_bf16(x2, c[0].get(self.layer_norm_weight), c[1].get(self.layer_norm_bias), ln, self.eps)
         h = torch.empty(x2.shape[0], self.ffn_hidden_size, dtype=torch.bfloat16, device=x.device)
-        pshattn.linear_bf16(ln, c[2].get(self.fc1_weight), c[3].get(self.fc1_bias), None, h, self.activation)
+        if self.hidden_size in FUSABLE_LN_WIDTHS:
+            pshattn.ln_linear_bf16(x2, c[0].get(self.layer_norm_weight), c[1].get(self.layer_norm_bias), self.eps,
+                                   c[2].get(self.fc1_weight), c[3].get(self.fc1_bias), None, h, self.activation)
+        else:
+            ln = torch.empty_like(x2)
+            pshattn.layernorm_bf16(x2, c[0].get(self.layer_norm_weight), c[1].get(self.layer_norm_bias), ln, self.eps)
+            pshattn.linear_bf16(ln, c[2].get(self.fc1_weight), c[3].get(self.fc1_bias), None, h, self.activation)
         y = torch.empty_like(x2)
         r2 = None if residual is None else as_bf16_2d(residual.reshape(-1, self.hidden_size))
         pshattn.linear_bf16(h, c[4].get(self.fc2_weight), c[5].get(self.fc2_bias), r2, y, None)

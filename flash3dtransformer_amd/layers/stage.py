@@ -9,7 +9,7 @@ from torch import nn
 from ..psh import bucket_scope
 from ..psh import dev_context as f3ddev
 from . import buck_swin, elem_wise
-from .nn_ops import apply_norm
+from .nn_ops import apply_norm, is_fusable_layernorm
 
 
 @dataclass(slots=True)
@@ -43,8 +43,12 @@ class XFMR(nn.Module):
         scope_bucks = self.swin_plan.gen_scopes_from_plan(N, reduced_feat.device)
         if f3ddev.get_nvtx():
             nvtx.range_push(self.NVTX_SCOPE)
-        x = apply_norm(self.norm, reduced_feat)
-        mid = self.bwa(x.view(1, N, C), scope_bucks, residual=reduced_feat.view(1, N, C)).view(N, C)
+        if is_fusable_layernorm(self.norm, C):   # norm -> qkv in one kernel
+            mid = self.bwa(reduced_feat.view(1, N, C), scope_bucks, residual=reduced_feat.view(1, N, C),
+                           pre_norm=self.norm).view(N, C)
+        else:
+            x = apply_norm(self.norm, reduced_feat)
+            mid = self.bwa(x.view(1, N, C), scope_bucks, residual=reduced_feat.view(1, N, C)).view(N, C)
         out = self.mlp(mid, residual=mid)
         if f3ddev.get_nvtx():
             nvtx.range_pop()

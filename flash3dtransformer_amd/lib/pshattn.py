@@ -352,6 +352,30 @@ def linear_bf16(x, w, bias, residual, y, act=None):
                                    _stream(dev)))
 
 
+def ln_linear_bf16(x, gamma, beta, eps, w, bias, residual, y, act=None):
+    """extension: y = act(LayerNorm(x) @ w.T + bias) + residual in one kernel (K in 32..512)"""
+    dev = assert_same_device([x, gamma, w, y])
+    assert_dtype([x, gamma, w, y], torch.bfloat16)
+    assert_contiguous([w, gamma])
+    if x.dim() != 2 or y.dim() != 2 or x.stride(1) != 1 or y.stride(1) != 1:
+        raise RuntimeError("ln_linear_bf16 expects 2-D row-major x and y")
+    m, k = x.shape
+    n = w.shape[0]
+    a = ACT[act] if not isinstance(act, int) else act
+    n_out = n // 2 if a == 2 else n
+    if w.shape[1] != k or tuple(y.shape) != (m, n_out) or gamma.shape[0] != k:
+        raise RuntimeError(f"ln_linear shape mismatch: x{tuple(x.shape)} w{tuple(w.shape)} y{tuple(y.shape)}")
+    ldr = 0
+    if residual is not None:
+        assert_dtype([residual], torch.bfloat16)
+        if tuple(residual.shape) != (m, n_out) or residual.stride(1) != 1:
+            raise RuntimeError("residual must be [m, n_out] row-major")
+        ldr = residual.stride(0)
+    _check(_load().f3d_ln_linear_bf16(_ptr(x), _u32(x.stride(0)), _ptr(gamma), _ptr(beta), _f32(eps), _ptr(w),
+                                      _ptr(bias), _ptr(residual), _u32(ldr), _ptr(y), _u32(y.stride(0)), _u32(m),
+                                      _u32(n), _u32(k), _u32(a), _i32(dev), _stream(dev)))
+
+
 def layernorm_bf16(x, gamma, beta, y, eps=1e-5):
     """extension: LayerNorm over the last axis, fp32 statistics"""
     assert_contiguous([x, gamma, y])

@@ -163,6 +163,16 @@ int f3d_linear_bf16(const f3d_bf16_t* x, uint32_t ldx, const f3d_bf16_t* w, cons
                     const f3d_bf16_t* residual, uint32_t ldr, f3d_bf16_t* y, uint32_t ldy, uint32_t m,
                     uint32_t n, uint32_t k, uint32_t act, int device, void* stream);
 
+/* LayerNorm fused into the following linear layer: y = act(LayerNorm(x; gamma, beta, eps) · wᵀ + bias)
+ * + residual, the `norm -> qkv` and `LayerNormMLP` front halves of flash3dxfmr/layers/stage.py:94-99.
+ * Same tensor contract as f3d_linear_bf16 with k in {32, 64, 128, 256}; gamma [k] bf16, beta [k]
+ * bf16 or NULL.  The normalised activations are rounded to bf16 before the product, as a separate
+ * LayerNorm module would emit them. */
+int f3d_ln_linear_bf16(const f3d_bf16_t* x, uint32_t ldx, const f3d_bf16_t* gamma, const f3d_bf16_t* beta, float eps,
+                       const f3d_bf16_t* w, const f3d_bf16_t* bias, const f3d_bf16_t* residual, uint32_t ldr,
+                       f3d_bf16_t* y, uint32_t ldy, uint32_t m, uint32_t n, uint32_t k, uint32_t act, int device,
+                       void* stream);
+
 /* LayerNorm over the last axis, fp32 statistics (norm callables of flash3dxfmr/layers/stage.py:67).
  * x,y [m,c] bf16; gamma,beta [c] bf16 (beta may be NULL). */
 int f3d_layernorm_bf16(const f3d_bf16_t* x, const f3d_bf16_t* gamma, const f3d_bf16_t* beta, f3d_bf16_t* y,

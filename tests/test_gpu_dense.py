@@ -75,6 +75,31 @@ def test_linear_epilogues(oracle, M, N, K, act, use_bias, use_res):
     _close(y, ref)
 
 
+@pytest.mark.parametrize("M,N,K,act,use_res", [
+    (5000, 768, 256, None, False),       # norm -> qkv of the C=256 block
+    (5000, 2048, 256, "swiglu", False),  # LayerNormMLP front half
+    (333, 96, 32, "gelu", True),
+    (1000, 192, 64, None, True),
+    (2049, 256, 128, "relu", False),
+])
+def test_layernorm_fused_linear(oracle, M, N, K, act, use_res):
+    from flash3dtransformer_amd.lib import pshattn
+    x, w = _rand((M, K), 1, scale=2.0) + 0.3, _rand((N, K), 2, scale=1 / math.sqrt(K))
+    g, b, bias = _rand((K,), 3) + 1.0, _rand((K,), 4, scale=0.2), _rand((N,), 5)
+    n_out = N // 2 if act == "swiglu" else N
+    res = _rand((M, n_out), 6) if use_res else None
+    y = torch.full((M, n_out), 9.0, dtype=torch.bfloat16, device=DEV)
+    pshattn.ln_linear_bf16(x.to(DEV), g.to(DEV), b.to(DEV), 1e-5, w.to(DEV), bias.to(DEV),
+                           None if res is None else res.to(DEV), y, act)
+    torch.cuda.synchronize()
+    ln = oracle.layernorm(x, g, b, 1e-5).to(torch.bfloat16).float()
+    lin = oracle.linear(ln, w, bias).to(torch.bfloat16).float()
+    ref = {"swiglu": oracle.swiglu, "gelu": oracle.gelu, "relu": torch.relu, None: lambda t: t}[act](lin)
+    if res is not None:
+        ref = ref.to(torch.bfloat16).float() + res.float()
+    _close(y, ref, tol=3e-2)
+
+
 def test_linear_strided_views():
     """x and y may be column slices of wider buffers (row stride > width)"""
     from flash3dtransformer_amd.lib import pshattn
