@@ -19,6 +19,9 @@ COMMON = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc",
     # packed fp32 VALU ops are kept out of the generated code on purpose
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # MFMA accumulators live in ordinary VGPRs (unified register file on gfx90a+): the softmax and the
+    # epilogues read them without v_accvgpr moves
+    "-mllvm", "-amdgpu-mfma-vgpr-form",
     "-Wall", "-Wno-unused-function", "-Wno-unknown-warning-option",
 ]
 # bit-exact integer / quantiser kernels: no fused multiply-add contraction

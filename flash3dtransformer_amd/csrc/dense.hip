@@ -214,87 +214,115 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_kernel(
   }
 }
 
-// ---- LayerNorm: one wave per row, row kept in registers, fp32 two-pass statistics ----------------
-template <int VPL>  // 16-byte chunks per lane: C <= 64 * 8 * VPL
+// ---- LayerNorm: LPR lanes per row (a wave covers 64 / LPR rows), the row kept in registers, fp32
+//      two-pass statistics.  LPR * VPL 16-byte chunks cover a row. ----
+template <int LPR, int VPL>
 __global__ __launch_bounds__(256) void layernorm_kernel(const uint16_t* __restrict__ x,
                                                         const uint16_t* __restrict__ gamma,
                                                         const uint16_t* __restrict__ beta, uint16_t* __restrict__ y,
                                                         uint32_t M, uint32_t C, float eps) {
-  const uint32_t row = blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave;
-  const uint32_t lane = threadIdx.x % kWave;
-  if (row >= M) return;
+  constexpr int RPW = kWave / LPR;  // rows per wave
+  const uint32_t lane = threadIdx.x % kWave, sub = lane % LPR;
+  const uint32_t row = (blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave) * RPW + lane / LPR;
+  const bool row_ok = row < M;
   const uint32_t nchunk = C / 8;
-  float v[VPL][8];
+  u32x4_t v[VPL];
   float sum = 0.f;
 #pragma unroll
   for (int i = 0; i < VPL; ++i) {
-    const uint32_t c = lane + i * kWave;
-    if (c < nchunk) {
-      const U16x8 t = *reinterpret_cast<const U16x8*>(x + (size_t)row * C + c * 8);
+    const uint32_t c = sub + i * LPR;
+    v[i] = u32x4_t{0u, 0u, 0u, 0u};
+    if (row_ok && c < nchunk) v[i] = *reinterpret_cast<const u32x4_t*>(x + (size_t)row * C + c * 8);
 #pragma unroll
-      for (int e = 0; e < 8; ++e) { v[i][e] = bf16_bits_to_float(t.v[e]); sum += v[i][e]; }
-    } else {
-#pragma unroll
-      for (int e = 0; e < 8; ++e) v[i][e] = 0.f;
-    }
+    for (int e = 0; e < 4; ++e) sum += bf16_lo(v[i][e]) + bf16_hi(v[i][e]);
   }
 #pragma unroll
-  for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off, kWave);
+  for (int off = LPR / 2; off > 0; off >>= 1) sum += __shfl_xor(sum, off, kWave);
   const float mean = sum / (float)C;
   float sq = 0.f;
 #pragma unroll
   for (int i = 0; i < VPL; ++i) {
-    const uint32_t c = lane + i * kWave;
+    const uint32_t c = sub + i * LPR;
     if (c < nchunk) {
 #pragma unroll
-      for (int e = 0; e < 8; ++e) { const float d = v[i][e] - mean; sq += d * d; }
+      for (int e = 0; e < 4; ++e) {
+        const float d0 = bf16_lo(v[i][e]) - mean, d1 = bf16_hi(v[i][e]) - mean;
+        sq += d0 * d0 + d1 * d1;
+      }
     }
   }
 #pragma unroll
-  for (int off = 32; off > 0; off >>= 1) sq += __shfl_xor(sq, off, kWave);
+  for (int off = LPR / 2; off > 0; off >>= 1) sq += __shfl_xor(sq, off, kWave);
   const float rstd = rsqrtf(sq / (float)C + eps);
 #pragma unroll
   for (int i = 0; i < VPL; ++i) {
-    const uint32_t c = lane + i * kWave;
-    if (c < nchunk) {
-      const U16x8 g = *reinterpret_cast<const U16x8*>(gamma + c * 8);
-      U16x8 b, t;
-      if (beta) b = *reinterpret_cast<const U16x8*>(beta + c * 8);
+    const uint32_t c = sub + i * LPR;
+    if (row_ok && c < nchunk) {
+      const u32x4_t g = *reinterpret_cast<const u32x4_t*>(gamma + c * 8);
+      u32x4_t b = {0u, 0u, 0u, 0u}, t;
+      if (beta) b = *reinterpret_cast<const u32x4_t*>(beta + c * 8);
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        float f = (v[i][e] - mean) * rstd * bf16_bits_to_float(g.v[e]);
-        if (beta) f += bf16_bits_to_float(b.v[e]);
-        t.v[e] = float_to_bf16_bits(f);
+      for (int e = 0; e < 4; ++e) {
+        const float f0 = (bf16_lo(v[i][e]) - mean) * rstd * bf16_lo(g[e]) + bf16_lo(b[e]);
+        const float f1 = (bf16_hi(v[i][e]) - mean) * rstd * bf16_hi(g[e]) + bf16_hi(b[e]);
+        t[e] = pack_bf16x2(f0, f1);
       }
-      *reinterpret_cast<U16x8*>(y + (size_t)row * C + c * 8) = t;
+      *reinterpret_cast<u32x4_t*>(y + (size_t)row * C + c * 8) = t;
     }
   }
 }
 
-// ---- coordinate embedding: y[r, :] = bf16(coord[r, :]) wT + bias, w [C,3] -------------------------
+static void launch_layernorm(const uint16_t* x, const uint16_t* gamma, const uint16_t* beta, uint16_t* y, uint32_t m,
+                             uint32_t c, float eps, hipStream_t s) {
+  const uint32_t nchunk = c / 8;
+#define F3D_LN(LPR, VPL)                                                                                       \
+  hipLaunchKernelGGL((layernorm_kernel<LPR, VPL>), dim3(cdiv_u32(m, 4 * (kWave / LPR))), dim3(256), 0, s, x, gamma, \
+                     beta, y, m, c, eps)
+  if (nchunk <= 4) F3D_LN(4, 1);
+  else if (nchunk <= 8) F3D_LN(8, 1);
+  else if (nchunk <= 16) F3D_LN(16, 1);
+  else if (nchunk <= 32) F3D_LN(32, 1);
+  else if (nchunk <= 64) F3D_LN(64, 1);
+  else if (nchunk <= 128) F3D_LN(64, 2);
+  else if (nchunk <= 256) F3D_LN(64, 4);
+  else F3D_LN(64, 8);
+#undef F3D_LN
+}
+
+// ---- coordinate embedding: y[r, :] = bf16(coord[r, :]) wT + bias, w [C,3].  A thread owns one
+//      8-channel chunk (its 24 weights and 8 biases stay in registers) and walks down the rows;
+//      the C/8 threads of a row write one contiguous burst. ----
 __global__ __launch_bounds__(256) void coord_embed_kernel(const uint16_t* __restrict__ coord,
                                                           const uint16_t* __restrict__ w,
                                                           const uint16_t* __restrict__ bias, uint16_t* __restrict__ y,
-                                                          uint32_t M, uint32_t C) {
-  const size_t gid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+                                                          uint32_t M, uint32_t C, uint32_t rows_per_block) {
   const uint32_t cpr = C / 8;
-  const uint32_t row = (uint32_t)(gid / cpr), ch = (uint32_t)(gid % cpr) * 8;
-  if (row >= M) return;
-  float p[3];
-#pragma unroll
-  for (int d = 0; d < 3; ++d)  // fp16 -> bf16 cast of the layer input (psh_ops.py:67)
-    p[d] = bf16_bits_to_float(float_to_bf16_bits(half_bits_to_float(coord[3 * (size_t)row + d])));
-  U16x8 t;
+  const uint32_t slots = blockDim.x / cpr;              // rows handled concurrently by the block
+  const uint32_t ch = (threadIdx.x % cpr) * 8, slot = threadIdx.x / cpr;
+  if (slot >= slots) return;
+  float wx[8], wy[8], wz[8], bb[8];
 #pragma unroll
   for (int e = 0; e < 8; ++e) {
     const uint16_t* wr = w + (size_t)(ch + e) * 3;
-    float f = p[0] * bf16_bits_to_float(wr[0]);
-    f = __builtin_fmaf(p[1], bf16_bits_to_float(wr[1]), f);
-    f = __builtin_fmaf(p[2], bf16_bits_to_float(wr[2]), f);
-    if (bias) f += bf16_bits_to_float(bias[ch + e]);
-    t.v[e] = float_to_bf16_bits(f);
+    wx[e] = bf16_bits_to_float(wr[0]); wy[e] = bf16_bits_to_float(wr[1]); wz[e] = bf16_bits_to_float(wr[2]);
+    bb[e] = bias ? bf16_bits_to_float(bias[ch + e]) : 0.f;
   }
-  *reinterpret_cast<U16x8*>(y + (size_t)row * C + ch) = t;
+  const uint32_t r_begin = blockIdx.x * rows_per_block;
+  const uint32_t r_end = min(r_begin + rows_per_block, M);
+  for (uint32_t row = r_begin + slot; row < r_end; row += slots) {
+    float p[3];
+#pragma unroll
+    for (int d = 0; d < 3; ++d)  // fp16 -> bf16 cast of the layer input (psh_ops.py:67)
+      p[d] = bf16_bits_to_float(float_to_bf16_bits(half_bits_to_float(coord[3 * (size_t)row + d])));
+    u32x4_t t;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      float f0 = __builtin_fmaf(p[2], wz[2 * e], __builtin_fmaf(p[1], wy[2 * e], p[0] * wx[2 * e])) + bb[2 * e];
+      float f1 = __builtin_fmaf(p[2], wz[2 * e + 1], __builtin_fmaf(p[1], wy[2 * e + 1], p[0] * wx[2 * e + 1])) + bb[2 * e + 1];
+      t[e] = pack_bf16x2(f0, f1);
+    }
+    *reinterpret_cast<u32x4_t*>(y + (size_t)row * C + ch) = t;
+  }
 }
 
 // ---- y = act(x * scale[c] + shift[c]) --------------------------------------------------------------
@@ -401,8 +429,7 @@ int f3d_ln_linear_bf16(const f3d_bf16_t* x, uint32_t ldx, const f3d_bf16_t* gamm
     uint16_t* tmp = (uint16_t*)workspace(device, (size_t)m * k * sizeof(uint16_t));
     if (!tmp) return F3D_ERR_RUNTIME;
     F3D_CHECK_ARG(ldx == k, "LayerNorm+Linear on a strided input needs an output width that is a multiple of 64");
-    const dim3 grid(cdiv_u32(m, 4)), block(256);
-    hipLaunchKernelGGL(layernorm_kernel<1>, grid, block, 0, s, x, gamma, beta, tmp, m, k, eps);
+    launch_layernorm(x, gamma, beta, tmp, m, k, eps, s);
     int rc = launch_gemm(false, tmp, k, w, k, bias, residual, ldr, y, ldy, m, n, k, act, s);
     if (rc != F3D_OK) return rc;
   }
@@ -437,11 +464,7 @@ int f3d_layernorm_bf16(const f3d_bf16_t* x, const f3d_bf16_t* gamma, const f3d_b
   F3D_CHECK_ARG(guard.ok, "cannot select device %d", device);
   hipStream_t s = (hipStream_t)stream;
   SyncBracket sync(s);
-  const dim3 grid(cdiv_u32(m, 4)), block(256);
-  if (c <= 512) hipLaunchKernelGGL(layernorm_kernel<1>, grid, block, 0, s, x, gamma, beta, y, m, c, eps);
-  else if (c <= 1024) hipLaunchKernelGGL(layernorm_kernel<2>, grid, block, 0, s, x, gamma, beta, y, m, c, eps);
-  else if (c <= 2048) hipLaunchKernelGGL(layernorm_kernel<4>, grid, block, 0, s, x, gamma, beta, y, m, c, eps);
-  else hipLaunchKernelGGL(layernorm_kernel<8>, grid, block, 0, s, x, gamma, beta, y, m, c, eps);
+  launch_layernorm(x, gamma, beta, y, m, c, eps, s);
   F3D_CHECK_HIP(hipGetLastError());
   return F3D_OK;
 }
@@ -450,14 +473,17 @@ int f3d_coord_embed_bf16(const f3d_half_t* coord, const f3d_bf16_t* w, const f3d
                          uint32_t m, uint32_t c, int device, void* stream) {
   using namespace f3d;
   F3D_CHECK_ARG(coord && w && y, "null tensor pointer");
-  F3D_CHECK_ARG(c % 8 == 0 && c > 0, "embedding width %u must be a positive multiple of 8", c);
+  F3D_CHECK_ARG(c % 8 == 0 && c > 0 && c <= 2048, "embedding width %u must be a multiple of 8 in [8, 2048]", c);
   if (m == 0) return F3D_OK;
   DeviceGuard guard(device);
   F3D_CHECK_ARG(guard.ok, "cannot select device %d", device);
   hipStream_t s = (hipStream_t)stream;
   SyncBracket sync(s);
-  const size_t total = (size_t)m * (c / 8);
-  hipLaunchKernelGGL(coord_embed_kernel, dim3((uint32_t)((total + 255) / 256)), dim3(256), 0, s, coord, w, bias, y, m, c);
+  const uint32_t slots = 256 / (c / 8);
+  uint32_t rows_per_block = slots * 16;                       // 16 rows per thread amortise the weight loads
+  while (rows_per_block > slots && cdiv_u32(m, rows_per_block) < 1024) rows_per_block /= 2;
+  hipLaunchKernelGGL(coord_embed_kernel, dim3(cdiv_u32(m, rows_per_block)), dim3(256), 0, s, coord, w, bias, y, m, c,
+                     rows_per_block);
   F3D_CHECK_HIP(hipGetLastError());
   return F3D_OK;
 }

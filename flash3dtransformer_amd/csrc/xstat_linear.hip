@@ -334,7 +334,9 @@ bool launch_xstat_linear(const uint16_t* x, uint32_t ldx, const uint16_t* gamma,
   if (M == 0) return true;
   if (N % 64 != 0) return false;     // chunks of 64 output features (32 value + 32 gate for swiglu) must be full
   if (ln && K == 512) return false;  // 128 row values per lane plus the fp32 statistics do not fit the register file
-  static const int mt_env = getenv("F3D_XS_MT") ? atoi(getenv("F3D_XS_MT")) : 0;
+  // One 32-row tile per wave (MT = 1) leaves room for two workgroups per CU, which measured faster than
+  // MT = 2 at every shape of the model; F3D_XS_MT=2 selects the larger panel for experiments.
+  static const int mt_env = getenv("F3D_XS_MT") ? atoi(getenv("F3D_XS_MT")) : 1;
 #define F3D_XS_CASE(KK, MTT)                                                                                        \
   case KK: {                                                                                                        \
     const size_t lds = (size_t)2 * kXsChunk * (KK + 8) * 2;                                                         \
