@@ -40,7 +40,7 @@ struct AttnCfg {
   static constexpr int VROW = KT + 8;                   // padded LDS row of Vt (elements)
   static constexpr int CHUNKS = KT * D / 8;             // 16-byte chunks per K (or V) tile
   static constexpr int NCH = (CHUNKS + kAttnThreads - 1) / kAttnThreads;
-  static constexpr int LDS_BYTES = (KT * KROW + D * VROW) * 2;
+  static constexpr int LDS_BYTES = (KT * KROW + D * VROW) * 2;   // plus 8 bytes per scope entry
 };
 
 template <int D, int KT>
@@ -53,6 +53,10 @@ __global__ __launch_bounds__(kAttnThreads) void buck_swin_fwd_kernel(
   extern __shared__ __attribute__((aligned(16))) uint16_t lds_attn[];
   uint16_t* sK = lds_attn;                  // [KT][KROW]
   uint16_t* sVt = lds_attn + KT * C::KROW;  // [D][VROW]
+  // per scope entry: bucket id and number of valid keys (0 for an id outside the sequence), read once
+  // from global memory so that the tile loop never waits on a scalar load
+  uint32_t* s_bucket = reinterpret_cast<uint32_t*>(lds_attn + KT * C::KROW + D * C::VROW);
+  int32_t* s_len = reinterpret_cast<int32_t*>(s_bucket + scope_size);
 
   // XCD-aware remap: hardware deals consecutive workgroup ids round-robin to the 8 XCDs
   const uint32_t work = (blockIdx.x % kNumXcd) * work_per_xcd + blockIdx.x / kNumXcd;
@@ -71,12 +75,18 @@ __global__ __launch_bounds__(kAttnThreads) void buck_swin_fwd_kernel(
   // ---- this wave's 32 query rows ----
   const uint32_t q_local = qb * kQBlock;                 // row offset inside the scope
   const uint32_t n_bucket = seq_len / bs;
-  const uint32_t q_bucket = my_scope[q_local / bs];
+  for (uint32_t j = tid; j < scope_size; j += kAttnThreads) {
+    const uint32_t b = my_scope[j];
+    s_bucket[j] = b;
+    s_len[j] = b >= n_bucket ? 0 : (kv_len ? min(max(kv_len[b], 0), (int32_t)bs) : (int32_t)bs);
+  }
+  __syncthreads();
+  const uint32_t q_bucket = s_bucket[q_local / bs];
   if (q_bucket >= n_bucket) return;  // a scope entry outside the sequence names no rows (uniform per workgroup)
   const uint32_t q_in_bucket = (q_local % bs) + wave * 32 + lq;
   const uint32_t q_row = q_bucket * bs + q_in_bucket;
   const size_t tok0 = (size_t)batch * seq_len;
-  const int32_t q_valid_len = kv_len ? min(max(kv_len[q_bucket], 0), (int32_t)bs) : (int32_t)bs;
+  const int32_t q_valid_len = s_len[q_local / bs];
 
   bf16x8_t qf[C::KSTEPS];
   {
@@ -95,11 +105,7 @@ __global__ __launch_bounds__(kAttnThreads) void buck_swin_fwd_kernel(
   // ---- KV tile iteration state ----
   const uint32_t tiles_per_bucket = bs / KT;
   uint32_t jb = 0, kt = 0;  // scope bucket index, tile inside the bucket
-  auto bucket_len = [&](uint32_t j) -> int32_t {  // valid keys of scope bucket j; 0 for an out-of-range bucket id
-    const uint32_t b = my_scope[j];
-    if (b >= n_bucket) return 0;
-    return kv_len ? min(max(kv_len[b], 0), (int32_t)bs) : (int32_t)bs;
-  };
+  auto bucket_len = [&](uint32_t j) -> int32_t { return s_len[j]; };
   auto settle = [&]() {  // advance (jb, kt) to the next tile that holds at least one valid key
     while (jb < scope_size) {
       if ((int32_t)(kt * KT) < bucket_len(jb)) return true;
@@ -110,7 +116,7 @@ __global__ __launch_bounds__(kAttnThreads) void buck_swin_fwd_kernel(
 
   u32x4_t rk[C::NCH], rv[C::NCH];
   auto fetch = [&](uint32_t j, uint32_t t) {
-    const size_t row0 = tok0 + (size_t)my_scope[j] * bs + t * KT;
+    const size_t row0 = tok0 + (size_t)s_bucket[j] * bs + t * KT;
 #pragma unroll
     for (int i = 0; i < C::NCH; ++i) {
       const uint32_t c = tid + i * kAttnThreads;
@@ -194,8 +200,10 @@ __global__ __launch_bounds__(kAttnThreads) void buck_swin_fwd_kernel(
     for (int i = 0; i < C::NSUB * 16; i += 2) {
       const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[i], scale_log2, -m_use));
       const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[i + 1], scale_log2, -m_use));
-      psum += p0 + p1;
       pb[i / 2] = pack_bf16x2(p0, p1);
+      // row sum of the bf16-rounded probabilities (what the PV product sees): one dot2 per pair
+      psum = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, pb[i / 2]),
+                                             __builtin_bit_cast(bf16x2_t, 0x3F803F80u), psum, false);
     }
     l_run = l_run * alpha + psum;
     // the running maximum settles after the first tiles: rescale the accumulators only when some
@@ -250,6 +258,356 @@ __global__ __launch_bounds__(kAttnThreads) void buck_swin_fwd_kernel(
   }
 }
 
+// ---- resident variant ---------------------------------------------------------------------------
+// When a scope holds 256 or 512 tokens and head_dim <= 32 (the shape of every block of the Flash3D
+// model: one 512-row bucket per scope, 32-wide heads) the K and V of a (scope, head) fit in LDS
+// twice.  One persistent workgroup walks a list of (batch, scope, head) items: wave w owns the scope's
+// query rows [32w, 32w+32) and runs them against all key tiles without any barrier, while the NEXT
+// item's K / V stream from HBM straight into the other LDS buffer (global_load ... lds, no registers)
+// and its Q into eight registers.  One barrier per item.
+//
+// LDS layout of one buffer: K [T][D] then V [T][D], both row-major exactly as the direct loads write
+// them (a wave's 64 lanes fill 1 KB = 1024/(2D) consecutive rows).  K rows carry no padding: the
+// 16-byte chunk c of row r is stored at position c ^ swz(r), swz(r) = (r / (128/D)) mod (D/8), which
+// spreads the 32 rows of a ds_read_b128 over all banks.  V is read with ds_read_b64_tr_b16, which hands
+// lane i of a 16-lane block column i%4 of the four 8-byte pieces addressed by lanes i/4 + {0,4,8,12}:
+// with lane r pointing at key r/4, features 4(r%4).., a lane receives one feature of four consecutive
+// keys, i.e. the MFMA A operand of V^T, with no transposed copy of V anywhere.
+//
+// The softmax reference m_ref of a query row is subtracted INSIDE the score MFMA: Q is pre-multiplied
+// by log2(e)/sqrt(D) (one bf16 rounding) and one extra k-step multiplies a column of ones (key side) by
+// -m_ref (query side), so the accumulator leaves the matrix core as the exponent and the VALU only
+// exponentiates.  Softmax is shift-invariant, so m_ref need not be the running maximum: it is set from
+// the first tile with a valid key and moved only when a tile's row sum would pass 2^60, which keeps
+// every value far inside fp32 / bf16 range.  m_ref is kept bf16-representable, so the shift is exact.
+constexpr int kResMaxScope = 8;  // buckets per scope the LDS tables hold
+typedef short i16x4_t __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) void lds_void_t;
+typedef __attribute__((address_space(3))) i16x4_t lds_i16x4_t;
+
+template <int D, int T>
+constexpr size_t resident_lds_bytes() {
+  return 2 * (size_t)2 * T * D * 2 + 3 * kResMaxScope * 8;
+}
+
+template <int D, int T>
+__global__ __launch_bounds__(2 * T) __attribute__((amdgpu_waves_per_eu(4, 4))) void buck_swin_fwd_resident_kernel(
+    const uint16_t* __restrict__ q, const uint16_t* __restrict__ k, const uint16_t* __restrict__ v, uint32_t ld,
+    uint16_t* __restrict__ o, float* __restrict__ lse, const uint32_t* __restrict__ scope_buckets,
+    uint32_t num_scope, uint32_t scope_size, uint32_t bs, uint32_t seq_len, uint32_t num_head,
+    const int32_t* __restrict__ kv_len, float scale_log2, uint32_t n_items, uint32_t items_per_xcd,
+    uint32_t n_slots) {
+  constexpr int KT = 64;
+  constexpr int KSTEPS = D / 16;
+  constexpr int NSUB = KT / 32;
+  constexpr int CPK = D / 8;               // 16-byte chunks per row
+  constexpr int ROWB = D * 2;              // bytes per K / V row in LDS
+  constexpr int RPB = 1024 / ROWB;         // rows one direct-load instruction fills
+  constexpr int BLK_PER_WAVE = 32 / RPB;   // wave w fills the rows [32w, 32w+32) of K and of V
+  constexpr int SWZ_DIV = 16 / CPK;        // rows sharing one swizzle value
+  constexpr int OPB = T * ROWB;            // bytes of one operand (K or V)
+  constexpr int BUF = 2 * OPB;             // bytes of one K + V buffer
+  constexpr int N_TILES = T / KT;
+  extern __shared__ __attribute__((aligned(16))) char lds_res[];
+  uint32_t (*s_bucket)[kResMaxScope] = reinterpret_cast<uint32_t (*)[kResMaxScope]>(lds_res + 2 * BUF);
+  int32_t (*s_len)[kResMaxScope] = reinterpret_cast<int32_t (*)[kResMaxScope]>(lds_res + 2 * BUF + 3 * kResMaxScope * 4);
+
+  const uint32_t tid = threadIdx.x, wave = tid / kWave, lane = tid % kWave;
+  const uint32_t lq = lane & 31u, half = lane >> 5;
+  const uint32_t n_bucket = seq_len / bs;
+  const uint32_t xcd = blockIdx.x % kNumXcd, slot = blockIdx.x / kNumXcd;
+  const uint32_t item_lo = xcd * items_per_xcd + slot;
+  const uint32_t item_hi = min((xcd + 1) * items_per_xcd, n_items);
+  if (item_lo >= item_hi) return;        // whole workgroup: no barrier has been passed yet
+  const uint32_t my_items = (item_hi - item_lo + n_slots - 1) / n_slots;
+
+  // item -> (batch, scope, head); the element offset of (first token of the batch, head) is uniform, the
+  // per-thread part (row inside the sequence, chunk) fits 32 bits (checked by the host)
+  auto item_scope = [&](uint32_t it) { return (it / num_head) % num_scope; };
+  auto item_base = [&](uint32_t it) {
+    return (size_t)(it / (num_head * num_scope)) * seq_len * ld + (size_t)(it % num_head) * D;
+  };
+
+  // bucket ids / valid lengths of one item's scope, handled by the first scope_size threads
+  uint32_t tb = 0;
+  int32_t tl = 0;
+  auto load_table_ids = [&](uint32_t it) {
+    if (tid < scope_size) tb = scope_buckets[(size_t)item_scope(it) * scope_size + tid];
+  };
+  auto load_table_len = [&]() {
+    if (tid < scope_size) tl = tb >= n_bucket ? 0 : (kv_len ? min(max(kv_len[tb], 0), (int32_t)bs) : (int32_t)bs);
+  };
+  auto store_table = [&](uint32_t tslot) {
+    if (tid < scope_size) {
+      s_bucket[tslot][tid] = tb;
+      s_len[tslot][tid] = tl;
+    }
+  };
+
+  // direct HBM -> LDS loads of one item's K and V rows [32 wave, 32 wave + 32)
+  auto issue_kv = [&](uint32_t it, uint32_t tslot, char* buf) {
+    const size_t base = item_base(it);
+#pragma unroll
+    for (int i = 0; i < BLK_PER_WAVE; ++i) {
+      const uint32_t blk = __builtin_amdgcn_readfirstlane(wave * BLK_PER_WAVE + i);
+      const uint32_t row = blk * RPB + lane / CPK, pos = lane % CPK;
+      const uint32_t j = (blk * RPB) / bs;               // uniform: a block never straddles buckets
+      if (s_len[tslot][j] > 0) {
+        const uint32_t rowoff = ((s_bucket[tslot][j] * bs + (row - j * bs)) * ld) * 2u;
+        const uint32_t ck = pos ^ ((row / SWZ_DIV) & (CPK - 1));
+        __builtin_amdgcn_global_load_lds(reinterpret_cast<const char*>(k + base) + (rowoff + ck * 16u),
+                                         (lds_void_t*)(buf + blk * 1024), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds(reinterpret_cast<const char*>(v + base) + (rowoff + pos * 16u),
+                                         (lds_void_t*)(buf + OPB + blk * 1024), 16, 0, 0);
+      }
+    }
+  };
+  // this wave's 32 query rows sit at scope-local rows [32 wave, 32 wave + 32)
+  const uint32_t q_local = wave * 32;
+  const uint32_t qj = q_local / bs;
+  const uint32_t q_in_bucket = (q_local - qj * bs) + lq;
+  u32x4_t qraw[KSTEPS];
+  auto issue_q = [&](uint32_t it, uint32_t tslot) {
+    const uint32_t qb = s_bucket[tslot][qj];
+    const uint32_t off = (((qb < n_bucket ? qb : 0u) * bs + q_in_bucket) * ld + half * 8) * 2u;
+    const char* qp = reinterpret_cast<const char*>(q + item_base(it));
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) qraw[ks] = *reinterpret_cast<const u32x4_t*>(qp + (off + ks * 32u));
+  };
+
+  // ---- prologue: tables of the first two items, K / V / Q of the first ----
+  load_table_ids(item_lo);
+  load_table_len();
+  store_table(0);
+  if (my_items > 1) {
+    load_table_ids(item_lo + n_slots);
+    load_table_len();
+    store_table(1);
+  }
+  __syncthreads();
+  issue_q(item_lo, 0);
+  issue_kv(item_lo, 0, lds_res);
+  __builtin_amdgcn_s_waitcnt(0);
+  __syncthreads();
+
+  // per-lane LDS byte offsets inside a buffer
+  const uint32_t k_off = lq * ROWB + ((half ^ ((lq / SWZ_DIV) & (CPK - 1))) * 16u);   // k-step ks: ^ (ks * 32)
+  const uint32_t l16 = lane & 15u, d_base = 16u * ((lane >> 4) & 1u);
+  const uint32_t v_off = OPB + (4u * half + l16 / 4u) * ROWB + (d_base + 4u * (l16 & 3u)) * 2u;
+  const bool v_lane = D >= 32 || d_base < (uint32_t)D;   // lanes whose V^T row exists
+
+  const bf16x8_t ones_k = __builtin_bit_cast(bf16x8_t, u32x4_t{half == 0 ? 0x00003F80u : 0u, 0u, 0u, 0u});
+  for (uint32_t n = 0; n < my_items; ++n) {
+    const uint32_t item = item_lo + n * n_slots;
+    const uint32_t tcur = n % 3, tnext = (n + 1) % 3, tnext2 = (n + 2) % 3;
+    const bool has_next = n + 1 < my_items;
+    const char* sbuf = lds_res + (n & 1u) * BUF;
+    const uint32_t q_bucket = s_bucket[tcur][qj];
+    const bool q_exists = q_bucket < n_bucket;             // uniform per wave
+    const uint32_t q_row = (q_exists ? q_bucket : 0u) * bs + q_in_bucket;
+    const int32_t q_valid_len = s_len[tcur][qj];
+
+    // Q of this item arrived during the previous one: scale and round once
+    bf16x8_t qf[KSTEPS];
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) {
+      u32x4_t sc;
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        sc[e] = pack_bf16x2(bf16_lo(qraw[ks][e]) * scale_log2, bf16_hi(qraw[ks][e]) * scale_log2);
+      qf[ks] = __builtin_bit_cast(bf16x8_t, sc);
+    }
+    // put the next item's operands in flight
+    if (has_next) {
+      issue_q(item + n_slots, tnext);
+      issue_kv(item + n_slots, tnext, lds_res + ((n + 1) & 1u) * BUF);
+    }
+    if (n + 2 < my_items) load_table_ids(item + 2 * n_slots);
+
+    bf16x8_t bias_q = __builtin_bit_cast(bf16x8_t, u32x4_t{0u, 0u, 0u, 0u});
+    float m_ref = -INFINITY;
+    f32x16_t acc;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[i] = 0.f;
+    float l_run = 0.f;
+    for (uint32_t t = 0; t < (uint32_t)N_TILES; ++t) {
+      if (t == (uint32_t)(N_TILES / 2) && n + 2 < my_items) load_table_len();
+      const uint32_t key0 = t * KT;
+      const uint32_t jb = key0 / bs;
+      const int32_t in_b = (int32_t)(key0 - jb * bs);
+      const int32_t cur_len = s_len[tcur][jb];
+      if (!q_exists || in_b >= cur_len) continue;   // nothing to do for this wave / tile (uniform)
+      const bool partial = in_b + KT > cur_len;
+      const char* kt = sbuf + key0 * ROWB + k_off;
+      const char* vt = sbuf + key0 * ROWB + v_off;
+      uint32_t pb[NSUB * 8];
+      float psum = 0.f;
+      bool slow = __ballot(m_ref == -INFINITY) != 0;   // some row has no reference yet
+      if (!slow) {
+        float s[NSUB * 16];
+#pragma unroll
+        for (int j = 0; j < NSUB; ++j) {
+          f32x16_t sacc;
+#pragma unroll
+          for (int i = 0; i < 16; ++i) sacc[i] = 0.f;
+          sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ones_k, bias_q, sacc, 0, 0, 0);
+#pragma unroll
+          for (int ks = 0; ks < KSTEPS; ++ks) {
+            const bf16x8_t kf = *reinterpret_cast<const bf16x8_t*>(kt + j * 32 * ROWB + ((k_off ^ (ks * 32u)) - k_off));
+            sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[ks], sacc, 0, 0, 0);
+          }
+#pragma unroll
+          for (int i = 0; i < 16; ++i) s[j * 16 + i] = sacc[i];
+        }
+        if (partial) {
+#pragma unroll
+          for (int j = 0; j < NSUB; ++j)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+              const int32_t key = in_b + j * 32 + (i / 4) * 8 + half * 4 + (i % 4);
+              if (key >= cur_len) s[j * 16 + i] = -INFINITY;
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < NSUB * 16; i += 2) {
+          pb[i / 2] = pack_bf16x2(__builtin_amdgcn_exp2f(s[i]), __builtin_amdgcn_exp2f(s[i + 1]));
+          psum = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, pb[i / 2]),
+                                                 __builtin_bit_cast(bf16x2_t, 0x3F803F80u), psum, false);
+        }
+        slow = __ballot(!(psum < 0x1p60f)) != 0;       // also catches inf / nan
+      }
+      if (slow) {
+        // (re)compute the tile against a fresh reference
+        float s[NSUB * 16];
+#pragma unroll
+        for (int j = 0; j < NSUB; ++j) {
+          f32x16_t sacc;
+#pragma unroll
+          for (int i = 0; i < 16; ++i) sacc[i] = 0.f;
+#pragma unroll
+          for (int ks = 0; ks < KSTEPS; ++ks) {
+            const bf16x8_t kf = *reinterpret_cast<const bf16x8_t*>(kt + j * 32 * ROWB + ((k_off ^ (ks * 32u)) - k_off));
+            sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[ks], sacc, 0, 0, 0);
+          }
+#pragma unroll
+          for (int i = 0; i < 16; ++i) s[j * 16 + i] = sacc[i];
+        }
+        if (partial) {
+#pragma unroll
+          for (int j = 0; j < NSUB; ++j)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+              const int32_t key = in_b + j * 32 + (i / 4) * 8 + half * 4 + (i % 4);
+              if (key >= cur_len) s[j * 16 + i] = -INFINITY;
+            }
+        }
+        float mx = s[0];
+#pragma unroll
+        for (int i = 1; i < NSUB * 16; ++i) mx = fmaxf(mx, s[i]);
+        mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
+        // the candidate is rounded to bf16 (it may land a hair below the true maximum: harmless)
+        const float m_cand =
+            mx == -INFINITY ? mx : __builtin_bit_cast(float, (uint32_t)float_to_bf16_bits(mx) << 16);
+        const float m_new = fmaxf(m_ref, m_cand);
+        const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+        const float alpha = __builtin_amdgcn_exp2f(m_ref - m_use);
+        m_ref = m_new;
+        const uint32_t neg_bits = (__builtin_bit_cast(uint32_t, m_use) >> 16) ^ 0x8000u;
+        bias_q = __builtin_bit_cast(bf16x8_t, u32x4_t{half == 0 ? neg_bits : 0u, 0u, 0u, 0u});
+        l_run *= alpha;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[i] *= alpha;
+        psum = 0.f;
+#pragma unroll
+        for (int i = 0; i < NSUB * 16; i += 2) {
+          pb[i / 2] = pack_bf16x2(__builtin_amdgcn_exp2f(s[i] - m_use), __builtin_amdgcn_exp2f(s[i + 1] - m_use));
+          psum = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, pb[i / 2]),
+                                                 __builtin_bit_cast(bf16x2_t, 0x3F803F80u), psum, false);
+        }
+      }
+      l_run += psum;
+#pragma unroll
+      for (int j = 0; j < NSUB; ++j)
+#pragma unroll
+        for (int kk = 0; kk < 2; ++kk) {
+          u32x4_t praw = {pb[j * 8 + kk * 4 + 0], pb[j * 8 + kk * 4 + 1], pb[j * 8 + kk * 4 + 2],
+                          pb[j * 8 + kk * 4 + 3]};
+          const bf16x8_t pfrag = __builtin_bit_cast(bf16x8_t, praw);
+          // slots 0..3 of this lane: keys 16kk + 4 half + 0..3, slots 4..7: the same + 8
+          i16x4_t lo = {0, 0, 0, 0}, hi = {0, 0, 0, 0};
+          if (v_lane) {
+            lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_t*)(vt + (j * 32 + kk * 16) * ROWB));
+            hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_t*)(vt + (j * 32 + kk * 16 + 8) * ROWB));
+          }
+          const bf16x8_t vf = __builtin_bit_cast(bf16x8_t, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+          acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pfrag, acc, 0, 0, 0);
+        }
+    }
+    // This wave's direct loads (issued a whole item ago) must have landed before the barrier below;
+    // wait for them BEFORE the output stores are issued, so that the stores stay fire-and-forget
+    // (vmcnt = 0, other counters untouched).
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+    if (q_exists) {   // a scope entry outside the sequence names no rows
+      const float l_tot = l_run + __shfl_xor(l_run, 32, kWave);
+      const bool row_ok = (int32_t)q_in_bucket < q_valid_len && l_tot > 0.f;
+      const float inv = row_ok ? 1.0f / l_tot : 0.f;
+      // uniform 64-bit base of (batch element, head) + 32-bit lane offset
+      const size_t obase = (size_t)(item / (num_head * num_scope)) * seq_len * num_head + item % num_head;
+      char* op = reinterpret_cast<char*>(o + obase * D);
+      const uint32_t orow_b = q_row * num_head * D * 2u;
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const uint32_t d0 = g * 8 + half * 4;
+        if (D >= 32 || d0 < (uint32_t)D) {
+          uint2 w;
+          w.x = pack_bf16x2(acc[g * 4 + 0] * inv, acc[g * 4 + 1] * inv);
+          w.y = pack_bf16x2(acc[g * 4 + 2] * inv, acc[g * 4 + 3] * inv);
+          *reinterpret_cast<uint2*>(op + (orow_b + d0 * 2u)) = w;
+        }
+      }
+      if (half == 0) {
+        const float ln2 = 0.69314718055994530942f;
+        *reinterpret_cast<float*>(reinterpret_cast<char*>(lse + obase) + q_row * num_head * 4u) =
+            row_ok ? (m_ref + __builtin_amdgcn_logf(l_tot)) * ln2 : 0.f;
+      }
+    }
+    if (n + 2 < my_items) store_table(tnext2);
+    __syncthreads();   // next buffer is complete; this buffer is free for the item after next
+  }
+}
+
+template <int D, int T>
+static int launch_attn_resident(const uint16_t* q, const uint16_t* k, const uint16_t* v, uint32_t ld, uint16_t* o,
+                                float* lse, const uint32_t* scope_buckets, uint32_t num_scope, uint32_t scope_size,
+                                uint32_t bs, uint32_t batch, uint32_t seq_len, uint32_t num_head,
+                                const int32_t* kv_len, int device, hipStream_t s) {
+  const uint64_t n_items64 = (uint64_t)batch * num_scope * num_head;
+  if (n_items64 == 0) return F3D_OK;
+  if (n_items64 > 0x7FFFFFF0ull) {
+    set_error("attention problem too large for one launch (%llu items)", (unsigned long long)n_items64);
+    return F3D_ERR_INVALID;
+  }
+  const uint32_t n_items = (uint32_t)n_items64;
+  int n_cu = 0;
+  F3D_CHECK_HIP(hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, device));
+  constexpr size_t lds = resident_lds_bytes<D, T>();
+  const uint32_t wg_per_cu = (2 * T <= 512 && 2 * lds <= 160 * 1024) ? 2u : 1u;
+  // workgroups: a multiple of the XCD count, no more than the chip holds at once, no more than items need
+  const uint32_t items_per_xcd = cdiv_u32(n_items, kNumXcd);
+  const uint32_t n_slots = std::max(1u, std::min((uint32_t)n_cu * wg_per_cu / kNumXcd, items_per_xcd));
+  const float scale_log2 = 1.4426950408889634f / sqrtf((float)D);
+  static bool attr_set[64] = {};   // raise the dynamic LDS limit once per instantiation and device
+  if (device < 0 || device >= 64 || !attr_set[device]) {
+    F3D_CHECK_HIP(hipFuncSetAttribute((const void*)buck_swin_fwd_resident_kernel<D, T>,
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    if (device >= 0 && device < 64) attr_set[device] = true;
+  }
+  hipLaunchKernelGGL((buck_swin_fwd_resident_kernel<D, T>), dim3(n_slots * kNumXcd), dim3(2 * T), lds, s, q, k, v, ld,
+                     o, lse, scope_buckets, num_scope, scope_size, bs, seq_len, num_head, kv_len, scale_log2, n_items,
+                     items_per_xcd, n_slots);
+  return F3D_OK;
+}
+
 template <int D, int KT>
 static int launch_attn(const uint16_t* q, const uint16_t* k, const uint16_t* v, uint32_t ld, uint16_t* o, float* lse,
                        const uint32_t* scope_buckets, uint32_t num_scope, uint32_t scope_size, uint32_t bs,
@@ -264,7 +622,8 @@ static int launch_attn(const uint16_t* q, const uint16_t* k, const uint16_t* v, 
   const uint32_t n_work = (uint32_t)n_work64;
   const uint32_t per_xcd = cdiv_u32(n_work, kNumXcd);
   const float scale_log2 = 1.4426950408889634f / sqrtf((float)D);
-  hipLaunchKernelGGL((buck_swin_fwd_kernel<D, KT>), dim3(per_xcd * kNumXcd), dim3(kAttnThreads), C::LDS_BYTES, s, q, k,
+  hipLaunchKernelGGL((buck_swin_fwd_kernel<D, KT>), dim3(per_xcd * kNumXcd), dim3(kAttnThreads),
+                     C::LDS_BYTES + scope_size * 8, s, q, k,
                      v, ld, o, lse, scope_buckets, num_scope, scope_size, bs, seq_len, num_head, kv_len, scale_log2,
                      n_work, per_xcd);
   return F3D_OK;
@@ -284,6 +643,7 @@ int f3d_buck_swin_fwd_strided(const f3d_bf16_t* q, const f3d_bf16_t* k, const f3
                 "No kernel found for head_dim=%u (supported: 16, 32, 64, 128)", head_dim);
   F3D_CHECK_ARG(bucket_size >= 128 && bucket_size % 128 == 0, "bucket_size=%u must be a multiple of 128",
                 bucket_size);
+  F3D_CHECK_ARG(scope_size >= 1 && scope_size <= 8192, "scope_size=%u outside [1, 8192]", scope_size);
   F3D_CHECK_ARG(seq_len % bucket_size == 0, "sequence length %u is not a multiple of bucket_size=%u", seq_len,
                 bucket_size);
   F3D_CHECK_ARG(qkv_row_stride >= num_head * head_dim && qkv_row_stride % 8 == 0,
@@ -296,6 +656,23 @@ int f3d_buck_swin_fwd_strided(const f3d_bf16_t* q, const f3d_bf16_t* k, const f3
   hipStream_t s = (hipStream_t)stream;
   SyncBracket sync(s);
   int rc;
+  // scopes of 256 or 512 tokens with narrow heads: K / V resident in LDS, persistent workgroups
+  const uint32_t scope_tokens = scope_size * bucket_size;
+  if (head_dim <= 32 && scope_size <= (uint32_t)kResMaxScope && (scope_tokens == 256 || scope_tokens == 512) &&
+      (uint64_t)seq_len * qkv_row_stride * 2 < (1ull << 32)) {
+#define F3D_RES(DD, TT)                                                                                         \
+  rc = launch_attn_resident<DD, TT>(q, k, v, qkv_row_stride, o, lse, scope_buckets, num_scope, scope_size,      \
+                                    bucket_size, batch, seq_len, num_head, kv_len, device, s)
+    if (head_dim == 16) {
+      if (scope_tokens == 256) F3D_RES(16, 256); else F3D_RES(16, 512);
+    } else {
+      if (scope_tokens == 256) F3D_RES(32, 256); else F3D_RES(32, 512);
+    }
+#undef F3D_RES
+    if (rc != F3D_OK) return rc;
+    F3D_CHECK_HIP(hipGetLastError());
+    return F3D_OK;
+  }
 #define F3D_ATTN(DD, KK)                                                                                            \
   rc = launch_attn<DD, KK>(q, k, v, qkv_row_stride, o, lse, scope_buckets, num_scope, scope_size, bucket_size, batch, \
                            seq_len, num_head, kv_len, s)
