@@ -14,6 +14,7 @@
 // accumulator layout yields; V is staged in that same order).  Softmax runs in the exp2 domain with
 // fp32 accumulation.  Workgroup ids are remapped so that the workgroups of one scope (which share
 // K/V and the 512-byte token rows) land on the same XCD and its L2.
+#include <type_traits>
 #include "f3d_device.h"
 #include "f3d_internal.h"
 
@@ -274,16 +275,28 @@ __global__ __launch_bounds__(kAttnThreads) void buck_swin_fwd_kernel(
 // with lane r pointing at key r/4, features 4(r%4).., a lane receives one feature of four consecutive
 // keys, i.e. the MFMA A operand of V^T, with no transposed copy of V anywhere.
 //
-// The softmax reference m_ref of a query row is subtracted INSIDE the score MFMA: Q is pre-multiplied
-// by log2(e)/sqrt(D) (one bf16 rounding) and one extra k-step multiplies a column of ones (key side) by
-// -m_ref (query side), so the accumulator leaves the matrix core as the exponent and the VALU only
-// exponentiates.  Softmax is shift-invariant, so m_ref need not be the running maximum: it is set from
-// the first tile with a valid key and moved only when a tile's row sum would pass 2^60, which keeps
-// every value far inside fp32 / bf16 range.  m_ref is kept bf16-representable, so the shift is exact.
-constexpr int kResMaxScope = 8;  // buckets per scope the LDS tables hold
+// Softmax without a running maximum (fast pass): Q is pre-multiplied by log2(e)/sqrt(D) (one bf16
+// rounding), so the score MFMA emits exponents and the VALU only exponentiates: P = 2^S with the
+// reference fixed at zero.  Softmax is shift-invariant and fp32 / bf16 share an 8-bit exponent, so this
+// is exact as long as the numbers stay in range; a wave whose step row sum reaches 2^24, or whose total
+// row sum stays under 2^-24 (scores that large also magnify the rounding of the pre-scaled Q), redoes
+// its item with the general pass: unscaled Q, scale applied in fp32, running maximum, masks.  Items with
+// masked or missing keys always take the general pass.
+constexpr int kResMaxScope = 4;  // buckets per scope: at most 512 tokens in buckets of at least 128
 typedef short i16x4_t __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) void lds_void_t;
 typedef __attribute__((address_space(3))) i16x4_t lds_i16x4_t;
+
+// 16 bytes per lane from global memory straight into LDS: lane l of the wave lands at lds + 16 l.
+// gbase and lds are wave-uniform, voff is the lane's byte offset from gbase.
+__device__ __forceinline__ void lds_dma16(const void* gbase, uint32_t voff, const char* lds) {
+  const uint32_t lds_addr =
+      __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(__attribute__((address_space(3))) const char*)lds);
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+               :
+               : "s"(lds_addr), "v"(voff), "s"(gbase)
+               : "memory", "m0");
+}
 
 template <int D, int T>
 constexpr size_t resident_lds_bytes() {
@@ -355,10 +368,11 @@ __global__ __launch_bounds__(2 * T) __attribute__((amdgpu_waves_per_eu(4, 4))) v
       if (s_len[tslot][j] > 0) {
         const uint32_t rowoff = ((s_bucket[tslot][j] * bs + (row - j * bs)) * ld) * 2u;
         const uint32_t ck = pos ^ ((row / SWZ_DIV) & (CPK - 1));
-        __builtin_amdgcn_global_load_lds(reinterpret_cast<const char*>(k + base) + (rowoff + ck * 16u),
-                                         (lds_void_t*)(buf + blk * 1024), 16, 0, 0);
-        __builtin_amdgcn_global_load_lds(reinterpret_cast<const char*>(v + base) + (rowoff + pos * 16u),
-                                         (lds_void_t*)(buf + OPB + blk * 1024), 16, 0, 0);
+        // Issued as inline assembly on purpose: the compiler then keeps no record of LDS writes in
+        // flight and does not put a full vmcnt wait in front of the tile loop's LDS reads (they read the
+        // OTHER buffer).  The wait that matters is the explicit one before the per-item barrier.
+        lds_dma16(k + base, rowoff + ck * 16u, buf + blk * 1024);
+        lds_dma16(v + base, rowoff + pos * 16u, buf + OPB + blk * 1024);
       }
     }
   };
@@ -396,7 +410,6 @@ __global__ __launch_bounds__(2 * T) __attribute__((amdgpu_waves_per_eu(4, 4))) v
   const uint32_t v_off = OPB + (4u * half + l16 / 4u) * ROWB + (d_base + 4u * (l16 & 3u)) * 2u;
   const bool v_lane = D >= 32 || d_base < (uint32_t)D;   // lanes whose V^T row exists
 
-  const bf16x8_t ones_k = __builtin_bit_cast(bf16x8_t, u32x4_t{half == 0 ? 0x00003F80u : 0u, 0u, 0u, 0u});
   for (uint32_t n = 0; n < my_items; ++n) {
     const uint32_t item = item_lo + n * n_slots;
     const uint32_t tcur = n % 3, tnext = (n + 1) % 3, tnext2 = (n + 2) % 3;
@@ -423,126 +436,189 @@ __global__ __launch_bounds__(2 * T) __attribute__((amdgpu_waves_per_eu(4, 4))) v
       issue_kv(item + n_slots, tnext, lds_res + ((n + 1) & 1u) * BUF);
     }
     if (n + 2 < my_items) load_table_ids(item + 2 * n_slots);
+    // valid key counts of the (at most four) buckets of this scope, as wave-uniform scalars
+    static_assert(kResMaxScope == 4, "four bucket lengths are kept in scalars");
+    const int32_t blen0 = __builtin_amdgcn_readfirstlane(s_len[tcur][0]);
+    const int32_t blen1 = __builtin_amdgcn_readfirstlane(scope_size > 1 ? s_len[tcur][1] : 0);
+    const int32_t blen2 = __builtin_amdgcn_readfirstlane(scope_size > 2 ? s_len[tcur][2] : 0);
+    const int32_t blen3 = __builtin_amdgcn_readfirstlane(scope_size > 3 ? s_len[tcur][3] : 0);
 
-    bf16x8_t bias_q = __builtin_bit_cast(bf16x8_t, u32x4_t{0u, 0u, 0u, 0u});
-    float m_ref = -INFINITY;
+    float m_ref = 0.f;        // reference subtracted from the scaled scores
     f32x16_t acc;
-#pragma unroll
-    for (int i = 0; i < 16; ++i) acc[i] = 0.f;
     float l_run = 0.f;
-    for (uint32_t t = 0; t < (uint32_t)N_TILES; ++t) {
-      if (t == (uint32_t)(N_TILES / 2) && n + 2 < my_items) load_table_len();
-      const uint32_t key0 = t * KT;
-      const uint32_t jb = key0 / bs;
-      const int32_t in_b = (int32_t)(key0 - jb * bs);
-      const int32_t cur_len = s_len[tcur][jb];
-      if (!q_exists || in_b >= cur_len) continue;   // nothing to do for this wave / tile (uniform)
-      const bool partial = in_b + KT > cur_len;
-      const char* kt = sbuf + key0 * ROWB + k_off;
-      const char* vt = sbuf + key0 * ROWB + v_off;
-      uint32_t pb[NSUB * 8];
-      float psum = 0.f;
-      bool slow = __ballot(m_ref == -INFINITY) != 0;   // some row has no reference yet
-      if (!slow) {
-        float s[NSUB * 16];
+    constexpr uint32_t NSTEP = T / 32, QSTEP = NSTEP / 4;
+
+    // scores of one step: S^T[key][query] = K Q'^T (already in the exponent's units)
+    auto qk = [&](uint32_t st) {
+      f32x16_t sacc;
 #pragma unroll
-        for (int j = 0; j < NSUB; ++j) {
-          f32x16_t sacc;
+      for (int i = 0; i < 16; ++i) sacc[i] = 0.f;
+      const char* kt = sbuf + st * 32u * ROWB;
 #pragma unroll
-          for (int i = 0; i < 16; ++i) sacc[i] = 0.f;
-          sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ones_k, bias_q, sacc, 0, 0, 0);
-#pragma unroll
-          for (int ks = 0; ks < KSTEPS; ++ks) {
-            const bf16x8_t kf = *reinterpret_cast<const bf16x8_t*>(kt + j * 32 * ROWB + ((k_off ^ (ks * 32u)) - k_off));
-            sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[ks], sacc, 0, 0, 0);
-          }
-#pragma unroll
-          for (int i = 0; i < 16; ++i) s[j * 16 + i] = sacc[i];
-        }
-        if (partial) {
-#pragma unroll
-          for (int j = 0; j < NSUB; ++j)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) {
-              const int32_t key = in_b + j * 32 + (i / 4) * 8 + half * 4 + (i % 4);
-              if (key >= cur_len) s[j * 16 + i] = -INFINITY;
-            }
-        }
-#pragma unroll
-        for (int i = 0; i < NSUB * 16; i += 2) {
-          pb[i / 2] = pack_bf16x2(__builtin_amdgcn_exp2f(s[i]), __builtin_amdgcn_exp2f(s[i + 1]));
-          psum = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, pb[i / 2]),
-                                                 __builtin_bit_cast(bf16x2_t, 0x3F803F80u), psum, false);
-        }
-        slow = __ballot(!(psum < 0x1p60f)) != 0;       // also catches inf / nan
+      for (int ks = 0; ks < KSTEPS; ++ks) {
+        const bf16x8_t kf = *reinterpret_cast<const bf16x8_t*>(kt + (k_off ^ (ks * 32u)));
+        sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[ks], sacc, 0, 0, 0);
       }
-      if (slow) {
-        // (re)compute the tile against a fresh reference
-        float s[NSUB * 16];
+      return sacc;
+    };
+    // V^T operand of a step: slots 0..3 of a lane are keys 16kk + 4 half + 0..3, slots 4..7 the same + 8
+    auto load_v = [&](uint32_t st, bf16x8_t (&vf)[2]) {
+      const char* vt = sbuf + st * 32u * ROWB + v_off;
 #pragma unroll
-        for (int j = 0; j < NSUB; ++j) {
-          f32x16_t sacc;
-#pragma unroll
-          for (int i = 0; i < 16; ++i) sacc[i] = 0.f;
-#pragma unroll
-          for (int ks = 0; ks < KSTEPS; ++ks) {
-            const bf16x8_t kf = *reinterpret_cast<const bf16x8_t*>(kt + j * 32 * ROWB + ((k_off ^ (ks * 32u)) - k_off));
-            sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[ks], sacc, 0, 0, 0);
-          }
-#pragma unroll
-          for (int i = 0; i < 16; ++i) s[j * 16 + i] = sacc[i];
+      for (int kk = 0; kk < 2; ++kk) {
+        i16x4_t lo = {0, 0, 0, 0}, hi = {0, 0, 0, 0};
+        if (v_lane) {
+          lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_t*)(vt + (kk * 16) * ROWB));
+          hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_t*)(vt + (kk * 16 + 8) * ROWB));
         }
-        if (partial) {
+        vf[kk] = __builtin_bit_cast(bf16x8_t, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+      }
+    };
+    // P = 2^S as bf16 pairs, row sum from the rounded values
+    auto exp_pack = [&](const f32x16_t& sc, uint32_t (&pb)[8], float& psum) {
+      psum = 0.f;
 #pragma unroll
-          for (int j = 0; j < NSUB; ++j)
+      for (int i = 0; i < 16; i += 2) {
+        pb[i / 2] = pack_bf16x2(__builtin_amdgcn_exp2f(sc[i]), __builtin_amdgcn_exp2f(sc[i + 1]));
+        psum = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, pb[i / 2]),
+                                               __builtin_bit_cast(bf16x2_t, 0x3F803F80u), psum, false);
+      }
+    };
+    auto pv = [&](const uint32_t (&pb)[8], const bf16x8_t (&vf)[2]) {
 #pragma unroll
-            for (int i = 0; i < 16; ++i) {
-              const int32_t key = in_b + j * 32 + (i / 4) * 8 + half * 4 + (i % 4);
-              if (key >= cur_len) s[j * 16 + i] = -INFINITY;
-            }
+      for (int kk = 0; kk < 2; ++kk) {
+        const u32x4_t praw = {pb[kk * 4 + 0], pb[kk * 4 + 1], pb[kk * 4 + 2], pb[kk * 4 + 3]};
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[kk], __builtin_bit_cast(bf16x8_t, praw), acc, 0, 0, 0);
+      }
+    };
+
+    // ---- fast pass: every key valid, reference fixed at zero ----
+    // One step starts the score MFMAs of step st+1, exponentiates step st on the VALU while they run,
+    // then feeds P V^T of step st to the matrix core.  A row sum at or above 2^24 only raises
+    // `suspect`; the item is then redone by the general pass below.
+    bool suspect = false;
+    auto fast_step = [&](auto next_tag, f32x16_t& s_cur, f32x16_t& s_nxt, uint32_t st) {
+      if (decltype(next_tag)::value) s_nxt = qk(st + 1);
+      bf16x8_t vf[2];
+      load_v(st, vf);
+      uint32_t pb[8];
+      float psum;
+      exp_pack(s_cur, pb, psum);
+      suspect = suspect || !(psum < 0x1p24f);   // also catches inf / nan
+      l_run += psum;
+      pv(pb, vf);
+    };
+    // The SIMD arbiter favours its oldest wave; left alone, that wave finishes its steps early and
+    // idles at the barrier while the youngest runs the tail alone.  Each wave therefore lowers its own
+    // priority as it advances (quarter by quarter), so a wave that is behind is served first.
+    auto quarter_prio = [&](uint32_t qd) {
+      switch (qd) {
+        case 0: __builtin_amdgcn_s_setprio(3); break;
+        case 1: __builtin_amdgcn_s_setprio(2); break;
+        case 2: __builtin_amdgcn_s_setprio(1); break;
+        default: __builtin_amdgcn_s_setprio(0); break;
+      }
+    };
+    auto fast_pass = [&]() {
+      m_ref = 0.f;
+      suspect = false;
+      l_run = 0.f;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[i] = 0.f;
+      f32x16_t s_a = qk(0), s_b;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) s_b[i] = 0.f;
+      for (uint32_t qd = 0; qd < 4; ++qd) {
+        quarter_prio(qd);
+        const uint32_t st_end = (qd + 1) * QSTEP - (qd == 3 ? 2 : 0);
+        for (uint32_t st = qd * QSTEP; st < st_end; st += 2) {
+          fast_step(std::true_type{}, s_a, s_b, st);
+          fast_step(std::true_type{}, s_b, s_a, st + 1);
         }
-        float mx = s[0];
+      }
+      fast_step(std::true_type{}, s_a, s_b, NSTEP - 2);
+      fast_step(std::false_type{}, s_b, s_a, NSTEP - 1);
+      __builtin_amdgcn_s_setprio(3);
+    };
+
+    // ---- general pass: masked keys, running-maximum softmax with the scale applied in fp32 ----
+    // (one step at a time, no overlap; Q is read again because the fast pass only keeps the pre-scaled copy)
+    auto general_pass = [&]() {
+      bf16x8_t qr[KSTEPS];
+      {
+        const uint32_t off = ((q_row * ld) + half * 8) * 2u;
+        const char* qp = reinterpret_cast<const char*>(q + item_base(item));
 #pragma unroll
-        for (int i = 1; i < NSUB * 16; ++i) mx = fmaxf(mx, s[i]);
+        for (int ks = 0; ks < KSTEPS; ++ks) qr[ks] = *reinterpret_cast<const bf16x8_t*>(qp + (off + ks * 32u));
+      }
+      m_ref = -INFINITY;
+      l_run = 0.f;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[i] = 0.f;
+      for (uint32_t st = 0; st < NSTEP; ++st) {
+        // step st covers the 32 keys [32 st, 32 st + 32): position inside its bucket and that bucket's length
+        const uint32_t jb = (st * 32u) / bs;
+        const int32_t in_b = (int32_t)(st * 32u - jb * bs);
+        const int32_t len = jb == 0 ? blen0 : jb == 1 ? blen1 : jb == 2 ? blen2 : blen3;
+        if (in_b >= len) continue;          // no valid key in this step (uniform)
+        f32x16_t sc;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) sc[i] = 0.f;
+        const char* kt = sbuf + st * 32u * ROWB;
+#pragma unroll
+        for (int ks = 0; ks < KSTEPS; ++ks) {
+          const bf16x8_t kf = *reinterpret_cast<const bf16x8_t*>(kt + (k_off ^ (ks * 32u)));
+          sc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qr[ks], sc, 0, 0, 0);
+        }
+        bf16x8_t vf[2];
+        load_v(st, vf);
+        if (in_b + 32 > len) {
+          // register i of a lane is key (i/4)*8 + 4 half + i%4 of the step
+          const int32_t thr = len - in_b - (int32_t)half * 4;
+#pragma unroll
+          for (int i = 0; i < 16; ++i)
+            if ((i / 4) * 8 + (i % 4) >= thr) sc[i] = -INFINITY;
+        }
+        float mx = sc[0];
+#pragma unroll
+        for (int i = 1; i < 16; ++i) mx = fmaxf(mx, sc[i]);
         mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
-        // the candidate is rounded to bf16 (it may land a hair below the true maximum: harmless)
-        const float m_cand =
-            mx == -INFINITY ? mx : __builtin_bit_cast(float, (uint32_t)float_to_bf16_bits(mx) << 16);
-        const float m_new = fmaxf(m_ref, m_cand);
+        const float m_new = fmaxf(m_ref, mx * scale_log2);
         const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
         const float alpha = __builtin_amdgcn_exp2f(m_ref - m_use);
         m_ref = m_new;
-        const uint32_t neg_bits = (__builtin_bit_cast(uint32_t, m_use) >> 16) ^ 0x8000u;
-        bias_q = __builtin_bit_cast(bf16x8_t, u32x4_t{half == 0 ? neg_bits : 0u, 0u, 0u, 0u});
-        l_run *= alpha;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) sc[i] = __builtin_fmaf(sc[i], scale_log2, -m_use);
+        uint32_t pb[8];
+        float psum;
+        exp_pack(sc, pb, psum);
+        l_run = l_run * alpha + psum;
 #pragma unroll
         for (int i = 0; i < 16; ++i) acc[i] *= alpha;
-        psum = 0.f;
-#pragma unroll
-        for (int i = 0; i < NSUB * 16; i += 2) {
-          pb[i / 2] = pack_bf16x2(__builtin_amdgcn_exp2f(s[i] - m_use), __builtin_amdgcn_exp2f(s[i + 1] - m_use));
-          psum = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, pb[i / 2]),
-                                                 __builtin_bit_cast(bf16x2_t, 0x3F803F80u), psum, false);
-        }
+        pv(pb, vf);
       }
-      l_run += psum;
+      if (m_ref == -INFINITY) m_ref = 0.f;
+    };
+
+    const bool any_valid = blen0 > 0 || blen1 > 0 || blen2 > 0 || blen3 > 0;
+    const bool all_full = blen0 == (int32_t)bs && (scope_size < 2 || blen1 == (int32_t)bs) &&
+                          (scope_size < 3 || blen2 == (int32_t)bs) && (scope_size < 4 || blen3 == (int32_t)bs);
+    if (q_exists && any_valid) {
+      bool redo = !all_full;
+      if (all_full) {
+        fast_pass();
+        // redo with a moving reference if any row sum left the safe range
+        const float l_chk = l_run + __shfl_xor(l_run, 32, kWave);
+        redo = __ballot(suspect || !(l_chk > 0x1p-24f)) != 0;
+      }
+      if (redo) general_pass();
+    } else {
+      l_run = 0.f;
 #pragma unroll
-      for (int j = 0; j < NSUB; ++j)
-#pragma unroll
-        for (int kk = 0; kk < 2; ++kk) {
-          u32x4_t praw = {pb[j * 8 + kk * 4 + 0], pb[j * 8 + kk * 4 + 1], pb[j * 8 + kk * 4 + 2],
-                          pb[j * 8 + kk * 4 + 3]};
-          const bf16x8_t pfrag = __builtin_bit_cast(bf16x8_t, praw);
-          // slots 0..3 of this lane: keys 16kk + 4 half + 0..3, slots 4..7: the same + 8
-          i16x4_t lo = {0, 0, 0, 0}, hi = {0, 0, 0, 0};
-          if (v_lane) {
-            lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_t*)(vt + (j * 32 + kk * 16) * ROWB));
-            hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_t*)(vt + (j * 32 + kk * 16 + 8) * ROWB));
-          }
-          const bf16x8_t vf = __builtin_bit_cast(bf16x8_t, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
-          acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pfrag, acc, 0, 0, 0);
-        }
+      for (int i = 0; i < 16; ++i) acc[i] = 0.f;
     }
+    const float m_run = m_ref;
+    if (n + 2 < my_items) load_table_len();
     // This wave's direct loads (issued a whole item ago) must have landed before the barrier below;
     // wait for them BEFORE the output stores are issued, so that the stores stay fire-and-forget
     // (vmcnt = 0, other counters untouched).
@@ -568,7 +644,7 @@ __global__ __launch_bounds__(2 * T) __attribute__((amdgpu_waves_per_eu(4, 4))) v
       if (half == 0) {
         const float ln2 = 0.69314718055994530942f;
         *reinterpret_cast<float*>(reinterpret_cast<char*>(lse + obase) + q_row * num_head * 4u) =
-            row_ok ? (m_ref + __builtin_amdgcn_logf(l_tot)) * ln2 : 0.f;
+            row_ok ? (m_run + __builtin_amdgcn_logf(l_tot)) * ln2 : 0.f;
       }
     }
     if (n + 2 < my_items) store_table(tnext2);

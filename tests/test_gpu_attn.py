@@ -119,6 +119,36 @@ def test_padding_masks_extension(oracle):
     assert (O - o_ref).abs().max() <= TOL and (LSE - lse_ref).abs().max() <= TOL
 
 
+@pytest.mark.parametrize("D,bs,scope_size", [(32, 512, 1), (16, 256, 2), (32, 128, 2)])
+@pytest.mark.parametrize("kind", ["huge", "tiny", "ramp"])
+def test_softmax_range_extremes(oracle, kind, D, bs, scope_size):
+    """Scores far from zero: exponent sums beyond 2^60 ("huge"), below 2^-60 for every key ("tiny"), and a
+    row maximum that keeps growing along the keys ("ramp").  The LDS-resident kernel first runs with a
+    fixed softmax reference and must fall back to a moving one for such rows; results follow the oracle."""
+    B, H = 1, 2
+    L = 4 * bs * scope_size
+    g = torch.Generator().manual_seed(99)
+    Q = torch.randn(B, L, H, D, generator=g)
+    K = torch.randn(B, L, H, D, generator=g)
+    V = torch.randn(B, L, H, D, generator=g)
+    if kind == "huge":
+        Q, K = Q * 4.0, K * 4.0
+    elif kind == "tiny":
+        Q = Q.abs() * 0.25 + 3.0
+        K = -(K.abs() * 0.25 + 3.0)
+    else:
+        K = K * torch.linspace(0.1, 6.0, L).view(1, L, 1, 1)
+        Q = Q * 3.0
+    Q, K, V = Q.to(torch.bfloat16), K.to(torch.bfloat16), V.to(torch.bfloat16)
+    scopes = np.arange(L // bs, dtype=np.uint32).reshape(-1, scope_size)
+    O, LSE = _run(Q, K, V, scopes, bs)
+    o_ref, lse_ref = oracle.buck_swin_fwd(Q, K, V, scopes, bs)
+    assert torch.isfinite(O).all() and torch.isfinite(LSE).all()
+    # near one-hot rows: the error is the bf16 rounding of V-sized outputs
+    assert (O - o_ref).abs().max() <= 4e-2
+    assert ((LSE - lse_ref).abs() <= 2e-2 + 4e-3 * lse_ref.abs()).all()
+
+
 def test_c2_full_size_strided_qkv(oracle):
     """BASELINE config 2 at full size: L = 131,072 (2 x 65,536), H = 8, D = 32, bucket 512, scope of 1
     bucket, Q/K/V ~ N(0,1)/sqrt(32) taken as column slices of one [L, 3C] projection output.
