@@ -45,7 +45,8 @@ __device__ __forceinline__ float pair_sum(float v) { return v + __shfl_xor(v, 32
 
 // EPI: 0 = bias only, 1 = runtime activation and / or residual
 template <int K, int MT, bool LN, bool SWIGLU, int EPI>
-__global__ __launch_bounds__(kXsThreads) void xstat_linear_kernel(
+__global__ __launch_bounds__(kXsThreads) __attribute__((amdgpu_waves_per_eu((MT == 1 && K <= 256) ? 2 : 1, (MT == 1 && K <= 256) ? 2 : 1)))
+void xstat_linear_kernel(
     const uint16_t* __restrict__ x, uint32_t ldx, const uint16_t* __restrict__ gamma,
     const uint16_t* __restrict__ beta, float eps, const uint16_t* __restrict__ w,
     const uint16_t* __restrict__ bias, const uint16_t* __restrict__ residual, uint32_t ldr,
@@ -89,24 +90,33 @@ __global__ __launch_bounds__(kXsThreads) void xstat_linear_kernel(
     }
   }
   if (LN) {
+    // Statistics in one sweep over the packed registers (sums of d = x - x0 and d^2, shifted by the
+    // row's first element so that the variance does not cancel), then a second sweep that normalises
+    // in place.  The register fence between the sweeps keeps the compiler from holding all K values of
+    // a row as fp32 across them, which would double the kernel's register footprint.
     float mean[MT], rstd[MT];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
-      float s = 0.f;
-#pragma unroll
-      for (int ks = 0; ks < KS; ++ks)
-#pragma unroll
-        for (int e = 0; e < 8; ++e) s += (float)xf[mt][ks][e];
-      mean[mt] = pair_sum(s) * (1.0f / K);
-      float q = 0.f;
+      const float x0 = __shfl((float)xf[mt][0][0], lq, kWave);   // lane lq (half 0) holds element 0 of row lq
+      float s = 0.f, q = 0.f;
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks)
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
-          const float d = (float)xf[mt][ks][e] - mean[mt];
-          q += d * d;
+          const float d = (float)xf[mt][ks][e] - x0;
+          s += d;
+          q = __builtin_fmaf(d, d, q);
         }
-      rstd[mt] = rsqrtf(pair_sum(q) * (1.0f / K) + eps);
+      const float sm = pair_sum(s) * (1.0f / K);
+      const float var = fmaxf(pair_sum(q) * (1.0f / K) - sm * sm, 0.f);
+      mean[mt] = x0 + sm;
+      rstd[mt] = rsqrtf(var + eps);
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        u32x4_t raw = __builtin_bit_cast(u32x4_t, xf[mt][ks]);
+        asm volatile("" : "+v"(raw));
+        xf[mt][ks] = __builtin_bit_cast(bf16x8_t, raw);
+      }
     }
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
@@ -251,9 +261,6 @@ __global__ __launch_bounds__(kXsThreads) void xstat_linear_kernel(
               t[e] = pack_bf16x2(bf16_lo(t[e]) + bf16_lo(rres[e]), bf16_hi(t[e]) + bf16_hi(rres[e]));
           }
         }
-#ifdef F3D_XS_SKIP_STORE
-        if (t[0] == 0x12345678u)
-#endif
         *reinterpret_cast<u32x4_t*>(y + (size_t)row * ldy + colbase + ch) = t;
       }
     };
