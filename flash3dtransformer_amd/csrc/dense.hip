@@ -345,9 +345,9 @@ __global__ __launch_bounds__(256) void affine_act_kernel(const uint16_t* __restr
   *reinterpret_cast<U16x8*>(y + (size_t)row * C + ch) = o;
 }
 
-bool launch_xstat_linear(const uint16_t* x, uint32_t ldx, const uint16_t* gamma, const uint16_t* beta, float eps,
-                         const uint16_t* w, const uint16_t* bias, const uint16_t* residual, uint32_t ldr, uint16_t* y,
-                         uint32_t ldy, uint32_t M, uint32_t N, uint32_t K, uint32_t act, hipStream_t s);
+int launch_xstat_linear(const uint16_t* x, uint32_t ldx, const uint16_t* gamma, const uint16_t* beta, float eps,
+                        const uint16_t* w, const uint16_t* bias, const uint16_t* residual, uint32_t ldr, uint16_t* y,
+                        uint32_t ldy, uint32_t M, uint32_t N, uint32_t K, uint32_t act, int device, hipStream_t s);
 
 static int launch_gemm(bool b_trans, const uint16_t* x, uint32_t ldx, const uint16_t* w, uint32_t ldw,
                        const uint16_t* bias, const uint16_t* residual, uint32_t ldr, uint16_t* y, uint32_t ldy,
@@ -396,10 +396,9 @@ int f3d_linear_bf16(const f3d_bf16_t* x, uint32_t ldx, const f3d_bf16_t* w, cons
   hipStream_t s = (hipStream_t)stream;
   SyncBracket sync(s);
   // small inner dimensions: row-panel kernel (x read once, w streamed); otherwise the tiled GEMM
-  if (!launch_xstat_linear(x, ldx, nullptr, nullptr, 0.f, w, bias, residual, ldr, y, ldy, m, n, k, act, s)) {
-    int rc = launch_gemm(false, x, ldx, w, k, bias, residual, ldr, y, ldy, m, n, k, act, s);
-    if (rc != F3D_OK) return rc;
-  }
+  int rc = launch_xstat_linear(x, ldx, nullptr, nullptr, 0.f, w, bias, residual, ldr, y, ldy, m, n, k, act, device, s);
+  if (rc == F3D_ERR_UNSUPPORTED) rc = launch_gemm(false, x, ldx, w, k, bias, residual, ldr, y, ldy, m, n, k, act, s);
+  if (rc != F3D_OK) return rc;
   F3D_CHECK_HIP(hipGetLastError());
   return F3D_OK;
 }
@@ -424,15 +423,16 @@ int f3d_ln_linear_bf16(const f3d_bf16_t* x, uint32_t ldx, const f3d_bf16_t* gamm
   F3D_CHECK_ARG(guard.ok, "cannot select device %d", device);
   hipStream_t s = (hipStream_t)stream;
   SyncBracket sync(s);
-  if (!launch_xstat_linear(x, ldx, gamma, beta, eps, w, bias, residual, ldr, y, ldy, m, n, k, act, s)) {
+  int rc = launch_xstat_linear(x, ldx, gamma, beta, eps, w, bias, residual, ldr, y, ldy, m, n, k, act, device, s);
+  if (rc == F3D_ERR_UNSUPPORTED) {
     // shape outside the fused kernel: normalise into the per-device workspace, then the tiled GEMM
     uint16_t* tmp = (uint16_t*)workspace(device, (size_t)m * k * sizeof(uint16_t));
     if (!tmp) return F3D_ERR_RUNTIME;
     F3D_CHECK_ARG(ldx == k, "LayerNorm+Linear on a strided input needs an output width that is a multiple of 64");
     launch_layernorm(x, gamma, beta, tmp, m, k, eps, s);
-    int rc = launch_gemm(false, tmp, k, w, k, bias, residual, ldr, y, ldy, m, n, k, act, s);
-    if (rc != F3D_OK) return rc;
+    rc = launch_gemm(false, tmp, k, w, k, bias, residual, ldr, y, ldy, m, n, k, act, s);
   }
+  if (rc != F3D_OK) return rc;
   F3D_CHECK_HIP(hipGetLastError());
   return F3D_OK;
 }

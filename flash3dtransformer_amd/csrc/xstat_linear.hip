@@ -1,18 +1,27 @@
 // Row-panel ("x-stationary") linear layers for gfx950: y = act(LN?(x) wT + bias) (+ residual) for the
-// small inner dimensions of the Flash3D blocks (K = channels, 32..512).
+// small inner dimensions of the Flash3D blocks (K = channels, 32..256).
 //
 // Stands where the reference runs LayerNorm followed by torch.nn.Linear / te.Linear
 // (flash3dxfmr/layers/stage.py:94-97, buck_swin.py:185,194, hourglass.py:99,181-183).
 //
 // Why not an output-tiled GEMM: with K this small a 128x128 tile re-reads 128 KB of operands per
 // 8 MFLOP, which saturates L2 long before the matrix cores.  Here a workgroup owns a panel of
-// 128 * MT rows of x for ALL output columns: every wave keeps its 32 * MT rows, already in the MFMA
-// B-operand layout, in registers for the whole kernel (x is read from HBM exactly once, and because
-// a lane pair holds a complete row the LayerNorm statistics are in-register sums plus one lane
-// exchange), while w streams through LDS in chunks of 64 output features, double buffered, one
-// barrier per chunk.  Each LDS fragment read feeds MT MFMAs.  The product is formed transposed
-// (A = w rows, B = x rows) so a lane owns 4 consecutive output columns of one row for the epilogue
-// (bias, GELU / SiLU / ReLU / swiglu, residual, bf16 store).
+// 32 * MT * WAVES rows of x for ALL output columns: every wave keeps its 32 * MT rows, already in the
+// MFMA B-operand layout, in registers for the whole kernel (x is read from HBM exactly once), while w
+// streams through LDS in chunks of 64 output features.  Each 16-byte LDS fragment read feeds MT MFMAs;
+// with MT = 1 the LDS read port is as busy as the matrix cores, so the large configuration uses MT = 2.
+// The product is formed transposed (A = w rows, B = x rows) so a lane owns 4 consecutive output columns
+// of one row for the epilogue (bias, GELU / SiLU / ReLU / swiglu, residual, bf16 store).
+//
+// w chunks travel HBM/L2 -> LDS directly (global_load ... lds, no staging registers), three buffers deep:
+// chunk c+2 is requested when chunk c starts.  Rows are unpadded; the 16-byte piece p of chunk-row r sits
+// at position p ^ swz(r), which spreads the 32 rows of one fragment read over all banks.
+//
+// LayerNorm is folded algebraically instead of being applied to x:
+//     LN(x) wT + b  =  rstd * (x w'T - mean * wsum) + b',   w' = w * gamma,  wsum[n] = sum_k w'[n][k],
+//                                                            b' = b + w beta.
+// A small kernel prepares w' (bf16), wsum and b' (fp32) per call; the main kernel then only needs the row
+// statistics (one sweep over the registers that hold x) and two fused multiply-adds per output element.
 #include "f3d_device.h"
 #include "f3d_internal.h"
 #include <stdlib.h>
@@ -23,8 +32,9 @@ namespace f3d {
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16_t;
 
-constexpr int kXsThreads = 256;
-constexpr int kXsChunk = 64;  // output features per w chunk (two 32-wide MFMA tiles)
+constexpr int kXsChunk = 64;   // w rows per chunk (two 32-wide MFMA tiles)
+constexpr int kXsBufs = 3;     // w chunk buffers in LDS
+constexpr int kPatchRow = 40;  // epilogue patch: 32 output columns + 8 pad (80-byte pitch keeps 16-byte alignment)
 
 __device__ __forceinline__ float fast_silu(float a) {
   // a * sigmoid(a) with the hardware exp2 / rcp
@@ -43,58 +53,113 @@ __device__ __forceinline__ float xs_act(float v, uint32_t act) {
 // sum over the two lanes (l, l ^ 32) that share a row
 __device__ __forceinline__ float pair_sum(float v) { return v + __shfl_xor(v, 32, kWave); }
 
-// EPI: 0 = bias only, 1 = runtime activation and / or residual
-template <int K, int MT, bool LN, bool SWIGLU, int EPI>
-__global__ __launch_bounds__(kXsThreads) __attribute__((amdgpu_waves_per_eu((MT == 1 && K <= 256) ? 2 : 1, (MT == 1 && K <= 256) ? 2 : 1)))
-void xstat_linear_kernel(
-    const uint16_t* __restrict__ x, uint32_t ldx, const uint16_t* __restrict__ gamma,
-    const uint16_t* __restrict__ beta, float eps, const uint16_t* __restrict__ w,
-    const uint16_t* __restrict__ bias, const uint16_t* __restrict__ residual, uint32_t ldr,
-    uint16_t* __restrict__ y, uint32_t ldy, uint32_t M, uint32_t N, uint32_t act) {
+// 16 bytes per lane from global memory straight into LDS: lane l of the wave lands at lds + 16 l.
+// gbase and lds are wave-uniform, voff is the lane's byte offset from gbase.  Inline assembly on
+// purpose: the compiler keeps no record of these loads, so it never guards LDS reads of OTHER buffers
+// with a full vmcnt wait; the waits that matter are written out below.
+__device__ __forceinline__ void xs_lds_dma16(const void* gbase, uint32_t voff, const char* lds) {
+  const uint32_t lds_addr =
+      __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(__attribute__((address_space(3))) const char*)lds);
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+               :
+               : "s"(lds_addr), "v"(voff), "s"(gbase)
+               : "memory", "m0");
+}
+
+// s_waitcnt vmcnt(n) for a small run-time n (the instruction takes an immediate)
+__device__ __forceinline__ void xs_wait_vm(uint32_t n) {
+  switch (n) {
+    case 0: __builtin_amdgcn_s_waitcnt(0x0F70); break;
+    case 1: __builtin_amdgcn_s_waitcnt(0x0F71); break;
+    case 2: __builtin_amdgcn_s_waitcnt(0x0F72); break;
+    case 3: __builtin_amdgcn_s_waitcnt(0x0F73); break;
+    case 4: __builtin_amdgcn_s_waitcnt(0x0F74); break;
+    case 5: __builtin_amdgcn_s_waitcnt(0x0F75); break;
+    case 6: __builtin_amdgcn_s_waitcnt(0x0F76); break;
+    default: __builtin_amdgcn_s_waitcnt(0x0F70); break;
+  }
+}
+
+template <int K>
+struct XsGeom {
+  static constexpr int CPR = K / 8;                       // 16-byte pieces per w row
+  static constexpr int ROWB = K * 2;                      // bytes per w row
+  static constexpr int CHUNK_BYTES = kXsChunk * ROWB;
+  static constexpr int RP = CPR >= 16 ? 1 : 16 / CPR;     // rows sharing one swizzle value
+  static constexpr int SWZ_MASK = (CPR < 16 ? CPR : 16) - 1;
+  static constexpr int N_DMA = CPR;                       // direct-load instructions per chunk (64 pieces each)
+  static constexpr int KP = K < 128 ? K : 128;            // columns per transposition pass of the x prologue
+  __host__ __device__ static constexpr uint32_t swz(uint32_t row) { return (row / RP) & SWZ_MASK; }
+};
+
+template <int K, int WAVES>
+constexpr size_t xs_lds_bytes() {
+  using G = XsGeom<K>;
+  const size_t wbuf = (size_t)kXsBufs * G::CHUNK_BYTES;
+  const size_t xpatch = (size_t)WAVES * 32 * (G::KP + 8) * 2;
+  const size_t front = wbuf > xpatch ? wbuf : xpatch;
+  return front + (size_t)WAVES * 32 * kPatchRow * 2 + (size_t)2 * kXsBufs * kXsChunk * 4;
+}
+
+// EPI: 0 = bias only, 1 = runtime activation and / or residual.
+// With LN the kernel expects w = w', bias = b' (fp32), wsum (fp32) as prepared by ln_fold_kernel.
+template <int K, int MT, int WAVES, bool LN, bool SWIGLU, int EPI>
+__global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2))) void xstat_linear_kernel(
+    const uint16_t* __restrict__ x, uint32_t ldx, float eps, const uint16_t* __restrict__ w,
+    const uint16_t* __restrict__ bias, const float* __restrict__ bias_f, const float* __restrict__ wsum,
+    const uint16_t* __restrict__ residual, uint32_t ldr, uint16_t* __restrict__ y, uint32_t ldy, uint32_t M,
+    uint32_t N, uint32_t act) {
+  using G = XsGeom<K>;
   constexpr int KS = K / 16;             // MFMA k-steps
-  constexpr int WROW = K + 8;            // padded LDS row (elements)
-  constexpr int CHUNK_ELEMS = kXsChunk * WROW;
-  constexpr int CPR = K / 8;             // 16-byte chunks per row
-  constexpr int NLOAD = (kXsChunk * CPR + kXsThreads - 1) / kXsThreads;
-  extern __shared__ __attribute__((aligned(16))) uint16_t lds_xs[];  // 2 x [64][WROW] w chunks
-  __shared__ __attribute__((aligned(16))) float s_bias[2][kXsChunk];
-  constexpr int kPatchRow = 40;  // 32 output columns + 8 pad (80-byte pitch keeps 16-byte alignment)
-  __shared__ __attribute__((aligned(16))) uint16_t lds_patch[4 * 32 * kPatchRow];
+  constexpr int ROWB = G::ROWB;
+  constexpr int NT = 64 * WAVES;
+  constexpr int ROWS_WG = 32 * MT * WAVES;
+  extern __shared__ __attribute__((aligned(1024))) char lds_xs[];
+  constexpr size_t kFront = (size_t)kXsBufs * G::CHUNK_BYTES > (size_t)WAVES * 32 * (G::KP + 8) * 2
+                                ? (size_t)kXsBufs * G::CHUNK_BYTES
+                                : (size_t)WAVES * 32 * (G::KP + 8) * 2;
+  uint16_t* lds_patch = reinterpret_cast<uint16_t*>(lds_xs + kFront);
+  float (*s_bias)[kXsChunk] = reinterpret_cast<float (*)[kXsChunk]>(lds_xs + kFront + (size_t)WAVES * 32 * kPatchRow * 2);
+  float (*s_wsum)[kXsChunk] = s_bias + kXsBufs;
 
-  const uint32_t tid = threadIdx.x, wave = tid / kWave, lane = tid % kWave;
+  const uint32_t tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid / kWave), lane = tid % kWave;
   const uint32_t lq = lane & 31u, half = lane >> 5;
-  const uint32_t row0 = blockIdx.x * (128 * MT) + wave * (32 * MT);
+  const uint32_t row0 = blockIdx.x * ROWS_WG + wave * (32 * MT);
 
-  // ---- this wave's x rows -> registers in the B-operand layout.  Loaded row-contiguously
-  //      (a row is one burst across CPR lanes) and transposed through a wave-private LDS patch ----
+  // ---- this wave's x rows -> registers in the B-operand layout.  Loaded row-contiguously and
+  //      transposed through a wave-private LDS patch, KP columns at a time ----
   bf16x8_t xf[MT][KS];
   {
-    uint16_t* patch = lds_xs + wave * (32 * WROW);   // 4 x 32 x WROW elements fit in one w buffer pair
-    constexpr int RPI = kWave / CPR > 0 ? kWave / CPR : 1;          // rows per load instruction
-    constexpr int LPR = CPR < kWave ? CPR : kWave;                  // lanes per row
-    constexpr int XLOADS = (32 * CPR) / kWave;                      // load instructions per m-tile
+    constexpr int KP = G::KP, PROW = KP + 8, PCPR = KP / 8;
+    uint16_t* patch = reinterpret_cast<uint16_t*>(lds_xs) + wave * (32 * PROW);
+    constexpr int XLOADS = (32 * PCPR) / kWave;
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
+    for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-      for (int i = 0; i < XLOADS; ++i) {
-        const uint32_t id = lane + i * kWave;
-        const uint32_t rr = id / CPR, kc = (id % CPR) * 8;
-        const uint32_t r = min(row0 + mt * 32 + rr, M - 1);
-        const u32x4_t v = *reinterpret_cast<const u32x4_t*>(x + (size_t)r * ldx + kc);
-        *reinterpret_cast<u32x4_t*>(patch + rr * WROW + kc) = v;
+      for (int kp = 0; kp < K / KP; ++kp) {
+        u32x4_t v[XLOADS];
+#pragma unroll
+        for (int i = 0; i < XLOADS; ++i) {
+          const uint32_t id = lane + i * kWave;
+          const uint32_t rr = id / PCPR, kc = (id % PCPR) * 8;
+          const uint32_t r = min(row0 + mt * 32 + rr, M - 1);
+          v[i] = *reinterpret_cast<const u32x4_t*>(x + (size_t)r * ldx + kp * KP + kc);
+        }
+#pragma unroll
+        for (int i = 0; i < XLOADS; ++i) {
+          const uint32_t id = lane + i * kWave;
+          const uint32_t rr = id / PCPR, kc = (id % PCPR) * 8;
+          *reinterpret_cast<u32x4_t*>(patch + rr * PROW + kc) = v[i];
+        }
+#pragma unroll
+        for (int ks = 0; ks < KP / 16; ++ks)
+          xf[mt][kp * (KP / 16) + ks] = *reinterpret_cast<const bf16x8_t*>(patch + lq * PROW + ks * 16 + half * 8);
       }
-      (void)RPI; (void)LPR;
-#pragma unroll
-      for (int ks = 0; ks < KS; ++ks)
-        xf[mt][ks] = *reinterpret_cast<const bf16x8_t*>(patch + lq * WROW + ks * 16 + half * 8);
-    }
   }
+  // LayerNorm statistics of this lane's rows: one sweep, sums of d = x - x0 and d^2, shifted by the row's
+  // first element so that the variance does not cancel
+  float ln_a[MT], ln_b[MT];   // y = ln_a * acc + (ln_b * wsum + bias'),  ln_a = rstd, ln_b = -rstd * mean
   if (LN) {
-    // Statistics in one sweep over the packed registers (sums of d = x - x0 and d^2, shifted by the
-    // row's first element so that the variance does not cancel), then a second sweep that normalises
-    // in place.  The register fence between the sweeps keeps the compiler from holding all K values of
-    // a row as fp32 across them, which would double the kernel's register footprint.
-    float mean[MT], rstd[MT];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
       const float x0 = __shfl((float)xf[mt][0][0], lq, kWave);   // lane lq (half 0) holds element 0 of row lq
@@ -109,94 +174,95 @@ void xstat_linear_kernel(
         }
       const float sm = pair_sum(s) * (1.0f / K);
       const float var = fmaxf(pair_sum(q) * (1.0f / K) - sm * sm, 0.f);
-      mean[mt] = x0 + sm;
-      rstd[mt] = rsqrtf(var + eps);
-#pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        u32x4_t raw = __builtin_bit_cast(u32x4_t, xf[mt][ks]);
-        asm volatile("" : "+v"(raw));
-        xf[mt][ks] = __builtin_bit_cast(bf16x8_t, raw);
-      }
-    }
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-      const bf16x8_t g = *reinterpret_cast<const bf16x8_t*>(gamma + ks * 16 + half * 8);
-      bf16x8_t b;
-      if (beta) b = *reinterpret_cast<const bf16x8_t*>(beta + ks * 16 + half * 8);
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          float v = ((float)xf[mt][ks][e] - mean[mt]) * rstd[mt] * (float)g[e];
-          if (beta) v += (float)b[e];
-          xf[mt][ks][e] = (__bf16)v;  // the normalised activations are bf16, as a separate LayerNorm would emit
-        }
+      ln_a[mt] = rsqrtf(var + eps);
+      ln_b[mt] = -ln_a[mt] * (x0 + sm);
     }
   }
-  __syncthreads();  // the transpose patches are dead; the space now holds w chunks
+  __syncthreads();  // the transposition patches are dead; the space now holds w chunks
 
   // ---- w chunk streaming ----
   const uint32_t n_out = SWIGLU ? N / 2 : N;
   // a swiglu chunk pairs 32 value rows with their 32 gate rows; a plain chunk is 64 consecutive rows
   constexpr uint32_t COLS = SWIGLU ? 32u : (uint32_t)kXsChunk;   // output columns per chunk
-  const uint32_t nchunk = (n_out + COLS - 1) / COLS;
+  const uint32_t nchunk = n_out / COLS;   // the launcher only takes shapes whose chunks are all full
   auto w_row = [&](uint32_t c, uint32_t r) -> uint32_t {  // weight row behind chunk-local row r
     if (!SWIGLU) return c * kXsChunk + r;
     return r < 32 ? c * 32 + r : n_out + c * 32 + (r - 32);
   };
-  // the launcher only takes shapes whose chunks are all full (N % 64 == 0), so no row guard is needed
-  static_assert((kXsChunk * CPR) % kXsThreads == 0, "w chunk must split evenly over the workgroup");
-  // two register sets: chunk c+2 is requested while chunk c is computed, so a w fetch has two chunk
-  // computations to land before it is staged
-  u32x4_t rwA[NLOAD], rwB[NLOAD];
-  float rbA = 0.f, rbB = 0.f;
-  auto fetch = [&](uint32_t c, u32x4_t (&rw)[NLOAD], float& rb) {
+  // direct loads of chunk c into buffer slot: instruction q fills LDS bytes [1024 q, 1024 q + 1024) of the
+  // buffer, i.e. chunk rows [q * 64 / CPR, ...); wave v issues instructions v, v + WAVES, ...
+  constexpr uint32_t kMyDmaMax = (G::N_DMA + WAVES - 1) / WAVES;
+  const uint32_t my_dma = G::N_DMA / WAVES + (wave < (uint32_t)(G::N_DMA % WAVES) ? 1u : 0u);
+  auto dma_chunk = [&](uint32_t c, uint32_t slot) {
+    const char* buf = lds_xs + slot * G::CHUNK_BYTES;
 #pragma unroll
-    for (int i = 0; i < NLOAD; ++i) {
-      const uint32_t id = tid + i * kXsThreads;
-      const uint32_t r = id / CPR, kc = (id % CPR) * 8;
-      rw[i] = *reinterpret_cast<const u32x4_t*>(w + (size_t)w_row(c, r) * K + kc);
+    for (uint32_t i = 0; i < kMyDmaMax; ++i) {
+      const uint32_t qi = wave + i * WAVES;
+      if (qi < (uint32_t)G::N_DMA) {
+        const uint32_t r = (qi * 64u + lane) / G::CPR, p = lane % G::CPR;   // chunk row and position of this lane's piece
+        const uint32_t piece = p ^ G::swz(r);
+        xs_lds_dma16(w, (w_row(c, r) * K + piece * 8u) * 2u, buf + qi * 1024);
+      }
     }
-    if (bias) rb = bf16_bits_to_float(bias[w_row(c, tid & (kXsChunk - 1))]);
   };
-  auto stage = [&](uint32_t c, const u32x4_t (&rw)[NLOAD], float rb) {
-    uint16_t* dst = lds_xs + (c & 1u) * CHUNK_ELEMS;
-#pragma unroll
-    for (int i = 0; i < NLOAD; ++i) {
-      const uint32_t id = tid + i * kXsThreads;
-      const uint32_t r = id / CPR, kc = (id % CPR) * 8;
-      *reinterpret_cast<u32x4_t*>(dst + r * WROW + kc) = rw[i];
+  // bias (and wsum) of a chunk: every wave issues the same loads so that the wait constants below hold
+  // for all of them; wave 0 parks the values in LDS one chunk later
+  float rb = 0.f, rs = 0.f;
+  auto load_bias = [&](uint32_t c) {
+    const uint32_t n = w_row(c, lane);
+    if (LN) {
+      rb = bias_f[n];
+      rs = wsum[n];
+    } else {
+      rb = bias ? bf16_bits_to_float(bias[n]) : 0.f;
     }
-    if (tid < kXsChunk) s_bias[c & 1u][tid] = rb;
+  };
+  auto park_bias = [&](uint32_t slot) {
+    if (wave == 0) {
+      s_bias[slot][lane] = rb;
+      if (LN) s_wsum[slot][lane] = rs;
+    }
   };
 
-  const bool wg_full = (blockIdx.x + 1) * (128 * MT) <= M;
+  const bool wg_full = (blockIdx.x + 1) * ROWS_WG <= M;
   // Workgroups walk the output columns in rotated order: at any moment different workgroups write
   // different column ranges, which spreads the stores over the HBM channels (with a power-of-two row
   // pitch every workgroup would otherwise hit the same channels at the same time).
   const uint32_t c_start = (blockIdx.x * 5u) % nchunk;
   auto actual = [&](uint32_t i) -> uint32_t { const uint32_t t = i + c_start; return t >= nchunk ? t - nchunk : t; };
-  fetch(actual(0), rwA, rbA);
-  if (nchunk > 1) fetch(actual(1), rwB, rbB);
-  stage(0, rwA, rbA);
-  if (nchunk > 2) fetch(actual(2), rwA, rbA);
+
+  dma_chunk(actual(0), 0);
+  if (nchunk > 1) dma_chunk(actual(1), 1);
+  load_bias(actual(0));
+  park_bias(0);
+  if (nchunk > 1) load_bias(actual(1));
+  __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): the first two chunks have landed
   __syncthreads();
-  // Order inside one step: MFMAs of chunk ci -> stage chunk ci+1 into the other LDS buffer -> request
-  // chunk ci+3 into the register set just freed -> epilogue stores of chunk ci -> barrier.  The stores
-  // are the youngest memory operations when the step ends, so nothing waits on them until a whole
-  // chunk of MFMA work later.
-  auto chunk_body = [&](auto parity, uint32_t ci) {
-    constexpr bool odd = decltype(parity)::value;
-    const uint32_t c = actual(ci);   // ci: position in this workgroup's order (selects LDS buffer / register set)
-    const uint16_t* sw = lds_xs + (ci & 1u) * CHUNK_ELEMS;
-    const float* sb = s_bias[ci & 1u];
-    // accumulators start from the bias: acc[nt][mt][g*4+r] <-> column nt*32 + g*8 + half*4 + r
+
+  // per-lane byte offset of its fragment inside a chunk buffer; k-step ks is reached by ^ (32 ks)
+  const uint32_t frag_off = lq * ROWB + (((half ^ G::swz(lq)) & (uint32_t)(G::CPR - 1)) << 4);
+  uint16_t* patch = lds_patch + wave * (32 * kPatchRow);
+
+  for (uint32_t ci = 0; ci < nchunk; ++ci) {
+    const uint32_t c = actual(ci);
+    const uint32_t slot = ci % kXsBufs;
+    const bool more = ci + 2 < nchunk;
+    // request chunk ci+2 (its buffer was last read in chunk ci-1, which every wave has left)
+    if (more) dma_chunk(actual(ci + 2), (ci + 2) % kXsBufs);
+    if (ci + 1 < nchunk) park_bias((ci + 1) % kXsBufs);
+    if (more) load_bias(actual(ci + 2));
+
+    const char* sw = lds_xs + slot * G::CHUNK_BYTES;
+    const float* sb = s_bias[slot];
+    // accumulators: acc[nt][mt][g*4+r] <-> column nt*32 + g*8 + half*4 + r; they start from the bias
+    // (from zero with LN, where the bias enters the correction below)
     f32x16_t acc[2][MT];
 #pragma unroll
     for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
-        const float4 b4 = *reinterpret_cast<const float4*>(sb + nt * 32 + g * 8 + half * 4);
+        float4 b4 = {0.f, 0.f, 0.f, 0.f};
+        if (!LN) b4 = *reinterpret_cast<const float4*>(sb + nt * 32 + g * 8 + half * 4);
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
           acc[nt][mt][g * 4 + 0] = b4.x; acc[nt][mt][g * 4 + 1] = b4.y;
@@ -204,12 +270,12 @@ void xstat_linear_kernel(
         }
       }
     // w fragments are read kAhead k-steps before the MFMAs that consume them
-    constexpr int kAhead = KS < 4 ? KS : 4;
+    constexpr int kAhead = KS < 2 ? KS : 2;
     bf16x8_t wf[KS][2];
     auto read_frag = [&](int ks) {
+      const char* p = sw + (frag_off ^ (uint32_t)(ks * 32));
 #pragma unroll
-      for (int nt = 0; nt < 2; ++nt)
-        wf[ks][nt] = *reinterpret_cast<const bf16x8_t*>(sw + (nt * 32 + lq) * WROW + ks * 16 + half * 8);
+      for (int nt = 0; nt < 2; ++nt) wf[ks][nt] = *reinterpret_cast<const bf16x8_t*>(p + nt * 32 * ROWB);
     };
 #pragma unroll
     for (int ks = 0; ks < kAhead; ++ks) read_frag(ks);
@@ -229,17 +295,32 @@ void xstat_linear_kernel(
       __builtin_amdgcn_sched_group_barrier(0x008, 2 * MT, 0);
       if (ks + kAhead < KS) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
     }
-    // next chunk into the other LDS buffer, then refill the freed register set two chunks ahead
-    if (ci + 1 < nchunk) {
-      if constexpr (odd) stage(ci + 1, rwA, rbA); else stage(ci + 1, rwB, rbB);
-    }
-    if (ci + 3 < nchunk) {
-      if constexpr (odd) fetch(actual(ci + 3), rwA, rbA); else fetch(actual(ci + 3), rwB, rbB);
-    }
+    // Everything this wave issued before this chunk's direct loads has completed once at most that many
+    // operations are outstanding; that includes its share of chunk ci+1 (requested one chunk ago).  The
+    // count deliberately ignores the bias loads (wherever the compiler places them, the wait is then
+    // exact or slightly early, never late).  The epilogue stores below are younger and never waited on.
+    if (more) xs_wait_vm(my_dma); else __builtin_amdgcn_s_waitcnt(0x0F70);
+
     // ---- epilogue: the wave's 32 x 32 result tiles go through a wave-private LDS patch so that
     //      the global stores are row-contiguous 16-byte pieces (4 lanes = 64 bytes of one row) ----
     const uint32_t col0 = c * COLS;   // first output column of the chunk
-    uint16_t* patch = lds_patch + wave * (32 * kPatchRow);
+    if (LN) {
+      const float* ss = s_wsum[slot];
+#pragma unroll
+      for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const float4 b4 = *reinterpret_cast<const float4*>(sb + nt * 32 + g * 8 + half * 4);
+          const float4 s4 = *reinterpret_cast<const float4*>(ss + nt * 32 + g * 8 + half * 4);
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt) {
+            acc[nt][mt][g * 4 + 0] = __builtin_fmaf(ln_a[mt], acc[nt][mt][g * 4 + 0], __builtin_fmaf(ln_b[mt], s4.x, b4.x));
+            acc[nt][mt][g * 4 + 1] = __builtin_fmaf(ln_a[mt], acc[nt][mt][g * 4 + 1], __builtin_fmaf(ln_b[mt], s4.y, b4.y));
+            acc[nt][mt][g * 4 + 2] = __builtin_fmaf(ln_a[mt], acc[nt][mt][g * 4 + 2], __builtin_fmaf(ln_b[mt], s4.z, b4.z));
+            acc[nt][mt][g * 4 + 3] = __builtin_fmaf(ln_a[mt], acc[nt][mt][g * 4 + 3], __builtin_fmaf(ln_b[mt], s4.w, b4.w));
+          }
+        }
+    }
     auto flush_tile = [&](auto full_tag, int mt, uint32_t colbase) {
       // patch holds rows [mt*32, mt*32+32) x 32 columns starting at output column colbase
       constexpr bool kFull = decltype(full_tag)::value;
@@ -300,68 +381,107 @@ void xstat_linear_kernel(
     };
     if (wg_full) epilogue(std::true_type{}); else epilogue(std::false_type{});
     __syncthreads();
-  };
-  for (uint32_t c = 0; c < nchunk; c += 2) {
-    chunk_body(std::false_type{}, c);
-    if (c + 1 < nchunk) chunk_body(std::true_type{}, c + 1);
   }
 }
 
-template <int K, int MT>
-static void launch_k(bool ln_in, bool swiglu, dim3 grid, size_t lds, hipStream_t s, const uint16_t* x, uint32_t ldx,
-                     const uint16_t* gamma, const uint16_t* beta, float eps, const uint16_t* w, const uint16_t* bias,
-                     const uint16_t* residual, uint32_t ldr, uint16_t* y, uint32_t ldy, uint32_t M, uint32_t N,
-                     uint32_t act) {
-  const bool general = act != F3D_ACT_NONE || residual != nullptr;
-#define F3D_XS(L, S)                                                                                                  \
-  do {                                                                                                                \
-    if (general)                                                                                                      \
-      hipLaunchKernelGGL((xstat_linear_kernel<K, MT, L, S, 1>), grid, dim3(kXsThreads), lds, s, x, ldx, gamma, beta,   \
-                         eps, w, bias, residual, ldr, y, ldy, M, N, act);                                             \
-    else                                                                                                              \
-      hipLaunchKernelGGL((xstat_linear_kernel<K, MT, L, S, 0>), grid, dim3(kXsThreads), lds, s, x, ldx, gamma, beta,   \
-                         eps, w, bias, residual, ldr, y, ldy, M, N, act);                                             \
-  } while (0)
-  constexpr bool kLnOk = K <= 256;
-  const bool ln = ln_in && kLnOk;
-  if (ln && swiglu) F3D_XS(kLnOk, true);
-  else if (ln) F3D_XS(kLnOk, false);
-  else if (swiglu) F3D_XS(false, true);
-  else F3D_XS(false, false);
-#undef F3D_XS
+// w' = bf16(w * gamma), wsum[n] = sum_k w'[n][k] (of the rounded values the matrix core will see),
+// b'[n] = bias[n] + sum_k w[n][k] * beta[k].  One wave per output feature.
+__global__ __launch_bounds__(256) void ln_fold_kernel(const uint16_t* __restrict__ w, const uint16_t* __restrict__ gamma,
+                                                      const uint16_t* __restrict__ beta,
+                                                      const uint16_t* __restrict__ bias, uint16_t* __restrict__ wp,
+                                                      float* __restrict__ wsum, float* __restrict__ bp, uint32_t N,
+                                                      uint32_t K) {
+  const uint32_t n = blockIdx.x * 4 + threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  if (n >= N) return;
+  float s = 0.f, t = 0.f;
+  for (uint32_t k = lane; k < K; k += kWave) {
+    const float wv = bf16_bits_to_float(w[(size_t)n * K + k]);
+    const uint16_t r = float_to_bf16_bits(wv * bf16_bits_to_float(gamma[k]));
+    wp[(size_t)n * K + k] = r;
+    s += bf16_bits_to_float(r);
+    if (beta) t = __builtin_fmaf(wv, bf16_bits_to_float(beta[k]), t);
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    s += __shfl_xor(s, o, kWave);
+    t += __shfl_xor(t, o, kWave);
+  }
+  if (lane == 0) {
+    wsum[n] = s;
+    bp[n] = t + (bias ? bf16_bits_to_float(bias[n]) : 0.f);
+  }
 }
 
-// Returns false when the shape is not covered (the caller then uses the tiled GEMM).
-bool launch_xstat_linear(const uint16_t* x, uint32_t ldx, const uint16_t* gamma, const uint16_t* beta, float eps,
-                         const uint16_t* w, const uint16_t* bias, const uint16_t* residual, uint32_t ldr, uint16_t* y,
-                         uint32_t ldy, uint32_t M, uint32_t N, uint32_t K, uint32_t act, hipStream_t s) {
+template <int K, int MT, int WAVES>
+static int launch_k(bool ln, bool swiglu, hipStream_t s, const uint16_t* x, uint32_t ldx, float eps,
+                    const uint16_t* w, const uint16_t* bias, const float* bias_f, const float* wsum,
+                    const uint16_t* residual, uint32_t ldr, uint16_t* y, uint32_t ldy, uint32_t M, uint32_t N,
+                    uint32_t act, int device) {
+  const bool general = act != F3D_ACT_NONE || residual != nullptr;
+  const dim3 grid(cdiv_u32(M, 32 * MT * WAVES)), block(64 * WAVES);
+  constexpr size_t lds = xs_lds_bytes<K, WAVES>();
+#define F3D_XS(L, S, E)                                                                                            \
+  do {                                                                                                             \
+    static bool attr_set[64] = {};                                                                                 \
+    auto kern = xstat_linear_kernel<K, MT, WAVES, L, S, E>;                                                        \
+    if (device < 0 || device >= 64 || !attr_set[device]) {                                                         \
+      F3D_CHECK_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds)); \
+      if (device >= 0 && device < 64) attr_set[device] = true;                                                     \
+    }                                                                                                              \
+    hipLaunchKernelGGL(kern, grid, block, lds, s, x, ldx, eps, w, bias, bias_f, wsum, residual, ldr, y, ldy, M, N, \
+                       act);                                                                                       \
+  } while (0)
+  if (ln && swiglu) { if (general) F3D_XS(true, true, 1); else F3D_XS(true, true, 0); }
+  else if (ln) { if (general) F3D_XS(true, false, 1); else F3D_XS(true, false, 0); }
+  else if (swiglu) { if (general) F3D_XS(false, true, 1); else F3D_XS(false, true, 0); }
+  else { if (general) F3D_XS(false, false, 1); else F3D_XS(false, false, 0); }
+#undef F3D_XS
+  return F3D_OK;
+}
+
+// Returns F3D_OK when launched, F3D_ERR_UNSUPPORTED when the shape is not covered (the caller then uses
+// the tiled GEMM), another code on failure.
+int launch_xstat_linear(const uint16_t* x, uint32_t ldx, const uint16_t* gamma, const uint16_t* beta, float eps,
+                        const uint16_t* w, const uint16_t* bias, const uint16_t* residual, uint32_t ldr, uint16_t* y,
+                        uint32_t ldy, uint32_t M, uint32_t N, uint32_t K, uint32_t act, int device, hipStream_t s) {
   const bool ln = gamma != nullptr;
   const bool swiglu = act == F3D_ACT_SWIGLU;
   const uint32_t run_act = swiglu ? (uint32_t)F3D_ACT_NONE : act;
-  if (M == 0) return true;
-  if (N % 64 != 0) return false;     // chunks of 64 output features (32 value + 32 gate for swiglu) must be full
-  if (ln && K == 512) return false;  // 128 row values per lane plus the fp32 statistics do not fit the register file
-  // One 32-row tile per wave (MT = 1) leaves room for two workgroups per CU, which measured faster than
-  // MT = 2 at every shape of the model; F3D_XS_MT=2 selects the larger panel for experiments.
-  static const int mt_env = getenv("F3D_XS_MT") ? atoi(getenv("F3D_XS_MT")) : 1;
-#define F3D_XS_CASE(KK, MTT)                                                                                        \
-  case KK: {                                                                                                        \
-    const size_t lds = (size_t)2 * kXsChunk * (KK + 8) * 2;                                                         \
-    if (mt_env == 1 || MTT == 1)                                                                                    \
-      launch_k<KK, 1>(ln, swiglu, dim3(cdiv_u32(M, 128)), lds, s, x, ldx, gamma, beta, eps, w, bias, residual,      \
-                      ldr, y, ldy, M, N, run_act);                                                                  \
-    else                                                                                                            \
-      launch_k<KK, 2>(ln, swiglu, dim3(cdiv_u32(M, 256)), lds, s, x, ldx, gamma, beta, eps, w, bias, residual,      \
-                      ldr, y, ldy, M, N, run_act);                                                                  \
-    return true;                                                                                                    \
+  if (M == 0) return F3D_OK;
+  if (N % 64 != 0) return F3D_ERR_UNSUPPORTED;   // chunks of 64 w rows (32 value + 32 gate for swiglu) must be full
+  if (K != 32 && K != 64 && K != 128 && K != 256) return F3D_ERR_UNSUPPORTED;
+  if ((uint64_t)N * K * 2 >= (1ull << 32)) return F3D_ERR_UNSUPPORTED;   // 32-bit byte offsets into w
+  const float* bias_f = nullptr;
+  const float* wsum = nullptr;
+  if (ln) {
+    // per call: w' (bf16 [N][K]), wsum and b' (fp32 [N]) in the per-device workspace
+    const size_t wp_bytes = ((size_t)N * K * 2 + 255) & ~(size_t)255;
+    char* ws = (char*)workspace(device, wp_bytes + (size_t)N * 8);
+    if (!ws) return F3D_ERR_RUNTIME;
+    uint16_t* wp = (uint16_t*)ws;
+    float* ws_sum = (float*)(ws + wp_bytes);
+    float* ws_bias = ws_sum + N;
+    hipLaunchKernelGGL(ln_fold_kernel, dim3(cdiv_u32(N, 4)), dim3(256), 0, s, w, gamma, beta, bias, wp, ws_sum, ws_bias,
+                       N, K);
+    w = wp;
+    wsum = ws_sum;
+    bias_f = ws_bias;
   }
+  // Large panels (64 rows per wave, 8 waves) when there are enough rows to fill the chip with them,
+  // otherwise 32 rows per wave in 4-wave workgroups.
+  const bool big = M >= 512u * 256u;
+#define F3D_XS_CASE(KK)                                                                                                  \
+  case KK:                                                                                                               \
+    return big ? launch_k<KK, 2, 8>(ln, swiglu, s, x, ldx, eps, w, bias, bias_f, wsum, residual, ldr, y, ldy, M, N,      \
+                                    run_act, device)                                                                     \
+               : launch_k<KK, 1, 4>(ln, swiglu, s, x, ldx, eps, w, bias, bias_f, wsum, residual, ldr, y, ldy, M, N,      \
+                                    run_act, device);
   switch (K) {
-    F3D_XS_CASE(32, 2)
-    F3D_XS_CASE(64, 2)
-    F3D_XS_CASE(128, 2)
-    F3D_XS_CASE(256, 2)
-    F3D_XS_CASE(512, 1)
-    default: return false;
+    F3D_XS_CASE(32)
+    F3D_XS_CASE(64)
+    F3D_XS_CASE(128)
+    F3D_XS_CASE(256)
+    default: return F3D_ERR_UNSUPPORTED;
   }
 #undef F3D_XS_CASE
 }

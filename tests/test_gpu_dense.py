@@ -92,12 +92,25 @@ def test_layernorm_fused_linear(oracle, M, N, K, act, use_res):
     pshattn.ln_linear_bf16(x.to(DEV), g.to(DEV), b.to(DEV), 1e-5, w.to(DEV), bias.to(DEV),
                            None if res is None else res.to(DEV), y, act)
     torch.cuda.synchronize()
+    acts = {"swiglu": oracle.swiglu, "gelu": oracle.gelu, "relu": torch.relu, None: lambda t: t}
+    # the reference's sequence of bf16 roundings (LayerNorm output, Linear output) ...
     ln = oracle.layernorm(x, g, b, 1e-5).to(torch.bfloat16).float()
     lin = oracle.linear(ln, w, bias).to(torch.bfloat16).float()
-    ref = {"swiglu": oracle.swiglu, "gelu": oracle.gelu, "relu": torch.relu, None: lambda t: t}[act](lin)
+    ref = acts[act](lin)
+    # ... and the same mathematics without any intermediate rounding
+    exact = acts[act](oracle.linear(oracle.layernorm(x, g, b, 1e-5), w, bias))
     if res is not None:
         ref = ref.to(torch.bfloat16).float() + res.float()
-    _close(y, ref, tol=3e-2)
+        exact = exact + res.float()
+    # The kernel folds LayerNorm into the weights (w * gamma rounded to bf16, statistics applied to the fp32
+    # accumulators), so its roundings fall in other places than the reference's.  It must sit as close to the
+    # exact result as the reference's own rounding sequence does (bf16 output rounding included in both).
+    yf = y.float().cpu()
+    err_ref = (ref.to(torch.bfloat16).float() - exact).abs()
+    err_us = (yf - exact).abs()
+    scale = exact.abs().clamp(min=1.0)
+    assert (err_us / scale).max() <= 1.5 * (err_ref / scale).max() + 4e-3, (err_us.max(), err_ref.max())
+    assert err_us.mean() <= 1.25 * err_ref.mean() + 1e-4, (err_us.mean(), err_ref.mean())
 
 
 def test_linear_strided_views():
