@@ -25,6 +25,9 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
 MFMA_BF16_PEAK_TFLOPS = 2500.0
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by a copy kernel of known
+# size, see profiles/); filled in for the kernels that have been measured, None otherwise
+TRAFFIC_BYTES_PER_LAUNCH = {}
 
 
 def ev_time(fn, iters, warmup=3):
@@ -140,26 +143,47 @@ def main():
         Wn, Bn, Wq, Bq, Wp, Bp = bw(blk.norm.weight), bw(blk.norm.bias), bw(blk.bwa.qkv.weight), bw(blk.bwa.qkv.bias), bw(blk.bwa.proj.weight), bw(blk.bwa.proj.bias)
         W1, B1, W2, B2 = bw(mlp.fc1_weight), bw(mlp.fc1_bias), bw(mlp.fc2_weight), bw(mlp.fc2_bias)
         q, k, v = (t.view(1, n_pad, H, C // H) for t in qkv.chunk(3, dim=-1))
+        Wm, Bm = bw(mlp.layer_norm_weight), bw(mlp.layer_norm_bias)
+        # the launches the step above makes, one by one (LayerNorm is fused into the qkv and fc1 kernels)
         ops = {
             "psh_scatter": lambda: psh_main.batch_bucket_scatter(coords, seps, BS, n_pad, HASH),
-            "layernorm": lambda: pshattn.layernorm_bf16(feat, Wn, Bn, ln_out, 1e-5),
-            "qkv_gemm": lambda: pshattn.linear_bf16(ln_out, Wq, Bq, None, qkv, None),
+            "ln_qkv": lambda: pshattn.ln_linear_bf16(feat, Wn, Bn, 1e-5, Wq, Bq, None, qkv, None),
             "attention": lambda: pshattn.buck_swin_fwd(q, k, v, o, lse, scopes, BS),
-            "proj_gemm": lambda: pshattn.linear_bf16(o.view(n_pad, C), Wp, Bp, feat, mid, None),
-            "fc1_gemm": lambda: pshattn.linear_bf16(ln_out, W1, B1, None, hid, args.mlp),
-            "fc2_gemm": lambda: pshattn.linear_bf16(hid, W2, B2, mid, y, None),
+            "proj_residual": lambda: pshattn.linear_bf16(o.view(n_pad, C), Wp, Bp, feat, mid, None),
+            "ln_fc1_act": lambda: pshattn.ln_linear_bf16(mid, Wm, Bm, 1e-5, W1, B1, None, hid, args.mlp),
+            "fc2_residual": lambda: pshattn.linear_bf16(hid, W2, B2, mid, y, None),
         }
         breakdown = {name: ev_time(fn, 20) for name, fn in ops.items()}
     fc1_n = 2 * HID if args.mlp == "swiglu" else HID
-    flops = {"qkv_gemm": 2.0 * n_pad * C * 3 * C, "proj_gemm": 2.0 * n_pad * C * C,
-             "fc1_gemm": 2.0 * n_pad * C * fc1_n, "fc2_gemm": 2.0 * n_pad * HID * C,
+    flops = {"ln_qkv": 2.0 * n_pad * C * 3 * C, "proj_residual": 2.0 * n_pad * C * C,
+             "ln_fc1_act": 2.0 * n_pad * C * fc1_n, "fc2_residual": 2.0 * n_pad * HID * C,
              "attention": 4.0 * n_pad * BS * SCOPE * C}
-    dominant = max(("attention", "qkv_gemm", "proj_gemm", "fc1_gemm", "fc2_gemm"), key=lambda kname: breakdown[kname])
-    ach = flops[dominant] / (breakdown[dominant] * 1e-3) / 1e12
-    roofline = {"kernel": {"attention": "buck_swin_fwd_kernel<32,128>"}.get(dominant, "gemm_bf16_kernel"),
-                "op": dominant, "bound": "mfma", "achieved": round(ach, 2), "peak": MFMA_BF16_PEAK_TFLOPS,
-                "unit": "TFLOP/s", "frac": round(ach / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None,
-                "avg_launch_ms": round(breakdown[dominant], 4), "algorithmic_flop_per_launch": flops[dominant]}
+    # algorithmic HBM bytes per launch (bf16 activations in and out, weights negligible)
+    hbm_bytes = {"ln_qkv": 2.0 * n_pad * (C + 3 * C), "proj_residual": 2.0 * n_pad * 3 * C,
+                 "ln_fc1_act": 2.0 * n_pad * (C + HID), "fc2_residual": 2.0 * n_pad * (HID + 2 * C),
+                 "attention": 2.0 * n_pad * 4 * C + 4.0 * n_pad * H}
+    kernels = {"attention": "buck_swin_fwd_resident_kernel<32,512>",
+               "ln_qkv": "xstat_linear_kernel<256,2,8,3,LN> + ln_fold_kernel",
+               "ln_fc1_act": "xstat_linear_kernel<256,2,8,3,LN,swiglu> + ln_fold_kernel",
+               "proj_residual": "xstat_linear_kernel<256,2,8,3,residual>",
+               "fc2_residual": "gemm_bf16_kernel<false>"}
+    dominant = max(flops, key=lambda kname: breakdown[kname])
+    t_dom = breakdown[dominant] * 1e-3
+    ach = flops[dominant] / t_dom / 1e12
+    # the binding roof is the one with the larger minimum time
+    t_mfma, t_hbm = flops[dominant] / (MFMA_BF16_PEAK_TFLOPS * 1e12), hbm_bytes[dominant] / (HBM_PEAK_GBS * 1e9)
+    if t_mfma >= t_hbm:
+        roofline = {"kernel": kernels[dominant], "op": dominant, "bound": "mfma", "achieved": round(ach, 2),
+                    "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(ach / MFMA_BF16_PEAK_TFLOPS, 4)}
+    else:
+        gbs = hbm_bytes[dominant] / t_dom / 1e9
+        roofline = {"kernel": kernels[dominant], "op": dominant, "bound": "hbm", "achieved": round(gbs, 1),
+                    "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4)}
+    roofline.update({"traffic": TRAFFIC_BYTES_PER_LAUNCH.get(dominant), "avg_launch_ms": round(breakdown[dominant], 4),
+                     "algorithmic_flop_per_launch": flops[dominant],
+                     "algorithmic_hbm_bytes_per_launch": hbm_bytes[dominant]})
+    per_op = {kname: {"ms": round(breakdown[kname], 4), "tflops": round(flops[kname] / breakdown[kname] / 1e9, 1),
+                      "hbm_gbs": round(hbm_bytes[kname] / breakdown[kname] / 1e6, 1)} for kname in flops}
 
     sub = {}
     if not args.no_sub_metrics:
@@ -176,6 +200,7 @@ def main():
                    "mlp_hidden": HID, "bucket_size": BS, "scope_size": SCOPE, "hash_type": HASH},
         "roofline": roofline,
         "breakdown_ms": {kname: round(vv, 4) for kname, vv in breakdown.items()},
+        "per_op": per_op,
         "sub_metrics": sub,
     }
     if not args.no_cpu_baseline:

@@ -19,11 +19,12 @@ COMMON = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc",
     # packed fp32 VALU ops are kept out of the generated code on purpose
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-    # MFMA accumulators live in ordinary VGPRs (unified register file on gfx90a+): the softmax and the
-    # epilogues read them without v_accvgpr moves
-    "-mllvm", "-amdgpu-mfma-vgpr-form",
     "-Wall", "-Wno-unused-function", "-Wno-unknown-warning-option",
 ]
+# MFMA accumulators live in ordinary VGPRs (unified register file on gfx90a+): the softmax and the
+# epilogues read them without v_accvgpr moves
+VGPR_FORM = ["-mllvm", "-amdgpu-mfma-vgpr-form"]
+NO_VGPR_FORM = set()
 # bit-exact integer / quantiser kernels: no fused multiply-add contraction
 EXACT = {"psh_bucket.hip", "subbuck_pool.hip", "unpool.hip"}
 
@@ -36,6 +37,8 @@ def _compile(src):
     obj = os.path.join(OBJ_DIR, src.replace(".hip", ".o"))
     cmd = ["hipcc", "-c", os.path.join(HERE, src), "-o", obj] + COMMON
     cmd += ["-ffp-contract=off"] if src in EXACT else ["-ffp-contract=fast"]
+    if src not in NO_VGPR_FORM:
+        cmd += VGPR_FORM
     p = subprocess.run(cmd, capture_output=True, text=True)
     err = "\n".join(l for l in p.stderr.splitlines() if "not a recognized feature for this target" not in l)
     if p.returncode != 0:

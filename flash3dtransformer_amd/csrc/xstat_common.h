@@ -1,0 +1,77 @@
+// Pieces shared by the row-panel linear kernels and the fused feed-forward kernel.
+#pragma once
+#include "f3d_device.h"
+#include "f3d_internal.h"
+#include <stdlib.h>
+#include <type_traits>
+
+namespace f3d {
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16_t;
+
+constexpr int kXsChunk = 64;   // w rows per chunk (two 32-wide MFMA tiles)
+constexpr int kXsBufs = 3;     // w chunk buffers in LDS
+constexpr int kPatchRow = 40;  // epilogue patch: 32 output columns + 8 pad (80-byte pitch keeps 16-byte alignment)
+
+__device__ __forceinline__ float fast_silu(float a) {
+  // a * sigmoid(a) with the hardware exp2 / rcp
+  return a * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * a));
+}
+
+__device__ __forceinline__ float xs_act(float v, uint32_t act) {
+  switch (act) {
+    case F3D_ACT_GELU: return 0.5f * v * (1.0f + erff(v * 0.70710678118654752440f));
+    case F3D_ACT_SILU: return fast_silu(v);
+    case F3D_ACT_RELU: return v > 0.f ? v : 0.f;
+    default: return v;
+  }
+}
+
+// sum over the two lanes (l, l ^ 32) that share a row
+__device__ __forceinline__ float pair_sum(float v) { return v + __shfl_xor(v, 32, kWave); }
+
+// 16 bytes per lane from global memory straight into LDS: lane l of the wave lands at lds + 16 l.
+// gbase and lds are wave-uniform, voff is the lane's byte offset from gbase.  Inline assembly on
+// purpose: the compiler keeps no record of these loads, so it never guards LDS reads of OTHER buffers
+// with a full vmcnt wait; the waits that matter are written out below.
+__device__ __forceinline__ void xs_lds_dma16(const void* gbase, uint32_t voff, const char* lds) {
+  const uint32_t lds_addr =
+      __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(__attribute__((address_space(3))) const char*)lds);
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+               :
+               : "s"(lds_addr), "v"(voff), "s"(gbase)
+               : "memory", "m0");
+}
+
+// s_waitcnt vmcnt(n) for a small run-time n (the instruction takes an immediate)
+__device__ __forceinline__ void xs_wait_vm(uint32_t n) {
+  switch (n) {
+    case 0: __builtin_amdgcn_s_waitcnt(0x0F70); break;
+    case 1: __builtin_amdgcn_s_waitcnt(0x0F71); break;
+    case 2: __builtin_amdgcn_s_waitcnt(0x0F72); break;
+    case 3: __builtin_amdgcn_s_waitcnt(0x0F73); break;
+    case 4: __builtin_amdgcn_s_waitcnt(0x0F74); break;
+    case 5: __builtin_amdgcn_s_waitcnt(0x0F75); break;
+    case 6: __builtin_amdgcn_s_waitcnt(0x0F76); break;
+    default: __builtin_amdgcn_s_waitcnt(0x0F70); break;
+  }
+}
+
+template <int K>
+struct XsGeom {
+  static constexpr int CPR = K / 8;                       // 16-byte pieces per w row
+  static constexpr int ROWB = K * 2;                      // bytes per w row
+  static constexpr int CHUNK_BYTES = kXsChunk * ROWB;
+  static constexpr int RP = CPR >= 16 ? 1 : 16 / CPR;     // rows sharing one swizzle value
+  static constexpr int SWZ_MASK = (CPR < 16 ? CPR : 16) - 1;
+  static constexpr int N_DMA = CPR;                       // direct-load instructions per chunk (64 pieces each)
+  static constexpr int KP = K < 128 ? K : 128;            // columns per transposition pass of the x prologue
+  __host__ __device__ static constexpr uint32_t swz(uint32_t row) { return (row / RP) & SWZ_MASK; }
+};
+
+// w' = bf16(w * gamma), wsum and b' (fp32) for the algebraic LayerNorm fold (defined with the linear kernels)
+void launch_ln_fold(const uint16_t* w, const uint16_t* gamma, const uint16_t* beta, const uint16_t* bias, uint16_t* wp,
+                    float* wsum, float* bp, uint32_t N, uint32_t K, hipStream_t s);
+
+}  // namespace f3d

@@ -22,88 +22,23 @@
 //                                                            b' = b + w beta.
 // A small kernel prepares w' (bf16), wsum and b' (fp32) per call; the main kernel then only needs the row
 // statistics (one sweep over the registers that hold x) and two fused multiply-adds per output element.
-#include "f3d_device.h"
-#include "f3d_internal.h"
-#include <stdlib.h>
-#include <type_traits>
+#include "xstat_common.h"
 
 namespace f3d {
 
-typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
-typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16_t;
-
-constexpr int kXsChunk = 64;   // w rows per chunk (two 32-wide MFMA tiles)
-constexpr int kXsBufs = 3;     // w chunk buffers in LDS
-constexpr int kPatchRow = 40;  // epilogue patch: 32 output columns + 8 pad (80-byte pitch keeps 16-byte alignment)
-
-__device__ __forceinline__ float fast_silu(float a) {
-  // a * sigmoid(a) with the hardware exp2 / rcp
-  return a * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * a));
-}
-
-__device__ __forceinline__ float xs_act(float v, uint32_t act) {
-  switch (act) {
-    case F3D_ACT_GELU: return 0.5f * v * (1.0f + erff(v * 0.70710678118654752440f));
-    case F3D_ACT_SILU: return fast_silu(v);
-    case F3D_ACT_RELU: return v > 0.f ? v : 0.f;
-    default: return v;
-  }
-}
-
-// sum over the two lanes (l, l ^ 32) that share a row
-__device__ __forceinline__ float pair_sum(float v) { return v + __shfl_xor(v, 32, kWave); }
-
-// 16 bytes per lane from global memory straight into LDS: lane l of the wave lands at lds + 16 l.
-// gbase and lds are wave-uniform, voff is the lane's byte offset from gbase.  Inline assembly on
-// purpose: the compiler keeps no record of these loads, so it never guards LDS reads of OTHER buffers
-// with a full vmcnt wait; the waits that matter are written out below.
-__device__ __forceinline__ void xs_lds_dma16(const void* gbase, uint32_t voff, const char* lds) {
-  const uint32_t lds_addr =
-      __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(__attribute__((address_space(3))) const char*)lds);
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-               :
-               : "s"(lds_addr), "v"(voff), "s"(gbase)
-               : "memory", "m0");
-}
-
-// s_waitcnt vmcnt(n) for a small run-time n (the instruction takes an immediate)
-__device__ __forceinline__ void xs_wait_vm(uint32_t n) {
-  switch (n) {
-    case 0: __builtin_amdgcn_s_waitcnt(0x0F70); break;
-    case 1: __builtin_amdgcn_s_waitcnt(0x0F71); break;
-    case 2: __builtin_amdgcn_s_waitcnt(0x0F72); break;
-    case 3: __builtin_amdgcn_s_waitcnt(0x0F73); break;
-    case 4: __builtin_amdgcn_s_waitcnt(0x0F74); break;
-    case 5: __builtin_amdgcn_s_waitcnt(0x0F75); break;
-    case 6: __builtin_amdgcn_s_waitcnt(0x0F76); break;
-    default: __builtin_amdgcn_s_waitcnt(0x0F70); break;
-  }
-}
-
-template <int K>
-struct XsGeom {
-  static constexpr int CPR = K / 8;                       // 16-byte pieces per w row
-  static constexpr int ROWB = K * 2;                      // bytes per w row
-  static constexpr int CHUNK_BYTES = kXsChunk * ROWB;
-  static constexpr int RP = CPR >= 16 ? 1 : 16 / CPR;     // rows sharing one swizzle value
-  static constexpr int SWZ_MASK = (CPR < 16 ? CPR : 16) - 1;
-  static constexpr int N_DMA = CPR;                       // direct-load instructions per chunk (64 pieces each)
-  static constexpr int KP = K < 128 ? K : 128;            // columns per transposition pass of the x prologue
-  __host__ __device__ static constexpr uint32_t swz(uint32_t row) { return (row / RP) & SWZ_MASK; }
-};
-
-template <int K, int WAVES>
+template <int K, int WAVES, int NBUF>
 constexpr size_t xs_lds_bytes() {
   using G = XsGeom<K>;
-  const size_t wbuf = (size_t)kXsBufs * G::CHUNK_BYTES;
+  const size_t wbuf = (size_t)NBUF * G::CHUNK_BYTES;
   const size_t xpatch = (size_t)WAVES * 32 * (G::KP + 8) * 2;
   const size_t front = wbuf > xpatch ? wbuf : xpatch;
-  return front + (size_t)WAVES * 32 * kPatchRow * 2 + (size_t)2 * kXsBufs * kXsChunk * 4;
+  return front + (size_t)WAVES * 32 * kPatchRow * 2 + (size_t)2 * NBUF * kXsChunk * 4;
 }
 
 // EPI: 0 = bias only, 1 = runtime activation and / or residual.
 // With LN the kernel expects w = w', bias = b' (fp32), wsum (fp32) as prepared by ln_fold_kernel.
-template <int K, int MT, int WAVES, bool LN, bool SWIGLU, int EPI>
+// NBUF: w chunk buffers in LDS (chunk c + NBUF - 1 is requested when chunk c starts).
+template <int K, int MT, int WAVES, int NBUF, bool LN, bool SWIGLU, int EPI>
 __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2))) void xstat_linear_kernel(
     const uint16_t* __restrict__ x, uint32_t ldx, float eps, const uint16_t* __restrict__ w,
     const uint16_t* __restrict__ bias, const float* __restrict__ bias_f, const float* __restrict__ wsum,
@@ -115,12 +50,13 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
   constexpr int NT = 64 * WAVES;
   constexpr int ROWS_WG = 32 * MT * WAVES;
   extern __shared__ __attribute__((aligned(1024))) char lds_xs[];
-  constexpr size_t kFront = (size_t)kXsBufs * G::CHUNK_BYTES > (size_t)WAVES * 32 * (G::KP + 8) * 2
-                                ? (size_t)kXsBufs * G::CHUNK_BYTES
+  constexpr size_t kFront = (size_t)NBUF * G::CHUNK_BYTES > (size_t)WAVES * 32 * (G::KP + 8) * 2
+                                ? (size_t)NBUF * G::CHUNK_BYTES
                                 : (size_t)WAVES * 32 * (G::KP + 8) * 2;
+  constexpr uint32_t kAheadChunks = NBUF - 1;
   uint16_t* lds_patch = reinterpret_cast<uint16_t*>(lds_xs + kFront);
   float (*s_bias)[kXsChunk] = reinterpret_cast<float (*)[kXsChunk]>(lds_xs + kFront + (size_t)WAVES * 32 * kPatchRow * 2);
-  float (*s_wsum)[kXsChunk] = s_bias + kXsBufs;
+  float (*s_wsum)[kXsChunk] = s_bias + NBUF;
 
   const uint32_t tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid / kWave), lane = tid % kWave;
   const uint32_t lq = lane & 31u, half = lane >> 5;
@@ -232,11 +168,11 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
   auto actual = [&](uint32_t i) -> uint32_t { const uint32_t t = i + c_start; return t >= nchunk ? t - nchunk : t; };
 
   dma_chunk(actual(0), 0);
-  if (nchunk > 1) dma_chunk(actual(1), 1);
+  if (kAheadChunks > 1 && nchunk > 1) dma_chunk(actual(1), 1);
   load_bias(actual(0));
   park_bias(0);
   if (nchunk > 1) load_bias(actual(1));
-  __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): the first two chunks have landed
+  __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): the first chunk(s) have landed
   __syncthreads();
 
   // per-lane byte offset of its fragment inside a chunk buffer; k-step ks is reached by ^ (32 ks)
@@ -245,12 +181,12 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
 
   for (uint32_t ci = 0; ci < nchunk; ++ci) {
     const uint32_t c = actual(ci);
-    const uint32_t slot = ci % kXsBufs;
-    const bool more = ci + 2 < nchunk;
-    // request chunk ci+2 (its buffer was last read in chunk ci-1, which every wave has left)
-    if (more) dma_chunk(actual(ci + 2), (ci + 2) % kXsBufs);
-    if (ci + 1 < nchunk) park_bias((ci + 1) % kXsBufs);
-    if (more) load_bias(actual(ci + 2));
+    const uint32_t slot = ci % NBUF;
+    const bool more = ci + kAheadChunks < nchunk;
+    // request chunk ci + NBUF - 1 (its buffer was last read in chunk ci-1, which every wave has left)
+    if (more) dma_chunk(actual(ci + kAheadChunks), (ci + kAheadChunks) % NBUF);
+    if (ci + 1 < nchunk) park_bias((ci + 1) % NBUF);
+    if (ci + 2 < nchunk) load_bias(actual(ci + 2));
 
     const char* sw = lds_xs + slot * G::CHUNK_BYTES;
     const float* sb = s_bias[slot];
@@ -299,7 +235,7 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
     // operations are outstanding; that includes its share of chunk ci+1 (requested one chunk ago).  The
     // count deliberately ignores the bias loads (wherever the compiler places them, the wait is then
     // exact or slightly early, never late).  The epilogue stores below are younger and never waited on.
-    if (more) xs_wait_vm(my_dma); else __builtin_amdgcn_s_waitcnt(0x0F70);
+    if (more && kAheadChunks > 1) xs_wait_vm(my_dma); else __builtin_amdgcn_s_waitcnt(0x0F70);
 
     // ---- epilogue: the wave's 32 x 32 result tiles go through a wave-private LDS patch so that
     //      the global stores are row-contiguous 16-byte pieces (4 lanes = 64 bytes of one row) ----
@@ -412,18 +348,23 @@ __global__ __launch_bounds__(256) void ln_fold_kernel(const uint16_t* __restrict
   }
 }
 
-template <int K, int MT, int WAVES>
+void launch_ln_fold(const uint16_t* w, const uint16_t* gamma, const uint16_t* beta, const uint16_t* bias, uint16_t* wp,
+                    float* wsum, float* bp, uint32_t N, uint32_t K, hipStream_t s) {
+  hipLaunchKernelGGL(ln_fold_kernel, dim3(cdiv_u32(N, 4)), dim3(256), 0, s, w, gamma, beta, bias, wp, wsum, bp, N, K);
+}
+
+template <int K, int MT, int WAVES, int NBUF>
 static int launch_k(bool ln, bool swiglu, hipStream_t s, const uint16_t* x, uint32_t ldx, float eps,
                     const uint16_t* w, const uint16_t* bias, const float* bias_f, const float* wsum,
                     const uint16_t* residual, uint32_t ldr, uint16_t* y, uint32_t ldy, uint32_t M, uint32_t N,
                     uint32_t act, int device) {
   const bool general = act != F3D_ACT_NONE || residual != nullptr;
   const dim3 grid(cdiv_u32(M, 32 * MT * WAVES)), block(64 * WAVES);
-  constexpr size_t lds = xs_lds_bytes<K, WAVES>();
+  constexpr size_t lds = xs_lds_bytes<K, WAVES, NBUF>();
 #define F3D_XS(L, S, E)                                                                                            \
   do {                                                                                                             \
     static bool attr_set[64] = {};                                                                                 \
-    auto kern = xstat_linear_kernel<K, MT, WAVES, L, S, E>;                                                        \
+    auto kern = xstat_linear_kernel<K, MT, WAVES, NBUF, L, S, E>;                                                       \
     if (device < 0 || device >= 64 || !attr_set[device]) {                                                         \
       F3D_CHECK_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds)); \
       if (device >= 0 && device < 64) attr_set[device] = true;                                                     \
@@ -461,21 +402,21 @@ int launch_xstat_linear(const uint16_t* x, uint32_t ldx, const uint16_t* gamma, 
     uint16_t* wp = (uint16_t*)ws;
     float* ws_sum = (float*)(ws + wp_bytes);
     float* ws_bias = ws_sum + N;
-    hipLaunchKernelGGL(ln_fold_kernel, dim3(cdiv_u32(N, 4)), dim3(256), 0, s, w, gamma, beta, bias, wp, ws_sum, ws_bias,
-                       N, K);
+    launch_ln_fold(w, gamma, beta, bias, wp, ws_sum, ws_bias, N, K, s);
     w = wp;
     wsum = ws_sum;
     bias_f = ws_bias;
   }
-  // Large panels (64 rows per wave, 8 waves) when there are enough rows to fill the chip with them,
-  // otherwise 32 rows per wave in 4-wave workgroups.
+  // Large panels (64 rows per wave, 8 waves, 3 chunk buffers: one workgroup per CU) when there are enough
+  // rows to fill the chip with them, otherwise 32 rows per wave in 4-wave workgroups with 2 buffers.
+  // (Two 4-wave workgroups of 64-row waves per CU measured 6% slower than one 8-wave workgroup.)
   const bool big = M >= 512u * 256u;
 #define F3D_XS_CASE(KK)                                                                                                  \
   case KK:                                                                                                               \
-    return big ? launch_k<KK, 2, 8>(ln, swiglu, s, x, ldx, eps, w, bias, bias_f, wsum, residual, ldr, y, ldy, M, N,      \
-                                    run_act, device)                                                                     \
-               : launch_k<KK, 1, 4>(ln, swiglu, s, x, ldx, eps, w, bias, bias_f, wsum, residual, ldr, y, ldy, M, N,      \
-                                    run_act, device);
+    return big ? launch_k<KK, 2, 8, 3>(ln, swiglu, s, x, ldx, eps, w, bias, bias_f, wsum, residual, ldr, y, ldy, M, N,   \
+                                       run_act, device)                                                                  \
+               : launch_k<KK, 1, 4, 2>(ln, swiglu, s, x, ldx, eps, w, bias, bias_f, wsum, residual, ldr, y, ldy, M, N,   \
+                                       run_act, device);
   switch (K) {
     F3D_XS_CASE(32)
     F3D_XS_CASE(64)

@@ -203,6 +203,7 @@ class LayerNormMLP(nn.Module):
     def forward(self, x: torch.Tensor, residual: torch.Tensor = None):
         x2 = as_bf16_2d(x.reshape(-1, self.hidden_size)).contiguous()
         c = self._c
+        r2 = None if residual is None else as_bf16_2d(residual.reshape(-1, self.hidden_size))
         h = torch.empty(x2.shape[0], self.ffn_hidden_size, dtype=torch.bfloat16, device=x.device)
         if self.hidden_size in FUSABLE_LN_WIDTHS:
             pshattn.ln_linear_bf16(x2, c[0].get(self.layer_norm_weight), c[1].get(self.layer_norm_bias), self.eps,
@@ -212,6 +213,5 @@ class LayerNormMLP(nn.Module):
             pshattn.layernorm_bf16(x2, c[0].get(self.layer_norm_weight), c[1].get(self.layer_norm_bias), ln, self.eps)
             pshattn.linear_bf16(ln, c[2].get(self.fc1_weight), c[3].get(self.fc1_bias), None, h, self.activation)
         y = torch.empty_like(x2)
-        r2 = None if residual is None else as_bf16_2d(residual.reshape(-1, self.hidden_size))
         pshattn.linear_bf16(h, c[4].get(self.fc2_weight), c[5].get(self.fc2_bias), r2, y, None)
         return forward_only(y.view(x.shape), "LayerNormMLP", x, self.fc1_weight)
