@@ -34,8 +34,21 @@ def cdiv_int(a: torch.Tensor, b):
     return (a + (b - 1)) / b
 
 
+_HOST_SIZES = {}   # (data_ptr, shape, version) of the last separator tensors seen -> their sizes on the host
+
+
 def host_sizes(seps: torch.Tensor):
     """Cloud sizes as a Python list with a single device->host copy (the reference pays one
-    `.item()` sync per statistic, psh_main.py:47,102)."""
+    `.item()` sync per statistic, psh_main.py:47,102).  The copy is a host-device synchronisation, so
+    the answer is remembered per separator tensor: the same tensor (same storage, unchanged since)
+    costs nothing the next time, and the host can queue a whole step ahead of the GPU."""
+    key = (seps.data_ptr(), tuple(seps.shape), seps._version, str(seps.device))
+    hit = _HOST_SIZES.get(key)
+    if hit is not None:
+        return hit
     wide = seps.to(torch.int64).cpu()
-    return torch.diff(wide, prepend=wide.new_zeros(1)).tolist()
+    sizes = torch.diff(wide, prepend=wide.new_zeros(1)).tolist()
+    if len(_HOST_SIZES) > 64:
+        _HOST_SIZES.clear()
+    _HOST_SIZES[key] = sizes
+    return sizes

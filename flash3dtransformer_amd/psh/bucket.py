@@ -17,8 +17,17 @@ def probe_offset_list(shuffle_seed=None):
     return offs
 
 
+_PROBE_CACHE = {}   # (device, row_major, shuffle_seed) -> table on the device (read-only for every consumer)
+
+
 def generate_probe_offsets(device, row_major=True, shuffle_seed=None):
+    key = (str(device), bool(row_major), shuffle_seed)
+    hit = _PROBE_CACHE.get(key)
+    if hit is not None:
+        return hit
     t = torch.tensor(probe_offset_list(shuffle_seed), dtype=torch.int16)
     if not row_major:
         t = t.t()
-    return t.contiguous().to(device)
+    t = t.contiguous().to(device)
+    _PROBE_CACHE[key] = t
+    return t

@@ -37,27 +37,36 @@ class BucketScatterBuffers:
     scattered_coord: torch.Tensor
 
     @staticmethod
-    def create_buffers(coords: torch.Tensor, seps: torch.Tensor, bucket_size: int, pad_to: int, num_buck: int = None):
+    def create_buffers(coords: torch.Tensor, seps: torch.Tensor, bucket_size: int, pad_to: int, num_buck: int = None,
+                       debug_prefill: bool = True):
         """Allocation contract of the op (psh_main.py:31-67).  Prefills the kernels rely on:
         bucket_cntr = 0 (slots are counted up from it).  bucket_id = 1 and scattered_coord = NaN are the
-        reference's debugging prefills (its tests look for surviving NaNs); they are kept."""
+        reference's debugging prefills (its tests look for surviving NaNs); `debug_prefill=False` skips
+        them, which is safe here because the scatter kernel writes every row of both."""
         total_n, d = coords.shape
         dev = coords.device
         if num_buck is None:
             num_buck, _, _ = bucket_geometry(seps, bucket_size)
         b = seps.shape[0]
+        zeros = torch.zeros(2, b, num_buck, dtype=torch.uint32, device=dev)   # one fill for both counters
+        if debug_prefill:
+            bucket_id = torch.ones(total_n, dtype=torch.uint16, device=dev)
+            scattered = torch.full((pad_to, d), float("nan"), dtype=torch.float16, device=dev)
+        else:
+            bucket_id = torch.empty(total_n, dtype=torch.uint16, device=dev)
+            scattered = torch.empty(pad_to, d, dtype=torch.float16, device=dev)
         return BucketScatterBuffers(
-            bucket_id=torch.ones(total_n, dtype=torch.uint16, device=dev),
-            bucket_cntr=torch.zeros(b, num_buck, dtype=torch.uint32, device=dev),
+            bucket_id=bucket_id,
+            bucket_cntr=zeros[0],
             bucket_offs=torch.empty(total_n, dtype=torch.uint32, device=dev),
-            bucket_cumsum=torch.zeros(b, num_buck, dtype=torch.uint32, device=dev),
+            bucket_cumsum=zeros[1],
             probe_offs=f3dbuck.generate_probe_offsets(dev, row_major=True),
-            scattered_coord=torch.full((pad_to, d), float("nan"), dtype=torch.float16, device=dev),
+            scattered_coord=scattered,
         )
 
 
-def batch_bucket_scatter(coords: torch.Tensor, seps: torch.Tensor, bucket_size: int, pad_to: int, hash_op: int
-                         ) -> Tuple[torch.Tensor, BucketScatterBuffers]:
+def batch_bucket_scatter(coords: torch.Tensor, seps: torch.Tensor, bucket_size: int, pad_to: int, hash_op: int,
+                         debug_prefill: bool = False) -> Tuple[torch.Tensor, BucketScatterBuffers]:
     """coords [N,3] fp16 (clouds concatenated, `seps` inclusive cumulative sizes, uint32) ->
     scattered_coord [pad_to,3]: every cloud's points grouped by hash bucket (hash_op: 1 ZORDER_DIV,
     2 XORSUM_DIV, 3 ZORDER_MOD, 4 XORSUM_MOD), rows [N, pad_to) = 0.
@@ -66,7 +75,7 @@ def batch_bucket_scatter(coords: torch.Tensor, seps: torch.Tensor, bucket_size: 
     bounding box from one fused kernel instead of two torch reductions."""
     f3ddev.init_dev(coords.get_device())
     num_buck, divisor, max_n = bucket_geometry(seps, bucket_size)
-    buffers = BucketScatterBuffers.create_buffers(coords, seps, bucket_size, pad_to, num_buck)
+    buffers = BucketScatterBuffers.create_buffers(coords, seps, bucket_size, pad_to, num_buck, debug_prefill)
     bbox = torch.empty(2, 3, dtype=torch.float16, device=coords.device)
     pshattn.coord_bbox(coords, bbox[0], bbox[1])
     pshattn.batch_psh_scatter_pad_hash(
