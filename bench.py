@@ -26,8 +26,9 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by a copy kernel of known
-# size, see profiles/); filled in for the kernels that have been measured, None otherwise
-TRAFFIC_BYTES_PER_LAUNCH = {}
+# size, see profiles/encoder_stage_4x120k_hbm_traffic.md) at this bench's shapes
+TRAFFIC_BYTES_PER_LAUNCH = {"ln_fc1_act": 1.540e9, "ln_qkv": 1.064e9, "attention": 1.016e9,
+                            "proj_residual": 0.826e9, "fc2_residual": 1.516e9}
 
 
 def ev_time(fn, iters, warmup=3):
