@@ -179,20 +179,22 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
   const uint32_t frag_off = lq * ROWB + (((half ^ G::swz(lq)) & (uint32_t)(G::CPR - 1)) << 4);
   uint16_t* patch = lds_patch + wave * (32 * kPatchRow);
 
-  for (uint32_t ci = 0; ci < nchunk; ++ci) {
-    const uint32_t c = actual(ci);
-    const uint32_t slot = ci % NBUF;
-    const bool more = ci + kAheadChunks < nchunk;
-    // request chunk ci + NBUF - 1 (its buffer was last read in chunk ci-1, which every wave has left)
-    if (more) dma_chunk(actual(ci + kAheadChunks), (ci + kAheadChunks) % NBUF);
+  // accumulators: acc[nt][mt][g*4+r] <-> column nt*32 + g*8 + half*4 + r
+  f32x16_t acc[2][MT];
+
+  // stage 1: requests for chunk ci + NBUF - 1 (its buffer was last read in chunk ci-1, which every wave
+  // has left) and the bias hand-over
+  auto stage_request = [&](uint32_t ci) {
+    if (ci + kAheadChunks < nchunk) dma_chunk(actual(ci + kAheadChunks), (ci + kAheadChunks) % NBUF);
     if (ci + 1 < nchunk) park_bias((ci + 1) % NBUF);
     if (ci + 2 < nchunk) load_bias(actual(ci + 2));
-
+  };
+  // stage 2: the MFMAs of chunk ci; the accumulators start from the bias (from zero with LN, where the bias
+  // enters the correction of the epilogue)
+  auto stage_mfma = [&](uint32_t ci) {
+    const uint32_t slot = ci % NBUF;
     const char* sw = lds_xs + slot * G::CHUNK_BYTES;
     const float* sb = s_bias[slot];
-    // accumulators: acc[nt][mt][g*4+r] <-> column nt*32 + g*8 + half*4 + r; they start from the bias
-    // (from zero with LN, where the bias enters the correction below)
-    f32x16_t acc[2][MT];
 #pragma unroll
     for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
@@ -231,15 +233,13 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
       __builtin_amdgcn_sched_group_barrier(0x008, 2 * MT, 0);
       if (ks + kAhead < KS) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
     }
-    // Everything this wave issued before this chunk's direct loads has completed once at most that many
-    // operations are outstanding; that includes its share of chunk ci+1 (requested one chunk ago).  The
-    // count deliberately ignores the bias loads (wherever the compiler places them, the wait is then
-    // exact or slightly early, never late).  The epilogue stores below are younger and never waited on.
-    if (more && kAheadChunks > 1) xs_wait_vm(my_dma); else __builtin_amdgcn_s_waitcnt(0x0F70);
-
-    // ---- epilogue: the wave's 32 x 32 result tiles go through a wave-private LDS patch so that
-    //      the global stores are row-contiguous 16-byte pieces (4 lanes = 64 bytes of one row) ----
-    const uint32_t col0 = c * COLS;   // first output column of the chunk
+  };
+  // stage 3: epilogue of chunk ci: the wave's 32 x 32 result tiles go through a wave-private LDS patch so
+  // that the global stores are row-contiguous 16-byte pieces (4 lanes = 64 bytes of one row)
+  auto stage_epilogue = [&](uint32_t ci) {
+    const uint32_t slot = ci % NBUF;
+    const float* sb = s_bias[slot];
+    const uint32_t col0 = actual(ci) * COLS;   // first output column of the chunk
     if (LN) {
       const float* ss = s_wsum[slot];
 #pragma unroll
@@ -316,7 +316,40 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
       }
     };
     if (wg_full) epilogue(std::true_type{}); else epilogue(std::false_type{});
-    __syncthreads();
+  };
+  // "Everything this wave issued before chunk ci's requests has completed" holds once at most that many
+  // operations are outstanding, PROVIDED nothing younger than the requests has been issued yet; that
+  // includes this wave's share of chunk ci+1 (requested one chunk ago).  The count ignores the bias loads
+  // (wherever the compiler places them, the wait is then exact or slightly early, never late).
+  auto wait_next_chunk = [&](uint32_t ci) {
+    if (kAheadChunks > 1 && ci + kAheadChunks < nchunk) xs_wait_vm(my_dma); else __builtin_amdgcn_s_waitcnt(0x0F70);
+  };
+
+  // The two waves that share a SIMD (wave v and v + WAVES/2) run the stages of a barrier interval in
+  // complementary order, so that one's epilogue (VALU, LDS, stores) overlaps the other's MFMAs:
+  //   first half :  request(c)  mfma(c)      wait  epilogue(c)   | barrier
+  //   second half:  epilogue(c-1)  request(c)  mfma(c)  wait      | barrier      (+ epilogue(last) at the end)
+  // Both halves read chunk c's buffer inside the same interval, so the buffer rotation is unchanged; the
+  // late epilogue only reads the bias slot of chunk c-1, which with three slots is not rewritten before
+  // interval c+1.  The stores of a late epilogue are older than the requests that follow them, as the wait needs.
+  const bool late_half = NBUF >= 3 && WAVES >= 8 && wave >= (uint32_t)(WAVES / 2);
+  if (!late_half) {
+    for (uint32_t ci = 0; ci < nchunk; ++ci) {
+      stage_request(ci);
+      stage_mfma(ci);
+      wait_next_chunk(ci);
+      stage_epilogue(ci);
+      __syncthreads();
+    }
+  } else {
+    for (uint32_t ci = 0; ci < nchunk; ++ci) {
+      if (ci > 0) stage_epilogue(ci - 1);
+      stage_request(ci);
+      stage_mfma(ci);
+      wait_next_chunk(ci);
+      __syncthreads();
+    }
+    stage_epilogue(nchunk - 1);
   }
 }
 
