@@ -293,7 +293,40 @@ def sub_metrics(dev):
     out["pool_c3_reduce_mean"] = {"ms": round(ms_mean, 4), "gbs": gb(red_bytes, ms_mean), "frac_of_hbm_peak": round(gb(red_bytes, ms_mean) / HBM_PEAK_GBS, 4)}
     out["pool_c3_reduce_max"] = {"ms": round(ms_max, 4), "gbs": gb(red_bytes, ms_max), "frac_of_hbm_peak": round(gb(red_bytes, ms_max) / HBM_PEAK_GBS, 4)}
     out["unpool_c3"] = {"ms": round(ms_up, 4), "gbs": gb(up_bytes, ms_up), "frac_of_hbm_peak": round(gb(up_bytes, ms_up) / HBM_PEAK_GBS, 4)}
+    del coords, feat, res, up, sb
+    out["hourglass_c5"] = hourglass_c5(dev)
     return out
+
+
+def hourglass_c5(dev):
+    """whole-model forward, config 5: 4 sweeps x 250,000 points, 5 levels C = 32/64/128/256/512, heads = C/32,
+    bucket 512, scope of 1 bucket, pooling S = 2 (mean), swiglu MLP with hidden = 4C, hash 2"""
+    from flash3dtransformer_amd import layers as L, synth
+    from flash3dtransformer_amd.psh.bucket_scope import SwinPlan
+    bs, scope, S, hash_op = 512, 1, 2, 2
+    torch.manual_seed(1005)
+    ln = lambda ch: L.LayerNorm(ch)
+    spec = lambda c: L.XFMRSpecs(c, 4 * c, c // 32, True, SwinPlan("swin", bs, scope, 0), ln)
+    chans = [32, 64, 128, 256, 512]
+    levels = [L.F3DLevelSpecs([spec(c)], [spec(c)], "mean", bs * scope, ln if i + 1 < len(chans) else None, None,
+                              ln if i + 1 < len(chans) else None, None) for i, c in enumerate(chans)]
+    model = L.Flash3D(levels, bs, scope, hash_op, subbuck_size=S).to(dev).eval()
+    clouds = [synth.lidar_sweep(250_000, 1005 + i) for i in range(4)]
+    coords_np, seps_np = synth.batch_of(clouds)
+    coords = torch.from_numpy(coords_np).to(dev)
+    seps = torch.from_numpy(seps_np.view(np.int32)).to(dev).view(torch.uint32)
+    with torch.no_grad():
+        for _ in range(2):
+            model(coords, None, seps)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        iters = 5
+        for _ in range(iters):
+            model(coords, None, seps)
+        torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) / iters * 1e3
+    return {"ms": round(ms, 3), "mpts_per_s": round(coords.shape[0] / ms / 1e3, 1), "points": int(coords.shape[0]),
+            "levels": chans, "subbuck_size": S}
 
 
 if __name__ == "__main__":
