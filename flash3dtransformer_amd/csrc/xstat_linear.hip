@@ -120,9 +120,11 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
   const uint32_t n_out = SWIGLU ? N / 2 : N;
   // a swiglu chunk pairs 32 value rows with their 32 gate rows; a plain chunk is 64 consecutive rows
   constexpr uint32_t COLS = SWIGLU ? 32u : (uint32_t)kXsChunk;   // output columns per chunk
-  const uint32_t nchunk = n_out / COLS;   // the launcher only takes shapes whose chunks are all full
+  // swiglu chunks are always full (the launcher checks); a plain last chunk may hold only its first 32
+  // rows: the missing rows are read from the last valid one and their tile is not stored
+  const uint32_t nchunk = (n_out + COLS - 1) / COLS;
   auto w_row = [&](uint32_t c, uint32_t r) -> uint32_t {  // weight row behind chunk-local row r
-    if (!SWIGLU) return c * kXsChunk + r;
+    if (!SWIGLU) return min(c * kXsChunk + r, N - 1);
     return r < 32 ? c * 32 + r : n_out + c * 32 + (r - 32);
   };
   // direct loads of chunk c into buffer slot: instruction q fills LDS bytes [1024 q, 1024 q + 1024) of the
@@ -294,7 +296,7 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
               pk.y = pack_bf16x2(acc[nt][mt][g * 4 + 2], acc[nt][mt][g * 4 + 3]);
               *reinterpret_cast<uint2*>(patch + lq * kPatchRow + g * 8 + half * 4) = pk;
             }
-            flush_tile(full_tag, mt, col0 + nt * 32);
+            if (col0 + nt * 32 < N) flush_tile(full_tag, mt, col0 + nt * 32);
           }
         } else {
 #pragma unroll
@@ -422,7 +424,8 @@ int launch_xstat_linear(const uint16_t* x, uint32_t ldx, const uint16_t* gamma, 
   const bool swiglu = act == F3D_ACT_SWIGLU;
   const uint32_t run_act = swiglu ? (uint32_t)F3D_ACT_NONE : act;
   if (M == 0) return F3D_OK;
-  if (N % 64 != 0) return F3D_ERR_UNSUPPORTED;   // chunks of 64 w rows (32 value + 32 gate for swiglu) must be full
+  // whole 32-column tiles; a swiglu chunk pairs 32 value rows with 32 gate rows
+  if (swiglu ? N % 64 != 0 : N % 32 != 0) return F3D_ERR_UNSUPPORTED;
   if (K != 32 && K != 64 && K != 128 && K != 256) return F3D_ERR_UNSUPPORTED;
   if ((uint64_t)N * K * 2 >= (1ull << 32)) return F3D_ERR_UNSUPPORTED;   // 32-bit byte offsets into w
   const float* bias_f = nullptr;

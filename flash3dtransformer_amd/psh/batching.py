@@ -2,6 +2,8 @@
 inclusive cumulative point counts (reference: flash3dxfmr/psh/batching.py:13-40)."""
 from typing import List, Sequence
 
+import weakref
+
 import torch
 
 
@@ -34,21 +36,29 @@ def cdiv_int(a: torch.Tensor, b):
     return (a + (b - 1)) / b
 
 
-_HOST_SIZES = {}   # (data_ptr, shape, version) of the last separator tensors seen -> their sizes on the host
+_HOST_FACTS = {}   # id(separator tensor) -> (weak reference, tensor version, facts known on the host)
+
+
+def host_facts(seps: torch.Tensor) -> dict:
+    """Per-tensor memo for values derived from a separator tensor that live on the host.  Keyed by the
+    tensor OBJECT (a weak reference proves it is still the same one: a new tensor that happens to reuse
+    the address is a different object) and its version counter (in-place torch ops bump it)."""
+    key = id(seps)
+    hit = _HOST_FACTS.get(key)
+    if hit is not None and hit[0]() is seps and hit[1] == seps._version:
+        return hit[2]
+    facts = {}
+    _HOST_FACTS[key] = (weakref.ref(seps, lambda _r, k=key: _HOST_FACTS.pop(k, None)), seps._version, facts)
+    return facts
 
 
 def host_sizes(seps: torch.Tensor):
     """Cloud sizes as a Python list with a single device->host copy (the reference pays one
     `.item()` sync per statistic, psh_main.py:47,102).  The copy is a host-device synchronisation, so
-    the answer is remembered per separator tensor: the same tensor (same storage, unchanged since)
-    costs nothing the next time, and the host can queue a whole step ahead of the GPU."""
-    key = (seps.data_ptr(), tuple(seps.shape), seps._version, str(seps.device))
-    hit = _HOST_SIZES.get(key)
-    if hit is not None:
-        return hit
-    wide = seps.to(torch.int64).cpu()
-    sizes = torch.diff(wide, prepend=wide.new_zeros(1)).tolist()
-    if len(_HOST_SIZES) > 64:
-        _HOST_SIZES.clear()
-    _HOST_SIZES[key] = sizes
-    return sizes
+    the answer is remembered per separator tensor: the same tensor object, unchanged since, costs nothing
+    the next time, and the host can queue a whole step ahead of the GPU."""
+    facts = host_facts(seps)
+    if "sizes" not in facts:
+        wide = seps.to(torch.int64).cpu()
+        facts["sizes"] = torch.diff(wide, prepend=wide.new_zeros(1)).tolist()
+    return facts["sizes"]

@@ -9,11 +9,25 @@ from . import batching as f3dbatch
 
 def calc_red_sep_sizes(seps: torch.Tensor, subbuck_size: int):
     """Every cloud of n points pools to ceil(n / subbuck_size) rows: (total rows, per-cloud rows,
-    cumulative rows) with the dtype of `seps` (subbuck.py:40-53)."""
+    cumulative rows) with the dtype of `seps` (subbuck.py:40-53).  Computed on the host from the cloud
+    sizes (known there after one copy per separator tensor) and remembered per tensor, so a repeated
+    forward on the same batch neither synchronises nor uploads anything; the returned cumulative tensor
+    already carries its own sizes for the next level."""
     assert seps.dim() == 1, f"Seps dimension is expected to be 1, got {seps.dim()} instead"
-    sizes = f3dbatch.sep2sizes(seps.to(torch.int64))
-    red_sizes = torch.div(sizes + (subbuck_size - 1), subbuck_size, rounding_mode="floor")
-    return int(red_sizes.sum()), red_sizes.to(seps.dtype), torch.cumsum(red_sizes, dim=0).to(seps.dtype)
+    facts = f3dbatch.host_facts(seps)
+    key = ("reduced", int(subbuck_size))
+    if key not in facts:
+        sizes = f3dbatch.host_sizes(seps)
+        red = [(n + subbuck_size - 1) // subbuck_size for n in sizes]
+        cum, acc = [], 0
+        for r in red:
+            acc += r
+            cum.append(acc)
+        as_dev = lambda v: torch.tensor(v, dtype=torch.int64).to(seps.dtype).to(seps.device)
+        red_sizes, red_cum = as_dev(red), as_dev(cum)
+        f3dbatch.host_facts(red_cum)["sizes"] = red
+        facts[key] = (acc, red_sizes, red_cum)
+    return facts[key]
 
 
 @dcls.dataclass(slots=True)

@@ -48,6 +48,9 @@ def test_gemm_sm_bf16_reference_case():
     (1000, 1024, 256, "gelu", True, False),    # plain-GELU MLP variant, ragged M
     (777, 96, 64, "relu", False, False),
     (130, 136, 72, "silu", True, True),        # edges in M, N and K
+    (3000, 32, 128, None, True, True),         # half-full last chunk of the row-panel kernel (fc2 of a C=32 level)
+    (140000, 96, 32, None, True, False),       # the same in the 512-row configuration (qkv of a C=32 level)
+    (140000, 32, 32, "gelu", True, True),
 ])
 def test_linear_epilogues(oracle, M, N, K, act, use_bias, use_res):
     from flash3dtransformer_amd.lib import pshattn
@@ -79,6 +82,7 @@ def test_linear_epilogues(oracle, M, N, K, act, use_bias, use_res):
     (5000, 768, 256, None, False),       # norm -> qkv of the C=256 block
     (5000, 2048, 256, "swiglu", False),  # LayerNormMLP front half
     (333, 96, 32, "gelu", True),
+    (133000, 96, 32, None, False),       # norm -> qkv of a C=32 level, 512-row configuration, half-full chunk
     (1000, 192, 64, None, True),
     (2049, 256, 128, "relu", False),
 ])
