@@ -32,7 +32,7 @@ constexpr size_t xs_lds_bytes() {
   const size_t wbuf = (size_t)NBUF * G::CHUNK_BYTES;
   const size_t xpatch = (size_t)WAVES * 32 * (G::KP + 8) * 2;
   const size_t front = wbuf > xpatch ? wbuf : xpatch;
-  return front + (size_t)WAVES * 32 * kPatchRow * 2 + (size_t)2 * NBUF * kXsChunk * 4;
+  return front + (size_t)WAVES * 32 * kPatchRow * 2 + (size_t)NBUF * 1024;
 }
 
 // EPI: 0 = bias only, 1 = runtime activation and / or residual.
