@@ -29,8 +29,8 @@ __device__ __forceinline__ uint32_t tile_pos(uint32_t w, uint32_t j, uint32_t l)
   return w * (kWave * ITEMS) + j * kWave + l;
 }
 
-template <int ITEMS>
-__global__ __launch_bounds__(kPshThreads) void psh_hash_hist_kernel(
+template <int THREADS, int ITEMS>
+__global__ __launch_bounds__(THREADS) void psh_hash_hist_kernel(
     const uint16_t* __restrict__ coord, uint16_t* __restrict__ bucket_id, const uint32_t* __restrict__ batch_sep,
     const uint16_t* __restrict__ bbox_min, const uint16_t* __restrict__ bbox_max, uint32_t num_vox,
     uint32_t divisor16, uint32_t num_bucket, uint32_t hash_type, uint32_t* __restrict__ tile_hist,
@@ -39,10 +39,10 @@ __global__ __launch_bounds__(kPshThreads) void psh_hash_hist_kernel(
   const uint32_t cloud = blockIdx.y, tile = blockIdx.x, tid = threadIdx.x;
   const uint32_t start = cloud ? batch_sep[cloud - 1] : 0u;
   const uint32_t n = batch_sep[cloud] - start;
-  const uint32_t tile0 = tile * (kPshThreads * ITEMS);
+  const uint32_t tile0 = tile * (THREADS * ITEMS);
   if (tile0 >= n) return;  // uniform for the workgroup
 
-  for (uint32_t b = tid; b < num_bucket; b += kPshThreads) lds_hist[b] = 0u;
+  for (uint32_t b = tid; b < num_bucket; b += THREADS) lds_hist[b] = 0u;
   VoxAxis ax[3];
 #pragma unroll
   for (int d = 0; d < 3; ++d) ax[d] = make_vox_axis(bbox_min[d], bbox_max[d], num_vox);
@@ -66,7 +66,7 @@ __global__ __launch_bounds__(kPshThreads) void psh_hash_hist_kernel(
   }
   __syncthreads();
   uint32_t* out = tile_hist + ((size_t)cloud * max_tiles + tile) * num_bucket;
-  for (uint32_t b = tid; b < num_bucket; b += kPshThreads) out[b] = lds_hist[b];
+  for (uint32_t b = tid; b < num_bucket; b += THREADS) out[b] = lds_hist[b];
 }
 
 // ---- K2a: exclusive prefix of tile_hist over the tiles of a cloud -------------------------------
@@ -201,8 +201,12 @@ __global__ __launch_bounds__(kPshThreads) void psh_bucket_plan_kernel(
   for (uint32_t b = tid; b < num_bucket; b += kPshThreads) cumsum_counter[(size_t)cloud * num_bucket + b] = s_fin[b];
 }
 
-template <int ITEMS, bool REBAL>
-__global__ __launch_bounds__(kPshThreads) void psh_rank_scatter_kernel(
+// STAGE (large tiles): the tile's rows are first laid out in LDS in (bucket, slot) order and then written
+// run by run, so that a bucket's rows of this tile reach memory as one contiguous piece instead of
+// isolated 6-byte writes (each of which costs a whole memory burst).  Rows moved by the rebalance are
+// written directly.
+template <int THREADS, int ITEMS, bool REBAL, bool STAGE>
+__global__ __launch_bounds__(THREADS) void psh_rank_scatter_kernel(
     const uint16_t* __restrict__ coord, uint16_t* __restrict__ bucket_id,
     uint32_t* __restrict__ bucket_offset, const uint32_t* __restrict__ batch_sep, uint32_t batch_size,
     const uint32_t* __restrict__ tile_base, const uint32_t* __restrict__ bucket_counter,
@@ -213,10 +217,10 @@ __global__ __launch_bounds__(kPshThreads) void psh_rank_scatter_kernel(
   const uint32_t cloud = blockIdx.y, tile = blockIdx.x, tid = threadIdx.x;
 
   if (cloud == batch_size) {  // tail padding rows [total_n, pad_to_n)
-    const uint32_t row0 = total_n + tile * (kPshThreads * ITEMS);
+    const uint32_t row0 = total_n + tile * (THREADS * ITEMS);
 #pragma unroll
     for (int j = 0; j < ITEMS; ++j) {
-      const uint32_t r = row0 + j * kPshThreads + tid;
+      const uint32_t r = row0 + j * THREADS + tid;
       if (r < pad_to_n) {
         uint16_t* q = scatter_coord + 3 * (size_t)r;
         q[0] = pad_bits; q[1] = pad_bits; q[2] = pad_bits;
@@ -227,11 +231,11 @@ __global__ __launch_bounds__(kPshThreads) void psh_rank_scatter_kernel(
 
   const uint32_t start = cloud ? batch_sep[cloud - 1] : 0u;
   const uint32_t n = batch_sep[cloud] - start;
-  const uint32_t tile0 = tile * (kPshThreads * ITEMS);
+  const uint32_t tile0 = tile * (THREADS * ITEMS);
   if (tile0 >= n) return;
 
-  uint32_t* whist = lds;                               // [kPshWaves][NB] per-wave counts
-  uint32_t* row_base = lds + kPshWaves * num_bucket;   // [NB] first output row of the bucket (final layout)
+  uint32_t* whist = lds;                               // [(THREADS / kWave)][NB] per-wave counts
+  uint32_t* row_base = lds + (THREADS / kWave) * num_bucket;   // [NB] first output row of the bucket (final layout)
   uint32_t* slot_base = row_base + num_bucket;         // [NB] tile base inside the first-hash bucket
   uint32_t* s_cnt = slot_base + num_bucket;            // REBAL: [NB] first-hash counts
   uint32_t* s_over = s_cnt + num_bucket;               // REBAL: [NB] exclusive scan of the overflow
@@ -240,9 +244,9 @@ __global__ __launch_bounds__(kPshThreads) void psh_rank_scatter_kernel(
   const uint32_t* cs = cumsum_counter + (size_t)cloud * num_bucket;
   const uint32_t* fin = bucket_counter + (size_t)cloud * num_bucket;
   const uint32_t* pl = plan + (size_t)cloud * (3 * num_bucket + 4);
-  for (uint32_t b = tid; b < num_bucket; b += kPshThreads) {
+  for (uint32_t b = tid; b < num_bucket; b += THREADS) {
 #pragma unroll
-    for (int w = 0; w < kPshWaves; ++w) whist[w * num_bucket + b] = 0u;
+    for (int w = 0; w < (THREADS / kWave); ++w) whist[w * num_bucket + b] = 0u;
     slot_base[b] = tb[b];
     row_base[b] = start + (cs[b] - fin[b]);  // exclusive cumsum of the final counts
     if (REBAL) {
@@ -252,15 +256,24 @@ __global__ __launch_bounds__(kPshThreads) void psh_rank_scatter_kernel(
     }
   }
   const uint32_t tot_free = REBAL ? pl[3 * num_bucket] : 0u;
+  // STAGE: inclusive scan of the tile's own bucket counts, then the staged ids and rows
+  uint32_t* linc = s_free + num_bucket;                                     // [NB]
+  uint16_t* s_id = reinterpret_cast<uint16_t*>(linc + num_bucket + 4);      // [tile] first-hash bucket, 0xFFFF = written directly
+  uint16_t* s_xyz = s_id + THREADS * ITEMS;                                  // [tile][3]
   __syncthreads();
 
   const uint32_t w = tid / kWave, l = tid % kWave;
   uint32_t* mine = whist + w * num_bucket;
   uint32_t id[ITEMS], rank[ITEMS];
+  uint16_t px[ITEMS], py[ITEMS], pz[ITEMS];   // the rows, requested up front so that their latency hides behind the ranking
 #pragma unroll
   for (int j = 0; j < ITEMS; ++j) {
     const uint32_t local = tile0 + tile_pos<ITEMS>(w, j, l);
-    id[j] = (local < n) ? (uint32_t)bucket_id[(size_t)start + local] : 0xFFFFFFFFu;
+    const bool in = local < n;
+    const size_t g = (size_t)start + (in ? local : 0u);
+    id[j] = in ? (uint32_t)bucket_id[g] : 0xFFFFFFFFu;
+    const uint16_t* p = coord + 3 * g;
+    px[j] = p[0]; py[j] = p[1]; pz[j] = p[2];
   }
 #pragma unroll
   for (int j = 0; j < ITEMS; ++j) {
@@ -276,16 +289,21 @@ __global__ __launch_bounds__(kPshThreads) void psh_rank_scatter_kernel(
   }
   __syncthreads();
   // per-wave counts -> exclusive prefix over waves
-  for (uint32_t b = tid; b < num_bucket; b += kPshThreads) {
+  for (uint32_t b = tid; b < num_bucket; b += THREADS) {
     uint32_t run = 0;
 #pragma unroll
-    for (int ww = 0; ww < kPshWaves; ++ww) {
+    for (int ww = 0; ww < (THREADS / kWave); ++ww) {
       const uint32_t c = whist[ww * num_bucket + b];
       whist[ww * num_bucket + b] = run;
       run += c;
     }
+    if (STAGE) linc[b] = run;
   }
   __syncthreads();
+  if (STAGE) {
+    if (tid < kWave) wave0_inclusive_scan(linc, linc, num_bucket, tid);
+    __syncthreads();
+  }
 #pragma unroll
   for (int j = 0; j < ITEMS; ++j) {
     if (id[j] == 0xFFFFFFFFu) continue;
@@ -311,10 +329,34 @@ __global__ __launch_bounds__(kPshThreads) void psh_rank_scatter_kernel(
       bucket_id[g] = (uint16_t)bucket;
     }
     bucket_offset[g] = slot;
+    if (STAGE) {
+      const uint32_t first = id[j];
+      const uint32_t pos = (first ? linc[first - 1] : 0u) + mine[first] + rank[j];   // (bucket, slot) order inside the tile
+      const bool moved = REBAL && bucket != first;
+      s_id[pos] = moved ? (uint16_t)0xFFFFu : (uint16_t)first;
+      if (!moved) {
+        s_xyz[3 * pos + 0] = px[j]; s_xyz[3 * pos + 1] = py[j]; s_xyz[3 * pos + 2] = pz[j];
+        continue;
+      }
+    }
     const size_t dst = (size_t)row_base[bucket] + slot;
-    const uint16_t* p = coord + 3 * g;
     uint16_t* q = scatter_coord + 3 * dst;
-    q[0] = p[0]; q[1] = p[1]; q[2] = p[2];
+    q[0] = px[j]; q[1] = py[j]; q[2] = pz[j];
+  }
+  if (STAGE) {
+    __syncthreads();
+    const uint32_t total = linc[num_bucket - 1];
+#pragma unroll
+    for (int j = 0; j < ITEMS; ++j) {
+      const uint32_t pos = j * THREADS + tid;
+      if (pos >= total) break;
+      const uint32_t b = s_id[pos];
+      if (b == 0xFFFFu) continue;
+      // unmoved rows keep their first-hash bucket: slot = tile base + rank inside the tile
+      const size_t dst = (size_t)row_base[b] + slot_base[b] + (pos - (b ? linc[b - 1] : 0u));
+      uint16_t* q = scatter_coord + 3 * dst;
+      q[0] = s_xyz[3 * pos + 0]; q[1] = s_xyz[3 * pos + 1]; q[2] = s_xyz[3 * pos + 2];
+    }
   }
 }
 
@@ -375,16 +417,16 @@ static uint32_t pick_items(uint32_t instance_max_n, uint32_t batch_size) {
   return 1;
 }
 
-template <int ITEMS, bool REBAL>
+template <int THREADS, int ITEMS, bool REBAL, bool STAGE>
 static void launch_psh(const uint16_t* coord, uint16_t* bucket_id, uint32_t* bucket_counter, uint32_t* bucket_offset,
                        const uint32_t* batch_sep, uint32_t batch_size, uint32_t total_n, uint32_t num_bucket,
                        uint32_t divisor16, uint32_t bucket_size, uint32_t num_vox, const uint16_t* bbox_min,
                        const uint16_t* bbox_max, uint32_t* cumsum_counter, uint16_t* scatter_coord, uint32_t pad_to_n,
                        uint16_t pad_bits, uint32_t hash_type, uint32_t* tile_hist, uint32_t* cnt_ws, uint32_t* plan_ws,
                        uint32_t max_tiles, uint32_t nbits, hipStream_t stream) {
-  const uint32_t tile_pts = kPshThreads * ITEMS;
+  const uint32_t tile_pts = THREADS * ITEMS;
   if (max_tiles > 0 && batch_size > 0) {
-    hipLaunchKernelGGL(psh_hash_hist_kernel<ITEMS>, dim3(max_tiles, batch_size), dim3(kPshThreads),
+    hipLaunchKernelGGL((psh_hash_hist_kernel<THREADS, ITEMS>), dim3(max_tiles, batch_size), dim3(THREADS),
                        num_bucket * sizeof(uint32_t), stream, coord, bucket_id, batch_sep, bbox_min, bbox_max, num_vox,
                        divisor16, num_bucket, hash_type, tile_hist, max_tiles);
     hipLaunchKernelGGL(psh_tile_scan_kernel, dim3(cdiv_u32(num_bucket, kWave), batch_size), dim3(kScanWaves * kWave), 0,
@@ -396,8 +438,12 @@ static void launch_psh(const uint16_t* coord, uint16_t* bucket_id, uint32_t* buc
   const uint32_t pad_tiles = cdiv_u32(pad_to_n - total_n, tile_pts);
   const uint32_t gx = max_tiles > pad_tiles ? max_tiles : pad_tiles;
   if (gx > 0) {
-    hipLaunchKernelGGL((psh_rank_scatter_kernel<ITEMS, REBAL>), dim3(gx, batch_size + (pad_tiles ? 1 : 0)),
-                       dim3(kPshThreads), (kPshWaves + 5) * num_bucket * sizeof(uint32_t), stream, coord, bucket_id,
+    const size_t lds = ((size_t)(THREADS / kWave + 5) * num_bucket +
+                        (STAGE ? num_bucket + 4 + (size_t)2 * THREADS * ITEMS : 0)) * sizeof(uint32_t);
+    auto kern = psh_rank_scatter_kernel<THREADS, ITEMS, REBAL, STAGE>;
+    if (lds > 64 * 1024) (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    hipLaunchKernelGGL(kern, dim3(gx, batch_size + (pad_tiles ? 1 : 0)),
+                       dim3(THREADS), lds, stream, coord, bucket_id,
                        bucket_offset, batch_sep, batch_size, tile_hist, bucket_counter, cumsum_counter, plan_ws,
                        num_bucket, nbits, max_tiles, bucket_size, scatter_coord, total_n, pad_to_n, pad_bits);
   }
@@ -443,8 +489,11 @@ int f3d_batch_psh_scatter_pad_hash(const f3d_half_t* coord, uint16_t* bucket_id,
   DeviceGuard guard(device);
   F3D_CHECK_ARG(guard.ok, "cannot select device %d", device);
   hipStream_t s = (hipStream_t)stream;
-  const uint32_t items = pick_items(instance_max_n, batch_size);
-  const uint32_t tile_pts = kPshThreads * items;
+  // Inputs large enough to fill the chip with 8192-point tiles use 1024-thread workgroups that stage
+  // the scatter through LDS; smaller ones use 256-thread workgroups with tiles sized for parallelism.
+  const bool big = (uint64_t)cdiv_u32(instance_max_n, 8192u) * batch_size >= 512u;
+  const uint32_t items = big ? 8u : pick_items(instance_max_n, batch_size);
+  const uint32_t tile_pts = (big ? 1024u : (uint32_t)kPshThreads) * items;
   const uint32_t max_tiles = cdiv_u32(instance_max_n, tile_pts);
   const size_t hist_words = (size_t)batch_size * max_tiles * num_bucket;
   const size_t cnt_words = (size_t)batch_size * num_bucket;
@@ -461,24 +510,28 @@ int f3d_batch_psh_scatter_pad_hash(const f3d_half_t* coord, uint16_t* bucket_id,
   __builtin_memcpy(&pad_bits, &pad_h, 2);
 
   SyncBracket sync(s);
-#define F3D_PSH_CASE(I)                                                                                          \
-  case I:                                                                                                        \
-    if (rebal)                                                                                                   \
-      launch_psh<I, true>(coord, bucket_id, bucket_counter, bucket_offset, batch_sep, batch_size, total_n, num_bucket, \
-                          div16, bucket_size, num_vox, bbox_min, bbox_max, cumsum_counter, scatter_coord, pad_to_n,    \
-                          pad_bits, hash_type, tile_hist, cnt_ws, plan_ws, max_tiles, nbits, s);                 \
-    else                                                                                                         \
-      launch_psh<I, false>(coord, bucket_id, bucket_counter, bucket_offset, batch_sep, batch_size, total_n, num_bucket, \
-                           div16, bucket_size, num_vox, bbox_min, bbox_max, cumsum_counter, scatter_coord, pad_to_n,   \
-                           pad_bits, hash_type, tile_hist, cnt_ws, plan_ws, max_tiles, nbits, s);                \
+#define F3D_PSH_ARGS                                                                                              \
+  coord, bucket_id, bucket_counter, bucket_offset, batch_sep, batch_size, total_n, num_bucket, div16, bucket_size, \
+      num_vox, bbox_min, bbox_max, cumsum_counter, scatter_coord, pad_to_n, pad_bits, hash_type, tile_hist, cnt_ws, \
+      plan_ws, max_tiles, nbits, s
+#define F3D_PSH_CASE(I)                                                                  \
+  case I:                                                                                \
+    if (rebal) launch_psh<kPshThreads, I, true, false>(F3D_PSH_ARGS);                    \
+    else launch_psh<kPshThreads, I, false, false>(F3D_PSH_ARGS);                         \
     break;
-  switch (items) {
-    F3D_PSH_CASE(1)
-    F3D_PSH_CASE(2)
-    F3D_PSH_CASE(4)
-    F3D_PSH_CASE(8)
+  if (big) {
+    if (rebal) launch_psh<1024, 8, true, true>(F3D_PSH_ARGS);
+    else launch_psh<1024, 8, false, true>(F3D_PSH_ARGS);
+  } else {
+    switch (items) {
+      F3D_PSH_CASE(1)
+      F3D_PSH_CASE(2)
+      F3D_PSH_CASE(4)
+      F3D_PSH_CASE(8)
+    }
   }
 #undef F3D_PSH_CASE
+#undef F3D_PSH_ARGS
   F3D_CHECK_HIP(hipGetLastError());
   return F3D_OK;
 }

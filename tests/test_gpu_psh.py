@@ -149,6 +149,30 @@ def test_python_wrapper_and_saturating_size_properties(oracle):
     assert dst.unique().numel() == n_c * b
 
 
+@pytest.mark.parametrize("rebalance", [0, 1])
+def test_large_tile_configuration_bit_exact(oracle, rebalance):
+    """Batches big enough for the 8192-point tiles (LDS-staged scatter): 72 ragged clouds, 4.5 M points, half of
+    them clustered so that buckets overflow; ids, counts, slots and scattered rows bit-exact vs the oracle"""
+    from flash3dtransformer_amd import synth
+    rng = np.random.default_rng(77)
+    clouds = []
+    for i in range(72):
+        n = int(rng.integers(56000, 70000))
+        if i % 2:
+            clouds.append((rng.normal(0, 8.0, (n, 3)) * np.array([1.0, 1.0, 0.1])).astype(np.float32))
+        else:
+            clouds.append(rng.uniform(0, 51.2, (n, 3)).astype(np.float32))
+    clouds[5] = clouds[5][:8191]        # one tile minus one point
+    clouds[6] = clouds[6][:8193]        # one tile plus one point
+    coords, seps = synth.batch_of(clouds)
+    assert -(-max(len(c) for c in clouds) // 8192) * len(clouds) >= 512
+    out = _run_psh(coords, seps, 512, 2, 3072, oracle, rebalance=rebalance)
+    _check_against_oracle(coords, seps, out, 2, oracle, rebalance=rebalance)
+    assert not np.isnan(out["scat"]).any()
+    from flash3dtransformer_amd.lib import pshattn
+    pshattn.DeviceManagerSingleton.instance().set_psh_rebalance(1)
+
+
 @pytest.mark.parametrize("case", ["lidar", "uniform_exact_capacity", "ragged"])
 def test_rebalance_bit_exact_and_reference_invariants(oracle, case):
     """A4 (deterministic overflow rebalance + recycle): final ids, counts, slots and scattered rows
