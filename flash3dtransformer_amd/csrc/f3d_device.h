@@ -136,13 +136,16 @@ __device__ __forceinline__ uint32_t mask_rank(uint64_t mask) {
 // Lanes of the wave whose `key` (low `nbits` bits significant) equals this lane's, restricted to
 // lanes with `valid` set.  One ballot per key bit.
 __device__ __forceinline__ uint64_t match_any(uint32_t key, uint32_t nbits, bool valid) {
-  uint64_t mask = __ballot(valid);
+  const uint64_t all = __ballot(valid);
+  uint32_t lo = (uint32_t)all, hi = (uint32_t)(all >> 32);
   for (uint32_t k = 0; k < nbits; ++k) {
-    bool bit = (key >> k) & 1u;
-    uint64_t b = __ballot(bit);
-    mask &= bit ? b : ~b;
+    const int32_t sbit = __builtin_amdgcn_sbfe((int32_t)key, k, 1u);   // all ones where this lane's bit is set
+    const uint32_t sx = (uint32_t)sbit;
+    const uint64_t b = __ballot(sbit < 0);
+    lo &= ~((uint32_t)b ^ sx);                    // keep the lanes whose bit equals mine
+    hi &= ~((uint32_t)(b >> 32) ^ sx);
   }
-  return mask;
+  return ((uint64_t)hi << 32) | lo;
 }
 
 }  // namespace f3d

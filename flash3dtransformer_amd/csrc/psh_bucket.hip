@@ -201,10 +201,30 @@ __global__ __launch_bounds__(kPshThreads) void psh_bucket_plan_kernel(
   for (uint32_t b = tid; b < num_bucket; b += kPshThreads) cumsum_counter[(size_t)cloud * num_bucket + b] = s_fin[b];
 }
 
-// STAGE (large tiles): the tile's rows are first laid out in LDS in (bucket, slot) order and then written
-// run by run, so that a bucket's rows of this tile reach memory as one contiguous piece instead of
-// isolated 6-byte writes (each of which costs a whole memory burst).  Rows moved by the rebalance are
-// written directly.
+// Phases of one workgroup (one tile of THREADS * ITEMS points of one cloud):
+//   1. every wave ranks its points inside their first-hash buckets (match + one LDS atomic per group),
+//   2. the per-wave counts become exclusive prefixes over the waves,
+//   3. every point gets its stable slot; rows that stay in their first-hash bucket are written (or
+//      staged), rows in the overflow of a bucket are gathered densely over the lanes of the wave and
+//      resolved there, so the search for their new bucket runs once per 64 of them rather than once
+//      per 64 points,
+//   4. STAGE (large tiles): the tile's rows are laid out in LDS in (bucket, slot) order and written run
+//      by run, so that a bucket's rows of this tile reach memory as one contiguous piece instead of
+//      isolated 6-byte writes.
+// LDS layout in 32-bit words: head (per-wave counts [waves][NB]; STAGE reuses it for the staged rows,
+// x|y as one word per row followed by z as 16 bits per row), then row_base, slot_base, s_cnt, s_over,
+// s_free, [STAGE: linc, dst_base], then the tail (STAGE: staged bucket ids, 16 bits per row, which
+// phase 3 borrows for the per-wave overflow lists; otherwise those lists, 64 entries of 16 bytes per wave).
+template <int THREADS, int ITEMS, bool STAGE>
+__host__ __device__ constexpr size_t psh_scatter_lds_bytes(uint32_t num_bucket) {
+  const size_t waves = THREADS / kWave, tile = (size_t)THREADS * ITEMS;
+  const size_t wave_words = waves * num_bucket, row_words = tile * 3 / 2;
+  const size_t head = (STAGE && row_words > wave_words) ? row_words : wave_words;
+  const size_t tables = (size_t)(STAGE ? 7 : 5) * num_bucket;
+  const size_t tail = STAGE ? (tile / 2 > waves * 256 ? tile / 2 : waves * 256) : waves * 256;
+  return (head + tables + tail) * sizeof(uint32_t);
+}
+
 template <int THREADS, int ITEMS, bool REBAL, bool STAGE>
 __global__ __launch_bounds__(THREADS) void psh_rank_scatter_kernel(
     const uint16_t* __restrict__ coord, uint16_t* __restrict__ bucket_id,
@@ -214,10 +234,12 @@ __global__ __launch_bounds__(THREADS) void psh_rank_scatter_kernel(
     uint32_t nbits, uint32_t max_tiles, uint32_t bucket_size, uint16_t* __restrict__ scatter_coord, uint32_t total_n,
     uint32_t pad_to_n, uint16_t pad_bits) {
   extern __shared__ uint32_t lds[];
+  constexpr uint32_t kWaves = THREADS / kWave, kTile = THREADS * ITEMS;
+  static_assert(!STAGE || kTile / 2 >= kWaves * 256, "the staged ids must cover the per-wave overflow lists");
   const uint32_t cloud = blockIdx.y, tile = blockIdx.x, tid = threadIdx.x;
 
   if (cloud == batch_size) {  // tail padding rows [total_n, pad_to_n)
-    const uint32_t row0 = total_n + tile * (THREADS * ITEMS);
+    const uint32_t row0 = total_n + tile * kTile;
 #pragma unroll
     for (int j = 0; j < ITEMS; ++j) {
       const uint32_t r = row0 + j * THREADS + tid;
@@ -231,22 +253,32 @@ __global__ __launch_bounds__(THREADS) void psh_rank_scatter_kernel(
 
   const uint32_t start = cloud ? batch_sep[cloud - 1] : 0u;
   const uint32_t n = batch_sep[cloud] - start;
-  const uint32_t tile0 = tile * (THREADS * ITEMS);
+  const uint32_t tile0 = tile * kTile;
   if (tile0 >= n) return;
 
-  uint32_t* whist = lds;                               // [(THREADS / kWave)][NB] per-wave counts
-  uint32_t* row_base = lds + (THREADS / kWave) * num_bucket;   // [NB] first output row of the bucket (final layout)
+  const uint32_t head_words = (STAGE && kTile * 3 / 2 > kWaves * num_bucket) ? kTile * 3 / 2 : kWaves * num_bucket;
+  uint32_t* whist = lds;                               // [kWaves][NB] per-wave counts
+  uint32_t* row_base = lds + head_words;               // [NB] first output row of the bucket (final layout)
   uint32_t* slot_base = row_base + num_bucket;         // [NB] tile base inside the first-hash bucket
   uint32_t* s_cnt = slot_base + num_bucket;            // REBAL: [NB] first-hash counts
   uint32_t* s_over = s_cnt + num_bucket;               // REBAL: [NB] exclusive scan of the overflow
   uint32_t* s_free = s_over + num_bucket;              // REBAL: [NB] inclusive scan of the free capacity
+  uint32_t* linc = s_free + num_bucket;                // STAGE: [NB] inclusive scan of the tile's own bucket counts
+  uint32_t* dst_base = linc + num_bucket;              // STAGE: [NB] output row of staged position 0 of the bucket
+  uint32_t* tail = s_free + (STAGE ? 3 : 1) * num_bucket;
+  uint32_t* s_xy = lds;                                // STAGE: [tile] x | y << 16, over the per-wave counts
+  uint16_t* s_z = reinterpret_cast<uint16_t*>(lds + kTile);   // STAGE: [tile]
+  uint16_t* s_id = reinterpret_cast<uint16_t*>(tail);  // STAGE: [tile] first-hash bucket, 0xFFFF = written directly
+  const uint32_t w = tid / kWave, l = tid % kWave;
+  uint4* ov_list = reinterpret_cast<uint4*>(tail) + w * kWave;   // this wave's gathered overflow rows: unit, source, x|y, z
+
   const uint32_t* tb = tile_base + ((size_t)cloud * max_tiles + tile) * num_bucket;
   const uint32_t* cs = cumsum_counter + (size_t)cloud * num_bucket;
   const uint32_t* fin = bucket_counter + (size_t)cloud * num_bucket;
   const uint32_t* pl = plan + (size_t)cloud * (3 * num_bucket + 4);
   for (uint32_t b = tid; b < num_bucket; b += THREADS) {
 #pragma unroll
-    for (int w = 0; w < (THREADS / kWave); ++w) whist[w * num_bucket + b] = 0u;
+    for (uint32_t ww = 0; ww < kWaves; ++ww) whist[ww * num_bucket + b] = 0u;
     slot_base[b] = tb[b];
     row_base[b] = start + (cs[b] - fin[b]);  // exclusive cumsum of the final counts
     if (REBAL) {
@@ -256,16 +288,10 @@ __global__ __launch_bounds__(THREADS) void psh_rank_scatter_kernel(
     }
   }
   const uint32_t tot_free = REBAL ? pl[3 * num_bucket] : 0u;
-  // STAGE: inclusive scan of the tile's own bucket counts, then the staged ids and rows
-  uint32_t* linc = s_free + num_bucket;                                     // [NB]
-  uint16_t* s_id = reinterpret_cast<uint16_t*>(linc + num_bucket + 4);      // [tile] first-hash bucket, 0xFFFF = written directly
-  uint16_t* s_xyz = s_id + THREADS * ITEMS;                                  // [tile][3]
-  __syncthreads();
 
-  const uint32_t w = tid / kWave, l = tid % kWave;
-  uint32_t* mine = whist + w * num_bucket;
-  uint32_t id[ITEMS], rank[ITEMS];
-  uint16_t px[ITEMS], py[ITEMS], pz[ITEMS];   // the rows, requested up front so that their latency hides behind the ranking
+  // the tile's ids and rows, requested up front so that their latency hides behind the ranking
+  uint32_t id[ITEMS], rank[ITEMS], pxy[ITEMS];
+  uint16_t pz[ITEMS];
 #pragma unroll
   for (int j = 0; j < ITEMS; ++j) {
     const uint32_t local = tile0 + tile_pos<ITEMS>(w, j, l);
@@ -273,8 +299,12 @@ __global__ __launch_bounds__(THREADS) void psh_rank_scatter_kernel(
     const size_t g = (size_t)start + (in ? local : 0u);
     id[j] = in ? (uint32_t)bucket_id[g] : 0xFFFFFFFFu;
     const uint16_t* p = coord + 3 * g;
-    px[j] = p[0]; py[j] = p[1]; pz[j] = p[2];
+    pxy[j] = (uint32_t)p[0] | ((uint32_t)p[1] << 16);
+    pz[j] = p[2];
   }
+  __syncthreads();
+
+  uint32_t* mine = whist + w * num_bucket;
 #pragma unroll
   for (int j = 0; j < ITEMS; ++j) {
     const bool valid = id[j] != 0xFFFFFFFFu;
@@ -292,7 +322,7 @@ __global__ __launch_bounds__(THREADS) void psh_rank_scatter_kernel(
   for (uint32_t b = tid; b < num_bucket; b += THREADS) {
     uint32_t run = 0;
 #pragma unroll
-    for (int ww = 0; ww < (THREADS / kWave); ++ww) {
+    for (uint32_t ww = 0; ww < kWaves; ++ww) {
       const uint32_t c = whist[ww * num_bucket + b];
       whist[ww * num_bucket + b] = run;
       run += c;
@@ -303,17 +333,21 @@ __global__ __launch_bounds__(THREADS) void psh_rank_scatter_kernel(
   if (STAGE) {
     if (tid < kWave) wave0_inclusive_scan(linc, linc, num_bucket, tid);
     __syncthreads();
+    // staged position p of bucket b goes to row row_base[b] + slot_base[b] + (p - first staged position of b)
+    for (uint32_t b = tid; b < num_bucket; b += THREADS)
+      dst_base[b] = row_base[b] + slot_base[b] - (b ? linc[b - 1] : 0u);
   }
-#pragma unroll
-  for (int j = 0; j < ITEMS; ++j) {
-    if (id[j] == 0xFFFFFFFFu) continue;
-    const uint32_t local = tile0 + tile_pos<ITEMS>(w, j, l);
-    const size_t g = (size_t)start + local;
-    uint32_t bucket = id[j];
-    uint32_t slot = slot_base[bucket] + mine[bucket] + rank[j];  // stable slot in the first-hash bucket
-    if (REBAL && bucket != 0 && slot >= bucket_size) {
-      // k-th overflow unit of the cloud takes the k-th free unit; none left -> recycle bucket 0
-      const uint32_t k = s_over[bucket] + (slot - bucket_size);
+
+  // Rows in the overflow of their bucket: the k-th overflow unit of the cloud takes the k-th free unit;
+  // none left -> recycle bucket 0.  Lane i of the wave resolves the i-th gathered row.
+  uint32_t ov_n = 0;   // wave-uniform
+  auto resolve_overflow = [&]() {
+    __builtin_amdgcn_wave_barrier();
+    if (l < ov_n) {
+      const uint4 e = ov_list[l];
+      const uint32_t k = e.x;
+      const size_t g = (size_t)start + tile0 + (w * (kWave * ITEMS) + e.y);
+      uint32_t bucket, slot;
       if (k < tot_free) {
         uint32_t lo = 1, hi = num_bucket - 1;  // first bucket whose inclusive free count exceeds k
         while (lo < hi) {
@@ -327,23 +361,53 @@ __global__ __launch_bounds__(THREADS) void psh_rank_scatter_kernel(
         slot = s_cnt[0] + (k - tot_free);
       }
       bucket_id[g] = (uint16_t)bucket;
+      bucket_offset[g] = slot;
+      uint16_t* q = scatter_coord + 3 * ((size_t)row_base[bucket] + slot);
+      q[0] = (uint16_t)e.z; q[1] = (uint16_t)(e.z >> 16); q[2] = (uint16_t)e.w;
     }
-    bucket_offset[g] = slot;
-    if (STAGE) {
-      const uint32_t first = id[j];
-      const uint32_t pos = (first ? linc[first - 1] : 0u) + mine[first] + rank[j];   // (bucket, slot) order inside the tile
-      const bool moved = REBAL && bucket != first;
-      s_id[pos] = moved ? (uint16_t)0xFFFFu : (uint16_t)first;
-      if (!moved) {
-        s_xyz[3 * pos + 0] = px[j]; s_xyz[3 * pos + 1] = py[j]; s_xyz[3 * pos + 2] = pz[j];
-        continue;
+    __builtin_amdgcn_wave_barrier();
+    ov_n = 0;
+  };
+
+#pragma unroll
+  for (int j = 0; j < ITEMS; ++j) {
+    const bool valid = id[j] != 0xFFFFFFFFu;
+    const uint32_t bucket = valid ? id[j] : 0u;
+    const uint32_t in_tile = mine[bucket] + rank[j];
+    const uint32_t slot = slot_base[bucket] + in_tile;  // stable slot in the first-hash bucket
+    const bool over = REBAL && valid && bucket != 0 && slot >= bucket_size;
+    if (REBAL) {
+      const uint64_t ovm = __ballot(over);
+      if (ovm != 0) {
+        const uint32_t n_ov = (uint32_t)__popcll(ovm);
+        if (ov_n + n_ov > kWave) resolve_overflow();
+        if (over)
+          ov_list[ov_n + mask_rank(ovm)] = make_uint4(s_over[bucket] + (slot - bucket_size), j * kWave + l, pxy[j], pz[j]);
+        ov_n += n_ov;
       }
     }
-    const size_t dst = (size_t)row_base[bucket] + slot;
-    uint16_t* q = scatter_coord + 3 * dst;
-    q[0] = px[j]; q[1] = py[j]; q[2] = pz[j];
+    if (STAGE) rank[j] = ((bucket ? linc[bucket - 1] : 0u) + in_tile) | (over ? 0x80000000u : 0u);  // staged position
+    if (valid && !over) {
+      const size_t g = (size_t)start + tile0 + tile_pos<ITEMS>(w, j, l);
+      bucket_offset[g] = slot;
+      if (!STAGE) {
+        uint16_t* q = scatter_coord + 3 * ((size_t)row_base[bucket] + slot);
+        q[0] = (uint16_t)pxy[j]; q[1] = (uint16_t)(pxy[j] >> 16); q[2] = pz[j];
+      }
+    }
   }
+  if (REBAL) resolve_overflow();
+
   if (STAGE) {
+    __syncthreads();   // the per-wave counts and overflow lists are consumed: their space takes the rows and ids
+#pragma unroll
+    for (int j = 0; j < ITEMS; ++j) {
+      if (id[j] == 0xFFFFFFFFu) continue;
+      const uint32_t pos = rank[j] & 0x7FFFFFFFu;
+      s_id[pos] = (rank[j] >> 31) ? (uint16_t)0xFFFFu : (uint16_t)id[j];
+      s_xy[pos] = pxy[j];
+      s_z[pos] = pz[j];
+    }
     __syncthreads();
     const uint32_t total = linc[num_bucket - 1];
 #pragma unroll
@@ -352,10 +416,9 @@ __global__ __launch_bounds__(THREADS) void psh_rank_scatter_kernel(
       if (pos >= total) break;
       const uint32_t b = s_id[pos];
       if (b == 0xFFFFu) continue;
-      // unmoved rows keep their first-hash bucket: slot = tile base + rank inside the tile
-      const size_t dst = (size_t)row_base[b] + slot_base[b] + (pos - (b ? linc[b - 1] : 0u));
-      uint16_t* q = scatter_coord + 3 * dst;
-      q[0] = s_xyz[3 * pos + 0]; q[1] = s_xyz[3 * pos + 1]; q[2] = s_xyz[3 * pos + 2];
+      uint16_t* q = scatter_coord + 3 * (size_t)(dst_base[b] + pos);
+      const uint32_t xy = s_xy[pos];
+      q[0] = (uint16_t)xy; q[1] = (uint16_t)(xy >> 16); q[2] = s_z[pos];
     }
   }
 }
@@ -438,8 +501,7 @@ static void launch_psh(const uint16_t* coord, uint16_t* bucket_id, uint32_t* buc
   const uint32_t pad_tiles = cdiv_u32(pad_to_n - total_n, tile_pts);
   const uint32_t gx = max_tiles > pad_tiles ? max_tiles : pad_tiles;
   if (gx > 0) {
-    const size_t lds = ((size_t)(THREADS / kWave + 5) * num_bucket +
-                        (STAGE ? num_bucket + 4 + (size_t)2 * THREADS * ITEMS : 0)) * sizeof(uint32_t);
+    const size_t lds = psh_scatter_lds_bytes<THREADS, ITEMS, STAGE>(num_bucket);
     auto kern = psh_rank_scatter_kernel<THREADS, ITEMS, REBAL, STAGE>;
     if (lds > 64 * 1024) (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     hipLaunchKernelGGL(kern, dim3(gx, batch_size + (pad_tiles ? 1 : 0)),
@@ -491,9 +553,10 @@ int f3d_batch_psh_scatter_pad_hash(const f3d_half_t* coord, uint16_t* bucket_id,
   hipStream_t s = (hipStream_t)stream;
   // Inputs large enough to fill the chip with 8192-point tiles use 1024-thread workgroups that stage
   // the scatter through LDS; smaller ones use 256-thread workgroups with tiles sized for parallelism.
+  constexpr int kBigThreads = 1024, kBigItems = 8;
   const bool big = (uint64_t)cdiv_u32(instance_max_n, 8192u) * batch_size >= 512u;
-  const uint32_t items = big ? 8u : pick_items(instance_max_n, batch_size);
-  const uint32_t tile_pts = (big ? 1024u : (uint32_t)kPshThreads) * items;
+  const uint32_t items = big ? (uint32_t)kBigItems : pick_items(instance_max_n, batch_size);
+  const uint32_t tile_pts = (big ? (uint32_t)kBigThreads : (uint32_t)kPshThreads) * items;
   const uint32_t max_tiles = cdiv_u32(instance_max_n, tile_pts);
   const size_t hist_words = (size_t)batch_size * max_tiles * num_bucket;
   const size_t cnt_words = (size_t)batch_size * num_bucket;
@@ -520,8 +583,8 @@ int f3d_batch_psh_scatter_pad_hash(const f3d_half_t* coord, uint16_t* bucket_id,
     else launch_psh<kPshThreads, I, false, false>(F3D_PSH_ARGS);                         \
     break;
   if (big) {
-    if (rebal) launch_psh<1024, 8, true, true>(F3D_PSH_ARGS);
-    else launch_psh<1024, 8, false, true>(F3D_PSH_ARGS);
+    if (rebal) launch_psh<kBigThreads, kBigItems, true, true>(F3D_PSH_ARGS);
+    else launch_psh<kBigThreads, kBigItems, false, true>(F3D_PSH_ARGS);
   } else {
     switch (items) {
       F3D_PSH_CASE(1)
