@@ -411,8 +411,8 @@ int f3d_ln_linear_bf16(const f3d_bf16_t* x, uint32_t ldx, const f3d_bf16_t* gamm
   F3D_CHECK_ARG(x && gamma && w && y, "null tensor pointer");
   F3D_CHECK_ARG(act <= F3D_ACT_RELU, "unknown activation id %u", act);
   const uint32_t n_out = act == F3D_ACT_SWIGLU ? n / 2 : n;
-  F3D_CHECK_ARG(k == 32 || k == 64 || k == 128 || k == 256,
-                "No kernel found for LayerNorm+Linear with inner dimension K=%u (supported: 32, 64, 128, 256)", k);
+  F3D_CHECK_ARG(k == 32 || k == 64 || k == 128 || k == 256 || k == 512,
+                "No kernel found for LayerNorm+Linear with inner dimension K=%u (supported: 32, 64, 128, 256, 512)", k);
   F3D_CHECK_ARG(n_out % 8 == 0 && (act != F3D_ACT_SWIGLU || n % 64 == 0), "output width %u must be a multiple of 8", n_out);
   F3D_CHECK_ARG(ldx >= k && ldx % 8 == 0 && ldy >= n_out && ldy % 4 == 0 && (!residual || (ldr >= n_out && ldr % 4 == 0)),
                 "row strides must be aligned and cover a row (ldx=%u ldy=%u ldr=%u)", ldx, ldy, ldr);

@@ -1,5 +1,5 @@
 // Row-panel ("x-stationary") linear layers for gfx950: y = act(LN?(x) wT + bias) (+ residual) for the
-// small inner dimensions of the Flash3D blocks (K = channels, 32..256).
+// small inner dimensions of the Flash3D blocks (K = channels, 32..512).
 //
 // Stands where the reference runs LayerNorm followed by torch.nn.Linear / te.Linear
 // (flash3dxfmr/layers/stage.py:94-97, buck_swin.py:185,194, hourglass.py:99,181-183).
@@ -32,7 +32,7 @@ constexpr size_t xs_lds_bytes() {
   const size_t wbuf = (size_t)NBUF * G::CHUNK_BYTES;
   const size_t xpatch = (size_t)WAVES * 32 * (G::KP + 8) * 2;
   const size_t front = wbuf > xpatch ? wbuf : xpatch;
-  return front + (size_t)WAVES * 32 * kPatchRow * 2 + (size_t)NBUF * 1024;
+  return front + (size_t)WAVES * 32 * kPatchRow * 2 + (size_t)2 * NBUF * kXsChunk * 4;
 }
 
 // EPI: 0 = bias only, 1 = runtime activation and / or residual.
@@ -426,7 +426,7 @@ int launch_xstat_linear(const uint16_t* x, uint32_t ldx, const uint16_t* gamma, 
   if (M == 0) return F3D_OK;
   // whole 32-column tiles; a swiglu chunk pairs 32 value rows with 32 gate rows
   if (swiglu ? N % 64 != 0 : N % 32 != 0) return F3D_ERR_UNSUPPORTED;
-  if (K != 32 && K != 64 && K != 128 && K != 256) return F3D_ERR_UNSUPPORTED;
+  if (K != 32 && K != 64 && K != 128 && K != 256 && K != 512) return F3D_ERR_UNSUPPORTED;
   if ((uint64_t)N * K * 2 >= (1ull << 32)) return F3D_ERR_UNSUPPORTED;   // 32-bit byte offsets into w
   const float* bias_f = nullptr;
   const float* wsum = nullptr;
@@ -458,6 +458,10 @@ int launch_xstat_linear(const uint16_t* x, uint32_t ldx, const uint16_t* gamma, 
     F3D_XS_CASE(64)
     F3D_XS_CASE(128)
     F3D_XS_CASE(256)
+    case 512:
+      // 512 inner features fill the register budget with 32 rows per wave; two 64 KB chunk buffers
+      return launch_k<512, 1, 8, 2>(ln, swiglu, s, x, ldx, eps, w, bias, bias_f, wsum, residual, ldr, y, ldy, M, N,
+                                    run_act, device);
     default: return F3D_ERR_UNSUPPORTED;
   }
 #undef F3D_XS_CASE

@@ -111,7 +111,7 @@ class LayerNorm(nn.Module):
         return forward_only(y.view(x.shape), "LayerNorm", x, self.weight)
 
 
-FUSABLE_LN_WIDTHS = (32, 64, 128, 256)
+FUSABLE_LN_WIDTHS = (32, 64, 128, 256, 512)
 
 
 def is_fusable_layernorm(norm, width: int) -> bool:

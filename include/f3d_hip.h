@@ -165,7 +165,7 @@ int f3d_linear_bf16(const f3d_bf16_t* x, uint32_t ldx, const f3d_bf16_t* w, cons
 
 /* LayerNorm fused into the following linear layer: y = act(LayerNorm(x; gamma, beta, eps) · wᵀ + bias)
  * + residual, the `norm -> qkv` and `LayerNormMLP` front halves of flash3dxfmr/layers/stage.py:94-99.
- * Same tensor contract as f3d_linear_bf16 with k in {32, 64, 128, 256}; gamma [k] bf16, beta [k]
+ * Same tensor contract as f3d_linear_bf16 with k in {32, 64, 128, 256, 512}; gamma [k] bf16, beta [k]
  * bf16 or NULL.  LayerNorm is applied algebraically (w scaled by gamma and rounded to bf16, the row
  * statistics applied to the fp32 accumulators), so roundings fall in other places than in a separate
  * LayerNorm module followed by a Linear; the result is as close to the unrounded mathematics. */

@@ -51,6 +51,10 @@ def test_gemm_sm_bf16_reference_case():
     (3000, 32, 128, None, True, True),         # half-full last chunk of the row-panel kernel (fc2 of a C=32 level)
     (140000, 96, 32, None, True, False),       # the same in the 512-row configuration (qkv of a C=32 level)
     (140000, 32, 32, "gelu", True, True),
+    (3001, 1536, 512, None, True, False),      # qkv of a C=512 level: 512 inner features in the row-panel kernel, ragged M
+    (2500, 512, 512, None, True, True),        # out-projection + residual of that level
+    (2100, 2048, 512, "swiglu", True, False),  # its fc1
+    (700, 256, 512, "gelu", False, True),      # fc2 of a C=256 level
 ])
 def test_linear_epilogues(oracle, M, N, K, act, use_bias, use_res):
     from flash3dtransformer_amd.lib import pshattn
@@ -85,6 +89,8 @@ def test_linear_epilogues(oracle, M, N, K, act, use_bias, use_res):
     (133000, 96, 32, None, False),       # norm -> qkv of a C=32 level, 512-row configuration, half-full chunk
     (1000, 192, 64, None, True),
     (2049, 256, 128, "relu", False),
+    (1900, 1536, 512, None, False),      # norm -> qkv of a C=512 level
+    (1300, 2048, 512, "swiglu", True),   # norm -> fc1 -> gate of that level
 ])
 def test_layernorm_fused_linear(oracle, M, N, K, act, use_res):
     from flash3dtransformer_amd.lib import pshattn
