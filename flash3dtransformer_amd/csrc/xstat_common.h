@@ -70,8 +70,8 @@ struct XsGeom {
   __host__ __device__ static constexpr uint32_t swz(uint32_t row) { return (row / RP) & SWZ_MASK; }
 };
 
-// w' = bf16(w * gamma), wsum and b' (fp32) for the algebraic LayerNorm fold (defined with the linear kernels)
+// w' = bf16(w * gamma) and the per-feature table of the algebraic LayerNorm fold (defined with the linear kernels)
 void launch_ln_fold(const uint16_t* w, const uint16_t* gamma, const uint16_t* beta, const uint16_t* bias, uint16_t* wp,
-                    float* wsum, float* bp, uint32_t N, uint32_t K, hipStream_t s);
+                    uint16_t* lnx, uint32_t N, uint32_t K, hipStream_t s);
 
 }  // namespace f3d

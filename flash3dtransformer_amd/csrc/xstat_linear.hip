@@ -20,8 +20,11 @@
 // LayerNorm is folded algebraically instead of being applied to x:
 //     LN(x) wT + b  =  rstd * (x w'T - mean * wsum) + b',   w' = w * gamma,  wsum[n] = sum_k w'[n][k],
 //                                                            b' = b + w beta.
-// A small kernel prepares w' (bf16), wsum and b' (fp32) per call; the main kernel then only needs the row
-// statistics (one sweep over the registers that hold x) and two fused multiply-adds per output element.
+// A small kernel prepares w' (bf16) and, per output feature, wsum and b' split into high and low bf16 parts; the main
+// kernel needs the row statistics (one sweep over the registers that hold x) and applies the correction on the
+// matrix core: one extra k-step multiplies (wsum_hi, wsum_hi, wsum_lo, b'_hi, b'_hi, b'_lo) by the row's
+// (m_hi, m_lo, m_hi, s_hi, s_lo, s_hi), m = -mean, s = 1 / rstd, which adds -mean * wsum + s * b' to the
+// accumulator to 16 bits of mantissa; the epilogue then multiplies by rstd.
 #include "xstat_common.h"
 
 namespace f3d {
@@ -32,16 +35,16 @@ constexpr size_t xs_lds_bytes() {
   const size_t wbuf = (size_t)NBUF * G::CHUNK_BYTES;
   const size_t xpatch = (size_t)WAVES * 32 * (G::KP + 8) * 2;
   const size_t front = wbuf > xpatch ? wbuf : xpatch;
-  return front + (size_t)WAVES * 32 * kPatchRow * 2 + (size_t)2 * NBUF * kXsChunk * 4;
+  return front + (size_t)WAVES * 32 * kPatchRow * 2 + (size_t)NBUF * 1024;
 }
 
 // EPI: 0 = bias only, 1 = runtime activation and / or residual.
-// With LN the kernel expects w = w', bias = b' (fp32), wsum (fp32) as prepared by ln_fold_kernel.
+// With LN the kernel expects w = w' and the table lnx as prepared by ln_fold_kernel.
 // NBUF: w chunk buffers in LDS (chunk c + NBUF - 1 is requested when chunk c starts).
 template <int K, int MT, int WAVES, int NBUF, bool LN, bool SWIGLU, int EPI>
 __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2))) void xstat_linear_kernel(
     const uint16_t* __restrict__ x, uint32_t ldx, float eps, const uint16_t* __restrict__ w,
-    const uint16_t* __restrict__ bias, const float* __restrict__ bias_f, const float* __restrict__ wsum,
+    const uint16_t* __restrict__ bias, const uint16_t* __restrict__ lnx,
     const uint16_t* __restrict__ residual, uint32_t ldr, uint16_t* __restrict__ y, uint32_t ldy, uint32_t M,
     uint32_t N, uint32_t act) {
   using G = XsGeom<K>;
@@ -55,8 +58,9 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
                                 : (size_t)WAVES * 32 * (G::KP + 8) * 2;
   constexpr uint32_t kAheadChunks = NBUF - 1;
   uint16_t* lds_patch = reinterpret_cast<uint16_t*>(lds_xs + kFront);
-  float (*s_bias)[kXsChunk] = reinterpret_cast<float (*)[kXsChunk]>(lds_xs + kFront + (size_t)WAVES * 32 * kPatchRow * 2);
-  float (*s_wsum)[kXsChunk] = s_bias + NBUF;
+  // per chunk slot, 1 KB: the chunk's bias as fp32 (plain) or its 64 rows of the LayerNorm table (16 bytes each)
+  char* s_side = lds_xs + kFront + (size_t)WAVES * 32 * kPatchRow * 2;
+  auto s_bias = [&](uint32_t slot) -> float* { return reinterpret_cast<float*>(s_side + slot * 1024); };
 
   const uint32_t tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid / kWave), lane = tid % kWave;
   const uint32_t lq = lane & 31u, half = lane >> 5;
@@ -94,7 +98,8 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
   }
   // LayerNorm statistics of this lane's rows: one sweep, sums of d = x - x0 and d^2, shifted by the row's
   // first element so that the variance does not cancel
-  float ln_a[MT], ln_b[MT];   // y = ln_a * acc + (ln_b * wsum + bias'),  ln_a = rstd, ln_b = -rstd * mean
+  float ln_a[MT];             // rstd of this lane's row
+  float ln_m[MT], ln_s[MT];   // -mean and 1 / rstd: the correction k-step's B operand is rebuilt from them per chunk
   if (LN) {
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
@@ -111,7 +116,8 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
       const float sm = pair_sum(s) * (1.0f / K);
       const float var = fmaxf(pair_sum(q) * (1.0f / K) - sm * sm, 0.f);
       ln_a[mt] = rsqrtf(var + eps);
-      ln_b[mt] = -ln_a[mt] * (x0 + sm);
+      ln_m[mt] = -(x0 + sm);
+      ln_s[mt] = (var + eps) * ln_a[mt];
     }
   }
   __syncthreads();  // the transposition patches are dead; the space now holds w chunks
@@ -130,7 +136,7 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
   // direct loads of chunk c into buffer slot: instruction q fills LDS bytes [1024 q, 1024 q + 1024) of the
   // buffer, i.e. chunk rows [q * 64 / CPR, ...); wave v issues instructions v, v + WAVES, ...
   constexpr uint32_t kMyDmaMax = (G::N_DMA + WAVES - 1) / WAVES;
-  const uint32_t my_dma = G::N_DMA / WAVES + (wave < (uint32_t)(G::N_DMA % WAVES) ? 1u : 0u);
+  const uint32_t my_dma = G::N_DMA / WAVES + (wave < (uint32_t)(G::N_DMA % WAVES) ? 1u : 0u) + ((LN && wave == 0) ? 1u : 0u);
   auto dma_chunk = [&](uint32_t c, uint32_t slot) {
     const char* buf = lds_xs + slot * G::CHUNK_BYTES;
 #pragma unroll
@@ -142,24 +148,16 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
         xs_lds_dma16(w, (w_row(c, r) * K + piece * 8u) * 2u, buf + qi * 1024);
       }
     }
+    if (LN && wave == 0) xs_lds_dma16(lnx, w_row(c, lane) * 16u, s_side + slot * 1024);   // table rows of the chunk
   };
   // bias (and wsum) of a chunk: every wave issues the same loads so that the wait constants below hold
   // for all of them; wave 0 parks the values in LDS one chunk later
-  float rb = 0.f, rs = 0.f;
+  float rb = 0.f;
   auto load_bias = [&](uint32_t c) {
-    const uint32_t n = w_row(c, lane);
-    if (LN) {
-      rb = bias_f[n];
-      rs = wsum[n];
-    } else {
-      rb = bias ? bf16_bits_to_float(bias[n]) : 0.f;
-    }
+    if (!LN) rb = bias ? bf16_bits_to_float(bias[w_row(c, lane)]) : 0.f;
   };
   auto park_bias = [&](uint32_t slot) {
-    if (wave == 0) {
-      s_bias[slot][lane] = rb;
-      if (LN) s_wsum[slot][lane] = rs;
-    }
+    if (!LN && wave == 0) s_bias(slot)[lane] = rb;
   };
 
   const bool wg_full = (blockIdx.x + 1) * ROWS_WG <= M;
@@ -196,7 +194,7 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
   auto stage_mfma = [&](uint32_t ci) {
     const uint32_t slot = ci % NBUF;
     const char* sw = lds_xs + slot * G::CHUNK_BYTES;
-    const float* sb = s_bias[slot];
+    const float* sb = s_bias(slot);
 #pragma unroll
     for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
@@ -219,6 +217,34 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
     };
 #pragma unroll
     for (int ks = 0; ks < kAhead; ++ks) read_frag(ks);
+    if (LN) {
+      // correction k-step: the chunk's table rows against the row statistics
+      bf16x8_t tf[2];
+#pragma unroll
+      for (int nt = 0; nt < 2; ++nt) tf[nt] = *reinterpret_cast<const bf16x8_t*>(s_side + slot * 1024 + (nt * 32 + lq) * 16);
+      // B operand (m_hi, m_lo, m_hi, s_hi, s_lo, s_hi, 0, 0) in the lanes of the lower half, zeros in the upper
+      // half; built here from two floats per tile (kept opaque so that it is not hoisted into eight registers)
+      bf16x8_t xe[MT];
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        float m = ln_m[mt], sd = ln_s[mt];
+        asm volatile("" : "+v"(m), "+v"(sd));
+        const uint32_t hi = pack_bf16x2(m, sd);                                  // m_hi | s_hi << 16
+        const uint32_t lo = pack_bf16x2(m - bf16_lo(hi), sd - bf16_hi(hi));      // m_lo | s_lo << 16
+        u32x4_t d;
+        d[0] = (hi & 0xFFFFu) | (lo << 16);          // m_hi, m_lo
+        d[1] = hi;                                   // m_hi, s_hi
+        d[2] = (lo >> 16) | (hi & 0xFFFF0000u);      // s_lo, s_hi
+        d[3] = 0u;
+        if (half != 0) { d[0] = 0u; d[1] = 0u; d[2] = 0u; }
+        xe[mt] = __builtin_bit_cast(bf16x8_t, d);
+      }
+#pragma unroll
+      for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+          acc[nt][mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tf[nt], xe[mt], acc[nt][mt], 0, 0, 0);
+    }
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       if (ks + kAhead < KS) read_frag(ks + kAhead);
@@ -229,7 +255,8 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
           acc[nt][mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[ks][nt], xf[mt][ks], acc[nt][mt], 0, 0, 0);
     }
     // pin the issue order: kAhead k-steps of LDS reads first, then one k-step of reads per k-step of MFMAs
-    __builtin_amdgcn_sched_group_barrier(0x100, 2 * kAhead, 0);
+    __builtin_amdgcn_sched_group_barrier(0x100, 2 * kAhead + (LN ? 2 : 0), 0);
+    if (LN) __builtin_amdgcn_sched_group_barrier(0x008, 2 * MT, 0);
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       __builtin_amdgcn_sched_group_barrier(0x008, 2 * MT, 0);
@@ -240,24 +267,14 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
   // that the global stores are row-contiguous 16-byte pieces (4 lanes = 64 bytes of one row)
   auto stage_epilogue = [&](uint32_t ci) {
     const uint32_t slot = ci % NBUF;
-    const float* sb = s_bias[slot];
     const uint32_t col0 = actual(ci) * COLS;   // first output column of the chunk
     if (LN) {
-      const float* ss = s_wsum[slot];
 #pragma unroll
       for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          const float4 b4 = *reinterpret_cast<const float4*>(sb + nt * 32 + g * 8 + half * 4);
-          const float4 s4 = *reinterpret_cast<const float4*>(ss + nt * 32 + g * 8 + half * 4);
+        for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-          for (int mt = 0; mt < MT; ++mt) {
-            acc[nt][mt][g * 4 + 0] = __builtin_fmaf(ln_a[mt], acc[nt][mt][g * 4 + 0], __builtin_fmaf(ln_b[mt], s4.x, b4.x));
-            acc[nt][mt][g * 4 + 1] = __builtin_fmaf(ln_a[mt], acc[nt][mt][g * 4 + 1], __builtin_fmaf(ln_b[mt], s4.y, b4.y));
-            acc[nt][mt][g * 4 + 2] = __builtin_fmaf(ln_a[mt], acc[nt][mt][g * 4 + 2], __builtin_fmaf(ln_b[mt], s4.z, b4.z));
-            acc[nt][mt][g * 4 + 3] = __builtin_fmaf(ln_a[mt], acc[nt][mt][g * 4 + 3], __builtin_fmaf(ln_b[mt], s4.w, b4.w));
-          }
-        }
+          for (int e = 0; e < 16; ++e) acc[nt][mt][e] *= ln_a[mt];
     }
     auto flush_tile = [&](auto full_tag, int mt, uint32_t colbase) {
       // patch holds rows [mt*32, mt*32+32) x 32 columns starting at output column colbase
@@ -304,9 +321,9 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
             float hv[4];
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-              // fc1 output is bf16 before the gated activation
-              const uint32_t vg = pack_bf16x2(acc[0][mt][g * 4 + r], acc[1][mt][g * 4 + r]);
-              hv[r] = fast_silu(bf16_lo(vg)) * bf16_hi(vg);
+              // the gate is formed from the fp32 accumulators: one rounding (of the product) where the
+              // reference rounds fc1 to bf16 first and the product again
+              hv[r] = fast_silu(acc[0][mt][g * 4 + r]) * acc[1][mt][g * 4 + r];
             }
             uint2 pk;
             pk.x = pack_bf16x2(hv[0], hv[1]);
@@ -355,13 +372,14 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
   }
 }
 
-// w' = bf16(w * gamma), wsum[n] = sum_k w'[n][k] (of the rounded values the matrix core will see),
-// b'[n] = bias[n] + sum_k w[n][k] * beta[k].  One wave per output feature.
+// w' = bf16(w * gamma) and the table row of every output feature n:
+//   (wsum_hi, wsum_hi, wsum_lo, b'_hi, b'_hi, b'_lo, 0, 0) in bf16, with
+//   wsum[n] = sum_k w'[n][k] (of the rounded values the matrix core will see), b'[n] = bias[n] + sum_k w[n][k] * beta[k].
+// One wave per output feature.
 __global__ __launch_bounds__(256) void ln_fold_kernel(const uint16_t* __restrict__ w, const uint16_t* __restrict__ gamma,
                                                       const uint16_t* __restrict__ beta,
                                                       const uint16_t* __restrict__ bias, uint16_t* __restrict__ wp,
-                                                      float* __restrict__ wsum, float* __restrict__ bp, uint32_t N,
-                                                      uint32_t K) {
+                                                      uint16_t* __restrict__ lnx, uint32_t N, uint32_t K) {
   const uint32_t n = blockIdx.x * 4 + threadIdx.x / kWave, lane = threadIdx.x % kWave;
   if (n >= N) return;
   float s = 0.f, t = 0.f;
@@ -378,19 +396,23 @@ __global__ __launch_bounds__(256) void ln_fold_kernel(const uint16_t* __restrict
     t += __shfl_xor(t, o, kWave);
   }
   if (lane == 0) {
-    wsum[n] = s;
-    bp[n] = t + (bias ? bf16_bits_to_float(bias[n]) : 0.f);
+    const float b = t + (bias ? bf16_bits_to_float(bias[n]) : 0.f);
+    const uint16_t s_hi = float_to_bf16_bits(s), b_hi = float_to_bf16_bits(b);
+    const uint16_t s_lo = float_to_bf16_bits(s - bf16_bits_to_float(s_hi));
+    const uint16_t b_lo = float_to_bf16_bits(b - bf16_bits_to_float(b_hi));
+    uint16_t* row = lnx + (size_t)n * 8;
+    row[0] = s_hi; row[1] = s_hi; row[2] = s_lo; row[3] = b_hi; row[4] = b_hi; row[5] = b_lo; row[6] = 0; row[7] = 0;
   }
 }
 
 void launch_ln_fold(const uint16_t* w, const uint16_t* gamma, const uint16_t* beta, const uint16_t* bias, uint16_t* wp,
-                    float* wsum, float* bp, uint32_t N, uint32_t K, hipStream_t s) {
-  hipLaunchKernelGGL(ln_fold_kernel, dim3(cdiv_u32(N, 4)), dim3(256), 0, s, w, gamma, beta, bias, wp, wsum, bp, N, K);
+                    uint16_t* lnx, uint32_t N, uint32_t K, hipStream_t s) {
+  hipLaunchKernelGGL(ln_fold_kernel, dim3(cdiv_u32(N, 4)), dim3(256), 0, s, w, gamma, beta, bias, wp, lnx, N, K);
 }
 
 template <int K, int MT, int WAVES, int NBUF>
 static int launch_k(bool ln, bool swiglu, hipStream_t s, const uint16_t* x, uint32_t ldx, float eps,
-                    const uint16_t* w, const uint16_t* bias, const float* bias_f, const float* wsum,
+                    const uint16_t* w, const uint16_t* bias, const uint16_t* lnx,
                     const uint16_t* residual, uint32_t ldr, uint16_t* y, uint32_t ldy, uint32_t M, uint32_t N,
                     uint32_t act, int device) {
   const bool general = act != F3D_ACT_NONE || residual != nullptr;
@@ -404,7 +426,7 @@ static int launch_k(bool ln, bool swiglu, hipStream_t s, const uint16_t* x, uint
       F3D_CHECK_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds)); \
       if (device >= 0 && device < 64) attr_set[device] = true;                                                     \
     }                                                                                                              \
-    hipLaunchKernelGGL(kern, grid, block, lds, s, x, ldx, eps, w, bias, bias_f, wsum, residual, ldr, y, ldy, M, N, \
+    hipLaunchKernelGGL(kern, grid, block, lds, s, x, ldx, eps, w, bias, lnx, residual, ldr, y, ldy, M, N,          \
                        act);                                                                                       \
   } while (0)
   if (ln && swiglu) { if (general) F3D_XS(true, true, 1); else F3D_XS(true, true, 0); }
@@ -428,30 +450,28 @@ int launch_xstat_linear(const uint16_t* x, uint32_t ldx, const uint16_t* gamma, 
   if (swiglu ? N % 64 != 0 : N % 32 != 0) return F3D_ERR_UNSUPPORTED;
   if (K != 32 && K != 64 && K != 128 && K != 256 && K != 512) return F3D_ERR_UNSUPPORTED;
   if ((uint64_t)N * K * 2 >= (1ull << 32)) return F3D_ERR_UNSUPPORTED;   // 32-bit byte offsets into w
-  const float* bias_f = nullptr;
-  const float* wsum = nullptr;
+  const uint16_t* lnx = nullptr;
   if (ln) {
-    // per call: w' (bf16 [N][K]), wsum and b' (fp32 [N]) in the per-device workspace
+    // per call: w' (bf16 [N][K]) and the table (bf16 [N][8]) in the per-device workspace
     const size_t wp_bytes = ((size_t)N * K * 2 + 255) & ~(size_t)255;
-    char* ws = (char*)workspace(device, wp_bytes + (size_t)N * 8);
+    char* ws = (char*)workspace(device, wp_bytes + (size_t)N * 16);
     if (!ws) return F3D_ERR_RUNTIME;
     uint16_t* wp = (uint16_t*)ws;
-    float* ws_sum = (float*)(ws + wp_bytes);
-    float* ws_bias = ws_sum + N;
-    launch_ln_fold(w, gamma, beta, bias, wp, ws_sum, ws_bias, N, K, s);
+    uint16_t* table = (uint16_t*)(ws + wp_bytes);
+    launch_ln_fold(w, gamma, beta, bias, wp, table, N, K, s);
     w = wp;
-    wsum = ws_sum;
-    bias_f = ws_bias;
+    lnx = table;
   }
-  // Large panels (64 rows per wave, 8 waves, 3 chunk buffers: one workgroup per CU) when there are enough
-  // rows to fill the chip with them, otherwise 32 rows per wave in 4-wave workgroups with 2 buffers.
-  // (Two 4-wave workgroups of 64-row waves per CU measured 6% slower than one 8-wave workgroup.)
-  const bool big = M >= 512u * 256u;
+  // Large panels (64 rows per wave, 8 waves, 3 chunk buffers: one workgroup per CU) when their workgroups fill
+  // at least three quarters of the chip, otherwise 32 rows per wave in 4-wave workgroups with 2 buffers
+  // (measured at 125 k rows: large panels 12 % faster; at 62 k rows: small panels 30 % faster).
+  // (Two 4-wave workgroups of 64-row waves per CU measured 6 % slower than one 8-wave workgroup.)
+  const bool big = M >= 512u * 192u;
 #define F3D_XS_CASE(KK)                                                                                                  \
   case KK:                                                                                                               \
-    return big ? launch_k<KK, 2, 8, 3>(ln, swiglu, s, x, ldx, eps, w, bias, bias_f, wsum, residual, ldr, y, ldy, M, N,   \
+    return big ? launch_k<KK, 2, 8, 3>(ln, swiglu, s, x, ldx, eps, w, bias, lnx, residual, ldr, y, ldy, M, N,   \
                                        run_act, device)                                                                  \
-               : launch_k<KK, 1, 4, 2>(ln, swiglu, s, x, ldx, eps, w, bias, bias_f, wsum, residual, ldr, y, ldy, M, N,   \
+               : launch_k<KK, 1, 4, 2>(ln, swiglu, s, x, ldx, eps, w, bias, lnx, residual, ldr, y, ldy, M, N,   \
                                        run_act, device);
   switch (K) {
     F3D_XS_CASE(32)
@@ -460,7 +480,7 @@ int launch_xstat_linear(const uint16_t* x, uint32_t ldx, const uint16_t* gamma, 
     F3D_XS_CASE(256)
     case 512:
       // 512 inner features fill the register budget with 32 rows per wave; two 64 KB chunk buffers
-      return launch_k<512, 1, 8, 2>(ln, swiglu, s, x, ldx, eps, w, bias, bias_f, wsum, residual, ldr, y, ldy, M, N,
+      return launch_k<512, 1, 8, 2>(ln, swiglu, s, x, ldx, eps, w, bias, lnx, residual, ldr, y, ldy, M, N,
                                     run_act, device);
     default: return F3D_ERR_UNSUPPORTED;
   }
