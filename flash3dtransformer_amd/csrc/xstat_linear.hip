@@ -161,6 +161,8 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
   };
 
   const bool wg_full = (blockIdx.x + 1) * ROWS_WG <= M;
+  uint16_t* y_wg = y + (size_t)(blockIdx.x * ROWS_WG) * ldy;                  // wave-uniform bases
+  const uint16_t* res_wg = residual ? residual + (size_t)(blockIdx.x * ROWS_WG) * ldr : nullptr;
   // Workgroups walk the output columns in rotated order: at any moment different workgroups write
   // different column ranges, which spreads the stores over the HBM channels (with a power-of-two row
   // pitch every workgroup would otherwise hit the same channels at the same time).
@@ -208,7 +210,8 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
         }
       }
     // w fragments are read kAhead k-steps before the MFMAs that consume them
-    constexpr int kAhead = KS < 2 ? KS : 2;
+    // (one k-step for the plain 256-feature large panels: the registers of the second one would spill)
+    constexpr int kAhead = (KS < 2 || (K >= 256 && MT > 1 && !SWIGLU)) ? 1 : 2;
     bf16x8_t wf[KS][2];
     auto read_frag = [&](int ks) {
       const char* p = sw + (frag_off ^ (uint32_t)(ks * 32));
@@ -283,6 +286,8 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
       for (int h2 = 0; h2 < 2; ++h2) {
         const uint32_t rr = (lane >> 2) + h2 * 16, ch = (lane & 3u) * 8;
         const uint32_t row = row0 + mt * 32 + rr;
+        // element offsets from the workgroup's first row fit 32 bits (512 rows at most)
+        const uint32_t lrow = wave * (32 * MT) + mt * 32 + rr;
         u32x4_t t = *reinterpret_cast<const u32x4_t*>(patch + rr * kPatchRow + ch);
         if (!kFull && row >= M) continue;
         if (EPI == 1) {
@@ -291,13 +296,13 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
             for (int e = 0; e < 4; ++e) t[e] = pack_bf16x2(xs_act(bf16_lo(t[e]), act), xs_act(bf16_hi(t[e]), act));
           }
           if (residual) {
-            const u32x4_t rres = *reinterpret_cast<const u32x4_t*>(residual + (size_t)row * ldr + colbase + ch);
+            const u32x4_t rres = *reinterpret_cast<const u32x4_t*>(res_wg + (lrow * ldr + colbase + ch));
 #pragma unroll
             for (int e = 0; e < 4; ++e)
               t[e] = pack_bf16x2(bf16_lo(t[e]) + bf16_lo(rres[e]), bf16_hi(t[e]) + bf16_hi(rres[e]));
           }
         }
-        *reinterpret_cast<u32x4_t*>(y + (size_t)row * ldy + colbase + ch) = t;
+        *reinterpret_cast<u32x4_t*>(y_wg + (lrow * ldy + colbase + ch)) = t;
       }
     };
     auto epilogue = [&](auto full_tag) {
