@@ -27,8 +27,8 @@ HBM_PEAK_GBS = 8000.0
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by a copy kernel of known
 # size, see profiles/encoder_stage_4x120k_hbm_traffic.md) at this bench's shapes
-TRAFFIC_BYTES_PER_LAUNCH = {"ln_fc1_act": 1.540e9, "ln_qkv": 1.064e9, "attention": 1.016e9,
-                            "proj_residual": 0.826e9, "fc2_residual": 1.516e9}
+TRAFFIC_BYTES_PER_LAUNCH = {"ln_fc1_act": 1.557e9, "ln_qkv": 1.027e9, "attention": 1.017e9,
+                            "proj_residual": 0.770e9, "fc2_residual": 1.513e9}
 
 
 def ev_time(fn, iters, warmup=3):
@@ -96,6 +96,8 @@ def main():
     ap.add_argument("--mlp", default="swiglu", choices=["swiglu", "gelu"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-sub-metrics", action="store_true")
+    ap.add_argument("--sub-metrics-only", action="store_true",
+                    help="run only the per-kernel sub-metrics (configs 1, 2, 3, 5) and print them; for profiling those kernels")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU; the path shards by cloud without any exchange "
@@ -106,6 +108,9 @@ def main():
     from flash3dtransformer_amd.lib import pshattn
     from flash3dtransformer_amd.psh import psh_main
     dev = "cuda:0"
+    if args.sub_metrics_only:
+        print(json.dumps({"sub_metrics": sub_metrics(dev)}))
+        return
     C, HID, H, BS, SCOPE, HASH = 256, 1024, 8, 512, 1, 2
     clouds = [synth.lidar_sweep(120_000, 1004 + i) for i in range(4)]
     coords_np, seps_np = synth.batch_of(clouds)
