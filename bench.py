@@ -298,6 +298,19 @@ def sub_metrics(dev):
     out["pool_c3_reduce_mean"] = {"ms": round(ms_mean, 4), "gbs": gb(red_bytes, ms_mean), "frac_of_hbm_peak": round(gb(red_bytes, ms_mean) / HBM_PEAK_GBS, 4)}
     out["pool_c3_reduce_max"] = {"ms": round(ms_max, 4), "gbs": gb(red_bytes, ms_max), "frac_of_hbm_peak": round(gb(red_bytes, ms_max) / HBM_PEAK_GBS, 4)}
     out["unpool_c3"] = {"ms": round(ms_up, 4), "gbs": gb(up_bytes, ms_up), "frac_of_hbm_peak": round(gb(up_bytes, ms_up) / HBM_PEAK_GBS, 4)}
+    # backward of both (same shapes): reduce bwd reads grad R C 2 (+ input N C 2 for max) and writes N C 2;
+    # unpool bwd reads N C 2, writes N C 2 + R C 2
+    g_red = torch.randn(sb.reduced_feat.shape[0], C, generator=gg).to(torch.bfloat16).to(dev)
+    g_in, g_res, g_down = torch.zeros_like(feat), torch.zeros_like(res), torch.zeros_like(sb.reduced_feat)
+    ms_rb = ev_time(lambda: pshattn.batch_subbuck_reduce_backward(g_red, feat, sb.unpool_ind, g_in, S, 0), 30)
+    ms_rbm = ev_time(lambda: pshattn.batch_subbuck_reduce_backward(g_red, feat, sb.unpool_ind, g_in, S, 3), 30)
+    ms_ub = ev_time(lambda: pshattn.additive_unpool_bwd(g_res, g_down, res, sb.unpool_ind, S), 30)
+    rb_bytes, rbm_bytes = r * C * 2 + n * C * 2 + r * S * 4, r * C * 2 + 2 * n * C * 2 + r * S * 4
+    ub_bytes = 2 * n * C * 2 + r * C * 2 + r * S * 4
+    out["pool_c3_reduce_mean_bwd"] = {"ms": round(ms_rb, 4), "gbs": gb(rb_bytes, ms_rb), "frac_of_hbm_peak": round(gb(rb_bytes, ms_rb) / HBM_PEAK_GBS, 4)}
+    out["pool_c3_reduce_max_bwd"] = {"ms": round(ms_rbm, 4), "gbs": gb(rbm_bytes, ms_rbm), "frac_of_hbm_peak": round(gb(rbm_bytes, ms_rbm) / HBM_PEAK_GBS, 4)}
+    out["unpool_c3_bwd"] = {"ms": round(ms_ub, 4), "gbs": gb(ub_bytes, ms_ub), "frac_of_hbm_peak": round(gb(ub_bytes, ms_ub) / HBM_PEAK_GBS, 4)}
+    del g_red, g_in, g_res, g_down
     del coords, feat, res, up, sb
     out["hourglass_c5"] = hourglass_c5(dev)
     return out

@@ -26,7 +26,7 @@ COMMON = [
 VGPR_FORM = ["-mllvm", "-amdgpu-mfma-vgpr-form"]
 NO_VGPR_FORM = set()
 # bit-exact integer / quantiser kernels: no fused multiply-add contraction
-EXACT = {"psh_bucket.hip", "subbuck_pool.hip", "unpool.hip"}
+EXACT = {"psh_bucket.hip", "subbuck_pool.hip", "unpool.hip", "pool_bwd.hip"}
 
 
 def sources():

@@ -31,7 +31,13 @@ class SubbuckReduceFunction(Function):
 
     @staticmethod
     def backward(ctx, grad_reduced_feat, grad_buffers):
-        raise NotImplementedError("batch_subbuck_reduce_backward: the gfx950 library implements the forward pass only")
+        """only input_feat is differentiable (reference: layers/pooling.py:87-116)"""
+        input_feat, unpool_ind = ctx.saved_tensors
+        g = grad_reduced_feat if grad_reduced_feat.dtype == torch.bfloat16 else grad_reduced_feat.to(torch.bfloat16)
+        grad_input_feat = torch.zeros_like(input_feat)
+        pshattn.batch_subbuck_reduce_backward(g.contiguous(), input_feat, unpool_ind, grad_input_feat, ctx.subbuck_size,
+                                              ctx.reduction_op)
+        return None, grad_input_feat, None, None, None, None
 
 
 class InbucketPoolingLayer(nn.Module):

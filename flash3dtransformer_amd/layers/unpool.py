@@ -4,7 +4,7 @@ from torch import nn
 from torch.autograd import Function
 
 from ..lib import pshattn
-from ..psh.subbuck import SubbuckBuffers, UnpoolBuffers
+from ..psh.subbuck import SubbuckBuffers, UnpoolBuffers, UnpoolGradients
 
 
 class AdditiveUnpoolFunction(Function):
@@ -15,11 +15,19 @@ class AdditiveUnpoolFunction(Function):
         buf = UnpoolBuffers.create_unpool_buff(residual_feat)
         pshattn.additive_unpool_fwd(residual_feat, down_feat, buf.up_add_feat, buffers.unpool_ind, subbuck_size)
         ctx.subbuck_size = subbuck_size
+        ctx.subbuck_buffers = buffers
+        ctx.down_len = down_feat.shape[0]
         return buf.up_add_feat
 
     @staticmethod
     def backward(ctx, grad_up_add_feat):
-        raise NotImplementedError("additive_unpool_bwd: the gfx950 library implements the forward pass only")
+        """grad_res = the output gradient (identity branch), grad_down[i] = sum over the points pooled into row i
+        (reference: layers/unpool.py:50-77)"""
+        g = grad_up_add_feat if grad_up_add_feat.dtype == torch.bfloat16 else grad_up_add_feat.to(torch.bfloat16)
+        g = g.contiguous()
+        grads = UnpoolGradients.create_unpool_grad(g, ctx.subbuck_buffers, ctx.down_len)
+        pshattn.additive_unpool_bwd(grads.grad_res, grads.grad_down, g, ctx.subbuck_buffers.unpool_ind, ctx.subbuck_size)
+        return grads.grad_res, grads.grad_down, None, None
 
 
 class AdditiveUnpoolLayer(nn.Module):

@@ -237,8 +237,23 @@ def batch_subbuck_reduce(scattered_coord, scattered_feat, batch_sep, instance_ma
 
 
 def batch_subbuck_reduce_backward(grad_red_feat, input_feat, unpool_ind, grad_input_feat, subbuck_size, red_op):
-    """src/f3d_frontend.cu:68-71 — backward is outside the forward hot path this library implements"""
-    raise NotImplementedError("batch_subbuck_reduce_backward: the gfx950 library implements the forward path only")
+    """src/f3d_frontend.cu:68-71 -> src/psh/batch_subbuck_pooling_bwd_dispatcher.cu: gradient of the feature reduce.
+    grad_red_feat [>= R, C], input_feat / grad_input_feat [N, C] bf16, unpool_ind [R, S] uint32.  Rows of
+    grad_input_feat that no slot refers to keep the caller's content (the reference passes zeros)."""
+    ts = [grad_red_feat, input_feat, unpool_ind, grad_input_feat]
+    assert_contiguous(ts)
+    dev = assert_same_device(ts)
+    assert_dtype([grad_red_feat, input_feat, grad_input_feat], torch.bfloat16)
+    assert_dtype([unpool_ind], torch.uint32)
+    if input_feat.shape != grad_input_feat.shape:
+        raise RuntimeError(f"input_feat shape {tuple(input_feat.shape)} != grad_input_feat shape {tuple(grad_input_feat.shape)}")
+    if grad_red_feat.shape[1] != input_feat.shape[1] or grad_red_feat.shape[0] < unpool_ind.shape[0]:
+        raise RuntimeError(f"grad_red_feat shape {tuple(grad_red_feat.shape)} does not cover unpool_ind {tuple(unpool_ind.shape)}")
+    if unpool_ind.shape[1] != subbuck_size:
+        raise RuntimeError(f"unpool_ind width {unpool_ind.shape[1]} != subbuck_size {subbuck_size}")
+    _check(_load().f3d_subbuck_reduce_bwd(
+        _ptr(grad_red_feat), _ptr(input_feat), _ptr(unpool_ind), _ptr(grad_input_feat), _u32(input_feat.shape[0]),
+        _u32(unpool_ind.shape[0]), _u32(input_feat.shape[1]), _u32(subbuck_size), _u32(red_op), _i32(dev), _stream(dev)))
 
 
 def additive_unpool_fwd(res_feat, down_feat, up_add_feat, unpool_ind, subbuck_size):
@@ -262,8 +277,23 @@ def additive_unpool_fwd(res_feat, down_feat, up_add_feat, unpool_ind, subbuck_si
 
 
 def additive_unpool_bwd(grad_res, grad_down, grad_up_added, unpool_ind, subbuck_size):
-    """src/f3d_frontend.cu:103-105 — backward, not part of the forward hot path"""
-    raise NotImplementedError("additive_unpool_bwd: the gfx950 library implements the forward path only")
+    """src/f3d_frontend.cu:103-105 -> src/psh/additive_unpool_dispatcher.cu:81-134: grad_res[r] = grad_up_added[r]
+    for every pooled point r, grad_down[i] = sum over the points pooled into row i.  Rows of grad_res that no slot
+    refers to keep the caller's content (the reference passes zeros)."""
+    ts = [grad_res, grad_down, grad_up_added, unpool_ind]
+    assert_contiguous(ts)
+    dev = assert_same_device(ts)
+    assert_dtype([grad_res, grad_down, grad_up_added], torch.bfloat16)
+    assert_dtype([unpool_ind], torch.uint32)
+    if grad_res.shape != grad_up_added.shape:
+        raise RuntimeError(f"grad_res shape {tuple(grad_res.shape)} != grad_up_added shape {tuple(grad_up_added.shape)}")
+    if grad_down.shape[1] != grad_res.shape[1] or grad_down.shape[0] < unpool_ind.shape[0]:
+        raise RuntimeError(f"grad_down shape {tuple(grad_down.shape)} does not cover unpool_ind {tuple(unpool_ind.shape)}")
+    if unpool_ind.shape[1] != subbuck_size:
+        raise RuntimeError(f"unpool_ind width {unpool_ind.shape[1]} != subbuck_size {subbuck_size}")
+    _check(_load().f3d_additive_unpool_bwd(
+        _ptr(grad_res), _ptr(grad_down), _ptr(grad_up_added), _ptr(unpool_ind), _u32(grad_res.shape[0]),
+        _u32(unpool_ind.shape[0]), _u32(grad_res.shape[1]), _u32(subbuck_size), _i32(dev), _stream(dev)))
 
 
 # ---------------------------------------------------------------------------------------------

@@ -79,3 +79,21 @@ class UnpoolBuffers:
     @staticmethod
     def create_unpool_buff(residual_feat: torch.Tensor):
         return UnpoolBuffers(torch.empty_like(residual_feat))
+
+
+@dcls.dataclass(slots=True)
+class UnpoolGradients:
+    """gradient buffers of additive unpooling (reference: psh/subbuck.py:119-132): grad_res like the output
+    gradient, grad_down with the aligned row count of the pooled features; both start from zero because the
+    kernel leaves rows that no slot refers to untouched"""
+    grad_res: torch.Tensor
+    grad_down: torch.Tensor
+
+    @staticmethod
+    def create_unpool_grad(grad_up_added: torch.Tensor, sb: "SubbuckBuffers", down_len: int = None):
+        feat_dim = grad_up_added.shape[-1]
+        if down_len is None:
+            down_len = sb.reduced_feat.shape[0]
+        grad_res = torch.zeros_like(grad_up_added)
+        grad_down = torch.zeros(down_len, feat_dim, dtype=grad_up_added.dtype, device=grad_up_added.device)
+        return UnpoolGradients(grad_res, grad_down)

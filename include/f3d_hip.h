@@ -128,6 +128,25 @@ int f3d_additive_unpool_fwd(const f3d_bf16_t* res_feat, const f3d_bf16_t* down_f
                             const uint32_t* unpool_ind, uint32_t up_n, uint32_t down_n, uint32_t feat_dim,
                             uint32_t subbuck_size, int device, void* stream);
 
+/* ---- additive unpool backward: additive_unpool_bwd, src/f3d_frontend.cu:103-105, kernel
+ *      src/psh/additive_unpool.cuh:90-137, dispatcher src/psh/additive_unpool_dispatcher.cu:81-134 ----
+ * grad_res[r,:] = grad_up_added[r,:] for every r = unpool_ind[i,s] < up_n (rows no slot refers to keep the
+ * caller's content); grad_down[i,:] = bf16(sum over the valid slots of row i, slot order, fp32).
+ * grad_res, grad_up_added [up_n, feat_dim]; grad_down [>= down_n, feat_dim]; unpool_ind [down_n, subbuck_size]. */
+int f3d_additive_unpool_bwd(f3d_bf16_t* grad_res, f3d_bf16_t* grad_down, const f3d_bf16_t* grad_up_added,
+                            const uint32_t* unpool_ind, uint32_t up_n, uint32_t down_n, uint32_t feat_dim,
+                            uint32_t subbuck_size, int device, void* stream);
+
+/* ---- sub-bucket reduce backward: batch_subbuck_reduce_backward, src/f3d_frontend.cu:68-71, kernel
+ *      src/psh/batch_psh_subbuck_reduce_bwd.cuh:39-126 ----------------------------------------------------
+ * red_op 0 mean: bf16(grad / max(count,1)) to every valid slot; 1 sum: grad to every valid slot; 2 min / 3 max:
+ * grad to the first slot holding the strict winner of input_feat, zero to the other valid slots.
+ * Rows of grad_input_feat that no slot refers to keep the caller's content.
+ * grad_red_feat [>= reduced_n, feat_dim]; input_feat, grad_input_feat [total_n, feat_dim]. */
+int f3d_subbuck_reduce_bwd(const f3d_bf16_t* grad_red_feat, const f3d_bf16_t* input_feat, const uint32_t* unpool_ind,
+                           f3d_bf16_t* grad_input_feat, uint32_t total_n, uint32_t reduced_n, uint32_t feat_dim,
+                           uint32_t subbuck_size, uint32_t red_op, int device, void* stream);
+
 /* ---- bucketed attention forward: buck_swin_fwd, declared src/f3d_frontend.cu:90-92, called from
  *      flash3dxfmr/layers/buck_swin.py:57 (kernel source absent from the reference) --------------
  * q,k,v,o [batch,seq_len,num_head,head_dim] bf16 contiguous; lse [batch,seq_len,num_head] fp32;

@@ -522,3 +522,58 @@ int f3d_or_additive_unpool(const uint16_t *res_bf, const uint16_t *down_bf, uint
     }
   return 0;
 }
+
+/* ------------------------------------------------------------------------------------------ */
+/* backward of A8 and A7 — src/psh/additive_unpool.cuh:90-137,                                   */
+/* src/psh/batch_psh_subbuck_reduce_bwd.cuh:39-126                                              */
+/* ------------------------------------------------------------------------------------------ */
+int f3d_or_additive_unpool_bwd(uint16_t *grad_res, uint16_t *grad_down, const uint16_t *grad_up,
+                               const uint32_t *unpool_ind, uint32_t up_n, uint32_t down_n,
+                               uint32_t feat_dim, uint32_t subbuck_size) {
+  for (uint32_t i = 0; i < down_n; ++i)
+    for (uint32_t c = 0; c < feat_dim; ++c) {
+      float acc = 0.f;
+      for (uint32_t s = 0; s < subbuck_size; ++s) {
+        uint32_t r = unpool_ind[(size_t)i * subbuck_size + s];
+        if (r >= up_n) continue;
+        uint16_t g = grad_up[(size_t)r * feat_dim + c];
+        grad_res[(size_t)r * feat_dim + c] = g;
+        acc = acc + f3d_or_bf16_to_float(g);
+      }
+      grad_down[(size_t)i * feat_dim + c] = f3d_or_float_to_bf16(acc);
+    }
+  return 0;
+}
+
+/* The division of the mean is the correctly rounded fp32 quotient (the reference is built with fast math,
+ * whose approximate quotient can differ in the last fp32 bit, i.e. at rare bf16 rounding ties). */
+int f3d_or_reduce_feat_bwd(const uint16_t *grad_red, const uint16_t *input_bf, const uint32_t *unpool_ind,
+                           uint16_t *grad_in, uint32_t total_n, uint32_t reduced_n, uint32_t feat_dim,
+                           uint32_t subbuck_size, uint32_t red_op) {
+  if (red_op > 3) return -1;
+  for (uint32_t r = 0; r < reduced_n; ++r)
+    for (uint32_t c = 0; c < feat_dim; ++c) {
+      const uint32_t *ind = unpool_ind + (size_t)r * subbuck_size;
+      uint16_t g = grad_red[(size_t)r * feat_dim + c];
+      if (red_op <= 1) {
+        uint32_t cnt = 0;
+        for (uint32_t s = 0; s < subbuck_size; ++s) cnt += ind[s] < total_n;
+        uint16_t out = g;
+        if (red_op == 0) out = f3d_or_float_to_bf16(f3d_or_bf16_to_float(g) / (float)(cnt > 1 ? cnt : 1));
+        for (uint32_t s = 0; s < subbuck_size; ++s)
+          if (ind[s] < total_n) grad_in[(size_t)ind[s] * feat_dim + c] = out;
+      } else {
+        float best = (red_op == 3) ? -INFINITY : INFINITY;
+        uint32_t win = 0;
+        for (uint32_t s = 0; s < subbuck_size; ++s) {
+          if (ind[s] >= total_n) continue;
+          float v = f3d_or_bf16_to_float(input_bf[(size_t)ind[s] * feat_dim + c]);
+          int better = (red_op == 3) ? (v > best) : (v < best);
+          if (better) { best = v; win = s; }
+        }
+        for (uint32_t s = 0; s < subbuck_size; ++s)
+          if (ind[s] < total_n) grad_in[(size_t)ind[s] * feat_dim + c] = (s == win) ? g : 0;
+      }
+    }
+  return 0;
+}

@@ -257,6 +257,36 @@ def additive_unpool(res_bf, down_bf, unpool_ind, up_init=None):
     return up
 
 
+def additive_unpool_bwd(grad_up_bf, unpool_ind, down_rows=None, grad_res_init=None):
+    """backward of additive_unpool: returns (grad_res, grad_down) as bf16 bit patterns
+    (src/psh/additive_unpool.cuh:90-137); rows of grad_res that no slot refers to keep ``grad_res_init`` (zeros)."""
+    g = np.ascontiguousarray(grad_up_bf, dtype=np.uint16)
+    u = np.ascontiguousarray(unpool_ind, dtype=np.uint32)
+    n, c = g.shape
+    r, s = u.shape
+    grad_res = np.zeros_like(g) if grad_res_init is None else np.ascontiguousarray(grad_res_init, dtype=np.uint16).copy()
+    grad_down = np.zeros((r if down_rows is None else down_rows, c), dtype=np.uint16)
+    rc = lib().f3d_or_additive_unpool_bwd(_p(grad_res), _p(grad_down), _p(g), _p(u), ctypes.c_uint32(n),
+                                          ctypes.c_uint32(r), ctypes.c_uint32(c), ctypes.c_uint32(s))
+    assert rc == 0
+    return grad_res, grad_down
+
+
+def reduce_feat_bwd(grad_red_bf, input_bf, unpool_ind, red_op, grad_in_init=None):
+    """backward of reduce_feat (src/psh/batch_psh_subbuck_reduce_bwd.cuh:39-126): grad_input as bf16 bits"""
+    g = np.ascontiguousarray(grad_red_bf, dtype=np.uint16)
+    x = np.ascontiguousarray(input_bf, dtype=np.uint16)
+    u = np.ascontiguousarray(unpool_ind, dtype=np.uint32)
+    n, c = x.shape
+    r, s = u.shape
+    grad_in = np.zeros_like(x) if grad_in_init is None else np.ascontiguousarray(grad_in_init, dtype=np.uint16).copy()
+    rc = lib().f3d_or_reduce_feat_bwd(_p(g), _p(x), _p(u), _p(grad_in), ctypes.c_uint32(n), ctypes.c_uint32(r),
+                                      ctypes.c_uint32(c), ctypes.c_uint32(s), ctypes.c_uint32(red_op))
+    if rc != 0:
+        raise RuntimeError(f"oracle reduce_feat_bwd failed rc={rc}")
+    return grad_in
+
+
 # ---------------------------------------------------------------------------------------------
 # bf16 bit helpers (numpy)
 # ---------------------------------------------------------------------------------------------

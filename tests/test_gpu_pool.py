@@ -143,3 +143,72 @@ def test_pool_argument_errors():
         call(args(feat=f.float()))
     with pytest.raises(RuntimeError, match="not contiguous"):
         call(args(feat=torch.zeros(10, 16, dtype=torch.bfloat16, device=DEV)[:, ::2]))
+
+
+# ---------------------------------------------------------------------------------------------
+# backward ops (reference: additive_unpool_bwd, batch_subbuck_reduce_backward)
+# ---------------------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("S,op,n,C", [
+    (2, 0, 5000, 64), (3, 0, 4097, 24), (8, 0, 30000, 128), (4, 1, 1000, 40),
+    (2, 2, 3001, 16), (8, 3, 20000, 32), (3, 3, 999, 12),       # 12 channels: scalar path
+])
+def test_reduce_backward_bit_exact(oracle, S, op, n, C):
+    from flash3dtransformer_amd.lib import pshattn
+    rng = np.random.default_rng(S * 1000 + op * 10 + C)
+    coords = rng.uniform(-30, 30, (n, 3)).astype(np.float16)
+    seps = np.array([n // 3, n], dtype=np.uint32)
+    _, _, unpool, _, _ = oracle.subbuck_build(coords, seps, S, out_align=16)
+    r_al = -(-unpool.shape[0] // 16) * 16
+    x = bf16_bits(np.round(rng.normal(0, 1, (n, C)) * 4) / 4)           # coarse values: plenty of ties for min / max
+    g = bf16_bits(rng.normal(0, 1, (r_al, C)))
+    grad_in = torch.full((n, C), 7.0, dtype=torch.bfloat16, device=DEV)
+    pshattn.batch_subbuck_reduce_backward(t_bf16_bits(g), t_bf16_bits(x), t_u32(unpool), grad_in, S, op)
+    torch.cuda.synchronize()
+    want = oracle.reduce_feat_bwd(g, x, unpool, op, grad_in_init=bf16_bits(np.full((n, C), 7.0)))
+    assert np.array_equal(n_bf16_bits(grad_in), want)
+
+
+@pytest.mark.parametrize("S,n,C", [(2, 6000, 64), (3, 4099, 24), (8, 40000, 128), (2, 777, 12)])
+def test_unpool_backward_bit_exact(oracle, S, n, C):
+    from flash3dtransformer_amd.lib import pshattn
+    rng = np.random.default_rng(S + n + C)
+    r = -(-n // S) + 5
+    unpool = np.full((r, S), n + 3, dtype=np.uint32)
+    keep = rng.permutation(n)[: n - 30]                    # 30 rows are referred to by no slot
+    unpool.reshape(-1)[rng.permutation(r * S)[: keep.size]] = keep
+    g = bf16_bits(rng.normal(0, 1, (n, C)))
+    grad_res = torch.full((n, C), 3.0, dtype=torch.bfloat16, device=DEV)
+    grad_down = torch.full((r + 11, C), 5.0, dtype=torch.bfloat16, device=DEV)
+    pshattn.additive_unpool_bwd(grad_res, grad_down, t_bf16_bits(g), t_u32(unpool), S)
+    torch.cuda.synchronize()
+    want_res, want_down = oracle.additive_unpool_bwd(g, unpool, grad_res_init=bf16_bits(np.full((n, C), 3.0)))
+    assert np.array_equal(n_bf16_bits(grad_res), want_res)
+    got_down = n_bf16_bits(grad_down)
+    assert np.array_equal(got_down[:r], want_down)
+    assert np.array_equal(got_down[r:], bf16_bits(np.full((11, C), 5.0)))      # rows past the map are not written
+
+
+def test_pool_unpool_layers_backpropagate(oracle):
+    """gradients flow through InbucketPoolingLayer and AdditiveUnpoolLayer (reference autograd functions
+    layers/pooling.py:18-116, layers/unpool.py:18-77) and equal the oracle's composition"""
+    from flash3dtransformer_amd.layers.pooling import InbucketPoolingLayer
+    from flash3dtransformer_amd.layers.unpool import AdditiveUnpoolLayer
+    rng = np.random.default_rng(77)
+    n, C, S = 3000, 32, 2
+    coords = rng.uniform(-20, 20, (n, 3)).astype(np.float16)
+    seps = np.array([1700, n], dtype=np.uint32)
+    feat = torch.from_numpy(rng.normal(0, 1, (n, C)).astype(np.float32)).to(torch.bfloat16).to(DEV).requires_grad_(True)
+    res = torch.from_numpy(rng.normal(0, 1, (n, C)).astype(np.float32)).to(torch.bfloat16).to(DEV).requires_grad_(True)
+    pool, unpool_layer = InbucketPoolingLayer("mean", out_alignment=16, subbuck_size=S), AdditiveUnpoolLayer(S)
+    red, sb = pool(t_f16(coords), feat, t_u32(seps))
+    up = unpool_layer(res, red, sb)
+    w = torch.from_numpy(rng.normal(0, 1, (n, C)).astype(np.float32)).to(torch.bfloat16).to(DEV)
+    (up.float() * w.float()).sum().backward()
+    torch.cuda.synchronize()
+    # oracle: d up = w ; unpool bwd -> (grad_res, grad_down) ; reduce bwd(mean) of grad_down -> grad_feat
+    unpool = n_u32(sb.unpool_ind)
+    g_res, g_down = oracle.additive_unpool_bwd(n_bf16_bits(w), unpool, down_rows=red.shape[0])
+    g_feat = oracle.reduce_feat_bwd(g_down, n_bf16_bits(feat.detach()), unpool, 0)
+    assert np.array_equal(n_bf16_bits(res.grad), g_res)
+    assert np.array_equal(n_bf16_bits(feat.grad), g_feat)

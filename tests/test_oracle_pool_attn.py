@@ -197,3 +197,87 @@ def test_attention_closed_forms_and_masks(oracle):
     init = torch.full((B, L, H, D), 7.0)
     O, _ = oracle.buck_swin_fwd(Q, K, V, scopes[:1], bs, O_init=init)
     assert (O[:, bs:] == 7.0).all()
+
+
+# ---------------------------------------------------------------------------------------------
+# backward of the feature reduce and of additive unpooling
+# ---------------------------------------------------------------------------------------------
+
+def _random_inverse_map(rng, n, S, holes):
+    """an unpool_ind [R, S] in which every point appears once; `holes` extra empty slots are spread at random"""
+    r = -(-(n + holes) // S)
+    flat = np.full(r * S, n + 3, dtype=np.uint32)
+    pos = rng.permutation(r * S)[:n]
+    flat[pos] = rng.permutation(n).astype(np.uint32)
+    return flat.reshape(r, S)
+
+
+@pytest.mark.parametrize("S,op", [(2, 0), (3, 0), (8, 0), (4, 1), (2, 2), (8, 2), (3, 3), (8, 3)])
+def test_reduce_feat_bwd_vs_torch_autograd(oracle, S, op):
+    """gradient of gather + mean / sum / amin / amax (the forward formula of reference
+    tests/test_subbuck_reduce.py:131-147) by torch autograd in fp32, on inputs without ties (for which
+    amin / amax send the whole gradient to the single winner, as the reference kernel does)"""
+    rng = np.random.default_rng(100 * S + op)
+    n, C = 203, 12
+    unpool = _random_inverse_map(rng, n, S, holes=17)
+    # distinct bf16 values per column so that min / max have no ties
+    x = torch.stack([torch.from_numpy(rng.permutation(n).astype(np.float32)) * 0.25 - 20 for _ in range(C)], 1)
+    x = x.to(torch.bfloat16)
+    assert all(len(set(x[:, c].tolist())) == n for c in range(C))
+    g = torch.from_numpy(rng.normal(0, 1, (unpool.shape[0], C)).astype(np.float32)).to(torch.bfloat16)
+    got = oracle.reduce_feat_bwd(_bits(g), _bits(x), unpool, op)
+    # torch: masked gather, reduce, backward
+    xf = x.float().requires_grad_(True)
+    idx = torch.from_numpy(unpool.astype(np.int64))
+    valid = idx < n
+    gathered = xf[idx.clamp(max=n - 1)]                                  # [R, S, C]
+    if op <= 1:
+        red = (gathered * valid[..., None]).sum(1)
+        if op == 0:
+            red = red / valid.sum(1).clamp(min=1)[:, None]
+    else:
+        fill = float("inf") if op == 2 else float("-inf")
+        masked = torch.where(valid[..., None], gathered, torch.full_like(gathered, fill))
+        red = masked.amin(1) if op == 2 else masked.amax(1)
+        red = torch.where(valid.any(1)[:, None], red, torch.zeros_like(red))
+    red.backward(g.float())
+    want = xf.grad.to(torch.bfloat16)
+    assert np.array_equal(got, _bits(want))
+
+
+def test_reduce_feat_bwd_first_winner_on_ties_and_untouched_rows(oracle):
+    """ties go to the first slot that reaches the extreme (reference loop, strict comparison,
+    batch_psh_subbuck_reduce_bwd.cuh:96-104); rows that no slot refers to keep the prefill"""
+    x = _bits(torch.tensor([[1.0], [5.0], [5.0], [2.0], [7.0]], dtype=torch.bfloat16))
+    unpool = np.array([[3, 1, 2, 0]], dtype=np.uint32)            # values 2, 5, 5, 1 ; row 4 is never referred to
+    g = _bits(torch.tensor([[3.0]], dtype=torch.bfloat16))
+    prefill = _bits(torch.full((5, 1), 9.0, dtype=torch.bfloat16))
+    mx = oracle.reduce_feat_bwd(g, x, unpool, 3, grad_in_init=prefill)
+    f = lambda b: oracle.bf16_bits_to_f32(b).reshape(-1).tolist()
+    assert f(mx) == [0.0, 3.0, 0.0, 0.0, 9.0]                     # slot 1 (row 1) wins the tie against slot 2 (row 2)
+    mn = oracle.reduce_feat_bwd(g, x, unpool, 2, grad_in_init=prefill)
+    assert f(mn) == [3.0, 0.0, 0.0, 0.0, 9.0]
+    mean = oracle.reduce_feat_bwd(g, x, np.array([[3, 1, 2, 77]], dtype=np.uint32), 0, grad_in_init=prefill)
+    assert f(mean) == [9.0, 1.0, 1.0, 1.0, 9.0]                   # 3 valid slots share the gradient
+
+
+@pytest.mark.parametrize("S,C", [(2, 16), (3, 5), (8, 8)])
+def test_additive_unpool_bwd_vs_torch_autograd(oracle, S, C):
+    """up[r] = down[i] + res[r] (reference tests/test_unpooling.py:127-134) differentiated by torch in fp32:
+    grad_res is the output gradient on the pooled rows, grad_down the per-row sum rounded once to bf16"""
+    rng = np.random.default_rng(S * 10 + C)
+    n = 157
+    unpool = _random_inverse_map(rng, n, S, holes=9)
+    r = unpool.shape[0]
+    g = torch.from_numpy(rng.normal(0, 1, (n, C)).astype(np.float32)).to(torch.bfloat16)
+    grad_res, grad_down = oracle.additive_unpool_bwd(_bits(g), unpool, down_rows=r + 3)
+    res = torch.zeros(n, C, requires_grad=True)
+    down = torch.zeros(r + 3, C, requires_grad=True)
+    idx = torch.from_numpy(unpool.astype(np.int64))
+    rows = idx[idx < n]
+    src = torch.arange(r)[:, None].expand(r, S)[idx < n]
+    up = torch.zeros(n, C).index_add(0, rows, down[src]) + res      # every point appears exactly once
+    up.backward(g.float())
+    assert np.array_equal(grad_res, _bits(res.grad.to(torch.bfloat16)))
+    assert np.array_equal(grad_down, _bits(down.grad.to(torch.bfloat16)))
+    assert not grad_down[r:].any()
