@@ -38,7 +38,7 @@ constexpr size_t xs_lds_bytes() {
   return front + (size_t)WAVES * 32 * kPatchRow * 2 + (size_t)NBUF * 1024;
 }
 
-// EPI: 0 = bias only, 1 = runtime activation and / or residual.
+// EPI: 0 = bias only, 1 = runtime activation and / or residual, 2 = residual only (its pieces are prefetched).
 // With LN the kernel expects w = w' and the table lnx as prepared by ln_fold_kernel.
 // NBUF: w chunk buffers in LDS (chunk c + NBUF - 1 is requested when chunk c starts).
 template <int K, int MT, int WAVES, int NBUF, bool LN, bool SWIGLU, int EPI>
@@ -279,7 +279,25 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
 #pragma unroll
           for (int e = 0; e < 16; ++e) acc[nt][mt][e] *= ln_a[mt];
     }
-    auto flush_tile = [&](auto full_tag, int mt, uint32_t colbase) {
+    // Residual pieces of the whole chunk are requested up front (one memory latency for all of them, hidden
+    // behind the packing below) instead of one by one where they are added.  Rows past M read row M - 1.
+    constexpr int NT_OUT = SWIGLU ? 1 : 2;
+    u32x4_t rres[EPI == 2 ? MT : 1][NT_OUT][2];
+    if (EPI == 2) {
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int nt = 0; nt < NT_OUT; ++nt)
+#pragma unroll
+          for (int h2 = 0; h2 < 2; ++h2) {
+            const uint32_t rr = (lane >> 2) + h2 * 16, ch = (lane & 3u) * 8;
+            const uint32_t row = min(row0 + mt * 32 + rr, M - 1);
+            const uint32_t lrow = row - blockIdx.x * ROWS_WG;
+            if (col0 + nt * 32 < n_out)
+              rres[mt][nt][h2] = *reinterpret_cast<const u32x4_t*>(res_wg + (lrow * ldr + col0 + nt * 32 + ch));
+          }
+    }
+    auto flush_tile = [&](auto full_tag, int mt, int nt_out, uint32_t colbase) {
       // patch holds rows [mt*32, mt*32+32) x 32 columns starting at output column colbase
       constexpr bool kFull = decltype(full_tag)::value;
 #pragma unroll
@@ -296,11 +314,17 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
             for (int e = 0; e < 4; ++e) t[e] = pack_bf16x2(xs_act(bf16_lo(t[e]), act), xs_act(bf16_hi(t[e]), act));
           }
           if (residual) {
-            const u32x4_t rres = *reinterpret_cast<const u32x4_t*>(res_wg + (lrow * ldr + colbase + ch));
+            const u32x4_t rv = *reinterpret_cast<const u32x4_t*>(res_wg + (lrow * ldr + colbase + ch));
 #pragma unroll
             for (int e = 0; e < 4; ++e)
-              t[e] = pack_bf16x2(bf16_lo(t[e]) + bf16_lo(rres[e]), bf16_hi(t[e]) + bf16_hi(rres[e]));
+              t[e] = pack_bf16x2(bf16_lo(t[e]) + bf16_lo(rv[e]), bf16_hi(t[e]) + bf16_hi(rv[e]));
           }
+        }
+        if (EPI == 2) {
+          const u32x4_t rv = rres[EPI == 2 ? mt : 0][nt_out][h2];
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            t[e] = pack_bf16x2(bf16_lo(t[e]) + bf16_lo(rv[e]), bf16_hi(t[e]) + bf16_hi(rv[e]));
         }
         *reinterpret_cast<u32x4_t*>(y_wg + (lrow * ldy + colbase + ch)) = t;
       }
@@ -318,7 +342,7 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
               pk.y = pack_bf16x2(acc[nt][mt][g * 4 + 2], acc[nt][mt][g * 4 + 3]);
               *reinterpret_cast<uint2*>(patch + lq * kPatchRow + g * 8 + half * 4) = pk;
             }
-            if (col0 + nt * 32 < N) flush_tile(full_tag, mt, col0 + nt * 32);
+            if (col0 + nt * 32 < N) flush_tile(full_tag, mt, nt, col0 + nt * 32);
           }
         } else {
 #pragma unroll
@@ -335,7 +359,7 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
             pk.y = pack_bf16x2(hv[2], hv[3]);
             *reinterpret_cast<uint2*>(patch + lq * kPatchRow + g * 8 + half * 4) = pk;
           }
-          flush_tile(full_tag, mt, col0);
+          flush_tile(full_tag, mt, 0, col0);
         }
       }
     };
@@ -421,6 +445,7 @@ static int launch_k(bool ln, bool swiglu, hipStream_t s, const uint16_t* x, uint
                     const uint16_t* residual, uint32_t ldr, uint16_t* y, uint32_t ldy, uint32_t M, uint32_t N,
                     uint32_t act, int device) {
   const bool general = act != F3D_ACT_NONE || residual != nullptr;
+  const bool res_only = act == F3D_ACT_NONE && residual != nullptr;
   const dim3 grid(cdiv_u32(M, 32 * MT * WAVES)), block(64 * WAVES);
   constexpr size_t lds = xs_lds_bytes<K, WAVES, NBUF>();
 #define F3D_XS(L, S, E)                                                                                            \
@@ -434,10 +459,10 @@ static int launch_k(bool ln, bool swiglu, hipStream_t s, const uint16_t* x, uint
     hipLaunchKernelGGL(kern, grid, block, lds, s, x, ldx, eps, w, bias, lnx, residual, ldr, y, ldy, M, N,          \
                        act);                                                                                       \
   } while (0)
-  if (ln && swiglu) { if (general) F3D_XS(true, true, 1); else F3D_XS(true, true, 0); }
-  else if (ln) { if (general) F3D_XS(true, false, 1); else F3D_XS(true, false, 0); }
-  else if (swiglu) { if (general) F3D_XS(false, true, 1); else F3D_XS(false, true, 0); }
-  else { if (general) F3D_XS(false, false, 1); else F3D_XS(false, false, 0); }
+  if (ln && swiglu) { if (res_only) F3D_XS(true, true, 2); else if (general) F3D_XS(true, true, 1); else F3D_XS(true, true, 0); }
+  else if (ln) { if (res_only) F3D_XS(true, false, 2); else if (general) F3D_XS(true, false, 1); else F3D_XS(true, false, 0); }
+  else if (swiglu) { if (res_only) F3D_XS(false, true, 2); else if (general) F3D_XS(false, true, 1); else F3D_XS(false, true, 0); }
+  else { if (res_only) F3D_XS(false, false, 2); else if (general) F3D_XS(false, false, 1); else F3D_XS(false, false, 0); }
 #undef F3D_XS
   return F3D_OK;
 }
