@@ -239,7 +239,18 @@ def sub_metrics(dev):
     flm = 4.0 * float((kl.double() ** 2).sum()) * H * D
     out["attention_c2_masked"] = {"ms": round(ms, 4), "tflops": round(flm / ms / 1e9, 2),
                                   "algorithmic_gflop": round(flm / 1e9, 2)}
-    del qkv, q, k, v, o, lse
+    # backward on the same shape: five products of 2 T D per (query, head) (dV, dP, dS->dQ, dS->dK, and S once;
+    # the kernels recompute S once more, which is not counted)
+    d_o = torch.randn(1, L, H, D, generator=g).to(torch.bfloat16).to(dev)
+    dq, dk, dv = [torch.zeros(1, L, H, D, dtype=torch.bfloat16, device=dev) for _ in range(3)]
+    dlt = torch.zeros(1, L, H, dtype=torch.float32, device=dev)
+    pshattn.buck_swin_fwd(q, k, v, o, lse, sc, BS)
+    ms = ev_time(lambda: pshattn.buck_swin_bwd(q, k, v, o, d_o, lse, dlt, dq, dk, dv, sc, BS), 30)
+    flb = 10.0 * L * BS * H * D
+    out["attention_c2_backward"] = {"ms": round(ms, 4), "tflops": round(flb / ms / 1e9, 2),
+                                    "frac_of_bf16_mfma_peak": round(flb / ms / 1e9 / MFMA_BF16_PEAK_TFLOPS, 4),
+                                    "algorithmic_gflop": round(flb / 1e9, 2)}
+    del qkv, q, k, v, o, lse, d_o, dq, dk, dv, dlt
     # ---- PSH: config 1 (latency bound) and a saturating batch, 30 B/pt three-kernel accounting ----
     for name, n_c, b in (("psh_c1_32768", 32768, 1), ("psh_saturating_64x262144", 262144, 64)):
         gg = torch.Generator().manual_seed(1001)

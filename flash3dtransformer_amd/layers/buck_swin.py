@@ -13,8 +13,8 @@ from .nn_ops import Linear
 
 
 class BuckSwinFwdFunction(Function):
-    """O = attention(Q, K, V) inside every scope of buckets; keeps (Q, K, V, O, LSE) for a backward
-    pass that this library does not provide (buck_swin.py:20-95 of the reference)."""
+    """O = attention(Q, K, V) inside every scope of buckets; keeps (Q, K, V, O, LSE) for the backward
+    pass (buck_swin.py:20-95 of the reference)."""
 
     @staticmethod
     def forward(ctx, Q, K, V, scope_buckets, buck_size: int) -> torch.Tensor:
@@ -26,7 +26,12 @@ class BuckSwinFwdFunction(Function):
 
     @staticmethod
     def backward(ctx, grad_output) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, None, None]:
-        raise NotImplementedError("buck_swin_bwd: the gfx950 library implements the forward pass only")
+        Q, K, V, O, lse = ctx.saved_tensors
+        dO = grad_output if grad_output.dtype == torch.bfloat16 else grad_output.to(torch.bfloat16)
+        bwd = sa.BuckSwinBwdBuffers.create_buckswin_buffers(O, ctx.scope_buckets, ctx.buck_size)
+        pshattn.buck_swin_bwd(Q, K, V, O, dO.contiguous(), lse, bwd.Delta, bwd.dQ, bwd.dK, bwd.dV, ctx.scope_buckets,
+                              ctx.buck_size)
+        return bwd.dQ, bwd.dK, bwd.dV, None, None
 
 
 class BucketSwinAttention(nn.Module):

@@ -331,8 +331,32 @@ def buck_swin_fwd(Q, K, V, O, L, Scope_buckets, bucket_size, kv_len=None):
 
 
 def buck_swin_bwd(Q, K, V, O, dO, LSE, Delta, dQ, dK, dV, Scope_buckets, bucket_size):
-    """declared src/f3d_frontend.cu:94-97 — backward, not part of the forward hot path"""
-    raise NotImplementedError("buck_swin_bwd: the gfx950 library implements the forward path only")
+    """declared src/f3d_frontend.cu:94-97, called at flash3dxfmr/layers/buck_swin.py:90-92.
+    Q, K, V [B,L,H,D] bf16 (may be column slices of one projection output, equal strides); O, dO, dQ, dK, dV dense
+    [B,L,H,D] bf16; LSE (from the forward), Delta (written here: rowsum(dO * O)) [B,L,H] fp32.  Rows that no scope
+    covers are not written (pass zero-filled dQ / dK / dV).  Scopes of 256 or 512 tokens, head_dim 16 or 32."""
+    dev = assert_same_device([Q, K, V, O, dO, LSE, Delta, dQ, dK, dV, Scope_buckets])
+    assert_dtype([Q, K, V, O, dO, dQ, dK, dV], torch.bfloat16)
+    assert_dtype([LSE, Delta], torch.float32)
+    assert_dtype([Scope_buckets], torch.uint32)
+    assert_contiguous([O, dO, dQ, dK, dV, LSE, Delta, Scope_buckets])
+    if Q.dim() != 4 or any(t.shape != Q.shape for t in (K, V, O, dO, dQ, dK, dV)):
+        raise RuntimeError("Q/K/V/O/dO/dQ/dK/dV must share one [B,L,H,D] shape")
+    B, Ls, H, D = Q.shape
+    if tuple(LSE.shape) != (B, Ls, H) or tuple(Delta.shape) != (B, Ls, H):
+        raise RuntimeError(f"LSE / Delta shape must be {(B, Ls, H)}")
+    if Scope_buckets.dim() != 2:
+        raise RuntimeError("Scope_buckets must be [num_scopes, scope_size]")
+    for t in (Q, K, V):
+        if t.stride(3) != 1 or t.stride(2) != D or t.stride(0) != t.stride(1) * Ls or t.stride() != Q.stride():
+            raise RuntimeError("Q/K/V must be dense over (H, D) with identical strides")
+    rc = _load().f3d_buck_swin_bwd(
+        _ptr(Q), _ptr(K), _ptr(V), _u32(Q.stride(1)), _ptr(O), _ptr(dO), _ptr(LSE), _ptr(Delta), _ptr(dQ), _ptr(dK),
+        _ptr(dV), _ptr(Scope_buckets), _u32(Scope_buckets.shape[0]), _u32(Scope_buckets.shape[1]), _u32(bucket_size),
+        _u32(B), _u32(Ls), _u32(H), _u32(D), _i32(dev), _stream(dev))
+    if rc == 2:   # F3D_ERR_UNSUPPORTED: a shape outside the backward kernels
+        raise NotImplementedError(_load().f3d_last_error().decode("utf-8", "replace"))
+    _check(rc)
 
 
 # ---------------------------------------------------------------------------------------------

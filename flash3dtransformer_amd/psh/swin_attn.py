@@ -1,4 +1,4 @@
-"""Output buffers of the bucketed attention op (reference: flash3dxfmr/psh/swin_attn.py:13-24)."""
+"""Output buffers of the bucketed attention ops (reference: flash3dxfmr/psh/swin_attn.py:13-43)."""
 from dataclasses import dataclass
 
 import torch
@@ -16,3 +16,23 @@ class BuckSwinFwdBuffers:
         # every plan of bucket_scope.py covers all rows, so the model path never reads such a row
         return BuckSwinFwdBuffers(torch.empty(B, L, H, D, dtype=Q.dtype, device=Q.device),
                                   torch.zeros(B, L, H, dtype=torch.float32, device=Q.device))
+
+
+@dataclass(slots=True)
+class BuckSwinBwdBuffers:
+    """gradient buffers of the backward op (reference: psh/swin_attn.py:26-43): zero-filled, because rows that no
+    scope covers are not written; dense [B, L, H, D] whatever the layout of O"""
+    O: torch.Tensor
+    dQ: torch.Tensor
+    dK: torch.Tensor
+    dV: torch.Tensor
+    Scope_buckets: torch.Tensor
+    Delta: torch.Tensor
+    buck_size: int
+
+    @staticmethod
+    def create_buckswin_buffers(O: torch.Tensor, Scope_buckets: torch.Tensor, buck_size: int):
+        B, L, H, D = O.shape
+        Delta = torch.zeros(B, L, H, dtype=torch.float32, device=O.device)
+        mk = lambda: torch.zeros(B, L, H, D, dtype=O.dtype, device=O.device)
+        return BuckSwinBwdBuffers(O, mk(), mk(), mk(), Scope_buckets, Delta, buck_size)

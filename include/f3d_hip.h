@@ -147,6 +147,18 @@ int f3d_subbuck_reduce_bwd(const f3d_bf16_t* grad_red_feat, const f3d_bf16_t* in
                            f3d_bf16_t* grad_input_feat, uint32_t total_n, uint32_t reduced_n, uint32_t feat_dim,
                            uint32_t subbuck_size, uint32_t red_op, int device, void* stream);
 
+/* ---- bucketed attention backward: buck_swin_bwd, declared src/f3d_frontend.cu:94-97, called from
+ *      flash3dxfmr/layers/buck_swin.py:69-95 (kernel source absent from the reference) ------------
+ * q,k,v [batch,seq_len,num_head,head_dim] bf16 with row stride qkv_row_stride (elements); o, d_o, dq, dk, dv dense
+ * [batch,seq_len,num_head,head_dim] bf16; lse (from the forward), delta (output: rowsum(d_o * o))
+ * [batch,seq_len,num_head] fp32.  Rows that no scope covers are not written.  Supported: head_dim 16 or 32, scopes of
+ * 256 or 512 tokens in at most 4 buckets; anything else returns F3D_ERR_UNSUPPORTED. */
+int f3d_buck_swin_bwd(const f3d_bf16_t* q, const f3d_bf16_t* k, const f3d_bf16_t* v, uint32_t qkv_row_stride,
+                      const f3d_bf16_t* o, const f3d_bf16_t* d_o, const float* lse, float* delta, f3d_bf16_t* dq,
+                      f3d_bf16_t* dk, f3d_bf16_t* dv, const uint32_t* scope_buckets, uint32_t num_scope,
+                      uint32_t scope_size, uint32_t bucket_size, uint32_t batch, uint32_t seq_len, uint32_t num_head,
+                      uint32_t head_dim, int device, void* stream);
+
 /* ---- bucketed attention forward: buck_swin_fwd, declared src/f3d_frontend.cu:90-92, called from
  *      flash3dxfmr/layers/buck_swin.py:57 (kernel source absent from the reference) --------------
  * q,k,v,o [batch,seq_len,num_head,head_dim] bf16 contiguous; lse [batch,seq_len,num_head] fp32;

@@ -349,6 +349,36 @@ def buck_swin_fwd(Q, K, V, scope_buckets, bucket_size, kv_len=None, O_init=None,
     return O, LSE
 
 
+def buck_swin_bwd(Q, K, V, dO, scope_buckets, bucket_size):
+    """Backward of buck_swin_fwd (pshattn.buck_swin_bwd, declared src/f3d_frontend.cu:94-97; the formulas are the
+    ones the reference's tests take from autograd, tests/test_attn_bwd.py): per scope and head, with
+    P = softmax(Q Kt / sqrt(D)),  Delta = rowsum(dO * O),  dV = Pt dO,  dP = dO Vt,  dS = P * (dP - Delta),
+    dQ = dS K / sqrt(D),  dK = dSt Q / sqrt(D).  Rows no scope covers get zero gradients.
+    Returns (dQ, dK, dV, Delta) in fp32."""
+    import torch
+
+    B, L, H, D = Q.shape
+    scopes = torch.as_tensor(np.asarray(scope_buckets).astype(np.int64))
+    Qf, Kf, Vf, dOf = Q.float(), K.float(), V.float(), dO.float()
+    dQ, dK, dV = torch.zeros_like(Qf), torch.zeros_like(Kf), torch.zeros_like(Vf)
+    Delta = torch.zeros(B, L, H, dtype=torch.float32)
+    ar = torch.arange(bucket_size)
+    scale = 1.0 / math.sqrt(D)
+    for s in range(scopes.shape[0]):
+        rows = (scopes[s][:, None] * bucket_size + ar[None, :]).reshape(-1)
+        q, k, v, do = [t[:, rows].permute(0, 2, 1, 3) for t in (Qf, Kf, Vf, dOf)]   # [B,H,T,D]
+        p = torch.softmax(torch.matmul(q, k.transpose(-1, -2)) * scale, dim=-1)
+        o = torch.matmul(p, v)
+        delta = (do * o).sum(-1)                                                    # [B,H,T]
+        dp = torch.matmul(do, v.transpose(-1, -2))
+        ds = p * (dp - delta[..., None])
+        dQ[:, rows] = (torch.matmul(ds, k) * scale).permute(0, 2, 1, 3)
+        dK[:, rows] = (torch.matmul(ds.transpose(-1, -2), q) * scale).permute(0, 2, 1, 3)
+        dV[:, rows] = torch.matmul(p.transpose(-1, -2), do).permute(0, 2, 1, 3)
+        Delta[:, rows] = delta.permute(0, 2, 1)
+    return dQ, dK, dV, Delta
+
+
 def linear(x, w, b=None):
     """y = x @ w.T + b in fp32 (torch.nn.Linear semantics; layers/buck_swin.py:159,163)"""
     import torch

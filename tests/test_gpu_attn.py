@@ -200,3 +200,83 @@ def test_attention_argument_errors():
     pshattn.buck_swin_fwd(q, q, q, O, mk(1, 256, 2, dt=torch.float32), bad, 256)
     torch.cuda.synchronize()
     assert (O == 3.0).all()
+
+
+# ---------------------------------------------------------------------------------------------
+# backward (reference op buck_swin_bwd; its tests differentiate an SDPA oracle, tests/test_attn_bwd.py)
+# ---------------------------------------------------------------------------------------------
+
+def _run_bwd(Q, K, V, dO, scopes, bs, fused_buffer=False):
+    """forward then backward through the C ABI; Q/K/V optionally as column slices of one [B,L,3HD] buffer"""
+    from flash3dtransformer_amd.lib import pshattn
+    B, L, H, D = Q.shape
+    if fused_buffer:
+        qkv = torch.cat([Q.reshape(B, L, H * D), K.reshape(B, L, H * D), V.reshape(B, L, H * D)], dim=-1).to(DEV)
+        q, k, v = [t.view(B, L, H, D) for t in qkv.chunk(3, dim=-1)]
+    else:
+        q, k, v = Q.to(DEV), K.to(DEV), V.to(DEV)
+    O = torch.zeros(B, L, H, D, dtype=torch.bfloat16, device=DEV)
+    LSE = torch.zeros(B, L, H, dtype=torch.float32, device=DEV)
+    sc = torch.from_numpy(np.ascontiguousarray(scopes, dtype=np.uint32).view(np.int32)).to(DEV).view(torch.uint32)
+    pshattn.buck_swin_fwd(q, k, v, O, LSE, sc, bs)
+    dq, dk, dv = [torch.zeros(B, L, H, D, dtype=torch.bfloat16, device=DEV) for _ in range(3)]
+    delta = torch.zeros(B, L, H, dtype=torch.float32, device=DEV)
+    pshattn.buck_swin_bwd(q, k, v, O, dO.to(DEV), LSE, delta, dq, dk, dv, sc, bs)
+    torch.cuda.synchronize()
+    return [t.float().cpu() for t in (dq, dk, dv)] + [delta.cpu(), O.float().cpu()]
+
+
+def _check_grads(got, want, what):
+    for g, w, n in zip(got, want, ("dQ", "dK", "dV")):
+        err = (g - w).abs()
+        ref = max(1.0, w.abs().max().item())
+        assert err.max().item() <= TOL * ref, f"{what} {n}: max err {err.max().item()} at scale {ref}"
+        assert err.mean().item() <= 2e-3 * ref, f"{what} {n}: mean err {err.mean().item()}"
+
+
+@pytest.mark.parametrize("B,L,H,D,bs,scope_size,fused", [
+    (2, 2048, 2, 32, 512, 1, True),      # the model's block: one 512-token bucket per scope, Q/K/V slices of one buffer
+    (1, 1024, 3, 16, 256, 2, False),     # 512 tokens in two buckets, 16-wide heads
+    (2, 1024, 2, 32, 128, 2, True),      # 256-token scopes
+    (1, 1024, 1, 16, 128, 2, False),
+    (1, 2048, 4, 32, 128, 4, False),     # four buckets per scope
+])
+def test_backward_vs_oracle(oracle, B, L, H, D, bs, scope_size, fused):
+    Q, K, V = _qkv(7 + D + bs, B, L, H, D)
+    g = torch.Generator().manual_seed(3)
+    dO = torch.randn(B, L, H, D, generator=g).to(torch.bfloat16)
+    nb = L // bs
+    rng = np.random.default_rng(nb)
+    scopes = rng.permutation(nb).astype(np.uint32).reshape(nb // scope_size, scope_size)   # buckets in shuffled order
+    dq, dk, dv, delta, O = _run_bwd(Q, K, V, dO, scopes, bs, fused_buffer=fused)
+    wq, wk, wv, wdelta = oracle.buck_swin_bwd(Q, K, V, dO, scopes, bs)
+    _check_grads((dq, dk, dv), (wq, wk, wv), f"D={D} bs={bs} scope={scope_size}")
+    # Delta is formed from the bf16 O the forward wrote
+    assert (delta - (dO.float() * O).sum(-1)).abs().max().item() <= 1e-3 * max(1.0, wdelta.abs().max().item())
+
+
+def test_backward_leaves_uncovered_rows_untouched(oracle):
+    B, L, H, D, bs = 1, 2048, 2, 32, 512
+    Q, K, V = _qkv(21, B, L, H, D)
+    dO = torch.randn(B, L, H, D, generator=torch.Generator().manual_seed(4)).to(torch.bfloat16)
+    scopes = np.array([[2], [0]], dtype=np.uint32)                 # buckets 1 and 3 belong to no scope
+    dq, dk, dv, _, _ = _run_bwd(Q, K, V, dO, scopes, bs)
+    for t in (dq, dk, dv):
+        assert not t[:, 512:1024].any() and not t[:, 1536:].any()
+    wq, wk, wv, _ = oracle.buck_swin_bwd(Q, K, V, dO, scopes, bs)
+    _check_grads((dq, dk, dv), (wq, wk, wv), "partial cover")
+
+
+def test_attention_module_backpropagates(oracle):
+    """gradients reach Q, K, V through the autograd function of the layer API (reference: layers/buck_swin.py:20-95)"""
+    from flash3dtransformer_amd.layers.buck_swin import BucketSwinAttention
+    B, L, H, D, bs = 1, 1024, 2, 32, 512
+    Q, K, V = [t.to(DEV).requires_grad_(True) for t in _qkv(31, B, L, H, D)]
+    scopes = np.array([[0], [1]], dtype=np.uint32)
+    sc = torch.from_numpy(scopes.view(np.int32)).to(DEV).view(torch.uint32)
+    w = torch.randn(B, L, H, D, generator=torch.Generator().manual_seed(5)).to(torch.bfloat16)
+    O = BucketSwinAttention(bs)(Q, K, V, sc)
+    (O.float() * w.to(DEV).float()).sum().backward()
+    torch.cuda.synchronize()
+    wq, wk, wv, _ = oracle.buck_swin_bwd(Q.detach().cpu(), K.detach().cpu(), V.detach().cpu(), w, scopes, bs)
+    _check_grads([t.grad.float().cpu() for t in (Q, K, V)], (wq, wk, wv), "autograd")

@@ -114,9 +114,15 @@ def test_forward_only_ops_refuse_backward():
     y = lin(x)
     with pytest.raises(NotImplementedError):
         y.float().sum().backward()
+    # attention backward exists for the resident shapes only; other shapes say so
     from flash3dtransformer_amd.lib import pshattn
+    B, Ls, H, D = 1, 512, 1, 64
+    z = lambda *s_: torch.zeros(*s_, dtype=torch.bfloat16, device=DEV)
+    f = lambda *s_: torch.zeros(*s_, dtype=torch.float32, device=DEV)
+    sc = torch.zeros(1, 1, dtype=torch.int32, device=DEV).view(torch.uint32)
     with pytest.raises(NotImplementedError):
-        pshattn.buck_swin_bwd(*([None] * 12))
+        pshattn.buck_swin_bwd(z(B, Ls, H, D), z(B, Ls, H, D), z(B, Ls, H, D), z(B, Ls, H, D), z(B, Ls, H, D), f(B, Ls, H),
+                              f(B, Ls, H), z(B, Ls, H, D), z(B, Ls, H, D), z(B, Ls, H, D), sc, 512)
 
 
 def test_state_dict_names_match_reference_module_tree():

@@ -281,3 +281,23 @@ def test_additive_unpool_bwd_vs_torch_autograd(oracle, S, C):
     assert np.array_equal(grad_res, _bits(res.grad.to(torch.bfloat16)))
     assert np.array_equal(grad_down, _bits(down.grad.to(torch.bfloat16)))
     assert not grad_down[r:].any()
+
+
+def test_attention_bwd_formulas_vs_autograd(oracle):
+    """the explicit backward formulas against torch autograd through the oracle's forward (the reference's own
+    tests differentiate an SDPA / FA2 oracle the same way, tests/test_attn_bwd.py)"""
+    rng = np.random.default_rng(11)
+    B, L, H, D, bs = 2, 512, 3, 16, 128
+    Q, K, V = [t.float().requires_grad_(True) for t in _qkv(rng, B, L, H, D)]
+    scopes = np.array([[1, 0], [3, 2]], dtype=np.uint32)
+    dO = torch.from_numpy(rng.normal(0, 1, (B, L, H, D)).astype(np.float32))
+    O, _ = oracle.buck_swin_fwd(Q, K, V, scopes, bs)
+    O.backward(dO)
+    dQ, dK, dV, Delta = oracle.buck_swin_bwd(Q.detach(), K.detach(), V.detach(), dO, scopes, bs)
+    for got, want in ((dQ, Q.grad), (dK, K.grad), (dV, V.grad)):
+        assert (got - want).abs().max().item() <= 2e-5 * max(1.0, want.abs().max().item())
+    assert (Delta - (dO * O.detach()).sum(-1)).abs().max().item() <= 1e-5
+    # a scope table that leaves buckets out: their rows get zero gradients
+    dQ2, dK2, dV2, _ = oracle.buck_swin_bwd(Q.detach(), K.detach(), V.detach(), dO, np.array([[1, 0]], dtype=np.uint32), bs)
+    assert not dQ2[:, 256:].any() and not dK2[:, 256:].any() and not dV2[:, 256:].any()
+    assert torch.equal(dQ2[:, :256], dQ[:, :256])
