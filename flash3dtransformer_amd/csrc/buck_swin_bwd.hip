@@ -15,8 +15,8 @@
 //         transposed from LDS (ds_read_b64_tr_b16).  Also writes Delta.
 //   dq  : a wave owns 32 QUERIES (Q, dO rows in registers, LSE and Delta one scalar per lane) and walks the key
 //         tiles; St = K Qt, dPt = V dOt, dQt += Kt dSt with Kt read transposed.
-// Every array that is read both ways is kept twice in LDS: once with the 16-byte pieces of a row XOR-swizzled
-// (conflict-free 128-bit operand reads) and once plain (the transposing reads address 8-byte pieces per lane).
+// LDS rows are unpadded with their 16-byte pieces XOR-swizzled (conflict-free 128-bit operand reads); the transposing
+// reads address 8-byte pieces per lane and apply the same swizzle to their addresses.
 // The score tile is computed twice (once per kernel), which keeps both kernels free of atomics: every output row
 // is written by exactly one wave.  Rows that no scope covers are not written (the caller passes zeros).
 #include <type_traits>
@@ -69,21 +69,35 @@ __device__ __forceinline__ void bwd_fill_rows(const uint16_t* gbase, uint32_t ld
   }
 }
 
-// A operand read transposed from a plain row-major LDS tile of 32 rows: lane (m = feature) gets, for k-step kk,
+// A operand read transposed from a swizzled LDS tile of 32 rows: lane (m = feature) gets, for k-step kk,
 // slots 0..3 = rows 16 kk + 4 half + 0..3 and slots 4..7 = the same + 8 (the order in which an accumulator tile
-// hands its rows to the next MFMA as a B operand)
+// hands its rows to the next MFMA as a B operand).  tr_lo / tr_hi are the lane's byte offsets for the two row
+// groups (their swizzle values differ); k-step kk adds 16 rows, which leaves the swizzle value unchanged.
 template <int D>
-__device__ __forceinline__ void bwd_load_tr(const char* tile, uint32_t tr_off, bool tr_lane, bf16x8_t (&f)[2]) {
+__device__ __forceinline__ void bwd_load_tr(const char* tile, uint32_t tr_lo, uint32_t tr_hi, bool tr_lane,
+                                            bf16x8_t (&f)[2]) {
   constexpr int ROWB = BwdGeom<D>::ROWB;
 #pragma unroll
   for (int kk = 0; kk < 2; ++kk) {
     i16x4_t lo = {0, 0, 0, 0}, hi = {0, 0, 0, 0};
     if (tr_lane) {
-      lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_t*)(tile + tr_off + (kk * 16) * ROWB));
-      hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_t*)(tile + tr_off + (kk * 16 + 8) * ROWB));
+      lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_t*)(tile + tr_lo + (kk * 16) * ROWB));
+      hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_t*)(tile + tr_hi + (kk * 16) * ROWB));
     }
     f[kk] = __builtin_bit_cast(bf16x8_t, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
   }
+}
+
+// the lane's byte offset of its 8-byte piece for the transposing reads: row 4 half + l16 / 4 + 8 hi of a 32-row
+// tile, features d_base + 4 (l16 % 4) .. + 3, with the row's swizzle applied to the 16-byte piece index
+template <int D>
+__device__ __forceinline__ uint32_t bwd_tr_offset(uint32_t lane, uint32_t hi) {
+  using G = BwdGeom<D>;
+  const uint32_t half = lane >> 5, l16 = lane & 15u, d_base = 16u * ((lane >> 4) & 1u);
+  const uint32_t row = 4u * half + l16 / 4u + 8u * hi;
+  const uint32_t colb = (d_base + 4u * (l16 & 3u)) * 2u;                    // byte column, a multiple of 8
+  const uint32_t piece = (colb / 16u) ^ ((row / G::SWZ_DIV) & (G::CPK - 1));
+  return row * G::ROWB + piece * 16u + (colb & 8u);
 }
 
 struct BwdItem {
@@ -102,11 +116,11 @@ __device__ __forceinline__ bool bwd_item(uint32_t n_items, uint32_t items_per_xc
 
 template <int D, int T>
 constexpr size_t bwd_dkdv_lds_bytes() {
-  return (size_t)4 * T * D * 2 + (size_t)2 * T * 4 + kBwdMaxScope * 4;
+  return (size_t)2 * T * D * 2 + (size_t)2 * T * 4 + kBwdMaxScope * 4;
 }
 template <int D, int T>
 constexpr size_t bwd_dq_lds_bytes() {
-  return (size_t)3 * T * D * 2 + kBwdMaxScope * 4;
+  return (size_t)2 * T * D * 2 + kBwdMaxScope * 4;
 }
 
 // ---- dK, dV (and Delta) -----------------------------------------------------------------------------
@@ -120,11 +134,9 @@ __global__ __launch_bounds__(2 * T) void buck_swin_bwd_dkdv_kernel(
   using G = BwdGeom<D>;
   constexpr int KSTEPS = G::KSTEPS, ROWB = G::ROWB, OPB = T * ROWB;
   extern __shared__ __attribute__((aligned(16))) char lds_bwd[];
-  char* sQs = lds_bwd;              // Q, swizzled pieces
-  char* sDs = lds_bwd + OPB;        // dO, swizzled pieces
-  char* sQu = lds_bwd + 2 * OPB;    // Q, plain
-  char* sDu = lds_bwd + 3 * OPB;    // dO, plain
-  float* s_lse2 = reinterpret_cast<float*>(lds_bwd + 4 * OPB);   // LSE in the exponent's units (x log2 e)
+  char* sQs = lds_bwd;              // Q
+  char* sDs = lds_bwd + OPB;        // dO
+  float* s_lse2 = reinterpret_cast<float*>(lds_bwd + 2 * OPB);   // LSE in the exponent's units (x log2 e)
   float* s_delta = s_lse2 + T;
   uint32_t* s_bucket = reinterpret_cast<uint32_t*>(s_delta + T);
 
@@ -145,9 +157,7 @@ __global__ __launch_bounds__(2 * T) void buck_swin_bwd_dkdv_kernel(
   const size_t base_l = (size_t)it.batch * seq_len * num_head + it.head;
 
   bwd_fill_rows<D, true>(q + base_qkv, ld, s_bucket, bs, wave, lane, sQs);
-  bwd_fill_rows<D, false>(q + base_qkv, ld, s_bucket, bs, wave, lane, sQu);
   bwd_fill_rows<D, true>(d_o + base_o, ldo, s_bucket, bs, wave, lane, sDs);
-  bwd_fill_rows<D, false>(d_o + base_o, ldo, s_bucket, bs, wave, lane, sDu);
 
   // this wave's 32 tokens: local rows [32 wave, 32 wave + 32), lane -> token lq
   const uint32_t loc = wave * 32 + lq;
@@ -191,9 +201,8 @@ __global__ __launch_bounds__(2 * T) void buck_swin_bwd_dkdv_kernel(
   __syncthreads();
 
   const uint32_t dir_off = lq * ROWB + ((half ^ ((lq / G::SWZ_DIV) & (G::CPK - 1))) * 16u);   // k-step ks: ^ (ks * 32)
-  const uint32_t l16 = lane & 15u, d_base = 16u * ((lane >> 4) & 1u);
-  const uint32_t tr_off = (4u * half + l16 / 4u) * ROWB + (d_base + 4u * (l16 & 3u)) * 2u;
-  const bool tr_lane = D >= 32 || d_base < (uint32_t)D;
+  const uint32_t tr_lo = bwd_tr_offset<D>(lane, 0), tr_hi = bwd_tr_offset<D>(lane, 1);
+  const bool tr_lane = D >= 32 || 16u * ((lane >> 4) & 1u) < (uint32_t)D;
 
   f32x16_t acc_dk, acc_dv;
 #pragma unroll
@@ -212,8 +221,8 @@ __global__ __launch_bounds__(2 * T) void buck_swin_bwd_dkdv_kernel(
       p_acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(da, vf[ks], p_acc, 0, 0, 0);   // dP[query][key]
     }
     bf16x8_t dot[2], qtr[2];
-    bwd_load_tr<D>(sDu + tile, tr_off, tr_lane, dot);
-    bwd_load_tr<D>(sQu + tile, tr_off, tr_lane, qtr);
+    bwd_load_tr<D>(sDs + tile, tr_lo, tr_hi, tr_lane, dot);
+    bwd_load_tr<D>(sQs + tile, tr_lo, tr_hi, tr_lane, qtr);
     // register i of a lane is query (i/4)*8 + 4 half + i%4 of the tile
     uint32_t pb[8], sb[8];
 #pragma unroll
@@ -270,10 +279,9 @@ __global__ __launch_bounds__(2 * T) void buck_swin_bwd_dq_kernel(
   using G = BwdGeom<D>;
   constexpr int KSTEPS = G::KSTEPS, ROWB = G::ROWB, OPB = T * ROWB;
   extern __shared__ __attribute__((aligned(16))) char lds_bwd[];
-  char* sKs = lds_bwd;             // K, swizzled pieces
-  char* sVs = lds_bwd + OPB;       // V, swizzled pieces
-  char* sKu = lds_bwd + 2 * OPB;   // K, plain
-  uint32_t* s_bucket = reinterpret_cast<uint32_t*>(lds_bwd + 3 * OPB);
+  char* sKs = lds_bwd;             // K
+  char* sVs = lds_bwd + OPB;       // V
+  uint32_t* s_bucket = reinterpret_cast<uint32_t*>(lds_bwd + 2 * OPB);
 
   BwdItem it;
   if (!bwd_item(n_items, items_per_xcd, num_scope, num_head, it)) return;
@@ -293,7 +301,6 @@ __global__ __launch_bounds__(2 * T) void buck_swin_bwd_dq_kernel(
 
   bwd_fill_rows<D, true>(k + base_qkv, ld, s_bucket, bs, wave, lane, sKs);
   bwd_fill_rows<D, true>(v + base_qkv, ld, s_bucket, bs, wave, lane, sVs);
-  bwd_fill_rows<D, false>(k + base_qkv, ld, s_bucket, bs, wave, lane, sKu);
 
   const uint32_t loc = wave * 32 + lq;
   const uint32_t lj = loc / bs;
@@ -315,9 +322,8 @@ __global__ __launch_bounds__(2 * T) void buck_swin_bwd_dq_kernel(
   __syncthreads();
 
   const uint32_t dir_off = lq * ROWB + ((half ^ ((lq / G::SWZ_DIV) & (G::CPK - 1))) * 16u);
-  const uint32_t l16 = lane & 15u, d_base = 16u * ((lane >> 4) & 1u);
-  const uint32_t tr_off = (4u * half + l16 / 4u) * ROWB + (d_base + 4u * (l16 & 3u)) * 2u;
-  const bool tr_lane = D >= 32 || d_base < (uint32_t)D;
+  const uint32_t tr_lo = bwd_tr_offset<D>(lane, 0), tr_hi = bwd_tr_offset<D>(lane, 1);
+  const bool tr_lane = D >= 32 || 16u * ((lane >> 4) & 1u) < (uint32_t)D;
 
   f32x16_t acc;
 #pragma unroll
@@ -335,7 +341,7 @@ __global__ __launch_bounds__(2 * T) void buck_swin_bwd_dq_kernel(
       p_acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, dof[ks], p_acc, 0, 0, 0);   // dPt[key][query]
     }
     bf16x8_t ktr[2];
-    bwd_load_tr<D>(sKu + tile, tr_off, tr_lane, ktr);
+    bwd_load_tr<D>(sKs + tile, tr_lo, tr_hi, tr_lane, ktr);
     uint32_t sb[8];
 #pragma unroll
     for (int i = 0; i < 16; i += 2) {
