@@ -3,8 +3,10 @@ norm + activation used around pooling.  Parameters are ordinary nn.Parameters (f
 a checkpoint of the reference's torch / TransformerEngine modules loads by name); the kernels run on
 bf16 copies that are refreshed whenever a parameter changes.
 
-The library implements the forward pass only: every op is wrapped in an autograd.Function whose
-backward raises, so a training loop fails loudly instead of silently dropping gradients.
+Forward runs on the HIP kernels.  Backward of these dense layers is not a kernel of this library: as the
+reference leaves it to torch / TransformerEngine, the autograd functions here differentiate a torch restatement
+of the same formula on the GPU (library GEMMs, fp32 accumulation).  The forward value never comes from that
+restatement.
 """
 import math
 
@@ -14,23 +16,65 @@ from torch import nn
 from ..lib import pshattn
 
 
-class _ForwardOnly(torch.autograd.Function):
-    """Marks the output of a forward-only kernel: asking for its gradient raises."""
+class _TorchBackward(torch.autograd.Function):
+    """Output of a HIP forward kernel whose gradient is taken through `ref_fn`, a torch restatement of the op
+    over the same inputs (None entries are passed through).  Inputs are re-read in fp32 for the backward."""
 
     @staticmethod
-    def forward(ctx, out, name, *deps):
-        ctx.name = name
+    def forward(ctx, out, ref_fn, *inputs):
+        ctx.ref_fn = ref_fn
+        ctx.is_tensor = [isinstance(t, torch.Tensor) for t in inputs]
+        ctx.save_for_backward(*[t for t in inputs if isinstance(t, torch.Tensor)])
         return out.view_as(out)
 
     @staticmethod
     def backward(ctx, grad):
-        raise NotImplementedError(f"{ctx.name}: the gfx950 library implements the forward pass only")
+        saved = list(ctx.saved_tensors)
+        ins, leaves = [], []
+        for is_t in ctx.is_tensor:
+            if not is_t:
+                ins.append(None)
+                continue
+            t = saved.pop(0)
+            leaf = t.detach().float().requires_grad_(True)
+            ins.append(leaf)
+            leaves.append((leaf, t))
+        with torch.enable_grad():
+            y = ctx.ref_fn(*ins)
+            grads = torch.autograd.grad(y, [l for l, _ in leaves], grad.float().reshape(y.shape), allow_unused=True)
+        out, gi = [None, None], iter(zip(grads, leaves))
+        for is_t in ctx.is_tensor:
+            if not is_t:
+                out.append(None)
+                continue
+            g, (_, orig) = next(gi)
+            out.append(None if g is None or not orig.requires_grad else g.to(orig.dtype).reshape(orig.shape))
+        return tuple(out)
 
 
-def forward_only(out: torch.Tensor, name: str, *deps) -> torch.Tensor:
-    if torch.is_grad_enabled() and any(isinstance(d, torch.Tensor) and d.requires_grad for d in deps):
-        return _ForwardOnly.apply(out, name, *deps)
+def torch_backward(out: torch.Tensor, ref_fn, *inputs) -> torch.Tensor:
+    """`out` = value from the HIP kernels; gradients flow to `inputs` through `ref_fn(*inputs)`"""
+    if torch.is_grad_enabled() and any(isinstance(t, torch.Tensor) and t.requires_grad for t in inputs):
+        return _TorchBackward.apply(out, ref_fn, *inputs)
     return out
+
+
+def _act_ref(z: torch.Tensor, act):
+    if act is None:
+        return z
+    if act == "swiglu":
+        h = z.shape[-1] // 2
+        return torch.nn.functional.silu(z[..., :h]) * z[..., h:]
+    return {"gelu": torch.nn.functional.gelu, "relu": torch.relu, "silu": torch.nn.functional.silu}[act](z)
+
+
+def _linear_ref(act, eps):
+    """torch restatement of Linear.forward: (x, w, b, residual, ln_w, ln_b) -> y"""
+    def ref(x, w, b, residual, ln_w, ln_b):
+        h = x if ln_w is None else torch.nn.functional.layer_norm(x, (x.shape[-1],), ln_w, ln_b, eps)
+        y = _act_ref(torch.nn.functional.linear(h, w, b), act)
+        return y if residual is None else y + residual
+    return ref
 
 
 class _Bf16Cache:
@@ -88,7 +132,12 @@ class Linear(nn.Module):
             pshattn.ln_linear_bf16(x2, g, b, pre_norm.eps, self._w.get(self.weight), self._b.get(self.bias), r2, y, act)
         else:
             pshattn.linear_bf16(x2, self._w.get(self.weight), self._b.get(self.bias), r2, y, act)
-        return forward_only(y.view(*lead, n_out), "Linear", x, self.weight)
+        ln_w = None if pre_norm is None else pre_norm.weight
+        ln_b = None if pre_norm is None else pre_norm.bias
+        eps = 0.0 if pre_norm is None else pre_norm.eps
+        res_in = None if residual is None else residual.reshape(-1, n_out)
+        out = torch_backward(y, _linear_ref(act, eps), x.reshape(-1, x.shape[-1]), self.weight, self.bias, res_in, ln_w, ln_b)
+        return out.view(*lead, n_out)
 
     def extra_repr(self):
         return f"in_features={self.in_features}, out_features={self.out_features}, bias={self.bias is not None}"
@@ -108,7 +157,9 @@ class LayerNorm(nn.Module):
         x2 = as_bf16_2d(x.reshape(-1, x.shape[-1])).contiguous()
         y = torch.empty_like(x2)
         pshattn.layernorm_bf16(x2, self._w.get(self.weight), self._b.get(self.bias), y, self.eps)
-        return forward_only(y.view(x.shape), "LayerNorm", x, self.weight)
+        eps = self.eps
+        ref = lambda xx, w, b: torch.nn.functional.layer_norm(xx, (xx.shape[-1],), w, b, eps)
+        return torch_backward(y, ref, x.reshape(-1, x.shape[-1]), self.weight, self.bias).view(x.shape)
 
 
 FUSABLE_LN_WIDTHS = (32, 64, 128, 256, 512)
@@ -141,7 +192,9 @@ def apply_norm(norm: nn.Module, x: torch.Tensor) -> torch.Tensor:
         y = torch.empty_like(x2)
         b = None if norm.bias is None else norm.bias.detach().to(torch.bfloat16)
         pshattn.layernorm_bf16(x2, norm.weight.detach().to(torch.bfloat16), b, y, norm.eps)
-        return forward_only(y.view(x.shape), "LayerNorm", x, norm.weight)
+        eps = norm.eps
+        ref = lambda xx, w, bb: torch.nn.functional.layer_norm(xx, (xx.shape[-1],), w, bb, eps)
+        return torch_backward(y, ref, x.reshape(-1, x.shape[-1]), norm.weight, norm.bias).view(x.shape)
     return norm(x)
 
 
@@ -170,7 +223,11 @@ def apply_norm_act(norm, act, x: torch.Tensor) -> torch.Tensor:
         x2 = as_bf16_2d(x).contiguous()
         y = torch.empty_like(x2)
         pshattn.affine_act_bf16(x2, scale, shift, y, act_name)
-        return forward_only(y, "BatchNorm1d+act", x)
+        mean, var, bn_eps = norm.running_mean, norm.running_var, norm.eps
+
+        def ref(xx, w, b):   # eval-mode BatchNorm1d (running statistics are constants) then the activation
+            return _act_ref(torch.nn.functional.batch_norm(xx, mean.float(), var.float(), w, b, False, 0.0, bn_eps), act_name)
+        return torch_backward(y, ref, x, norm.weight if norm.affine else None, norm.bias if norm.affine else None)
     if norm is not None:
         x = apply_norm(norm, x)
     if act is not None:
@@ -214,4 +271,13 @@ class LayerNormMLP(nn.Module):
             pshattn.linear_bf16(ln, c[2].get(self.fc1_weight), c[3].get(self.fc1_bias), None, h, self.activation)
         y = torch.empty_like(x2)
         pshattn.linear_bf16(h, c[4].get(self.fc2_weight), c[5].get(self.fc2_bias), r2, y, None)
-        return forward_only(y.view(x.shape), "LayerNormMLP", x, self.fc1_weight)
+        act, eps = self.activation, self.eps
+
+        def ref(xx, res, ln_w, ln_b, w1, b1, w2, b2):
+            hh = torch.nn.functional.layer_norm(xx, (xx.shape[-1],), ln_w, ln_b, eps)
+            out = torch.nn.functional.linear(_act_ref(torch.nn.functional.linear(hh, w1, b1), act), w2, b2)
+            return out if res is None else out + res
+        res_in = None if residual is None else residual.reshape(-1, self.hidden_size)
+        out = torch_backward(y, ref, x.reshape(-1, self.hidden_size), res_in, self.layer_norm_weight, self.layer_norm_bias,
+                             self.fc1_weight, self.fc1_bias, self.fc2_weight, self.fc2_bias)
+        return out.view(x.shape)

@@ -7,7 +7,7 @@ from torch import nn
 from ..lib import pshattn
 from ..psh import arithmatic as f3darith
 from ..psh import psh_main as pm
-from .nn_ops import Linear, forward_only
+from .nn_ops import Linear, torch_backward
 
 
 class PSHScatterLayer(nn.Module):
@@ -40,4 +40,7 @@ class PSH3DCoordEmbedding(nn.Module):
         emb = torch.empty(pad_to, self.lin.out_features, dtype=torch.bfloat16, device=coords.device)
         lin = self.lin
         pshattn.coord_embed_bf16(scattered, lin._w.get(lin.weight), lin._b.get(lin.bias), emb)
-        return forward_only(emb, "PSH3DCoordEmbedding", lin.weight)
+        # the coordinates carry no gradient; the embedding's weights do (bf16 view of the fp16 coordinates, as the kernel reads them)
+        coord_f = scattered
+        ref = lambda w, b: torch.nn.functional.linear(coord_f.to(torch.bfloat16).float(), w, b)
+        return torch_backward(emb, ref, lin.weight, lin.bias)
