@@ -61,12 +61,13 @@ def make_block(C, hid, H, bs, scope, activation, seed):
 
 
 def cpu_baseline(clouds, emb, blk, C, H, bs, scope, hash_op, activation):
-    """the oracle pipeline on the first sweep only, all host cores for the torch part"""
+    """the oracle pipeline on the whole batch (the same 4 sweeps), repeated for about ten seconds of CPU work,
+    all host cores for the torch part"""
     from oracle import f3d_oracle as orc
     from flash3dtransformer_amd import synth
     cores = os.cpu_count() or 1
     torch.set_num_threads(cores)
-    coords, seps = synth.batch_of(clouds[:1])
+    coords, seps = synth.batch_of(clouds)
     n = coords.shape[0]
     align = bs * scope * 6
     pad_to = -(-n // align) * align
@@ -77,15 +78,18 @@ def cpu_baseline(clouds, emb, blk, C, H, bs, scope, hash_op, activation):
          "fc1.weight": f(blk.mlp.mlp.fc1_weight), "fc1.bias": f(blk.mlp.mlp.fc1_bias),
          "fc2.weight": f(blk.mlp.mlp.fc2_weight), "fc2.bias": f(blk.mlp.mlp.fc2_bias)}
     ew, eb = f(emb.lin.weight), f(emb.lin.bias)
-    t0 = time.perf_counter()
-    scat = orc.psh_scatter_coords(coords, seps, bs, pad_to, hash_op)
-    x = orc._r(orc.linear(torch.from_numpy(scat.astype(np.float32)).to(torch.bfloat16), ew, eb))
-    scopes = orc.gen_scopes(pad_to, bs, scope)
-    out = orc.xfmr_block(x, w, scopes, bs, H, activation)
+    passes, t0 = 0, time.perf_counter()
+    with torch.no_grad():
+        while passes < 2 or (time.perf_counter() - t0 < 10.0 and passes < 8):
+            scat = orc.psh_scatter_coords(coords, seps, bs, pad_to, hash_op)
+            x = orc._r(orc.linear(torch.from_numpy(scat.astype(np.float32)).to(torch.bfloat16), ew, eb))
+            scopes = orc.gen_scopes(pad_to, bs, scope)
+            out = orc.xfmr_block(x, w, scopes, bs, H, activation)
+            passes += 1
     dt = time.perf_counter() - t0
-    return {"value": n / dt / 1e6, "unit": "Mpts/s", "cores": cores, "kind": "port",
-            "sample": f"first of 4 sweeps ({n} points), one pass of the same stage through the oracle "
-                      f"(C PSH single-threaded + torch fp32 on {cores} threads), {dt:.2f} s"}, out
+    return {"value": n * passes / dt / 1e6, "unit": "Mpts/s", "cores": cores, "kind": "port",
+            "sample": f"{passes} passes of the whole stage on the same 4 sweeps ({n} points) through the oracle "
+                      f"(C PSH single-threaded + torch fp32 on {cores} threads), {dt:.1f} s of CPU work"}, out
 
 
 def main():
