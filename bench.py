@@ -275,6 +275,28 @@ def sub_metrics(dev):
                      "frac_of_hbm_peak": round(byts / ms / 1e6 / HBM_PEAK_GBS, 4),
                      "mpts_per_s": round(n_c * b / ms / 1e3, 1)}
         del coords, buf
+    # ---- permutation index + feature scatter and the way back: 4 x 120,000 points, 256 bf16 channels ----
+    n_c, b, C = 120000, 4, 256
+    gg = torch.Generator().manual_seed(1004)
+    coords = (torch.rand(n_c * b, 3, generator=gg) * 51.2).to(torch.float16).to(dev)
+    seps = (torch.arange(1, b + 1, dtype=torch.int32) * n_c).to(dev).view(torch.uint32)
+    pad_to = -(-n_c * b // 3072) * 3072
+    _, buf = psh_main.batch_bucket_scatter(coords, seps, 512, pad_to, 2)
+    feat = torch.randn(n_c * b, C, generator=gg).to(torch.bfloat16).to(dev)
+    index = torch.empty(pad_to, dtype=torch.uint32, device=dev)
+    sfeat = torch.empty(pad_to, C, dtype=torch.bfloat16, device=dev)
+    back = torch.empty_like(feat)
+    ms_s = ev_time(lambda: pshattn.psh_scatter_feat_index(buf.bucket_id, buf.bucket_cntr, buf.bucket_offs, seps,
+                                                          buf.bucket_cumsum, index, feat, sfeat), 30)
+    ms_r = ev_time(lambda: pshattn.permute_rows(index, sfeat, back, False), 30)
+    s_bytes = n_c * b * (2 + 4 + C * 2) + pad_to * (4 + C * 2)
+    r_bytes = pad_to * 4 + 2 * n_c * b * C * 2
+    gbs = lambda b_, ms_: round(b_ / ms_ / 1e6, 1)
+    out["psh_feat_scatter_4x120k_c256"] = {"ms": round(ms_s, 4), "gbs": gbs(s_bytes, ms_s),
+                                           "frac_of_hbm_peak": round(gbs(s_bytes, ms_s) / HBM_PEAK_GBS, 4)}
+    out["psh_restore_order_4x120k_c256"] = {"ms": round(ms_r, 4), "gbs": gbs(r_bytes, ms_r),
+                                            "frac_of_hbm_peak": round(gbs(r_bytes, ms_r) / HBM_PEAK_GBS, 4)}
+    del coords, buf, feat, index, sfeat, back
     # ---- pooling / unpooling, config 3: 262,144 points x 128 channels, S = 8 ----
     n, C, S = 262144, 128, 8
     gg = torch.Generator().manual_seed(1003)

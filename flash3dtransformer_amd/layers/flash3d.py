@@ -7,6 +7,7 @@ import torch.cuda.nvtx as nvtx
 from torch import nn
 
 from ..psh import dev_context as f3ddev
+from ..psh import psh_main as pm
 from . import hourglass as f3dhourglass
 from . import psh_ops
 from . import stage as f3dstage
@@ -43,15 +44,18 @@ class Flash3D(nn.Module):
     forward(coords [N,3] fp16, input_feat, seps [B] uint32) -> [pad_to, C_out] bf16, rows in PSH
     (scattered) order, pad_to = N rounded up to buck_size * scope_size * 6.
 
-    As in the reference, `input_feat` is accepted and not used: the first-level features are the
-    embedded scattered coordinates.  Unlike the reference, which hands the UNSCATTERED coordinates
-    to the tree next to scattered features (flash3d.py:162-163), the tree receives the scattered
-    coordinates, with the pad rows counted into the last cloud, so that pooling groups the rows it
-    actually pools."""
+    By default, as in the reference, `input_feat` is accepted and not used: the first-level features are
+    the embedded scattered coordinates.  With `in_feat_dim` set, `input_feat` [N, in_feat_dim] is moved to
+    PSH order by the scatter's permutation index, projected by `input_proj` (a parameter the reference does
+    not have) and added to the coordinate embedding.  Unlike the reference, which hands the UNSCATTERED
+    coordinates to the tree next to scattered features (flash3d.py:162-163), the tree receives the
+    scattered coordinates, with the pad rows counted into the last cloud, so that pooling groups the rows
+    it actually pools.  `to_input_order(out)` brings per-point rows of the last forward back to the order
+    the points came in."""
     NVTX_SCOPE = "Flash3D"
 
     def __init__(self, level_specs: List[F3DLevelSpecs], buck_size: int, scope_size: int, top_level_hash,
-                 subbuck_size: int = 2):
+                 subbuck_size: int = 2, in_feat_dim: int = None):
         super().__init__()
         f3ddev.set_sync_stream(False)
         emb_chann = level_specs[0].encoder_specs[0].channels
@@ -62,6 +66,15 @@ class Flash3D(nn.Module):
         self.scope_size = scope_size
         self.subbuck_size = subbuck_size
         self.module_tree = self.build_module(0)
+        self.in_feat_dim = in_feat_dim
+        self._in_feat_pad = 0
+        if in_feat_dim is not None:
+            # the matrix-core linear takes inner widths in multiples of 8: narrower point features are zero-padded
+            self._in_feat_pad = -in_feat_dim % 8
+            self.input_proj = Linear(in_feat_dim + self._in_feat_pad, emb_chann)
+        self._last_index = None
+        self._last_n = 0
+        self._last_seps = None
 
     def build_module(self, level: int) -> nn.Module:
         if level >= len(self.level_specs):
@@ -94,6 +107,20 @@ class Flash3D(nn.Module):
             nvtx.range_push(self.NVTX_SCOPE)
         psh_feat = self.psh_scatter(coords, seps, self.first_hashtype)
         scattered = self.psh_scatter.last_scattered_coord
+        self._last_index, self._last_n, self._last_seps = None, coords.shape[0], seps
+        if self.in_feat_dim is not None:
+            if input_feat is None or input_feat.shape != (coords.shape[0], self.in_feat_dim):
+                raise RuntimeError(f"input_feat must be [{coords.shape[0]}, {self.in_feat_dim}]")
+            feat = input_feat.to(torch.bfloat16)
+            if self._in_feat_pad:
+                feat = torch.nn.functional.pad(feat, (0, self._in_feat_pad))
+            if feat.requires_grad:
+                index, _ = pm.batch_scatter_index(self.psh_scatter.last_buffers, seps)
+                feat = psh_ops.to_psh_order(feat, index)
+            else:
+                index, feat = pm.batch_scatter_index(self.psh_scatter.last_buffers, seps, feat)
+            self._last_index = index
+            psh_feat = psh_feat + self.input_proj(feat)
         tree_seps = seps
         if scattered.shape[0] != coords.shape[0]:
             tree_seps = seps.clone()
@@ -102,3 +129,12 @@ class Flash3D(nn.Module):
         if f3ddev.get_nvtx():
             nvtx.range_pop()
         return out
+
+    def to_input_order(self, out: torch.Tensor) -> torch.Tensor:
+        """Rows of a per-point tensor of the last forward ([pad_to, ...], PSH order) in the order the points
+        came in ([N, ...]); differentiable."""
+        if self._last_index is None:
+            if self._last_seps is None:
+                raise RuntimeError("to_input_order needs a forward call first")
+            self._last_index, _ = pm.batch_scatter_index(self.psh_scatter.last_buffers, self._last_seps)
+        return psh_ops.to_input_order(out, self._last_index, self._last_n)

@@ -10,6 +10,38 @@ from ..psh import psh_main as pm
 from .nn_ops import Linear, torch_backward
 
 
+class _PermuteRows(torch.autograd.Function):
+    """Row permutation by a PSH out-to-in index; the gradient of one direction is the other direction."""
+
+    @staticmethod
+    def forward(ctx, x, index, n_out: int, gather: bool):
+        out = torch.empty((n_out,) + tuple(x.shape[1:]), dtype=x.dtype, device=x.device)
+        if not gather:
+            out.zero_()      # rows that the index does not name
+        pshattn.permute_rows(index, x.contiguous(), out, gather)
+        ctx.index, ctx.n_in, ctx.gather = index, x.shape[0], gather
+        return out
+
+    @staticmethod
+    def backward(ctx, grad):
+        g = torch.empty((ctx.n_in,) + tuple(grad.shape[1:]), dtype=grad.dtype, device=grad.device)
+        if ctx.gather:
+            g.zero_()
+        pshattn.permute_rows(ctx.index, grad.contiguous(), g, not ctx.gather)
+        return g, None, None, None
+
+
+def to_psh_order(x: torch.Tensor, index: torch.Tensor) -> torch.Tensor:
+    """x [N, ...] in input order -> [pad_to, ...] in PSH (scattered) order, pad rows zero; index: the out-to-in
+    index of psh_main.batch_scatter_index"""
+    return _PermuteRows.apply(x, index, index.shape[0], True)
+
+
+def to_input_order(y: torch.Tensor, index: torch.Tensor, n: int) -> torch.Tensor:
+    """y [pad_to, ...] in PSH order -> [n, ...] in the order the points came in (pad rows dropped)"""
+    return _PermuteRows.apply(y, index, n, False)
+
+
 class PSHScatterLayer(nn.Module):
     def __init__(self, bucket_size: int = 512) -> None:
         super().__init__()
@@ -32,11 +64,13 @@ class PSH3DCoordEmbedding(nn.Module):
         self.feat_dtype = feat_dtype
         self.lin = Linear(3, emb_dim)
         self.last_scattered_coord = None
+        self.last_buffers = None
 
     def forward(self, coords, seps, hash_op):
         pad_to = f3darith.cdiv(coords.shape[0], self.alignment) * self.alignment
-        scattered, _ = pm.batch_bucket_scatter(coords, seps, self.bucket_size, pad_to, hash_op)
+        scattered, buffers = pm.batch_bucket_scatter(coords, seps, self.bucket_size, pad_to, hash_op)
         self.last_scattered_coord = scattered
+        self.last_buffers = buffers
         emb = torch.empty(pad_to, self.lin.out_features, dtype=torch.bfloat16, device=coords.device)
         lin = self.lin
         pshattn.coord_embed_bf16(scattered, lin._w.get(lin.weight), lin._b.get(lin.bias), emb)

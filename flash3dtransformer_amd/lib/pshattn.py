@@ -156,6 +156,66 @@ def batch_psh_scatter(coord, bucket_id, bucket_counter, bucket_offset, batch_sep
                                probe_offsets, cumsum_counter, scatter_coord, 0.0, 3)
 
 
+def _row_bytes(t) -> int:
+    n = t.element_size()
+    for d in t.shape[1:]:
+        n *= d
+    return n
+
+
+def psh_scatter_feat_index(bucket_id, bucket_counter, bucket_offset, batch_sep, cumsum_counter, scatter_idx_out2in,
+                           feat=None, scattered_feat=None):
+    """Completes src/psh/batch_psh_bucket.cuh:617-753: after a batch_psh_scatter* call on the same buffers,
+    scatter_idx_out2in[dst] = src (pad rows: N + 3) and, with `feat`, scattered_feat[dst] = feat[src] (pad rows
+    zero).  feat [N, ...] and scattered_feat [pad_to, ...] of one dtype and trailing shape."""
+    ts = [bucket_id, bucket_counter, bucket_offset, batch_sep, cumsum_counter, scatter_idx_out2in]
+    if (feat is None) != (scattered_feat is None):
+        raise RuntimeError("feat and scattered_feat come together")
+    if feat is not None:
+        ts += [feat, scattered_feat]
+        if feat.dtype != scattered_feat.dtype or feat.shape[1:] != scattered_feat.shape[1:]:
+            raise RuntimeError(f"feat {tuple(feat.shape)} {feat.dtype} and scattered_feat "
+                               f"{tuple(scattered_feat.shape)} {scattered_feat.dtype} differ in row shape or dtype")
+        if feat.shape[0] != bucket_id.shape[0] or scattered_feat.shape[0] != scatter_idx_out2in.shape[0]:
+            raise RuntimeError("feat needs one row per point and scattered_feat one per index entry")
+    assert_contiguous(ts)
+    dev = assert_same_device(ts)
+    assert_dtype([bucket_counter, bucket_offset, batch_sep, cumsum_counter, scatter_idx_out2in], torch.uint32)
+    assert_dtype([bucket_id], torch.uint16)
+    if bucket_counter.shape != cumsum_counter.shape or bucket_counter.shape[0] != batch_sep.shape[0]:
+        raise RuntimeError("bucket_counter and cumsum_counter must both be [batch, num_bucket]")
+    row_bytes = 0 if feat is None else _row_bytes(feat)
+    _check(_load().f3d_psh_scatter_feat_index(
+        _ptr(bucket_id), _ptr(bucket_offset), _ptr(bucket_counter), _ptr(cumsum_counter), _ptr(batch_sep),
+        _u32(batch_sep.shape[0]), _u32(bucket_id.shape[0]), _u32(bucket_counter.shape[1]),
+        _ptr(feat), _u32(row_bytes), _ptr(scatter_idx_out2in), _ptr(scattered_feat),
+        _u32(scatter_idx_out2in.shape[0]), _i32(dev), _stream(dev)))
+
+
+def permute_rows(index, src, dst, gather: bool):
+    """Row permutation by a PSH index.  gather: dst[r] = src[index[r]] (zero where index[r] >= len(src)), dst has
+    len(index) rows.  not gather: dst[index[r]] = src[r] where index[r] < len(dst), src has len(index) rows."""
+    ts = [index, src, dst]
+    assert_contiguous(ts)
+    dev = assert_same_device(ts)
+    assert_dtype([index], torch.uint32)
+    if src.dtype != dst.dtype or src.shape[1:] != dst.shape[1:]:
+        raise RuntimeError(f"src {tuple(src.shape)} {src.dtype} and dst {tuple(dst.shape)} {dst.dtype} differ in row "
+                           f"shape or dtype")
+    n_index, n_other = ((dst.shape[0], src.shape[0]) if gather else (src.shape[0], dst.shape[0]))
+    if index.shape[0] != n_index:
+        raise RuntimeError(f"index has {index.shape[0]} entries, the indexed side {n_index} rows")
+    if n_index == 0:
+        return
+    if n_other == 0:
+        if gather:
+            dst.zero_()
+        return
+    _check(_load().f3d_permute_rows(_ptr(index), _ptr(src), _ptr(dst), _u32(n_index), _u32(n_other),
+                                    _u32(_row_bytes(src)), _u32(1 if gather else 0), _i32(dev),
+                                    _stream(dev)))
+
+
 def coord_bbox(coord, bbox_min, bbox_max):
     """extension: one-pass whole-batch bounding box (replaces torch.min/max of psh_main.py:117-118)"""
     assert_contiguous([coord, bbox_min, bbox_max])

@@ -2,7 +2,7 @@
 (reference: flash3dxfmr/psh/psh_main.py:21-125)."""
 import math
 from dataclasses import dataclass
-from typing import Tuple
+from typing import Tuple, Optional
 
 import torch
 
@@ -35,6 +35,7 @@ class BucketScatterBuffers:
     bucket_cumsum: torch.Tensor
     probe_offs: torch.Tensor
     scattered_coord: torch.Tensor
+    scatter_index: Optional[torch.Tensor] = None   # filled by batch_scatter_index
 
     @staticmethod
     def create_buffers(coords: torch.Tensor, seps: torch.Tensor, bucket_size: int, pad_to: int, num_buck: int = None,
@@ -83,3 +84,23 @@ def batch_bucket_scatter(coords: torch.Tensor, seps: torch.Tensor, bucket_size: 
         bucket_size, NUM_VOX, bbox[0], bbox[1], buffers.probe_offs, buffers.bucket_cumsum,
         buffers.scattered_coord, 0.0, hash_op)
     return buffers.scattered_coord, buffers
+
+
+def batch_scatter_index(buffers: BucketScatterBuffers, seps: torch.Tensor,
+                        feat: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
+    """Out-to-in permutation index of a finished batch_bucket_scatter, uint32 [pad_to]: row r of the scattered
+    layout holds input row index[r]; the pad rows hold N + 3 (batch_psh_bucket.cuh:678, :735).  With `feat`
+    [N, ...] also returns the features in scattered order with zero pad rows, moved in the same pass (the step
+    batch_psh_cumsum_scatter_feat_index_postpad_ker, batch_psh_bucket.cuh:617-753, announces and never reaches).
+    The index is kept in `buffers.scatter_index`."""
+    pad_to = buffers.scattered_coord.shape[0]
+    dev = buffers.scattered_coord.device
+    index = torch.empty(pad_to, dtype=torch.uint32, device=dev)
+    out = None
+    if feat is not None:
+        feat = feat.contiguous()
+        out = torch.empty((pad_to,) + tuple(feat.shape[1:]), dtype=feat.dtype, device=dev)
+    pshattn.psh_scatter_feat_index(buffers.bucket_id, buffers.bucket_cntr, buffers.bucket_offs, seps,
+                                   buffers.bucket_cumsum, index, feat, out)
+    buffers.scatter_index = index
+    return index, out

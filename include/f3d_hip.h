@@ -128,6 +128,29 @@ int f3d_additive_unpool_fwd(const f3d_bf16_t* res_feat, const f3d_bf16_t* down_f
                             const uint32_t* unpool_ind, uint32_t up_n, uint32_t down_n, uint32_t feat_dim,
                             uint32_t subbuck_size, int device, void* stream);
 
+/* ---- PSH permutation index and feature scatter: completes batch_psh_cumsum_scatter_feat_index_postpad_ker,
+ *      src/psh/batch_psh_bucket.cuh:617-753 (unfinished in the reference: it writes the index, :735, and the pad
+ *      value total_N + 3, :678, and moves no feature) ------------------------------------------------------------
+ * Runs after f3d_batch_psh_scatter_pad_hash on that call's bucket_id / bucket_offset / bucket_counter /
+ * cumsum_counter / batch_sep.  scatter_idx_out2in[dst] = src for every input row, = total_n + 3 for the pad rows
+ * [total_n, pad_to_n); with feat != NULL also scattered_feat[dst] = feat[src] (rows of row_bytes bytes, any even
+ * size) and zero pad rows.  scatter_idx_out2in [pad_to_n]; feat [total_n] rows; scattered_feat [pad_to_n] rows. */
+int f3d_psh_scatter_feat_index(const uint16_t* bucket_id, const uint32_t* bucket_offset,
+                               const uint32_t* bucket_counter, const uint32_t* cumsum_counter,
+                               const uint32_t* batch_sep, uint32_t batch_size, uint32_t total_n, uint32_t num_bucket,
+                               const void* feat, uint32_t row_bytes, uint32_t* scatter_idx_out2in,
+                               void* scattered_feat, uint32_t pad_to_n, int device, void* stream);
+
+/* Row permutation by such an index (no counterpart in the reference, which never reaches this step; it is what
+ * src/psh/batch_psh_bucket.cuh:617-753 prepares the index for).
+ * gather != 0: out[r] = index[r] < n_other ? in[index[r]] : 0   for r < n_index  (in: n_other rows, out: n_index rows)
+ * gather == 0: out[index[r]] = in[r] where index[r] < n_other   for r < n_index  (in: n_index rows, out: n_other rows;
+ *              rows of out that no index names keep the caller's content).
+ * With the out-to-in index, gather moves input-order rows to PSH order and the other direction restores the input
+ * order; each is the other's gradient. */
+int f3d_permute_rows(const uint32_t* index, const void* in, void* out, uint32_t n_index, uint32_t n_other,
+                     uint32_t row_bytes, uint32_t gather, int device, void* stream);
+
 /* ---- additive unpool backward: additive_unpool_bwd, src/f3d_frontend.cu:103-105, kernel
  *      src/psh/additive_unpool.cuh:90-137, dispatcher src/psh/additive_unpool_dispatcher.cu:81-134 ----
  * grad_res[r,:] = grad_up_added[r,:] for every r = unpool_ind[i,s] < up_n (rows no slot refers to keep the

@@ -9,6 +9,8 @@
  * Pins (what keeps the oracle itself honest, see tests/test_oracle_*.py):
  *   vox/hash      : closed forms + known answers + bit-loop Morton brute force
  *   claim/scatter : scoreboard invariant + cumsum identity + multiset equality
+ *   index/features: index is a bijection per cloud; gathering the input coordinates by it gives
+ *                   the scattered coordinates of the scatter step, bit for bit
  *   reduce/unpool : numpy library routines on the same inputs
  *   sub-buckets   : structural invariants of tests/test_subbuck_reduce.py:486-631
  *
@@ -278,6 +280,39 @@ int f3d_or_cumsum_scatter_pad(const uint16_t *coord_h, uint32_t total_n, const u
   uint16_t pad_h = f3d_or_float_to_half(pad_num);
   for (size_t r = total_n; r < pad_to; ++r)
     for (int d = 0; d < 3; ++d) scattered_h[3 * r + d] = pad_h;
+  return 0;
+}
+
+/* ------------------------------------------------------------------------------------------ */
+/* Permutation index + feature scatter — src/psh/batch_psh_bucket.cuh:617-753 (the reference      */
+/* writes scatter_idx_out2in[dst] = src, :725-736, and total_N + 3 into the pad rows, :670-679;    */
+/* the feature move it announces is the same assignment on rows of row_bytes bytes).               */
+/* cumsum_counter is the inclusive prefix that f3d_or_cumsum_scatter_pad leaves behind.            */
+/* ------------------------------------------------------------------------------------------ */
+
+int f3d_or_scatter_feat_index(uint32_t total_n, const uint32_t *batch_sep, uint32_t batch_size,
+                              uint32_t num_bucket, const uint16_t *bucket_id, const uint32_t *bucket_offset,
+                              const uint32_t *cumsum_counter, const uint8_t *feat, uint32_t row_bytes,
+                              uint32_t *idx_out2in, uint8_t *scattered_feat, uint32_t pad_to) {
+  if (pad_to < total_n) return -1;
+  uint32_t start = 0;
+  for (uint32_t b = 0; b < batch_size; ++b) {
+    uint32_t end = batch_sep[b];
+    const uint32_t *cs = cumsum_counter + (size_t)b * num_bucket;
+    for (uint32_t i = start; i < end; ++i) {
+      uint32_t id = bucket_id[i];
+      uint32_t base = id ? cs[id - 1] : 0u;
+      size_t dst = (size_t)start + base + bucket_offset[i];
+      if (dst >= total_n) return -2;
+      idx_out2in[dst] = i;
+      if (feat) memcpy(scattered_feat + dst * row_bytes, feat + (size_t)i * row_bytes, row_bytes);
+    }
+    start = end;
+  }
+  for (size_t r = total_n; r < pad_to; ++r) {
+    idx_out2in[r] = total_n + 3u;
+    if (feat) memset(scattered_feat + r * row_bytes, 0, row_bytes);
+  }
   return 0;
 }
 

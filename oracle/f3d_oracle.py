@@ -196,6 +196,30 @@ def cumsum_scatter_pad(coord_h, seps, num_bucket, bucket_id, counter, offset, pa
     return cumsum, scattered.view(np.float16)
 
 
+def scatter_feat_index(seps, num_bucket, bucket_id, offset, cumsum, pad_to, feat=None):
+    """out-to-in permutation index of the PSH scatter (pad rows: N + 3) and, with `feat` [N, ...], the features in
+    PSH order with zero pad rows (src/psh/batch_psh_bucket.cuh:617-753)"""
+    seps = np.ascontiguousarray(seps, dtype=np.uint32)
+    bid = np.ascontiguousarray(bucket_id, dtype=np.uint16)
+    n, b = bid.shape[0], seps.shape[0]
+    idx = np.full(pad_to, 0xFFFFFFFF, dtype=np.uint32)
+    f = out = None
+    row_bytes = 0
+    if feat is not None:
+        f = np.ascontiguousarray(feat)
+        row_bytes = f.dtype.itemsize * int(np.prod(f.shape[1:], dtype=np.int64))
+        out = np.full((pad_to,) + f.shape[1:], 0, dtype=f.dtype)
+        out.view(np.uint8)[...] = 0xA5
+    rc = lib().f3d_or_scatter_feat_index(
+        ctypes.c_uint32(n), _p(seps), ctypes.c_uint32(b), ctypes.c_uint32(num_bucket), _p(bid),
+        _p(np.ascontiguousarray(offset, dtype=np.uint32)), _p(np.ascontiguousarray(cumsum, dtype=np.uint32)),
+        _p(f) if f is not None else None, ctypes.c_uint32(row_bytes), _p(idx),
+        _p(out) if out is not None else None, ctypes.c_uint32(pad_to))
+    if rc != 0:
+        raise RuntimeError(f"oracle scatter_feat_index failed rc={rc}")
+    return (idx, out) if feat is not None else idx
+
+
 def scoreboard(bucket_id, counter, offset, seps):
     """0 when every (cloud, bucket, slot < count) is claimed exactly once (bucket_sanitizer_cpu.cpp:92-176)"""
     seps = np.ascontiguousarray(seps, dtype=np.uint32)

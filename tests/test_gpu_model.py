@@ -232,6 +232,43 @@ def test_two_level_model_backward_reaches_every_parameter():
     assert losses[-1] < losses[0], losses
 
 
+def test_model_consumes_point_features_and_restores_input_order():
+    """Flash3D(in_feat_dim=4): the per-point features (KITTI-style x, y, z, intensity rows) reach the first level
+    through the PSH permutation, `input_proj` trains, and `to_input_order` returns rows in the order the points
+    came in: permuting the input points permutes that output the same way (bucket slots follow input order, so the
+    comparison is through the point's coordinates: same multiset of (coord, output) rows per cloud)."""
+    from flash3dtransformer_amd import layers as L, synth
+    from flash3dtransformer_amd.psh.bucket_scope import SwinPlan
+    bs, scope = 256, 1
+    torch.manual_seed(2)
+    ln = lambda ch: L.LayerNorm(ch)
+    spec = lambda c, h: L.XFMRSpecs(c, 2 * c, h, True, SwinPlan("swin", bs, scope, 0), ln)
+    levels = [L.F3DLevelSpecs([spec(32, 1)], [spec(32, 1)], "mean", 256, None, None, None, None)]
+    model = L.Flash3D(levels, bs, scope, 2, in_feat_dim=4).to(DEV)
+    assert "input_proj.weight" in model.state_dict()
+    rng = np.random.default_rng(8)
+    coords, seps = synth.batch_of([rng.normal(0, 10, (n, 3)).astype(np.float32) for n in (9000, 8200)])
+    n = coords.shape[0]
+    c = torch.from_numpy(coords).to(DEV)
+    s = torch.from_numpy(seps.view(np.int32)).to(DEV).view(torch.uint32)
+    feat = torch.randn(n, 4, device=DEV)
+    out = model(c, feat, s)
+    per_point = model.to_input_order(out)
+    assert per_point.shape == (n, out.shape[1]) and torch.isfinite(per_point.float()).all()
+    # rows of the scattered output and rows in input order are the same rows, related by the index
+    idx = model._last_index.view(torch.int32)[:n].long()
+    assert torch.equal(out[:n], per_point[idx])
+    # the features matter, and their projection receives a gradient
+    out0 = model(c, torch.zeros_like(feat), s)
+    assert (out0.float() - out.float()).abs().max().item() > 1e-3
+    feat_g = feat.clone().requires_grad_(True)
+    model.to_input_order(model(c, feat_g, s)).float().square().mean().backward()
+    assert model.input_proj.weight.grad.abs().max().item() > 0
+    assert feat_g.grad is not None and feat_g.grad.abs().max().item() > 0
+    with pytest.raises(RuntimeError, match="input_feat must be"):
+        model(c, feat[:, :3], s)
+
+
 def test_state_dict_names_match_reference_module_tree():
     """parameter names a reference checkpoint would carry (flash3dxfmr/layers/*.py module attributes;
     TransformerEngine's LayerNormMLP / Linear parameter names)"""

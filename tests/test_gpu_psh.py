@@ -34,7 +34,7 @@ def _run_psh(coords, seps, bucket_size, hash_op, pad_align, oracle, rebalance=0)
     torch.cuda.synchronize()
     return dict(nb=nb, div=div, pad_to=pad_to, ids=n_u16(bucket_id), cnt=n_u32(cntr), off=n_u32(offs),
                 cumsum=n_u32(cumsum), scat=n_f16(scat), bmin=n_f16(bmin), bmax=n_f16(bmax),
-                t=(bucket_id, cntr, offs, s))
+                t=(bucket_id, cntr, offs, s), t_cumsum=cumsum)
 
 
 def _check_against_oracle(coords, seps, out, hash_op, oracle, rebalance=0, bucket_size=512):
@@ -200,3 +200,95 @@ def test_rebalance_bit_exact_and_reference_invariants(oracle, case):
         maxcnt = torch.from_numpy(out["cnt"].max(1).astype(np.int32)).to(DEV).view(torch.uint32)
         pshattn.batch_bucket_sanitizer_cpu(bucket_id, cntr, offs, table, res, s, maxcnt, b, out["nb"])
     pshattn.DeviceManagerSingleton.instance().set_psh_rebalance(1)
+
+
+@pytest.mark.parametrize("sizes,bucket_size,rebalance,feat_shape,feat_dtype", [
+    ([20000, 17001, 23456], 512, 1, (64,), torch.bfloat16),     # 128-byte rows: 8 lanes x 16 B
+    ([9000, 0, 8000], 256, 0, (1,), torch.bfloat16),            # 2-byte rows, an empty cloud
+    ([70000, 300, 65000, 1], 512, 1, (4,), torch.float32),      # KITTI-style [n, 4] float rows
+    ([33000, 31000], 512, 1, (3, 5), torch.float16),            # 30-byte rows: 2-byte units, 16 lanes
+    ([300000, 280000], 512, 1, (256,), torch.bfloat16),         # 512-byte rows at the large-tile configuration
+])
+def test_scatter_index_and_features_bit_exact(oracle, sizes, bucket_size, rebalance, feat_shape, feat_dtype):
+    """Permutation index + feature scatter (batch_psh_bucket.cuh:617-753) against the oracle, bit for bit; the
+    index must also reproduce the coordinate scatter of the bucketing call itself, and permute_rows must move rows
+    both ways."""
+    from flash3dtransformer_amd.lib import pshattn
+    rng = np.random.default_rng(sum(sizes) + 1)
+    pts = np.concatenate([rng.normal(0, 20, (n, 3)) + rng.uniform(-5, 5, 3) for n in sizes]).astype(np.float16)
+    seps = np.cumsum(sizes).astype(np.uint32)
+    n = pts.shape[0]
+    out = _run_psh(pts, seps, bucket_size, 2, bucket_size * 6, oracle, rebalance=rebalance)
+    bucket_id, cntr, offs, s = out["t"]
+    pad_to = out["pad_to"]
+    g = torch.Generator().manual_seed(7)
+    feat = torch.randn((n,) + feat_shape, generator=g).to(feat_dtype).to(DEV)
+    index = torch.full((pad_to,), 0xFFFFFFF, dtype=torch.int32, device=DEV).view(torch.uint32)
+    sfeat = torch.full((pad_to,) + feat_shape, 7.0, dtype=feat_dtype, device=DEV)
+    pshattn.psh_scatter_feat_index(bucket_id, cntr, offs, s, out["t_cumsum"], index, feat, sfeat)
+    index_only = torch.empty_like(index)
+    pshattn.psh_scatter_feat_index(bucket_id, cntr, offs, s, out["t_cumsum"], index_only)
+    torch.cuda.synchronize()
+    bits = {2: torch.int16, 4: torch.int32}[feat.element_size()]
+    feat_np = feat.cpu().view(bits).numpy()
+    ref_idx, ref_feat = oracle.scatter_feat_index(seps, out["nb"], out["ids"], out["off"], out["cumsum"], pad_to, feat_np)
+    idx = n_u32(index)
+    assert np.array_equal(idx, ref_idx) and np.array_equal(n_u32(index_only), ref_idx)
+    assert np.array_equal(sfeat.cpu().view(bits).numpy(), ref_feat)
+    # independent of the oracle: the index reproduces the bucketing call's own coordinate scatter
+    assert np.array_equal(pts[idx[:n]].view(np.uint16), out["scat"][:n].view(np.uint16))
+    assert (idx[n:] == n + 3).all()
+    # permute_rows: gather by the index = the fused feature scatter; the other direction restores the input
+    gathered = torch.full_like(sfeat, 3.0)
+    pshattn.permute_rows(index, feat, gathered, True)
+    restored = torch.full_like(feat, 5.0)
+    pshattn.permute_rows(index, gathered, restored, False)
+    torch.cuda.synchronize()
+    assert torch.equal(gathered.view(bits), sfeat.view(bits))
+    assert torch.equal(restored.view(bits), feat.view(bits))
+
+
+def test_scatter_index_misaligned_rows_and_errors():
+    """Rows whose base address is only 2-byte aligned fall back to narrower units; bad arguments raise."""
+    from flash3dtransformer_amd.lib import pshattn
+    n, c = 1000, 24
+    g = torch.Generator().manual_seed(3)
+    perm = torch.randperm(n, generator=g).to(torch.int32)
+    index = torch.cat([perm, torch.full((24,), n + 3, dtype=torch.int32)]).to(DEV).view(torch.uint32)
+    base = torch.randn(n * c + 1, generator=g).to(torch.bfloat16).to(DEV)
+    src = base[1:].view(n, c)                       # 2-byte aligned rows
+    dst = torch.full((n + 24, c), 9.0, dtype=torch.bfloat16, device=DEV)
+    pshattn.permute_rows(index, src, dst, True)
+    torch.cuda.synchronize()
+    assert torch.equal(dst[:n], src[perm.to(DEV).long()]) and (dst[n:] == 0).all()
+    with pytest.raises(RuntimeError, match="row shape or dtype"):
+        pshattn.permute_rows(index, src, dst.float(), True)
+    with pytest.raises(RuntimeError, match="entries"):
+        pshattn.permute_rows(index[:10], src, dst, True)
+
+
+def test_layer_permutation_is_differentiable_and_model_takes_features():
+    """to_psh_order / to_input_order are each other's gradient; Flash3D with in_feat_dim consumes input_feat
+    and to_input_order returns per-point rows in the order the points came in."""
+    from flash3dtransformer_amd import synth
+    from flash3dtransformer_amd.layers import psh_ops
+    from flash3dtransformer_amd.psh import psh_main as pm
+    coords, seps = synth.batch_of([synth.uniform_cube(9000, 40.0, 5), synth.uniform_cube(8200, 40.0, 6)])
+    c, s = t_f16(coords), t_u32(seps)
+    n = coords.shape[0]
+    pad_to = -(-n // 1536) * 1536
+    scattered, buffers = pm.batch_bucket_scatter(c, s, 256, pad_to, 2)
+    index, _ = pm.batch_scatter_index(buffers, s)
+    x = torch.randn(n, 16, device=DEV).to(torch.bfloat16).requires_grad_(True)
+    y = psh_ops.to_psh_order(x, index)
+    w = torch.randn(pad_to, 16, device=DEV).to(torch.bfloat16)
+    (y.float() * w.float()).sum().backward()
+    idx = index.view(torch.int32)[:n].long()
+    assert torch.equal(y[:n], x.detach()[idx]) and (y[n:] == 0).all()
+    expect = torch.zeros(n, 16, dtype=torch.bfloat16, device=DEV)
+    expect[idx] = w[:n]
+    assert torch.equal(x.grad, expect)
+    back = psh_ops.to_input_order(y.detach(), index, n)
+    assert torch.equal(back, x.detach())
+    # coordinates gathered by the index are the scattered coordinates
+    assert torch.equal(psh_ops.to_psh_order(c, index)[:n], scattered[:n])

@@ -186,6 +186,37 @@ def test_scatter_cumsum_multiset_and_positions(oracle):
         start = int(end)
 
 
+@pytest.mark.parametrize("rebalance", [False, True])
+def test_scatter_index_is_the_scatter_permutation(oracle, rebalance):
+    """Pins the permutation index (batch_psh_bucket.cuh:617-753) by what fixes it without restating its formula:
+    it is a bijection on every cloud's row range, the input coordinates gathered by it are the scatter step's
+    output bit for bit, without rebalance it is the stable argsort by bucket id, and features ride along."""
+    rng = np.random.default_rng(11)
+    coords, seps = _cloud(rng, [9000, 0, 7777, 8300])
+    n = coords.shape[0]
+    nb, div, _ = oracle.psh_params(seps, 256)
+    mn, mx = coords.min(0), coords.max(0)
+    ids, cnt, off = oracle.psh_claim(coords, seps, mn, mx, 0xFFFF, div, nb, 2)
+    if rebalance:
+        ids, cnt, off = oracle.psh_rebalance(ids, cnt, off, seps, 256)
+    pad_to = -(-n // 1536) * 1536
+    cumsum, scat = oracle.cumsum_scatter_pad(coords, seps, nb, ids, cnt, off, pad_to, 0.0)
+    feat = rng.integers(0, 2 ** 16, (n, 5), dtype=np.uint16)
+    idx, sfeat = oracle.scatter_feat_index(seps, nb, ids, off, cumsum, pad_to, feat)
+    assert np.array_equal(idx, oracle.scatter_feat_index(seps, nb, ids, off, cumsum, pad_to))
+    assert (idx[n:] == n + 3).all() and (sfeat[n:] == 0).all()
+    start = 0
+    for end in seps:
+        end = int(end)
+        assert np.array_equal(np.sort(idx[start:end]), np.arange(start, end, dtype=np.uint32))
+        if not rebalance:
+            order = np.argsort(ids[start:end], kind="stable")
+            assert np.array_equal(idx[start:end], start + order)
+        start = end
+    assert np.array_equal(coords[idx[:n]].view(np.uint16), scat[:n].view(np.uint16))
+    assert np.array_equal(feat[idx[:n]], sfeat[:n])
+
+
 def test_helpers_closed_forms(oracle):
     for v in range(1, 3000):
         p = oracle.round_next_two_power(v)
