@@ -167,16 +167,30 @@ def main():
     fc1_n = 2 * HID if args.mlp == "swiglu" else HID
     flops = {"ln_qkv": 2.0 * n_pad * C * 3 * C, "proj_residual": 2.0 * n_pad * C * C,
              "ln_fc1_act": 2.0 * n_pad * C * fc1_n, "fc2_residual": 2.0 * n_pad * HID * C,
+             "ln_mlp_residual": 2.0 * n_pad * C * fc1_n + 2.0 * n_pad * HID * C,
              "attention": 4.0 * n_pad * BS * SCOPE * C}
     # algorithmic HBM bytes per launch (bf16 activations in and out, weights negligible)
     hbm_bytes = {"ln_qkv": 2.0 * n_pad * (C + 3 * C), "proj_residual": 2.0 * n_pad * 3 * C,
                  "ln_fc1_act": 2.0 * n_pad * (C + HID), "fc2_residual": 2.0 * n_pad * (HID + 2 * C),
+                 "ln_mlp_residual": 2.0 * n_pad * 2 * C,      # x (also the residual) in, y out
                  "attention": 2.0 * n_pad * 4 * C + 4.0 * n_pad * H}
     kernels = {"attention": "buck_swin_fwd_resident_kernel<32,512>",
                "ln_qkv": "xstat_linear_kernel<256,2,8,3,LN> + ln_fold_kernel",
                "ln_fc1_act": "xstat_linear_kernel<256,2,8,3,LN,swiglu> + ln_fold_kernel",
                "proj_residual": "xstat_linear_kernel<256,2,8,3,residual>",
-               "fc2_residual": "gemm_bf16_kernel<false>"}
+               "fc2_residual": "gemm_bf16_kernel<false>",
+               "ln_mlp_residual": "ln_mlp_swiglu_kernel<256> + ln_fold_kernel + mlp_w2_prep_kernel"}
+    flops = {kname: vv for kname, vv in flops.items() if kname in breakdown}
+    # the one-kernel gated MLP (not part of the timed step: the layers use it on request only), same tensors
+    fused_mlp = None
+    if args.mlp == "swiglu":
+        with torch.no_grad():
+            ms_f = ev_time(lambda: pshattn.ln_mlp_swiglu_bf16(mid, Wm, Bm, 1e-5, W1, B1, W2, B2, mid, y), 20)
+        fl_f = 2.0 * n_pad * C * fc1_n + 2.0 * n_pad * HID * C
+        fused_mlp = {"kernel": "ln_mlp_swiglu_kernel<256> + ln_fold_kernel + mlp_w2_prep_kernel", "ms": round(ms_f, 4),
+                     "tflops": round(fl_f / ms_f / 1e9, 1), "frac_of_bf16_mfma_peak": round(fl_f / ms_f / 1e9 / MFMA_BF16_PEAK_TFLOPS, 4),
+                     "two_kernel_ms": round(breakdown["ln_fc1_act"] + breakdown["fc2_residual"], 4),
+                     "hidden_activation_bytes_not_allocated": int(n_pad) * HID * 2}
     dominant = max(flops, key=lambda kname: breakdown[kname])
     t_dom = breakdown[dominant] * 1e-3
     ach = flops[dominant] / t_dom / 1e12
@@ -211,6 +225,7 @@ def main():
         "roofline": roofline,
         "breakdown_ms": {kname: round(vv, 4) for kname, vv in breakdown.items()},
         "per_op": per_op,
+        "fused_mlp_on_request": fused_mlp,
         "sub_metrics": sub,
     }
     if not args.no_cpu_baseline:

@@ -490,6 +490,35 @@ def ln_linear_bf16(x, gamma, beta, eps, w, bias, residual, y, act=None):
                                       _u32(n), _u32(k), _u32(a), _i32(dev), _stream(dev)))
 
 
+def ln_mlp_swiglu_bf16(x, gamma, beta, eps, w1, b1, w2, b2, residual, y) -> bool:
+    """extension: y = (silu(LN(x) w1[:h].T + b1[:h]) * (LN(x) w1[h:].T + b1[h:])) w2.T + b2 (+ residual) in one kernel
+    (te.LayerNormMLP with swiglu + the residual add, elem_wise.py:22-26, stage.py:94-97).  Returns False, leaving y
+    untouched, when no fused kernel covers the widths (the caller then runs ln_linear_bf16 + linear_bf16)."""
+    dev = assert_same_device([x, gamma, w1, w2, y])
+    assert_dtype([x, gamma, w1, w2, y], torch.bfloat16)
+    assert_contiguous([w1, w2, gamma])
+    if x.dim() != 2 or y.dim() != 2 or x.stride(1) != 1 or y.stride(1) != 1:
+        raise RuntimeError("ln_mlp_swiglu_bf16 expects 2-D row-major x and y")
+    m, c = x.shape
+    hidden = w2.shape[1]
+    if tuple(w1.shape) != (2 * hidden, c) or w2.shape[0] != c or tuple(y.shape) != (m, c) or gamma.shape[0] != c:
+        raise RuntimeError(f"ln_mlp shape mismatch: x{tuple(x.shape)} w1{tuple(w1.shape)} w2{tuple(w2.shape)} "
+                           f"y{tuple(y.shape)}")
+    ldr = 0
+    if residual is not None:
+        assert_dtype([residual], torch.bfloat16)
+        if tuple(residual.shape) != (m, c) or residual.stride(1) != 1:
+            raise RuntimeError("residual must be [m, c] row-major")
+        ldr = residual.stride(0)
+    rc = _load().f3d_ln_mlp_swiglu_bf16(_ptr(x), _u32(x.stride(0)), _ptr(gamma), _ptr(beta), _f32(eps), _ptr(w1),
+                                        _ptr(b1), _ptr(w2), _ptr(b2), _ptr(residual), _u32(ldr), _ptr(y),
+                                        _u32(y.stride(0)), _u32(m), _u32(c), _u32(hidden), _i32(dev), _stream(dev))
+    if rc == 2:
+        return False
+    _check(rc)
+    return True
+
+
 def layernorm_bf16(x, gamma, beta, y, eps=1e-5):
     """extension: LayerNorm over the last axis, fp32 statistics"""
     assert_contiguous([x, gamma, y])

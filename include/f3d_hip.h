@@ -228,6 +228,20 @@ int f3d_ln_linear_bf16(const f3d_bf16_t* x, uint32_t ldx, const f3d_bf16_t* gamm
                        f3d_bf16_t* y, uint32_t ldy, uint32_t m, uint32_t n, uint32_t k, uint32_t act, int device,
                        void* stream);
 
+/* The whole gated MLP of a block in one kernel:
+ *   y = (silu(LN(x) w1[:h]ᵀ + b1[:h]) * (LN(x) w1[h:]ᵀ + b1[h:])) w2ᵀ + b2 (+ residual),
+ * te.LayerNormMLP(activation = "swiglu") followed by the residual add (flash3dxfmr/layers/elem_wise.py:22-26,
+ * stage.py:94-97).  x [m,c] (row stride ldx), gamma [c], beta [c] or NULL, w1 [2 hidden, c] (value rows, then gate
+ * rows), b1 [2 hidden] or NULL, w2 [c, hidden], b2 [c] or NULL, residual [m,c] or NULL (row stride ldr), y [m,c] (row
+ * stride ldy), all bf16.  The hidden activations are rounded to bf16 as a separate fc1 kernel would store them and
+ * never leave the registers.  c in {128, 256}, hidden a multiple of 32; anything else returns F3D_ERR_UNSUPPORTED
+ * without touching y (use f3d_ln_linear_bf16 with F3D_ACT_SWIGLU followed by f3d_linear_bf16).  Uses the per-device
+ * workspace like f3d_ln_linear_bf16. */
+int f3d_ln_mlp_swiglu_bf16(const f3d_bf16_t* x, uint32_t ldx, const f3d_bf16_t* gamma, const f3d_bf16_t* beta, float eps,
+                           const f3d_bf16_t* w1, const f3d_bf16_t* b1, const f3d_bf16_t* w2, const f3d_bf16_t* b2,
+                           const f3d_bf16_t* residual, uint32_t ldr, f3d_bf16_t* y, uint32_t ldy, uint32_t m,
+                           uint32_t c, uint32_t hidden, int device, void* stream);
+
 /* LayerNorm over the last axis, fp32 statistics (norm callables of flash3dxfmr/layers/stage.py:67).
  * x,y [m,c] bf16; gamma,beta [c] bf16 (beta may be NULL). */
 int f3d_layernorm_bf16(const f3d_bf16_t* x, const f3d_bf16_t* gamma, const f3d_bf16_t* beta, f3d_bf16_t* y,

@@ -173,3 +173,73 @@ def test_dense_argument_errors():
         pshattn.layernorm_bf16(mk(4, 12), mk(12), mk(12), mk(4, 12))
     with pytest.raises(RuntimeError, match="gemm shape mismatch"):
         pshattn.gemm_sm_bf16(mk(8, 16), mk(8, 16), mk(8, 16))
+
+
+@pytest.mark.parametrize("M,C,H,use_res,use_bias", [
+    (4096, 256, 1024, True, True),      # the C = 256 block's MLP
+    (1000, 256, 512, False, True),      # ragged M, no residual
+    (777, 128, 512, True, False),       # C = 128, no biases
+    (300, 256, 32, True, True),         # a single hidden chunk
+    (70000, 128, 256, True, True),      # many workgroups
+])
+def test_fused_mlp_matches_two_kernel_path(oracle, M, C, H, use_res, use_bias):
+    """The one-kernel gated MLP against (a) the LayerNorm+fc1+swiglu kernel followed by the fc2+residual kernel, whose
+    roundings it reproduces (same folded weights, hidden activations rounded to bf16; only the fp32 summation order
+    of fc2 differs), and (b) the unrounded mathematics, next to the reference's own rounding sequence."""
+    from flash3dtransformer_amd.lib import pshattn
+    x = (_rand((M, C), 1, scale=2.0) + 0.3).to(DEV)
+    g, b = (_rand((C,), 3) + 1.0).to(DEV), _rand((C,), 4, scale=0.2).to(DEV)
+    w1, w2 = _rand((2 * H, C), 2, scale=1 / math.sqrt(C)).to(DEV), _rand((C, H), 5, scale=1 / math.sqrt(H)).to(DEV)
+    b1 = _rand((2 * H,), 6).to(DEV) if use_bias else None
+    b2 = _rand((C,), 7).to(DEV) if use_bias else None
+    res = _rand((M, C), 8).to(DEV) if use_res else None
+    y = torch.full((M, C), 9.0, dtype=torch.bfloat16, device=DEV)
+    assert pshattn.ln_mlp_swiglu_bf16(x, g, b, 1e-5, w1, b1, w2, b2, res, y)
+    hid = torch.empty(M, H, dtype=torch.bfloat16, device=DEV)
+    y2 = torch.empty_like(y)
+    pshattn.ln_linear_bf16(x, g, b, 1e-5, w1, b1, None, hid, "swiglu")
+    pshattn.linear_bf16(hid, w2, b2, res, y2, None)
+    torch.cuda.synchronize()
+    d = (y.float() - y2.float()).abs()
+    scale = y2.float().abs().clamp(min=1.0)
+    assert (d / scale).max().item() <= 2 ** -6, (d / scale).max().item()          # at most two bf16 steps apart
+    assert (d > 0).float().mean().item() < 0.02                                     # and almost always equal
+    # (b) against the unrounded mathematics: at least as close as the reference's own sequence of bf16 roundings
+    # (LayerNorm output, fc1 output, gated product, fc2 output, residual sum)
+    xc, gc, bc, w1c, w2c = x.cpu(), g.cpu(), b.cpu(), w1.cpu(), w2.cpu()
+    b1c, b2c = (None if b1 is None else b1.cpu()), (None if b2 is None else b2.cpu())
+    rb = lambda t: t.to(torch.bfloat16).float()
+    exact = oracle.linear(oracle.swiglu(oracle.linear(oracle.layernorm(xc, gc, bc, 1e-5), w1c, b1c)), w2c, b2c)
+    ref = rb(oracle.linear(rb(oracle.swiglu(rb(oracle.linear(rb(oracle.layernorm(xc, gc, bc, 1e-5)), w1c, b1c)))), w2c, b2c))
+    if res is not None:
+        exact = exact + res.float().cpu()
+        ref = rb(ref + res.float().cpu())
+    scale = exact.abs().clamp(min=1.0)
+    err_us, err_ref = (y.float().cpu() - exact).abs() / scale, (ref - exact).abs() / scale
+    assert err_us.max() <= 1.5 * err_ref.max() + 4e-3, (err_us.max(), err_ref.max())
+    assert err_us.mean() <= 1.25 * err_ref.mean() + 1e-4, (err_us.mean(), err_ref.mean())
+
+
+def test_fused_mlp_unsupported_width_is_reported():
+    from flash3dtransformer_amd.lib import pshattn
+    mk = lambda *s: torch.zeros(*s, dtype=torch.bfloat16, device=DEV)
+    y = torch.full((64, 64), 3.0, dtype=torch.bfloat16, device=DEV)
+    assert not pshattn.ln_mlp_swiglu_bf16(mk(64, 64), mk(64), mk(64), 1e-5, mk(256, 64), None, mk(64, 128), None, None, y)
+    assert (y == 3.0).all()
+
+
+def test_layernorm_mlp_layer_fused_on_request():
+    """LayerNormMLP(fused=True) routes through the one-kernel gated MLP and agrees with the default two-kernel
+    path; gradients flow through it like through the default."""
+    from flash3dtransformer_amd.layers.nn_ops import LayerNormMLP
+    torch.manual_seed(5)
+    a, b = LayerNormMLP(256, 512).to(DEV), LayerNormMLP(256, 512, fused=True).to(DEV)
+    b.load_state_dict(a.state_dict())
+    x = torch.randn(3000, 256, device=DEV).to(torch.bfloat16)
+    ya, yb = a(x, residual=x), b(x, residual=x)
+    d = (ya.float() - yb.float()).abs() / ya.float().abs().clamp(min=1.0)
+    assert d.max().item() <= 2 ** -6
+    xg = x.clone().requires_grad_(True)
+    b(xg, residual=xg).float().square().mean().backward()
+    assert xg.grad is not None and torch.isfinite(xg.grad.float()).all() and xg.grad.abs().max().item() > 0
+    assert b.fc2_weight.grad.abs().max().item() > 0
