@@ -22,10 +22,13 @@
 // The hidden activations (M x H bf16, 1 GB at 482 k rows x 1024) are never allocated.  Measured on MI355X at
 // 482,304 rows, C = 256, H = 1024 against the LayerNorm+fc1+gate kernel followed by the fc2+residual kernel:
 // 0.94 ms against 0.98 ms on the activations of a block with small random weights, 1.04 ms against 0.97 ms on
-// unit-variance random tensors.  With one wave per SIMD the matrix core is busy about a third of the time (a single
-// wave's products issue at about half the rate that two waves reach together; shortening the vector and LDS work
-// between them changed nothing), so this kernel is a memory saving, not yet a speed-up, and the layers use it on
-// request only.
+// unit-variance random tensors.  With one wave per SIMD the matrix core is busy about a third of the time.  A lone
+// wave does reach 2.06 PFLOP/s on back-to-back products with two independent accumulators, and four waves per CU read
+// LDS at 295 B/ns, so neither the product issue rate nor LDS bandwidth is the limit: the chunk loop has about 1000
+// instructions for its 101 products, and with a single wave per SIMD nothing but the matrix core's own latency
+// overlaps with their issue.  Two waves per SIMD need at most 256 registers per wave, which x (128) and the fc2
+// accumulators (256) do not allow at C = 256.  So this kernel is a memory saving, not yet a speed-up, and the layers
+// use it on request only.
 #include "xstat_common.h"
 
 namespace f3d {
