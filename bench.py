@@ -27,8 +27,8 @@ HBM_PEAK_GBS = 8000.0
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by a copy kernel of known
 # size, see profiles/encoder_stage_4x120k_hbm_traffic.md) at this bench's shapes
-TRAFFIC_BYTES_PER_LAUNCH = {"ln_fc1_act": 1.557e9, "ln_qkv": 1.027e9, "attention": 1.017e9,
-                            "proj_residual": 0.770e9, "fc2_residual": 1.513e9}
+TRAFFIC_BYTES_PER_LAUNCH = {"ln_fc1_act": 1.554e9, "ln_qkv": 1.027e9, "attention": 1.016e9,
+                            "proj_residual": 0.768e9, "fc2_residual": 1.513e9, "ln_mlp_residual": 0.807e9}
 
 
 def ev_time(fn, iters, warmup=3):
@@ -190,6 +190,7 @@ def main():
         fused_mlp = {"kernel": "ln_mlp_swiglu_kernel<256> + ln_fold_kernel + mlp_w2_prep_kernel", "ms": round(ms_f, 4),
                      "tflops": round(fl_f / ms_f / 1e9, 1), "frac_of_bf16_mfma_peak": round(fl_f / ms_f / 1e9 / MFMA_BF16_PEAK_TFLOPS, 4),
                      "two_kernel_ms": round(breakdown["ln_fc1_act"] + breakdown["fc2_residual"], 4),
+                     "traffic": TRAFFIC_BYTES_PER_LAUNCH["ln_mlp_residual"],
                      "hidden_activation_bytes_not_allocated": int(n_pad) * HID * 2}
     dominant = max(flops, key=lambda kname: breakdown[kname])
     t_dom = breakdown[dominant] * 1e-3
