@@ -178,7 +178,7 @@ def main():
                "ln_qkv": "xstat_linear_kernel<256,2,8,3,LN> + ln_fold_kernel",
                "ln_fc1_act": "xstat_linear_kernel<256,2,8,3,LN,swiglu> + ln_fold_kernel",
                "proj_residual": "xstat_linear_kernel<256,2,8,3,residual>",
-               "fc2_residual": "gemm_bf16_kernel<false>",
+               "fc2_residual": "ystat_linear_kernel<256> + ys_w_prep_kernel",
                "ln_mlp_residual": "ln_mlp_swiglu_kernel<256> + ln_fold_kernel + mlp_w2_prep_kernel"}
     flops = {kname: vv for kname, vv in flops.items() if kname in breakdown}
     # the one-kernel gated MLP (not part of the timed step: the layers use it on request only), same tensors

@@ -348,6 +348,10 @@ __global__ __launch_bounds__(256) void affine_act_kernel(const uint16_t* __restr
 int launch_xstat_linear(const uint16_t* x, uint32_t ldx, const uint16_t* gamma, const uint16_t* beta, float eps,
                         const uint16_t* w, const uint16_t* bias, const uint16_t* residual, uint32_t ldr, uint16_t* y,
                         uint32_t ldy, uint32_t M, uint32_t N, uint32_t K, uint32_t act, int device, hipStream_t s);
+// output-panel kernel for long inner dimensions and 128 / 256 outputs (ystat_linear.hip); F3D_ERR_UNSUPPORTED otherwise
+int launch_ystat_linear(const uint16_t* x, uint32_t ldx, const uint16_t* w, const uint16_t* bias,
+                        const uint16_t* residual, uint32_t ldr, uint16_t* y, uint32_t ldy, uint32_t M, uint32_t N,
+                        uint32_t K, uint32_t act, int device, hipStream_t s);
 
 static int launch_gemm(bool b_trans, const uint16_t* x, uint32_t ldx, const uint16_t* w, uint32_t ldw,
                        const uint16_t* bias, const uint16_t* residual, uint32_t ldr, uint16_t* y, uint32_t ldy,
@@ -395,8 +399,10 @@ int f3d_linear_bf16(const f3d_bf16_t* x, uint32_t ldx, const f3d_bf16_t* w, cons
   F3D_CHECK_ARG(guard.ok, "cannot select device %d", device);
   hipStream_t s = (hipStream_t)stream;
   SyncBracket sync(s);
-  // small inner dimensions: row-panel kernel (x read once, w streamed); otherwise the tiled GEMM
+  // small inner dimensions: row-panel kernel (x read once, w streamed); long inner dimensions with 128 / 256 outputs:
+  // output-panel kernel (x streamed once, y in registers); otherwise the tiled GEMM
   int rc = launch_xstat_linear(x, ldx, nullptr, nullptr, 0.f, w, bias, residual, ldr, y, ldy, m, n, k, act, device, s);
+  if (rc == F3D_ERR_UNSUPPORTED) rc = launch_ystat_linear(x, ldx, w, bias, residual, ldr, y, ldy, m, n, k, act, device, s);
   if (rc == F3D_ERR_UNSUPPORTED) rc = launch_gemm(false, x, ldx, w, k, bias, residual, ldr, y, ldy, m, n, k, act, s);
   if (rc != F3D_OK) return rc;
   F3D_CHECK_HIP(hipGetLastError());

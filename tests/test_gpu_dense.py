@@ -55,6 +55,9 @@ def test_gemm_sm_bf16_reference_case():
     (2500, 512, 512, None, True, True),        # out-projection + residual of that level
     (2100, 2048, 512, "swiglu", True, False),  # its fc1
     (700, 256, 512, "gelu", False, True),      # fc2 of a C=256 level
+    (40000, 256, 1024, None, True, True),      # fc2 + residual of the C=256 block at a size the output-panel kernel takes
+    (33001, 128, 640, None, False, False),     # the same kernel: 128 outputs, ragged M, 20 chunks, no bias, no residual
+    (35000, 256, 544, None, True, False),      # 17 chunks
 ])
 def test_linear_epilogues(oracle, M, N, K, act, use_bias, use_res):
     from flash3dtransformer_amd.lib import pshattn
