@@ -246,3 +246,31 @@ def test_layernorm_mlp_layer_fused_on_request():
     b(xg, residual=xg).float().square().mean().backward()
     assert xg.grad is not None and torch.isfinite(xg.grad.float()).all() and xg.grad.abs().max().item() > 0
     assert b.fc2_weight.grad.abs().max().item() > 0
+
+
+def test_fused_mlp_and_output_panel_kernel_at_bench_size():
+    """482,304 rows x 256 channels, hidden 1024 (the bench's MLP): the one-kernel MLP against LayerNorm+fc1+gate
+    followed by fc2+residual (which at this size runs the output-panel kernel), and the output-panel kernel against
+    the tiled GEMM on a row slice small enough to fall back to it."""
+    from flash3dtransformer_amd.lib import pshattn
+    M, C, H = 482304, 256, 1024
+    x = (_rand((M, C), 11, scale=1.5)).to(DEV)
+    g, b = (_rand((C,), 3) + 1.0).to(DEV), _rand((C,), 4, scale=0.2).to(DEV)
+    w1, w2 = _rand((2 * H, C), 2, scale=1 / math.sqrt(C)).to(DEV), _rand((C, H), 5, scale=1 / math.sqrt(H)).to(DEV)
+    b1, b2 = _rand((2 * H,), 6).to(DEV), _rand((C,), 7).to(DEV)
+    y = torch.empty(M, C, dtype=torch.bfloat16, device=DEV)
+    assert pshattn.ln_mlp_swiglu_bf16(x, g, b, 1e-5, w1, b1, w2, b2, x, y)
+    hid = torch.empty(M, H, dtype=torch.bfloat16, device=DEV)
+    y2 = torch.empty_like(y)
+    pshattn.ln_linear_bf16(x, g, b, 1e-5, w1, b1, None, hid, "swiglu")
+    pshattn.linear_bf16(hid, w2, b2, x, y2, None)                     # output-panel kernel (K = 1024 > 512, many rows)
+    torch.cuda.synchronize()
+    # one bf16 step of the fc2 output before the residual add, whose magnitude is at most |y| + |residual|
+    d = (y.float() - y2.float()).abs() / (y2.float().abs() + x.float().abs()).clamp(min=1.0)
+    assert d.max().item() <= 2 ** -6 and (d > 0).float().mean().item() < 0.02
+    n_small = 20000                                                   # fewer rows than the output-panel kernel takes
+    y3 = torch.empty(n_small, C, dtype=torch.bfloat16, device=DEV)
+    pshattn.linear_bf16(hid[-n_small:], w2, b2, x[-n_small:], y3, None)   # tiled GEMM
+    torch.cuda.synchronize()
+    d = (y2[-n_small:].float() - y3.float()).abs() / (y3.float().abs() + x[-n_small:].float().abs()).clamp(min=1.0)
+    assert d.max().item() <= 2 ** -6 and (d > 0).float().mean().item() < 0.02
