@@ -269,6 +269,31 @@ def test_model_consumes_point_features_and_restores_input_order():
         model(c, feat[:, :3], s)
 
 
+def test_restore_input_order_without_point_features():
+    """Default model (input_feat ignored, as in the reference): to_input_order builds the permutation index on demand;
+    row i of its result is the output row of input point i (checked through the scattered coordinates)."""
+    from flash3dtransformer_amd import layers as L, synth
+    from flash3dtransformer_amd.psh.bucket_scope import SwinPlan
+    bs = 256
+    torch.manual_seed(3)
+    ln = lambda ch: L.LayerNorm(ch)
+    spec = lambda c, h: L.XFMRSpecs(c, 2 * c, h, True, SwinPlan("swin", bs, 1, 0), ln)
+    model = L.Flash3D([L.F3DLevelSpecs([spec(32, 1)], [spec(32, 1)], "mean", 256, None, None, None, None)], bs, 1, 2).to(DEV)
+    with pytest.raises(RuntimeError, match="forward call first"):
+        model.to_input_order(torch.zeros(4, 32, device=DEV))
+    rng = np.random.default_rng(9)
+    coords, seps = synth.batch_of([rng.normal(0, 10, (n, 3)).astype(np.float32) for n in (9000, 8200)])
+    c = torch.from_numpy(coords).to(DEV)
+    s = torch.from_numpy(seps.view(np.int32)).to(DEV).view(torch.uint32)
+    with torch.no_grad():
+        out = model(c, None, s)
+        scattered = model.psh_scatter.last_scattered_coord
+        assert torch.equal(model.to_input_order(scattered), c)        # the scattered coordinates come back in input order
+        per_point = model.to_input_order(out)
+    idx = model._last_index.view(torch.int32)[:c.shape[0]].long()
+    assert torch.equal(out[:c.shape[0]], per_point[idx])
+
+
 def test_state_dict_names_match_reference_module_tree():
     """parameter names a reference checkpoint would carry (flash3dxfmr/layers/*.py module attributes;
     TransformerEngine's LayerNormMLP / Linear parameter names)"""
