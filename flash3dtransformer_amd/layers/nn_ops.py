@@ -1,7 +1,8 @@
 """HIP-backed building blocks of the layer API: Linear, LayerNorm, LayerNormMLP and the fused
 norm + activation used around pooling.  Parameters are ordinary nn.Parameters (fp32 by default, so
 a checkpoint of the reference's torch / TransformerEngine modules loads by name); the kernels run on
-bf16 copies that are refreshed whenever a parameter changes.
+bf16 copies: made anew on every training-mode or gradient-enabled forward, kept between eval-mode forwards
+under no_grad (see _Bf16Cache for when such a copy is dropped).
 
 Forward runs on the HIP kernels.  Backward of these dense layers is not a kernel of this library: as the
 reference leaves it to torch / TransformerEngine, the autograd functions here differentiate a torch restatement
@@ -78,20 +79,71 @@ def _linear_ref(act, eps):
 
 
 class _Bf16Cache:
-    """bf16 device copy of a parameter, rebuilt when the parameter is modified or moved"""
+    """bf16 device copy of a parameter for the kernels.
+
+    A parameter that already is bf16 is handed over as it is (always current).  An fp32 master parameter is cast
+    again on every forward while gradients are enabled or the owning module is in training mode, which is what the
+    reference's autocast forward does; only an eval-mode forward under no_grad keeps the copy between calls.  That
+    copy is dropped when the parameter's address or version changes, on train() / eval(), on load_state_dict and by
+    refresh_weights().  In-place edits through `.data` leave address and version alone: after one of those in eval
+    mode call refresh_weights(model)."""
 
     def __init__(self):
         self._key = None
         self._val = None
 
-    def get(self, p: torch.Tensor) -> torch.Tensor:
+    def clear(self):
+        self._key = self._val = None
+
+    def get(self, p: torch.Tensor, training: bool = False) -> torch.Tensor:
         if p is None:
             return None
+        if p.dtype == torch.bfloat16 and p.is_contiguous():
+            return p.detach()
+        if training or torch.is_grad_enabled():
+            self.clear()
+            return p.detach().to(torch.bfloat16).contiguous()
         key = (p.data_ptr(), p._version, p.dtype, p.device)
         if key != self._key:
             self._val = p.detach().to(torch.bfloat16).contiguous()
             self._key = key
         return self._val
+
+
+class _CachedParamModule(nn.Module):
+    """nn.Module whose kernels read bf16 copies of its parameters (`_Bf16Cache` attributes or lists of them)"""
+
+    def _bf16_caches(self):
+        for v in self.__dict__.values():
+            if isinstance(v, _Bf16Cache):
+                yield v
+            elif isinstance(v, (list, tuple)):
+                for c in v:
+                    if isinstance(c, _Bf16Cache):
+                        yield c
+
+    def refresh_weights(self):
+        for c in self._bf16_caches():
+            c.clear()
+
+    def train(self, mode: bool = True):
+        self.refresh_weights()
+        return super().train(mode)
+
+    def _load_from_state_dict(self, state_dict, prefix, *args, **kwargs):
+        # TransformerEngine modules of the reference store one `_extra_state` entry each (fp8 recipe state, of no use
+        # to a bf16 kernel): dropped, so that such a checkpoint loads with strict=True
+        state_dict.pop(prefix + "_extra_state", None)
+        self.refresh_weights()
+        return super()._load_from_state_dict(state_dict, prefix, *args, **kwargs)
+
+
+def refresh_weights(module: nn.Module) -> None:
+    """Drops every cached bf16 weight copy under `module`; needed only after in-place edits through `.data`
+    (EMA swaps, manual re-initialisation) on a model that stays in eval mode under no_grad."""
+    for m in module.modules():
+        if isinstance(m, _CachedParamModule):
+            m.refresh_weights()
 
 
 def as_bf16_2d(x: torch.Tensor) -> torch.Tensor:
@@ -102,7 +154,7 @@ def as_bf16_2d(x: torch.Tensor) -> torch.Tensor:
     return x
 
 
-class Linear(nn.Module):
+class Linear(_CachedParamModule):
     """y = act(x W^T + b) (+ residual) on MFMA; parameter names match torch.nn.Linear / te.Linear"""
 
     def __init__(self, in_features: int, out_features: int, bias: bool = True):
@@ -129,9 +181,9 @@ class Linear(nn.Module):
         r2 = None if residual is None else as_bf16_2d(residual.reshape(-1, n_out))
         if pre_norm is not None:
             g, b = norm_params_bf16(pre_norm)
-            pshattn.ln_linear_bf16(x2, g, b, pre_norm.eps, self._w.get(self.weight), self._b.get(self.bias), r2, y, act)
+            pshattn.ln_linear_bf16(x2, g, b, pre_norm.eps, self._w.get(self.weight, self.training), self._b.get(self.bias, self.training), r2, y, act)
         else:
-            pshattn.linear_bf16(x2, self._w.get(self.weight), self._b.get(self.bias), r2, y, act)
+            pshattn.linear_bf16(x2, self._w.get(self.weight, self.training), self._b.get(self.bias, self.training), r2, y, act)
         ln_w = None if pre_norm is None else pre_norm.weight
         ln_b = None if pre_norm is None else pre_norm.bias
         eps = 0.0 if pre_norm is None else pre_norm.eps
@@ -143,7 +195,7 @@ class Linear(nn.Module):
         return f"in_features={self.in_features}, out_features={self.out_features}, bias={self.bias is not None}"
 
 
-class LayerNorm(nn.Module):
+class LayerNorm(_CachedParamModule):
     """LayerNorm over the last axis with fp32 statistics; parameter names match nn.LayerNorm / te.LayerNorm"""
 
     def __init__(self, normalized_shape: int, eps: float = 1e-5):
@@ -156,7 +208,7 @@ class LayerNorm(nn.Module):
     def forward(self, x: torch.Tensor):
         x2 = as_bf16_2d(x.reshape(-1, x.shape[-1])).contiguous()
         y = torch.empty_like(x2)
-        pshattn.layernorm_bf16(x2, self._w.get(self.weight), self._b.get(self.bias), y, self.eps)
+        pshattn.layernorm_bf16(x2, self._w.get(self.weight, self.training), self._b.get(self.bias, self.training), y, self.eps)
         eps = self.eps
         ref = lambda xx, w, b: torch.nn.functional.layer_norm(xx, (xx.shape[-1],), w, b, eps)
         return torch_backward(y, ref, x.reshape(-1, x.shape[-1]), self.weight, self.bias).view(x.shape)
@@ -177,7 +229,7 @@ def is_fusable_layernorm(norm, width: int) -> bool:
 
 def norm_params_bf16(norm):
     if isinstance(norm, LayerNorm):
-        return norm._w.get(norm.weight), norm._b.get(norm.bias)
+        return norm._w.get(norm.weight, norm.training), norm._b.get(norm.bias, norm.training)
     b = None if norm.bias is None else norm.bias.detach().to(torch.bfloat16).contiguous()
     return norm.weight.detach().to(torch.bfloat16).contiguous(), b
 
@@ -236,7 +288,7 @@ def apply_norm_act(norm, act, x: torch.Tensor) -> torch.Tensor:
     return x
 
 
-class LayerNormMLP(nn.Module):
+class LayerNormMLP(_CachedParamModule):
     """LayerNorm -> fc1 -> activation -> fc2, the role te.LayerNormMLP plays in the reference
     (flash3dxfmr/layers/elem_wise.py:22-26).  Parameter names follow TransformerEngine
     (layer_norm_weight/bias, fc1_weight/bias, fc2_weight/bias).  activation "swiglu": fc1 has
@@ -270,20 +322,20 @@ class LayerNormMLP(nn.Module):
         # on request, the whole gated MLP in one kernel where one exists (hidden activations stay in registers) ...
         fused = (self.fused and self.activation == "swiglu" and self.hidden_size in FUSED_MLP_WIDTHS
                  and self.ffn_hidden_size % 32 == 0
-                 and pshattn.ln_mlp_swiglu_bf16(x2, c[0].get(self.layer_norm_weight), c[1].get(self.layer_norm_bias),
-                                                self.eps, c[2].get(self.fc1_weight), c[3].get(self.fc1_bias),
-                                                c[4].get(self.fc2_weight), c[5].get(self.fc2_bias), r2, y))
+                 and pshattn.ln_mlp_swiglu_bf16(x2, c[0].get(self.layer_norm_weight, self.training), c[1].get(self.layer_norm_bias, self.training),
+                                                self.eps, c[2].get(self.fc1_weight, self.training), c[3].get(self.fc1_bias, self.training),
+                                                c[4].get(self.fc2_weight, self.training), c[5].get(self.fc2_bias, self.training), r2, y))
         if not fused:
             # ... otherwise LayerNorm + fc1 + activation, then fc2 + residual
             h = torch.empty(x2.shape[0], self.ffn_hidden_size, dtype=torch.bfloat16, device=x.device)
             if self.hidden_size in FUSABLE_LN_WIDTHS:
-                pshattn.ln_linear_bf16(x2, c[0].get(self.layer_norm_weight), c[1].get(self.layer_norm_bias), self.eps,
-                                       c[2].get(self.fc1_weight), c[3].get(self.fc1_bias), None, h, self.activation)
+                pshattn.ln_linear_bf16(x2, c[0].get(self.layer_norm_weight, self.training), c[1].get(self.layer_norm_bias, self.training), self.eps,
+                                       c[2].get(self.fc1_weight, self.training), c[3].get(self.fc1_bias, self.training), None, h, self.activation)
             else:
                 ln = torch.empty_like(x2)
-                pshattn.layernorm_bf16(x2, c[0].get(self.layer_norm_weight), c[1].get(self.layer_norm_bias), ln, self.eps)
-                pshattn.linear_bf16(ln, c[2].get(self.fc1_weight), c[3].get(self.fc1_bias), None, h, self.activation)
-            pshattn.linear_bf16(h, c[4].get(self.fc2_weight), c[5].get(self.fc2_bias), r2, y, None)
+                pshattn.layernorm_bf16(x2, c[0].get(self.layer_norm_weight, self.training), c[1].get(self.layer_norm_bias, self.training), ln, self.eps)
+                pshattn.linear_bf16(ln, c[2].get(self.fc1_weight, self.training), c[3].get(self.fc1_bias, self.training), None, h, self.activation)
+            pshattn.linear_bf16(h, c[4].get(self.fc2_weight, self.training), c[5].get(self.fc2_bias, self.training), r2, y, None)
         act, eps = self.activation, self.eps
 
         def ref(xx, res, ln_w, ln_b, w1, b1, w2, b2):

@@ -73,7 +73,7 @@ class PSH3DCoordEmbedding(nn.Module):
         self.last_buffers = buffers
         emb = torch.empty(pad_to, self.lin.out_features, dtype=torch.bfloat16, device=coords.device)
         lin = self.lin
-        pshattn.coord_embed_bf16(scattered, lin._w.get(lin.weight), lin._b.get(lin.bias), emb)
+        pshattn.coord_embed_bf16(scattered, lin._w.get(lin.weight, lin.training), lin._b.get(lin.bias, lin.training), emb)
         # the coordinates carry no gradient; the embedding's weights do (bf16 view of the fp16 coordinates, as the kernel reads them)
         coord_f = scattered
         ref = lambda w, b: torch.nn.functional.linear(coord_f.to(torch.bfloat16).float(), w, b)

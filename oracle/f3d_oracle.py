@@ -7,6 +7,13 @@ never does.
 
 Arrays are numpy: fp16 coordinates as ``np.float16``, bf16 features as raw ``np.uint16`` bit
 patterns, counters as ``np.uint32`` / ``np.uint16`` (the reference's CounterT / HashT).
+
+Pins (tests/test_oracle_*.py, tests/test_golden.py): every function below is held to known answers, brute force or
+a numpy / torch library routine of the same quantity, except one.  PARITY UNPINNED: ``swiglu`` -- which half of
+fc1's output te.LayerNormMLP(activation="swiglu") gates is fixed by TransformerEngine, which is not in this image
+and which no test of the reference checks; the function itself (silu of the first half times the second) is held
+to torch.nn.functional.silu.  The model-level functions (xfmr_block, stage_forward, flash3d_forward) only compose
+pinned functions in the order of the reference's layer files, cited at each.
 """
 import ctypes
 import math
@@ -478,3 +485,88 @@ def bn_act(x, bn, act):
     elif act == "relu":
         x = _r(torch.relu(x))
     return x
+
+
+def norm_act(x, p, act):
+    """optional norm then optional activation, each rounded to bf16.  `p` is None, a LayerNorm dict
+    (weight, bias, eps) or an eval-mode BatchNorm1d dict (weight, bias, mean, var, eps): the callables the
+    reference passes as pool_norm / unpool_norm (tests/test_psh_hourglass.py:103-106)"""
+    import torch
+    if p is not None and "mean" in p:
+        return bn_act(x, p, act)
+    if p is not None:
+        x = _r(torch.nn.functional.layer_norm(x.float(), (x.shape[-1],), p["weight"], p["bias"], p.get("eps", 1e-5)))
+    return bn_act(x, None, act)
+
+
+XFMR_KEYS = {"norm.weight": "norm.weight", "norm.bias": "norm.bias", "qkv.weight": "bwa.qkv.weight",
+             "qkv.bias": "bwa.qkv.bias", "proj.weight": "bwa.proj.weight", "proj.bias": "bwa.proj.bias",
+             "ln.weight": "mlp.mlp.layer_norm_weight", "ln.bias": "mlp.mlp.layer_norm_bias",
+             "fc1.weight": "mlp.mlp.fc1_weight", "fc1.bias": "mlp.mlp.fc1_bias",
+             "fc2.weight": "mlp.mlp.fc2_weight", "fc2.bias": "mlp.mlp.fc2_bias"}
+
+
+def _norm_params(sd, prefix, eps_bn=1e-3):
+    if prefix + "weight" not in sd:
+        return None
+    p = {"weight": sd[prefix + "weight"], "bias": sd[prefix + "bias"]}
+    if prefix + "running_mean" in sd:
+        p.update(mean=sd[prefix + "running_mean"], var=sd[prefix + "running_var"], eps=eps_bn)
+    return p
+
+
+def stage_forward(sd, prefix, coord_h, x, seps, levels, level, bs, scope, S, trace=None):
+    """Stage.forward (layers/stage.py:171-197) around HourglassModule.forward (layers/hourglass.py:268-293) or the
+    LeafModule (layers/flash3d.py:25-38), recursively.  `sd`: state dict of fp32 CPU tensors holding bf16 values
+    (norm statistics fp32); `levels[level]`: dict(heads, n_enc, n_dec, red_op, pool_align, pool_act, unpool_act,
+    bn_eps).  x [n, C] fp32 holding bf16 values, coord_h [n, 3] fp16, seps inclusive cumulative sizes whose last
+    entry is n."""
+    import torch
+    cfg = levels[level]
+    n = x.shape[0]
+    scopes = gen_scopes(n, bs, scope)
+    w = lambda pre: {k: sd[pre + v] for k, v in XFMR_KEYS.items() if pre + v in sd}
+    for i in range(cfg["n_enc"]):
+        x = xfmr_block(x, w(f"{prefix}encoder_blocks.{i}."), scopes, bs, cfg["heads"], cfg.get("activation", "swiglu"))
+    if trace is not None:
+        trace.append(("enc", level, x))
+    mid = prefix + "middle."
+    if level + 1 == len(levels):
+        x = _r(linear(x, sd[mid + "proj.weight"], sd[mid + "proj.bias"]))
+    else:
+        proj = _r(linear(x, sd[mid + "pooling.proj.weight"], sd[mid + "pooling.proj.bias"]))
+        _, _, unpool, red_coord, red_sep = subbuck_build(coord_h, seps, S, out_align=cfg["pool_align"])
+        r_al = red_coord.shape[0]
+        red = torch.from_numpy(bf16_bits_to_f32(reduce_feat(f32_to_bf16_bits(proj.numpy()), unpool, cfg["red_op"],
+                                                              r_aligned=r_al)))
+        red = norm_act(red, _norm_params(sd, mid + "pooling.norm.", cfg.get("bn_eps", 1e-3)), cfg.get("pool_act"))
+        sub_sep = np.array(red_sep, dtype=np.uint32).copy()
+        sub_sep[-1] = r_al
+        if trace is not None:
+            trace.append(("pool", level, unpool, red_coord))
+        sub = stage_forward(sd, mid + "submodule.", red_coord, red, sub_sep, levels, level + 1, bs, scope, S, trace)
+        un = mid + "unpooling."
+        pd = norm_act(_r(linear(sub, sd[un + "proj.0.weight"], sd[un + "proj.0.bias"])),
+                      _norm_params(sd, un + "proj.norm.", cfg.get("bn_eps", 1e-3)), cfg.get("unpool_act"))
+        ps = norm_act(_r(linear(proj, sd[un + "proj_skip.0.weight"], sd[un + "proj_skip.0.bias"])),
+                      _norm_params(sd, un + "proj_skip.norm.", cfg.get("bn_eps", 1e-3)), cfg.get("unpool_act"))
+        up = additive_unpool(f32_to_bf16_bits(ps.numpy()), f32_to_bf16_bits(pd.numpy()), unpool)
+        x = torch.from_numpy(bf16_bits_to_f32(up))
+    for i in range(cfg["n_dec"]):
+        x = xfmr_block(x, w(f"{prefix}decoder_blocks.{i}."), scopes, bs, cfg["heads"], cfg.get("activation", "swiglu"))
+    return x
+
+
+def flash3d_forward(sd, coord_h, seps, levels, bs, scope, hash_op, S, trace=None):
+    """Flash3D.forward (layers/flash3d.py:148-166) with the scattered coordinates routed down the tree and the pad
+    rows counted into the last cloud.  Returns (output [pad_to, C] fp32 holding bf16 values, scattered coords)."""
+    import torch
+    n = coord_h.shape[0]
+    align = bs * scope * 6
+    pad_to = -(-n // align) * align
+    scat = psh_scatter_coords(coord_h, seps, bs, pad_to, hash_op)
+    x = _r(linear(torch.from_numpy(scat.astype(np.float32)).to(torch.bfloat16), sd["psh_scatter.lin.weight"],
+                  sd["psh_scatter.lin.bias"]))
+    tree_seps = np.array(seps, dtype=np.uint32).copy()
+    tree_seps[-1] = pad_to
+    return stage_forward(sd, "module_tree.", scat, x, tree_seps, levels, 0, bs, scope, S, trace), scat

@@ -31,7 +31,8 @@ def test_gemm_sm_bf16_reference_case():
     o = torch.zeros(M, N, dtype=torch.bfloat16, device=DEV)
     pshattn.gemm_sm_bf16(a, b, o)
     ref = a.float().cpu() @ b.float().cpu()
-    assert torch.allclose(o.float().cpu(), ref, atol=1e-2 * K ** 0.5, rtol=1e-2)
+    # the reference's own bar for this op (tests/test_gemm.py:35 of the reference)
+    assert torch.allclose(o.float().cpu(), ref, atol=1e-2, rtol=1e-2)
     # general shapes, which the reference op rejects
     for (M, N, K) in [(300, 72, 40), (1, 8, 8), (1000, 520, 264)]:
         a, b = _rand((M, K), M).to(DEV), _rand((K, N), N).to(DEV)

@@ -1,0 +1,54 @@
+"""Host-side logic of the layer modules that needs no GPU: when the bf16 weight copies the kernels read are made anew,
+and loading a checkpoint that carries TransformerEngine's per-module `_extra_state` entries."""
+import torch
+
+from flash3dtransformer_amd import layers as L
+from flash3dtransformer_amd.layers import nn_ops
+
+
+def test_bf16_weight_copy_follows_the_parameter():
+    lin = L.Linear(8, 4)
+    w0 = lin._w.get(lin.weight, lin.training)
+    # training mode or enabled gradients: every call casts again, so an edit through .data is seen at once
+    lin.weight.data.mul_(0)
+    assert lin._w.get(lin.weight, lin.training).abs().max().item() == 0 and w0.abs().max().item() > 0
+    lin.weight.data.normal_()
+    lin.eval()
+    with torch.no_grad():
+        a = lin._w.get(lin.weight, lin.training)
+        assert lin._w.get(lin.weight, lin.training) is a                 # kept between eval-mode forwards
+        lin.weight.mul_(2.0)                                             # ordinary in-place edit: version moves
+        b = lin._w.get(lin.weight, lin.training)
+        assert b is not a and torch.equal(b, lin.weight.to(torch.bfloat16))
+        lin.weight.data.zero_()                                          # through .data: invisible ...
+        assert lin._w.get(lin.weight, lin.training) is b
+        L.refresh_weights(lin)                                           # ... until the copies are dropped
+        assert lin._w.get(lin.weight, lin.training).abs().max().item() == 0
+        lin.weight.data.fill_(1.0)
+        lin.eval()                                                       # a mode call drops them too
+        assert lin._w.get(lin.weight, lin.training).min().item() == 1.0
+    # a bf16 parameter is handed over itself
+    lin16 = L.Linear(8, 4).to(torch.bfloat16).eval()
+    with torch.no_grad():
+        assert lin16._w.get(lin16.weight, False).data_ptr() == lin16.weight.data_ptr()
+
+
+def test_load_state_dict_drops_copies_and_accepts_extra_state():
+    mlp = L.LayerNormMLP(32, 64).eval()
+    with torch.no_grad():
+        old = mlp._c[2].get(mlp.fc1_weight, False)
+        sd = {k: torch.zeros_like(v) for k, v in mlp.state_dict().items()}
+        sd["_extra_state"] = None           # what te.LayerNormMLP stores beside its parameters
+        mlp.load_state_dict(sd, strict=True)
+        new = mlp._c[2].get(mlp.fc1_weight, False)
+    assert new.abs().max().item() == 0 and old.abs().max().item() > 0
+    # nested: the reference's MLP wrapper holds te.LayerNormMLP as `.mlp`, te.Linear as the leaf `.proj`
+    blk = L.MLP(32, 64)
+    sd = dict(blk.state_dict())
+    sd["mlp._extra_state"] = torch.zeros(1)
+    blk.load_state_dict(sd, strict=True)
+    lin = L.Linear(8, 4)
+    sd = dict(lin.state_dict())
+    sd["_extra_state"] = None
+    lin.load_state_dict(sd, strict=True)
+    assert isinstance(lin, nn_ops._CachedParamModule)

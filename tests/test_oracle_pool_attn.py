@@ -301,3 +301,48 @@ def test_attention_bwd_formulas_vs_autograd(oracle):
     dQ2, dK2, dV2, _ = oracle.buck_swin_bwd(Q.detach(), K.detach(), V.detach(), dO, np.array([[1, 0]], dtype=np.uint32), bs)
     assert not dQ2[:, 256:].any() and not dK2[:, 256:].any() and not dV2[:, 256:].any()
     assert torch.equal(dQ2[:, :256], dQ[:, :256])
+
+
+@pytest.mark.parametrize("act", [None, "gelu", "relu"])
+def test_bn_act_vs_torch_batch_norm(oracle, act):
+    """eval-mode BatchNorm1d (+ GELU / ReLU) of the oracle against torch.nn.functional.batch_norm(training=False) and the
+    library activations on random statistics (the reference's pool_norm / unpool_norm callables,
+    tests/test_psh_hourglass.py:103-106: BatchNorm1d(eps=1e-3) then GELU)"""
+    g = torch.Generator().manual_seed(17)
+    n, c = 513, 40
+    x = (torch.randn(n, c, generator=g) * 2).to(torch.bfloat16).float()
+    bn = {"weight": torch.rand(c, generator=g) + 0.5, "bias": torch.randn(c, generator=g) * 0.3,
+          "mean": torch.randn(c, generator=g) * 0.5, "var": torch.rand(c, generator=g) * 2 + 0.1, "eps": 1e-3}
+    got = oracle.bn_act(x, bn, act)
+    want = torch.nn.functional.batch_norm(x, bn["mean"], bn["var"], bn["weight"], bn["bias"], False, 0.0, bn["eps"])
+    # the library may associate (x - mean) * rstd * w + b differently: at most one bf16 step before the activation
+    want_r = want.to(torch.bfloat16).float()
+    pre = oracle.bn_act(x, bn, None)
+    assert (pre - want).abs().max().item() <= 2 ** -8 * max(1.0, want.abs().max().item())
+    assert (pre != want_r).float().mean().item() < 0.01
+    if act == "gelu":
+        want_a = torch.nn.functional.gelu(pre).to(torch.bfloat16).float()
+    elif act == "relu":
+        want_a = torch.relu(pre)
+    else:
+        want_a = pre
+    assert torch.equal(got, want_a)
+    # a module says the same: nn.BatchNorm1d in eval mode with those statistics
+    m = torch.nn.BatchNorm1d(c, eps=1e-3).eval()
+    with torch.no_grad():
+        m.weight.copy_(bn["weight"]); m.bias.copy_(bn["bias"])
+        m.running_mean.copy_(bn["mean"]); m.running_var.copy_(bn["var"])
+        assert torch.allclose(m(x), want, atol=1e-6, rtol=1e-6)
+    # a dropped shift, a forgotten eps or var used as std would all fail the comparison above; make sure of one
+    wrong = (x - bn["mean"]) / torch.sqrt(bn["var"]) * bn["weight"] + bn["bias"]
+    assert (wrong - want).abs().max().item() > 2 ** -8 * max(1.0, want.abs().max().item())
+
+
+def test_norm_act_layernorm_vs_torch(oracle):
+    g = torch.Generator().manual_seed(18)
+    x = torch.randn(100, 64, generator=g).to(torch.bfloat16).float()
+    p = {"weight": torch.rand(64, generator=g) + 0.5, "bias": torch.randn(64, generator=g) * 0.1, "eps": 1e-5}
+    want = torch.nn.functional.layer_norm(x, (64,), p["weight"], p["bias"], 1e-5).to(torch.bfloat16).float()
+    assert torch.equal(oracle.norm_act(x, p, None), want)
+    assert torch.equal(oracle.norm_act(x, p, "gelu"), torch.nn.functional.gelu(want).to(torch.bfloat16).float())
+    assert torch.equal(oracle.norm_act(x, None, None), x)
