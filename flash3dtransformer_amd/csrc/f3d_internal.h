@@ -19,6 +19,10 @@ void set_error(const char* fmt, ...) __attribute__((format(printf, 1, 2)));
 // Returns nullptr (and sets the error) on allocation failure.
 void* workspace(int device, size_t bytes);
 
+// This device's copy of the fixed scratch array behind f3d_batch_psh_scatter_pad_hash_noalloc (resolved on the first
+// call per device; f3d_init_dev_info does it ahead of time).  nullptr + error message on failure.
+uint32_t* psh_noalloc_scratch(int device);
+
 bool sync_stream_enabled();
 uint32_t global_seed();
 int rebalance_mode();

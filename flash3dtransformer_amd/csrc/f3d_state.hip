@@ -32,6 +32,7 @@ void* workspace(int device, size_t bytes) {
   std::lock_guard<std::mutex> lk(g_mu);
   Ws& w = g_ws[device];
   if (w.bytes >= bytes && w.ptr) return w.ptr;
+  DeviceGuard guard(device);
   // Work queued on the old buffer must finish before it is released.
   if (w.ptr) {
     (void)hipDeviceSynchronize();
@@ -39,7 +40,6 @@ void* workspace(int device, size_t bytes) {
     w.ptr = nullptr;
     w.bytes = 0;
   }
-  DeviceGuard guard(device);
   size_t want = bytes < (size_t(1) << 20) ? (size_t(1) << 20) : bytes + bytes / 4;
   void* p = nullptr;
   hipError_t e = hipMalloc(&p, want);
@@ -67,6 +67,7 @@ int f3d_init_dev_info(int device) {
   F3D_CHECK_HIP(hipGetDeviceCount(&n));
   // The reference silently ignores a device that does not exist (device_manager.cu:59-60).
   if (device < 0 || device >= n) return F3D_OK;
+  if (!f3d::psh_noalloc_scratch(device)) return F3D_ERR_RUNTIME;
   return f3d::workspace(device, 1) ? F3D_OK : F3D_ERR_RUNTIME;
 }
 

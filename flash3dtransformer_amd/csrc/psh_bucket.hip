@@ -14,6 +14,8 @@
 //                   write bucket_offset and scatter the coordinate row; extra workgroups fill the pad rows
 // No global atomics, no dependence on workgroup scheduling: bucket ids, counts AND slots are a pure
 // function of the input.  HBM traffic per point: K1 6 B read + 2 B write, K3 8 B read + 10 B write.
+#include <mutex>
+
 #include "f3d_device.h"
 #include "f3d_internal.h"
 
@@ -511,19 +513,53 @@ static void launch_psh(const uint16_t* coord, uint16_t* bucket_id, uint32_t* buc
   }
 }
 
-}  // namespace f3d
 
-extern "C" {
+// ---- scratch memory of the entry point that allocates nothing ---------------------------------------
+// f3d_batch_psh_scatter_pad_hash_noalloc keeps the tile histograms, first-hash counts and the rebalance
+// plan in this array instead of the grow-only workspace.  Every GPU the library runs on holds its own copy
+// until the process ends.  The name `scratch` is a host-side stand-in for the symbol, not a device
+// address: host code only ever uses the per-device address that hipGetSymbolAddress returned.
+constexpr size_t kNoAllocScratchWords = F3D_PSH_NOALLOC_SCRATCH_BYTES / sizeof(uint32_t);
+static __device__ __align__(256) uint32_t scratch[kNoAllocScratchWords];
 
-int f3d_batch_psh_scatter_pad_hash(const f3d_half_t* coord, uint16_t* bucket_id, uint32_t* bucket_counter,
-                                   uint32_t* bucket_offset, const uint32_t* batch_sep, uint32_t batch_size,
-                                   uint32_t total_n, uint32_t instance_max_n, uint32_t num_bucket,
-                                   uint32_t bucket_divisor, uint32_t bucket_size, uint32_t num_vox,
-                                   const f3d_half_t* bbox_min, const f3d_half_t* bbox_max,
-                                   const int16_t* probe_offsets, uint32_t* cumsum_counter,
-                                   f3d_half_t* scatter_coord, uint32_t pad_to_n, float pad_num,
-                                   uint32_t hash_type, int device, void* stream) {
-  using namespace f3d;
+constexpr int kMaxDevices = 64;
+static std::mutex g_scratch_mu;
+static uint32_t* g_scratch_ptr[kMaxDevices] = {};
+
+// Address of this device's copy of `scratch`; resolved once per device, with that device current.
+// Returns nullptr (and sets the error) on failure.
+uint32_t* psh_noalloc_scratch(int device) {
+  if (device < 0 || device >= kMaxDevices) {
+    set_error("device index %d outside [0, %d)", device, kMaxDevices);
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> lk(g_scratch_mu);
+  if (g_scratch_ptr[device]) return g_scratch_ptr[device];
+  DeviceGuard guard(device);
+  if (!guard.ok) {
+    set_error("cannot select device %d", device);
+    return nullptr;
+  }
+  void* ptr = nullptr;
+  const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+  if (e != hipSuccess || ptr == nullptr) {
+    set_error("hipGetSymbolAddress(scratch) failed on device %d: %s", device, hipGetErrorString(e));
+    return nullptr;
+  }
+  g_scratch_ptr[device] = static_cast<uint32_t*>(ptr);
+  return g_scratch_ptr[device];
+}
+
+// Checks, kernel selection and the four launches shared by the two entry points.  `ws` = scratch memory of
+// `ws_words` 32-bit words, or nullptr: then the library's grow-only workspace is used (and may be allocated).
+static int psh_run(const f3d_half_t* coord, uint16_t* bucket_id, uint32_t* bucket_counter,
+                   uint32_t* bucket_offset, const uint32_t* batch_sep, uint32_t batch_size,
+                   uint32_t total_n, uint32_t instance_max_n, uint32_t num_bucket,
+                   uint32_t bucket_divisor, uint32_t bucket_size, uint32_t num_vox,
+                   const f3d_half_t* bbox_min, const f3d_half_t* bbox_max,
+                   const int16_t* probe_offsets, uint32_t* cumsum_counter,
+                   f3d_half_t* scatter_coord, uint32_t pad_to_n, float pad_num,
+                   uint32_t hash_type, int device, void* stream, bool no_alloc) {
   // The probe table is part of the reference signature; the deterministic rebalance below does not
   // probe (see psh_bucket_plan_kernel) and never reads it.
   (void)probe_offsets;
@@ -548,8 +584,6 @@ int f3d_batch_psh_scatter_pad_hash(const f3d_half_t* coord, uint16_t* bucket_id,
                 "null tensor pointer");
   if (pad_to_n == 0) return F3D_OK;
 
-  DeviceGuard guard(device);
-  F3D_CHECK_ARG(guard.ok, "cannot select device %d", device);
   hipStream_t s = (hipStream_t)stream;
   // Inputs large enough to fill the chip with 8192-point tiles use 1024-thread workgroups that stage
   // the scatter through LDS; smaller ones use 256-thread workgroups with tiles sized for parallelism.
@@ -561,7 +595,16 @@ int f3d_batch_psh_scatter_pad_hash(const f3d_half_t* coord, uint16_t* bucket_id,
   const size_t hist_words = (size_t)batch_size * max_tiles * num_bucket;
   const size_t cnt_words = (size_t)batch_size * num_bucket;
   const size_t plan_words = (size_t)batch_size * (3 * num_bucket + 4);
-  uint32_t* tile_hist = (uint32_t*)workspace(device, (hist_words + cnt_words + plan_words + 4) * sizeof(uint32_t));
+  const size_t ws_words = hist_words + cnt_words + plan_words + 4;
+  if (no_alloc && ws_words > kNoAllocScratchWords) {
+      set_error("f3d_batch_psh_scatter_pad_hash_noalloc: this batch needs %zu bytes of scratch memory (%u clouds x %u "
+              "tiles x %u buckets), the fixed scratch array holds %zu; use f3d_batch_psh_scatter_pad_hash",
+              ws_words * sizeof(uint32_t), batch_size, max_tiles, num_bucket, kNoAllocScratchWords * sizeof(uint32_t));
+    return F3D_ERR_UNSUPPORTED;
+  }
+  DeviceGuard guard(device);
+  F3D_CHECK_ARG(guard.ok, "cannot select device %d", device);
+  uint32_t* tile_hist = no_alloc ? psh_noalloc_scratch(device) : (uint32_t*)workspace(device, ws_words * sizeof(uint32_t));
   if (!tile_hist) return F3D_ERR_RUNTIME;
   uint32_t* cnt_ws = tile_hist + hist_words;
   uint32_t* plan_ws = cnt_ws + cnt_words;
@@ -597,6 +640,36 @@ int f3d_batch_psh_scatter_pad_hash(const f3d_half_t* coord, uint16_t* bucket_id,
 #undef F3D_PSH_ARGS
   F3D_CHECK_HIP(hipGetLastError());
   return F3D_OK;
+}
+
+}  // namespace f3d
+
+extern "C" {
+
+int f3d_batch_psh_scatter_pad_hash(const f3d_half_t* coord, uint16_t* bucket_id, uint32_t* bucket_counter,
+                                   uint32_t* bucket_offset, const uint32_t* batch_sep, uint32_t batch_size,
+                                   uint32_t total_n, uint32_t instance_max_n, uint32_t num_bucket,
+                                   uint32_t bucket_divisor, uint32_t bucket_size, uint32_t num_vox,
+                                   const f3d_half_t* bbox_min, const f3d_half_t* bbox_max,
+                                   const int16_t* probe_offsets, uint32_t* cumsum_counter,
+                                   f3d_half_t* scatter_coord, uint32_t pad_to_n, float pad_num,
+                                   uint32_t hash_type, int device, void* stream) {
+  return f3d::psh_run(coord, bucket_id, bucket_counter, bucket_offset, batch_sep, batch_size, total_n, instance_max_n,
+                      num_bucket, bucket_divisor, bucket_size, num_vox, bbox_min, bbox_max, probe_offsets,
+                      cumsum_counter, scatter_coord, pad_to_n, pad_num, hash_type, device, stream, false);
+}
+
+int f3d_batch_psh_scatter_pad_hash_noalloc(const f3d_half_t* coord, uint16_t* bucket_id, uint32_t* bucket_counter,
+                                           uint32_t* bucket_offset, const uint32_t* batch_sep, uint32_t batch_size,
+                                           uint32_t total_n, uint32_t instance_max_n, uint32_t num_bucket,
+                                           uint32_t bucket_divisor, uint32_t bucket_size, uint32_t num_vox,
+                                           const f3d_half_t* bbox_min, const f3d_half_t* bbox_max,
+                                           const int16_t* probe_offsets, uint32_t* cumsum_counter,
+                                           f3d_half_t* scatter_coord, uint32_t pad_to_n, float pad_num,
+                                           uint32_t hash_type, int device, void* stream) {
+  return f3d::psh_run(coord, bucket_id, bucket_counter, bucket_offset, batch_sep, batch_size, total_n, instance_max_n,
+                      num_bucket, bucket_divisor, bucket_size, num_vox, bbox_min, bbox_max, probe_offsets,
+                      cumsum_counter, scatter_coord, pad_to_n, pad_num, hash_type, device, stream, true);
 }
 
 int f3d_coord_bbox(const f3d_half_t* coord, uint32_t total_n, f3d_half_t* bbox_min, f3d_half_t* bbox_max, int device,

@@ -117,16 +117,21 @@ class DeviceManagerSingleton:
 
 def batch_psh_scatter_pad_hash(coord, bucket_id, bucket_counter, bucket_offset, batch_sep, instance_max_N,
                                num_bucket, bucket_divisor, bucket_size, num_vox, bbox_min, bbox_max,
-                               probe_offsets, cumsum_counter, scatter_coord, pad_num, hash_type):
-    """src/f3d_frontend.cu:52-58 -> src/psh/batch_psh_bucket_dispatcher.cu:221-326"""
+                               probe_offsets, cumsum_counter, scatter_coord, pad_num, hash_type, no_alloc=False):
+    """src/f3d_frontend.cu:52-58 -> src/psh/batch_psh_bucket_dispatcher.cu:221-326.
+    no_alloc=True takes the entry point that allocates nothing (fixed scratch array in the library, no
+    counterpart in the reference; bbox_min / bbox_max must then be contiguous already)."""
     ts = [coord, bucket_id, bucket_counter, bucket_offset, batch_sep, probe_offsets, cumsum_counter, scatter_coord]
     assert_contiguous(ts)
     dev = assert_same_device(ts + [bbox_min, bbox_max])
     assert_dtype([coord, bbox_min, bbox_max, scatter_coord], torch.float16)
     assert_dtype([bucket_counter, bucket_offset, batch_sep, cumsum_counter], torch.uint32)
     assert_dtype([bucket_id], torch.uint16)
+    if no_alloc:
+        assert_contiguous([bbox_min, bbox_max])
     bbox_min, bbox_max = bbox_min.contiguous(), bbox_max.contiguous()
-    _check(_load().f3d_batch_psh_scatter_pad_hash(
+    fn = _load().f3d_batch_psh_scatter_pad_hash_noalloc if no_alloc else _load().f3d_batch_psh_scatter_pad_hash
+    _check(fn(
         _ptr(coord), _ptr(bucket_id), _ptr(bucket_counter), _ptr(bucket_offset), _ptr(batch_sep),
         _u32(batch_sep.shape[0]), _u32(coord.shape[0]), _u32(instance_max_N), _u32(num_bucket),
         _u32(bucket_divisor), _u32(bucket_size), _u32(num_vox), _ptr(bbox_min), _ptr(bbox_max),

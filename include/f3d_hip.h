@@ -82,6 +82,27 @@ int f3d_batch_psh_scatter_pad_hash(const f3d_half_t* coord, uint16_t* bucket_id,
                                    f3d_half_t* scatter_coord, uint32_t pad_to_n, float pad_num,
                                    uint32_t hash_type, int device, void* stream);
 
+/* The same op for callers that cannot allocate device memory: code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc.  No counterpart in the reference.  Same arguments, same results bit for bit; the
+ * tile histograms, first-hash counts and rebalance plan live in a fixed array of F3D_PSH_NOALLOC_SCRATCH_BYTES that
+ * every GPU the library runs on holds until the process ends, instead of the library's grow-only workspace.  The
+ * call makes no hipMalloc / hipFree and calls no allocating routine.  A batch that needs more scratch memory
+ * (about batch_size * tiles_per_cloud * num_bucket 32-bit words; 4 clouds x 250,000 points need 4.1 MB, 64 clouds x
+ * 262,144 points 4.7 MB) is rejected with F3D_ERR_UNSUPPORTED and a message.  The array's per-device
+ * address is looked up once per device: by f3d_init_dev_info(device), else by the first call on that device (call
+ * f3d_init_dev_info before a stream capture).  All calls on one GPU share the array, so calls that overlap on one
+ * GPU (two streams, two threads) race; calls ordered on one stream do not.  Nothing in it needs clearing between
+ * calls: every word a launch reads was written earlier in the same call. */
+#define F3D_PSH_NOALLOC_SCRATCH_BYTES (8u << 20)
+int f3d_batch_psh_scatter_pad_hash_noalloc(const f3d_half_t* coord, uint16_t* bucket_id, uint32_t* bucket_counter,
+                                           uint32_t* bucket_offset, const uint32_t* batch_sep, uint32_t batch_size,
+                                           uint32_t total_n, uint32_t instance_max_n, uint32_t num_bucket,
+                                           uint32_t bucket_divisor, uint32_t bucket_size, uint32_t num_vox,
+                                           const f3d_half_t* bbox_min, const f3d_half_t* bbox_max,
+                                           const int16_t* probe_offsets, uint32_t* cumsum_counter,
+                                           f3d_half_t* scatter_coord, uint32_t pad_to_n, float pad_num,
+                                           uint32_t hash_type, int device, void* stream);
+
 /* Overflow handling of the bucketing op (src/psh/batch_psh_bucket.cuh:154-246, 259-382).
  * 0 = hash + claim only (every point stays in its first-hash bucket);
  * 1 = deterministic probe rebalance + recycle (default). */

@@ -62,3 +62,25 @@ def test_psh_argument_errors_match_reference(lib):
     assert _psh_call(lib, hash_type=0) == 1
     # src/common/kernel_dispatcher.cuh:73-82
     assert _psh_call(lib, num_bucket=48, divisor=2048) == 2 and b"No kernel found" in lib.f3d_last_error()
+
+
+def test_no_alloc_psh_rejects_batches_beyond_its_scratch_array(lib):
+    """the entry point that allocates nothing says so when a batch does not fit its fixed scratch array
+    (argument validation: no GPU is touched)"""
+    u32, vp = ctypes.c_uint32, ctypes.c_void_p
+    dummy = vp(16)
+
+    def call(batch, per_cloud, nb):
+        div = -(-65535 // nb)
+        return lib.f3d_batch_psh_scatter_pad_hash_noalloc(
+            dummy, dummy, dummy, dummy, dummy, u32(batch), u32(batch * per_cloud), u32(per_cloud), u32(nb), u32(div),
+            u32(512), u32(0xFFFF), dummy, dummy, dummy, dummy, dummy, u32(batch * per_cloud), ctypes.c_float(0.0),
+            u32(1), ctypes.c_int(0), vp(0))
+    assert call(256, 262144, 512) == 2
+    msg = lib.f3d_last_error()
+    assert b"scratch" in msg and b"f3d_batch_psh_scatter_pad_hash" in msg
+    # the same argument errors as the allocating entry point come first
+    assert lib.f3d_batch_psh_scatter_pad_hash_noalloc(
+        dummy, dummy, dummy, dummy, dummy, u32(1), u32(512), u32(512), u32(64), u32(512), u32(512), u32(0xFFFF), dummy,
+        dummy, dummy, dummy, dummy, u32(512), ctypes.c_float(0.0), u32(1), ctypes.c_int(0), vp(0)) == 1
+    assert b"bucket divisor too small" in lib.f3d_last_error()
