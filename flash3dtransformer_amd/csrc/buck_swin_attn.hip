@@ -278,10 +278,21 @@ __global__ __launch_bounds__(kAttnThreads) void buck_swin_fwd_kernel(
 // Softmax without a running maximum (fast pass): Q is pre-multiplied by log2(e)/sqrt(D) (one bf16
 // rounding), so the score MFMA emits exponents and the VALU only exponentiates: P = 2^S with the
 // reference fixed at zero.  Softmax is shift-invariant and fp32 / bf16 share an 8-bit exponent, so this
-// is exact as long as the numbers stay in range; a wave whose step row sum reaches 2^24, or whose total
-// row sum stays under 2^-24 (scores that large also magnify the rounding of the pre-scaled Q), redoes
-// its item with the general pass: unscaled Q, scale applied in fp32, running maximum, masks.  Items with
-// masked or missing keys always take the general pass.
+// is exact as long as the numbers stay in range; a wave whose total row sum reaches 2^24 or stays under
+// 2^-24 (scores that large also magnify the rounding of the pre-scaled Q) redoes its item with the general
+// pass: unscaled Q, scale applied in fp32, running maximum.  Masked keys of a one-bucket scope are handled
+// inside the fast pass (steps past the valid length are skipped, the boundary step gets -inf scores);
+// scopes of several buckets of which some are partly valid take the general pass.
+// f(std::integral_constant<uint32_t, 0>) ... f(std::integral_constant<uint32_t, N - 1>): a loop whose counter is a
+// constant expression inside the body (immediate LDS offsets, statically indexed register arrays)
+template <uint32_t N, uint32_t I = 0, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+  if constexpr (I < N) {
+    f(std::integral_constant<uint32_t, I>{});
+    static_for<N, I + 1>(f);
+  }
+}
+
 constexpr int kResMaxScope = 4;  // buckets per scope: at most 512 tokens in buckets of at least 128
 typedef short i16x4_t __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) void lds_void_t;
@@ -448,19 +459,6 @@ __global__ __launch_bounds__(2 * T) __attribute__((amdgpu_waves_per_eu(4, 4))) v
     float l_run = 0.f;
     constexpr uint32_t NSTEP = T / 32, QSTEP = NSTEP / 4;
 
-    // scores of one step: S^T[key][query] = K Q'^T (already in the exponent's units)
-    auto qk = [&](uint32_t st) {
-      f32x16_t sacc;
-#pragma unroll
-      for (int i = 0; i < 16; ++i) sacc[i] = 0.f;
-      const char* kt = sbuf + st * 32u * ROWB;
-#pragma unroll
-      for (int ks = 0; ks < KSTEPS; ++ks) {
-        const bf16x8_t kf = *reinterpret_cast<const bf16x8_t*>(kt + (k_off ^ (ks * 32u)));
-        sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[ks], sacc, 0, 0, 0);
-      }
-      return sacc;
-    };
     // V^T operand of a step: slots 0..3 of a lane are keys 16kk + 4 half + 0..3, slots 4..7 the same + 8
     auto load_v = [&](uint32_t st, bf16x8_t (&vf)[2]) {
       const char* vt = sbuf + st * 32u * ROWB + v_off;
@@ -492,52 +490,70 @@ __global__ __launch_bounds__(2 * T) __attribute__((amdgpu_waves_per_eu(4, 4))) v
       }
     };
 
-    // ---- fast pass: every key valid, reference fixed at zero ----
-    // One step starts the score MFMAs of step st+1, exponentiates step st on the VALU while they run,
-    // then feeds P V^T of step st to the matrix core.  A row sum at or above 2^24 only raises
-    // `suspect`; the item is then redone by the general pass below.
-    bool suspect = false;
-    auto fast_step = [&](auto next_tag, f32x16_t& s_cur, f32x16_t& s_nxt, uint32_t st) {
-      if (decltype(next_tag)::value) s_nxt = qk(st + 1);
-      bf16x8_t vf[2];
-      load_v(st, vf);
-      uint32_t pb[8];
-      float psum;
-      exp_pack(s_cur, pb, psum);
-      suspect = suspect || !(psum < 0x1p24f);   // also catches inf / nan
-      l_run += psum;
-      pv(pb, vf);
+    // ---- fast pass: reference fixed at zero; one bucket per scope may be partly valid ----
+    // Fully unrolled over the steps of the scope (LDS offsets are immediates).  Step st issues the score MFMAs
+    // of step st+1 from K fragments that were read a step earlier, requests the K fragments of step st+2 and
+    // its own V fragments, exponentiates step st on the VALU while the matrix core runs, and ends with P V^T
+    // of step st.  `n_valid` steps hold valid keys (a prefix of the scope); in the last of them only the first
+    // `tail_keys` keys are valid and the others get a score of -inf (2^-inf = 0 exactly).  The row sum is
+    // chained through the dot2 accumulator; whether it left the safe range is looked at once per item.
+    auto load_k = [&](uint32_t st, bf16x8_t (&kf)[KSTEPS]) {
+      const char* kt = sbuf + st * 32u * ROWB;
+#pragma unroll
+      for (int ks = 0; ks < KSTEPS; ++ks) kf[ks] = *reinterpret_cast<const bf16x8_t*>(kt + (k_off ^ (ks * 32u)));
+    };
+    auto qk_from = [&](const bf16x8_t (&kf)[KSTEPS]) {
+      f32x16_t sacc;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) sacc[i] = 0.f;
+#pragma unroll
+      for (int ks = 0; ks < KSTEPS; ++ks) sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[ks], qf[ks], sacc, 0, 0, 0);
+      return sacc;
     };
     // The SIMD arbiter favours its oldest wave; left alone, that wave finishes its steps early and
     // idles at the barrier while the youngest runs the tail alone.  Each wave therefore lowers its own
     // priority as it advances (quarter by quarter), so a wave that is behind is served first.
-    auto quarter_prio = [&](uint32_t qd) {
-      switch (qd) {
-        case 0: __builtin_amdgcn_s_setprio(3); break;
-        case 1: __builtin_amdgcn_s_setprio(2); break;
-        case 2: __builtin_amdgcn_s_setprio(1); break;
-        default: __builtin_amdgcn_s_setprio(0); break;
-      }
-    };
-    auto fast_pass = [&]() {
+    auto fast_pass = [&](uint32_t n_valid, int32_t tail_keys) {
       m_ref = 0.f;
-      suspect = false;
       l_run = 0.f;
 #pragma unroll
       for (int i = 0; i < 16; ++i) acc[i] = 0.f;
-      f32x16_t s_a = qk(0), s_b;
+      bf16x8_t kf[2][KSTEPS];
+      load_k(0, kf[0]);
+      if (NSTEP > 1) load_k(1, kf[1]);
+      f32x16_t sc[2];
+      sc[0] = qk_from(kf[0]);
+      __builtin_amdgcn_s_setprio(3);
+      static_for<NSTEP>([&](auto st_c) {
+        constexpr uint32_t st = decltype(st_c)::value;
+        if (st < n_valid) {                 // uniform
+          if (st == QSTEP) __builtin_amdgcn_s_setprio(2);
+          if (st == 2 * QSTEP) __builtin_amdgcn_s_setprio(1);
+          if (st == 3 * QSTEP) __builtin_amdgcn_s_setprio(0);
+          f32x16_t& s_cur = sc[st & 1u];
+          if constexpr (st + 1 < NSTEP) sc[(st + 1) & 1u] = qk_from(kf[(st + 1) & 1u]);
+          if constexpr (st + 2 < NSTEP) load_k(st + 2, kf[st & 1u]);
+          bf16x8_t vf[2];
+          load_v(st, vf);
+          if (st + 1 == n_valid && tail_keys < 32) {
+            // (the empty asm keeps this a branch taken once per item instead of selects in every step)
+            asm volatile("; boundary step: mask the keys past the valid length");
+            // register i of a lane is key (i/4)*8 + 4 half + i%4 of the step
+            const int32_t thr = tail_keys - (int32_t)half * 4;
 #pragma unroll
-      for (int i = 0; i < 16; ++i) s_b[i] = 0.f;
-      for (uint32_t qd = 0; qd < 4; ++qd) {
-        quarter_prio(qd);
-        const uint32_t st_end = (qd + 1) * QSTEP - (qd == 3 ? 2 : 0);
-        for (uint32_t st = qd * QSTEP; st < st_end; st += 2) {
-          fast_step(std::true_type{}, s_a, s_b, st);
-          fast_step(std::true_type{}, s_b, s_a, st + 1);
+            for (int i = 0; i < 16; ++i)
+              if ((i / 4) * 8 + (i % 4) >= thr) s_cur[i] = -INFINITY;
+          }
+          uint32_t pb[8];
+#pragma unroll
+          for (int i = 0; i < 16; i += 2) {
+            pb[i / 2] = pack_bf16x2(__builtin_amdgcn_exp2f(s_cur[i]), __builtin_amdgcn_exp2f(s_cur[i + 1]));
+            l_run = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, pb[i / 2]),
+                                                    __builtin_bit_cast(bf16x2_t, 0x3F803F80u), l_run, false);
+          }
+          pv(pb, vf);
         }
-      }
-      fast_step(std::true_type{}, s_a, s_b, NSTEP - 2);
-      fast_step(std::false_type{}, s_b, s_a, NSTEP - 1);
+      });
       __builtin_amdgcn_s_setprio(3);
     };
 
@@ -603,13 +619,19 @@ __global__ __launch_bounds__(2 * T) __attribute__((amdgpu_waves_per_eu(4, 4))) v
     const bool any_valid = blen0 > 0 || blen1 > 0 || blen2 > 0 || blen3 > 0;
     const bool all_full = blen0 == (int32_t)bs && (scope_size < 2 || blen1 == (int32_t)bs) &&
                           (scope_size < 3 || blen2 == (int32_t)bs) && (scope_size < 4 || blen3 == (int32_t)bs);
-    if (q_exists && any_valid) {
-      bool redo = !all_full;
-      if (all_full) {
-        fast_pass();
-        // redo with a moving reference if any row sum left the safe range
+    // queries at or beyond the valid length of their bucket produce zeros: a wave that owns only such rows has
+    // nothing to compute (uniform per wave)
+    const bool wave_has_rows = (int32_t)(q_local - qj * bs) < q_valid_len;
+    if (q_exists && any_valid && wave_has_rows) {
+      // the fast pass takes scopes whose keys are all valid, and one-bucket scopes with a valid prefix
+      bool redo = !(all_full || scope_size == 1);
+      if (!redo) {
+        const uint32_t n_valid = all_full ? NSTEP : (uint32_t)(blen0 + 31) / 32u;
+        const int32_t tail_keys = all_full ? 32 : blen0 - (int32_t)(n_valid - 1) * 32;
+        fast_pass(n_valid, tail_keys);
+        // redo with a moving reference if any row sum left the safe range (also catches inf / nan)
         const float l_chk = l_run + __shfl_xor(l_run, 32, kWave);
-        redo = __ballot(suspect || !(l_chk > 0x1p-24f)) != 0;
+        redo = __ballot(!(l_chk > 0x1p-24f) || !(l_chk < 0x1p24f)) != 0;
       }
       if (redo) general_pass();
     } else {

@@ -33,8 +33,16 @@ def sources():
     return sorted(f for f in os.listdir(HERE) if f.endswith(".hip"))
 
 
-def _compile(src):
+def _newest_header():
+    return max(os.path.getmtime(os.path.join(d, f)) for d in (HERE, os.path.join(os.path.dirname(PKG), "include"))
+               for f in os.listdir(d) if f.endswith(".h"))
+
+
+def _compile(src, incremental=False):
     obj = os.path.join(OBJ_DIR, src.replace(".hip", ".o"))
+    if incremental and os.path.exists(obj) and os.path.getmtime(obj) > max(
+            os.path.getmtime(os.path.join(HERE, src)), _newest_header(), os.path.getmtime(__file__)):
+        return obj
     cmd = ["hipcc", "-c", os.path.join(HERE, src), "-o", obj] + COMMON
     cmd += ["-ffp-contract=off"] if src in EXACT else ["-ffp-contract=fast"]
     if src not in NO_VGPR_FORM:
@@ -48,13 +56,15 @@ def _compile(src):
     return obj
 
 
-def build(verbose=True, jobs=None):
+def build(verbose=True, jobs=None, incremental=False):
+    """incremental=True keeps objects that are newer than their source, every header and this file (a developer's
+    shortcut: `python -m flash3dtransformer_amd.csrc.build -i`); the default compiles everything."""
     os.makedirs(OBJ_DIR, exist_ok=True)
     os.makedirs(os.path.dirname(LIB), exist_ok=True)
     srcs = sources()
     jobs = jobs or min(len(srcs), int(os.environ.get("MAX_JOBS", "8")))
     with ThreadPoolExecutor(max_workers=jobs) as ex:
-        objs = list(ex.map(_compile, srcs))
+        objs = list(ex.map(lambda f: _compile(f, incremental), srcs))
     cmd = ["hipcc", "-shared", "-fPIC", "--offload-arch=gfx950", "-fno-gpu-rdc", "-o", LIB] + objs
     p = subprocess.run(cmd, capture_output=True, text=True)
     if p.returncode != 0:
@@ -65,4 +75,4 @@ def build(verbose=True, jobs=None):
 
 
 if __name__ == "__main__":
-    build()
+    build(incremental="-i" in sys.argv[1:])
