@@ -5,8 +5,8 @@
 // batch row, every scope (a row of scope_buckets) and every head: softmax(Q Kt / sqrt(D)) V over the
 // rows of the scope's buckets, plus the natural-log LSE.
 //
-// Kernel shape: one 256-thread workgroup (4 waves) per (batch, scope, head, 128-query block); each
-// wave owns 32 query rows.  K and V of the scope stream through LDS in tiles of KT keys (K row-major,
+// Streaming kernel (any scope size, head_dim up to 128): one 256-thread workgroup (4 waves) per (batch, scope,
+// head, 128-query block); each wave owns 32 query rows.  K and V of the scope stream through LDS in tiles of KT keys (K row-major,
 // V transposed), prefetched into registers one tile ahead.  Scores are computed TRANSPOSED,
 // St = K Qt with v_mfma_f32_32x32x16_bf16, so that a lane holds 16 keys of ONE query: the softmax
 // max / sum run inside the lane plus one exchange with lane^32, and the bf16 P values are already in
@@ -259,30 +259,6 @@ __global__ __launch_bounds__(kAttnThreads) void buck_swin_fwd_kernel(
   }
 }
 
-// ---- resident variant ---------------------------------------------------------------------------
-// When a scope holds 256 or 512 tokens and head_dim <= 32 (the shape of every block of the Flash3D
-// model: one 512-row bucket per scope, 32-wide heads) the K and V of a (scope, head) fit in LDS
-// twice.  One persistent workgroup walks a list of (batch, scope, head) items: wave w owns the scope's
-// query rows [32w, 32w+32) and runs them against all key tiles without any barrier, while the NEXT
-// item's K / V stream from HBM straight into the other LDS buffer (global_load ... lds, no registers)
-// and its Q into eight registers.  One barrier per item.
-//
-// LDS layout of one buffer: K [T][D] then V [T][D], both row-major exactly as the direct loads write
-// them (a wave's 64 lanes fill 1 KB = 1024/(2D) consecutive rows).  K rows carry no padding: the
-// 16-byte chunk c of row r is stored at position c ^ swz(r), swz(r) = (r / (128/D)) mod (D/8), which
-// spreads the 32 rows of a ds_read_b128 over all banks.  V is read with ds_read_b64_tr_b16, which hands
-// lane i of a 16-lane block column i%4 of the four 8-byte pieces addressed by lanes i/4 + {0,4,8,12}:
-// with lane r pointing at key r/4, features 4(r%4).., a lane receives one feature of four consecutive
-// keys, i.e. the MFMA A operand of V^T, with no transposed copy of V anywhere.
-//
-// Softmax without a running maximum (fast pass): Q is pre-multiplied by log2(e)/sqrt(D) (one bf16
-// rounding), so the score MFMA emits exponents and the VALU only exponentiates: P = 2^S with the
-// reference fixed at zero.  Softmax is shift-invariant and fp32 / bf16 share an 8-bit exponent, so this
-// is exact as long as the numbers stay in range; a wave whose total row sum reaches 2^24 or stays under
-// 2^-24 (scores that large also magnify the rounding of the pre-scaled Q) redoes its item with the general
-// pass: unscaled Q, scale applied in fp32, running maximum.  Masked keys of a one-bucket scope are handled
-// inside the fast pass (steps past the valid length are skipped, the boundary step gets -inf scores);
-// scopes of several buckets of which some are partly valid take the general pass.
 // f(std::integral_constant<uint32_t, 0>) ... f(std::integral_constant<uint32_t, N - 1>): a loop whose counter is a
 // constant expression inside the body (immediate LDS offsets, statically indexed register arrays)
 template <uint32_t N, uint32_t I = 0, class F>
@@ -295,6 +271,7 @@ __device__ __forceinline__ void static_for(F&& f) {
 
 constexpr int kResMaxScope = 4;  // buckets per scope: at most 512 tokens in buckets of at least 128
 typedef short i16x4_t __attribute__((ext_vector_type(4)));
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
 typedef __attribute__((address_space(3))) void lds_void_t;
 typedef __attribute__((address_space(3))) i16x4_t lds_i16x4_t;
 
@@ -309,34 +286,69 @@ __device__ __forceinline__ void lds_dma16(const void* gbase, uint32_t voff, cons
                : "memory", "m0");
 }
 
-template <int D, int T>
-constexpr size_t resident_lds_bytes() {
-  return 2 * (size_t)2 * T * D * 2 + 3 * kResMaxScope * 8;
+// ---- scope-resident kernel --------------------------------------------------------------------------
+// When a scope holds 256 or 512 tokens and head_dim <= 32 (the shape of every block of the Flash3D model: one
+// 512-row bucket per scope, 32-wide heads) the K and V of a (batch, scope, head) item fit in LDS twice.  One
+// persistent workgroup of WAVES waves walks a list of items: the current item's K and V sit in one LDS buffer
+// (2 T D bytes each) while the next item's stream HBM -> LDS directly (global_load ... lds, no registers) into the
+// other and its Q into registers; one barrier per item.  A wave owns QB = T / (32 WAVES) blocks of 32 queries
+// (one with the T / 32 waves the launcher picks: four waves per SIMD at under 128 registers, nothing spills, so no
+// scratch reload ever waits behind the direct loads in flight) and walks the flattened sequence (step, block):
+// every K / V fragment read from LDS feeds all of its blocks.
+//
+// LDS layout of one buffer: K [T][D] then V [T][D], both row-major exactly as the direct loads write them (a
+// wave's 64 lanes fill 1 KB = 1024/(2D) consecutive rows).  K rows carry no padding: the 16-byte chunk c of row r
+// is stored at position c ^ swz(r), swz(r) = (r / (128/D)) mod (D/8), which spreads the 32 rows of a ds_read_b128
+// over all banks.  V is read with ds_read_b64_tr_b16, which hands lane i of a 16-lane block column i%4 of the four
+// 8-byte pieces addressed by lanes i/4 + {0,4,8,12}: with lane r pointing at key r/4, features 4(r%4).., a lane
+// receives one feature of four consecutive keys, i.e. the MFMA A operand of V^T, with no transposed copy of V
+// anywhere.  Scores are computed transposed (S^T = K Q^T, a lane holds 16 keys of one query), so the packed P
+// values already are the B operand of O^T += V^T P^T.
+//
+// Softmax without a running maximum (fast pass): Q is pre-multiplied by log2(e)/sqrt(D) (one bf16 rounding), so
+// the score MFMA emits exponents and the VALU only exponentiates and packs: P = 2^S with the reference fixed at
+// zero.  Softmax is shift-invariant and fp32 / bf16 share an 8-bit exponent, so this is exact as long as the
+// numbers stay in range; a wave whose total row sum reaches 2^24 or stays under 2^-24 (scores that large also
+// magnify the rounding of the pre-scaled Q) redoes its item with the general pass: unscaled Q, scale applied in
+// fp32, running maximum.  Masked keys of a one-bucket scope are handled inside the fast pass (steps past the
+// valid length are skipped, the boundary step gets -inf scores, 2^-inf = 0 exactly); scopes of several buckets of
+// which some are partly valid take the general pass.
+//
+// What bounds the pass is the vector unit's issue port: per 32 x 32 scores a wave issues 16 v_exp_f32 (two slots
+// each), 8 v_cvt_pk_bf16_f32 and six MFMAs (each holds the port for about ten clocks), some 240 clocks against
+// 160 clocks of matrix-core time.  Hence: the scores of the next (step, block) are issued before the
+// exponentials of the current one, so that the matrix core works under them; the row sums come from the matrix
+// core too (one 16x16x32 product of P with a 0 / 1 selector per 16 keys, a quarter of a score product, instead
+// of eight dot instructions on the vector unit); the steps are fully unrolled (LDS offsets are immediates, no
+// address arithmetic); the next item's loads are issued a few per step (all at once they hold every wave at the
+// memory pipeline's door for a microsecond with the SIMDs idle).
+template <int D, int T, int WAVES>
+constexpr size_t scope_lds_bytes() {
+  return (size_t)2 * 2 * T * D * 2;
 }
 
-template <int D, int T>
-__global__ __launch_bounds__(2 * T) __attribute__((amdgpu_waves_per_eu(4, 4))) void buck_swin_fwd_resident_kernel(
+template <int D, int T, int WAVES>
+__global__ __launch_bounds__(64 * WAVES) void buck_swin_fwd_scope_kernel(
     const uint16_t* __restrict__ q, const uint16_t* __restrict__ k, const uint16_t* __restrict__ v, uint32_t ld,
     uint16_t* __restrict__ o, float* __restrict__ lse, const uint32_t* __restrict__ scope_buckets,
     uint32_t num_scope, uint32_t scope_size, uint32_t bs, uint32_t seq_len, uint32_t num_head,
     const int32_t* __restrict__ kv_len, float scale_log2, uint32_t n_items, uint32_t items_per_xcd,
     uint32_t n_slots) {
-  constexpr int KT = 64;
+  constexpr int QB = T / (32 * WAVES);     // 32-query blocks per wave
   constexpr int KSTEPS = D / 16;
-  constexpr int NSUB = KT / 32;
   constexpr int CPK = D / 8;               // 16-byte chunks per row
   constexpr int ROWB = D * 2;              // bytes per K / V row in LDS
   constexpr int RPB = 1024 / ROWB;         // rows one direct-load instruction fills
-  constexpr int BLK_PER_WAVE = 32 / RPB;   // wave w fills the rows [32w, 32w+32) of K and of V
+  constexpr int BPW = T / RPB / WAVES;     // direct-load instructions per wave and operand
   constexpr int SWZ_DIV = 16 / CPK;        // rows sharing one swizzle value
   constexpr int OPB = T * ROWB;            // bytes of one operand (K or V)
   constexpr int BUF = 2 * OPB;             // bytes of one K + V buffer
-  constexpr int N_TILES = T / KT;
-  extern __shared__ __attribute__((aligned(16))) char lds_res[];
-  uint32_t (*s_bucket)[kResMaxScope] = reinterpret_cast<uint32_t (*)[kResMaxScope]>(lds_res + 2 * BUF);
-  int32_t (*s_len)[kResMaxScope] = reinterpret_cast<int32_t (*)[kResMaxScope]>(lds_res + 2 * BUF + 3 * kResMaxScope * 4);
+  constexpr uint32_t NSTEP = T / 32;
+  static_assert(QB >= 1 && BPW >= 1 && (T / WAVES) % 32 == 0 && (T / WAVES) % RPB == 0, "a wave owns whole 32-query blocks and whole direct-load blocks");
+  extern __shared__ __attribute__((aligned(16))) char lds_scope[];
 
-  const uint32_t tid = threadIdx.x, wave = tid / kWave, lane = tid % kWave;
+  const uint32_t tid = threadIdx.x, lane = tid % kWave;
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(tid / kWave);
   const uint32_t lq = lane & 31u, half = lane >> 5;
   const uint32_t n_bucket = seq_len / bs;
   const uint32_t xcd = blockIdx.x % kNumXcd, slot = blockIdx.x / kNumXcd;
@@ -345,120 +357,174 @@ __global__ __launch_bounds__(2 * T) __attribute__((amdgpu_waves_per_eu(4, 4))) v
   if (item_lo >= item_hi) return;        // whole workgroup: no barrier has been passed yet
   const uint32_t my_items = (item_hi - item_lo + n_slots - 1) / n_slots;
 
-  // item -> (batch, scope, head); the element offset of (first token of the batch, head) is uniform, the
-  // per-thread part (row inside the sequence, chunk) fits 32 bits (checked by the host)
-  auto item_scope = [&](uint32_t it) { return (it / num_head) % num_scope; };
-  auto item_base = [&](uint32_t it) {
-    return (size_t)(it / (num_head * num_scope)) * seq_len * ld + (size_t)(it % num_head) * D;
-  };
-
-  // bucket ids / valid lengths of one item's scope, handled by the first scope_size threads
-  uint32_t tb = 0;
-  int32_t tl = 0;
-  auto load_table_ids = [&](uint32_t it) {
-    if (tid < scope_size) tb = scope_buckets[(size_t)item_scope(it) * scope_size + tid];
-  };
-  auto load_table_len = [&]() {
-    if (tid < scope_size) tl = tb >= n_bucket ? 0 : (kv_len ? min(max(kv_len[tb], 0), (int32_t)bs) : (int32_t)bs);
-  };
-  auto store_table = [&](uint32_t tslot) {
-    if (tid < scope_size) {
-      s_bucket[tslot][tid] = tb;
-      s_len[tslot][tid] = tl;
-    }
-  };
-
-  // direct HBM -> LDS loads of one item's K and V rows [32 wave, 32 wave + 32)
-  auto issue_kv = [&](uint32_t it, uint32_t tslot, char* buf) {
-    const size_t base = item_base(it);
-#pragma unroll
-    for (int i = 0; i < BLK_PER_WAVE; ++i) {
-      const uint32_t blk = __builtin_amdgcn_readfirstlane(wave * BLK_PER_WAVE + i);
-      const uint32_t row = blk * RPB + lane / CPK, pos = lane % CPK;
-      const uint32_t j = (blk * RPB) / bs;               // uniform: a block never straddles buckets
-      if (s_len[tslot][j] > 0) {
-        const uint32_t rowoff = ((s_bucket[tslot][j] * bs + (row - j * bs)) * ld) * 2u;
-        const uint32_t ck = pos ^ ((row / SWZ_DIV) & (CPK - 1));
-        // Issued as inline assembly on purpose: the compiler then keeps no record of LDS writes in
-        // flight and does not put a full vmcnt wait in front of the tile loop's LDS reads (they read the
-        // OTHER buffer).  The wait that matters is the explicit one before the per-item barrier.
-        lds_dma16(k + base, rowoff + ck * 16u, buf + blk * 1024);
-        lds_dma16(v + base, rowoff + pos * 16u, buf + OPB + blk * 1024);
-      }
-    }
-  };
-  // this wave's 32 query rows sit at scope-local rows [32 wave, 32 wave + 32)
-  const uint32_t q_local = wave * 32;
-  const uint32_t qj = q_local / bs;
-  const uint32_t q_in_bucket = (q_local - qj * bs) + lq;
-  u32x4_t qraw[KSTEPS];
-  auto issue_q = [&](uint32_t it, uint32_t tslot) {
-    const uint32_t qb = s_bucket[tslot][qj];
-    const uint32_t off = (((qb < n_bucket ? qb : 0u) * bs + q_in_bucket) * ld + half * 8) * 2u;
-    const char* qp = reinterpret_cast<const char*>(q + item_base(it));
-#pragma unroll
-    for (int ks = 0; ks < KSTEPS; ++ks) qraw[ks] = *reinterpret_cast<const u32x4_t*>(qp + (off + ks * 32u));
-  };
-
-  // ---- prologue: tables of the first two items, K / V / Q of the first ----
-  load_table_ids(item_lo);
-  load_table_len();
-  store_table(0);
-  if (my_items > 1) {
-    load_table_ids(item_lo + n_slots);
-    load_table_len();
-    store_table(1);
-  }
-  __syncthreads();
-  issue_q(item_lo, 0);
-  issue_kv(item_lo, 0, lds_res);
-  __builtin_amdgcn_s_waitcnt(0);
-  __syncthreads();
-
-  // per-lane LDS byte offsets inside a buffer
+  // per-lane LDS byte offsets of the fragment reads
   const uint32_t k_off = lq * ROWB + ((half ^ ((lq / SWZ_DIV) & (CPK - 1))) * 16u);   // k-step ks: ^ (ks * 32)
   const uint32_t l16 = lane & 15u, d_base = 16u * ((lane >> 4) & 1u);
   const uint32_t v_off = OPB + (4u * half + l16 / 4u) * ROWB + (d_base + 4u * (l16 & 3u)) * 2u;
   const bool v_lane = D >= 32 || d_base < (uint32_t)D;   // lanes whose V^T row exists
+  // per-lane byte offsets of the direct loads inside a block of RPB rows: lane l fills LDS bytes [16 l, 16 l + 16)
+  // of the block, i.e. row l / CPK, chunk l % CPK; for K that chunk holds the row's chunk (l % CPK) ^ swizzle(row)
+  const uint32_t dma_row = lane / CPK, dma_pos = lane % CPK;
+  const uint32_t dma_k = (dma_row * ld + (dma_pos ^ ((dma_row / SWZ_DIV) & (CPK - 1))) * 8u) * 2u;
+  const uint32_t dma_v = (dma_row * ld + dma_pos * 8u) * 2u;
+  // Row-sum selector, the A operand of a 16x16x32 product whose B operand is a P fragment in the layout of the
+  // 32x32x16 product (lane = query lane % 32, keys 8 (lane / 32) ..): as a 16x16x32 operand the fragment's lane is
+  // (column lane % 16, k-block lane / 16), so even k-blocks hold queries 0-15 and odd ones queries 16-31.  Rows
+  // 0-7 of the selector take the even k-blocks, rows 8-15 the odd ones: lanes 0-31 of the result hold the row sums
+  // of queries 0-15 (lane % 16), lanes 32-63 those of queries 16-31, every register the same number.
+  bf16x8_t ones_sel;
+  {
+    const uint32_t m = lane & 15u, kb = lane >> 4;
+    const __bf16 val = ((m < 8u) == ((kb & 1u) == 0u)) ? (__bf16)1.0f : (__bf16)0.0f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) ones_sel[e] = val;
+  }
+  const uint32_t l_src = (lq < 16u ? 0u : 32u) + (lq & 15u);
+
+  // ---- item -> (batch, scope, head) and the scope's bucket ids / valid key counts ----
+  // Lane j < scope_size of every wave reads bucket j of an item's scope (two dependent loads, issued long before
+  // their use); the consumer broadcasts them into scalars.
+  auto item_base = [&](uint32_t it) {     // element offset of (first token of the batch element, head), uniform
+    return (size_t)(it / (num_head * num_scope)) * seq_len * ld + (size_t)(it % num_head) * D;
+  };
+  auto load_ids = [&](uint32_t it) -> uint32_t {
+    return lane < scope_size ? scope_buckets[(size_t)((it / num_head) % num_scope) * scope_size + lane] : 0xFFFFFFFFu;
+  };
+  auto load_len = [&](uint32_t ids) -> int32_t {
+    return ids >= n_bucket ? 0 : (kv_len ? min(max(kv_len[ids], 0), (int32_t)bs) : (int32_t)bs);
+  };
+  struct Scope {
+    uint32_t bkt[kResMaxScope];
+    int32_t len[kResMaxScope];
+  };
+  auto broadcast = [&](uint32_t ids, int32_t lens) {
+    Scope sc;
+#pragma unroll
+    for (int j = 0; j < kResMaxScope; ++j) {
+      sc.bkt[j] = __builtin_amdgcn_readlane(ids, j);
+      sc.len[j] = __builtin_amdgcn_readlane(lens, j);
+    }
+    return sc;
+  };
+  auto bucket_of = [&](const Scope& sc, uint32_t j) { return j == 0 ? sc.bkt[0] : j == 1 ? sc.bkt[1] : j == 2 ? sc.bkt[2] : sc.bkt[3]; };
+  auto len_of = [&](const Scope& sc, uint32_t j) { return j == 0 ? sc.len[0] : j == 1 ? sc.len[1] : j == 2 ? sc.len[2] : sc.len[3]; };
+
+  // K and V rows [wave T/WAVES, (wave + 1) T/WAVES) of an item go straight into an LDS buffer, 2 BPW direct loads of
+  // 1 KB per wave: load i < BPW is K block i of the wave, load BPW + i its V block i.  kv_base() is the byte offset of
+  // the wave's first row (valid when kv_wanted()).  Issued as inline assembly on purpose: the compiler then keeps no
+  // record of LDS writes in flight and puts no full vmcnt wait in front of the fragment reads (they read the OTHER
+  // buffer).  The wait that matters is the explicit one before the per-item barrier.
+  const uint32_t kv_row0 = wave * (T / WAVES), kv_j = kv_row0 / bs;     // a wave's rows never straddle buckets
+  auto kv_wanted = [&](const Scope& sc) { return len_of(sc, kv_j) > 0; };
+  auto kv_base = [&](uint32_t it, const Scope& sc) {
+    return item_base(it) * 2u + (size_t)(bucket_of(sc, kv_j) * bs + (kv_row0 - kv_j * bs)) * ld * 2u;
+  };
+  auto issue_kv_one = [&](size_t goff, uint32_t i, char* buf) {
+    const uint32_t blk = wave * BPW + (i < (uint32_t)BPW ? i : i - BPW);
+    const size_t g = goff + (size_t)(i < (uint32_t)BPW ? i : i - BPW) * RPB * ld * 2u;
+    if (i < (uint32_t)BPW) lds_dma16(reinterpret_cast<const char*>(k) + g, dma_k, buf + blk * 1024);
+    else lds_dma16(reinterpret_cast<const char*>(v) + g, dma_v, buf + OPB + blk * 1024);
+  };
+  // row inside the sequence of query lq of block b (0 when the scope entry names no bucket of the sequence)
+  auto q_row_of = [&](const Scope& sc, uint32_t b) {
+    const uint32_t q_local = (wave * QB + b) * 32u, qj = q_local / bs, id = bucket_of(sc, qj);
+    return (id < n_bucket ? id : 0u) * bs + (q_local - qj * bs) + lq;
+  };
+  u32x4_t qraw[QB][KSTEPS];
+  auto issue_q_one = [&](uint32_t it, const Scope& sc, auto b_c) {
+    constexpr uint32_t b = decltype(b_c)::value;
+    const char* qp = reinterpret_cast<const char*>(q + item_base(it));
+    const uint32_t off = (q_row_of(sc, b) * ld + half * 8u) * 2u;      // fits 32 bits (checked by the host)
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) qraw[b][ks] = *reinterpret_cast<const u32x4_t*>(qp + (off + ks * 32u));
+  };
+
+  // ---- prologue: the first item's scope, K / V / Q; the second item's bucket ids ----
+  Scope cur;
+  {
+    const uint32_t ids = load_ids(item_lo);
+    cur = broadcast(ids, load_len(ids));
+  }
+  uint32_t nxt_ids = my_items > 1 ? load_ids(item_lo + n_slots) : 0xFFFFFFFFu;
+  int32_t nxt_len = load_len(nxt_ids);
+  static_for<QB>([&](auto b_c) { issue_q_one(item_lo, cur, b_c); });
+  if (kv_wanted(cur)) {
+    const size_t goff = kv_base(item_lo, cur);
+#pragma unroll
+    for (uint32_t i = 0; i < 2u * BPW; ++i) issue_kv_one(goff, i, lds_scope);
+  }
+  __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
+  __syncthreads();
 
   for (uint32_t n = 0; n < my_items; ++n) {
     const uint32_t item = item_lo + n * n_slots;
-    const uint32_t tcur = n % 3, tnext = (n + 1) % 3, tnext2 = (n + 2) % 3;
     const bool has_next = n + 1 < my_items;
-    const char* sbuf = lds_res + (n & 1u) * BUF;
-    const uint32_t q_bucket = s_bucket[tcur][qj];
-    const bool q_exists = q_bucket < n_bucket;             // uniform per wave
-    const uint32_t q_row = (q_exists ? q_bucket : 0u) * bs + q_in_bucket;
-    const int32_t q_valid_len = s_len[tcur][qj];
+    const char* const sbuf = lds_scope + (n & 1u) * BUF;
 
-    // Q of this item arrived during the previous one: scale and round once
-    bf16x8_t qf[KSTEPS];
+    // Q of this item arrived during the previous one: scale into the exponent's units and round once
+    bf16x8_t qf[QB][KSTEPS];
 #pragma unroll
-    for (int ks = 0; ks < KSTEPS; ++ks) {
-      u32x4_t sc;
+    for (int b = 0; b < QB; ++b)
 #pragma unroll
-      for (int e = 0; e < 4; ++e)
-        sc[e] = pack_bf16x2(bf16_lo(qraw[ks][e]) * scale_log2, bf16_hi(qraw[ks][e]) * scale_log2);
-      qf[ks] = __builtin_bit_cast(bf16x8_t, sc);
-    }
-    // put the next item's operands in flight
-    if (has_next) {
-      issue_q(item + n_slots, tnext);
-      issue_kv(item + n_slots, tnext, lds_res + ((n + 1) & 1u) * BUF);
-    }
-    if (n + 2 < my_items) load_table_ids(item + 2 * n_slots);
-    // valid key counts of the (at most four) buckets of this scope, as wave-uniform scalars
-    static_assert(kResMaxScope == 4, "four bucket lengths are kept in scalars");
-    const int32_t blen0 = __builtin_amdgcn_readfirstlane(s_len[tcur][0]);
-    const int32_t blen1 = __builtin_amdgcn_readfirstlane(scope_size > 1 ? s_len[tcur][1] : 0);
-    const int32_t blen2 = __builtin_amdgcn_readfirstlane(scope_size > 2 ? s_len[tcur][2] : 0);
-    const int32_t blen3 = __builtin_amdgcn_readfirstlane(scope_size > 3 ? s_len[tcur][3] : 0);
+      for (int ks = 0; ks < KSTEPS; ++ks) {
+        u32x4_t sc;
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          sc[e] = pack_bf16x2(bf16_lo(qraw[b][ks][e]) * scale_log2, bf16_hi(qraw[b][ks][e]) * scale_log2);
+        qf[b][ks] = __builtin_bit_cast(bf16x8_t, sc);
+      }
+    // The next item's operands go in flight during the first half of this item's passes, a few vector-memory
+    // instructions per step (issued all at once they would hold every wave of the workgroup at the memory pipeline's door for a
+    // microsecond or two with the SIMDs idle): `vm_next` counts those already issued, 2 BPW direct loads of K / V
+    // first, then the Q rows of the wave's QB blocks.
+    Scope nxt = broadcast(nxt_ids, nxt_len);
+    constexpr uint32_t VM_OPS = 2u * BPW + QB, VM_PER_STEP = (VM_OPS + NSTEP / 2 - 1) / (NSTEP / 2);   // all in the first half
+    const bool nxt_kv = has_next && kv_wanted(nxt);
+    const size_t nxt_goff = nxt_kv ? kv_base(item + n_slots, nxt) : 0;
+    char* const nxt_buf = lds_scope + ((n + 1) & 1u) * BUF;
+    auto issue_vm = [&](auto i_c) {
+      constexpr uint32_t i = decltype(i_c)::value;
+      if constexpr (i < 2u * BPW) {
+        if (nxt_kv) issue_kv_one(nxt_goff, i, nxt_buf);
+      } else if constexpr (i < VM_OPS) {
+        if (has_next) issue_q_one(item + n_slots, nxt, std::integral_constant<uint32_t, i - 2u * BPW>{});
+      }
+    };
+    uint32_t vm_next = 0;
+    nxt_ids = n + 2 < my_items ? load_ids(item + 2 * n_slots) : 0xFFFFFFFFu;
 
-    float m_ref = 0.f;        // reference subtracted from the scaled scores
-    f32x16_t acc;
-    float l_run = 0.f;
-    constexpr uint32_t NSTEP = T / 32, QSTEP = NSTEP / 4;
+    // per block: do its rows exist / are they valid (uniform), how many of them, which rows
+    uint32_t q_row[QB];
+    bool q_live[QB], q_exists[QB];
+    int32_t q_len[QB];
+#pragma unroll
+    for (int b = 0; b < QB; ++b) {
+      const uint32_t q_local = (wave * QB + b) * 32u, qj = q_local / bs;
+      const int32_t in_b = (int32_t)(q_local - qj * bs);
+      q_exists[b] = bucket_of(cur, qj) < n_bucket;
+      q_len[b] = len_of(cur, qj) - in_b;               // valid rows of the block, counted from its first row
+      q_live[b] = q_exists[b] && q_len[b] > 0;
+      q_row[b] = q_row_of(cur, b);
+    }
 
+    f32x16_t acc[QB];
+    f32x4_t lacc[QB];
+    float m_ref[QB], l_fin[QB];
+#pragma unroll
+    for (int b = 0; b < QB; ++b) {
+      m_ref[b] = 0.f;
+      l_fin[b] = 0.f;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) lacc[b][i] = 0.f;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[b][i] = 0.f;
+    }
+
+    auto load_k = [&](uint32_t st, bf16x8_t (&kf)[KSTEPS]) {
+      const char* kt = sbuf + st * 32u * ROWB;
+#pragma unroll
+      for (int ks = 0; ks < KSTEPS; ++ks) kf[ks] = *reinterpret_cast<const bf16x8_t*>(kt + (k_off ^ (ks * 32u)));
+    };
     // V^T operand of a step: slots 0..3 of a lane are keys 16kk + 4 half + 0..3, slots 4..7 the same + 8
     auto load_v = [&](uint32_t st, bf16x8_t (&vf)[2]) {
       const char* vt = sbuf + st * 32u * ROWB + v_off;
@@ -472,213 +538,221 @@ __global__ __launch_bounds__(2 * T) __attribute__((amdgpu_waves_per_eu(4, 4))) v
         vf[kk] = __builtin_bit_cast(bf16x8_t, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
       }
     };
-    // P = 2^S as bf16 pairs, row sum from the rounded values
-    auto exp_pack = [&](const f32x16_t& sc, uint32_t (&pb)[8], float& psum) {
-      psum = 0.f;
-#pragma unroll
-      for (int i = 0; i < 16; i += 2) {
-        pb[i / 2] = pack_bf16x2(__builtin_amdgcn_exp2f(sc[i]), __builtin_amdgcn_exp2f(sc[i + 1]));
-        psum = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, pb[i / 2]),
-                                               __builtin_bit_cast(bf16x2_t, 0x3F803F80u), psum, false);
-      }
-    };
-    auto pv = [&](const uint32_t (&pb)[8], const bf16x8_t (&vf)[2]) {
-#pragma unroll
-      for (int kk = 0; kk < 2; ++kk) {
-        const u32x4_t praw = {pb[kk * 4 + 0], pb[kk * 4 + 1], pb[kk * 4 + 2], pb[kk * 4 + 3]};
-        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[kk], __builtin_bit_cast(bf16x8_t, praw), acc, 0, 0, 0);
-      }
-    };
-
-    // ---- fast pass: reference fixed at zero; one bucket per scope may be partly valid ----
-    // Fully unrolled over the steps of the scope (LDS offsets are immediates).  Step st issues the score MFMAs
-    // of step st+1 from K fragments that were read a step earlier, requests the K fragments of step st+2 and
-    // its own V fragments, exponentiates step st on the VALU while the matrix core runs, and ends with P V^T
-    // of step st.  `n_valid` steps hold valid keys (a prefix of the scope); in the last of them only the first
-    // `tail_keys` keys are valid and the others get a score of -inf (2^-inf = 0 exactly).  The row sum is
-    // chained through the dot2 accumulator; whether it left the safe range is looked at once per item.
-    auto load_k = [&](uint32_t st, bf16x8_t (&kf)[KSTEPS]) {
-      const char* kt = sbuf + st * 32u * ROWB;
-#pragma unroll
-      for (int ks = 0; ks < KSTEPS; ++ks) kf[ks] = *reinterpret_cast<const bf16x8_t*>(kt + (k_off ^ (ks * 32u)));
-    };
-    auto qk_from = [&](const bf16x8_t (&kf)[KSTEPS]) {
+    auto scores = [&](const bf16x8_t (&kf)[KSTEPS], const bf16x8_t (&qq)[KSTEPS]) {
       f32x16_t sacc;
 #pragma unroll
       for (int i = 0; i < 16; ++i) sacc[i] = 0.f;
 #pragma unroll
-      for (int ks = 0; ks < KSTEPS; ++ks) sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[ks], qf[ks], sacc, 0, 0, 0);
+      for (int ks = 0; ks < KSTEPS; ++ks) sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[ks], qq[ks], sacc, 0, 0, 0);
       return sacc;
     };
-    // The SIMD arbiter favours its oldest wave; left alone, that wave finishes its steps early and
-    // idles at the barrier while the youngest runs the tail alone.  Each wave therefore lowers its own
-    // priority as it advances (quarter by quarter), so a wave that is behind is served first.
-    auto fast_pass = [&](uint32_t n_valid, int32_t tail_keys) {
-      m_ref = 0.f;
-      l_run = 0.f;
+    // P V^T and the row sums of one (step, block)
+    auto pv_rowsum = [&](const uint32_t (&pb)[8], const bf16x8_t (&vf)[2], f32x16_t& a, f32x4_t& la) {
 #pragma unroll
-      for (int i = 0; i < 16; ++i) acc[i] = 0.f;
-      bf16x8_t kf[2][KSTEPS];
-      load_k(0, kf[0]);
-      if (NSTEP > 1) load_k(1, kf[1]);
-      f32x16_t sc[2];
-      sc[0] = qk_from(kf[0]);
-      __builtin_amdgcn_s_setprio(3);
-      static_for<NSTEP>([&](auto st_c) {
-        constexpr uint32_t st = decltype(st_c)::value;
-        if (st < n_valid) {                 // uniform
-          if (st == QSTEP) __builtin_amdgcn_s_setprio(2);
-          if (st == 2 * QSTEP) __builtin_amdgcn_s_setprio(1);
-          if (st == 3 * QSTEP) __builtin_amdgcn_s_setprio(0);
-          f32x16_t& s_cur = sc[st & 1u];
-          if constexpr (st + 1 < NSTEP) sc[(st + 1) & 1u] = qk_from(kf[(st + 1) & 1u]);
-          if constexpr (st + 2 < NSTEP) load_k(st + 2, kf[st & 1u]);
-          bf16x8_t vf[2];
+      for (int kk = 0; kk < 2; ++kk) {
+        const u32x4_t praw = {pb[kk * 4 + 0], pb[kk * 4 + 1], pb[kk * 4 + 2], pb[kk * 4 + 3]};
+        const bf16x8_t pf = __builtin_bit_cast(bf16x8_t, praw);
+        a = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[kk], pf, a, 0, 0, 0);
+        la = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones_sel, pf, la, 0, 0, 0);
+      }
+    };
+
+    // ---- fast pass: scopes whose keys are all valid, and one-bucket scopes with a valid prefix (steps past it are
+    //      skipped, the boundary step gets -inf scores: 2^-inf = 0 exactly) ----
+    const bool any_valid = cur.len[0] > 0 || cur.len[1] > 0 || cur.len[2] > 0 || cur.len[3] > 0;
+    const bool all_full = cur.len[0] == (int32_t)bs && (scope_size < 2 || cur.len[1] == (int32_t)bs) &&
+                          (scope_size < 3 || cur.len[2] == (int32_t)bs) && (scope_size < 4 || cur.len[3] == (int32_t)bs);
+    bool any_live = false;
+#pragma unroll
+    for (int b = 0; b < QB; ++b) any_live = any_live || q_live[b];
+    bool redo = false;
+    if (any_valid && any_live) {
+      redo = !(all_full || scope_size == 1);
+      if (!redo) {
+        const uint32_t n_full = all_full ? NSTEP : (uint32_t)cur.len[0] / 32u;        // steps whose 32 keys are all valid
+        const int32_t tail_keys = all_full ? 0 : cur.len[0] - (int32_t)n_full * 32;   // valid keys of the step after them
+        {
+          bf16x8_t kf[2][KSTEPS], vf[2][2];
+          f32x16_t sc[2];
+          load_k(0, kf[0]);
+          load_v(0, vf[0]);
+          sc[0] = scores(kf[0], qf[0]);
+          static_for<NSTEP>([&](auto st_c) {
+            constexpr uint32_t st = decltype(st_c)::value;
+            if (st < n_full) {               // uniform
+              // The SIMD arbiter favours its oldest wave; left alone, that wave finishes early and idles at the
+              // barrier while the other runs the tail alone.  Each wave lowers its own priority as it advances, so
+              // the wave that is behind is served first.
+              if constexpr (st % (NSTEP / 4) == 0) __builtin_amdgcn_s_setprio(3 - (int)(st / (NSTEP / 4)));
+              static_for<VM_PER_STEP>([&](auto j_c) {
+                issue_vm(std::integral_constant<uint32_t, st * VM_PER_STEP + decltype(j_c)::value>{});
+              });
+              vm_next = (st + 1) * VM_PER_STEP;
+              if constexpr (st + 1 < NSTEP) {
+                load_k(st + 1, kf[(st + 1) & 1u]);
+                load_v(st + 1, vf[(st + 1) & 1u]);
+              }
+              static_for<QB>([&](auto b_c) {
+                constexpr uint32_t b = decltype(b_c)::value;
+                constexpr uint32_t u = st * QB + b;          // position in the flattened (step, block) sequence
+                // the scores of the next (step, block) start now
+                if constexpr (b + 1 < QB) sc[(u + 1) & 1u] = scores(kf[st & 1u], qf[b + 1]);
+                else if constexpr (st + 1 < NSTEP) sc[(u + 1) & 1u] = scores(kf[(st + 1) & 1u], qf[0]);
+                const f32x16_t& s_cur = sc[u & 1u];
+                uint32_t pb[8];
+#pragma unroll
+                for (int i = 0; i < 16; i += 2)
+                  pb[i / 2] = pack_bf16x2(__builtin_amdgcn_exp2f(s_cur[i]), __builtin_amdgcn_exp2f(s_cur[i + 1]));
+                pv_rowsum(pb, vf[st & 1u], acc[b], lacc[b]);
+              });
+            }
+          });
+        }
+        if (tail_keys > 0) {
+          // the boundary step, once per item and out of the pipeline: keys at or past the valid length get a
+          // score of -inf.  Register i of a lane is key (i/4)*8 + 4 half + i%4 of the step.
+          bf16x8_t kf[KSTEPS], vf[2];
+          load_k(n_full, kf);
+          load_v(n_full, vf);
+          const int32_t thr = tail_keys - (int32_t)half * 4;
+          static_for<QB>([&](auto b_c) {
+            constexpr uint32_t b = decltype(b_c)::value;
+            f32x16_t sc = scores(kf, qf[b]);
+            uint32_t pb[8];
+#pragma unroll
+            for (int i = 0; i < 16; i += 2) {
+              const float s0 = (i / 4) * 8 + (i % 4) >= thr ? -INFINITY : sc[i];
+              const float s1 = ((i + 1) / 4) * 8 + ((i + 1) % 4) >= thr ? -INFINITY : sc[i + 1];
+              pb[i / 2] = pack_bf16x2(__builtin_amdgcn_exp2f(s0), __builtin_amdgcn_exp2f(s1));
+            }
+            pv_rowsum(pb, vf, acc[b], lacc[b]);
+          });
+        }
+        // redo with a moving reference where a row sum left the safe range (also catches inf / nan)
+#pragma unroll
+        for (int b = 0; b < QB; ++b) {
+          l_fin[b] = __shfl(lacc[b][0], l_src, kWave);
+          redo = redo || (q_live[b] && __ballot(!(l_fin[b] > 0x1p-24f) || !(l_fin[b] < 0x1p24f)) != 0);
+        }
+      }
+    }
+    // ---- general pass: any mix of valid lengths, running-maximum softmax with the scale applied in fp32; one
+    //      (block, step) at a time, nothing overlapped ----
+    if (redo) {
+#pragma unroll 1
+      for (int b = 0; b < QB; ++b) {
+        // unscaled Q, read again: the fast pass keeps only its pre-scaled copy
+        bf16x8_t qr[KSTEPS];
+        {
+          const char* qp = reinterpret_cast<const char*>(q + item_base(item)) + (q_row_of(cur, b) * ld + half * 8u) * 2u;
+#pragma unroll
+          for (int ks = 0; ks < KSTEPS; ++ks) qr[ks] = *reinterpret_cast<const bf16x8_t*>(qp + ks * 32u);
+        }
+        float m_run = -INFINITY, l_run = 0.f;
+        f32x16_t a;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) a[i] = 0.f;
+#pragma unroll 1
+        for (uint32_t st = 0; st < NSTEP; ++st) {
+          // step st covers the 32 keys [32 st, 32 st + 32): position inside its bucket and that bucket's length
+          const uint32_t jb = (st * 32u) / bs;
+          const int32_t in_b = (int32_t)(st * 32u - jb * bs);
+          const int32_t len = len_of(cur, jb);
+          if (in_b >= len) continue;          // no valid key in this step (uniform)
+          bf16x8_t kf[KSTEPS], vf[2];
+          load_k(st, kf);
           load_v(st, vf);
-          if (st + 1 == n_valid && tail_keys < 32) {
-            // (the empty asm keeps this a branch taken once per item instead of selects in every step)
-            asm volatile("; boundary step: mask the keys past the valid length");
-            // register i of a lane is key (i/4)*8 + 4 half + i%4 of the step
-            const int32_t thr = tail_keys - (int32_t)half * 4;
+          f32x16_t sc = scores(kf, qr);
+          if (in_b + 32 > len) {
+            const int32_t thr = len - in_b - (int32_t)half * 4;
 #pragma unroll
             for (int i = 0; i < 16; ++i)
-              if ((i / 4) * 8 + (i % 4) >= thr) s_cur[i] = -INFINITY;
+              if ((i / 4) * 8 + (i % 4) >= thr) sc[i] = -INFINITY;
           }
+          float mx = sc[0];
+#pragma unroll
+          for (int i = 1; i < 16; ++i) mx = fmaxf(mx, sc[i]);
+          mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
+          const float m_new = fmaxf(m_run, mx * scale_log2);
+          const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+          const float alpha = __builtin_amdgcn_exp2f(m_run - m_use);
+          m_run = m_new;
           uint32_t pb[8];
+          float psum = 0.f;
 #pragma unroll
           for (int i = 0; i < 16; i += 2) {
-            pb[i / 2] = pack_bf16x2(__builtin_amdgcn_exp2f(s_cur[i]), __builtin_amdgcn_exp2f(s_cur[i + 1]));
-            l_run = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, pb[i / 2]),
-                                                    __builtin_bit_cast(bf16x2_t, 0x3F803F80u), l_run, false);
+            pb[i / 2] = pack_bf16x2(__builtin_amdgcn_exp2f(__builtin_fmaf(sc[i], scale_log2, -m_use)),
+                                    __builtin_amdgcn_exp2f(__builtin_fmaf(sc[i + 1], scale_log2, -m_use)));
+            psum = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, pb[i / 2]),
+                                                   __builtin_bit_cast(bf16x2_t, 0x3F803F80u), psum, false);
           }
-          pv(pb, vf);
+          l_run = l_run * alpha + psum;
+#pragma unroll
+          for (int i = 0; i < 16; ++i) a[i] *= alpha;
+#pragma unroll
+          for (int kk = 0; kk < 2; ++kk) {
+            const u32x4_t praw = {pb[kk * 4 + 0], pb[kk * 4 + 1], pb[kk * 4 + 2], pb[kk * 4 + 3]};
+            a = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[kk], __builtin_bit_cast(bf16x8_t, praw), a, 0, 0, 0);
+          }
         }
-      });
-      __builtin_amdgcn_s_setprio(3);
-    };
-
-    // ---- general pass: masked keys, running-maximum softmax with the scale applied in fp32 ----
-    // (one step at a time, no overlap; Q is read again because the fast pass only keeps the pre-scaled copy)
-    auto general_pass = [&]() {
-      bf16x8_t qr[KSTEPS];
-      {
-        const uint32_t off = ((q_row * ld) + half * 8) * 2u;
-        const char* qp = reinterpret_cast<const char*>(q + item_base(item));
-#pragma unroll
-        for (int ks = 0; ks < KSTEPS; ++ks) qr[ks] = *reinterpret_cast<const bf16x8_t*>(qp + (off + ks * 32u));
+        // hand the block's results to the epilogue through the variables the fast pass fills
+        static_for<QB>([&](auto b_c) {
+          constexpr uint32_t bb = decltype(b_c)::value;
+          if (bb == (uint32_t)b) {
+            acc[bb] = a;
+            l_fin[bb] = l_run + __shfl_xor(l_run, 32, kWave);
+            m_ref[bb] = (m_run == -INFINITY) ? 0.f : m_run;
+          }
+        });
       }
-      m_ref = -INFINITY;
-      l_run = 0.f;
-#pragma unroll
-      for (int i = 0; i < 16; ++i) acc[i] = 0.f;
-      for (uint32_t st = 0; st < NSTEP; ++st) {
-        // step st covers the 32 keys [32 st, 32 st + 32): position inside its bucket and that bucket's length
-        const uint32_t jb = (st * 32u) / bs;
-        const int32_t in_b = (int32_t)(st * 32u - jb * bs);
-        const int32_t len = jb == 0 ? blen0 : jb == 1 ? blen1 : jb == 2 ? blen2 : blen3;
-        if (in_b >= len) continue;          // no valid key in this step (uniform)
-        f32x16_t sc;
-#pragma unroll
-        for (int i = 0; i < 16; ++i) sc[i] = 0.f;
-        const char* kt = sbuf + st * 32u * ROWB;
-#pragma unroll
-        for (int ks = 0; ks < KSTEPS; ++ks) {
-          const bf16x8_t kf = *reinterpret_cast<const bf16x8_t*>(kt + (k_off ^ (ks * 32u)));
-          sc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qr[ks], sc, 0, 0, 0);
-        }
-        bf16x8_t vf[2];
-        load_v(st, vf);
-        if (in_b + 32 > len) {
-          // register i of a lane is key (i/4)*8 + 4 half + i%4 of the step
-          const int32_t thr = len - in_b - (int32_t)half * 4;
-#pragma unroll
-          for (int i = 0; i < 16; ++i)
-            if ((i / 4) * 8 + (i % 4) >= thr) sc[i] = -INFINITY;
-        }
-        float mx = sc[0];
-#pragma unroll
-        for (int i = 1; i < 16; ++i) mx = fmaxf(mx, sc[i]);
-        mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
-        const float m_new = fmaxf(m_ref, mx * scale_log2);
-        const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-        const float alpha = __builtin_amdgcn_exp2f(m_ref - m_use);
-        m_ref = m_new;
-#pragma unroll
-        for (int i = 0; i < 16; ++i) sc[i] = __builtin_fmaf(sc[i], scale_log2, -m_use);
-        uint32_t pb[8];
-        float psum;
-        exp_pack(sc, pb, psum);
-        l_run = l_run * alpha + psum;
-#pragma unroll
-        for (int i = 0; i < 16; ++i) acc[i] *= alpha;
-        pv(pb, vf);
-      }
-      if (m_ref == -INFINITY) m_ref = 0.f;
-    };
-
-    const bool any_valid = blen0 > 0 || blen1 > 0 || blen2 > 0 || blen3 > 0;
-    const bool all_full = blen0 == (int32_t)bs && (scope_size < 2 || blen1 == (int32_t)bs) &&
-                          (scope_size < 3 || blen2 == (int32_t)bs) && (scope_size < 4 || blen3 == (int32_t)bs);
-    // queries at or beyond the valid length of their bucket produce zeros: a wave that owns only such rows has
-    // nothing to compute (uniform per wave)
-    const bool wave_has_rows = (int32_t)(q_local - qj * bs) < q_valid_len;
-    if (q_exists && any_valid && wave_has_rows) {
-      // the fast pass takes scopes whose keys are all valid, and one-bucket scopes with a valid prefix
-      bool redo = !(all_full || scope_size == 1);
-      if (!redo) {
-        const uint32_t n_valid = all_full ? NSTEP : (uint32_t)(blen0 + 31) / 32u;
-        const int32_t tail_keys = all_full ? 32 : blen0 - (int32_t)(n_valid - 1) * 32;
-        fast_pass(n_valid, tail_keys);
-        // redo with a moving reference if any row sum left the safe range (also catches inf / nan)
-        const float l_chk = l_run + __shfl_xor(l_run, 32, kWave);
-        redo = __ballot(!(l_chk > 0x1p-24f) || !(l_chk < 0x1p24f)) != 0;
-      }
-      if (redo) general_pass();
-    } else {
-      l_run = 0.f;
-#pragma unroll
-      for (int i = 0; i < 16; ++i) acc[i] = 0.f;
     }
-    const float m_run = m_ref;
-    if (n + 2 < my_items) load_table_len();
-    // This wave's direct loads (issued a whole item ago) must have landed before the barrier below;
-    // wait for them BEFORE the output stores are issued, so that the stores stay fire-and-forget
-    // (vmcnt = 0, other counters untouched).
+    __builtin_amdgcn_s_setprio(3);
+    // whatever of the next item's loads the passes above did not issue (short or skipped passes)
+    static_for<VM_OPS>([&](auto i_c) {
+      if (decltype(i_c)::value >= vm_next) issue_vm(i_c);
+    });
+    nxt_len = load_len(nxt_ids);
+    // This wave's direct loads (issued during this item) must have landed before the barrier below; wait for them
+    // BEFORE the output stores are issued, so that the stores stay fire-and-forget (vmcnt = 0, other counters
+    // untouched).
     __builtin_amdgcn_s_waitcnt(0x0F70);
-    if (q_exists) {   // a scope entry outside the sequence names no rows
-      const float l_tot = l_run + __shfl_xor(l_run, 32, kWave);
-      const bool row_ok = (int32_t)q_in_bucket < q_valid_len && l_tot > 0.f;
+
+    // ---- epilogue: normalise, store O (bf16) and LSE ----
+    const size_t obase = (size_t)(item / (num_head * num_scope)) * seq_len * num_head + item % num_head;
+    char* const op = reinterpret_cast<char*>(o + obase * D);
+#pragma unroll
+    for (int b = 0; b < QB; ++b) {
+      if (!q_exists[b]) continue;          // a scope entry outside the sequence names no rows
+      const float l_tot = q_live[b] ? l_fin[b] : 0.f;
+      const bool row_ok = (int32_t)lq < q_len[b] && l_tot > 0.f;
       const float inv = row_ok ? 1.0f / l_tot : 0.f;
-      // uniform 64-bit base of (batch element, head) + 32-bit lane offset
-      const size_t obase = (size_t)(item / (num_head * num_scope)) * seq_len * num_head + item % num_head;
-      char* op = reinterpret_cast<char*>(o + obase * D);
-      const uint32_t orow_b = q_row * num_head * D * 2u;
+      const uint32_t orow_b = q_row[b] * num_head * D * 2u;
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
         const uint32_t d0 = g * 8 + half * 4;
         if (D >= 32 || d0 < (uint32_t)D) {
           uint2 w;
-          w.x = pack_bf16x2(acc[g * 4 + 0] * inv, acc[g * 4 + 1] * inv);
-          w.y = pack_bf16x2(acc[g * 4 + 2] * inv, acc[g * 4 + 3] * inv);
+          w.x = pack_bf16x2(acc[b][g * 4 + 0] * inv, acc[b][g * 4 + 1] * inv);
+          w.y = pack_bf16x2(acc[b][g * 4 + 2] * inv, acc[b][g * 4 + 3] * inv);
           *reinterpret_cast<uint2*>(op + (orow_b + d0 * 2u)) = w;
         }
       }
       if (half == 0) {
         const float ln2 = 0.69314718055994530942f;
-        *reinterpret_cast<float*>(reinterpret_cast<char*>(lse + obase) + q_row * num_head * 4u) =
-            row_ok ? (m_run + __builtin_amdgcn_logf(l_tot)) * ln2 : 0.f;
+        *reinterpret_cast<float*>(reinterpret_cast<char*>(lse + obase) + q_row[b] * num_head * 4u) =
+            row_ok ? (m_ref[b] + __builtin_amdgcn_logf(l_tot)) * ln2 : 0.f;
       }
     }
-    if (n + 2 < my_items) store_table(tnext2);
-    __syncthreads();   // next buffer is complete; this buffer is free for the item after next
+    cur = nxt;
+    __syncthreads();   // the next buffer is complete; this buffer is free for the item after next
   }
 }
 
-template <int D, int T>
-static int launch_attn_resident(const uint16_t* q, const uint16_t* k, const uint16_t* v, uint32_t ld, uint16_t* o,
-                                float* lse, const uint32_t* scope_buckets, uint32_t num_scope, uint32_t scope_size,
-                                uint32_t bs, uint32_t batch, uint32_t seq_len, uint32_t num_head,
-                                const int32_t* kv_len, int device, hipStream_t s) {
+template <int D, int T, int WAVES>
+static int launch_attn_scope(const uint16_t* q, const uint16_t* k, const uint16_t* v, uint32_t ld, uint16_t* o, float* lse,
+                             const uint32_t* scope_buckets, uint32_t num_scope, uint32_t scope_size, uint32_t bs,
+                             uint32_t batch, uint32_t seq_len, uint32_t num_head, const int32_t* kv_len, int device,
+                             hipStream_t s) {
   const uint64_t n_items64 = (uint64_t)batch * num_scope * num_head;
   if (n_items64 == 0) return F3D_OK;
   if (n_items64 > 0x7FFFFFF0ull) {
@@ -686,23 +760,27 @@ static int launch_attn_resident(const uint16_t* q, const uint16_t* k, const uint
     return F3D_ERR_INVALID;
   }
   const uint32_t n_items = (uint32_t)n_items64;
+  constexpr size_t lds = scope_lds_bytes<D, T, WAVES>();
+  // once per instantiation and device: raise the dynamic LDS limit, ask how many workgroups a CU holds
+  static int wg_per_cu[64] = {};
+  int per_cu = (device >= 0 && device < 64) ? wg_per_cu[device] : 0;
+  if (per_cu == 0) {
+    F3D_CHECK_HIP(hipFuncSetAttribute((const void*)buck_swin_fwd_scope_kernel<D, T, WAVES>,
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    F3D_CHECK_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, buck_swin_fwd_scope_kernel<D, T, WAVES>,
+                                                               64 * WAVES, lds));
+    if (per_cu < 1) per_cu = 1;
+    if (device >= 0 && device < 64) wg_per_cu[device] = per_cu;
+  }
   int n_cu = 0;
   F3D_CHECK_HIP(hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, device));
-  constexpr size_t lds = resident_lds_bytes<D, T>();
-  const uint32_t wg_per_cu = (2 * T <= 512 && 2 * lds <= 160 * 1024) ? 2u : 1u;
-  // workgroups: a multiple of the XCD count, no more than the chip holds at once, no more than items need
+  // persistent workgroups: a multiple of the XCD count, no more than the chip holds at once, no more than items need
   const uint32_t items_per_xcd = cdiv_u32(n_items, kNumXcd);
-  const uint32_t n_slots = std::max(1u, std::min((uint32_t)n_cu * wg_per_cu / kNumXcd, items_per_xcd));
+  const uint32_t n_slots = std::max(1u, std::min((uint32_t)n_cu * (uint32_t)per_cu / kNumXcd, items_per_xcd));
   const float scale_log2 = 1.4426950408889634f / sqrtf((float)D);
-  static bool attr_set[64] = {};   // raise the dynamic LDS limit once per instantiation and device
-  if (device < 0 || device >= 64 || !attr_set[device]) {
-    F3D_CHECK_HIP(hipFuncSetAttribute((const void*)buck_swin_fwd_resident_kernel<D, T>,
-                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    if (device >= 0 && device < 64) attr_set[device] = true;
-  }
-  hipLaunchKernelGGL((buck_swin_fwd_resident_kernel<D, T>), dim3(n_slots * kNumXcd), dim3(2 * T), lds, s, q, k, v, ld,
-                     o, lse, scope_buckets, num_scope, scope_size, bs, seq_len, num_head, kv_len, scale_log2, n_items,
-                     items_per_xcd, n_slots);
+  hipLaunchKernelGGL((buck_swin_fwd_scope_kernel<D, T, WAVES>), dim3(n_slots * kNumXcd), dim3(64 * WAVES), lds, s, q, k,
+                     v, ld, o, lse, scope_buckets, num_scope, scope_size, bs, seq_len, num_head, kv_len, scale_log2,
+                     n_items, items_per_xcd, n_slots);
   return F3D_OK;
 }
 
@@ -759,8 +837,8 @@ int f3d_buck_swin_fwd_strided(const f3d_bf16_t* q, const f3d_bf16_t* k, const f3
   if (head_dim <= 32 && scope_size <= (uint32_t)kResMaxScope && (scope_tokens == 256 || scope_tokens == 512) &&
       (uint64_t)seq_len * qkv_row_stride * 2 < (1ull << 32)) {
 #define F3D_RES(DD, TT)                                                                                         \
-  rc = launch_attn_resident<DD, TT>(q, k, v, qkv_row_stride, o, lse, scope_buckets, num_scope, scope_size,      \
-                                    bucket_size, batch, seq_len, num_head, kv_len, device, s)
+  rc = launch_attn_scope<DD, TT, TT / 32>(q, k, v, qkv_row_stride, o, lse, scope_buckets, num_scope, scope_size, \
+                                          bucket_size, batch, seq_len, num_head, kv_len, device, s)
     if (head_dim == 16) {
       if (scope_tokens == 256) F3D_RES(16, 256); else F3D_RES(16, 512);
     } else {
