@@ -85,8 +85,9 @@ def main():
     ap.add_argument("--mlp", default="swiglu", choices=["swiglu", "gelu"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-sub-metrics", action="store_true")
-    ap.add_argument("--sub-metrics-only", action="store_true",
-                    help="run only the per-kernel sub-metrics (configs 1, 2, 3, 5) and print them; for profiling those kernels")
+    ap.add_argument("--sub-metrics-only", nargs="*", default=None, metavar="GROUP",
+                    help="run only the per-kernel sub-metrics (configs 1, 2, 3, 5) and print them; for profiling those "
+                         "kernels.  Optional group names restrict the run: attention, psh, permute, pool, hourglass")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU; the path shards by cloud without any exchange "
@@ -97,8 +98,8 @@ def main():
     from flash3dtransformer_amd.lib import pshattn
     from flash3dtransformer_amd.psh import psh_main
     dev = "cuda:0"
-    if args.sub_metrics_only:
-        print(json.dumps({"sub_metrics": sub_metrics(dev)}))
+    if args.sub_metrics_only is not None:
+        print(json.dumps({"sub_metrics": sub_metrics(dev, set(args.sub_metrics_only) or None)}))
         return
     C, HID, H, BS, SCOPE, HASH = 256, 1024, 8, 512, 1, 2
     clouds = [synth.lidar_sweep(120_000, 1004 + i) for i in range(4)]
@@ -228,12 +229,20 @@ def main():
     print(json.dumps(result))
 
 
-def sub_metrics(dev):
+def sub_metrics(dev, only=None):
     """attention TFLOP/s on config 2, PSH GB/s (config 1 latency + saturating size), pooling and
-    unpooling GB/s on config 3 — each against its roofline"""
-    from flash3dtransformer_amd.lib import pshattn
-    from flash3dtransformer_amd.psh import psh_main, subbuck
+    unpooling GB/s on config 3 — each against its roofline.  `only`: a set of group names, or None for all"""
     out = {}
+    groups = {"attention": sub_attention, "psh": sub_psh, "permute": sub_permute, "pool": sub_pool,
+              "hourglass": lambda d, o: o.__setitem__("hourglass_c5", hourglass_c5(d))}
+    for name, fn in groups.items():
+        if only is None or name in only:
+            fn(dev, out)
+    return out
+
+
+def sub_attention(dev, out):
+    from flash3dtransformer_amd.lib import pshattn
     # ---- attention, config 2: L = 131,072, H = 8, D = 32, bucket 512, scope 1 ----
     L, H, D, BS = 131072, 8, 32, 512
     g = torch.Generator().manual_seed(1002)
@@ -264,6 +273,11 @@ def sub_metrics(dev):
                                     "frac_of_bf16_mfma_peak": round(flb / ms / 1e9 / MFMA_BF16_PEAK_TFLOPS, 4),
                                     "algorithmic_gflop": round(flb / 1e9, 2)}
     del qkv, q, k, v, o, lse, d_o, dq, dk, dv, dlt
+
+
+def sub_psh(dev, out):
+    from flash3dtransformer_amd.lib import pshattn
+    from flash3dtransformer_amd.psh import psh_main
     # ---- PSH: config 1 (latency bound) and a saturating batch, 30 B/pt three-kernel accounting ----
     for name, n_c, b in (("psh_c1_32768", 32768, 1), ("psh_saturating_64x262144", 262144, 64)):
         gg = torch.Generator().manual_seed(1001)
@@ -284,6 +298,11 @@ def sub_metrics(dev):
                      "frac_of_hbm_peak": round(byts / ms / 1e6 / HBM_PEAK_GBS, 4),
                      "mpts_per_s": round(n_c * b / ms / 1e3, 1)}
         del coords, buf
+
+
+def sub_permute(dev, out):
+    from flash3dtransformer_amd.lib import pshattn
+    from flash3dtransformer_amd.psh import psh_main
     # ---- permutation index + feature scatter and the way back: 4 x 120,000 points, 256 bf16 channels ----
     n_c, b, C = 120000, 4, 256
     gg = torch.Generator().manual_seed(1004)
@@ -306,6 +325,11 @@ def sub_metrics(dev):
     out["psh_restore_order_4x120k_c256"] = {"ms": round(ms_r, 4), "gbs": gbs(r_bytes, ms_r),
                                             "frac_of_hbm_peak": round(gbs(r_bytes, ms_r) / HBM_PEAK_GBS, 4)}
     del coords, buf, feat, index, sfeat, back
+
+
+def sub_pool(dev, out):
+    from flash3dtransformer_amd.lib import pshattn
+    from flash3dtransformer_amd.psh import subbuck
     # ---- pooling / unpooling, config 3: 262,144 points x 128 channels, S = 8 ----
     n, C, S = 262144, 128, 8
     gg = torch.Generator().manual_seed(1003)
@@ -358,8 +382,6 @@ def sub_metrics(dev):
     out["unpool_c3_bwd"] = {"ms": round(ms_ub, 4), "gbs": gb(ub_bytes, ms_ub), "frac_of_hbm_peak": round(gb(ub_bytes, ms_ub) / HBM_PEAK_GBS, 4)}
     del g_red, g_in, g_res, g_down
     del coords, feat, res, up, sb
-    out["hourglass_c5"] = hourglass_c5(dev)
-    return out
 
 
 def hourglass_c5(dev):

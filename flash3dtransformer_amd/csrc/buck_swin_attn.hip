@@ -286,6 +286,14 @@ __device__ __forceinline__ void lds_dma16(const void* gbase, uint32_t voff, cons
                : "memory", "m0");
 }
 
+// the same with the LDS address given as a (wave-uniform) 32-bit number
+__device__ __forceinline__ void lds_dma16_at(const void* gbase, uint32_t voff, uint32_t lds_addr) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+               :
+               : "s"(lds_addr), "v"(voff), "s"(gbase)
+               : "memory", "m0");
+}
+
 // ---- scope-resident kernel --------------------------------------------------------------------------
 // When a scope holds 256 or 512 tokens and head_dim <= 32 (the shape of every block of the Flash3D model: one
 // 512-row bucket per scope, 32-wide heads) the K and V of a (batch, scope, head) item fit in LDS twice.  One
@@ -381,33 +389,42 @@ __global__ __launch_bounds__(64 * WAVES) void buck_swin_fwd_scope_kernel(
   }
   const uint32_t l_src = (lq < 16u ? 0u : 32u) + (lq & 15u);
 
-  // ---- item -> (batch, scope, head) and the scope's bucket ids / valid key counts ----
-  // Lane j < scope_size of every wave reads bucket j of an item's scope (two dependent loads, issued long before
-  // their use); the consumer broadcasts them into scalars.
-  auto item_base = [&](uint32_t it) {     // element offset of (first token of the batch element, head), uniform
-    return (size_t)(it / (num_head * num_scope)) * seq_len * ld + (size_t)(it % num_head) * D;
+  // ---- item -> (head, scope, batch); the scope's bucket ids / valid key counts ----
+  // An item index is head + num_head (scope + num_scope batch).  A workgroup's items are n_slots apart: its position
+  // advances by a mixed-radix addition with carries, one division at the start and none per item (the scalar unit
+  // is shared by all waves of a SIMD, and every wave does this bookkeeping).
+  struct Pos {
+    uint32_t head, scope, batch;
   };
-  auto load_ids = [&](uint32_t it) -> uint32_t {
-    return lane < scope_size ? scope_buckets[(size_t)((it / num_head) % num_scope) * scope_size + lane] : 0xFFFFFFFFu;
+  const uint32_t d_head = n_slots % num_head, d_scope = (n_slots / num_head) % num_scope,
+                 d_batch = n_slots / (num_head * num_scope);
+  auto advance = [&](Pos p) {
+    p.head += d_head;
+    uint32_t carry = p.head >= num_head ? 1u : 0u;
+    p.head -= carry ? num_head : 0u;
+    p.scope += d_scope + carry;
+    carry = p.scope >= num_scope ? 1u : 0u;
+    p.scope -= carry ? num_scope : 0u;
+    p.batch += d_batch + carry;
+    return p;
+  };
+  auto in_base = [&](const Pos& p) {      // element offset of (first token of the batch element, head), uniform
+    return (size_t)p.batch * seq_len * ld + (size_t)p.head * D;
+  };
+  // Lane j < scope_size of every wave reads bucket j of an item's scope (two dependent loads, issued long before
+  // their use); the consumer picks entries with v_readlane.
+  auto load_ids = [&](const Pos& p) -> uint32_t {
+    return lane < scope_size ? scope_buckets[(size_t)p.scope * scope_size + lane] : 0xFFFFFFFFu;
   };
   auto load_len = [&](uint32_t ids) -> int32_t {
     return ids >= n_bucket ? 0 : (kv_len ? min(max(kv_len[ids], 0), (int32_t)bs) : (int32_t)bs);
   };
   struct Scope {
-    uint32_t bkt[kResMaxScope];
-    int32_t len[kResMaxScope];
+    uint32_t ids;     // lane j: bucket id of scope entry j (0xFFFFFFFF beyond scope_size)
+    int32_t len;      // lane j: its valid key count (0 for an id outside the sequence)
   };
-  auto broadcast = [&](uint32_t ids, int32_t lens) {
-    Scope sc;
-#pragma unroll
-    for (int j = 0; j < kResMaxScope; ++j) {
-      sc.bkt[j] = __builtin_amdgcn_readlane(ids, j);
-      sc.len[j] = __builtin_amdgcn_readlane(lens, j);
-    }
-    return sc;
-  };
-  auto bucket_of = [&](const Scope& sc, uint32_t j) { return j == 0 ? sc.bkt[0] : j == 1 ? sc.bkt[1] : j == 2 ? sc.bkt[2] : sc.bkt[3]; };
-  auto len_of = [&](const Scope& sc, uint32_t j) { return j == 0 ? sc.len[0] : j == 1 ? sc.len[1] : j == 2 ? sc.len[2] : sc.len[3]; };
+  auto bucket_of = [&](const Scope& sc, uint32_t j) { return (uint32_t)__builtin_amdgcn_readlane(sc.ids, j); };
+  auto len_of = [&](const Scope& sc, uint32_t j) { return (int32_t)__builtin_amdgcn_readlane(sc.len, j); };
 
   // K and V rows [wave T/WAVES, (wave + 1) T/WAVES) of an item go straight into an LDS buffer, 2 BPW direct loads of
   // 1 KB per wave: load i < BPW is K block i of the wave, load BPW + i its V block i.  kv_base() is the byte offset of
@@ -416,14 +433,16 @@ __global__ __launch_bounds__(64 * WAVES) void buck_swin_fwd_scope_kernel(
   // buffer).  The wait that matters is the explicit one before the per-item barrier.
   const uint32_t kv_row0 = wave * (T / WAVES), kv_j = kv_row0 / bs;     // a wave's rows never straddle buckets
   auto kv_wanted = [&](const Scope& sc) { return len_of(sc, kv_j) > 0; };
-  auto kv_base = [&](uint32_t it, const Scope& sc) {
-    return item_base(it) * 2u + (size_t)(bucket_of(sc, kv_j) * bs + (kv_row0 - kv_j * bs)) * ld * 2u;
+  auto kv_base = [&](const Pos& p, const Scope& sc) {
+    return in_base(p) * 2u + (size_t)(bucket_of(sc, kv_j) * bs + (kv_row0 - kv_j * bs)) * ld * 2u;
   };
-  auto issue_kv_one = [&](size_t goff, uint32_t i, char* buf) {
+  // LDS addresses as plain 32-bit numbers (a generic pointer costs a null check per conversion)
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)lds_scope;
+  auto issue_kv_one = [&](size_t goff, uint32_t i, uint32_t buf_addr) {
     const uint32_t blk = wave * BPW + (i < (uint32_t)BPW ? i : i - BPW);
     const size_t g = goff + (size_t)(i < (uint32_t)BPW ? i : i - BPW) * RPB * ld * 2u;
-    if (i < (uint32_t)BPW) lds_dma16(reinterpret_cast<const char*>(k) + g, dma_k, buf + blk * 1024);
-    else lds_dma16(reinterpret_cast<const char*>(v) + g, dma_v, buf + OPB + blk * 1024);
+    if (i < (uint32_t)BPW) lds_dma16_at(reinterpret_cast<const char*>(k) + g, dma_k, buf_addr + blk * 1024);
+    else lds_dma16_at(reinterpret_cast<const char*>(v) + g, dma_v, buf_addr + OPB + blk * 1024);
   };
   // row inside the sequence of query lq of block b (0 when the scope entry names no bucket of the sequence)
   auto q_row_of = [&](const Scope& sc, uint32_t b) {
@@ -431,33 +450,32 @@ __global__ __launch_bounds__(64 * WAVES) void buck_swin_fwd_scope_kernel(
     return (id < n_bucket ? id : 0u) * bs + (q_local - qj * bs) + lq;
   };
   u32x4_t qraw[QB][KSTEPS];
-  auto issue_q_one = [&](uint32_t it, const Scope& sc, auto b_c) {
+  auto issue_q_one = [&](const Pos& p, const Scope& sc, auto b_c) {
     constexpr uint32_t b = decltype(b_c)::value;
-    const char* qp = reinterpret_cast<const char*>(q + item_base(it));
+    const char* qp = reinterpret_cast<const char*>(q + in_base(p));
     const uint32_t off = (q_row_of(sc, b) * ld + half * 8u) * 2u;      // fits 32 bits (checked by the host)
 #pragma unroll
     for (int ks = 0; ks < KSTEPS; ++ks) qraw[b][ks] = *reinterpret_cast<const u32x4_t*>(qp + (off + ks * 32u));
   };
 
   // ---- prologue: the first item's scope, K / V / Q; the second item's bucket ids ----
-  Scope cur;
-  {
-    const uint32_t ids = load_ids(item_lo);
-    cur = broadcast(ids, load_len(ids));
-  }
-  uint32_t nxt_ids = my_items > 1 ? load_ids(item_lo + n_slots) : 0xFFFFFFFFu;
-  int32_t nxt_len = load_len(nxt_ids);
-  static_for<QB>([&](auto b_c) { issue_q_one(item_lo, cur, b_c); });
+  Pos p_cur = {item_lo % num_head, (item_lo / num_head) % num_scope, item_lo / (num_head * num_scope)};
+  Pos p_nxt = advance(p_cur);
+  Scope cur, nxt;
+  cur.ids = load_ids(p_cur);
+  cur.len = load_len(cur.ids);
+  nxt.ids = my_items > 1 ? load_ids(p_nxt) : 0xFFFFFFFFu;
+  nxt.len = load_len(nxt.ids);
+  static_for<QB>([&](auto b_c) { issue_q_one(p_cur, cur, b_c); });
   if (kv_wanted(cur)) {
-    const size_t goff = kv_base(item_lo, cur);
+    const size_t goff = kv_base(p_cur, cur);
 #pragma unroll
-    for (uint32_t i = 0; i < 2u * BPW; ++i) issue_kv_one(goff, i, lds_scope);
+    for (uint32_t i = 0; i < 2u * BPW; ++i) issue_kv_one(goff, i, lds0);
   }
   __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
   __syncthreads();
 
   for (uint32_t n = 0; n < my_items; ++n) {
-    const uint32_t item = item_lo + n * n_slots;
     const bool has_next = n + 1 < my_items;
     const char* const sbuf = lds_scope + (n & 1u) * BUF;
 
@@ -477,21 +495,22 @@ __global__ __launch_bounds__(64 * WAVES) void buck_swin_fwd_scope_kernel(
     // instructions per step (issued all at once they would hold every wave of the workgroup at the memory pipeline's door for a
     // microsecond or two with the SIMDs idle): `vm_next` counts those already issued, 2 BPW direct loads of K / V
     // first, then the Q rows of the wave's QB blocks.
-    Scope nxt = broadcast(nxt_ids, nxt_len);
     constexpr uint32_t VM_OPS = 2u * BPW + QB, VM_PER_STEP = (VM_OPS + NSTEP / 2 - 1) / (NSTEP / 2);   // all in the first half
     const bool nxt_kv = has_next && kv_wanted(nxt);
-    const size_t nxt_goff = nxt_kv ? kv_base(item + n_slots, nxt) : 0;
-    char* const nxt_buf = lds_scope + ((n + 1) & 1u) * BUF;
+    const size_t nxt_goff = nxt_kv ? kv_base(p_nxt, nxt) : 0;
+    const uint32_t nxt_buf = lds0 + ((n + 1) & 1u) * BUF;
     auto issue_vm = [&](auto i_c) {
       constexpr uint32_t i = decltype(i_c)::value;
       if constexpr (i < 2u * BPW) {
         if (nxt_kv) issue_kv_one(nxt_goff, i, nxt_buf);
       } else if constexpr (i < VM_OPS) {
-        if (has_next) issue_q_one(item + n_slots, nxt, std::integral_constant<uint32_t, i - 2u * BPW>{});
+        if (has_next) issue_q_one(p_nxt, nxt, std::integral_constant<uint32_t, i - 2u * BPW>{});
       }
     };
     uint32_t vm_next = 0;
-    nxt_ids = n + 2 < my_items ? load_ids(item + 2 * n_slots) : 0xFFFFFFFFu;
+    const Pos p_nxt2 = advance(p_nxt);
+    Scope nxt2;
+    nxt2.ids = n + 2 < my_items ? load_ids(p_nxt2) : 0xFFFFFFFFu;
 
     // per block: do its rows exist / are they valid (uniform), how many of them, which rows
     uint32_t q_row[QB];
@@ -559,9 +578,9 @@ __global__ __launch_bounds__(64 * WAVES) void buck_swin_fwd_scope_kernel(
 
     // ---- fast pass: scopes whose keys are all valid, and one-bucket scopes with a valid prefix (steps past it are
     //      skipped, the boundary step gets -inf scores: 2^-inf = 0 exactly) ----
-    const bool any_valid = cur.len[0] > 0 || cur.len[1] > 0 || cur.len[2] > 0 || cur.len[3] > 0;
-    const bool all_full = cur.len[0] == (int32_t)bs && (scope_size < 2 || cur.len[1] == (int32_t)bs) &&
-                          (scope_size < 3 || cur.len[2] == (int32_t)bs) && (scope_size < 4 || cur.len[3] == (int32_t)bs);
+    const bool any_valid = __ballot(cur.len > 0) != 0;
+    const bool all_full = __ballot(lane < scope_size && cur.len != (int32_t)bs) == 0;
+    const int32_t len0 = len_of(cur, 0);
     bool any_live = false;
 #pragma unroll
     for (int b = 0; b < QB; ++b) any_live = any_live || q_live[b];
@@ -569,12 +588,16 @@ __global__ __launch_bounds__(64 * WAVES) void buck_swin_fwd_scope_kernel(
     if (any_valid && any_live) {
       redo = !(all_full || scope_size == 1);
       if (!redo) {
-        const uint32_t n_full = all_full ? NSTEP : (uint32_t)cur.len[0] / 32u;        // steps whose 32 keys are all valid
-        const int32_t tail_keys = all_full ? 0 : cur.len[0] - (int32_t)n_full * 32;   // valid keys of the step after them
+        const uint32_t n_full = all_full ? NSTEP : (uint32_t)len0 / 32u;        // steps whose 32 keys are all valid
+        const int32_t tail_keys = all_full ? 0 : len0 - (int32_t)n_full * 32;   // valid keys of the step after them
         {
+          // K fragments are requested a whole step before the score product that reads them (with one block per
+          // wave that product belongs to the NEXT step, so they run two steps ahead), V fragments one step ahead
+          constexpr uint32_t K_AHEAD = QB == 1 ? 2u : 1u;
           bf16x8_t kf[2][KSTEPS], vf[2][2];
           f32x16_t sc[2];
           load_k(0, kf[0]);
+          if constexpr (K_AHEAD == 2 && NSTEP > 1) load_k(1, kf[1]);
           load_v(0, vf[0]);
           sc[0] = scores(kf[0], qf[0]);
           static_for<NSTEP>([&](auto st_c) {
@@ -588,16 +611,15 @@ __global__ __launch_bounds__(64 * WAVES) void buck_swin_fwd_scope_kernel(
                 issue_vm(std::integral_constant<uint32_t, st * VM_PER_STEP + decltype(j_c)::value>{});
               });
               vm_next = (st + 1) * VM_PER_STEP;
-              if constexpr (st + 1 < NSTEP) {
-                load_k(st + 1, kf[(st + 1) & 1u]);
-                load_v(st + 1, vf[(st + 1) & 1u]);
-              }
+              if constexpr (K_AHEAD == 1 && st + 1 < NSTEP) load_k(st + 1, kf[(st + 1) & 1u]);
+              if constexpr (st + 1 < NSTEP) load_v(st + 1, vf[(st + 1) & 1u]);
               static_for<QB>([&](auto b_c) {
                 constexpr uint32_t b = decltype(b_c)::value;
                 constexpr uint32_t u = st * QB + b;          // position in the flattened (step, block) sequence
                 // the scores of the next (step, block) start now
                 if constexpr (b + 1 < QB) sc[(u + 1) & 1u] = scores(kf[st & 1u], qf[b + 1]);
                 else if constexpr (st + 1 < NSTEP) sc[(u + 1) & 1u] = scores(kf[(st + 1) & 1u], qf[0]);
+                if constexpr (K_AHEAD == 2 && st + 2 < NSTEP) load_k(st + 2, kf[st & 1u]);
                 const f32x16_t& s_cur = sc[u & 1u];
                 uint32_t pb[8];
 #pragma unroll
@@ -644,7 +666,7 @@ __global__ __launch_bounds__(64 * WAVES) void buck_swin_fwd_scope_kernel(
         // unscaled Q, read again: the fast pass keeps only its pre-scaled copy
         bf16x8_t qr[KSTEPS];
         {
-          const char* qp = reinterpret_cast<const char*>(q + item_base(item)) + (q_row_of(cur, b) * ld + half * 8u) * 2u;
+          const char* qp = reinterpret_cast<const char*>(q + in_base(p_cur)) + (q_row_of(cur, b) * ld + half * 8u) * 2u;
 #pragma unroll
           for (int ks = 0; ks < KSTEPS; ++ks) qr[ks] = *reinterpret_cast<const bf16x8_t*>(qp + ks * 32u);
         }
@@ -711,14 +733,14 @@ __global__ __launch_bounds__(64 * WAVES) void buck_swin_fwd_scope_kernel(
     static_for<VM_OPS>([&](auto i_c) {
       if (decltype(i_c)::value >= vm_next) issue_vm(i_c);
     });
-    nxt_len = load_len(nxt_ids);
+    nxt2.len = load_len(nxt2.ids);
     // This wave's direct loads (issued during this item) must have landed before the barrier below; wait for them
     // BEFORE the output stores are issued, so that the stores stay fire-and-forget (vmcnt = 0, other counters
     // untouched).
     __builtin_amdgcn_s_waitcnt(0x0F70);
 
     // ---- epilogue: normalise, store O (bf16) and LSE ----
-    const size_t obase = (size_t)(item / (num_head * num_scope)) * seq_len * num_head + item % num_head;
+    const size_t obase = (size_t)p_cur.batch * seq_len * num_head + p_cur.head;
     char* const op = reinterpret_cast<char*>(o + obase * D);
 #pragma unroll
     for (int b = 0; b < QB; ++b) {
@@ -744,6 +766,9 @@ __global__ __launch_bounds__(64 * WAVES) void buck_swin_fwd_scope_kernel(
       }
     }
     cur = nxt;
+    nxt = nxt2;
+    p_cur = p_nxt;
+    p_nxt = p_nxt2;
     __syncthreads();   // the next buffer is complete; this buffer is free for the item after next
   }
 }
