@@ -328,10 +328,17 @@ def sub_permute(dev, out):
 
 
 def sub_pool(dev, out):
+    """pooling / unpooling and their backward: config 3 (262,144 points x 128 channels, S = 8: 77 / 144 MB working
+    sets, which stay inside the 256 MB Infinity Cache when a kernel is repeated, so these are latencies at the
+    configuration's size) and the same kernels on 4,194,304 points (1.2 / 2.3 GB working sets: the bandwidth figures)"""
+    _pool_case(dev, out, 262144, "c3", 30)
+    _pool_case(dev, out, 4194304, "4m", 10)
+
+
+def _pool_case(dev, out, n, tag, iters):
     from flash3dtransformer_amd.lib import pshattn
     from flash3dtransformer_amd.psh import subbuck
-    # ---- pooling / unpooling, config 3: 262,144 points x 128 channels, S = 8 ----
-    n, C, S = 262144, 128, 8
+    C, S = 128, 8
     gg = torch.Generator().manual_seed(1003)
     coords = (torch.rand(n, 3, generator=gg) * 51.2).to(torch.float16).to(dev)
     seps = (torch.arange(1, 5, dtype=torch.int32) * (n // 4)).to(dev).view(torch.uint32)
@@ -355,31 +362,36 @@ def sub_pool(dev, out):
                            u32(sb.unpool_ind.shape[0]), u32(S), u32(op), vp(sb.reduced_feat.data_ptr()),
                            u32(sb.reduced_feat.shape[0]), ci(0), st)
     up = torch.empty_like(res)
-    ms_b = ev_time(build, 30)
-    ms_mean = ev_time(lambda: reduce(0), 30)
-    ms_max = ev_time(lambda: reduce(3), 30)
-    ms_up = ev_time(lambda: pshattn.additive_unpool_fwd(res, sb.reduced_feat, up, sb.unpool_ind, S), 30)
+    ms_b = ev_time(build, iters)
+    ms_mean = ev_time(lambda: reduce(0), iters)
+    ms_max = ev_time(lambda: reduce(3), iters)
+    ms_up = ev_time(lambda: pshattn.additive_unpool_fwd(res, sb.reduced_feat, up, sb.unpool_ind, S), iters)
     r = n // S
     red_bytes = n * C * 2 + r * S * 4 + r * C * 2
     up_bytes = n * C * 2 + r * C * 2 + r * S * 4 + n * C * 2
     bld_bytes = n * 6 + n * 4 + n * 2 + r * S * 4 + r * 6
     gb = lambda b_, ms_: round(b_ / ms_ / 1e6, 1)
-    out["pool_c3_builder"] = {"ms": round(ms_b, 4), "gbs": gb(bld_bytes, ms_b), "frac_of_hbm_peak": round(gb(bld_bytes, ms_b) / HBM_PEAK_GBS, 4)}
-    out["pool_c3_reduce_mean"] = {"ms": round(ms_mean, 4), "gbs": gb(red_bytes, ms_mean), "frac_of_hbm_peak": round(gb(red_bytes, ms_mean) / HBM_PEAK_GBS, 4)}
-    out["pool_c3_reduce_max"] = {"ms": round(ms_max, 4), "gbs": gb(red_bytes, ms_max), "frac_of_hbm_peak": round(gb(red_bytes, ms_max) / HBM_PEAK_GBS, 4)}
-    out["unpool_c3"] = {"ms": round(ms_up, 4), "gbs": gb(up_bytes, ms_up), "frac_of_hbm_peak": round(gb(up_bytes, ms_up) / HBM_PEAK_GBS, 4)}
+
+    def put(name, ms, byts):
+        out[f"{name}_{tag}" if not name.startswith("pool") else name.replace("pool", f"pool_{tag}", 1)] = {
+            "ms": round(ms, 4), "gbs": gb(byts, ms), "frac_of_hbm_peak": round(gb(byts, ms) / HBM_PEAK_GBS, 4),
+            "working_set_mb": round(byts / 1e6, 1)}
+    put("pool_builder", ms_b, bld_bytes)
+    put("pool_reduce_mean", ms_mean, red_bytes)
+    put("pool_reduce_max", ms_max, red_bytes)
+    put("unpool", ms_up, up_bytes)
     # backward of both (same shapes): reduce bwd reads grad R C 2 (+ input N C 2 for max) and writes N C 2;
     # unpool bwd reads N C 2, writes N C 2 + R C 2
     g_red = torch.randn(sb.reduced_feat.shape[0], C, generator=gg).to(torch.bfloat16).to(dev)
     g_in, g_res, g_down = torch.zeros_like(feat), torch.zeros_like(res), torch.zeros_like(sb.reduced_feat)
-    ms_rb = ev_time(lambda: pshattn.batch_subbuck_reduce_backward(g_red, feat, sb.unpool_ind, g_in, S, 0), 30)
-    ms_rbm = ev_time(lambda: pshattn.batch_subbuck_reduce_backward(g_red, feat, sb.unpool_ind, g_in, S, 3), 30)
-    ms_ub = ev_time(lambda: pshattn.additive_unpool_bwd(g_res, g_down, res, sb.unpool_ind, S), 30)
+    ms_rb = ev_time(lambda: pshattn.batch_subbuck_reduce_backward(g_red, feat, sb.unpool_ind, g_in, S, 0), iters)
+    ms_rbm = ev_time(lambda: pshattn.batch_subbuck_reduce_backward(g_red, feat, sb.unpool_ind, g_in, S, 3), iters)
+    ms_ub = ev_time(lambda: pshattn.additive_unpool_bwd(g_res, g_down, res, sb.unpool_ind, S), iters)
     rb_bytes, rbm_bytes = r * C * 2 + n * C * 2 + r * S * 4, r * C * 2 + 2 * n * C * 2 + r * S * 4
     ub_bytes = 2 * n * C * 2 + r * C * 2 + r * S * 4
-    out["pool_c3_reduce_mean_bwd"] = {"ms": round(ms_rb, 4), "gbs": gb(rb_bytes, ms_rb), "frac_of_hbm_peak": round(gb(rb_bytes, ms_rb) / HBM_PEAK_GBS, 4)}
-    out["pool_c3_reduce_max_bwd"] = {"ms": round(ms_rbm, 4), "gbs": gb(rbm_bytes, ms_rbm), "frac_of_hbm_peak": round(gb(rbm_bytes, ms_rbm) / HBM_PEAK_GBS, 4)}
-    out["unpool_c3_bwd"] = {"ms": round(ms_ub, 4), "gbs": gb(ub_bytes, ms_ub), "frac_of_hbm_peak": round(gb(ub_bytes, ms_ub) / HBM_PEAK_GBS, 4)}
+    put("pool_reduce_mean_bwd", ms_rb, rb_bytes)
+    put("pool_reduce_max_bwd", ms_rbm, rbm_bytes)
+    put("unpool_bwd", ms_ub, ub_bytes)
     del g_red, g_in, g_res, g_down
     del coords, feat, res, up, sb
 

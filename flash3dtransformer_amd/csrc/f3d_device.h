@@ -94,11 +94,61 @@ __device__ __forceinline__ uint32_t zorder16(uint32_t vx, uint32_t vy, uint32_t 
   return (ys | (zs << 1) | (xs << 2)) & 0xFFFFu;
 }
 
+// Exact division of a 16-bit number by a 16-bit divisor with one multiply: q = mulhi(x, ceil(2^32 / d)) equals
+// floor(x / d) for all x, d < 2^16 (the rounding error of the reciprocal times x stays below 1 / d).
+struct Div16 {
+  uint32_t d, magic;
+};
+__host__ __device__ __forceinline__ Div16 make_div16(uint32_t d) {
+  Div16 r;
+  r.d = d;
+  r.magic = d > 1u ? (uint32_t)(0x100000000ull / d) + 1u : 0u;   // d = 1: quotient is x itself
+  return r;
+}
+__device__ __forceinline__ uint32_t div16(uint32_t x, const Div16& v) {
+  return v.d > 1u ? __umulhi(x, v.magic) : x;
+}
+
 // divisor16 / num_bucket16 are the 16-bit truncations the reference's HashT parameters apply
 __device__ __forceinline__ uint32_t first_hash(uint32_t vx, uint32_t vy, uint32_t vz, uint32_t hash_type,
                                                uint32_t divisor16, uint32_t num_bucket16) {
   uint32_t h = (hash_type & 1u) ? zorder16(vx, vy, vz) : ((vx ^ vy ^ vz) & 0xFFFFu);
   return (hash_type <= 2u) ? h / divisor16 : h % num_bucket16;
+}
+
+// The same with the divisor prepared once (dv = make_div16(divisor16) for hash types 1 / 2, of num_bucket16 for
+// 3 / 4) and the hash kind as compile-time constants, for the kernels that hash every point of a batch.
+template <bool ZORDER, bool MOD>
+__device__ __forceinline__ uint32_t first_hash_t(uint32_t vx, uint32_t vy, uint32_t vz, const Div16& dv) {
+  const uint32_t h = ZORDER ? zorder16(vx, vy, vz) : ((vx ^ vy ^ vz) & 0xFFFFu);
+  const uint32_t q = div16(h, dv);
+  return MOD ? h - q * dv.d : q;
+}
+
+// ---- wave-cooperative access to runs of short records ---------------------------------------------------------
+// A wave reads `bytes` consecutive bytes starting at the 2-byte aligned address `src` in aligned 16-byte pieces (lane
+// l takes pieces l, l + 64, ...) and parks them in a wave-private LDS area; the run then starts at byte
+// `returned shift` (0..14) of the area.  The first / last piece may reach up to 14 bytes before / past the run: they
+// lie in the same 16-byte block as a byte of the run, hence in a page of the same allocation, but a piece that starts
+// at or past `limit` (the end of the array) is not read.  MAXBYTES: largest run the caller passes.
+template <uint32_t MAXBYTES>
+constexpr uint32_t wave_run_area_bytes() {
+  return ((MAXBYTES + 14u + 15u) / 16u) * 16u;
+}
+template <uint32_t MAXBYTES>
+__device__ __forceinline__ uint32_t wave_fetch_run(const void* src, uint32_t bytes, const void* limit, char* area,
+                                                   uint32_t lane) {
+  const uintptr_t a = (uintptr_t)src, a0 = a & ~(uintptr_t)15, end = (uintptr_t)limit;
+  const uint32_t shift = (uint32_t)(a - a0);
+  const uint32_t pieces = (shift + bytes + 15u) / 16u;
+  constexpr uint32_t MAXP = wave_run_area_bytes<MAXBYTES>() / 16u;
+#pragma unroll
+  for (uint32_t i = 0; i * kWave < MAXP; ++i) {
+    const uint32_t p = lane + i * kWave;
+    if (p < pieces && a0 + 16u * p < end)
+      *reinterpret_cast<u32x4_t*>(area + 16u * p) = *reinterpret_cast<const u32x4_t*>(a0 + 16u * (uintptr_t)p);
+  }
+  return shift;
 }
 
 // ---- stateless RNG: 32-bit finaliser chained over (seed, a, b, c) -------------------------------

@@ -31,18 +31,29 @@ __device__ __forceinline__ uint32_t tile_pos(uint32_t w, uint32_t j, uint32_t l)
   return w * (kWave * ITEMS) + j * kWave + l;
 }
 
-template <int THREADS, int ITEMS>
+// The coordinate rows of a wave's 64 * ITEMS consecutive points are one run of 384 * ITEMS bytes: fetched in
+// 16-byte pieces into a wave-private LDS area and picked up from there, a few vector-memory instructions per wave
+// instead of three 2-byte loads per point (the memory pipeline is paced by instructions, not bytes, at that size).
+template <int THREADS, int ITEMS, bool ZORDER, bool MOD>
 __global__ __launch_bounds__(THREADS) void psh_hash_hist_kernel(
     const uint16_t* __restrict__ coord, uint16_t* __restrict__ bucket_id, const uint32_t* __restrict__ batch_sep,
-    const uint16_t* __restrict__ bbox_min, const uint16_t* __restrict__ bbox_max, uint32_t num_vox,
-    uint32_t divisor16, uint32_t num_bucket, uint32_t hash_type, uint32_t* __restrict__ tile_hist,
-    uint32_t max_tiles) {
-  extern __shared__ uint32_t lds_hist[];
+    const uint16_t* __restrict__ bbox_min, const uint16_t* __restrict__ bbox_max, uint32_t num_vox, Div16 dv,
+    uint32_t num_bucket, uint32_t total_n, uint32_t* __restrict__ tile_hist, uint32_t max_tiles) {
+  extern __shared__ __attribute__((aligned(16))) uint32_t lds_hist[];
+  constexpr uint32_t kRunBytes = 384u * ITEMS, kArea = wave_run_area_bytes<kRunBytes>();
   const uint32_t cloud = blockIdx.y, tile = blockIdx.x, tid = threadIdx.x;
   const uint32_t start = cloud ? batch_sep[cloud - 1] : 0u;
   const uint32_t n = batch_sep[cloud] - start;
   const uint32_t tile0 = tile * (THREADS * ITEMS);
   if (tile0 >= n) return;  // uniform for the workgroup
+
+  const uint32_t w = __builtin_amdgcn_readfirstlane(tid / kWave), l = tid % kWave;
+  char* area = reinterpret_cast<char*>(lds_hist + num_bucket) + w * kArea;
+  // this wave's rows [wave0, wave0 + rows) of the cloud
+  const uint32_t wave0 = tile0 + w * (kWave * ITEMS);
+  const uint32_t rows = wave0 < n ? min((uint32_t)(kWave * ITEMS), n - wave0) : 0u;
+  uint32_t shift = 0;
+  if (rows) shift = wave_fetch_run<kRunBytes>(coord + 3 * ((size_t)start + wave0), rows * 6u, coord + 3 * (size_t)total_n, area, l);
 
   for (uint32_t b = tid; b < num_bucket; b += THREADS) lds_hist[b] = 0u;
   VoxAxis ax[3];
@@ -50,19 +61,16 @@ __global__ __launch_bounds__(THREADS) void psh_hash_hist_kernel(
   for (int d = 0; d < 3; ++d) ax[d] = make_vox_axis(bbox_min[d], bbox_max[d], num_vox);
   __syncthreads();
 
-  const uint32_t w = tid / kWave, l = tid % kWave;
-  const uint32_t nb16 = num_bucket & 0xFFFFu;
 #pragma unroll
   for (int j = 0; j < ITEMS; ++j) {
-    const uint32_t local = tile0 + tile_pos<ITEMS>(w, j, l);
-    if (local < n) {
-      const size_t g = (size_t)start + local;
-      const uint16_t* p = coord + 3 * g;
+    const uint32_t t = j * kWave + l;               // position inside the wave's run: (j, l) order is input order
+    if (t < rows) {
+      const uint16_t* p = reinterpret_cast<const uint16_t*>(area + shift + 6u * t);
       uint32_t v[3];
 #pragma unroll
       for (int d = 0; d < 3; ++d) v[d] = vox1(half_bits_to_float(p[d]), ax[d]);
-      const uint32_t id = first_hash(v[0], v[1], v[2], hash_type, divisor16, nb16);
-      bucket_id[g] = (uint16_t)id;
+      const uint32_t id = first_hash_t<ZORDER, MOD>(v[0], v[1], v[2], dv);
+      bucket_id[(size_t)start + wave0 + t] = (uint16_t)id;
       atomicAdd(&lds_hist[id], 1u);
     }
   }
@@ -491,9 +499,14 @@ static void launch_psh(const uint16_t* coord, uint16_t* bucket_id, uint32_t* buc
                        uint32_t max_tiles, uint32_t nbits, hipStream_t stream) {
   const uint32_t tile_pts = THREADS * ITEMS;
   if (max_tiles > 0 && batch_size > 0) {
-    hipLaunchKernelGGL((psh_hash_hist_kernel<THREADS, ITEMS>), dim3(max_tiles, batch_size), dim3(THREADS),
-                       num_bucket * sizeof(uint32_t), stream, coord, bucket_id, batch_sep, bbox_min, bbox_max, num_vox,
-                       divisor16, num_bucket, hash_type, tile_hist, max_tiles);
+    // hash types 1 / 2 divide the 16-bit hash by the divisor, 3 / 4 take it modulo the bucket count
+    const bool zorder = (hash_type & 1u) != 0, mod = hash_type > 2u;
+    const Div16 dv = make_div16(mod ? (num_bucket & 0xFFFFu) : divisor16);
+    const size_t lds1 = num_bucket * sizeof(uint32_t) + (THREADS / kWave) * wave_run_area_bytes<384u * ITEMS>();
+    auto k1 = zorder ? (mod ? psh_hash_hist_kernel<THREADS, ITEMS, true, true> : psh_hash_hist_kernel<THREADS, ITEMS, true, false>)
+                     : (mod ? psh_hash_hist_kernel<THREADS, ITEMS, false, true> : psh_hash_hist_kernel<THREADS, ITEMS, false, false>);
+    hipLaunchKernelGGL(k1, dim3(max_tiles, batch_size), dim3(THREADS), lds1, stream, coord, bucket_id, batch_sep,
+                       bbox_min, bbox_max, num_vox, dv, num_bucket, total_n, tile_hist, max_tiles);
     hipLaunchKernelGGL(psh_tile_scan_kernel, dim3(cdiv_u32(num_bucket, kWave), batch_size), dim3(kScanWaves * kWave), 0,
                        stream, tile_hist, bucket_counter, cnt_ws, batch_sep, num_bucket, tile_pts, max_tiles);
     hipLaunchKernelGGL(psh_bucket_plan_kernel<REBAL>, dim3(batch_size), dim3(kPshThreads),

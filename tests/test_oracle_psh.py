@@ -275,3 +275,14 @@ def test_rebalance_invariants(oracle, case):
         dst[dst == 0] = nb                                                # recycle bucket comes last
         assert (np.diff(dst) >= 0).all()
         start = end
+
+
+def test_one_multiply_division_of_16_bit_numbers_is_exact():
+    """the hashing kernel divides the 16-bit hash by the bucket divisor with q = (x * (2^32 // d + 1)) >> 32
+    (csrc/f3d_device.h:div16); exact for every 16-bit x and every divisor a bucket geometry can produce"""
+    x = np.arange(65536, dtype=np.uint64)
+    for d in list(range(2, 70)) + [127, 128, 129, 255, 256, 257, 511, 512, 513, 1023, 1024, 1025, 2047, 2048, 2049,
+                                   4095, 4096, 21845, 32767, 32768, 65534, 65535]:
+        magic = np.uint64((1 << 32) // d + 1)
+        q = (x * magic) >> np.uint64(32)
+        assert np.array_equal(q, x // np.uint64(d)), d
