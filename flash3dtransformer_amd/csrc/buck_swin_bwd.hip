@@ -400,7 +400,7 @@ extern "C" int f3d_buck_swin_bwd(const f3d_bf16_t* q, const f3d_bf16_t* k, const
                                  const float* lse, float* delta, f3d_bf16_t* dq, f3d_bf16_t* dk, f3d_bf16_t* dv,
                                  const uint32_t* scope_buckets, uint32_t num_scope, uint32_t scope_size,
                                  uint32_t bucket_size, uint32_t batch, uint32_t seq_len, uint32_t num_head,
-                                 uint32_t head_dim, int device, void* stream) {
+                                 uint32_t head_dim, const int32_t* kv_len, int device, void* stream) {
   using namespace f3d;
   F3D_CHECK_ARG(q && k && v && o && d_o && lse && delta && dq && dk && dv && scope_buckets, "null tensor pointer");
   F3D_CHECK_ARG(bucket_size >= 128 && bucket_size % 128 == 0, "bucket_size=%u must be a multiple of 128",
@@ -413,11 +413,18 @@ extern "C" int f3d_buck_swin_bwd(const f3d_bf16_t* q, const f3d_bf16_t* k, const
   F3D_CHECK_ARG((((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)o | (uintptr_t)d_o | (uintptr_t)dq |
                   (uintptr_t)dk | (uintptr_t)dv) & 15u) == 0,
                 "q/k/v/o/dO/dQ/dK/dV must be 16-byte aligned");
+  F3D_CHECK_ARG(scope_size >= 1, "scope_size must be at least 1");
   const uint32_t scope_tokens = scope_size * bucket_size;
-  if (!((head_dim == 16 || head_dim == 32) && scope_size >= 1 && scope_size <= (uint32_t)kBwdMaxScope &&
-        (scope_tokens == 256 || scope_tokens == 512) && (uint64_t)seq_len * qkv_row_stride * 2 < (1ull << 32))) {
-    set_error("No backward kernel found for head_dim=%u, scope of %u x %u tokens (supported: head_dim 16 or 32, "
-              "scopes of 256 or 512 tokens in at most %d buckets)", head_dim, scope_size, bucket_size, kBwdMaxScope);
+  // the scope-resident kernels: small heads, a scope that fits LDS, no valid lengths, 32-bit row offsets
+  const bool resident = (head_dim == 16 || head_dim == 32) && scope_size <= (uint32_t)kBwdMaxScope &&
+                        (scope_tokens == 256 || scope_tokens == 512) && kv_len == nullptr &&
+                        (uint64_t)seq_len * qkv_row_stride * 2 < (1ull << 32);
+  if (!(head_dim == 16 || head_dim == 32 || head_dim == 64 || head_dim == 128)) {
+    set_error("No backward kernel found for head_dim=%u (supported: 16, 32, 64, 128)", head_dim);
+    return F3D_ERR_UNSUPPORTED;
+  }
+  if (!resident && (uint64_t)scope_size * 8 > 32 * 1024) {
+    set_error("attention backward: a scope of %u buckets exceeds the 4096 the scope table holds", scope_size);
     return F3D_ERR_UNSUPPORTED;
   }
   if (batch == 0 || num_scope == 0 || num_head == 0) return F3D_OK;
@@ -429,7 +436,10 @@ extern "C" int f3d_buck_swin_bwd(const f3d_bf16_t* q, const f3d_bf16_t* k, const
 #define F3D_BWD(DD, TT)                                                                                          \
   rc = launch_attn_bwd<DD, TT>(q, k, v, qkv_row_stride, o, d_o, lse, delta, dq, dk, dv, scope_buckets, num_scope, \
                                scope_size, bucket_size, batch, seq_len, num_head, device, s)
-  if (head_dim == 16) {
+  if (!resident) {
+    rc = launch_attn_bwd_stream(q, k, v, qkv_row_stride, o, d_o, lse, delta, dq, dk, dv, scope_buckets, num_scope,
+                                scope_size, bucket_size, batch, seq_len, num_head, head_dim, kv_len, device, s);
+  } else if (head_dim == 16) {
     if (scope_tokens == 256) F3D_BWD(16, 256); else F3D_BWD(16, 512);
   } else {
     if (scope_tokens == 256) F3D_BWD(32, 256); else F3D_BWD(32, 512);

@@ -19,7 +19,7 @@ COMMON = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc",
     # packed fp32 VALU ops are kept out of the generated code on purpose
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-    "-Wall", "-Wno-unused-function", "-Wno-unknown-warning-option",
+    "-Wall", "-Wno-unused-function", "-Wno-unknown-warning-option", "-Wno-inline-asm",
 ]
 # MFMA accumulators live in ordinary VGPRs (unified register file on gfx90a+): the softmax and the
 # epilogues read them without v_accvgpr moves

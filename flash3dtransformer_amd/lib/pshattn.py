@@ -395,12 +395,19 @@ def buck_swin_fwd(Q, K, V, O, L, Scope_buckets, bucket_size, kv_len=None):
         _u32(D), _ptr(kv_len), _i32(dev), _stream(dev)))
 
 
-def buck_swin_bwd(Q, K, V, O, dO, LSE, Delta, dQ, dK, dV, Scope_buckets, bucket_size):
+def buck_swin_bwd(Q, K, V, O, dO, LSE, Delta, dQ, dK, dV, Scope_buckets, bucket_size, kv_len=None):
     """declared src/f3d_frontend.cu:94-97, called at flash3dxfmr/layers/buck_swin.py:90-92.
     Q, K, V [B,L,H,D] bf16 (may be column slices of one projection output, equal strides); O, dO, dQ, dK, dV dense
     [B,L,H,D] bf16; LSE (from the forward), Delta (written here: rowsum(dO * O)) [B,L,H] fp32.  Rows that no scope
-    covers are not written (pass zero-filled dQ / dK / dV).  Scopes of 256 or 512 tokens, head_dim 16 or 32."""
-    dev = assert_same_device([Q, K, V, O, dO, LSE, Delta, dQ, dK, dV, Scope_buckets])
+    covers are not written (pass zero-filled dQ / dK / dV).  head_dim 16, 32, 64 or 128; scopes of any number of
+    buckets.  kv_len (extension, as in the forward): int32 [L / bucket_size] valid rows per bucket."""
+    dev = assert_same_device([Q, K, V, O, dO, LSE, Delta, dQ, dK, dV, Scope_buckets] +
+                             ([kv_len] if kv_len is not None else []))
+    if kv_len is not None:
+        assert_dtype([kv_len], torch.int32)
+        assert_contiguous([kv_len])
+        if kv_len.numel() != Q.shape[1] // bucket_size:
+            raise RuntimeError(f"kv_len must have L / bucket_size = {Q.shape[1] // bucket_size} entries")
     assert_dtype([Q, K, V, O, dO, dQ, dK, dV], torch.bfloat16)
     assert_dtype([LSE, Delta], torch.float32)
     assert_dtype([Scope_buckets], torch.uint32)
@@ -418,7 +425,7 @@ def buck_swin_bwd(Q, K, V, O, dO, LSE, Delta, dQ, dK, dV, Scope_buckets, bucket_
     rc = _load().f3d_buck_swin_bwd(
         _ptr(Q), _ptr(K), _ptr(V), _u32(Q.stride(1)), _ptr(O), _ptr(dO), _ptr(LSE), _ptr(Delta), _ptr(dQ), _ptr(dK),
         _ptr(dV), _ptr(Scope_buckets), _u32(Scope_buckets.shape[0]), _u32(Scope_buckets.shape[1]), _u32(bucket_size),
-        _u32(B), _u32(Ls), _u32(H), _u32(D), _i32(dev), _stream(dev))
+        _u32(B), _u32(Ls), _u32(H), _u32(D), _ptr(kv_len), _i32(dev), _stream(dev))
     if rc == 2:   # F3D_ERR_UNSUPPORTED: a shape outside the backward kernels
         raise NotImplementedError(_load().f3d_last_error().decode("utf-8", "replace"))
     _check(rc)

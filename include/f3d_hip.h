@@ -195,13 +195,16 @@ int f3d_subbuck_reduce_bwd(const f3d_bf16_t* grad_red_feat, const f3d_bf16_t* in
  *      flash3dxfmr/layers/buck_swin.py:69-95 (kernel source absent from the reference) ------------
  * q,k,v [batch,seq_len,num_head,head_dim] bf16 with row stride qkv_row_stride (elements); o, d_o, dq, dk, dv dense
  * [batch,seq_len,num_head,head_dim] bf16; lse (from the forward), delta (output: rowsum(d_o * o))
- * [batch,seq_len,num_head] fp32.  Rows that no scope covers are not written.  Supported: head_dim 16 or 32, scopes of
- * 256 or 512 tokens in at most 4 buckets; anything else returns F3D_ERR_UNSUPPORTED. */
+ * [batch,seq_len,num_head] fp32.  Rows that no scope covers are not written.  kv_len (may be NULL)
+ * [seq_len/bucket_size] i32 is the forward's extension: rows of a bucket at or past its valid length get zero
+ * gradients and add nothing to the others (they must still hold finite numbers).  Supported: head_dim 16, 32, 64 or
+ * 128, scopes of any number of buckets up to 4096 (the reference's test shapes, tests/test_attn_bwd.py: head_dim 64 and
+ * 128, 32 buckets of 256 in one scope); other head sizes return F3D_ERR_UNSUPPORTED. */
 int f3d_buck_swin_bwd(const f3d_bf16_t* q, const f3d_bf16_t* k, const f3d_bf16_t* v, uint32_t qkv_row_stride,
                       const f3d_bf16_t* o, const f3d_bf16_t* d_o, const float* lse, float* delta, f3d_bf16_t* dq,
                       f3d_bf16_t* dk, f3d_bf16_t* dv, const uint32_t* scope_buckets, uint32_t num_scope,
                       uint32_t scope_size, uint32_t bucket_size, uint32_t batch, uint32_t seq_len, uint32_t num_head,
-                      uint32_t head_dim, int device, void* stream);
+                      uint32_t head_dim, const int32_t* kv_len, int device, void* stream);
 
 /* ---- bucketed attention forward: buck_swin_fwd, declared src/f3d_frontend.cu:90-92, called from
  *      flash3dxfmr/layers/buck_swin.py:57 (kernel source absent from the reference) --------------

@@ -380,11 +380,13 @@ def buck_swin_fwd(Q, K, V, scope_buckets, bucket_size, kv_len=None, O_init=None,
     return O, LSE
 
 
-def buck_swin_bwd(Q, K, V, dO, scope_buckets, bucket_size):
+def buck_swin_bwd(Q, K, V, dO, scope_buckets, bucket_size, kv_len=None):
     """Backward of buck_swin_fwd (pshattn.buck_swin_bwd, declared src/f3d_frontend.cu:94-97; the formulas are the
     ones the reference's tests take from autograd, tests/test_attn_bwd.py): per scope and head, with
     P = softmax(Q Kt / sqrt(D)),  Delta = rowsum(dO * O),  dV = Pt dO,  dP = dO Vt,  dS = P * (dP - Delta),
     dQ = dS K / sqrt(D),  dK = dSt Q / sqrt(D).  Rows no scope covers get zero gradients.
+    ``kv_len`` (the forward's extension): P is the softmax over the valid keys, and zero on masked query rows, so
+    masked rows get zero gradients and Delta = 0.
     Returns (dQ, dK, dV, Delta) in fp32."""
     import torch
 
@@ -398,7 +400,15 @@ def buck_swin_bwd(Q, K, V, dO, scope_buckets, bucket_size):
     for s in range(scopes.shape[0]):
         rows = (scopes[s][:, None] * bucket_size + ar[None, :]).reshape(-1)
         q, k, v, do = [t[:, rows].permute(0, 2, 1, 3) for t in (Qf, Kf, Vf, dOf)]   # [B,H,T,D]
-        p = torch.softmax(torch.matmul(q, k.transpose(-1, -2)) * scale, dim=-1)
+        logits = torch.matmul(q, k.transpose(-1, -2)) * scale
+        if kv_len is not None:
+            kl = torch.as_tensor(np.asarray(kv_len).astype(np.int64))[scopes[s]]
+            valid = (ar[None, :] < kl[:, None]).reshape(-1)
+            logits = logits.masked_fill(~valid[None, None, None, :], float("-inf"))
+            p = torch.softmax(logits, dim=-1) if valid.any() else torch.zeros_like(logits)
+            p = torch.where(valid[None, None, :, None], p, torch.zeros_like(p))
+        else:
+            p = torch.softmax(logits, dim=-1)
         o = torch.matmul(p, v)
         delta = (do * o).sum(-1)                                                    # [B,H,T]
         dp = torch.matmul(do, v.transpose(-1, -2))

@@ -303,6 +303,31 @@ def test_attention_bwd_formulas_vs_autograd(oracle):
     assert torch.equal(dQ2[:, :256], dQ[:, :256])
 
 
+def test_attention_bwd_with_valid_lengths_vs_autograd(oracle):
+    """the masked backward against autograd through the oracle's masked forward (whose masks the forward tests pin):
+    a full bucket, a ragged one, a one-key bucket, and an empty bucket sharing a scope with a valid one"""
+    rng = np.random.default_rng(12)
+    B, L, H, D, bs = 1, 512, 2, 16, 128
+    Q, K, V = [t.float().requires_grad_(True) for t in _qkv(rng, B, L, H, D)]
+    scopes = np.array([[1, 0], [3, 2]], dtype=np.uint32)
+    kv_len = np.array([128, 77, 1, 0])
+    dO = torch.from_numpy(rng.normal(0, 1, (B, L, H, D)).astype(np.float32))
+    O, _ = oracle.buck_swin_fwd(Q, K, V, scopes, bs, kv_len=kv_len)
+    O.backward(dO)
+    dQ, dK, dV, Delta = oracle.buck_swin_bwd(Q.detach(), K.detach(), V.detach(), dO, scopes, bs, kv_len=kv_len)
+    for got, want in ((dQ, Q.grad), (dK, K.grad), (dV, V.grad)):
+        assert torch.isfinite(want).all()
+        assert (got - want).abs().max().item() <= 2e-5 * max(1.0, want.abs().max().item())
+    assert (Delta - (dO * O.detach()).sum(-1)).abs().max().item() <= 1e-5
+    for t in (dQ, dK, dV):
+        assert not t[:, 128 + 77:256].any() and not t[:, 257:].any() and t[:, :128 + 77].any()
+    assert torch.equal(dV[:, 256], dO[:, 256])      # the one-key bucket: P = 1
+    # lengths equal to the bucket size change nothing
+    same = oracle.buck_swin_bwd(Q.detach(), K.detach(), V.detach(), dO, scopes, bs, kv_len=np.full(4, bs))
+    plain = oracle.buck_swin_bwd(Q.detach(), K.detach(), V.detach(), dO, scopes, bs)
+    assert all(torch.equal(a, b) for a, b in zip(same, plain))
+
+
 @pytest.mark.parametrize("act", [None, "gelu", "relu"])
 def test_bn_act_vs_torch_batch_norm(oracle, act):
     """eval-mode BatchNorm1d (+ GELU / ReLU) of the oracle against torch.nn.functional.batch_norm(training=False) and the
