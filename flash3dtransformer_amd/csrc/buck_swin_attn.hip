@@ -769,7 +769,9 @@ __global__ __launch_bounds__(64 * WAVES) void buck_swin_fwd_scope_kernel(
     nxt = nxt2;
     p_cur = p_nxt;
     p_nxt = p_nxt2;
-    __syncthreads();   // the next buffer is complete; this buffer is free for the item after next
+    // the next buffer is complete; this buffer is free for the item after next.  Not __syncthreads(): that would wait
+    // for the output stores just issued
+    wg_barrier_lds();
   }
 }
 

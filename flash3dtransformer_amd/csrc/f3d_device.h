@@ -9,6 +9,12 @@ namespace f3d {
 
 constexpr int kWave = 64;
 
+// Workgroup barrier that waits for this wave's LDS operations only.  __syncthreads() also waits for every outstanding
+// global load and store of the wave (its release fence covers global memory), which serialises a loop whose stores
+// and direct-to-LDS loads are meant to stay in flight across the barrier; what such a loop needs from global memory
+// it waits for explicitly (s_waitcnt vmcnt).  The "memory" clobber keeps the compiler from moving accesses across.
+__device__ __forceinline__ void wg_barrier_lds() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
 // ---- 16-bit float bit patterns <-> fp32 -------------------------------------------------------
 
 __device__ __forceinline__ float half_bits_to_float(uint16_t h) {

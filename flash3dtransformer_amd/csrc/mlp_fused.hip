@@ -15,8 +15,8 @@
 // Per chunk the weights stream HBM/L2 -> LDS directly (global_load ... lds), three buffers deep: 64 rows of the
 // LayerNorm-folded w1 (row-major, 16-byte pieces XOR-swizzled) and the chunk's slice of w2, which the preparation
 // kernel stores fragment-major (the 64 lanes' 16-byte pieces of one fragment are consecutive), so its LDS reads are
-// linear.  LayerNorm is folded as in the row-panel linear kernel (w' = w * gamma, one extra k-step applies
-// -mean * wsum + b' / rstd, the gate epilogue multiplies by rstd).
+// linear.  LayerNorm as in the row-panel linear kernel: the rows are normalised in registers (bf16((x - mean) * rstd)),
+// w' = w * gamma, and one extra k-step starts the fc1 accumulators from b' = b1 + w1 beta.
 //
 // Matrix-core bound: 6 * M * C * H flops (fc1 value + gate, fc2) against HBM traffic of x, residual and y only.
 // The hidden activations (M x H bf16, 1 GB at 482 k rows x 1024) are never allocated.  Measured on MI355X at
@@ -47,9 +47,9 @@ struct MlpGeom {
   static constexpr int CH1 = G::CHUNK_BYTES;                // w1 chunk: 64 rows
   static constexpr int CH2 = K * 32 * 2;                    // w2 chunk: K outputs x 32 hidden
   static constexpr int N_DMA2 = CH2 / 1024;
-  // weight buffers, the table rows of the w1 slots, and the rows' (-mean, 1 / rstd) pairs (8 bytes per lane and row tile)
+  // weight buffers, the table rows of the w1 slots, and the x operands kept in LDS
   static constexpr size_t lds_bytes() {
-    return (size_t)kMlpBufs1 * (CH1 + 1024) + (size_t)kMlpBufs2 * CH2 + (size_t)kMlpWaves * kMlpMT * 64 * 8 +
+    return (size_t)kMlpBufs1 * (CH1 + 1024) + (size_t)kMlpBufs2 * CH2 +
            (size_t)kMlpWaves * kMlpMT * kMlpXTail * 1024;
   }
 };
@@ -80,10 +80,9 @@ __global__ __launch_bounds__(64 * kMlpWaves) __attribute__((amdgpu_waves_per_eu(
   extern __shared__ __attribute__((aligned(1024))) char lds_mlp[];
   char* w1buf = lds_mlp;
   char* w2buf = lds_mlp + (size_t)NB1 * MG::CH1;
-  char* s_side = w2buf + (size_t)NB2 * MG::CH2;   // per w1 slot: the chunk's 64 rows of the LayerNorm table
-  float2* s_stat = reinterpret_cast<float2*>(s_side + (size_t)NB1 * 1024);   // [wave][mt][lane]: (-mean, 1 / rstd)
+  char* s_side = w2buf + (size_t)NB2 * MG::CH2;   // per w1 slot: the chunk's 64 rows of the bias table
   constexpr int XT = kMlpXTail, KSR = K / 16 - XT;                            // k-steps whose x operand is in registers
-  bf16x8_t* s_xtail = reinterpret_cast<bf16x8_t*>(reinterpret_cast<char*>(s_stat) + (size_t)WAVES * MT * 64 * 8);   // [wave][mt][j][lane]
+  bf16x8_t* s_xtail = reinterpret_cast<bf16x8_t*>(s_side + (size_t)NB1 * 1024);   // [wave][mt][j][lane]
 
   const uint32_t tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid / kWave), lane = tid % kWave;
   const uint32_t lq = lane & 31u, half = lane >> 5;
@@ -124,8 +123,9 @@ __global__ __launch_bounds__(64 * kMlpWaves) __attribute__((amdgpu_waves_per_eu(
           xf[mt][kp * (KP / 16) + ks] = *reinterpret_cast<const bf16x8_t*>(patch + lq * PROW + ks * 16 + half * 8);
       }
   }
-  // LayerNorm statistics of this lane's rows (shifted by the row's first element against cancellation)
-  float ln_a[MT];   // rstd; (-mean, 1 / rstd) of the lane's rows are parked in LDS: they are needed once per chunk
+  // LayerNorm of this lane's rows in place: statistics (shifted by the row's first element against cancellation), then
+  // x <- bf16((x - mean) * rstd), one fragment at a time (kept opaque so that the floats of the first sweep are not
+  // held for the second)
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
     const float x0 = __shfl((float)xf[mt][0][0], lq, kWave);
@@ -140,8 +140,18 @@ __global__ __launch_bounds__(64 * kMlpWaves) __attribute__((amdgpu_waves_per_eu(
       }
     const float sm = pair_sum(s) * (1.0f / K);
     const float var = fmaxf(pair_sum(q) * (1.0f / K) - sm * sm, 0.f);
-    ln_a[mt] = rsqrtf(var + eps);
-    s_stat[(wave * MT + mt) * 64 + lane] = make_float2(-(x0 + sm), (var + eps) * ln_a[mt]);
+    const float rstd = rsqrtf(var + eps), shift = -(x0 + sm) * rstd;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      u32x4_t raw = __builtin_bit_cast(u32x4_t, xf[mt][ks]);
+      asm volatile("" : "+v"(raw));
+      u32x4_t pk;
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        pk[e] = pack_bf16x2(__builtin_fmaf(bf16_lo(raw[e]), rstd, shift), __builtin_fmaf(bf16_hi(raw[e]), rstd, shift));
+      asm volatile("" : "+v"(pk));
+      xf[mt][ks] = __builtin_bit_cast(bf16x8_t, pk);
+    }
   }
 
 #pragma unroll
@@ -230,24 +240,16 @@ __global__ __launch_bounds__(64 * kMlpWaves) __attribute__((amdgpu_waves_per_eu(
 #pragma unroll
     for (int ks = 0; ks < kAhead; ++ks) read_frag(ks);
     {
-      // LayerNorm correction k-step: table rows (wsum_hi, wsum_hi, wsum_lo, b'_hi, b'_hi, b'_lo, 0, 0) against
-      // (m_hi, m_lo, m_hi, s_hi, s_lo, s_hi, 0, 0) of the row, rebuilt here from two floats per tile
+      // bias k-step: the table rows (wsum_hi, wsum_hi, wsum_lo, b'_hi, b'_hi, b'_lo, 0, 0) against (0, 0, 0, 1, 0, 1, 0, 0)
+      // start the accumulators from b' = b'_hi + b'_lo (exact: products with 1 in fp32)
       bf16x8_t tf[2];
 #pragma unroll
       for (int nt = 0; nt < 2; ++nt) tf[nt] = *reinterpret_cast<const bf16x8_t*>(s_side + slot * 1024 + (nt * 32 + lq) * 16);
       bf16x8_t xe[MT];
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) {
-        const float2 ms = s_stat[(wave * MT + mt) * 64 + lane];
-        const float m = ms.x, sd = ms.y;
-        const uint32_t hi = pack_bf16x2(m, sd);
-        const uint32_t lo = pack_bf16x2(m - bf16_lo(hi), sd - bf16_hi(hi));
-        u32x4_t d;
-        d[0] = (hi & 0xFFFFu) | (lo << 16);
-        d[1] = hi;
-        d[2] = (lo >> 16) | (hi & 0xFFFF0000u);
-        d[3] = 0u;
-        if (half != 0) { d[0] = 0u; d[1] = 0u; d[2] = 0u; }
+        u32x4_t d = {0u, half == 0 ? 0x3F800000u : 0u, half == 0 ? 0x3F800000u : 0u, 0u};
+        asm volatile("" : "+v"(d));   // rebuilt per chunk: four registers are not worth holding
         xe[mt] = __builtin_bit_cast(bf16x8_t, d);
       }
       const f32x16_t zero = {};
@@ -270,10 +272,10 @@ __global__ __launch_bounds__(64 * kMlpWaves) __attribute__((amdgpu_waves_per_eu(
           acc1[nt][mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[ks][nt], xb[mt], acc1[nt][mt], 0, 0, 0);
     }
     // Pin the issue order (left alone, the scheduler sinks every LDS read to just before its first use, which
-    // exposes the whole LDS latency twice per k-step): the row statistics, the table rows and kAhead k-steps of
-    // fragments first, then the correction products, then per k-step its products followed by the reads of the
+    // exposes the whole LDS latency twice per k-step): the table rows and kAhead k-steps of
+    // fragments first, then the bias products, then per k-step its products followed by the reads of the
     // k-step kAhead later (w fragments, and the x operands that live in LDS)
-    __builtin_amdgcn_sched_group_barrier(0x100, MT + 2 + 2 * kAhead + (kAhead > KSR ? MT * (kAhead - KSR) : 0), 0);
+    __builtin_amdgcn_sched_group_barrier(0x100, 2 + 2 * kAhead + (kAhead > KSR ? MT * (kAhead - KSR) : 0), 0);
     __builtin_amdgcn_sched_group_barrier(0x008, 2 * MT, 0);
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
@@ -294,8 +296,8 @@ __global__ __launch_bounds__(64 * kMlpWaves) __attribute__((amdgpu_waves_per_eu(
   auto gate_piece = [&](int mt, int q) __attribute__((always_inline)) {
     const int s = q / 4, p = q % 4;
     const int e0 = (2 * s + p / 2) * 4 + (p % 2) * 2;   // accumulator index g * 4 + r of element 2 p
-    const float v0 = fast_silu(acc1[0][mt][e0] * ln_a[mt]) * (acc1[1][mt][e0] * ln_a[mt]);
-    const float v1 = fast_silu(acc1[0][mt][e0 + 1] * ln_a[mt]) * (acc1[1][mt][e0 + 1] * ln_a[mt]);
+    const float v0 = fast_silu(acc1[0][mt][e0]) * acc1[1][mt][e0];
+    const float v1 = fast_silu(acc1[0][mt][e0 + 1]) * acc1[1][mt][e0 + 1];
     hb[mt][s][p] = pack_bf16x2(v0, v1);
   };
   // fc2 of chunk c, row tile mt, output tiles ot and ot + 1 (two independent accumulators alternate)
@@ -468,7 +470,7 @@ int f3d_ln_mlp_swiglu_bf16(const f3d_bf16_t* x, uint32_t ldx, const f3d_bf16_t* 
   uint16_t* w2p = (uint16_t*)(ws + w1_bytes + tab_bytes);
   uint16_t* zero_bias = (uint16_t*)(ws + w1_bytes + tab_bytes + w2_bytes);
   if (!b2) b2 = zero_bias;
-  launch_ln_fold(w1, gamma, beta, b1, w1p, table, 2 * hidden, c, s);
+  launch_ln_fold(w1, gamma, beta, b1, w1p, table, nullptr, 2 * hidden, c, s);
   hipLaunchKernelGGL(mlp_w2_prep_kernel, dim3(cdiv_u32(c * hidden / 8, 256)), dim3(256), 0, s, w2, w2p, zero_bias, c, hidden);
   int rc;
   if (c == 256) rc = launch_mlp<256>(x, ldx, eps, w1p, table, w2p, b2, residual, ldr, y, ldy, m, hidden, device, s);

@@ -12,6 +12,7 @@ typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16_t;
 
 constexpr int kXsChunk = 64;   // w rows per chunk (two 32-wide MFMA tiles)
 constexpr int kXsBufs = 3;     // w chunk buffers in LDS
+constexpr int kXsBiasSlots = 3;  // per-chunk bias slots in LDS (256 bytes each)
 constexpr int kPatchRow = 40;  // epilogue patch: 32 output columns + 8 pad (80-byte pitch keeps 16-byte alignment)
 
 __device__ __forceinline__ float fast_silu(float a) {
@@ -44,18 +45,35 @@ __device__ __forceinline__ void xs_lds_dma16(const void* gbase, uint32_t voff, c
                : "memory", "m0");
 }
 
+// the same with 4 bytes per lane (lane l lands at lds + 4 l) and with 2 bytes per lane, zero-extended to 4
+__device__ __forceinline__ void xs_lds_dma4(const void* gbase, uint32_t voff, const char* lds) {
+  const uint32_t lds_addr =
+      __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(__attribute__((address_space(3))) const char*)lds);
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2"
+               :
+               : "s"(lds_addr), "v"(voff), "s"(gbase)
+               : "memory", "m0");
+}
+__device__ __forceinline__ void xs_lds_dma2(const void* gbase, uint32_t voff, const char* lds) {
+  const uint32_t lds_addr =
+      __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(__attribute__((address_space(3))) const char*)lds);
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_ushort %1, %2"
+               :
+               : "s"(lds_addr), "v"(voff), "s"(gbase)
+               : "memory", "m0");
+}
+
 // s_waitcnt vmcnt(n) for a small run-time n (the instruction takes an immediate)
 __device__ __forceinline__ void xs_wait_vm(uint32_t n) {
+  // vmcnt is split over bits 3:0 and 15:14 of the immediate; expcnt and lgkmcnt stay at "no wait"
+#define F3D_VM(N) case N: __builtin_amdgcn_s_waitcnt(0x0F70 | ((N) & 15) | (((N) >> 4) << 14)); break;
   switch (n) {
-    case 0: __builtin_amdgcn_s_waitcnt(0x0F70); break;
-    case 1: __builtin_amdgcn_s_waitcnt(0x0F71); break;
-    case 2: __builtin_amdgcn_s_waitcnt(0x0F72); break;
-    case 3: __builtin_amdgcn_s_waitcnt(0x0F73); break;
-    case 4: __builtin_amdgcn_s_waitcnt(0x0F74); break;
-    case 5: __builtin_amdgcn_s_waitcnt(0x0F75); break;
-    case 6: __builtin_amdgcn_s_waitcnt(0x0F76); break;
+    F3D_VM(0) F3D_VM(1) F3D_VM(2) F3D_VM(3) F3D_VM(4) F3D_VM(5) F3D_VM(6) F3D_VM(7) F3D_VM(8) F3D_VM(9) F3D_VM(10)
+    F3D_VM(11) F3D_VM(12) F3D_VM(13) F3D_VM(14) F3D_VM(15) F3D_VM(16) F3D_VM(17) F3D_VM(18) F3D_VM(19) F3D_VM(20)
+    F3D_VM(21) F3D_VM(22) F3D_VM(23) F3D_VM(24)
     default: __builtin_amdgcn_s_waitcnt(0x0F70); break;
   }
+#undef F3D_VM
 }
 
 template <int K>
@@ -70,8 +88,9 @@ struct XsGeom {
   __host__ __device__ static constexpr uint32_t swz(uint32_t row) { return (row / RP) & SWZ_MASK; }
 };
 
-// w' = bf16(w * gamma) and the per-feature table of the algebraic LayerNorm fold (defined with the linear kernels)
+// w' = bf16(w * gamma), the per-feature table (wsum and b' = b + w beta in bf16 parts) and, when bias32 is not null,
+// b' as fp32 (defined with the linear kernels)
 void launch_ln_fold(const uint16_t* w, const uint16_t* gamma, const uint16_t* beta, const uint16_t* bias, uint16_t* wp,
-                    uint16_t* lnx, uint32_t N, uint32_t K, hipStream_t s);
+                    uint16_t* lnx, float* bias32, uint32_t N, uint32_t K, hipStream_t s);
 
 }  // namespace f3d

@@ -17,14 +17,10 @@
 // chunk c+2 is requested when chunk c starts.  Rows are unpadded; the 16-byte piece p of chunk-row r sits
 // at position p ^ swz(r), which spreads the 32 rows of one fragment read over all banks.
 //
-// LayerNorm is folded algebraically instead of being applied to x:
-//     LN(x) wT + b  =  rstd * (x w'T - mean * wsum) + b',   w' = w * gamma,  wsum[n] = sum_k w'[n][k],
-//                                                            b' = b + w beta.
-// A small kernel prepares w' (bf16) and, per output feature, wsum and b' split into high and low bf16 parts; the main
-// kernel needs the row statistics (one sweep over the registers that hold x) and applies the correction on the
-// matrix core: one extra k-step multiplies (wsum_hi, wsum_hi, wsum_lo, b'_hi, b'_hi, b'_lo) by the row's
-// (m_hi, m_lo, m_hi, s_hi, s_lo, s_hi), m = -mean, s = 1 / rstd, which adds -mean * wsum + s * b' to the
-// accumulator to 16 bits of mantissa; the epilogue then multiplies by rstd.
+// LayerNorm is applied to the rows while they sit in registers: one sweep for the statistics, one that replaces
+// x by bf16((x - mean) * rstd) (the reference's LayerNorm also hands bf16 to its Linear).  gamma and beta are folded
+// into the weights by a small kernel:  LN(x) wT + b = xhat w'T + b',  w' = bf16(w * gamma),  b' = b + w beta (fp32).
+// The main loop then is the plain one with bias b'.
 #include "xstat_common.h"
 
 namespace f3d {
@@ -35,11 +31,11 @@ constexpr size_t xs_lds_bytes() {
   const size_t wbuf = (size_t)NBUF * G::CHUNK_BYTES;
   const size_t xpatch = (size_t)WAVES * 32 * (G::KP + 8) * 2;
   const size_t front = wbuf > xpatch ? wbuf : xpatch;
-  return front + (size_t)WAVES * 32 * kPatchRow * 2 + (size_t)NBUF * 1024;
+  return front + (size_t)WAVES * 32 * kPatchRow * 2 + (size_t)kXsBiasSlots * 256;
 }
 
 // EPI: 0 = bias only, 1 = runtime activation and / or residual, 2 = residual only (its pieces are prefetched).
-// With LN the kernel expects w = w' and the table lnx as prepared by ln_fold_kernel.
+// With LN the kernel expects w = w' and lnx = b' as fp32 [N], both prepared by ln_fold_kernel.
 // NBUF: w chunk buffers in LDS (chunk c + NBUF - 1 is requested when chunk c starts).
 template <int K, int MT, int WAVES, int NBUF, bool LN, bool SWIGLU, int EPI>
 __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2))) void xstat_linear_kernel(
@@ -58,9 +54,9 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
                                 : (size_t)WAVES * 32 * (G::KP + 8) * 2;
   constexpr uint32_t kAheadChunks = NBUF - 1;
   uint16_t* lds_patch = reinterpret_cast<uint16_t*>(lds_xs + kFront);
-  // per chunk slot, 1 KB: the chunk's bias as fp32 (plain) or its 64 rows of the LayerNorm table (16 bytes each)
+  // the bias of a chunk as fp32 (64 values), three slots: chunk c + 2 is parked while chunk c is being read
   char* s_side = lds_xs + kFront + (size_t)WAVES * 32 * kPatchRow * 2;
-  auto s_bias = [&](uint32_t slot) -> float* { return reinterpret_cast<float*>(s_side + slot * 1024); };
+  auto s_bias = [&](uint32_t c) -> float* { return reinterpret_cast<float*>(s_side + (c % kXsBiasSlots) * 256); };
 
   const uint32_t tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid / kWave), lane = tid % kWave;
   const uint32_t lq = lane & 31u, half = lane >> 5;
@@ -96,10 +92,8 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
           xf[mt][kp * (KP / 16) + ks] = *reinterpret_cast<const bf16x8_t*>(patch + lq * PROW + ks * 16 + half * 8);
       }
   }
-  // LayerNorm statistics of this lane's rows: one sweep, sums of d = x - x0 and d^2, shifted by the row's
-  // first element so that the variance does not cancel
-  float ln_a[MT];             // rstd of this lane's row
-  float ln_m[MT], ln_s[MT];   // -mean and 1 / rstd: the correction k-step's B operand is rebuilt from them per chunk
+  // LayerNorm of this lane's rows in place: one sweep for the sums of d = x - x0 and d^2 (shifted by the row's first
+  // element so that the variance does not cancel), one that writes bf16((x - mean) * rstd) back
   if (LN) {
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
@@ -115,9 +109,20 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
         }
       const float sm = pair_sum(s) * (1.0f / K);
       const float var = fmaxf(pair_sum(q) * (1.0f / K) - sm * sm, 0.f);
-      ln_a[mt] = rsqrtf(var + eps);
-      ln_m[mt] = -(x0 + sm);
-      ln_s[mt] = (var + eps) * ln_a[mt];
+      const float rstd = rsqrtf(var + eps), shift = -(x0 + sm) * rstd;
+      // one fragment at a time (kept opaque: otherwise the compiler holds every row element as a float from the first
+      // sweep to the second, 8 registers per fragment, and spills)
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        u32x4_t raw = __builtin_bit_cast(u32x4_t, xf[mt][ks]);
+        asm volatile("" : "+v"(raw));
+        u32x4_t pk;
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          pk[e] = pack_bf16x2(__builtin_fmaf(bf16_lo(raw[e]), rstd, shift), __builtin_fmaf(bf16_hi(raw[e]), rstd, shift));
+        asm volatile("" : "+v"(pk));
+        xf[mt][ks] = __builtin_bit_cast(bf16x8_t, pk);
+      }
     }
   }
   __syncthreads();  // the transposition patches are dead; the space now holds w chunks
@@ -136,8 +141,15 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
   // direct loads of chunk c into buffer slot: instruction q fills LDS bytes [1024 q, 1024 q + 1024) of the
   // buffer, i.e. chunk rows [q * 64 / CPR, ...); wave v issues instructions v, v + WAVES, ...
   constexpr uint32_t kMyDmaMax = (G::N_DMA + WAVES - 1) / WAVES;
-  const uint32_t my_dma = G::N_DMA / WAVES + (wave < (uint32_t)(G::N_DMA % WAVES) ? 1u : 0u) + ((LN && wave == 0) ? 1u : 0u);
-  auto dma_chunk = [&](uint32_t c, uint32_t slot) {
+  const bool bias_dma = LN || bias != nullptr;
+  const uint32_t my_dma = G::N_DMA / WAVES + (wave < (uint32_t)(G::N_DMA % WAVES) ? 1u : 0u) + ((bias_dma && wave == 0) ? 1u : 0u);
+  auto dma_chunk = [&](uint32_t c, uint32_t c_seq, uint32_t slot) {   // c: the chunk, c_seq: its place in this workgroup's order
+    // the chunk's 64 bias values go to its bias slot: fp32 b' with LN, else the bf16 bits zero-extended to a dword
+    if (wave == 0) {
+      char* sb = reinterpret_cast<char*>(s_bias(c_seq));
+      if (LN) xs_lds_dma4(lnx, w_row(c, lane) * 4u, sb);
+      else if (bias) xs_lds_dma2(bias, w_row(c, lane) * 2u, sb);
+    }
     const char* buf = lds_xs + slot * G::CHUNK_BYTES;
 #pragma unroll
     for (uint32_t i = 0; i < kMyDmaMax; ++i) {
@@ -148,18 +160,7 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
         xs_lds_dma16(w, (w_row(c, r) * K + piece * 8u) * 2u, buf + qi * 1024);
       }
     }
-    if (LN && wave == 0) xs_lds_dma16(lnx, w_row(c, lane) * 16u, s_side + slot * 1024);   // table rows of the chunk
   };
-  // bias (and wsum) of a chunk: every wave issues the same loads so that the wait constants below hold
-  // for all of them; wave 0 parks the values in LDS one chunk later
-  float rb = 0.f;
-  auto load_bias = [&](uint32_t c) {
-    if (!LN) rb = bias ? bf16_bits_to_float(bias[w_row(c, lane)]) : 0.f;
-  };
-  auto park_bias = [&](uint32_t slot) {
-    if (!LN && wave == 0) s_bias(slot)[lane] = rb;
-  };
-
   const bool wg_full = (blockIdx.x + 1) * ROWS_WG <= M;
   uint16_t* y_wg = y + (size_t)(blockIdx.x * ROWS_WG) * ldy;                  // wave-uniform bases
   const uint16_t* res_wg = residual ? residual + (size_t)(blockIdx.x * ROWS_WG) * ldr : nullptr;
@@ -169,11 +170,9 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
   const uint32_t c_start = (blockIdx.x * 5u) % nchunk;
   auto actual = [&](uint32_t i) -> uint32_t { const uint32_t t = i + c_start; return t >= nchunk ? t - nchunk : t; };
 
-  dma_chunk(actual(0), 0);
-  if (kAheadChunks > 1 && nchunk > 1) dma_chunk(actual(1), 1);
-  load_bias(actual(0));
-  park_bias(0);
-  if (nchunk > 1) load_bias(actual(1));
+  if (!bias_dma && tid < 64 * kXsBiasSlots) reinterpret_cast<float*>(s_side)[tid] = 0.f;   // no bias: zeros, once
+  dma_chunk(actual(0), 0, 0);
+  if (kAheadChunks > 1 && nchunk > 1) dma_chunk(actual(1), 1, 1);
   __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): the first chunk(s) have landed
   __syncthreads();
 
@@ -184,25 +183,25 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
   // accumulators: acc[nt][mt][g*4+r] <-> column nt*32 + g*8 + half*4 + r
   f32x16_t acc[2][MT];
 
-  // stage 1: requests for chunk ci + NBUF - 1 (its buffer was last read in chunk ci-1, which every wave
-  // has left) and the bias hand-over
+  // stage 1: requests for chunk ci + NBUF - 1 (its buffer and its bias slot were last read in chunk ci - 1, which
+  // every wave has left).  (Spread over the k-steps of stage 2 they break its issue pattern: measured 10 % slower.)
   auto stage_request = [&](uint32_t ci) {
-    if (ci + kAheadChunks < nchunk) dma_chunk(actual(ci + kAheadChunks), (ci + kAheadChunks) % NBUF);
-    if (ci + 1 < nchunk) park_bias((ci + 1) % NBUF);
-    if (ci + 2 < nchunk) load_bias(actual(ci + 2));
+    if (ci + kAheadChunks < nchunk) dma_chunk(actual(ci + kAheadChunks), ci + kAheadChunks, (ci + kAheadChunks) % NBUF);
   };
-  // stage 2: the MFMAs of chunk ci; the accumulators start from the bias (from zero with LN, where the bias
-  // enters the correction of the epilogue)
+  // stage 2: the MFMAs of chunk ci; the accumulators start from the bias
   auto stage_mfma = [&](uint32_t ci) {
     const uint32_t slot = ci % NBUF;
     const char* sw = lds_xs + slot * G::CHUNK_BYTES;
-    const float* sb = s_bias(slot);
+    const float* sb = s_bias(ci);
 #pragma unroll
     for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
-        float4 b4 = {0.f, 0.f, 0.f, 0.f};
-        if (!LN) b4 = *reinterpret_cast<const float4*>(sb + nt * 32 + g * 8 + half * 4);
+        float4 b4 = *reinterpret_cast<const float4*>(sb + nt * 32 + g * 8 + half * 4);
+        if (!LN) {   // bf16 bits in the low half of each dword
+          b4.x = __uint_as_float(__float_as_uint(b4.x) << 16); b4.y = __uint_as_float(__float_as_uint(b4.y) << 16);
+          b4.z = __uint_as_float(__float_as_uint(b4.z) << 16); b4.w = __uint_as_float(__float_as_uint(b4.w) << 16);
+        }
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
           acc[nt][mt][g * 4 + 0] = b4.x; acc[nt][mt][g * 4 + 1] = b4.y;
@@ -220,34 +219,6 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
     };
 #pragma unroll
     for (int ks = 0; ks < kAhead; ++ks) read_frag(ks);
-    if (LN) {
-      // correction k-step: the chunk's table rows against the row statistics
-      bf16x8_t tf[2];
-#pragma unroll
-      for (int nt = 0; nt < 2; ++nt) tf[nt] = *reinterpret_cast<const bf16x8_t*>(s_side + slot * 1024 + (nt * 32 + lq) * 16);
-      // B operand (m_hi, m_lo, m_hi, s_hi, s_lo, s_hi, 0, 0) in the lanes of the lower half, zeros in the upper
-      // half; built here from two floats per tile (kept opaque so that it is not hoisted into eight registers)
-      bf16x8_t xe[MT];
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt) {
-        float m = ln_m[mt], sd = ln_s[mt];
-        asm volatile("" : "+v"(m), "+v"(sd));
-        const uint32_t hi = pack_bf16x2(m, sd);                                  // m_hi | s_hi << 16
-        const uint32_t lo = pack_bf16x2(m - bf16_lo(hi), sd - bf16_hi(hi));      // m_lo | s_lo << 16
-        u32x4_t d;
-        d[0] = (hi & 0xFFFFu) | (lo << 16);          // m_hi, m_lo
-        d[1] = hi;                                   // m_hi, s_hi
-        d[2] = (lo >> 16) | (hi & 0xFFFF0000u);      // s_lo, s_hi
-        d[3] = 0u;
-        if (half != 0) { d[0] = 0u; d[1] = 0u; d[2] = 0u; }
-        xe[mt] = __builtin_bit_cast(bf16x8_t, d);
-      }
-#pragma unroll
-      for (int nt = 0; nt < 2; ++nt)
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt)
-          acc[nt][mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tf[nt], xe[mt], acc[nt][mt], 0, 0, 0);
-    }
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       if (ks + kAhead < KS) read_frag(ks + kAhead);
@@ -258,8 +229,7 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
           acc[nt][mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[ks][nt], xf[mt][ks], acc[nt][mt], 0, 0, 0);
     }
     // pin the issue order: kAhead k-steps of LDS reads first, then one k-step of reads per k-step of MFMAs
-    __builtin_amdgcn_sched_group_barrier(0x100, 2 * kAhead + (LN ? 2 : 0), 0);
-    if (LN) __builtin_amdgcn_sched_group_barrier(0x008, 2 * MT, 0);
+    __builtin_amdgcn_sched_group_barrier(0x100, 8 + 2 * kAhead, 0);   // the 8 bias reads come first
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       __builtin_amdgcn_sched_group_barrier(0x008, 2 * MT, 0);
@@ -271,14 +241,6 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
   auto stage_epilogue = [&](uint32_t ci) {
     const uint32_t slot = ci % NBUF;
     const uint32_t col0 = actual(ci) * COLS;   // first output column of the chunk
-    if (LN) {
-#pragma unroll
-      for (int nt = 0; nt < 2; ++nt)
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-          for (int e = 0; e < 16; ++e) acc[nt][mt][e] *= ln_a[mt];
-    }
     // Residual pieces of the whole chunk are requested up front (one memory latency for all of them, hidden
     // behind the packing below) instead of one by one where they are added.  Rows past M read row M - 1.
     constexpr int NT_OUT = SWIGLU ? 1 : 2;
@@ -365,21 +327,24 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
     };
     if (wg_full) epilogue(std::true_type{}); else epilogue(std::false_type{});
   };
-  // "Everything this wave issued before chunk ci's requests has completed" holds once at most that many
-  // operations are outstanding, PROVIDED nothing younger than the requests has been issued yet; that
-  // includes this wave's share of chunk ci+1 (requested one chunk ago).  The count ignores the bias loads
-  // (wherever the compiler places them, the wait is then exact or slightly early, never late).
+  // Chunk ci + 1 must have landed when the interval ends.  Its requests were issued one interval ago; since then this
+  // wave has issued the memory operations of one epilogue (stores, and the residual loads of EPI 2: kEpiOps of them
+  // when every row of the workgroup is stored) and the requests of chunk ci + 2 (my_dma).  Memory operations complete
+  // in order, so "at most that many outstanding" is the weakest wait that covers chunk ci + 1, and it does not wait
+  // for the stores.  Where the epilogue's count is not fixed (partial workgroup, run-time residual) the stores are
+  // not allowed for: the wait is then early, never late.
+  constexpr uint32_t kEpiOps = EPI == 1 ? 0u : (uint32_t)(MT * (SWIGLU ? 1 : 2) * 2 * (EPI == 2 ? 2 : 1));
+  const uint32_t wait_n = my_dma + (wg_full ? kEpiOps : 0u);
   auto wait_next_chunk = [&](uint32_t ci) {
-    if (kAheadChunks > 1 && ci + kAheadChunks < nchunk) xs_wait_vm(my_dma); else __builtin_amdgcn_s_waitcnt(0x0F70);
+    if (kAheadChunks > 1 && ci + kAheadChunks < nchunk) xs_wait_vm(wait_n); else __builtin_amdgcn_s_waitcnt(0x0F70);
   };
 
   // The two waves that share a SIMD (wave v and v + WAVES/2) run the stages of a barrier interval in
   // complementary order, so that one's epilogue (VALU, LDS, stores) overlaps the other's MFMAs:
   //   first half :  request(c)  mfma(c)      wait  epilogue(c)   | barrier
   //   second half:  epilogue(c-1)  request(c)  mfma(c)  wait      | barrier      (+ epilogue(last) at the end)
-  // Both halves read chunk c's buffer inside the same interval, so the buffer rotation is unchanged; the
-  // late epilogue only reads the bias slot of chunk c-1, which with three slots is not rewritten before
-  // interval c+1.  The stores of a late epilogue are older than the requests that follow them, as the wait needs.
+  // Both halves read chunk c's buffer and bias slot inside the same interval, so the rotations are unchanged.
+  // The stores of a late epilogue are older than the requests that follow them, as the wait needs.
   const bool late_half = NBUF >= 3 && WAVES >= 8 && wave >= (uint32_t)(WAVES / 2);
   if (!late_half) {
     for (uint32_t ci = 0; ci < nchunk; ++ci) {
@@ -387,7 +352,7 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
       stage_mfma(ci);
       wait_next_chunk(ci);
       stage_epilogue(ci);
-      __syncthreads();
+      wg_barrier_lds();
     }
   } else {
     for (uint32_t ci = 0; ci < nchunk; ++ci) {
@@ -395,20 +360,21 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
       stage_request(ci);
       stage_mfma(ci);
       wait_next_chunk(ci);
-      __syncthreads();
+      wg_barrier_lds();
     }
     stage_epilogue(nchunk - 1);
   }
 }
 
-// w' = bf16(w * gamma) and the table row of every output feature n:
+// w' = bf16(w * gamma), b' as fp32 (bias32, may be null) and the table row of every output feature n:
 //   (wsum_hi, wsum_hi, wsum_lo, b'_hi, b'_hi, b'_lo, 0, 0) in bf16, with
 //   wsum[n] = sum_k w'[n][k] (of the rounded values the matrix core will see), b'[n] = bias[n] + sum_k w[n][k] * beta[k].
 // One wave per output feature.
 __global__ __launch_bounds__(256) void ln_fold_kernel(const uint16_t* __restrict__ w, const uint16_t* __restrict__ gamma,
                                                       const uint16_t* __restrict__ beta,
                                                       const uint16_t* __restrict__ bias, uint16_t* __restrict__ wp,
-                                                      uint16_t* __restrict__ lnx, uint32_t N, uint32_t K) {
+                                                      uint16_t* __restrict__ lnx, float* __restrict__ bias32,
+                                                      uint32_t N, uint32_t K) {
   const uint32_t n = blockIdx.x * 4 + threadIdx.x / kWave, lane = threadIdx.x % kWave;
   if (n >= N) return;
   float s = 0.f, t = 0.f;
@@ -431,12 +397,13 @@ __global__ __launch_bounds__(256) void ln_fold_kernel(const uint16_t* __restrict
     const uint16_t b_lo = float_to_bf16_bits(b - bf16_bits_to_float(b_hi));
     uint16_t* row = lnx + (size_t)n * 8;
     row[0] = s_hi; row[1] = s_hi; row[2] = s_lo; row[3] = b_hi; row[4] = b_hi; row[5] = b_lo; row[6] = 0; row[7] = 0;
+    if (bias32) bias32[n] = b;
   }
 }
 
 void launch_ln_fold(const uint16_t* w, const uint16_t* gamma, const uint16_t* beta, const uint16_t* bias, uint16_t* wp,
-                    uint16_t* lnx, uint32_t N, uint32_t K, hipStream_t s) {
-  hipLaunchKernelGGL(ln_fold_kernel, dim3(cdiv_u32(N, 4)), dim3(256), 0, s, w, gamma, beta, bias, wp, lnx, N, K);
+                    uint16_t* lnx, float* bias32, uint32_t N, uint32_t K, hipStream_t s) {
+  hipLaunchKernelGGL(ln_fold_kernel, dim3(cdiv_u32(N, 4)), dim3(256), 0, s, w, gamma, beta, bias, wp, lnx, bias32, N, K);
 }
 
 template <int K, int MT, int WAVES, int NBUF>
@@ -482,15 +449,17 @@ int launch_xstat_linear(const uint16_t* x, uint32_t ldx, const uint16_t* gamma, 
   if ((uint64_t)N * K * 2 >= (1ull << 32)) return F3D_ERR_UNSUPPORTED;   // 32-bit byte offsets into w
   const uint16_t* lnx = nullptr;
   if (ln) {
-    // per call: w' (bf16 [N][K]) and the table (bf16 [N][8]) in the per-device workspace
+    // per call: w' (bf16 [N][K]), the table (bf16 [N][8], unused by this kernel) and b' (fp32 [N]) in the per-device
+    // workspace
     const size_t wp_bytes = ((size_t)N * K * 2 + 255) & ~(size_t)255;
-    char* ws = (char*)workspace(device, wp_bytes + (size_t)N * 16);
+    char* ws = (char*)workspace(device, wp_bytes + (size_t)N * 16 + (size_t)N * 4);
     if (!ws) return F3D_ERR_RUNTIME;
     uint16_t* wp = (uint16_t*)ws;
     uint16_t* table = (uint16_t*)(ws + wp_bytes);
-    launch_ln_fold(w, gamma, beta, bias, wp, table, N, K, s);
+    float* b32 = (float*)(ws + wp_bytes + (size_t)N * 16);
+    launch_ln_fold(w, gamma, beta, bias, wp, table, b32, N, K, s);
     w = wp;
-    lnx = table;
+    lnx = (const uint16_t*)b32;   // the kernel reads b' from here
   }
   // Large panels (64 rows per wave, 8 waves, 3 chunk buffers: one workgroup per CU) when their workgroups fill
   // at least three quarters of the chip, otherwise 32 rows per wave in 4-wave workgroups with 2 buffers

@@ -105,7 +105,7 @@ __global__ __launch_bounds__(64 * kYsWaves) __attribute__((amdgpu_waves_per_eu(2
   if (nchunk > 2) dma_chunk(2);
   // chunk 0 must have landed; up to two younger chunks may stay in flight
   ys_wait_vm(nchunk > 2 ? 2 * kPerChunk : (nchunk > 1 ? kPerChunk : 0));
-  __syncthreads();
+  wg_barrier_lds();
 
   for (uint32_t ci = 0; ci < nchunk; ++ci) {
     // chunk ci + 3 goes into the buffer of chunk ci - 1, which every wave has left
@@ -129,8 +129,9 @@ __global__ __launch_bounds__(64 * kYsWaves) __attribute__((amdgpu_waves_per_eu(2
     // chunk ci + 1 must have landed: what may stay in flight are the chunks after it that have been requested
     const uint32_t requested = min(ci + 3, nchunk - 1);     // youngest chunk requested so far
     ys_wait_vm(requested > ci + 1 ? (requested - (ci + 1)) * kPerChunk : 0);
-    __syncthreads();
+    wg_barrier_lds();   // not __syncthreads(): that would also wait for the chunks that are meant to stay in flight
   }
+
 
   // ---- output: bf16 (+ residual), through a wave-private LDS patch so that the stores are row-contiguous.  The
   //      residual pieces of the wave's whole panel are requested first: one memory latency for all of them ----

@@ -206,7 +206,9 @@ def test_fused_mlp_matches_two_kernel_path(oracle, M, C, H, use_res, use_bias):
     torch.cuda.synchronize()
     d = (y.float() - y2.float()).abs()
     scale = y2.float().abs().clamp(min=1.0)
-    assert (d / scale).max().item() <= 2 ** -6, (d / scale).max().item()          # at most two bf16 steps apart
+    # a hidden value that rounds the other way (the fused kernel forms b' from its two bf16 parts, the two-kernel path
+    # from fp32) moves an output by a step or two before the final rounding: at most four bf16 steps apart
+    assert (d / scale).max().item() <= 2 ** -5, (d / scale).max().item()
     assert (d > 0).float().mean().item() < 0.02                                     # and almost always equal
     # (b) against the unrounded mathematics: at least as close as the reference's own sequence of bf16 roundings
     # (LayerNorm output, fc1 output, gated product, fc2 output, residual sum)
@@ -232,17 +234,21 @@ def test_fused_mlp_unsupported_width_is_reported():
     assert (y == 3.0).all()
 
 
-def test_layernorm_mlp_layer_fused_on_request():
-    """LayerNormMLP(fused=True) routes through the one-kernel gated MLP and agrees with the default two-kernel
-    path; gradients flow through it like through the default."""
+def test_layernorm_mlp_layer_one_kernel_and_two_kernel_paths():
+    """LayerNormMLP(fused=True) routes through the one-kernel gated MLP, fused=False through LayerNorm+fc1+gate and
+    fc2+residual; the default picks by size and equals one of them bit for bit; gradients flow through either."""
     from flash3dtransformer_amd.layers.nn_ops import LayerNormMLP
     torch.manual_seed(5)
-    a, b = LayerNormMLP(256, 512).to(DEV), LayerNormMLP(256, 512, fused=True).to(DEV)
+    a, b, auto = LayerNormMLP(256, 512, fused=False).to(DEV), LayerNormMLP(256, 512, fused=True).to(DEV), LayerNormMLP(256, 512).to(DEV)
     b.load_state_dict(a.state_dict())
+    auto.load_state_dict(a.state_dict())
     x = torch.randn(3000, 256, device=DEV).to(torch.bfloat16)
     ya, yb = a(x, residual=x), b(x, residual=x)
     d = (ya.float() - yb.float()).abs() / ya.float().abs().clamp(min=1.0)
-    assert d.max().item() <= 2 ** -6
+    assert d.max().item() <= 2 ** -5
+    assert torch.equal(auto(x, residual=x), ya)                       # 3,000 rows of width 256: two kernels
+    big = torch.randn(70000, 256, device=DEV).to(torch.bfloat16)
+    assert torch.equal(auto(big, residual=big), b(big, residual=big))   # 70,000 rows: one kernel
     xg = x.clone().requires_grad_(True)
     b(xg, residual=xg).float().square().mean().backward()
     assert xg.grad is not None and torch.isfinite(xg.grad.float()).all() and xg.grad.abs().max().item() > 0
