@@ -301,7 +301,7 @@ class LayerNormMLP(_CachedParamModule):
         # fused: run the whole gated MLP as one kernel where one exists (widths 128 / 256): the hidden activations
         # [rows, ffn_hidden_size] are then never allocated.  None (default): where it is the faster path on MI355X
         # (measured against LayerNorm+fc1+gate followed by fc2+residual, hidden = 4 x width: width 128 at every row
-        # count, 4 to 30 % faster; width 256 from 60 k rows up, 2 to 19 % faster, and 12 to 44 % slower below)
+        # count, 19 to 41 % faster; width 256 from 32 k rows up, 6 to 23 % faster, and 11 % slower at 16 k rows)
         self.fused = fused
         assert activation in ("swiglu", "gelu")
         self.hidden_size, self.ffn_hidden_size, self.activation, self.eps = hidden_size, ffn_hidden_size, activation, eps
@@ -322,7 +322,7 @@ class LayerNormMLP(_CachedParamModule):
         r2 = None if residual is None else as_bf16_2d(residual.reshape(-1, self.hidden_size))
         y = torch.empty_like(x2)
         # on request, the whole gated MLP in one kernel where one exists (hidden activations stay in registers) ...
-        want_fused = self.fused if self.fused is not None else (self.hidden_size == 128 or x2.shape[0] >= 60000)
+        want_fused = self.fused if self.fused is not None else (self.hidden_size == 128 or x2.shape[0] >= 30000)
         fused = (want_fused and self.activation == "swiglu" and self.hidden_size in FUSED_MLP_WIDTHS
                  and self.ffn_hidden_size % 32 == 0
                  and pshattn.ln_mlp_swiglu_bf16(x2, c[0].get(self.layer_norm_weight, self.training), c[1].get(self.layer_norm_bias, self.training),
