@@ -417,9 +417,11 @@ def _pool_case(dev, out, n, tag, iters):
 def hourglass_c5(dev):
     """whole-model forward, config 5: 4 sweeps x 250,000 points, 5 levels C = 32/64/128/256/512, heads = C/32,
     bucket 512, scope of 1 bucket, pooling S = 2 (mean), swiglu MLP with hidden = 4C, hash 2.
-    `ms`: wall time per forward, forwards queued back to back.  `gpu_busy_ms`: the sum of the kernel durations of one
-    forward, from the profiler's kernel records (None when the profiler is not usable, e.g. under an outer tracer);
-    the difference is time the GPU waited for the host."""
+    `ms`: wall time per forward, forwards queued back to back.  `host_enqueue_ms`: the time the host needs to queue
+    one forward (the call returns before the GPU is done): below `ms`, the host runs ahead and per-call marshalling
+    is not what the GPU waits for.  `gpu_busy_ms`: the sum of the kernel durations of one forward, from the
+    profiler's kernel records (None when the profiler is not usable, e.g. under an outer tracer); `ms` minus it is
+    the idle time between consecutive kernels."""
     from flash3dtransformer_amd import configs
     model = configs.hourglass(1005).to(dev).eval()
     coords_np, seps_np, _ = configs.lidar_batch(4, 250_000, 1005)
@@ -434,6 +436,11 @@ def hourglass_c5(dev):
             out = model(coords, None, seps)
         torch.cuda.synchronize()
     ms = (time.perf_counter() - t0) / iters * 1e3
+    with torch.no_grad():
+        t0 = time.perf_counter()
+        model(coords, None, seps)
+        enqueue_ms = (time.perf_counter() - t0) * 1e3
+        torch.cuda.synchronize()
     busy, n_kernels = None, None
     if not os.environ.get("ROCPROFILER_REGISTER_FORCE_LOAD") and not os.environ.get("ROCP_TOOL_LIBRARIES"):
         try:
@@ -447,7 +454,8 @@ def hourglass_c5(dev):
             n_kernels = sum(e.count for e in ka) // iters
         except Exception as exc:   # noqa: BLE001 - the timing above stands without it
             print(f"bench.py: kernel records unavailable ({type(exc).__name__}: {exc})", file=sys.stderr)
-    return {"ms": round(ms, 3), "gpu_busy_ms": None if busy is None else round(busy, 3),
+    return {"ms": round(ms, 3), "host_enqueue_ms": round(enqueue_ms, 3),
+            "gpu_busy_ms": None if busy is None else round(busy, 3),
             "launches_per_forward": n_kernels, "mpts_per_s": round(coords.shape[0] / ms / 1e3, 1), "points": int(coords.shape[0]),
             "levels": list(configs.HOURGLASS["channels"]), "subbuck_size": configs.HOURGLASS["subbuck_size"],
             "finite": bool(torch.isfinite(out.float()).all().item())}
