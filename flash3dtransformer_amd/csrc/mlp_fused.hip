@@ -260,20 +260,24 @@ __global__ __launch_bounds__(64 * kMlpWaves) __attribute__((amdgpu_waves_per_eu(
   // ---- output: bf16(fc2) (+ residual), through a wave-private LDS patch so that the stores are row-contiguous ----
   uint16_t* y_wg = y + (size_t)(blockIdx.x * ROWS_WG) * ldy;
   const uint16_t* res_wg = residual ? residual + (size_t)(blockIdx.x * ROWS_WG) * ldr : nullptr;
+  // the residual pieces of the wave's whole panel are requested at once (x is dead: its registers take them): one
+  // memory latency for all of them instead of one per column tile
+  u32x4_t rres[OT][2];
+  if (residual) {
+#pragma unroll
+    for (int ot = 0; ot < OT; ++ot)
+#pragma unroll
+      for (int h2 = 0; h2 < 2; ++h2) {
+        const uint32_t rr = (lane >> 2) + h2 * 16, ch = (lane & 3u) * 8;
+        const uint32_t row = min(row0 + rr, M - 1);            // rows past M read row M - 1
+        rres[ot][h2] = *reinterpret_cast<const u32x4_t*>(res_wg + ((row - blockIdx.x * ROWS_WG) * ldr + ot * 32 + ch));
+      }
+  }
   __syncthreads();   // every wave is done with the weight buffers: their space takes the output patches
   static_assert((size_t)WAVES * 32 * kPatchRow * 2 <= (size_t)NB1 * MG::CH1, "the output patches alias the w1 buffers");
   uint16_t* patch = reinterpret_cast<uint16_t*>(lds_mlp) + wave * (32 * kPatchRow);
 #pragma unroll
   for (int ot = 0; ot < OT; ++ot) {
-    u32x4_t rv[2] = {};
-    if (residual) {
-#pragma unroll
-      for (int h2 = 0; h2 < 2; ++h2) {
-        const uint32_t rr = (lane >> 2) + h2 * 16, ch = (lane & 3u) * 8;
-        const uint32_t row = min(row0 + rr, M - 1);            // rows past M read row M - 1
-        rv[h2] = *reinterpret_cast<const u32x4_t*>(res_wg + ((row - blockIdx.x * ROWS_WG) * ldr + ot * 32 + ch));
-      }
-    }
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
       uint2 pk;
@@ -290,7 +294,7 @@ __global__ __launch_bounds__(64 * kMlpWaves) __attribute__((amdgpu_waves_per_eu(
       if (residual) {
 #pragma unroll
         for (int e = 0; e < 4; ++e)
-          t[e] = pack_bf16x2(bf16_lo(t[e]) + bf16_lo(rv[h2][e]), bf16_hi(t[e]) + bf16_hi(rv[h2][e]));
+          t[e] = pack_bf16x2(bf16_lo(t[e]) + bf16_lo(rres[ot][h2][e]), bf16_hi(t[e]) + bf16_hi(rres[ot][h2][e]));
       }
       if (row < M) *reinterpret_cast<u32x4_t*>(y_wg + (lrow * ldy + ot * 32 + ch)) = t;
     }
