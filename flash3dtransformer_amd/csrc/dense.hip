@@ -420,7 +420,7 @@ int f3d_ln_linear_bf16(const f3d_bf16_t* x, uint32_t ldx, const f3d_bf16_t* gamm
   F3D_CHECK_ARG(k == 32 || k == 64 || k == 128 || k == 256 || k == 512,
                 "No kernel found for LayerNorm+Linear with inner dimension K=%u (supported: 32, 64, 128, 256, 512)", k);
   F3D_CHECK_ARG(n_out % 8 == 0 && (act != F3D_ACT_SWIGLU || n % 64 == 0), "output width %u must be a multiple of 8", n_out);
-  F3D_CHECK_ARG(ldx >= k && ldx % 8 == 0 && ldy >= n_out && ldy % 4 == 0 && (!residual || (ldr >= n_out && ldr % 4 == 0)),
+  F3D_CHECK_ARG(ldx >= k && ldx % 8 == 0 && ldy >= n_out && ldy % 8 == 0 && (!residual || (ldr >= n_out && ldr % 8 == 0)),
                 "row strides must be aligned and cover a row (ldx=%u ldy=%u ldr=%u)", ldx, ldy, ldr);
   F3D_CHECK_ARG((((uintptr_t)x | (uintptr_t)w | (uintptr_t)y | (uintptr_t)residual | (uintptr_t)gamma | (uintptr_t)beta) & 15u) == 0,
                 "x/w/y/residual/gamma/beta must be 16-byte aligned");

@@ -6,6 +6,7 @@ import torch
 import torch.cuda.nvtx as nvtx
 from torch import nn
 
+from ..psh import batching as f3dbatch
 from ..psh import dev_context as f3ddev
 from ..psh import psh_main as pm
 from . import hourglass as f3dhourglass
@@ -123,8 +124,7 @@ class Flash3D(nn.Module):
             psh_feat = psh_feat + self.input_proj(feat)
         tree_seps = seps
         if scattered.shape[0] != coords.shape[0]:
-            tree_seps = seps.clone()
-            tree_seps.view(torch.int32)[-1] = scattered.shape[0]
+            tree_seps = f3dbatch.with_last_separator(seps, scattered.shape[0])
         out = self.module_tree(scattered, psh_feat, tree_seps)
         if f3ddev.get_nvtx():
             nvtx.range_pop()

@@ -6,6 +6,7 @@ import torch
 import torch.cuda.nvtx as nvtx
 from torch import nn
 
+from ..psh import batching as f3dbatch
 from ..psh import dev_context as f3ddev
 from ..psh import subbuck as f3dsubbuck
 from . import pooling, unpool
@@ -96,8 +97,7 @@ class HourglassModule(nn.Module):
         # level belongs to a cloud and is written by the unpooling on the way back.
         sub_sep = buffers.reduced_sep
         if buffers.reduced_feat.shape[0] != buffers.unpool_ind.shape[0]:
-            sub_sep = sub_sep.clone()
-            sub_sep.view(torch.int32)[-1] = buffers.reduced_feat.shape[0]
+            sub_sep = f3dbatch.with_last_separator(sub_sep, buffers.reduced_feat.shape[0])
         sub_out = self.submodule(buffers.reduced_coord, reduced_feat, sub_sep)
         output = self.unpooling(residual_feat, sub_out, buffers)
         if f3ddev.get_nvtx():

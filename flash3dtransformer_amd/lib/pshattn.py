@@ -75,6 +75,15 @@ def assert_dtype(tensors, dtype):
             raise RuntimeError(f"Tensor #{i} has dtype {t.dtype}, expected {dtype}.")
 
 
+def _check_vectors(dev_ref, tensors, dtype=torch.bfloat16):
+    """optional 1-D operands (bias, beta, ...): same device as the call, the wire dtype, contiguous"""
+    ts = [t for t in tensors if t is not None]
+    if ts:
+        assert_same_device([dev_ref] + ts)
+        assert_dtype(ts, dtype)
+        assert_contiguous(ts)
+
+
 class DeviceManagerSingleton:
     """src/common/device_manager.{cuh,cu}; bound at src/f3d_frontend.cu:115-120"""
     _inst = None
@@ -464,11 +473,10 @@ def linear_bf16(x, w, bias, residual, y, act=None):
     n_out = n // 2 if a == 2 else n
     if w.shape[1] != k or tuple(y.shape) != (m, n_out):
         raise RuntimeError(f"linear shape mismatch: x{tuple(x.shape)} w{tuple(w.shape)} y{tuple(y.shape)}")
-    if bias is not None:
-        assert_dtype([bias], torch.bfloat16)
-        assert_contiguous([bias])
+    _check_vectors(x, [bias])
     ldr = 0
     if residual is not None:
+        assert_same_device([x, residual])
         assert_dtype([residual], torch.bfloat16)
         if tuple(residual.shape) != (m, n_out) or residual.stride(1) != 1:
             raise RuntimeError("residual must be [m, n_out] row-major")
@@ -491,8 +499,10 @@ def ln_linear_bf16(x, gamma, beta, eps, w, bias, residual, y, act=None):
     n_out = n // 2 if a == 2 else n
     if w.shape[1] != k or tuple(y.shape) != (m, n_out) or gamma.shape[0] != k:
         raise RuntimeError(f"ln_linear shape mismatch: x{tuple(x.shape)} w{tuple(w.shape)} y{tuple(y.shape)}")
+    _check_vectors(x, [beta, bias])
     ldr = 0
     if residual is not None:
+        assert_same_device([x, residual])
         assert_dtype([residual], torch.bfloat16)
         if tuple(residual.shape) != (m, n_out) or residual.stride(1) != 1:
             raise RuntimeError("residual must be [m, n_out] row-major")
@@ -509,6 +519,7 @@ def ln_mlp_swiglu_bf16(x, gamma, beta, eps, w1, b1, w2, b2, residual, y) -> bool
     dev = assert_same_device([x, gamma, w1, w2, y])
     assert_dtype([x, gamma, w1, w2, y], torch.bfloat16)
     assert_contiguous([w1, w2, gamma])
+    _check_vectors(x, [beta, b1, b2])
     if x.dim() != 2 or y.dim() != 2 or x.stride(1) != 1 or y.stride(1) != 1:
         raise RuntimeError("ln_mlp_swiglu_bf16 expects 2-D row-major x and y")
     m, c = x.shape
@@ -536,6 +547,7 @@ def layernorm_bf16(x, gamma, beta, y, eps=1e-5):
     assert_contiguous([x, gamma, y])
     dev = assert_same_device([x, gamma, y])
     assert_dtype([x, gamma, y], torch.bfloat16)
+    _check_vectors(x, [beta])
     m, c = x.shape
     _check(_load().f3d_layernorm_bf16(_ptr(x), _ptr(gamma), _ptr(beta), _ptr(y), _u32(m), _u32(c), _f32(eps),
                                       _i32(dev), _stream(dev)))
@@ -547,6 +559,7 @@ def coord_embed_bf16(coord, w, bias, y):
     dev = assert_same_device([coord, w, y])
     assert_dtype([coord], torch.float16)
     assert_dtype([w, y], torch.bfloat16)
+    _check_vectors(coord, [bias])
     _check(_load().f3d_coord_embed_bf16(_ptr(coord), _ptr(w), _ptr(bias), _ptr(y), _u32(coord.shape[0]),
                                         _u32(w.shape[0]), _i32(dev), _stream(dev)))
 

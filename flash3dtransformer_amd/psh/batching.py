@@ -25,7 +25,25 @@ def sep2sizes(seps: torch.Tensor) -> torch.Tensor:
 
 
 def max_inslen_from_seps(seps: torch.Tensor) -> int:
-    return int(sep2sizes(seps.to(torch.int64)).max())
+    """largest cloud of the batch, from the host-side sizes (one device->host copy per separator tensor, then none)"""
+    return max(host_sizes(seps))
+
+
+def with_last_separator(seps: torch.Tensor, total: int) -> torch.Tensor:
+    """A copy of `seps` whose last entry is `total` (rows appended for alignment are counted into the last cloud).
+    The copy is made once per separator tensor and length, and the host-side sizes of the copy are derived from those
+    of `seps`, so handing it on costs no host synchronisation."""
+    facts = host_facts(seps)
+    key = ("with_last", int(total))
+    if key not in facts:
+        out = seps.clone()
+        out.view(torch.int32)[-1] = int(total)
+        if "sizes" in facts:
+            sizes = list(facts["sizes"])
+            sizes[-1] += int(total) - sum(sizes)
+            host_facts(out)["sizes"] = sizes
+        facts[key] = out
+    return facts[key]
 
 
 def bulk_to(ts: List[torch.Tensor], dest):
