@@ -152,29 +152,29 @@ __global__ __launch_bounds__(64 * kMlpWaves) __attribute__((amdgpu_waves_per_eu(
   const uint32_t nchunk = H / 32;
   static_assert(G::N_DMA % WAVES == 0 && MG::N_DMA2 % WAVES == 0, "direct loads split evenly over the waves");
   constexpr uint32_t kDma1 = G::N_DMA / WAVES, kDma2 = MG::N_DMA2 / WAVES;
+  // One direct load moves 64 pieces = RPD w1 rows. The lane's byte offset inside such a group (its row of the group,
+  // its piece of the row under the row's swizzle) is the same for every group the wave loads, because the groups of
+  // one wave lie a multiple of 16 rows apart and the swizzle has period 16; everything else about an address is
+  // uniform and goes into the scalar base. (Addresses recomputed per load in vector registers cost the issuing wave
+  // about 60 cycles of dependent arithmetic each, with the matrix pipeline idle.)
+  constexpr uint32_t RPD = 64 / G::CPR;
+  static_assert((WAVES * RPD) % 16 == 0 && G::RP == 1 && 32 % RPD == 0, "one lane offset serves all groups of a wave");
+  const uint32_t w1_lane_off = ((lane / G::CPR) * K + (((lane % G::CPR) ^ G::swz(wave * RPD + lane / G::CPR)) * 8u)) * 2u;
+  const uint32_t tab_lane_off = (lane < 32 ? lane : H + lane - 32) * 16u;
   auto dma_chunk = [&](uint32_t c) __attribute__((always_inline)) {
-    // the lane's address parts are recomputed per chunk from an opaque copy of the lane number: hoisted out of the
-    // loop they would occupy registers that the loop does not have (and a spilled address is reloaded through the
-    // same counter the direct loads complete on)
-    uint32_t lane_o = lane;
-    asm volatile("" : "+v"(lane_o));
-    const uint32_t lane = lane_o;
     const char* b1 = w1buf + (c % NB1) * MG::CH1;
 #pragma unroll
     for (uint32_t i = 0; i < kDma1; ++i) {
-      const uint32_t qi = wave + i * WAVES;
-      const uint32_t r = (qi * 64u + lane) / G::CPR, p = lane % G::CPR;      // chunk row, position of the lane's piece
-      const uint32_t wrow = r < 32 ? c * 32u + r : H + c * 32u + (r - 32u);   // value rows, then gate rows
-      xs_lds_dma16(w1p, (wrow * K + (p ^ G::swz(r)) * 8u) * 2u, b1 + qi * 1024);
+      const uint32_t qi = wave + i * WAVES, r0 = qi * RPD;                       // first chunk row of the group
+      const uint32_t wrow0 = r0 < 32 ? c * 32u + r0 : H + c * 32u + (r0 - 32u);   // value rows, then gate rows
+      xs_lds_dma16(reinterpret_cast<const char*>(w1p) + (size_t)wrow0 * (K * 2), w1_lane_off, b1 + qi * 1024);
     }
     const char* b2 = w2buf + (c % NB2) * MG::CH2;
 #pragma unroll
     for (uint32_t i = 0; i < kDma2; ++i)
-      xs_lds_dma16(reinterpret_cast<const char*>(w2p) + (size_t)c * MG::CH2, (wave + i * WAVES) * 1024u + lane * 16u,
+      xs_lds_dma16(reinterpret_cast<const char*>(w2p) + (size_t)c * MG::CH2 + (wave + i * WAVES) * 1024u, lane * 16u,
                    b2 + (wave + i * WAVES) * 1024);
-    if (wave == 0)
-      xs_lds_dma16(reinterpret_cast<const char*>(lnx) + (size_t)c * 512, (lane < 32 ? lane : H + lane - 32) * 16u,
-                   s_side + (c % NB1) * 1024);
+    if (wave == 0) xs_lds_dma16(reinterpret_cast<const char*>(lnx) + (size_t)c * 512, tab_lane_off, s_side + (c % NB1) * 1024);
   };
   dma_chunk(0);
   __builtin_amdgcn_s_waitcnt(0x0F70);
