@@ -28,10 +28,12 @@
 //
 // 6 * M * C * H flops (fc1 value + gate, fc2) against HBM traffic of x, residual and y only: the hidden activations
 // (M x H bf16, 1 GB at 482 k rows x 1024) are never allocated.  Measured on MI355X against the LayerNorm+fc1+gate
-// kernel followed by the fc2+residual kernel: 482,304 rows, C = 256, H = 1024: 0.78 ms against 0.94 ms; 250 k rows,
-// C = 128, H = 512: 0.145 ms against 0.224 ms.  (A first form with 64 rows per wave and one wave per SIMD, whose
+// kernel followed by the fc2+residual kernel: 482,304 rows, C = 256, H = 1024: 0.75 ms against 0.94 ms; 250 k rows,
+// C = 128, H = 512: 0.138 ms against 0.224 ms.  (A first form with 64 rows per wave and one wave per SIMD, whose
 // register file the x rows (128) and the fc2 accumulators (256) fill, took 0.87 ms: with a single wave per SIMD
 // nothing overlaps the issue of the roughly 1000 instructions that go with the 100 products of a chunk.)
+#include <algorithm>
+
 #include "xstat_common.h"
 
 namespace f3d {
@@ -302,6 +304,193 @@ __global__ __launch_bounds__(64 * kMlpWaves) __attribute__((amdgpu_waves_per_eu(
 }
 
 
+// Narrow layers (C = 32 / 64): all of w1', its table and w2 fit into LDS at once (7 / 13 KB per 32 hidden features), so
+// a workgroup loads them once and then its waves walk 32-row tiles of x independently, with no barrier and no weight
+// traffic per tile: the kernel moves x, the residual and y and nothing else. Same arithmetic as the streaming kernel
+// above, stage by stage. What bounds it is the gate: per hidden feature and row one exp2 and one reciprocal
+// (transcendental rate) and four ordinary operations, about 350 vector-ALU cycles per 16 hidden features of a tile
+// against 128 / 224 cycles of matrix core. Measured on MI355X against the two-kernel path, launches of the weight
+// preparation included: 1 M rows, C = 32, H = 128: 0.069 ms against 0.200 ms; 500 k rows, C = 64, H = 256: 0.091 ms
+// against 0.198 ms; 3,000 rows: 0.017 ms against 0.024 / 0.026 ms.
+constexpr int kMlpSmallWaves = 8;
+
+template <int K>
+__host__ __device__ constexpr size_t mlp_small_lds_bytes(uint32_t H) {
+  return (size_t)(H / 32) * (64 * K * 2 + K * 64 + 1024) + (size_t)kMlpSmallWaves * 32 * (K + 8) * 2;
+}
+
+template <int K>
+__global__ __launch_bounds__(64 * kMlpSmallWaves) void ln_mlp_swiglu_small_kernel(
+    const uint16_t* __restrict__ x, uint32_t ldx, float eps, const uint16_t* __restrict__ w1p,
+    const uint16_t* __restrict__ lnx, const uint16_t* __restrict__ w2p, const uint16_t* __restrict__ bias2,
+    const uint16_t* __restrict__ residual, uint32_t ldr, uint16_t* __restrict__ y, uint32_t ldy, uint32_t M,
+    uint32_t H) {
+  using G = XsGeom<K>;
+  constexpr int KS = K / 16, ROWB = G::ROWB, WAVES = kMlpSmallWaves, OT = K / 32;
+  constexpr int CH1 = 64 * ROWB, CH2 = K * 64, N2 = CH2 / 1024, PROW = K + 8, PCPR = K / 8;
+  static_assert(K == 32 || K == 64, "narrow layers only");
+  static_assert(32 * kPatchRow <= 32 * PROW, "the output patch fits into the wave's transposition patch");
+  extern __shared__ __attribute__((aligned(1024))) char lds_mlp[];
+  const uint32_t nchunk = H / 32;
+  char* w1buf = lds_mlp;
+  char* w2buf = w1buf + (size_t)nchunk * CH1;
+  char* s_side = w2buf + (size_t)nchunk * CH2;
+  const uint32_t tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid / kWave), lane = tid % kWave;
+  const uint32_t lq = lane & 31u, half = lane >> 5;
+  uint16_t* patch = reinterpret_cast<uint16_t*>(s_side + (size_t)nchunk * 1024) + wave * (32 * PROW);
+
+  // ---- every weight of the layer -> LDS, the direct loads dealt out over the waves ----
+  {
+    constexpr uint32_t per = G::N_DMA + N2 + 1;
+    for (uint32_t pi = wave; pi < nchunk * per; pi += WAVES) {
+      const uint32_t c = pi / per, j = pi % per;
+      if (j < (uint32_t)G::N_DMA) {
+        const uint32_t r = (j * 64u + lane) / G::CPR, pc = lane % G::CPR;      // chunk row, position of the lane's piece
+        const uint32_t wrow = r < 32 ? c * 32u + r : H + c * 32u + (r - 32u);   // value rows, then gate rows
+        xs_lds_dma16(w1p, (wrow * K + (pc ^ G::swz(r)) * 8u) * 2u, w1buf + c * CH1 + j * 1024);
+      } else if (j < (uint32_t)G::N_DMA + N2) {
+        const uint32_t q = j - G::N_DMA;
+        xs_lds_dma16(w2p, c * CH2 + q * 1024u + lane * 16u, w2buf + c * CH2 + q * 1024);
+      } else {
+        xs_lds_dma16(lnx, (lane < 32 ? c * 32u + lane : H + c * 32u + lane - 32u) * 16u, s_side + c * 1024);
+      }
+    }
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+    __syncthreads();
+  }
+
+  const uint32_t trow = lq < 16 ? lq : lq + 16;
+  const uint32_t frag_off = trow * ROWB + (((half ^ G::swz(trow)) & (uint32_t)(G::CPR - 1)) << 4);
+  const uint32_t ntiles = (M + 31) / 32;
+  // the rows of a tile as the lanes load them (row-contiguous 16-byte pieces); the next tile's are requested while the
+  // current one is computed
+  constexpr int XLOADS = (32 * PCPR) / kWave;
+  u32x4_t xv[XLOADS];
+  auto request_x = [&](uint32_t tile) __attribute__((always_inline)) {
+#pragma unroll
+    for (int i = 0; i < XLOADS; ++i) {
+      const uint32_t id = lane + i * kWave;
+      const uint32_t rr = id / PCPR, kc = (id % PCPR) * 8;
+      const uint32_t r = min(tile * 32 + rr, M - 1);
+      xv[i] = *reinterpret_cast<const u32x4_t*>(x + (size_t)r * ldx + kc);
+    }
+  };
+  const uint32_t tile_step = gridDim.x * WAVES;
+  if (blockIdx.x * WAVES + wave < ntiles) request_x(blockIdx.x * WAVES + wave);
+  for (uint32_t tile = blockIdx.x * WAVES + wave; tile < ntiles; tile += tile_step) {
+    const uint32_t row0 = tile * 32;
+    // ---- the tile's rows of x -> registers (B-operand layout) through the wave's patch ----
+    bf16x8_t xf[KS];
+#pragma unroll
+    for (int i = 0; i < XLOADS; ++i) {
+      const uint32_t id = lane + i * kWave;
+      const uint32_t rr = id / PCPR, kc = (id % PCPR) * 8;
+      *reinterpret_cast<u32x4_t*>(patch + rr * PROW + kc) = xv[i];
+    }
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+      xf[ks] = *reinterpret_cast<const bf16x8_t*>(patch + lq * PROW + ks * 16 + half * 8);
+    if (tile + tile_step < ntiles) request_x(tile + tile_step);
+    // the residual rows of the tile, requested now, used at the end
+    u32x4_t rres[OT][2];
+    if (residual) {
+#pragma unroll
+      for (int ot = 0; ot < OT; ++ot)
+#pragma unroll
+        for (int h2 = 0; h2 < 2; ++h2) {
+          const uint32_t rr = (lane >> 2) + h2 * 16, ch = (lane & 3u) * 8;
+          const uint32_t row = min(row0 + rr, M - 1);
+          rres[ot][h2] = *reinterpret_cast<const u32x4_t*>(residual + ((size_t)row * ldr + ot * 32 + ch));
+        }
+    }
+    // LayerNorm in place: x <- bf16((x - mean) * rstd), statistics shifted by the row's first element
+    {
+      const float x0 = __shfl((float)xf[0][0], lq, kWave);
+      float sm = 0.f, sq = 0.f;
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const float d = (float)xf[ks][e] - x0;
+          sm += d;
+          sq = __builtin_fmaf(d, d, sq);
+        }
+      const float mean = pair_sum(sm) * (1.0f / K);
+      const float var = fmaxf(pair_sum(sq) * (1.0f / K) - mean * mean, 0.f);
+      const float rstd = rsqrtf(var + eps), shift = -(x0 + mean) * rstd;
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        const u32x4_t raw = __builtin_bit_cast(u32x4_t, xf[ks]);
+        u32x4_t pk;
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          pk[e] = pack_bf16x2(__builtin_fmaf(bf16_lo(raw[e]), rstd, shift), __builtin_fmaf(bf16_hi(raw[e]), rstd, shift));
+        xf[ks] = __builtin_bit_cast(bf16x8_t, pk);
+      }
+    }
+    // fc2 accumulators start from the bias: acc2[ot][g*4+r] <-> output column ot*32 + g*8 + half*4 + r of row lq
+    f32x16_t acc2[OT];
+#pragma unroll
+    for (int ot = 0; ot < OT; ++ot)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const uint2 bb = *reinterpret_cast<const uint2*>(bias2 + ot * 32 + g * 8 + half * 4);
+        acc2[ot][g * 4 + 0] = bf16_lo(bb.x); acc2[ot][g * 4 + 1] = bf16_hi(bb.x);
+        acc2[ot][g * 4 + 2] = bf16_lo(bb.y); acc2[ot][g * 4 + 3] = bf16_hi(bb.y);
+      }
+    for (uint32_t c = 0; c < nchunk; ++c) {
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        // fc1 of the half: rows 0-15 value, 16-31 gate; the bias k-step first (table row against (0, 0, 0, 1, 0, 1, 0, 0))
+        const char* sw = w1buf + c * CH1 + h * 16 * ROWB;
+        const bf16x8_t tf = *reinterpret_cast<const bf16x8_t*>(s_side + c * 1024 + (trow + h * 16) * 16);
+        u32x4_t d = {0u, half == 0 ? 0x3F800000u : 0u, half == 0 ? 0x3F800000u : 0u, 0u};
+        const f32x16_t zero = {};
+        f32x16_t acc1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tf, __builtin_bit_cast(bf16x8_t, d), zero, 0, 0, 0);
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+          const bf16x8_t wf = *reinterpret_cast<const bf16x8_t*>(sw + (frag_off ^ (uint32_t)(ks * 32)));
+          acc1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf, xf[ks], acc1, 0, 0, 0);
+        }
+        u32x4_t hb;
+#pragma unroll
+        for (int p = 0; p < 4; ++p)
+          hb[p] = pack_bf16x2(fast_silu(acc1[2 * p]) * acc1[2 * p + 8], fast_silu(acc1[2 * p + 1]) * acc1[2 * p + 9]);
+        const char* s2 = w2buf + c * CH2 + lane * 16 + h * 1024;
+#pragma unroll
+        for (int ot = 0; ot < OT; ++ot) {
+          const bf16x8_t f = *reinterpret_cast<const bf16x8_t*>(s2 + ot * 2048);
+          acc2[ot] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f, __builtin_bit_cast(bf16x8_t, hb), acc2[ot], 0, 0, 0);
+        }
+      }
+    }
+    // ---- output: bf16(fc2) (+ residual) through the wave's patch, row-contiguous stores ----
+#pragma unroll
+    for (int ot = 0; ot < OT; ++ot) {
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        uint2 pk;
+        pk.x = pack_bf16x2(acc2[ot][g * 4 + 0], acc2[ot][g * 4 + 1]);
+        pk.y = pack_bf16x2(acc2[ot][g * 4 + 2], acc2[ot][g * 4 + 3]);
+        *reinterpret_cast<uint2*>(patch + lq * kPatchRow + g * 8 + half * 4) = pk;
+      }
+#pragma unroll
+      for (int h2 = 0; h2 < 2; ++h2) {
+        const uint32_t rr = (lane >> 2) + h2 * 16, ch = (lane & 3u) * 8;
+        const uint32_t row = row0 + rr;
+        u32x4_t t = *reinterpret_cast<const u32x4_t*>(patch + rr * kPatchRow + ch);
+        if (residual) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            t[e] = pack_bf16x2(bf16_lo(t[e]) + bf16_lo(rres[ot][h2][e]), bf16_hi(t[e]) + bf16_hi(rres[ot][h2][e]));
+        }
+        if (row < M) *reinterpret_cast<u32x4_t*>(y + ((size_t)row * ldy + ot * 32 + ch)) = t;
+      }
+    }
+  }
+}
+
+
 // w2 [C][H] row-major -> fragment-major per chunk of 32 hidden features:
 //   w2p[(((c * C/32 + ot) * 2 + s) * 64 + half * 32 + lq) * 8 + e] = w2[ot * 32 + lq][c * 32 + (2 s + e / 4) * 8 + half * 4 + e % 4]
 // One thread per 16-byte piece.
@@ -337,6 +526,31 @@ static int launch_mlp(const uint16_t* x, uint32_t ldx, float eps, const uint16_t
 }
 
 
+template <int K>
+static int launch_mlp_small(const uint16_t* x, uint32_t ldx, float eps, const uint16_t* w1p, const uint16_t* lnx,
+                            const uint16_t* w2p, const uint16_t* bias2, const uint16_t* residual, uint32_t ldr,
+                            uint16_t* y, uint32_t ldy, uint32_t M, uint32_t H, int device, hipStream_t s) {
+  const size_t lds = mlp_small_lds_bytes<K>(H);
+  static int cus[64] = {};
+  static size_t attr_lds[64] = {};
+  int n_cu = 256;
+  if (device >= 0 && device < 64) {
+    if (!cus[device]) F3D_CHECK_HIP(hipDeviceGetAttribute(&cus[device], hipDeviceAttributeMultiprocessorCount, device));
+    n_cu = cus[device];
+  }
+  auto kern = ln_mlp_swiglu_small_kernel<K>;
+  if (device < 0 || device >= 64 || attr_lds[device] < lds) {
+    F3D_CHECK_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    if (device >= 0 && device < 64) attr_lds[device] = lds;
+  }
+  // as many resident workgroups as the LDS allows; each wave then walks its share of the 32-row tiles
+  const uint32_t per_cu = (uint32_t)std::max<size_t>(1, std::min<size_t>(4, (160 * 1024) / lds));
+  const uint32_t wgs = std::min<uint32_t>(cdiv_u32(cdiv_u32(M, 32), kMlpSmallWaves), (uint32_t)n_cu * per_cu);
+  hipLaunchKernelGGL(kern, dim3(wgs), dim3(64 * kMlpSmallWaves), lds, s, x, ldx, eps, w1p, lnx, w2p, bias2, residual, ldr,
+                     y, ldy, M, H);
+  return F3D_OK;
+}
+
 }  // namespace f3d
 
 extern "C" {
@@ -347,9 +561,11 @@ int f3d_ln_mlp_swiglu_bf16(const f3d_bf16_t* x, uint32_t ldx, const f3d_bf16_t* 
                            uint32_t c, uint32_t hidden, int device, void* stream) {
   using namespace f3d;
   F3D_CHECK_ARG(x && gamma && w1 && w2 && y, "null tensor pointer");
-  if (!(c == 128 || c == 256) || hidden == 0 || hidden % 32 != 0 || (uint64_t)hidden * c * 4 >= (1ull << 32)) {
-    set_error("No fused MLP kernel for width %u with hidden width %u (widths 128 and 256, hidden a multiple of 32)", c,
-              hidden);
+  const bool narrow = c == 32 || c == 64;
+  if (!(narrow || c == 128 || c == 256) || hidden == 0 || hidden % 32 != 0 || (uint64_t)hidden * c * 4 >= (1ull << 32) ||
+      (c == 32 && mlp_small_lds_bytes<32>(hidden) > 160 * 1024) || (c == 64 && mlp_small_lds_bytes<64>(hidden) > 160 * 1024)) {
+    set_error("No fused MLP kernel for width %u with hidden width %u (widths 128 and 256 with hidden a multiple of 32; "
+              "widths 32 and 64 while all weights fit into LDS: hidden <= 640 / 288)", c, hidden);
     return F3D_ERR_UNSUPPORTED;
   }
   F3D_CHECK_ARG(ldx >= c && ldx % 8 == 0 && ldy >= c && ldy % 8 == 0 && (!residual || (ldr >= c && ldr % 8 == 0)),
@@ -376,6 +592,8 @@ int f3d_ln_mlp_swiglu_bf16(const f3d_bf16_t* x, uint32_t ldx, const f3d_bf16_t* 
   hipLaunchKernelGGL(mlp_w2_prep_kernel, dim3(cdiv_u32(c * hidden / 8, 256)), dim3(256), 0, s, w2, w2p, zero_bias, c, hidden);
   int rc;
   if (c == 256) rc = launch_mlp<256>(x, ldx, eps, w1p, table, w2p, b2, residual, ldr, y, ldy, m, hidden, device, s);
+  else if (c == 32) rc = launch_mlp_small<32>(x, ldx, eps, w1p, table, w2p, b2, residual, ldr, y, ldy, m, hidden, device, s);
+  else if (c == 64) rc = launch_mlp_small<64>(x, ldx, eps, w1p, table, w2p, b2, residual, ldr, y, ldy, m, hidden, device, s);
   else rc = launch_mlp<128>(x, ldx, eps, w1p, table, w2p, b2, residual, ldr, y, ldy, m, hidden, device, s);
   if (rc != F3D_OK) return rc;
   F3D_CHECK_HIP(hipGetLastError());

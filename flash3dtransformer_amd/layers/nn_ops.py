@@ -215,7 +215,7 @@ class LayerNorm(_CachedParamModule):
 
 
 FUSABLE_LN_WIDTHS = (32, 64, 128, 256, 512)
-FUSED_MLP_WIDTHS = (128, 256)      # widths the one-kernel gated MLP covers
+FUSED_MLP_WIDTHS = (32, 64, 128, 256)      # widths the one-kernel gated MLP covers (32 / 64: while the weights fit into LDS)
 
 
 def is_fusable_layernorm(norm, width: int) -> bool:
@@ -298,9 +298,10 @@ class LayerNormMLP(_CachedParamModule):
     def __init__(self, hidden_size: int, ffn_hidden_size: int, activation: str = "swiglu", eps: float = 1e-5,
                  fused: bool = None):
         super().__init__()
-        # fused: run the whole gated MLP as one kernel where one exists (widths 128 / 256): the hidden activations
-        # [rows, ffn_hidden_size] are then never allocated.  None (default): where it is the faster path on MI355X
-        # (measured against LayerNorm+fc1+gate followed by fc2+residual, hidden = 4 x width: width 128 at every row
+        # fused: run the whole gated MLP as one kernel where one exists (widths 32 / 64 / 128 / 256): the hidden
+        # activations [rows, ffn_hidden_size] are then never allocated.  None (default): where it is the faster path on
+        # MI355X (measured against LayerNorm+fc1+gate followed by fc2+residual, hidden = 4 x width: widths 32 and 64
+        # at every row count, 27 % faster at 3 k rows and 2.2 to 2.9 x at 0.5 to 1 M rows; width 128 at every row
         # count, 19 to 41 % faster; width 256 from 32 k rows up, 6 to 23 % faster, and 11 % slower at 16 k rows)
         self.fused = fused
         assert activation in ("swiglu", "gelu")
@@ -322,7 +323,7 @@ class LayerNormMLP(_CachedParamModule):
         r2 = None if residual is None else as_bf16_2d(residual.reshape(-1, self.hidden_size))
         y = torch.empty_like(x2)
         # on request, the whole gated MLP in one kernel where one exists (hidden activations stay in registers) ...
-        want_fused = self.fused if self.fused is not None else (self.hidden_size == 128 or x2.shape[0] >= 30000)
+        want_fused = self.fused if self.fused is not None else (self.hidden_size <= 128 or x2.shape[0] >= 30000)
         fused = (want_fused and self.activation == "swiglu" and self.hidden_size in FUSED_MLP_WIDTHS
                  and self.ffn_hidden_size % 32 == 0
                  and pshattn.ln_mlp_swiglu_bf16(x2, c[0].get(self.layer_norm_weight, self.training), c[1].get(self.layer_norm_bias, self.training),

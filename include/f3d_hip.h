@@ -258,8 +258,9 @@ int f3d_ln_linear_bf16(const f3d_bf16_t* x, uint32_t ldx, const f3d_bf16_t* gamm
  * stage.py:94-97).  x [m,c] (row stride ldx), gamma [c], beta [c] or NULL, w1 [2 hidden, c] (value rows, then gate
  * rows), b1 [2 hidden] or NULL, w2 [c, hidden], b2 [c] or NULL, residual [m,c] or NULL (row stride ldr), y [m,c] (row
  * stride ldy), all bf16.  The hidden activations are rounded to bf16 as a separate fc1 kernel would store them and
- * never leave the registers.  c in {128, 256}, hidden a multiple of 32; anything else returns F3D_ERR_UNSUPPORTED
- * without touching y (use f3d_ln_linear_bf16 with F3D_ACT_SWIGLU followed by f3d_linear_bf16).  Uses the per-device
+ * never leave the registers.  c in {128, 256} with hidden a multiple of 32 (weights stream through LDS), or c in
+ * {32, 64} with hidden a multiple of 32 up to 640 / 288 (all weights resident in LDS, each wave walks row tiles on its
+ * own); anything else returns F3D_ERR_UNSUPPORTED without touching y (use f3d_ln_linear_bf16 with F3D_ACT_SWIGLU followed by f3d_linear_bf16).  Uses the per-device
  * workspace like f3d_ln_linear_bf16. */
 int f3d_ln_mlp_swiglu_bf16(const f3d_bf16_t* x, uint32_t ldx, const f3d_bf16_t* gamma, const f3d_bf16_t* beta, float eps,
                            const f3d_bf16_t* w1, const f3d_bf16_t* b1, const f3d_bf16_t* w2, const f3d_bf16_t* b2,

@@ -185,6 +185,11 @@ def test_dense_argument_errors():
     (777, 128, 512, True, False),       # C = 128, no biases
     (300, 256, 32, True, True),         # a single hidden chunk
     (70000, 128, 256, True, True),      # many workgroups
+    (5000, 32, 128, True, True),        # narrow layers: all weights resident in LDS, waves walk the row tiles
+    (100000, 64, 256, True, True),      # ... more tiles than resident waves
+    (333, 64, 64, False, False),        # ... ragged M, no residual, no biases
+    (1000, 32, 640, True, True),        # ... the largest hidden width that fits at C = 32
+    (40, 64, 288, True, False),         # ... and at C = 64; fewer rows than one workgroup's waves
 ])
 def test_fused_mlp_matches_two_kernel_path(oracle, M, C, H, use_res, use_bias):
     """The one-kernel gated MLP against (a) the LayerNorm+fc1+swiglu kernel followed by the fc2+residual kernel, whose
@@ -230,8 +235,12 @@ def test_fused_mlp_unsupported_width_is_reported():
     from flash3dtransformer_amd.lib import pshattn
     mk = lambda *s: torch.zeros(*s, dtype=torch.bfloat16, device=DEV)
     y = torch.full((64, 64), 3.0, dtype=torch.bfloat16, device=DEV)
-    assert not pshattn.ln_mlp_swiglu_bf16(mk(64, 64), mk(64), mk(64), 1e-5, mk(256, 64), None, mk(64, 128), None, None, y)
+    # C = 64 with a hidden width whose weights do not fit into LDS; C = 512
+    assert not pshattn.ln_mlp_swiglu_bf16(mk(64, 64), mk(64), mk(64), 1e-5, mk(640, 64), None, mk(64, 320), None, None, y)
     assert (y == 3.0).all()
+    y5 = torch.full((64, 512), 3.0, dtype=torch.bfloat16, device=DEV)
+    assert not pshattn.ln_mlp_swiglu_bf16(mk(64, 512), mk(512), mk(512), 1e-5, mk(128, 512), None, mk(512, 64), None, None, y5)
+    assert (y5 == 3.0).all()
 
 
 def test_layernorm_mlp_layer_one_kernel_and_two_kernel_paths():
