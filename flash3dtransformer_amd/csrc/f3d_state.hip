@@ -35,7 +35,13 @@ void* workspace(int device, size_t bytes) {
   DeviceGuard guard(device);
   // Work queued on the old buffer must finish before it is released.
   if (w.ptr) {
-    (void)hipDeviceSynchronize();
+    // (refused while a stream of this thread is being captured: the caller gets an error instead of a broken graph)
+    const hipError_t es = hipDeviceSynchronize();
+    if (es != hipSuccess) {
+      set_error("the workspace of device %d must grow from %zu to %zu bytes, but the device cannot be synchronised (%s): "
+                "warm the shapes up outside stream capture", device, w.bytes, bytes, hipGetErrorString(es));
+      return nullptr;
+    }
     (void)hipFree(w.ptr);
     w.ptr = nullptr;
     w.bytes = 0;

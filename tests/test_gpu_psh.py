@@ -79,6 +79,31 @@ def test_ragged_batches_bit_exact(oracle, sizes, bucket_size):
         assert (out["scat"][n:] == 0).all() and not np.isnan(out["scat"]).any()
 
 
+@pytest.mark.parametrize("sizes,bucket_size", [
+    ([5000, 8192, 1, 0, 777], 64),         # clouds of at most 8192 points, an empty and a one-point cloud
+    ([16384, 12000, 3], 512),              # exactly 16,384
+    ([32768, 16385, 20000, 0], 512),       # exactly 32,768, one point more than 16,384, an empty last cloud
+])
+@pytest.mark.parametrize("rebalance", [0, 1])
+def test_small_clouds_bit_exact(oracle, sizes, bucket_size, rebalance):
+    """Small clouds at the tile-size boundaries, half of each cloud clustered so that buckets overflow and the
+    rebalance plan is in use, empty and one-point clouds, pad rows, all four hash types; ids, counts, slots and
+    scattered rows bit-exact vs the oracle."""
+    from flash3dtransformer_amd.lib import pshattn
+    rng = np.random.default_rng(sum(sizes) + rebalance)
+    pts = np.concatenate([np.concatenate([rng.normal(0, 2.0, (n // 2, 3)), rng.uniform(-30, 30, (n - n // 2, 3))])
+                          for n in sizes]).astype(np.float16)
+    seps = np.cumsum(sizes).astype(np.uint32)
+    for hash_op in (1, 2, 3, 4):
+        out = _run_psh(pts, seps, bucket_size, hash_op, bucket_size * 6, oracle, rebalance=rebalance)
+        _check_against_oracle(pts, seps, out, hash_op, oracle, rebalance=rebalance, bucket_size=bucket_size)
+        n = pts.shape[0]
+        assert (out["scat"][n:] == 0).all() and not np.isnan(out["scat"]).any()
+        if rebalance:
+            assert (out["cnt"][:, 1:] <= bucket_size).all()
+    pshattn.DeviceManagerSingleton.instance().set_psh_rebalance(1)
+
+
 def test_lidar_batch_reference_invariants(oracle):
     """4 synthetic sweeps (heavily clustered): the reference's three checks, through its own
     sanitizer entry point"""
