@@ -64,7 +64,7 @@ __global__ __launch_bounds__(64 * kMlpWaves) __attribute__((amdgpu_waves_per_eu(
     const uint16_t* __restrict__ x, uint32_t ldx, float eps, const uint16_t* __restrict__ w1p,
     const uint16_t* __restrict__ lnx, const uint16_t* __restrict__ w2p, const uint16_t* __restrict__ bias2,
     const uint16_t* __restrict__ residual, uint32_t ldr, uint16_t* __restrict__ y, uint32_t ldy, uint32_t M,
-    uint32_t H) {
+    uint32_t H, uint32_t main_wgs, uint32_t tail_rows) {
   using G = XsGeom<K>;
   using MG = MlpGeom<K>;
   constexpr int KS = K / 16, ROWB = G::ROWB, WAVES = kMlpWaves, NB1 = kMlpBufs, NB2 = kMlpBufs, OT = MG::OT;
@@ -77,7 +77,13 @@ __global__ __launch_bounds__(64 * kMlpWaves) __attribute__((amdgpu_waves_per_eu(
 
   const uint32_t tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid / kWave), lane = tid % kWave;
   const uint32_t lq = lane & 31u, half = lane >> 5;
-  const uint32_t row0 = blockIdx.x * ROWS_WG + wave * 32;
+  // Workgroups [0, main_wgs) own 256 rows each; the workgroups after them share what is left in panels of tail_rows
+  // rows (a multiple of 32, at most 256), of which only the first tail_rows / 32 waves have rows: the last, partly
+  // filled turn of the chip then runs with fewer waves per SIMD and ends sooner.
+  const bool in_tail = blockIdx.x >= main_wgs;
+  const uint32_t wg_row0 = in_tail ? main_wgs * ROWS_WG + (blockIdx.x - main_wgs) * tail_rows : blockIdx.x * ROWS_WG;
+  const uint32_t row0 = wg_row0 + wave * 32;
+  const bool has_rows = (wave * 32 < (in_tail ? tail_rows : (uint32_t)ROWS_WG)) && row0 < M;
 
   // ---- this wave's 32 rows of x -> registers (B-operand layout), through a wave-private transposition patch ----
   bf16x8_t xf[KS];
@@ -250,6 +256,16 @@ __global__ __launch_bounds__(64 * kMlpWaves) __attribute__((amdgpu_waves_per_eu(
     __builtin_amdgcn_sched_barrier(0);
   };
 
+  if (!has_rows) {
+    // a wave without rows only carries its share of the weight requests and keeps the barriers in step
+    for (uint32_t ci = 0; ci < nchunk; ++ci) {
+      if (ci + 1 < nchunk) dma_chunk(ci + 1);
+      __builtin_amdgcn_s_waitcnt(0x0F70);
+      wg_barrier_lds();
+    }
+    __syncthreads();
+    return;
+  }
   for (uint32_t ci = 0; ci < nchunk; ++ci) {
     // chunk ci + 1 goes into the buffers of chunk ci - 1, which every wave has left
     if (ci + 1 < nchunk) dma_chunk(ci + 1);
@@ -260,8 +276,8 @@ __global__ __launch_bounds__(64 * kMlpWaves) __attribute__((amdgpu_waves_per_eu(
   }
 
   // ---- output: bf16(fc2) (+ residual), through a wave-private LDS patch so that the stores are row-contiguous ----
-  uint16_t* y_wg = y + (size_t)(blockIdx.x * ROWS_WG) * ldy;
-  const uint16_t* res_wg = residual ? residual + (size_t)(blockIdx.x * ROWS_WG) * ldr : nullptr;
+  uint16_t* y_wg = y + (size_t)wg_row0 * ldy;
+  const uint16_t* res_wg = residual ? residual + (size_t)wg_row0 * ldr : nullptr;
   // the residual pieces of the wave's whole panel are requested at once (x is dead: its registers take them): one
   // memory latency for all of them instead of one per column tile
   u32x4_t rres[OT][2];
@@ -272,7 +288,7 @@ __global__ __launch_bounds__(64 * kMlpWaves) __attribute__((amdgpu_waves_per_eu(
       for (int h2 = 0; h2 < 2; ++h2) {
         const uint32_t rr = (lane >> 2) + h2 * 16, ch = (lane & 3u) * 8;
         const uint32_t row = min(row0 + rr, M - 1);            // rows past M read row M - 1
-        rres[ot][h2] = *reinterpret_cast<const u32x4_t*>(res_wg + ((row - blockIdx.x * ROWS_WG) * ldr + ot * 32 + ch));
+        rres[ot][h2] = *reinterpret_cast<const u32x4_t*>(res_wg + ((row - wg_row0) * ldr + ot * 32 + ch));
       }
   }
   __syncthreads();   // every wave is done with the weight buffers: their space takes the output patches
@@ -520,8 +536,25 @@ static int launch_mlp(const uint16_t* x, uint32_t ldx, float eps, const uint16_t
     F3D_CHECK_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     if (device >= 0 && device < 64) attr_set[device] = true;
   }
-  hipLaunchKernelGGL(kern, dim3(cdiv_u32(M, 32 * kMlpWaves)), dim3(64 * kMlpWaves), lds, s, x, ldx, eps, w1p, lnx, w2p,
-                     bias2, residual, ldr, y, ldy, M, H);
+  // Whole turns of the chip run 256-row workgroups; what is left over is spread over all CUs in panels of fewer rows
+  // (fewer waves with work per workgroup), so that the last turn is shorter than a full one.
+  static int cus[64] = {};
+  int n_cu = 256;
+  if (device >= 0 && device < 64) {
+    if (!cus[device]) F3D_CHECK_HIP(hipDeviceGetAttribute(&cus[device], hipDeviceAttributeMultiprocessorCount, device));
+    n_cu = cus[device];
+  }
+  constexpr uint32_t kRows = 32 * kMlpWaves;
+  const uint32_t panels = cdiv_u32(M, kRows);
+  uint32_t main_wgs = panels, tail_rows = kRows, tail_wgs = 0;
+  if (panels > (uint32_t)n_cu && panels % (uint32_t)n_cu != 0) {
+    main_wgs = panels / (uint32_t)n_cu * (uint32_t)n_cu;
+    const uint32_t left = M - main_wgs * kRows;
+    tail_rows = cdiv_u32(cdiv_u32(left, (uint32_t)n_cu), 32u) * 32u;
+    tail_wgs = cdiv_u32(left, tail_rows);
+  }
+  hipLaunchKernelGGL(kern, dim3(main_wgs + tail_wgs), dim3(64 * kMlpWaves), lds, s, x, ldx, eps, w1p, lnx, w2p, bias2, residual,
+                     ldr, y, ldy, M, H, main_wgs, tail_rows);
   return F3D_OK;
 }
 
