@@ -24,7 +24,7 @@
 // LayerNorm-folded w1 (row-major, 16-byte pieces XOR-swizzled) and the chunk's slice of w2, which the preparation
 // kernel stores fragment-major (the 64 lanes' 16-byte pieces of one fragment are consecutive), so its LDS reads are
 // linear.  LayerNorm as in the row-panel linear kernel: the rows are normalised in registers (bf16((x - mean) * rstd)),
-// w' = w * gamma, and one extra k-step starts the fc1 accumulators from b' = b1 + w1 beta.
+// w' = w * gamma, and the fc1 accumulators start from b' = b1 + w1 beta (fp32, fetched per chunk next to the weights).
 //
 // 6 * M * C * H flops (fc1 value + gate, fc2) against HBM traffic of x, residual and y only: the hidden activations
 // (M x H bf16, 1 GB at 482 k rows x 1024) are never allocated.  Measured on MI355X against the LayerNorm+fc1+gate
@@ -48,7 +48,7 @@ struct MlpGeom {
   static constexpr int CH1 = G::CHUNK_BYTES;                // w1 chunk: 64 rows
   static constexpr int CH2 = K * 32 * 2;                    // w2 chunk: K outputs x 32 hidden
   static constexpr int N_DMA2 = CH2 / 1024;
-  // weight buffers and the table rows of the w1 slots; at least the prologue's transposition patches
+  // weight buffers and the b' slots of the w1 buffers; at least the prologue's transposition patches
   static constexpr size_t lds_bytes() {
     const size_t loop = (size_t)kMlpBufs * (CH1 + 1024 + CH2);
     const size_t patches = (size_t)kMlpWaves * 32 * (G::KP + 8) * 2;
@@ -56,13 +56,13 @@ struct MlpGeom {
   }
 };
 
-// w1p: LayerNorm-folded fc1 weight [2 H][K] (value rows then gate rows), lnx: its table [2 H][8] (ln_fold_kernel);
+// w1p: LayerNorm-folded fc1 weight [2 H][K] (value rows then gate rows), b32: b' = b1 + w1 beta as fp32 [2 H] (ln_fold_kernel);
 // w2p: fc2 weight, fragment-major per chunk (mlp_w2_prep_kernel); bias2 [K] (zeros when the layer has none);
 // H: hidden width, multiple of 32.
 template <int K>
 __global__ __launch_bounds__(64 * kMlpWaves) __attribute__((amdgpu_waves_per_eu(2, 2))) void ln_mlp_swiglu_kernel(
     const uint16_t* __restrict__ x, uint32_t ldx, float eps, const uint16_t* __restrict__ w1p,
-    const uint16_t* __restrict__ lnx, const uint16_t* __restrict__ w2p, const uint16_t* __restrict__ bias2,
+    const float* __restrict__ b32, const uint16_t* __restrict__ w2p, const uint16_t* __restrict__ bias2,
     const uint16_t* __restrict__ residual, uint32_t ldr, uint16_t* __restrict__ y, uint32_t ldy, uint32_t M,
     uint32_t H, uint32_t main_wgs, uint32_t tail_rows) {
   using G = XsGeom<K>;
@@ -73,7 +73,7 @@ __global__ __launch_bounds__(64 * kMlpWaves) __attribute__((amdgpu_waves_per_eu(
   extern __shared__ __attribute__((aligned(1024))) char lds_mlp[];
   char* w1buf = lds_mlp;
   char* w2buf = lds_mlp + (size_t)NB1 * MG::CH1;
-  char* s_side = w2buf + (size_t)NB2 * MG::CH2;   // per w1 slot: 64 rows of the bias table
+  char* s_side = w2buf + (size_t)NB2 * MG::CH2;   // per w1 slot: b' of the chunk's 64 fc1 features (fp32; 1 KB apart)
 
   const uint32_t tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid / kWave), lane = tid % kWave;
   const uint32_t lq = lane & 31u, half = lane >> 5;
@@ -156,7 +156,7 @@ __global__ __launch_bounds__(64 * kMlpWaves) __attribute__((amdgpu_waves_per_eu(
   __builtin_amdgcn_s_waitcnt(0x0F70);
   __syncthreads();   // the transposition patches are dead; the space now holds weight chunks
 
-  // ---- weight streaming: per chunk 64 rows of w1 (N_DMA kilobytes), K x 32 of w2 (N_DMA2), 64 table rows (wave 0) ----
+  // ---- weight streaming: per chunk 64 rows of w1 (N_DMA kilobytes), K x 32 of w2 (N_DMA2), the 64 values of b' (wave 0) ----
   const uint32_t nchunk = H / 32;
   static_assert(G::N_DMA % WAVES == 0 && MG::N_DMA2 % WAVES == 0, "direct loads split evenly over the waves");
   constexpr uint32_t kDma1 = G::N_DMA / WAVES, kDma2 = MG::N_DMA2 / WAVES;
@@ -168,7 +168,7 @@ __global__ __launch_bounds__(64 * kMlpWaves) __attribute__((amdgpu_waves_per_eu(
   constexpr uint32_t RPD = 64 / G::CPR;
   static_assert((WAVES * RPD) % 16 == 0 && G::RP == 1 && 32 % RPD == 0, "one lane offset serves all groups of a wave");
   const uint32_t w1_lane_off = ((lane / G::CPR) * K + (((lane % G::CPR) ^ G::swz(wave * RPD + lane / G::CPR)) * 8u)) * 2u;
-  const uint32_t tab_lane_off = (lane < 32 ? lane : H + lane - 32) * 16u;
+  const uint32_t tab_lane_off = (lane < 32 ? lane : H + lane - 32) * 4u;
   auto dma_chunk = [&](uint32_t c) __attribute__((always_inline)) {
     const char* b1 = w1buf + (c % NB1) * MG::CH1;
 #pragma unroll
@@ -182,7 +182,7 @@ __global__ __launch_bounds__(64 * kMlpWaves) __attribute__((amdgpu_waves_per_eu(
     for (uint32_t i = 0; i < kDma2; ++i)
       xs_lds_dma16(reinterpret_cast<const char*>(w2p) + (size_t)c * MG::CH2 + (wave + i * WAVES) * 1024u, lane * 16u,
                    b2 + (wave + i * WAVES) * 1024);
-    if (wave == 0) xs_lds_dma16(reinterpret_cast<const char*>(lnx) + (size_t)c * 512, tab_lane_off, s_side + (c % NB1) * 1024);
+    if (wave == 0) xs_lds_dma4(reinterpret_cast<const char*>(b32) + (size_t)c * 128, tab_lane_off, s_side + (c % NB1) * 1024);
   };
   dma_chunk(0);
   __builtin_amdgcn_s_waitcnt(0x0F70);
@@ -205,22 +205,19 @@ __global__ __launch_bounds__(64 * kMlpWaves) __attribute__((amdgpu_waves_per_eu(
 #pragma unroll
     for (int ks = 0; ks < kAhead; ++ks) read_frag(ks);
     {
-      // bias k-step: the table rows (wsum_hi, wsum_hi, wsum_lo, b'_hi, b'_hi, b'_lo, 0, 0) against (0, 0, 0, 1, 0, 1, 0, 0)
-      const bf16x8_t tf = *reinterpret_cast<const bf16x8_t*>(s_side + slot * 1024 + (trow + h * 16) * 16);
-      u32x4_t d = {0u, half == 0 ? 0x3F800000u : 0u, half == 0 ? 0x3F800000u : 0u, 0u};
-      asm volatile("" : "+v"(d));
-      const f32x16_t zero = {};
-      acc1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tf, __builtin_bit_cast(bf16x8_t, d), zero, 0, 0, 0);
+      // the accumulators start from b' (fp32, 64 per chunk: the 32 value features, then the 32 gate features)
+      const float* sb = reinterpret_cast<const float*>(s_side + slot * 1024) + h * 16 + half * 4;
+      const float4 v0 = *reinterpret_cast<const float4*>(sb), v1 = *reinterpret_cast<const float4*>(sb + 8);
+      const float4 g0 = *reinterpret_cast<const float4*>(sb + 32), g1 = *reinterpret_cast<const float4*>(sb + 40);
+      acc1[0] = v0.x; acc1[1] = v0.y; acc1[2] = v0.z; acc1[3] = v0.w; acc1[4] = v1.x; acc1[5] = v1.y; acc1[6] = v1.z; acc1[7] = v1.w;
+      acc1[8] = g0.x; acc1[9] = g0.y; acc1[10] = g0.z; acc1[11] = g0.w; acc1[12] = g1.x; acc1[13] = g1.y; acc1[14] = g1.z; acc1[15] = g1.w;
     }
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       if (ks + kAhead < KS) read_frag(ks + kAhead);
       acc1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[ks], xf[ks], acc1, 0, 0, 0);
     }
-    // issue order: the table row and kAhead k-steps of fragments, the bias product, then per k-step its product
-    // followed by the reads of the k-step kAhead later
-    __builtin_amdgcn_sched_group_barrier(0x100, 1 + kAhead, 0);
-    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+    __builtin_amdgcn_sched_group_barrier(0x100, 4 + kAhead, 0);
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
@@ -320,7 +317,7 @@ __global__ __launch_bounds__(64 * kMlpWaves) __attribute__((amdgpu_waves_per_eu(
 }
 
 
-// Narrow layers (C = 32 / 64): all of w1', its table and w2 fit into LDS at once (7 / 13 KB per 32 hidden features), so
+// Narrow layers (C = 32 / 64): all of w1', b' and w2 fit into LDS at once (7 / 13 KB per 32 hidden features), so
 // a workgroup loads them once and then its waves walk 32-row tiles of x independently, with no barrier and no weight
 // traffic per tile: the kernel moves x, the residual and y and nothing else. Same arithmetic as the streaming kernel
 // above, stage by stage. What bounds it is the gate: per hidden feature and row one exp2 and one reciprocal
@@ -338,7 +335,7 @@ __host__ __device__ constexpr size_t mlp_small_lds_bytes(uint32_t H) {
 template <int K>
 __global__ __launch_bounds__(64 * kMlpSmallWaves) void ln_mlp_swiglu_small_kernel(
     const uint16_t* __restrict__ x, uint32_t ldx, float eps, const uint16_t* __restrict__ w1p,
-    const uint16_t* __restrict__ lnx, const uint16_t* __restrict__ w2p, const uint16_t* __restrict__ bias2,
+    const float* __restrict__ b32, const uint16_t* __restrict__ w2p, const uint16_t* __restrict__ bias2,
     const uint16_t* __restrict__ residual, uint32_t ldr, uint16_t* __restrict__ y, uint32_t ldy, uint32_t M,
     uint32_t H) {
   using G = XsGeom<K>;
@@ -368,7 +365,7 @@ __global__ __launch_bounds__(64 * kMlpSmallWaves) void ln_mlp_swiglu_small_kerne
         const uint32_t q = j - G::N_DMA;
         xs_lds_dma16(w2p, c * CH2 + q * 1024u + lane * 16u, w2buf + c * CH2 + q * 1024);
       } else {
-        xs_lds_dma16(lnx, (lane < 32 ? c * 32u + lane : H + c * 32u + lane - 32u) * 16u, s_side + c * 1024);
+        xs_lds_dma4(b32, (lane < 32 ? c * 32u + lane : H + c * 32u + lane - 32u) * 4u, s_side + c * 1024);
       }
     }
     __builtin_amdgcn_s_waitcnt(0x0F70);
@@ -457,12 +454,13 @@ __global__ __launch_bounds__(64 * kMlpSmallWaves) void ln_mlp_swiglu_small_kerne
     for (uint32_t c = 0; c < nchunk; ++c) {
 #pragma unroll
       for (int h = 0; h < 2; ++h) {
-        // fc1 of the half: rows 0-15 value, 16-31 gate; the bias k-step first (table row against (0, 0, 0, 1, 0, 1, 0, 0))
+        // fc1 of the half: rows 0-15 value, 16-31 gate; the accumulators start from b' (fp32: the chunk's 32 value
+        // features, then its 32 gate features)
         const char* sw = w1buf + c * CH1 + h * 16 * ROWB;
-        const bf16x8_t tf = *reinterpret_cast<const bf16x8_t*>(s_side + c * 1024 + (trow + h * 16) * 16);
-        u32x4_t d = {0u, half == 0 ? 0x3F800000u : 0u, half == 0 ? 0x3F800000u : 0u, 0u};
-        const f32x16_t zero = {};
-        f32x16_t acc1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tf, __builtin_bit_cast(bf16x8_t, d), zero, 0, 0, 0);
+        const float* sb = reinterpret_cast<const float*>(s_side + c * 1024) + h * 16 + half * 4;
+        const float4 v0 = *reinterpret_cast<const float4*>(sb), v1 = *reinterpret_cast<const float4*>(sb + 8);
+        const float4 g0 = *reinterpret_cast<const float4*>(sb + 32), g1 = *reinterpret_cast<const float4*>(sb + 40);
+        f32x16_t acc1 = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w, g0.x, g0.y, g0.z, g0.w, g1.x, g1.y, g1.z, g1.w};
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
           const bf16x8_t wf = *reinterpret_cast<const bf16x8_t*>(sw + (frag_off ^ (uint32_t)(ks * 32)));
@@ -525,7 +523,7 @@ __global__ __launch_bounds__(256) void mlp_w2_prep_kernel(const uint16_t* __rest
 
 
 template <int K>
-static int launch_mlp(const uint16_t* x, uint32_t ldx, float eps, const uint16_t* w1p, const uint16_t* lnx,
+static int launch_mlp(const uint16_t* x, uint32_t ldx, float eps, const uint16_t* w1p, const float* b32,
                            const uint16_t* w2p, const uint16_t* bias2, const uint16_t* residual, uint32_t ldr, uint16_t* y,
                            uint32_t ldy, uint32_t M, uint32_t H, int device, hipStream_t s) {
   constexpr size_t lds = MlpGeom<K>::lds_bytes();
@@ -553,14 +551,14 @@ static int launch_mlp(const uint16_t* x, uint32_t ldx, float eps, const uint16_t
     tail_rows = cdiv_u32(cdiv_u32(left, (uint32_t)n_cu), 32u) * 32u;
     tail_wgs = cdiv_u32(left, tail_rows);
   }
-  hipLaunchKernelGGL(kern, dim3(main_wgs + tail_wgs), dim3(64 * kMlpWaves), lds, s, x, ldx, eps, w1p, lnx, w2p, bias2, residual,
+  hipLaunchKernelGGL(kern, dim3(main_wgs + tail_wgs), dim3(64 * kMlpWaves), lds, s, x, ldx, eps, w1p, b32, w2p, bias2, residual,
                      ldr, y, ldy, M, H, main_wgs, tail_rows);
   return F3D_OK;
 }
 
 
 template <int K>
-static int launch_mlp_small(const uint16_t* x, uint32_t ldx, float eps, const uint16_t* w1p, const uint16_t* lnx,
+static int launch_mlp_small(const uint16_t* x, uint32_t ldx, float eps, const uint16_t* w1p, const float* b32,
                             const uint16_t* w2p, const uint16_t* bias2, const uint16_t* residual, uint32_t ldr,
                             uint16_t* y, uint32_t ldy, uint32_t M, uint32_t H, int device, hipStream_t s) {
   const size_t lds = mlp_small_lds_bytes<K>(H);
@@ -579,7 +577,7 @@ static int launch_mlp_small(const uint16_t* x, uint32_t ldx, float eps, const ui
   // as many resident workgroups as the LDS allows; each wave then walks its share of the 32-row tiles
   const uint32_t per_cu = (uint32_t)std::max<size_t>(1, std::min<size_t>(4, (160 * 1024) / lds));
   const uint32_t wgs = std::min<uint32_t>(cdiv_u32(cdiv_u32(M, 32), kMlpSmallWaves), (uint32_t)n_cu * per_cu);
-  hipLaunchKernelGGL(kern, dim3(wgs), dim3(64 * kMlpSmallWaves), lds, s, x, ldx, eps, w1p, lnx, w2p, bias2, residual, ldr,
+  hipLaunchKernelGGL(kern, dim3(wgs), dim3(64 * kMlpSmallWaves), lds, s, x, ldx, eps, w1p, b32, w2p, bias2, residual, ldr,
                      y, ldy, M, H);
   return F3D_OK;
 }
@@ -611,23 +609,24 @@ int f3d_ln_mlp_swiglu_bf16(const f3d_bf16_t* x, uint32_t ldx, const f3d_bf16_t* 
   F3D_CHECK_ARG(guard.ok, "cannot select device %d", device);
   hipStream_t s = (hipStream_t)stream;
   SyncBracket sync(s);
-  // per call, in the per-device workspace: w1' (bf16 [2H][C]), its table (bf16 [2H][8]), w2 fragment-major (bf16 [C][H]),
-  // a zero bias [C]
-  const size_t w1_bytes = (size_t)2 * hidden * c * 2, tab_bytes = (size_t)2 * hidden * 16, w2_bytes = (size_t)hidden * c * 2;
-  char* ws = (char*)workspace(device, w1_bytes + tab_bytes + w2_bytes + (size_t)c * 2);
+  // per call, in the per-device workspace: w1' (bf16 [2H][C]), b' (fp32 [2H]), w2 fragment-major (bf16 [C][H]), a zero
+  // bias [C]
+  const size_t w1_bytes = (size_t)2 * hidden * c * 2, b32_bytes = (((size_t)2 * hidden * 4) + 255) & ~(size_t)255;
+  const size_t w2_bytes = (size_t)hidden * c * 2;
+  char* ws = (char*)workspace(device, w1_bytes + b32_bytes + w2_bytes + (size_t)c * 2);
   if (!ws) return F3D_ERR_RUNTIME;
   uint16_t* w1p = (uint16_t*)ws;
-  uint16_t* table = (uint16_t*)(ws + w1_bytes);
-  uint16_t* w2p = (uint16_t*)(ws + w1_bytes + tab_bytes);
-  uint16_t* zero_bias = (uint16_t*)(ws + w1_bytes + tab_bytes + w2_bytes);
+  float* b32 = (float*)(ws + w1_bytes);
+  uint16_t* w2p = (uint16_t*)(ws + w1_bytes + b32_bytes);
+  uint16_t* zero_bias = (uint16_t*)(ws + w1_bytes + b32_bytes + w2_bytes);
   if (!b2) b2 = zero_bias;
-  launch_ln_fold(w1, gamma, beta, b1, w1p, table, nullptr, 2 * hidden, c, s);
+  launch_ln_fold(w1, gamma, beta, b1, w1p, b32, 2 * hidden, c, s);
   hipLaunchKernelGGL(mlp_w2_prep_kernel, dim3(cdiv_u32(c * hidden / 8, 256)), dim3(256), 0, s, w2, w2p, zero_bias, c, hidden);
   int rc;
-  if (c == 256) rc = launch_mlp<256>(x, ldx, eps, w1p, table, w2p, b2, residual, ldr, y, ldy, m, hidden, device, s);
-  else if (c == 32) rc = launch_mlp_small<32>(x, ldx, eps, w1p, table, w2p, b2, residual, ldr, y, ldy, m, hidden, device, s);
-  else if (c == 64) rc = launch_mlp_small<64>(x, ldx, eps, w1p, table, w2p, b2, residual, ldr, y, ldy, m, hidden, device, s);
-  else rc = launch_mlp<128>(x, ldx, eps, w1p, table, w2p, b2, residual, ldr, y, ldy, m, hidden, device, s);
+  if (c == 256) rc = launch_mlp<256>(x, ldx, eps, w1p, b32, w2p, b2, residual, ldr, y, ldy, m, hidden, device, s);
+  else if (c == 32) rc = launch_mlp_small<32>(x, ldx, eps, w1p, b32, w2p, b2, residual, ldr, y, ldy, m, hidden, device, s);
+  else if (c == 64) rc = launch_mlp_small<64>(x, ldx, eps, w1p, b32, w2p, b2, residual, ldr, y, ldy, m, hidden, device, s);
+  else rc = launch_mlp<128>(x, ldx, eps, w1p, b32, w2p, b2, residual, ldr, y, ldy, m, hidden, device, s);
   if (rc != F3D_OK) return rc;
   F3D_CHECK_HIP(hipGetLastError());
   return F3D_OK;

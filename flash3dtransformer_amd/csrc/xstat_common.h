@@ -88,9 +88,8 @@ struct XsGeom {
   __host__ __device__ static constexpr uint32_t swz(uint32_t row) { return (row / RP) & SWZ_MASK; }
 };
 
-// w' = bf16(w * gamma), the per-feature table (wsum and b' = b + w beta in bf16 parts) and, when bias32 is not null,
-// b' as fp32 (defined with the linear kernels)
+// w' = bf16(w * gamma) and b' = b + w beta as fp32 (defined with the linear kernels)
 void launch_ln_fold(const uint16_t* w, const uint16_t* gamma, const uint16_t* beta, const uint16_t* bias, uint16_t* wp,
-                    uint16_t* lnx, float* bias32, uint32_t N, uint32_t K, hipStream_t s);
+                    float* bias32, uint32_t N, uint32_t K, hipStream_t s);
 
 }  // namespace f3d

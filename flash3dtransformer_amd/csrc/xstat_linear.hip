@@ -366,44 +366,27 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
   }
 }
 
-// w' = bf16(w * gamma), b' as fp32 (bias32, may be null) and the table row of every output feature n:
-//   (wsum_hi, wsum_hi, wsum_lo, b'_hi, b'_hi, b'_lo, 0, 0) in bf16, with
-//   wsum[n] = sum_k w'[n][k] (of the rounded values the matrix core will see), b'[n] = bias[n] + sum_k w[n][k] * beta[k].
-// One wave per output feature.
+// w' = bf16(w * gamma) and b'[n] = bias[n] + sum_k w[n][k] * beta[k] as fp32.  One wave per output feature.
 __global__ __launch_bounds__(256) void ln_fold_kernel(const uint16_t* __restrict__ w, const uint16_t* __restrict__ gamma,
                                                       const uint16_t* __restrict__ beta,
                                                       const uint16_t* __restrict__ bias, uint16_t* __restrict__ wp,
-                                                      uint16_t* __restrict__ lnx, float* __restrict__ bias32,
-                                                      uint32_t N, uint32_t K) {
+                                                      float* __restrict__ bias32, uint32_t N, uint32_t K) {
   const uint32_t n = blockIdx.x * 4 + threadIdx.x / kWave, lane = threadIdx.x % kWave;
   if (n >= N) return;
-  float s = 0.f, t = 0.f;
+  float t = 0.f;
   for (uint32_t k = lane; k < K; k += kWave) {
     const float wv = bf16_bits_to_float(w[(size_t)n * K + k]);
-    const uint16_t r = float_to_bf16_bits(wv * bf16_bits_to_float(gamma[k]));
-    wp[(size_t)n * K + k] = r;
-    s += bf16_bits_to_float(r);
+    wp[(size_t)n * K + k] = float_to_bf16_bits(wv * bf16_bits_to_float(gamma[k]));
     if (beta) t = __builtin_fmaf(wv, bf16_bits_to_float(beta[k]), t);
   }
 #pragma unroll
-  for (int o = 32; o > 0; o >>= 1) {
-    s += __shfl_xor(s, o, kWave);
-    t += __shfl_xor(t, o, kWave);
-  }
-  if (lane == 0) {
-    const float b = t + (bias ? bf16_bits_to_float(bias[n]) : 0.f);
-    const uint16_t s_hi = float_to_bf16_bits(s), b_hi = float_to_bf16_bits(b);
-    const uint16_t s_lo = float_to_bf16_bits(s - bf16_bits_to_float(s_hi));
-    const uint16_t b_lo = float_to_bf16_bits(b - bf16_bits_to_float(b_hi));
-    uint16_t* row = lnx + (size_t)n * 8;
-    row[0] = s_hi; row[1] = s_hi; row[2] = s_lo; row[3] = b_hi; row[4] = b_hi; row[5] = b_lo; row[6] = 0; row[7] = 0;
-    if (bias32) bias32[n] = b;
-  }
+  for (int o = 32; o > 0; o >>= 1) t += __shfl_xor(t, o, kWave);
+  if (lane == 0) bias32[n] = t + (bias ? bf16_bits_to_float(bias[n]) : 0.f);
 }
 
 void launch_ln_fold(const uint16_t* w, const uint16_t* gamma, const uint16_t* beta, const uint16_t* bias, uint16_t* wp,
-                    uint16_t* lnx, float* bias32, uint32_t N, uint32_t K, hipStream_t s) {
-  hipLaunchKernelGGL(ln_fold_kernel, dim3(cdiv_u32(N, 4)), dim3(256), 0, s, w, gamma, beta, bias, wp, lnx, bias32, N, K);
+                    float* bias32, uint32_t N, uint32_t K, hipStream_t s) {
+  hipLaunchKernelGGL(ln_fold_kernel, dim3(cdiv_u32(N, 4)), dim3(256), 0, s, w, gamma, beta, bias, wp, bias32, N, K);
 }
 
 template <int K, int MT, int WAVES, int NBUF>
@@ -449,15 +432,13 @@ int launch_xstat_linear(const uint16_t* x, uint32_t ldx, const uint16_t* gamma, 
   if ((uint64_t)N * K * 2 >= (1ull << 32)) return F3D_ERR_UNSUPPORTED;   // 32-bit byte offsets into w
   const uint16_t* lnx = nullptr;
   if (ln) {
-    // per call: w' (bf16 [N][K]), the table (bf16 [N][8], unused by this kernel) and b' (fp32 [N]) in the per-device
-    // workspace
+    // per call: w' (bf16 [N][K]) and b' (fp32 [N]) in the per-device workspace
     const size_t wp_bytes = ((size_t)N * K * 2 + 255) & ~(size_t)255;
-    char* ws = (char*)workspace(device, wp_bytes + (size_t)N * 16 + (size_t)N * 4);
+    char* ws = (char*)workspace(device, wp_bytes + (size_t)N * 4);
     if (!ws) return F3D_ERR_RUNTIME;
     uint16_t* wp = (uint16_t*)ws;
-    uint16_t* table = (uint16_t*)(ws + wp_bytes);
-    float* b32 = (float*)(ws + wp_bytes + (size_t)N * 16);
-    launch_ln_fold(w, gamma, beta, bias, wp, table, b32, N, K, s);
+    float* b32 = (float*)(ws + wp_bytes);
+    launch_ln_fold(w, gamma, beta, bias, wp, b32, N, K, s);
     w = wp;
     lnx = (const uint16_t*)b32;   // the kernel reads b' from here
   }

@@ -211,8 +211,9 @@ def test_fused_mlp_matches_two_kernel_path(oracle, M, C, H, use_res, use_bias):
     torch.cuda.synchronize()
     d = (y.float() - y2.float()).abs()
     scale = y2.float().abs().clamp(min=1.0)
-    # a hidden value that rounds the other way (the fused kernel forms b' from its two bf16 parts, the two-kernel path
-    # from fp32) moves an output by a step or two before the final rounding: at most four bf16 steps apart
+    # a hidden value that rounds the other way (the two paths sum fc1 in different orders: the fused kernel starts its
+    # accumulators from b', the other adds it last) moves an output by a step or two before the final rounding: at most
+    # four bf16 steps apart
     assert (d / scale).max().item() <= 2 ** -5, (d / scale).max().item()
     assert (d > 0).float().mean().item() < 0.02                                     # and almost always equal
     # (b) against the unrounded mathematics: at least as close as the reference's own sequence of bf16 roundings
