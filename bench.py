@@ -90,8 +90,9 @@ def main():
                          "kernels.  Optional group names restrict the run: attention, psh, permute, pool, hourglass")
     args = ap.parse_args()
     if args.gpus != 1:
-        print("bench.py: this build runs on ONE GPU; the path shards by cloud without any exchange "
-              "(see DESIGN.md), and no multi-GPU figure is produced. Re-run with --gpus 1.", file=sys.stderr)
+        print("bench.py: this build runs on ONE GPU; the path shards by cloud without any exchange between GPUs (each cloud "
+              "is bucketed, pooled and attended to on its own), and no multi-GPU figure is produced. Re-run with --gpus 1.",
+              file=sys.stderr)
         sys.exit(2)
 
     from flash3dtransformer_amd import synth
