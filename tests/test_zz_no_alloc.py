@@ -76,3 +76,47 @@ def test_no_alloc_entry_point_says_when_a_batch_does_not_fit():
         pshattn.batch_psh_scatter_pad_hash(coords, buf.bucket_id, buf.bucket_cntr, buf.bucket_offs, seps, mx, nb, div,
                                            512, 0xFFFF, bb, bb + 1, buf.probe_offs, buf.bucket_cumsum,
                                            buf.scattered_coord, 0.0, 1, no_alloc=True)
+
+
+def test_no_alloc_entry_point_in_a_captured_graph_replays_to_the_eager_result():
+    """A caller that captures its stream (the kind of caller the entry point is for): the call sits in a HIP graph next
+    to the fill kernel that clears the counters; every replay, with eager work and synchronisations of the program in
+    between, leaves exactly what the eager call leaves."""
+    from flash3dtransformer_amd import configs, synth
+    from flash3dtransformer_amd.lib import pshattn
+    from flash3dtransformer_amd.psh import psh_main
+    pshattn.DeviceManagerSingleton.instance().init_dev_info(0)
+    pshattn.DeviceManagerSingleton.instance().set_psh_rebalance(1)
+    coords, seps, _ = configs.lidar_batch(2, 60_000, 1010)
+    coords, seps = configs.to_device(coords, seps, DEV)
+    nb, div, mx = psh_main.bucket_geometry(seps, 512)
+    pad_to = -(-coords.shape[0] // 3072) * 3072
+    buf = psh_main.BucketScatterBuffers.create_buffers(coords, seps, 512, pad_to, nb)
+    bb_min, bb_max = coords.min(0)[0].contiguous(), coords.max(0)[0].contiguous()
+
+    def run():
+        buf.bucket_cntr.zero_()
+        pshattn.batch_psh_scatter_pad_hash(coords, buf.bucket_id, buf.bucket_cntr, buf.bucket_offs, seps, mx, nb, div,
+                                           512, 0xFFFF, bb_min, bb_max, buf.probe_offs, buf.bucket_cumsum,
+                                           buf.scattered_coord, 0.0, 2, no_alloc=True)
+    names = ("bucket_id", "bucket_cntr", "bucket_offs", "bucket_cumsum", "scattered_coord")
+    run()
+    torch.cuda.synchronize()
+    want = {n: getattr(buf, n).clone() for n in names}
+    graph, side = torch.cuda.CUDAGraph(), torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        run()                                      # warm-up on the capture stream
+        torch.cuda.synchronize()
+        with torch.cuda.graph(graph, stream=side):
+            run()
+    torch.cuda.synchronize()
+    for _ in range(4):
+        for n in ("bucket_id", "bucket_offs", "bucket_cumsum", "scattered_coord"):
+            getattr(buf, n).view(torch.int16).fill_(0x3C00)         # stale contents the replay must overwrite
+        x = torch.randn(512, 512, device=DEV)
+        assert torch.isfinite((x @ x).sum()).item()                 # eager work and a synchronisation in between
+        graph.replay()
+        torch.cuda.synchronize()
+        for n in names:
+            bits = {2: torch.int16, 4: torch.int32}[want[n].element_size()]
+            assert torch.equal(getattr(buf, n).view(bits), want[n].view(bits)), n
