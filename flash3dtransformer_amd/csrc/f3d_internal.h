@@ -55,13 +55,18 @@ int rebalance_mode();
 
 // RAII bracket reproducing the reference's optional stream synchronisation around an op
 // (src/psh/batch_psh_bucket_dispatcher.cu:278-280, 323-325).
+// A stream that is being captured is left alone (synchronising it would invalidate the capture).
 struct SyncBracket {
   hipStream_t s;
-  explicit SyncBracket(hipStream_t stream) : s(stream) {
-    if (sync_stream_enabled()) (void)hipStreamSynchronize(s);
+  bool on;
+  explicit SyncBracket(hipStream_t stream) : s(stream), on(false) {
+    if (!sync_stream_enabled()) return;
+    hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+    on = hipStreamIsCapturing(s, &st) == hipSuccess && st == hipStreamCaptureStatusNone;
+    if (on) (void)hipStreamSynchronize(s);
   }
   ~SyncBracket() {
-    if (sync_stream_enabled()) (void)hipStreamSynchronize(s);
+    if (on) (void)hipStreamSynchronize(s);
   }
 };
 

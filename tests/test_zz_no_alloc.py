@@ -87,6 +87,9 @@ def test_no_alloc_entry_point_in_a_captured_graph_replays_to_the_eager_result():
     from flash3dtransformer_amd.psh import psh_main
     pshattn.DeviceManagerSingleton.instance().init_dev_info(0)
     pshattn.DeviceManagerSingleton.instance().set_psh_rebalance(1)
+    # the optional synchronisation around every op stays switched on, as earlier tests leave it: the library must not
+    # synchronise a stream that is being captured
+    pshattn.DeviceManagerSingleton.instance().set_sync_stream(True)
     coords, seps, _ = configs.lidar_batch(2, 60_000, 1010)
     coords, seps = configs.to_device(coords, seps, DEV)
     nb, div, mx = psh_main.bucket_geometry(seps, 512)
