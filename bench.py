@@ -184,7 +184,7 @@ def main():
                "ln_fc1_act": "xstat_linear_kernel<256,2,8,3,LN,swiglu> + ln_fold_kernel",
                "proj_residual": "xstat_linear_kernel<256,2,8,3,residual>",
                "fc2_residual": "ystat_linear_kernel<256> + ys_w_prep_kernel",
-               "ln_mlp_residual": "ln_mlp_swiglu_kernel<256> + ln_fold_kernel + mlp_w2_prep_kernel"}
+               "ln_mlp_residual": "ln_mlp_swiglu_kernel<256> + mlp_prep_kernel"}
     flops = {kname: vv for kname, vv in flops.items() if kname in breakdown}
     # the two-kernel form of the MLP (what the layer runs below 60 k rows, or with fused=False), same tensors
     two_kernel_mlp = None

@@ -56,8 +56,8 @@ struct MlpGeom {
   }
 };
 
-// w1p: LayerNorm-folded fc1 weight [2 H][K] (value rows then gate rows), b32: b' = b1 + w1 beta as fp32 [2 H] (ln_fold_kernel);
-// w2p: fc2 weight, fragment-major per chunk (mlp_w2_prep_kernel); bias2 [K] (zeros when the layer has none);
+// w1p: LayerNorm-folded fc1 weight [2 H][K] (value rows then gate rows), b32: b' = b1 + w1 beta as fp32 [2 H] (mlp_prep_kernel);
+// w2p: fc2 weight, fragment-major per chunk (mlp_prep_kernel); bias2 [K] (zeros when the layer has none);
 // H: hidden width, multiple of 32.
 template <int K>
 __global__ __launch_bounds__(64 * kMlpWaves) __attribute__((amdgpu_waves_per_eu(2, 2))) void ln_mlp_swiglu_kernel(
@@ -508,9 +508,19 @@ __global__ __launch_bounds__(64 * kMlpSmallWaves) void ln_mlp_swiglu_small_kerne
 // w2 [C][H] row-major -> fragment-major per chunk of 32 hidden features:
 //   w2p[(((c * C/32 + ot) * 2 + s) * 64 + half * 32 + lq) * 8 + e] = w2[ot * 32 + lq][c * 32 + (2 s + e / 4) * 8 + half * 4 + e % 4]
 // One thread per 16-byte piece.
-__global__ __launch_bounds__(256) void mlp_w2_prep_kernel(const uint16_t* __restrict__ w2, uint16_t* __restrict__ w2p,
-                                                          uint16_t* __restrict__ zero_bias, uint32_t C, uint32_t H) {
-  const uint32_t piece = blockIdx.x * blockDim.x + threadIdx.x;
+// The LayerNorm fold of w1 (one wave per fc1 feature, blocks [0, fold_blocks)) rides in the same launch.
+__global__ __launch_bounds__(256) void mlp_prep_kernel(const uint16_t* __restrict__ w1, const uint16_t* __restrict__ gamma,
+                                                       const uint16_t* __restrict__ beta, const uint16_t* __restrict__ b1,
+                                                       uint16_t* __restrict__ w1p, float* __restrict__ b32,
+                                                       uint32_t fold_blocks, const uint16_t* __restrict__ w2,
+                                                       uint16_t* __restrict__ w2p, uint16_t* __restrict__ zero_bias,
+                                                       uint32_t C, uint32_t H) {
+  if (blockIdx.x < fold_blocks) {
+    const uint32_t n = blockIdx.x * 4 + threadIdx.x / kWave;
+    if (n < 2 * H) ln_fold_row(w1, gamma, beta, b1, w1p, b32, C, n, threadIdx.x % kWave);
+    return;
+  }
+  const uint32_t piece = (blockIdx.x - fold_blocks) * blockDim.x + threadIdx.x;
   if (piece < C / 8) *reinterpret_cast<uint4*>(zero_bias + piece * 8) = make_uint4(0u, 0u, 0u, 0u);   // stands in for a missing bias
   if (piece >= C * H / 8) return;
   const uint32_t lq = piece % 32, half = (piece / 32) % 2, s = (piece / 64) % 2;
@@ -620,8 +630,9 @@ int f3d_ln_mlp_swiglu_bf16(const f3d_bf16_t* x, uint32_t ldx, const f3d_bf16_t* 
   uint16_t* w2p = (uint16_t*)(ws + w1_bytes + b32_bytes);
   uint16_t* zero_bias = (uint16_t*)(ws + w1_bytes + b32_bytes + w2_bytes);
   if (!b2) b2 = zero_bias;
-  launch_ln_fold(w1, gamma, beta, b1, w1p, b32, 2 * hidden, c, s);
-  hipLaunchKernelGGL(mlp_w2_prep_kernel, dim3(cdiv_u32(c * hidden / 8, 256)), dim3(256), 0, s, w2, w2p, zero_bias, c, hidden);
+  const uint32_t fold_blocks = cdiv_u32(2 * hidden, 4);
+  hipLaunchKernelGGL(mlp_prep_kernel, dim3(fold_blocks + cdiv_u32(c * hidden / 8, 256)), dim3(256), 0, s, w1, gamma, beta, b1,
+                     w1p, b32, fold_blocks, w2, w2p, zero_bias, c, hidden);
   int rc;
   if (c == 256) rc = launch_mlp<256>(x, ldx, eps, w1p, b32, w2p, b2, residual, ldr, y, ldy, m, hidden, device, s);
   else if (c == 32) rc = launch_mlp_small<32>(x, ldx, eps, w1p, b32, w2p, b2, residual, ldr, y, ldy, m, hidden, device, s);

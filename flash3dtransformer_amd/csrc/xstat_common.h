@@ -88,6 +88,23 @@ struct XsGeom {
   __host__ __device__ static constexpr uint32_t swz(uint32_t row) { return (row / RP) & SWZ_MASK; }
 };
 
+// One wave folds one output feature n of a LayerNorm into the Linear behind it: w'[n][:] = bf16(w[n][:] * gamma) and
+// b'[n] = bias[n] + sum_k w[n][k] * beta[k] as fp32.
+__device__ __forceinline__ void ln_fold_row(const uint16_t* __restrict__ w, const uint16_t* __restrict__ gamma,
+                                            const uint16_t* __restrict__ beta, const uint16_t* __restrict__ bias,
+                                            uint16_t* __restrict__ wp, float* __restrict__ bias32, uint32_t K, uint32_t n,
+                                            uint32_t lane) {
+  float t = 0.f;
+  for (uint32_t k = lane; k < K; k += kWave) {
+    const float wv = bf16_bits_to_float(w[(size_t)n * K + k]);
+    wp[(size_t)n * K + k] = float_to_bf16_bits(wv * bf16_bits_to_float(gamma[k]));
+    if (beta) t = __builtin_fmaf(wv, bf16_bits_to_float(beta[k]), t);
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) t += __shfl_xor(t, o, kWave);
+  if (lane == 0) bias32[n] = t + (bias ? bf16_bits_to_float(bias[n]) : 0.f);
+}
+
 // w' = bf16(w * gamma) and b' = b + w beta as fp32 (defined with the linear kernels)
 void launch_ln_fold(const uint16_t* w, const uint16_t* gamma, const uint16_t* beta, const uint16_t* bias, uint16_t* wp,
                     float* bias32, uint32_t N, uint32_t K, hipStream_t s);

@@ -373,15 +373,7 @@ __global__ __launch_bounds__(256) void ln_fold_kernel(const uint16_t* __restrict
                                                       float* __restrict__ bias32, uint32_t N, uint32_t K) {
   const uint32_t n = blockIdx.x * 4 + threadIdx.x / kWave, lane = threadIdx.x % kWave;
   if (n >= N) return;
-  float t = 0.f;
-  for (uint32_t k = lane; k < K; k += kWave) {
-    const float wv = bf16_bits_to_float(w[(size_t)n * K + k]);
-    wp[(size_t)n * K + k] = float_to_bf16_bits(wv * bf16_bits_to_float(gamma[k]));
-    if (beta) t = __builtin_fmaf(wv, bf16_bits_to_float(beta[k]), t);
-  }
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) t += __shfl_xor(t, o, kWave);
-  if (lane == 0) bias32[n] = t + (bias ? bf16_bits_to_float(bias[n]) : 0.f);
+  ln_fold_row(w, gamma, beta, bias, wp, bias32, K, n, lane);
 }
 
 void launch_ln_fold(const uint16_t* w, const uint16_t* gamma, const uint16_t* beta, const uint16_t* bias, uint16_t* wp,
