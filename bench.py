@@ -27,8 +27,8 @@ HBM_PEAK_GBS = 8000.0
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by a copy kernel of known
 # size, see profiles/encoder_stage_4x120k_hbm_traffic.md) at this bench's shapes
-TRAFFIC_BYTES_PER_LAUNCH = {"ln_fc1_act": 1.617e9, "ln_qkv": 1.022e9, "attention": 1.017e9,
-                            "proj_residual": 0.764e9, "fc2_residual": 1.848e9, "ln_mlp_residual": 0.832e9}
+TRAFFIC_BYTES_PER_LAUNCH = {"ln_fc1_act": 1.613e9, "ln_qkv": 1.022e9, "attention": 1.019e9,
+                            "proj_residual": 0.763e9, "fc2_residual": 1.847e9, "ln_mlp_residual": 0.849e9}
 
 
 def ev_time(fn, iters, warmup=3):
