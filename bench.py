@@ -87,7 +87,7 @@ def main():
     ap.add_argument("--no-sub-metrics", action="store_true")
     ap.add_argument("--sub-metrics-only", nargs="*", default=None, metavar="GROUP",
                     help="run only the per-kernel sub-metrics (configs 1, 2, 3, 5) and print them; for profiling those "
-                         "kernels.  Optional group names restrict the run: attention, psh, permute, pool, hourglass")
+                         "kernels.  Optional group names restrict the run: attention, psh, permute, pool, hourglass, mfma")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU; the path shards by cloud without any exchange between GPUs (each cloud "
@@ -249,11 +249,25 @@ def sub_metrics(dev, only=None):
     unpooling GB/s on config 3 — each against its roofline.  `only`: a set of group names, or None for all"""
     out = {}
     groups = {"attention": sub_attention, "psh": sub_psh, "permute": sub_permute, "pool": sub_pool,
-              "hourglass": lambda d, o: o.__setitem__("hourglass_c5", hourglass_c5(d))}
+              "hourglass": lambda d, o: o.__setitem__("hourglass_c5", hourglass_c5(d)), "mfma": sub_mfma_rate}
     for name, fn in groups.items():
         if only is None or name in only:
             fn(dev, out)
     return out
+
+
+def sub_mfma_rate(dev, out):
+    """what the matrix cores of this GPU sustain on dense bf16 products with nothing else running (register operands,
+    4 waves per SIMD): with random operands the power budget sets the clock, with a zero operand the data-sheet rate
+    is reached.  Context for the `frac` figures, which are priced against the data-sheet 2.5 PFLOP/s."""
+    from flash3dtransformer_amd.lib import pshattn
+    sink = torch.zeros(1, dtype=torch.float32, device=dev)
+    wgs, iters = 1024, 100000
+    flop = wgs * 4 * iters * 8 * 32768.0
+    for name, ra, rb in (("random_operands", True, True), ("one_zero_operand", False, True)):
+        ms = ev_time(lambda: pshattn.probe_mfma_bf16(wgs, iters, ra, rb, sink), 3, warmup=1)
+        out["mfma_bf16_dense_rate_" + name] = {"ms": round(ms, 3), "tflops": round(flop / ms / 1e9, 1),
+                                               "frac_of_bf16_mfma_peak": round(flop / ms / 1e9 / MFMA_BF16_PEAK_TFLOPS, 4)}
 
 
 def sub_attention(dev, out):

@@ -542,6 +542,15 @@ def ln_mlp_swiglu_bf16(x, gamma, beta, eps, w1, b1, w2, b2, residual, y) -> bool
     return True
 
 
+def probe_mfma_bf16(workgroups: int, iters: int, random_a: bool, random_b: bool, sink: torch.Tensor):
+    """measurement aid: workgroups x 4 waves x iters x 8 dense bf16 MFMA products (32,768 flops each) on register
+    operands, pseudo-random or zero; the caller times it (see bench.py)"""
+    assert_dtype([sink], torch.float32)
+    dev = assert_same_device([sink])
+    _check(_load().f3d_probe_mfma_bf16(_u32(workgroups), _u32(iters), _u32(1 if random_a else 0),
+                                       _u32(1 if random_b else 0), _ptr(sink), _i32(dev), _stream(dev)))
+
+
 def layernorm_bf16(x, gamma, beta, y, eps=1e-5):
     """extension: LayerNorm over the last axis, fp32 statistics"""
     assert_contiguous([x, gamma, y])

@@ -226,6 +226,14 @@ int f3d_buck_swin_fwd_strided(const f3d_bf16_t* q, const f3d_bf16_t* k, const f3
                               uint32_t bucket_size, uint32_t batch, uint32_t seq_len, uint32_t num_head,
                               uint32_t head_dim, const int32_t* kv_len, int device, void* stream);
 
+/* ---- measurement aid (no counterpart in the reference, not on the hot path) -------------------
+ * Runs `workgroups` x 4 waves x `iters` x 8 back-to-back v_mfma_f32_32x32x16_bf16 products (32,768 flops each) on
+ * register operands that are pseudo-random (random_a / random_b != 0) or zero, so that a caller timing it sees the rate
+ * the matrix cores sustain under the power budget (random operands) and at the data-sheet clock (a zero operand).
+ * sink: one float of device memory (never written). */
+int f3d_probe_mfma_bf16(uint32_t workgroups, uint32_t iters, uint32_t random_a, uint32_t random_b, float* sink,
+                        int device, void* stream);
+
 /* ---- dense layers --------------------------------------------------------------------------
  * gemm_sm_bf16(A[M,K], B[K,N], O[M,N]) — src/f3d_frontend.cu:87-88, src/psh/gemm_dispatcher.cu;
  * the reference only accepts M == 128, this one any shape with K % 8 == 0 and N % 8 == 0. */

@@ -291,3 +291,15 @@ def test_fused_mlp_and_output_panel_kernel_at_bench_size():
     torch.cuda.synchronize()
     d = (y2[-n_small:].float() - y3.float()).abs() / (y3.float().abs() + x[-n_small:].float().abs()).clamp(min=1.0)
     assert d.max().item() <= 2 ** -6 and (d > 0).float().mean().item() < 0.02
+
+
+def test_mfma_rate_probe_runs():
+    """the measurement aid behind bench.py's `mfma_bf16_dense_rate_*`: launches, finishes, leaves its sink alone"""
+    from flash3dtransformer_amd.lib import pshattn
+    sink = torch.full((1,), 5.0, dtype=torch.float32, device=DEV)
+    for ra, rb in ((True, True), (False, True)):
+        pshattn.probe_mfma_bf16(64, 100, ra, rb, sink)
+    torch.cuda.synchronize()
+    assert sink.item() == 5.0
+    with pytest.raises(RuntimeError, match="out of range"):
+        pshattn.probe_mfma_bf16(0, 100, True, True, sink)
