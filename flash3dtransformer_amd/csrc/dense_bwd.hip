@@ -1,0 +1,461 @@
+// Backward of the dense layers for gfx950: weight / bias gradient of a linear layer, LayerNorm backward and the
+// backward of the gated activation.  The input gradient of a linear layer is itself a linear layer (dx = dy · w), so it
+// runs on the forward kernels with the transposed weight.
+//
+// The reference takes these from torch.nn.Linear / TransformerEngine autograd (flash3dxfmr/layers/buck_swin.py:159-163,
+// elem_wise.py:22-26, stage.py:94-99); nothing of it lives in the reference's own sources.
+//
+// Weight gradient  dw[n][k] = sum_m dy[m][n] x[m][k]  (fp32 out, bf16 in):
+//   the reduction runs over the rows, which is the slow axis of both operands in memory, so both MFMA operands are
+//   read TRANSPOSED from LDS (ds_read_b64_tr_b16: a lane receives four consecutive rows of one column).  A workgroup of
+//   eight waves (4 x 2, two per SIMD) owns a 256 x 256 tile of dw and one slab of rows; a wave holds 64 x 128 of it in
+//   128 accumulator registers and skips the 32 x 32 blocks that lie outside dw.  64-row stages go global -> registers
+//   -> LDS (row pitch = row bytes + 32, which spreads the four rows of a transposing read over all banks),
+//   double-buffered, one barrier per stage.  Slabs are sized so that the launch is one round of the chip; every slab
+//   writes its partial tile to the workspace and a second kernel sums the slabs in a fixed order (no atomics: the
+//   result does not depend on scheduling).  The bias gradient is summed on the vector unit from the dy pieces a
+//   thread stages anyway (always the same 8 columns), in the workgroups of the first k-tile.
+#include "f3d_device.h"
+#include "f3d_internal.h"
+
+namespace f3d {
+namespace {
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x16_t __attribute__((ext_vector_type(16)));
+typedef short i16x4_t __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) i16x4_t lds_i16x4_t;
+
+constexpr int kXcd = 8;
+constexpr int kWgThreads = 512;
+constexpr int kWgNT = 256, kWgKT = 256, kWgMT = 64;
+constexpr int kPitchA = kWgNT * 2 + 32, kPitchB = kWgKT * 2 + 32;   // bytes
+constexpr int kTileA = kWgMT * kPitchA, kTileB = kWgMT * kPitchB;
+constexpr int kWgBuf = kTileA + kTileB;
+constexpr int kWgLds = 2 * kWgBuf;
+constexpr int kPiecesA = kWgMT * (kWgNT / 8) / kWgThreads;   // 16-byte pieces per thread and stage
+constexpr int kPiecesB = kWgMT * (kWgKT / 8) / kWgThreads;
+static_assert(kPitchA % 128 == 32 && kPitchB % 128 == 32, "four consecutive rows cover all banks");
+static_assert(kWgThreads % (kWgNT / 8) == 0, "a thread stages the same dy columns in every piece");
+static_assert(kWgLds <= 160 * 1024 && (kWgThreads / (kWgNT / 8)) * kWgNT * 4 <= kWgLds, "LDS budget");
+
+// two transposing reads -> one 8-value MFMA operand: slots 0..3 = rows r .. r+3, slots 4..7 = rows r+4 .. r+7 of the
+// lane's column (the same row order for both operands, so the products pair up)
+__device__ __forceinline__ bf16x8_t read_tr8(const char* p, int pitch) {
+  const i16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_t*)p);
+  const i16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_t*)(p + 4 * pitch));
+  return __builtin_bit_cast(bf16x8_t, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+}
+
+__global__ __launch_bounds__(kWgThreads) void linear_wgrad_kernel(
+    const uint16_t* __restrict__ dy, uint32_t lddy, const uint16_t* __restrict__ x, uint32_t ldx,
+    float* __restrict__ part_w, float* __restrict__ part_b, uint32_t M, uint32_t N, uint32_t K, uint32_t n_tiles,
+    uint32_t k_tiles, uint32_t slabs, uint32_t slab_rows, uint32_t items_per_xcd) {
+  extern __shared__ __attribute__((aligned(16))) char lds_wg[];
+  // workgroups of one XCD take consecutive items, so the tiles of one slab (which re-read the same rows of x and
+  // dy) meet in one L2
+  const uint32_t tiles = n_tiles * k_tiles, n_items = tiles * slabs;
+  const uint32_t item = (blockIdx.x % kXcd) * items_per_xcd + blockIdx.x / kXcd;
+  if (blockIdx.x / kXcd >= items_per_xcd || item >= n_items) return;
+  const uint32_t slab = item / tiles, tile = item % tiles;
+  const uint32_t n0 = (tile / k_tiles) * kWgNT, k0 = (tile % k_tiles) * kWgKT;
+  const uint32_t m_begin = slab * slab_rows, m_end = min(M, m_begin + slab_rows);
+  const uint32_t tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
+  const uint32_t nw = wave >> 1, kw = wave & 1u;   // 4 x 2 waves
+  const bool with_bias = part_b != nullptr && k0 == 0;     // uniform over the workgroup
+  // 32 x 32 blocks of this wave's 64 x 128 that lie inside dw
+  const uint32_t n_w = n0 + nw * 64u, k_w = k0 + kw * 128u;
+  const uint32_t ni = n_w >= N ? 0u : min(2u, (N - n_w + 31u) / 32u), nj = k_w >= K ? 0u : min(4u, (K - k_w + 31u) / 32u);
+  float colsum[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) colsum[e] = 0.f;
+
+  // ---- staging: which 16-byte pieces this thread moves ----
+  u32x4_t ra[kPiecesA], rb[kPiecesB];
+  auto fetch = [&](uint32_t m0) {
+#pragma unroll
+    for (int i = 0; i < kPiecesA; ++i) {
+      const uint32_t idx = tid + kWgThreads * i, row = idx / (kWgNT / 8), pc = idx % (kWgNT / 8);
+      ra[i] = u32x4_t{0u, 0u, 0u, 0u};
+      if (m0 + row < m_end && n0 + pc * 8 < N)
+        ra[i] = *reinterpret_cast<const u32x4_t*>(dy + (size_t)(m0 + row) * lddy + n0 + pc * 8);
+    }
+#pragma unroll
+    for (int i = 0; i < kPiecesB; ++i) {
+      const uint32_t idx = tid + kWgThreads * i, row = idx / (kWgKT / 8), pc = idx % (kWgKT / 8);
+      rb[i] = u32x4_t{0u, 0u, 0u, 0u};
+      if (m0 + row < m_end && k0 + pc * 8 < K)
+        rb[i] = *reinterpret_cast<const u32x4_t*>(x + (size_t)(m0 + row) * ldx + k0 + pc * 8);
+    }
+  };
+  auto stash = [&](char* buf) {
+#pragma unroll
+    for (int i = 0; i < kPiecesA; ++i) {
+      const uint32_t idx = tid + kWgThreads * i, row = idx / (kWgNT / 8), pc = idx % (kWgNT / 8);
+      *reinterpret_cast<u32x4_t*>(buf + row * kPitchA + pc * 16) = ra[i];
+      if (with_bias) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) { colsum[2 * e] += bf16_lo(ra[i][e]); colsum[2 * e + 1] += bf16_hi(ra[i][e]); }
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < kPiecesB; ++i) {
+      const uint32_t idx = tid + kWgThreads * i, row = idx / (kWgKT / 8), pc = idx % (kWgKT / 8);
+      *reinterpret_cast<u32x4_t*>(buf + kTileA + row * kPitchB + pc * 16) = rb[i];
+    }
+  };
+
+  // ---- the lane's place in a transposing read: lane p of a 16-lane block points at row p / 4, columns 4 (p % 4).. ----
+  const uint32_t half = lane >> 5, p16 = lane & 15u, cgrp = (lane >> 4) & 1u;
+  const uint32_t a_off = (8u * half + p16 / 4u) * kPitchA + (nw * 64u + 16u * cgrp + 4u * (p16 & 3u)) * 2u;
+  const uint32_t b_off = kTileA + (8u * half + p16 / 4u) * kPitchB + (kw * 128u + 16u * cgrp + 4u * (p16 & 3u)) * 2u;
+
+  f32x16_t acc[2][4];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+  const uint32_t n_stage = m_end > m_begin ? (m_end - m_begin + kWgMT - 1) / kWgMT : 0u;
+  if (n_stage) {
+    fetch(m_begin);
+    stash(lds_wg);
+  }
+  __syncthreads();
+  for (uint32_t st = 0; st < n_stage; ++st) {
+    const char* buf = lds_wg + (st & 1u) * kWgBuf;
+    const bool more = st + 1 < n_stage;
+    if (more) fetch(m_begin + (st + 1) * kWgMT);
+#pragma unroll
+    for (int ks = 0; ks < kWgMT / 16; ++ks) {
+      bf16x8_t fa[2], fb[4];
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+        if ((uint32_t)i < ni) fa[i] = read_tr8(buf + a_off + ks * 16 * kPitchA + i * 64, kPitchA);
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        if ((uint32_t)j < nj) fb[j] = read_tr8(buf + b_off + ks * 16 * kPitchB + j * 64, kPitchB);
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          if ((uint32_t)i < ni && (uint32_t)j < nj)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[j], acc[i][j], 0, 0, 0);
+    }
+    if (more) stash(lds_wg + ((st + 1) & 1u) * kWgBuf);
+    __syncthreads();
+  }
+
+  // ---- this slab's partial tile: accumulator slot e of a lane is row 8 (e / 4) + 4 half + e % 4, column lane % 32 ----
+  float* pw = part_w + (size_t)slab * N * K;
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+      const uint32_t n = n0 + nw * 64u + 32u * i + 8u * (e / 4) + 4u * half + (e % 4);
+      if (n >= N) continue;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const uint32_t k = k0 + kw * 128u + 32u * j + (lane & 31u);
+        if (k < K) pw[(size_t)n * K + k] = acc[i][j][e];
+      }
+    }
+  }
+  // ---- bias gradient: the 16 threads that staged the same 8 columns meet in LDS (the stage buffers are dead) ----
+  if (with_bias) {
+    constexpr int kGroups = kWgThreads / (kWgNT / 8);
+    float* s_cs = reinterpret_cast<float*>(lds_wg);
+    const uint32_t pc = tid % (kWgNT / 8), grp = tid / (kWgNT / 8);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) s_cs[grp * kWgNT + pc * 8 + e] = colsum[e];
+    __syncthreads();
+    if (tid < (uint32_t)kWgNT && n0 + tid < N) {
+      float t = 0.f;
+      for (int g = 0; g < kGroups; ++g) t += s_cs[g * kWgNT + tid];
+      part_b[(size_t)slab * N + n0 + tid] = t;
+    }
+  }
+}
+
+// out[i] = (accumulate ? out[i] : 0) + sum over p of part[p][i], p ascending
+__global__ __launch_bounds__(256) void sum_partials_kernel(const float* __restrict__ part, uint32_t n_part, size_t len,
+                                                           float* __restrict__ out, uint32_t accumulate) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= len) return;
+  float s = accumulate ? out[i] : 0.f;
+  for (uint32_t p = 0; p < n_part; ++p) s += part[(size_t)p * len + i];
+  out[i] = s;
+}
+
+// ---- LayerNorm backward: LPR lanes per row, 8 channels per lane.
+//   xhat = (x - mean) rstd, g = dh gamma, dx = rstd (g - mean(g) - xhat mean(g xhat)) (+ dres),
+//   dgamma = sum_rows dh xhat, dbeta = sum_rows dh.  A thread walks rows with a grid stride and keeps its 8 + 8 column
+//   sums in registers; the workgroup combines them through LDS and writes one partial per workgroup. ----
+template <int LPR>
+__global__ __launch_bounds__(256) void layernorm_bwd_kernel(const uint16_t* __restrict__ x, uint32_t ldx,
+                                                            const uint16_t* dh, uint32_t lddh,
+                                                            const uint16_t* __restrict__ gamma,
+                                                            const uint16_t* dres, uint32_t lddr,
+                                                            uint16_t* dx, uint32_t lddx,
+                                                            float* __restrict__ part, uint32_t M, float eps) {
+  constexpr int C = LPR * 8, RPB = 256 / LPR;
+  __shared__ float s_col[256][17];
+  const uint32_t tid = threadIdx.x, sub = tid % LPR, slot = tid / LPR;
+  float g8[8], dg[8], db[8];
+  {
+    const u32x4_t g = *reinterpret_cast<const u32x4_t*>(gamma + sub * 8);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) { g8[2 * e] = bf16_lo(g[e]); g8[2 * e + 1] = bf16_hi(g[e]); }
+  }
+#pragma unroll
+  for (int e = 0; e < 8; ++e) dg[e] = db[e] = 0.f;
+  // every lane of a row group runs the same number of iterations (the shuffles need all of them)
+  for (uint32_t base = blockIdx.x * RPB; base < M; base += gridDim.x * RPB) {
+    const uint32_t row = base + slot;
+    const bool ok = row < M;
+    u32x4_t vx = {0u, 0u, 0u, 0u}, vd = {0u, 0u, 0u, 0u}, vr = {0u, 0u, 0u, 0u};
+    if (ok) {
+      vx = *reinterpret_cast<const u32x4_t*>(x + (size_t)row * ldx + sub * 8);
+      vd = *reinterpret_cast<const u32x4_t*>(dh + (size_t)row * lddh + sub * 8);
+      if (dres) vr = *reinterpret_cast<const u32x4_t*>(dres + (size_t)row * lddr + sub * 8);
+    }
+    float xv[8], dv[8];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      xv[2 * e] = bf16_lo(vx[e]); xv[2 * e + 1] = bf16_hi(vx[e]);
+      dv[2 * e] = bf16_lo(vd[e]); dv[2 * e + 1] = bf16_hi(vd[e]);
+    }
+    float sum = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) sum += xv[e];
+#pragma unroll
+    for (int off = LPR / 2; off > 0; off >>= 1) sum += __shfl_xor(sum, off, kWave);
+    const float mean = sum / (float)C;
+    float sq = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) { xv[e] -= mean; sq += xv[e] * xv[e]; }
+#pragma unroll
+    for (int off = LPR / 2; off > 0; off >>= 1) sq += __shfl_xor(sq, off, kWave);
+    const float rstd = rsqrtf(sq / (float)C + eps);
+    float s1 = 0.f, s2 = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      xv[e] *= rstd;                       // xhat
+      const float g = dv[e] * g8[e];
+      s1 += g; s2 += g * xv[e];
+      dg[e] += dv[e] * xv[e]; db[e] += dv[e];   // rows past the end contribute zeros (dh = 0)
+    }
+#pragma unroll
+    for (int off = LPR / 2; off > 0; off >>= 1) {
+      s1 += __shfl_xor(s1, off, kWave);
+      s2 += __shfl_xor(s2, off, kWave);
+    }
+    s1 /= (float)C; s2 /= (float)C;
+    if (ok) {
+      u32x4_t t;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        float f0 = rstd * (dv[2 * e] * g8[2 * e] - s1 - xv[2 * e] * s2) + bf16_lo(vr[e]);
+        float f1 = rstd * (dv[2 * e + 1] * g8[2 * e + 1] - s1 - xv[2 * e + 1] * s2) + bf16_hi(vr[e]);
+        t[e] = pack_bf16x2(f0, f1);
+      }
+      *reinterpret_cast<u32x4_t*>(dx + (size_t)row * lddx + sub * 8) = t;
+    }
+  }
+#pragma unroll
+  for (int e = 0; e < 8; ++e) { s_col[tid][e] = dg[e]; s_col[tid][8 + e] = db[e]; }
+  __syncthreads();
+  // thread (sub, e) for e < 16 sums the RPB row slots of its column
+  for (uint32_t o = tid; o < LPR * 16u; o += 256u) {
+    const uint32_t su = o / 16u, e = o % 16u;
+    float s = 0.f;
+    for (uint32_t r = 0; r < (uint32_t)RPB; ++r) s += s_col[r * LPR + su][e];
+    // partial layout per workgroup: dgamma [C] then dbeta [C]
+    part[(size_t)blockIdx.x * 2u * C + (e / 8u) * C + su * 8u + (e % 8u)] = s;
+  }
+}
+
+// ---- gated activation backward: a = silu(z1) z2, dz1 = da z2 s (1 + z1 (1 - s)), dz2 = da silu(z1), s = sigmoid(z1);
+//      z = [z1 | z2] per row.  dz may alias z and a may alias da (a thread reads its pieces before it writes them). ----
+__global__ __launch_bounds__(256) void swiglu_bwd_kernel(const uint16_t* z, uint32_t ldz, const uint16_t* da,
+                                                         uint32_t ldda, uint16_t* dz, uint32_t lddz, uint16_t* a,
+                                                         uint32_t lda, uint32_t M, uint32_t H) {
+  const size_t gid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const uint32_t cpr = H / 8;
+  const uint32_t row = (uint32_t)(gid / cpr), ch = (uint32_t)(gid % cpr) * 8;
+  if (row >= M) return;
+  const u32x4_t v1 = *reinterpret_cast<const u32x4_t*>(z + (size_t)row * ldz + ch);
+  const u32x4_t v2 = *reinterpret_cast<const u32x4_t*>(z + (size_t)row * ldz + H + ch);
+  const u32x4_t vd = *reinterpret_cast<const u32x4_t*>(da + (size_t)row * ldda + ch);
+  u32x4_t o1, o2, oa;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    float r1[2], r2[2], ra[2];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const float z1 = h ? bf16_hi(v1[e]) : bf16_lo(v1[e]);
+      const float z2 = h ? bf16_hi(v2[e]) : bf16_lo(v2[e]);
+      const float d = h ? bf16_hi(vd[e]) : bf16_lo(vd[e]);
+      const float s = 1.f / (1.f + __expf(-z1));
+      const float sl = z1 * s;
+      ra[h] = sl * z2;
+      r1[h] = d * z2 * s * (1.f + z1 * (1.f - s));
+      r2[h] = d * sl;
+    }
+    o1[e] = pack_bf16x2(r1[0], r1[1]);
+    o2[e] = pack_bf16x2(r2[0], r2[1]);
+    oa[e] = pack_bf16x2(ra[0], ra[1]);
+  }
+  *reinterpret_cast<u32x4_t*>(dz + (size_t)row * lddz + ch) = o1;
+  *reinterpret_cast<u32x4_t*>(dz + (size_t)row * lddz + H + ch) = o2;
+  if (a) *reinterpret_cast<u32x4_t*>(a + (size_t)row * lda + ch) = oa;
+}
+
+// dgamma / dbeta from the per-workgroup partial rows [dgamma | dbeta].  A workgroup owns 16 columns; its 64 row
+// groups each sum every 64th partial row (independent loads, so many are in flight), then one thread per column adds
+// the 64 group sums in ascending order: a fixed summation tree.
+__global__ __launch_bounds__(1024) void ln_bwd_reduce_kernel(const float* __restrict__ part, uint32_t n_part, uint32_t C,
+                                                             float* __restrict__ dgamma, float* __restrict__ dbeta,
+                                                             uint32_t accumulate) {
+  __shared__ float s_red[64][17];
+  const uint32_t tid = threadIdx.x, col = blockIdx.x * 16u + (tid & 15u), rg = tid >> 4;
+  float s = 0.f;
+  if (col < 2u * C)
+    for (uint32_t p = rg; p < n_part; p += 64u) s += part[(size_t)p * 2u * C + col];
+  s_red[rg][tid & 15u] = s;
+  __syncthreads();
+  if (tid < 16u && col < 2u * C) {
+    float* out = col < C ? dgamma + col : dbeta + (col - C);
+    float t = accumulate ? *out : 0.f;
+    for (uint32_t r = 0; r < 64u; ++r) t += s_red[r][tid];
+    *out = t;
+  }
+}
+
+int n_cu_of(int device, uint32_t* n_cu) {
+  int v = 0;
+  F3D_CHECK_HIP(hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, device));
+  *n_cu = v > 0 ? (uint32_t)v : 256u;
+  return F3D_OK;
+}
+
+}  // namespace
+}  // namespace f3d
+
+extern "C" {
+
+int f3d_linear_wgrad_bf16(const f3d_bf16_t* dy, uint32_t lddy, const f3d_bf16_t* x, uint32_t ldx, float* dw, float* db,
+                          uint32_t m, uint32_t n, uint32_t k, uint32_t accumulate, int device, void* stream) {
+  using namespace f3d;
+  F3D_CHECK_ARG(((dy && x) || m == 0) && dw, "null tensor pointer");
+  F3D_CHECK_ARG(n > 0 && k > 0 && n % 8 == 0 && k % 8 == 0, "n=%u and k=%u must be positive multiples of 8", n, k);
+  F3D_CHECK_ARG(lddy >= n && lddy % 8 == 0 && ldx >= k && ldx % 8 == 0,
+                "row strides must be multiples of 8 and cover a row (lddy=%u ldx=%u)", lddy, ldx);
+  F3D_CHECK_ARG((((uintptr_t)dy | (uintptr_t)x) & 15u) == 0, "dy / x must be 16-byte aligned");
+  DeviceGuard guard(device);
+  F3D_CHECK_ARG(guard.ok, "cannot select device %d", device);
+  hipStream_t s = (hipStream_t)stream;
+  SyncBracket sync(s);
+  uint32_t n_cu = 0;
+  if (int rc = n_cu_of(device, &n_cu)) return rc;
+  const uint32_t n_tiles = cdiv_u32(n, kWgNT), k_tiles = cdiv_u32(k, kWgKT), tiles = n_tiles * k_tiles;
+  // one round of the chip: as many row slabs as there are compute units per tile
+  uint32_t slabs = tiles >= n_cu ? 1u : n_cu / tiles;
+  const uint32_t stages = cdiv_u32(m, kWgMT);
+  if (slabs > stages) slabs = stages ? stages : 1u;
+  const uint32_t slab_rows = cdiv_u32(cdiv_u32(m, slabs), kWgMT) * kWgMT;
+  if (m) slabs = cdiv_u32(m, slab_rows);
+  const size_t nk = (size_t)n * k;
+  const size_t part_w_bytes = (size_t)slabs * nk * 4, part_b_bytes = db ? (size_t)slabs * n * 4 : 0;
+  char* ws = (char*)workspace(device, part_w_bytes + part_b_bytes);
+  if (!ws) return F3D_ERR_RUNTIME;
+  float* part_w = (float*)ws;
+  float* part_b = db ? (float*)(ws + part_w_bytes) : nullptr;
+  static bool attr_set[64] = {};
+  if (device >= 0 && device < 64 && !attr_set[device]) {
+    F3D_CHECK_HIP(hipFuncSetAttribute((const void*)linear_wgrad_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, kWgLds));
+    attr_set[device] = true;
+  }
+  const uint32_t n_items = tiles * slabs, items_per_xcd = cdiv_u32(n_items, kXcd);
+  hipLaunchKernelGGL(linear_wgrad_kernel, dim3(items_per_xcd * kXcd), dim3(kWgThreads), kWgLds, s, dy, lddy, x, ldx,
+                     part_w, part_b, m, n, k, n_tiles, k_tiles, slabs, slab_rows, items_per_xcd);
+  hipLaunchKernelGGL(sum_partials_kernel, dim3((uint32_t)((nk + 255) / 256)), dim3(256), 0, s, part_w, slabs, nk, dw,
+                     accumulate);
+  if (db)
+    hipLaunchKernelGGL(sum_partials_kernel, dim3(cdiv_u32(n, 256)), dim3(256), 0, s, part_b, slabs, (size_t)n, db,
+                       accumulate);
+  F3D_CHECK_HIP(hipGetLastError());
+  return F3D_OK;
+}
+
+int f3d_layernorm_bwd_bf16(const f3d_bf16_t* x, uint32_t ldx, const f3d_bf16_t* dh, uint32_t lddh,
+                           const f3d_bf16_t* gamma, const f3d_bf16_t* dres, uint32_t lddr, f3d_bf16_t* dx, uint32_t lddx,
+                           float* dgamma, float* dbeta, uint32_t m, uint32_t c, float eps, uint32_t accumulate,
+                           int device, void* stream) {
+  using namespace f3d;
+  F3D_CHECK_ARG(((x && dh && dx) || m == 0) && gamma && dgamma && dbeta, "null tensor pointer");
+  if (!(c == 32 || c == 64 || c == 128 || c == 256 || c == 512)) {
+    set_error("No kernel found for LayerNorm backward at width %u (supported: 32, 64, 128, 256, 512)", c);
+    return F3D_ERR_UNSUPPORTED;
+  }
+  F3D_CHECK_ARG(ldx >= c && ldx % 8 == 0 && lddh >= c && lddh % 8 == 0 && lddx >= c && lddx % 8 == 0 &&
+                    (!dres || (lddr >= c && lddr % 8 == 0)),
+                "row strides must be multiples of 8 and cover a row");
+  F3D_CHECK_ARG((((uintptr_t)x | (uintptr_t)dh | (uintptr_t)gamma | (uintptr_t)dres | (uintptr_t)dx) & 15u) == 0,
+                "x / dh / gamma / dres / dx must be 16-byte aligned");
+  DeviceGuard guard(device);
+  F3D_CHECK_ARG(guard.ok, "cannot select device %d", device);
+  hipStream_t s = (hipStream_t)stream;
+  SyncBracket sync(s);
+  uint32_t n_cu = 0;
+  if (int rc = n_cu_of(device, &n_cu)) return rc;
+  const uint32_t rpb = 256u / (c / 8u);
+  uint32_t wgs = cdiv_u32(m, rpb);
+  if (wgs > n_cu * 8u) wgs = n_cu * 8u;
+  if (wgs == 0) wgs = 1;
+  float* part = (float*)workspace(device, (size_t)wgs * 2u * c * 4u);
+  if (!part) return F3D_ERR_RUNTIME;
+#define F3D_LNB(LPR)                                                                                                \
+  hipLaunchKernelGGL((layernorm_bwd_kernel<LPR>), dim3(wgs), dim3(256), 0, s, x, ldx, dh, lddh, gamma, dres, lddr, \
+                     dx, lddx, part, m, eps)
+  switch (c) {
+    case 32: F3D_LNB(4); break;
+    case 64: F3D_LNB(8); break;
+    case 128: F3D_LNB(16); break;
+    case 256: F3D_LNB(32); break;
+    default: F3D_LNB(64); break;
+  }
+#undef F3D_LNB
+  hipLaunchKernelGGL(ln_bwd_reduce_kernel, dim3(cdiv_u32(2u * c, 16)), dim3(1024), 0, s, part, wgs, c, dgamma, dbeta,
+                     accumulate);
+  F3D_CHECK_HIP(hipGetLastError());
+  return F3D_OK;
+}
+
+int f3d_swiglu_bwd_bf16(const f3d_bf16_t* z, uint32_t ldz, const f3d_bf16_t* da, uint32_t ldda, f3d_bf16_t* dz,
+                        uint32_t lddz, f3d_bf16_t* a, uint32_t lda, uint32_t m, uint32_t hidden, int device,
+                        void* stream) {
+  using namespace f3d;
+  F3D_CHECK_ARG(z && da && dz, "null tensor pointer");
+  F3D_CHECK_ARG(hidden > 0 && hidden % 8 == 0, "hidden=%u must be a positive multiple of 8", hidden);
+  F3D_CHECK_ARG(ldz >= 2 * hidden && ldz % 8 == 0 && lddz >= 2 * hidden && lddz % 8 == 0 && ldda >= hidden &&
+                    ldda % 8 == 0 && (!a || (lda >= hidden && lda % 8 == 0)),
+                "row strides must be multiples of 8 and cover a row");
+  F3D_CHECK_ARG((((uintptr_t)z | (uintptr_t)da | (uintptr_t)dz | (uintptr_t)a) & 15u) == 0,
+                "z / da / dz / a must be 16-byte aligned");
+  if (m == 0) return F3D_OK;
+  DeviceGuard guard(device);
+  F3D_CHECK_ARG(guard.ok, "cannot select device %d", device);
+  hipStream_t s = (hipStream_t)stream;
+  SyncBracket sync(s);
+  const size_t threads = (size_t)m * (hidden / 8);
+  F3D_CHECK_ARG((threads + 255) / 256 <= 0x7FFFFFFFull, "too many rows");
+  hipLaunchKernelGGL(swiglu_bwd_kernel, dim3((uint32_t)((threads + 255) / 256)), dim3(256), 0, s, z, ldz, da, ldda, dz,
+                     lddz, a, lda, m, hidden);
+  F3D_CHECK_HIP(hipGetLastError());
+  return F3D_OK;
+}
+
+}  // extern "C"

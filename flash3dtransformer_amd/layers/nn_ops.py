@@ -4,9 +4,13 @@ a checkpoint of the reference's torch / TransformerEngine modules loads by name)
 bf16 copies: made anew on every training-mode or gradient-enabled forward, kept between eval-mode forwards
 under no_grad (see _Bf16Cache for when such a copy is dropped).
 
-Forward runs on the HIP kernels.  Backward of these dense layers is not a kernel of this library: as the
-reference leaves it to torch / TransformerEngine, the autograd functions here differentiate a torch restatement
-of the same formula on the GPU (library GEMMs, fp32 accumulation).  The forward value never comes from that
+Forward runs on the HIP kernels.  So does the backward of Linear (optionally with a LayerNorm in front and a
+residual), LayerNorm and the gated LayerNormMLP on bf16 activations: weight / bias gradients from the transposing
+MFMA kernel, input gradients from the forward linear kernels on the transposed weight, LayerNorm and gate backward
+as one pass each (`_LinearGrad`, `_LayerNormGrad`, `_GatedMLPGrad`).  What those kernels do not cover (other
+activations inside a Linear, widths that are not a multiple of 8, LayerNorm widths other than 32 ... 512, fp32
+activations) differentiates a torch restatement of the same formula on the GPU instead (`_TorchBackward`), which
+is where the reference gets all of it (torch / TransformerEngine autograd).  The forward value never comes from a
 restatement.
 """
 import math
@@ -154,6 +158,145 @@ def as_bf16_2d(x: torch.Tensor) -> torch.Tensor:
     return x
 
 
+def _grad_out(g, like):
+    """a gradient tensor in the dtype and shape autograd expects for `like`"""
+    return g.to(like.dtype).reshape(like.shape)
+
+
+def _transposed_bf16(w16: torch.Tensor) -> torch.Tensor:
+    return w16.t().contiguous()
+
+
+def _ln_backward(x2, dh, g16, dres, eps, need_dx=True):
+    """(dx bf16, dgamma fp32, dbeta fp32) of LayerNorm at rows x2 for the output gradient dh (+ dres added to dx)"""
+    c = x2.shape[1]
+    dx = torch.empty(x2.shape, dtype=torch.bfloat16, device=x2.device)
+    dg = torch.empty(c, dtype=torch.float32, device=x2.device)
+    db = torch.empty(c, dtype=torch.float32, device=x2.device)
+    pshattn.layernorm_bwd_bf16(x2, dh, g16, dres, dx, dg, db, eps)
+    return dx, dg, db
+
+
+class _LayerNormGrad(torch.autograd.Function):
+    """y = LayerNorm(x) computed by the HIP forward; gradient by f3d_layernorm_bwd_bf16"""
+
+    @staticmethod
+    def forward(ctx, y, x, weight, bias, eps, g16):
+        ctx.save_for_backward(x, weight, bias, g16)
+        ctx.eps = eps
+        return y.view_as(y)
+
+    @staticmethod
+    def backward(ctx, dy):
+        x, weight, bias, g16 = ctx.saved_tensors
+        dx, dg, db = _ln_backward(as_bf16_2d(x), as_bf16_2d(dy.reshape(x.shape)), g16, None, ctx.eps)
+        return (None, _grad_out(dx, x) if ctx.needs_input_grad[1] else None,
+                _grad_out(dg, weight) if ctx.needs_input_grad[2] else None,
+                _grad_out(db, bias) if bias is not None and ctx.needs_input_grad[3] else None, None, None)
+
+
+class _LinearGrad(torch.autograd.Function):
+    """y = [LayerNorm](x) @ w.T + b (+ residual) computed by the HIP forward; gradient by the HIP backward kernels:
+    dw, db = f3d_linear_wgrad_bf16(dy, h), dh = f3d_linear_bf16(dy, w.T), then LayerNorm backward if there is one"""
+
+    @staticmethod
+    def forward(ctx, y, x, weight, bias, residual, ln_w, ln_b, eps, w16, g16, b16):
+        ctx.save_for_backward(x, weight, bias, residual, ln_w, ln_b, w16, g16, b16)
+        ctx.eps = eps
+        return y.view_as(y)
+
+    @staticmethod
+    def backward(ctx, dy):
+        x, weight, bias, residual, ln_w, ln_b, w16, g16, b16 = ctx.saved_tensors
+        need = ctx.needs_input_grad
+        dy2 = as_bf16_2d(dy)
+        x2 = as_bf16_2d(x)
+        m, k = x2.shape
+        n = dy2.shape[1]
+        dev = x2.device
+        if ln_w is not None:
+            h = torch.empty(m, k, dtype=torch.bfloat16, device=dev)
+            pshattn.layernorm_bf16(x2.contiguous(), g16, b16, h, ctx.eps)
+        else:
+            h = x2
+        dw = db = dx = dg = dbeta = None
+        if need[2] or (bias is not None and need[3]):
+            dw = torch.empty(n, k, dtype=torch.float32, device=dev)
+            db = torch.empty(n, dtype=torch.float32, device=dev) if bias is not None else None
+            pshattn.linear_wgrad_bf16(dy2, h, dw, db)
+        if need[1] or (ln_w is not None and (need[5] or need[6])):
+            dh = torch.empty(m, k, dtype=torch.bfloat16, device=dev)
+            pshattn.linear_bf16(dy2, _transposed_bf16(w16), None, None, dh, None)
+            if ln_w is not None:
+                dx, dg, dbeta = _ln_backward(x2, dh, g16, None, ctx.eps)
+            else:
+                dx = dh
+        return (None, _grad_out(dx, x) if need[1] else None, _grad_out(dw, weight) if need[2] else None,
+                _grad_out(db, bias) if bias is not None and need[3] else None,
+                _grad_out(dy2, residual) if residual is not None and need[4] else None,
+                _grad_out(dg, ln_w) if ln_w is not None and need[5] else None,
+                _grad_out(dbeta, ln_b) if ln_b is not None and need[6] else None, None, None, None, None)
+
+
+class _GatedMLPGrad(torch.autograd.Function):
+    """y = fc2(silu(z1) * z2) + b2 (+ residual), [z1 | z2] = LayerNorm(x) @ w1.T + b1, computed by the HIP forward.
+    The backward recomputes LayerNorm(x) and z (the forward keeps neither), then runs
+    da = dy @ w2, (dz, a) = gate backward in place, dw2 = dy.T a, dw1 = dz.T h, dh = dz @ w1, LayerNorm backward.
+    When the residual is the layer's own input, its gradient dy is added to dx inside the LayerNorm backward."""
+
+    @staticmethod
+    def forward(ctx, y, x, residual, ln_w, ln_b, w1, b1, w2, b2, eps, g16, be16, w1_16, b1_16, w2_16):
+        ctx.save_for_backward(x, residual, ln_w, ln_b, w1, b1, w2, b2, g16, be16, w1_16, b1_16, w2_16)
+        ctx.eps = eps
+        return y.view_as(y)
+
+    @staticmethod
+    def backward(ctx, dy):
+        x, residual, ln_w, ln_b, w1, b1, w2, b2, g16, be16, w1_16, b1_16, w2_16 = ctx.saved_tensors
+        need = ctx.needs_input_grad
+        dy2 = as_bf16_2d(dy)
+        x2 = as_bf16_2d(x).contiguous()
+        m, c = x2.shape
+        hid = w2_16.shape[1]
+        dev = x2.device
+        bf = dict(dtype=torch.bfloat16, device=dev)
+        f32 = dict(dtype=torch.float32, device=dev)
+        h = torch.empty(m, c, **bf)
+        pshattn.layernorm_bf16(x2, g16, be16, h, ctx.eps)
+        z = torch.empty(m, 2 * hid, **bf)
+        pshattn.linear_bf16(h, w1_16, b1_16, None, z, None)
+        da = torch.empty(m, hid, **bf)
+        pshattn.linear_bf16(dy2, _transposed_bf16(w2_16), None, None, da, None)
+        pshattn.swiglu_bwd_bf16(z, da, z, da)          # z <- dz, da <- a
+        dz, a = z, da
+        dw2, db2 = torch.empty(c, hid, **f32), torch.empty(c, **f32)
+        pshattn.linear_wgrad_bf16(dy2, a, dw2, db2)
+        dw1, db1 = torch.empty(2 * hid, c, **f32), torch.empty(2 * hid, **f32)
+        pshattn.linear_wgrad_bf16(dz, h, dw1, db1)
+        pshattn.linear_bf16(dz, _transposed_bf16(w1_16), None, None, h, None)     # h <- dh
+        # a residual that is the input itself: one gradient tensor for both routes
+        shared = (residual is not None and need[1] and need[2] and residual.data_ptr() == x.data_ptr()
+                  and residual.shape == x.shape and residual.dtype == x.dtype and residual.stride() == x.stride())
+        dx, dg, dbeta = _ln_backward(x2, h, g16, dy2 if shared else None, ctx.eps)
+        d_res = None
+        if residual is not None and need[2] and not shared:
+            d_res = _grad_out(dy2, residual)
+        return (None, _grad_out(dx, x) if need[1] else None, d_res,
+                _grad_out(dg, ln_w) if need[3] else None, _grad_out(dbeta, ln_b) if ln_b is not None and need[4] else None,
+                _grad_out(dw1, w1) if need[5] else None, _grad_out(db1, b1) if b1 is not None and need[6] else None,
+                _grad_out(dw2, w2) if need[7] else None, _grad_out(db2, b2) if b2 is not None and need[8] else None,
+                None, None, None, None, None, None)
+
+
+def _grad_wanted(*tensors) -> bool:
+    return torch.is_grad_enabled() and any(isinstance(t, torch.Tensor) and t.requires_grad for t in tensors)
+
+
+def _hip_backward_covers(x: torch.Tensor, *widths) -> bool:
+    """bf16 activations on the GPU and widths the backward kernels take"""
+    return x.is_cuda and x.dtype == torch.bfloat16 and all(w % 8 == 0 for w in widths)
+
+
 class Linear(_CachedParamModule):
     """y = act(x W^T + b) (+ residual) on MFMA; parameter names match torch.nn.Linear / te.Linear"""
 
@@ -179,16 +322,25 @@ class Linear(_CachedParamModule):
         n_out = self.out_features // 2 if act == "swiglu" else self.out_features
         y = out if out is not None else torch.empty(x2.shape[0], n_out, dtype=torch.bfloat16, device=x.device)
         r2 = None if residual is None else as_bf16_2d(residual.reshape(-1, n_out))
+        w16, b16 = self._w.get(self.weight, self.training), self._b.get(self.bias, self.training)
+        g = b = None
         if pre_norm is not None:
             g, b = norm_params_bf16(pre_norm)
-            pshattn.ln_linear_bf16(x2, g, b, pre_norm.eps, self._w.get(self.weight, self.training), self._b.get(self.bias, self.training), r2, y, act)
+            pshattn.ln_linear_bf16(x2, g, b, pre_norm.eps, w16, b16, r2, y, act)
         else:
-            pshattn.linear_bf16(x2, self._w.get(self.weight, self.training), self._b.get(self.bias, self.training), r2, y, act)
+            pshattn.linear_bf16(x2, w16, b16, r2, y, act)
         ln_w = None if pre_norm is None else pre_norm.weight
         ln_b = None if pre_norm is None else pre_norm.bias
         eps = 0.0 if pre_norm is None else pre_norm.eps
+        x_in = x.reshape(-1, x.shape[-1])
         res_in = None if residual is None else residual.reshape(-1, n_out)
-        out = torch_backward(y, _linear_ref(act, eps), x.reshape(-1, x.shape[-1]), self.weight, self.bias, res_in, ln_w, ln_b)
+        if not _grad_wanted(x_in, self.weight, self.bias, res_in, ln_w, ln_b):
+            return y.view(*lead, n_out)
+        if act is None and _hip_backward_covers(x_in, self.in_features, self.out_features) and (
+                pre_norm is None or (self.in_features in pshattn.LN_BWD_WIDTHS and g is not None)):
+            out = _LinearGrad.apply(y, x_in, self.weight, self.bias, res_in, ln_w, ln_b, eps, w16, g, b)
+        else:
+            out = torch_backward(y, _linear_ref(act, eps), x_in, self.weight, self.bias, res_in, ln_w, ln_b)
         return out.view(*lead, n_out)
 
     def extra_repr(self):
@@ -208,10 +360,15 @@ class LayerNorm(_CachedParamModule):
     def forward(self, x: torch.Tensor):
         x2 = as_bf16_2d(x.reshape(-1, x.shape[-1])).contiguous()
         y = torch.empty_like(x2)
-        pshattn.layernorm_bf16(x2, self._w.get(self.weight, self.training), self._b.get(self.bias, self.training), y, self.eps)
+        g16 = self._w.get(self.weight, self.training)
+        pshattn.layernorm_bf16(x2, g16, self._b.get(self.bias, self.training), y, self.eps)
+        x_in = x.reshape(-1, x.shape[-1])
+        if _grad_wanted(x_in, self.weight, self.bias) and _hip_backward_covers(x_in) \
+                and self.normalized_shape in pshattn.LN_BWD_WIDTHS:
+            return _LayerNormGrad.apply(y, x_in, self.weight, self.bias, self.eps, g16).view(x.shape)
         eps = self.eps
         ref = lambda xx, w, b: torch.nn.functional.layer_norm(xx, (xx.shape[-1],), w, b, eps)
-        return torch_backward(y, ref, x.reshape(-1, x.shape[-1]), self.weight, self.bias).view(x.shape)
+        return torch_backward(y, ref, x_in, self.weight, self.bias).view(x.shape)
 
 
 FUSABLE_LN_WIDTHS = (32, 64, 128, 256, 512)
@@ -244,7 +401,12 @@ def apply_norm(norm: nn.Module, x: torch.Tensor) -> torch.Tensor:
         x2 = as_bf16_2d(x.reshape(-1, x.shape[-1])).contiguous()
         y = torch.empty_like(x2)
         b = None if norm.bias is None else norm.bias.detach().to(torch.bfloat16)
-        pshattn.layernorm_bf16(x2, norm.weight.detach().to(torch.bfloat16), b, y, norm.eps)
+        g16 = norm.weight.detach().to(torch.bfloat16)
+        pshattn.layernorm_bf16(x2, g16, b, y, norm.eps)
+        x_in = x.reshape(-1, x.shape[-1])
+        if _grad_wanted(x_in, norm.weight, norm.bias) and _hip_backward_covers(x_in) \
+                and x.shape[-1] in pshattn.LN_BWD_WIDTHS:
+            return _LayerNormGrad.apply(y, x_in, norm.weight, norm.bias, norm.eps, g16).view(x.shape)
         eps = norm.eps
         ref = lambda xx, w, bb: torch.nn.functional.layer_norm(xx, (xx.shape[-1],), w, bb, eps)
         return torch_backward(y, ref, x.reshape(-1, x.shape[-1]), norm.weight, norm.bias).view(x.shape)
@@ -319,34 +481,38 @@ class LayerNormMLP(_CachedParamModule):
 
     def forward(self, x: torch.Tensor, residual: torch.Tensor = None):
         x2 = as_bf16_2d(x.reshape(-1, self.hidden_size)).contiguous()
-        c = self._c
+        params = (self.layer_norm_weight, self.layer_norm_bias, self.fc1_weight, self.fc1_bias, self.fc2_weight, self.fc2_bias)
+        g16, be16, w1_16, b1_16, w2_16, b2_16 = (c.get(p, self.training) for c, p in zip(self._c, params))
         r2 = None if residual is None else as_bf16_2d(residual.reshape(-1, self.hidden_size))
         y = torch.empty_like(x2)
         # on request, the whole gated MLP in one kernel where one exists (hidden activations stay in registers) ...
         want_fused = self.fused if self.fused is not None else (self.hidden_size <= 128 or x2.shape[0] >= 30000)
         fused = (want_fused and self.activation == "swiglu" and self.hidden_size in FUSED_MLP_WIDTHS
                  and self.ffn_hidden_size % 32 == 0
-                 and pshattn.ln_mlp_swiglu_bf16(x2, c[0].get(self.layer_norm_weight, self.training), c[1].get(self.layer_norm_bias, self.training),
-                                                self.eps, c[2].get(self.fc1_weight, self.training), c[3].get(self.fc1_bias, self.training),
-                                                c[4].get(self.fc2_weight, self.training), c[5].get(self.fc2_bias, self.training), r2, y))
+                 and pshattn.ln_mlp_swiglu_bf16(x2, g16, be16, self.eps, w1_16, b1_16, w2_16, b2_16, r2, y))
         if not fused:
             # ... otherwise LayerNorm + fc1 + activation, then fc2 + residual
             h = torch.empty(x2.shape[0], self.ffn_hidden_size, dtype=torch.bfloat16, device=x.device)
             if self.hidden_size in FUSABLE_LN_WIDTHS:
-                pshattn.ln_linear_bf16(x2, c[0].get(self.layer_norm_weight, self.training), c[1].get(self.layer_norm_bias, self.training), self.eps,
-                                       c[2].get(self.fc1_weight, self.training), c[3].get(self.fc1_bias, self.training), None, h, self.activation)
+                pshattn.ln_linear_bf16(x2, g16, be16, self.eps, w1_16, b1_16, None, h, self.activation)
             else:
                 ln = torch.empty_like(x2)
-                pshattn.layernorm_bf16(x2, c[0].get(self.layer_norm_weight, self.training), c[1].get(self.layer_norm_bias, self.training), ln, self.eps)
-                pshattn.linear_bf16(ln, c[2].get(self.fc1_weight, self.training), c[3].get(self.fc1_bias, self.training), None, h, self.activation)
-            pshattn.linear_bf16(h, c[4].get(self.fc2_weight, self.training), c[5].get(self.fc2_bias, self.training), r2, y, None)
+                pshattn.layernorm_bf16(x2, g16, be16, ln, self.eps)
+                pshattn.linear_bf16(ln, w1_16, b1_16, None, h, self.activation)
+            pshattn.linear_bf16(h, w2_16, b2_16, r2, y, None)
+        x_in = x.reshape(-1, self.hidden_size)
+        res_in = None if residual is None else residual.reshape(-1, self.hidden_size)
+        if not _grad_wanted(x_in, res_in, *params):
+            return y.view(x.shape)
+        if self.activation == "swiglu" and self.hidden_size in pshattn.LN_BWD_WIDTHS \
+                and _hip_backward_covers(x_in, self.ffn_hidden_size) and (res_in is None or res_in.dtype == torch.bfloat16):
+            out = _GatedMLPGrad.apply(y, x_in, res_in, *params, self.eps, g16, be16, w1_16, b1_16, w2_16)
+            return out.view(x.shape)
         act, eps = self.activation, self.eps
 
         def ref(xx, res, ln_w, ln_b, w1, b1, w2, b2):
             hh = torch.nn.functional.layer_norm(xx, (xx.shape[-1],), ln_w, ln_b, eps)
             out = torch.nn.functional.linear(_act_ref(torch.nn.functional.linear(hh, w1, b1), act), w2, b2)
             return out if res is None else out + res
-        res_in = None if residual is None else residual.reshape(-1, self.hidden_size)
-        out = torch_backward(y, ref, x.reshape(-1, self.hidden_size), res_in, self.layer_norm_weight, self.layer_norm_bias,
-                             self.fc1_weight, self.fc1_bias, self.fc2_weight, self.fc2_bias)
+        out = torch_backward(y, ref, x_in, res_in, *params)
         return out.view(x.shape)

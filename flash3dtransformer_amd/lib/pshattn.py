@@ -562,6 +562,68 @@ def layernorm_bf16(x, gamma, beta, y, eps=1e-5):
                                       _i32(dev), _stream(dev)))
 
 
+def _rows2d(ts, dtype=torch.bfloat16):
+    for t in ts:
+        if t.dim() != 2 or t.stride(1) != 1:
+            raise RuntimeError("expected 2-D row-major tensors")
+    assert_dtype(ts, dtype)
+
+
+def linear_wgrad_bf16(dy, x, dw, db=None, accumulate=False):
+    """extension: dw[n,k] (+)= dy.T @ x, db[n] (+)= dy.sum(0), fp32 outputs (gradient of y = x @ w.T + b)"""
+    dev = assert_same_device([dy, x, dw])
+    _rows2d([dy, x])
+    assert_dtype([dw], torch.float32)
+    assert_contiguous([dw])
+    m, n = dy.shape
+    k = x.shape[1]
+    if x.shape[0] != m or tuple(dw.shape) != (n, k):
+        raise RuntimeError(f"wgrad shape mismatch: dy{tuple(dy.shape)} x{tuple(x.shape)} dw{tuple(dw.shape)}")
+    if db is not None:
+        _check_vectors(dy, [db], torch.float32)
+        if tuple(db.shape) != (n,):
+            raise RuntimeError("db must be [n]")
+    _check(_load().f3d_linear_wgrad_bf16(_ptr(dy), _u32(dy.stride(0)), _ptr(x), _u32(x.stride(0)), _ptr(dw), _ptr(db),
+                                         _u32(m), _u32(n), _u32(k), _u32(1 if accumulate else 0), _i32(dev),
+                                         _stream(dev)))
+
+
+LN_BWD_WIDTHS = (32, 64, 128, 256, 512)
+
+
+def layernorm_bwd_bf16(x, dh, gamma, dres, dx, dgamma, dbeta, eps=1e-5, accumulate=False):
+    """extension: LayerNorm backward (dx, dgamma, dbeta) with an optional extra gradient `dres` added to dx"""
+    dev = assert_same_device([x, dh, gamma, dx, dgamma, dbeta])
+    _rows2d([x, dh, dx] + ([dres] if dres is not None else []))
+    _check_vectors(x, [gamma])
+    _check_vectors(x, [dgamma, dbeta], torch.float32)
+    m, c = x.shape
+    for t in (dh, dx, dres):
+        if t is not None and tuple(t.shape) != (m, c):
+            raise RuntimeError("layernorm_bwd: x, dh, dx, dres must share one shape")
+    if tuple(gamma.shape) != (c,) or tuple(dgamma.shape) != (c,) or tuple(dbeta.shape) != (c,):
+        raise RuntimeError("layernorm_bwd: gamma, dgamma, dbeta must be [c]")
+    rc = _load().f3d_layernorm_bwd_bf16(_ptr(x), _u32(x.stride(0)), _ptr(dh), _u32(dh.stride(0)), _ptr(gamma),
+                                        _ptr(dres), _u32(dres.stride(0) if dres is not None else 0), _ptr(dx),
+                                        _u32(dx.stride(0)), _ptr(dgamma), _ptr(dbeta), _u32(m), _u32(c), _f32(eps),
+                                        _u32(1 if accumulate else 0), _i32(dev), _stream(dev))
+    if rc == 2:
+        raise NotImplementedError(_load().f3d_last_error().decode("utf-8", "replace"))
+    _check(rc)
+
+
+def swiglu_bwd_bf16(z, da, dz, a=None):
+    """extension: backward of a = silu(z[:, :h]) * z[:, h:]; dz may be z itself and a may be da itself"""
+    dev = assert_same_device([z, da, dz])
+    _rows2d([z, da, dz] + ([a] if a is not None else []))
+    m, h = da.shape
+    if tuple(z.shape) != (m, 2 * h) or tuple(dz.shape) != (m, 2 * h) or (a is not None and tuple(a.shape) != (m, h)):
+        raise RuntimeError("swiglu_bwd shape mismatch")
+    _check(_load().f3d_swiglu_bwd_bf16(_ptr(z), _u32(z.stride(0)), _ptr(da), _u32(da.stride(0)), _ptr(dz),
+                                       _u32(dz.stride(0)), _ptr(a), _u32(a.stride(0) if a is not None else 0),
+                                       _u32(m), _u32(h), _i32(dev), _stream(dev)))
+
+
 def coord_embed_bf16(coord, w, bias, y):
     """extension: y = bf16(coord) @ w.T + bias for w [C,3] (PSH3DCoordEmbedding, psh_ops.py:64-67)"""
     assert_contiguous([coord, w, y])

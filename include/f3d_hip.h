@@ -291,6 +291,37 @@ int f3d_coord_embed_bf16(const f3d_half_t* coord, const f3d_bf16_t* w, const f3d
 int f3d_affine_act_bf16(const f3d_bf16_t* x, const float* scale, const float* shift, f3d_bf16_t* y, uint32_t m,
                         uint32_t c, uint32_t act, int device, void* stream);
 
+/* ---- backward of the dense layers ---------------------------------------------------------------
+ * The reference takes these from torch / TransformerEngine autograd (flash3dxfmr/layers/buck_swin.py:159-163,
+ * elem_wise.py:22-26, stage.py:94-99: nn.Linear, te.LayerNormMLP, the norms); the input gradient of a linear layer is
+ * f3d_linear_bf16 with the transposed weight (dx = dy · w).
+ *
+ * Weight and bias gradient of y = x · wᵀ + b:  dw[n,k] = sum_m dy[m,n] x[m,k],  db[n] = sum_m dy[m,n].
+ * dy [m,n] bf16 (row stride lddy), x [m,k] bf16 (row stride ldx), dw [n,k] fp32, db [n] fp32 or NULL; n % 8 == 0,
+ * k % 8 == 0; fp32 accumulation in a fixed order (bit-reproducible).  accumulate != 0 adds to dw / db.  Uses the
+ * per-device workspace like f3d_ln_linear_bf16. */
+int f3d_linear_wgrad_bf16(const f3d_bf16_t* dy, uint32_t lddy, const f3d_bf16_t* x, uint32_t ldx, float* dw, float* db,
+                          uint32_t m, uint32_t n, uint32_t k, uint32_t accumulate, int device, void* stream);
+
+/* LayerNorm backward: with xhat = (x - mean) rstd and g = dh * gamma,
+ *   dx = rstd (g - mean(g) - xhat mean(g xhat)) (+ dres),  dgamma = sum_rows dh xhat,  dbeta = sum_rows dh.
+ * x, dh, dx [m,c] bf16 (row strides ldx, lddh, lddx), gamma [c] bf16, dres [m,c] bf16 or NULL (a gradient that
+ * reaches x by another route, e.g. the residual connection; row stride lddr), dgamma, dbeta [c] fp32 (accumulate != 0
+ * adds to them).  c in {32, 64, 128, 256, 512}, else F3D_ERR_UNSUPPORTED.  dx may alias dh or dres.  Uses the
+ * per-device workspace. */
+int f3d_layernorm_bwd_bf16(const f3d_bf16_t* x, uint32_t ldx, const f3d_bf16_t* dh, uint32_t lddh,
+                           const f3d_bf16_t* gamma, const f3d_bf16_t* dres, uint32_t lddr, f3d_bf16_t* dx, uint32_t lddx,
+                           float* dgamma, float* dbeta, uint32_t m, uint32_t c, float eps, uint32_t accumulate,
+                           int device, void* stream);
+
+/* Backward of the gated activation a = silu(z[:, :h]) * z[:, h:] (F3D_ACT_SWIGLU):
+ *   dz[:, :h] = da * z2 * s (1 + z1 (1 - s)),  dz[:, h:] = da * silu(z1),  s = sigmoid(z1).
+ * z, dz [m,2h] bf16, da [m,h] bf16, a [m,h] bf16 or NULL (the recomputed activation, which the weight gradient of
+ * the following layer needs).  dz may alias z and a may alias da. */
+int f3d_swiglu_bwd_bf16(const f3d_bf16_t* z, uint32_t ldz, const f3d_bf16_t* da, uint32_t ldda, f3d_bf16_t* dz,
+                        uint32_t lddz, f3d_bf16_t* a, uint32_t lda, uint32_t m, uint32_t hidden, int device,
+                        void* stream);
+
 #ifdef __cplusplus
 }
 #endif
