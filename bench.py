@@ -87,7 +87,8 @@ def main():
     ap.add_argument("--no-sub-metrics", action="store_true")
     ap.add_argument("--sub-metrics-only", nargs="*", default=None, metavar="GROUP",
                     help="run only the per-kernel sub-metrics (configs 1, 2, 3, 5) and print them; for profiling those "
-                         "kernels.  Optional group names restrict the run: attention, psh, permute, pool, hourglass, mfma")
+                         "kernels.  Optional group names restrict the run: attention, psh, permute, pool, hourglass, mfma, "
+                         "backward")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU; the path shards by cloud without any exchange between GPUs (each cloud "
@@ -249,7 +250,8 @@ def sub_metrics(dev, only=None):
     unpooling GB/s on config 3 — each against its roofline.  `only`: a set of group names, or None for all"""
     out = {}
     groups = {"attention": sub_attention, "psh": sub_psh, "permute": sub_permute, "pool": sub_pool,
-              "hourglass": lambda d, o: o.__setitem__("hourglass_c5", hourglass_c5(d)), "mfma": sub_mfma_rate}
+              "hourglass": lambda d, o: o.__setitem__("hourglass_c5", hourglass_c5(d)), "mfma": sub_mfma_rate,
+              "backward": sub_backward}
     for name, fn in groups.items():
         if only is None or name in only:
             fn(dev, out)
@@ -268,6 +270,55 @@ def sub_mfma_rate(dev, out):
         ms = ev_time(lambda: pshattn.probe_mfma_bf16(wgs, iters, ra, rb, sink), 3, warmup=1)
         out["mfma_bf16_dense_rate_" + name] = {"ms": round(ms, 3), "tflops": round(flop / ms / 1e9, 1),
                                                "frac_of_bf16_mfma_peak": round(flop / ms / 1e9 / MFMA_BF16_PEAK_TFLOPS, 4)}
+
+
+def sub_backward(dev, out):
+    """backward of the dense layers at the headline workload's shapes (480,000 rows, C = 256, hidden 1024): the weight
+    gradient GEMMs (2 M N K flops against the MFMA roof, M (N + K) 2 bytes against the HBM roof: the two are close for
+    these shapes), LayerNorm and gate backward (one pass each, against the HBM roof), and forward + backward of the
+    three dense layers of a block through the layer API"""
+    from flash3dtransformer_amd.lib import pshattn
+    from flash3dtransformer_amd import layers as L
+    M, C, HID = 480_000, 256, 1024
+    gg = torch.Generator().manual_seed(1007)
+    rnd = lambda *shape: torch.randn(*shape, generator=gg).to(torch.bfloat16).to(dev)
+    for name, n, k in (("qkv", 3 * C, C), ("proj", C, C), ("fc1", 2 * HID, C), ("fc2", C, HID)):
+        dy, x = rnd(M, n), rnd(M, k)
+        dw, db = torch.empty(n, k, device=dev), torch.empty(n, device=dev)
+        ms = ev_time(lambda: pshattn.linear_wgrad_bf16(dy, x, dw, db), 10)
+        tf, gbs = 2.0 * M * n * k / ms / 1e9, M * (n + k) * 2.0 / ms / 1e6
+        out[f"wgrad_{name}_{n}x{k}"] = {"ms": round(ms, 4), "tflops": round(tf, 1), "frac_of_bf16_mfma_peak": round(tf / MFMA_BF16_PEAK_TFLOPS, 4),
+                                        "gbs": round(gbs, 1), "frac_of_hbm_peak": round(gbs / HBM_PEAK_GBS, 4)}
+        del dy, x
+    x, dh = rnd(M, C), rnd(M, C)
+    g16, dx = torch.ones(C, dtype=torch.bfloat16, device=dev), torch.empty(M, C, dtype=torch.bfloat16, device=dev)
+    dg, dbeta = torch.empty(C, device=dev), torch.empty(C, device=dev)
+    ms = ev_time(lambda: pshattn.layernorm_bwd_bf16(x, dh, g16, None, dx, dg, dbeta), 10)
+    gbs = M * C * 6.0 / ms / 1e6
+    out["layernorm_bwd_256"] = {"ms": round(ms, 4), "gbs": round(gbs, 1), "frac_of_hbm_peak": round(gbs / HBM_PEAK_GBS, 4)}
+    del x, dh, dx
+    z, da = rnd(M, 2 * HID), rnd(M, HID)
+    ms = ev_time(lambda: pshattn.swiglu_bwd_bf16(z, da, z, da), 10)
+    gbs = M * HID * 12.0 / ms / 1e6
+    out["swiglu_bwd_1024"] = {"ms": round(ms, 4), "gbs": round(gbs, 1), "frac_of_hbm_peak": round(gbs / HBM_PEAK_GBS, 4)}
+    del z, da
+    torch.manual_seed(1007)
+    ln = L.LayerNorm(C).to(dev)
+    qkv, proj, mlp = L.Linear(C, 3 * C).to(dev), L.Linear(C, C).to(dev), L.LayerNormMLP(C, HID).to(dev)
+    for name, f in (("ln_qkv", lambda t: qkv(t, pre_norm=ln)), ("proj_residual", lambda t: proj(t, residual=t)),
+                    ("ln_mlp_residual", lambda t: mlp(t, residual=t))):
+        xin = rnd(M, C).requires_grad_(True)
+        gy = torch.randn_like(f(xin))
+
+        def step():
+            f(xin).backward(gy)
+
+        def fwd():
+            with torch.no_grad():
+                f(xin)
+        out[f"layer_fwd_bwd_{name}"] = {"fwd_ms": round(ev_time(fwd, 5), 4), "fwd_bwd_ms": round(ev_time(step, 5), 4)}
+        del xin, gy
+    torch.cuda.empty_cache()
 
 
 def sub_attention(dev, out):

@@ -128,21 +128,26 @@ __global__ __launch_bounds__(kWgThreads) void linear_wgrad_kernel(
     const char* buf = lds_wg + (st & 1u) * kWgBuf;
     const bool more = st + 1 < n_stage;
     if (more) fetch(m_begin + (st + 1) * kWgMT);
-#pragma unroll
-    for (int ks = 0; ks < kWgMT / 16; ++ks) {
-      bf16x8_t fa[2], fb[4];
+    // operands of k-step ks + 1 are requested before the products of k-step ks are issued
+    bf16x8_t fa[2][2], fb[2][4];
+    auto frags = [&](int ks, bf16x8_t (&a)[2], bf16x8_t (&b)[4]) {
 #pragma unroll
       for (int i = 0; i < 2; ++i)
-        if ((uint32_t)i < ni) fa[i] = read_tr8(buf + a_off + ks * 16 * kPitchA + i * 64, kPitchA);
+        if ((uint32_t)i < ni) a[i] = read_tr8(buf + a_off + ks * 16 * kPitchA + i * 64, kPitchA);
 #pragma unroll
       for (int j = 0; j < 4; ++j)
-        if ((uint32_t)j < nj) fb[j] = read_tr8(buf + b_off + ks * 16 * kPitchB + j * 64, kPitchB);
+        if ((uint32_t)j < nj) b[j] = read_tr8(buf + b_off + ks * 16 * kPitchB + j * 64, kPitchB);
+    };
+    frags(0, fa[0], fb[0]);
+#pragma unroll
+    for (int ks = 0; ks < kWgMT / 16; ++ks) {
+      if (ks + 1 < kWgMT / 16) frags(ks + 1, fa[(ks + 1) & 1], fb[(ks + 1) & 1]);
 #pragma unroll
       for (int i = 0; i < 2; ++i)
 #pragma unroll
         for (int j = 0; j < 4; ++j)
           if ((uint32_t)i < ni && (uint32_t)j < nj)
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[j], acc[i][j], 0, 0, 0);
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[ks & 1][i], fb[ks & 1][j], acc[i][j], 0, 0, 0);
     }
     if (more) stash(lds_wg + ((st + 1) & 1u) * kWgBuf);
     __syncthreads();
@@ -179,14 +184,31 @@ __global__ __launch_bounds__(kWgThreads) void linear_wgrad_kernel(
   }
 }
 
-// out[i] = (accumulate ? out[i] : 0) + sum over p of part[p][i], p ascending
-__global__ __launch_bounds__(256) void sum_partials_kernel(const float* __restrict__ part, uint32_t n_part, size_t len,
-                                                           float* __restrict__ out, uint32_t accumulate) {
-  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= len) return;
-  float s = accumulate ? out[i] : 0.f;
-  for (uint32_t p = 0; p < n_part; ++p) s += part[(size_t)p * len + i];
-  out[i] = s;
+// out[i] = (accumulate ? out[i] : 0) + sum over p of part[p][i].  A workgroup owns 256 consecutive elements (64 lanes x
+// 4 floats, len % 4 == 0); its 16 partial groups each sum every 16th partial (independent 16-byte loads), then the
+// first group adds the 16 group sums in ascending order: a fixed summation tree.
+__global__ __launch_bounds__(1024) void sum_partials_kernel(const float* __restrict__ part, uint32_t n_part, size_t len,
+                                                            float* __restrict__ out, uint32_t accumulate) {
+  __shared__ float4 s_sum[16][64];
+  const uint32_t tid = threadIdx.x, l = tid & 63u, g = tid >> 6;
+  const size_t i = ((size_t)blockIdx.x * 64u + l) * 4u;
+  float4 s = {0.f, 0.f, 0.f, 0.f};
+  if (i < len)
+    for (uint32_t p = g; p < n_part; p += 16u) {
+      const float4 v = *reinterpret_cast<const float4*>(part + (size_t)p * len + i);
+      s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
+    }
+  s_sum[g][l] = s;
+  __syncthreads();
+  if (g == 0 && i < len) {
+    float4 t = {0.f, 0.f, 0.f, 0.f};
+    if (accumulate) t = *reinterpret_cast<const float4*>(out + i);
+    for (int r = 0; r < 16; ++r) {
+      const float4 v = s_sum[r][l];
+      t.x += v.x; t.y += v.y; t.z += v.z; t.w += v.w;
+    }
+    *reinterpret_cast<float4*>(out + i) = t;
+  }
 }
 
 // ---- LayerNorm backward: LPR lanes per row, 8 channels per lane.
@@ -353,7 +375,8 @@ int f3d_linear_wgrad_bf16(const f3d_bf16_t* dy, uint32_t lddy, const f3d_bf16_t*
   F3D_CHECK_ARG(n > 0 && k > 0 && n % 8 == 0 && k % 8 == 0, "n=%u and k=%u must be positive multiples of 8", n, k);
   F3D_CHECK_ARG(lddy >= n && lddy % 8 == 0 && ldx >= k && ldx % 8 == 0,
                 "row strides must be multiples of 8 and cover a row (lddy=%u ldx=%u)", lddy, ldx);
-  F3D_CHECK_ARG((((uintptr_t)dy | (uintptr_t)x) & 15u) == 0, "dy / x must be 16-byte aligned");
+  F3D_CHECK_ARG((((uintptr_t)dy | (uintptr_t)x | (uintptr_t)dw | (uintptr_t)db) & 15u) == 0,
+                "dy / x / dw / db must be 16-byte aligned");
   DeviceGuard guard(device);
   F3D_CHECK_ARG(guard.ok, "cannot select device %d", device);
   hipStream_t s = (hipStream_t)stream;
@@ -381,10 +404,10 @@ int f3d_linear_wgrad_bf16(const f3d_bf16_t* dy, uint32_t lddy, const f3d_bf16_t*
   const uint32_t n_items = tiles * slabs, items_per_xcd = cdiv_u32(n_items, kXcd);
   hipLaunchKernelGGL(linear_wgrad_kernel, dim3(items_per_xcd * kXcd), dim3(kWgThreads), kWgLds, s, dy, lddy, x, ldx,
                      part_w, part_b, m, n, k, n_tiles, k_tiles, slabs, slab_rows, items_per_xcd);
-  hipLaunchKernelGGL(sum_partials_kernel, dim3((uint32_t)((nk + 255) / 256)), dim3(256), 0, s, part_w, slabs, nk, dw,
+  hipLaunchKernelGGL(sum_partials_kernel, dim3((uint32_t)((nk + 255) / 256)), dim3(1024), 0, s, part_w, slabs, nk, dw,
                      accumulate);
   if (db)
-    hipLaunchKernelGGL(sum_partials_kernel, dim3(cdiv_u32(n, 256)), dim3(256), 0, s, part_b, slabs, (size_t)n, db,
+    hipLaunchKernelGGL(sum_partials_kernel, dim3(cdiv_u32(n, 256)), dim3(1024), 0, s, part_b, slabs, (size_t)n, db,
                        accumulate);
   F3D_CHECK_HIP(hipGetLastError());
   return F3D_OK;
