@@ -9,12 +9,12 @@
 //   the reduction runs over the rows, which is the slow axis of both operands in memory, so both MFMA operands are
 //   read TRANSPOSED from LDS (ds_read_b64_tr_b16: a lane receives four consecutive rows of one column).  A workgroup of
 //   eight waves (4 x 2, two per SIMD) owns a 256 x 256 tile of dw and one slab of rows; a wave holds 64 x 128 of it in
-//   128 accumulator registers and skips the 32 x 32 blocks that lie outside dw.  64-row stages go global -> registers
-//   -> LDS (row pitch = row bytes + 32, which spreads the four rows of a transposing read over all banks),
-//   double-buffered, one barrier per stage.  Slabs are sized so that the launch is one round of the chip; every slab
-//   writes its partial tile to the workspace and a second kernel sums the slabs in a fixed order (no atomics: the
-//   result does not depend on scheduling).  The bias gradient is summed on the vector unit from the dy pieces a
-//   thread stages anyway (always the same 8 columns), in the workgroups of the first k-tile.
+//   128 accumulator registers and skips the 32 x 32 blocks that lie outside dw.  32-row stages stream HBM -> LDS
+//   directly (global_load ... lds, no registers) through four stage buffers, so three stages are in flight behind the
+//   one being multiplied; one barrier per stage.  Slabs are sized so that the launch is one round of the chip; every
+//   slab writes its partial tile to the workspace and a second kernel sums the slabs in a fixed order (no atomics: the
+//   result does not depend on scheduling).  The bias gradient rides along in the waves of the first k-tile as one more
+//   product with a matrix of ones.
 #include "f3d_device.h"
 #include "f3d_internal.h"
 
@@ -27,26 +27,41 @@ typedef short i16x4_t __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) i16x4_t lds_i16x4_t;
 
 constexpr int kXcd = 8;
-constexpr int kWgThreads = 512;
-constexpr int kWgNT = 256, kWgKT = 256, kWgMT = 64;
-constexpr int kPitchA = kWgNT * 2 + 32, kPitchB = kWgKT * 2 + 32;   // bytes
-constexpr int kTileA = kWgMT * kPitchA, kTileB = kWgMT * kPitchB;
-constexpr int kWgBuf = kTileA + kTileB;
-constexpr int kWgLds = 2 * kWgBuf;
-constexpr int kPiecesA = kWgMT * (kWgNT / 8) / kWgThreads;   // 16-byte pieces per thread and stage
-constexpr int kPiecesB = kWgMT * (kWgKT / 8) / kWgThreads;
-static_assert(kPitchA % 128 == 32 && kPitchB % 128 == 32, "four consecutive rows cover all banks");
-static_assert(kWgThreads % (kWgNT / 8) == 0, "a thread stages the same dy columns in every piece");
-static_assert(kWgLds <= 160 * 1024 && (kWgThreads / (kWgNT / 8)) * kWgNT * 4 <= kWgLds, "LDS budget");
+constexpr int kWgThreads = 512, kWgWaves = kWgThreads / kWave;
+constexpr int kWgNT = 256, kWgKT = 256;      // tile of dw per workgroup
+constexpr int kWgMT = 32;                    // rows per stage
+constexpr int kWgNBuf = 4;                   // stage buffers: three stages in flight behind the one being multiplied
+constexpr int kRowB = 512;                   // bytes per LDS row of either operand tile (256 bf16, no padding)
+constexpr int kTileB = kWgMT * kRowB;        // one operand tile of a stage
+constexpr int kWgBuf = 2 * kTileB;
+constexpr int kWgLds = kWgNBuf * kWgBuf;
+constexpr int kDmaPerTile = kTileB / 1024 / kWgWaves;   // direct loads (1 KB each) per wave, operand and stage
+static_assert(kWgNT == 256 && kWgKT == 256 && kRowB == 512, "one direct load fills two LDS rows of 32 pieces");
+static_assert(kDmaPerTile * kWgWaves * 1024 == kTileB && kWgLds <= 160 * 1024, "stage geometry");
+
+// 16 bytes per lane from global memory straight into LDS: lane l of the wave lands at lds + 16 l
+__device__ __forceinline__ void wg_dma16(const void* gbase, uint32_t voff, const char* lds) {
+  const uint32_t lds_addr =
+      __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(__attribute__((address_space(3))) const char*)lds);
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+               :
+               : "s"(lds_addr), "v"(voff), "s"(gbase)
+               : "memory", "m0");
+}
 
 // two transposing reads -> one 8-value MFMA operand: slots 0..3 = rows r .. r+3, slots 4..7 = rows r+4 .. r+7 of the
 // lane's column (the same row order for both operands, so the products pair up)
-__device__ __forceinline__ bf16x8_t read_tr8(const char* p, int pitch) {
+__device__ __forceinline__ bf16x8_t read_tr8(const char* p) {
   const i16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_t*)p);
-  const i16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_t*)(p + 4 * pitch));
+  const i16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_t*)(p + 4 * kRowB));
   return __builtin_bit_cast(bf16x8_t, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
 }
 
+// LDS layout of an operand tile: row r at r * 512 bytes, its 16-byte piece c stored at position c ^ 4 (r % 4).  The
+// direct loads write positions linearly (a lane picks the global piece that belongs at its position).  A transposing
+// read has 32 lanes touch 64 bytes of each of four consecutive rows; the swizzle sends the four rows to the four
+// 64-byte quarters of the 256 bytes the 64 banks serve per clock (without it the rows, a multiple of 256 bytes apart,
+// would all meet in the same banks).
 __global__ __launch_bounds__(kWgThreads) void linear_wgrad_kernel(
     const uint16_t* __restrict__ dy, uint32_t lddy, const uint16_t* __restrict__ x, uint32_t ldx,
     float* __restrict__ part_w, float* __restrict__ part_b, uint32_t M, uint32_t N, uint32_t K, uint32_t n_tiles,
@@ -60,83 +75,99 @@ __global__ __launch_bounds__(kWgThreads) void linear_wgrad_kernel(
   const uint32_t slab = item / tiles, tile = item % tiles;
   const uint32_t n0 = (tile / k_tiles) * kWgNT, k0 = (tile % k_tiles) * kWgKT;
   const uint32_t m_begin = slab * slab_rows, m_end = min(M, m_begin + slab_rows);
-  const uint32_t tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
-  const uint32_t nw = wave >> 1, kw = wave & 1u;   // 4 x 2 waves
-  const bool with_bias = part_b != nullptr && k0 == 0;     // uniform over the workgroup
+  const uint32_t tid = threadIdx.x, lane = tid % kWave;
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+  // 4 x 2 waves; the two waves of a SIMD (wave, wave + 4) sit in different k halves
+  const uint32_t nw = wave & 3u, kw = wave >> 2;
+  const bool with_bias = part_b != nullptr && k0 == 0 && kw == 0;
   // 32 x 32 blocks of this wave's 64 x 128 that lie inside dw
   const uint32_t n_w = n0 + nw * 64u, k_w = k0 + kw * 128u;
   const uint32_t ni = n_w >= N ? 0u : min(2u, (N - n_w + 31u) / 32u), nj = k_w >= K ? 0u : min(4u, (K - k_w + 31u) / 32u);
-  float colsum[8];
-#pragma unroll
-  for (int e = 0; e < 8; ++e) colsum[e] = 0.f;
 
-  // ---- staging: which 16-byte pieces this thread moves ----
-  u32x4_t ra[kPiecesA], rb[kPiecesB];
-  auto fetch = [&](uint32_t m0) {
+  // ---- direct loads: instruction q of a tile fills rows 2q, 2q + 1; this wave issues q = kDmaPerTile wave + i.
+  //      Pieces beyond the last column are clamped to the last valid piece (they only reach blocks of dw that are
+  //      never stored), rows beyond the slab to its last row (and zeroed in LDS once they have landed). ----
+  const uint32_t pieces_a = min(32u, (N - n0) / 8u), pieces_b = min(32u, (K - k0) / 8u);
+  uint32_t d_row[kDmaPerTile], d_ca[kDmaPerTile], d_cb[kDmaPerTile];
 #pragma unroll
-    for (int i = 0; i < kPiecesA; ++i) {
-      const uint32_t idx = tid + kWgThreads * i, row = idx / (kWgNT / 8), pc = idx % (kWgNT / 8);
-      ra[i] = u32x4_t{0u, 0u, 0u, 0u};
-      if (m0 + row < m_end && n0 + pc * 8 < N)
-        ra[i] = *reinterpret_cast<const u32x4_t*>(dy + (size_t)(m0 + row) * lddy + n0 + pc * 8);
-    }
+  for (int i = 0; i < kDmaPerTile; ++i) {
+    const uint32_t q = kDmaPerTile * wave + i;
+    d_row[i] = 2u * q + lane / 32u;
+    const uint32_t c = (lane & 31u) ^ ((d_row[i] & 3u) << 2);
+    d_ca[i] = min(c, pieces_a - 1u) * 16u;
+    d_cb[i] = min(c, pieces_b - 1u) * 16u;
+  }
+  auto issue = [&](uint32_t st) {
+    const uint32_t m0 = m_begin + st * kWgMT, last = m_end - 1u - m0;   // m0 < m_end
+    const char* ga = reinterpret_cast<const char*>(dy + (size_t)m0 * lddy + n0);
+    const char* gb = reinterpret_cast<const char*>(x + (size_t)m0 * ldx + k0);
+    char* buf = lds_wg + (st % kWgNBuf) * kWgBuf;
 #pragma unroll
-    for (int i = 0; i < kPiecesB; ++i) {
-      const uint32_t idx = tid + kWgThreads * i, row = idx / (kWgKT / 8), pc = idx % (kWgKT / 8);
-      rb[i] = u32x4_t{0u, 0u, 0u, 0u};
-      if (m0 + row < m_end && k0 + pc * 8 < K)
-        rb[i] = *reinterpret_cast<const u32x4_t*>(x + (size_t)(m0 + row) * ldx + k0 + pc * 8);
-    }
-  };
-  auto stash = [&](char* buf) {
-#pragma unroll
-    for (int i = 0; i < kPiecesA; ++i) {
-      const uint32_t idx = tid + kWgThreads * i, row = idx / (kWgNT / 8), pc = idx % (kWgNT / 8);
-      *reinterpret_cast<u32x4_t*>(buf + row * kPitchA + pc * 16) = ra[i];
-      if (with_bias) {
-#pragma unroll
-        for (int e = 0; e < 4; ++e) { colsum[2 * e] += bf16_lo(ra[i][e]); colsum[2 * e + 1] += bf16_hi(ra[i][e]); }
-      }
-    }
-#pragma unroll
-    for (int i = 0; i < kPiecesB; ++i) {
-      const uint32_t idx = tid + kWgThreads * i, row = idx / (kWgKT / 8), pc = idx % (kWgKT / 8);
-      *reinterpret_cast<u32x4_t*>(buf + kTileA + row * kPitchB + pc * 16) = rb[i];
+    for (int i = 0; i < kDmaPerTile; ++i) {
+      const uint32_t r = min(d_row[i], last), q = kDmaPerTile * wave + i;
+      wg_dma16(ga, r * lddy * 2u + d_ca[i], buf + q * 1024);
+      wg_dma16(gb, r * ldx * 2u + d_cb[i], buf + kTileB + q * 1024);
     }
   };
 
-  // ---- the lane's place in a transposing read: lane p of a 16-lane block points at row p / 4, columns 4 (p % 4).. ----
+  // ---- the lane's place in a transposing read: lane p of a 16-lane block points at row p / 4, columns 4 (p % 4)..;
+  //      the swizzle value 4 (row % 4) = 4 (p / 4) is the same for every row the lane ever reads ----
   const uint32_t half = lane >> 5, p16 = lane & 15u, cgrp = (lane >> 4) & 1u;
-  const uint32_t a_off = (8u * half + p16 / 4u) * kPitchA + (nw * 64u + 16u * cgrp + 4u * (p16 & 3u)) * 2u;
-  const uint32_t b_off = kTileA + (8u * half + p16 / 4u) * kPitchB + (kw * 128u + 16u * cgrp + 4u * (p16 & 3u)) * 2u;
-
-  f32x16_t acc[2][4];
+  const uint32_t row_off = (8u * half + p16 / 4u) * kRowB, sw = (p16 / 4u) << 2, in_piece = 8u * (p16 & 1u);
+  uint32_t a_off[2], b_off[4];
 #pragma unroll
   for (int i = 0; i < 2; ++i)
+    a_off[i] = row_off + (((nw * 8u + 4u * i + 2u * cgrp + ((p16 & 3u) >> 1)) ^ sw) << 4) + in_piece;
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+    b_off[j] = kTileB + row_off + (((kw * 16u + 4u * j + 2u * cgrp + ((p16 & 3u) >> 1)) ^ sw) << 4) + in_piece;
+
+  f32x16_t acc[2][4], accb[2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+#pragma unroll
+    for (int e = 0; e < 16; ++e) accb[i][e] = 0.f;
 #pragma unroll
     for (int j = 0; j < 4; ++j)
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+  }
+  bf16x8_t ones;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) ones[e] = (__bf16)1.0f;
 
   const uint32_t n_stage = m_end > m_begin ? (m_end - m_begin + kWgMT - 1) / kWgMT : 0u;
-  if (n_stage) {
-    fetch(m_begin);
-    stash(lds_wg);
-  }
-  __syncthreads();
+#pragma unroll
+  for (int st = 0; st < kWgNBuf - 1; ++st)
+    if ((uint32_t)st < n_stage) issue(st);
   for (uint32_t st = 0; st < n_stage; ++st) {
-    const char* buf = lds_wg + (st & 1u) * kWgBuf;
-    const bool more = st + 1 < n_stage;
-    if (more) fetch(m_begin + (st + 1) * kWgMT);
+    char* buf = lds_wg + (st % kWgNBuf) * kWgBuf;
+    // this wave's loads of stage st have landed once at most the loads of the later stages are outstanding
+    const uint32_t later = min(n_stage - 1u - st, (uint32_t)kWgNBuf - 2u);
+    if (later == 2u) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(4 * kDmaPerTile) : "memory");
+    else if (later == 1u) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * kDmaPerTile) : "memory");
+    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    const uint32_t rows_left = m_end - (m_begin + st * kWgMT);
+    if (rows_left < (uint32_t)kWgMT) {   // rows past the slab: zeros
+#pragma unroll
+      for (int i = 0; i < kDmaPerTile; ++i)
+        if (d_row[i] >= rows_left) {
+          const uint32_t pos = (kDmaPerTile * wave + i) * 1024u + lane * 16u;
+          *reinterpret_cast<u32x4_t*>(buf + pos) = u32x4_t{0u, 0u, 0u, 0u};
+          *reinterpret_cast<u32x4_t*>(buf + kTileB + pos) = u32x4_t{0u, 0u, 0u, 0u};
+        }
+    }
+    wg_barrier_lds();   // every wave's part of stage st is in LDS; every wave is done with stage st - 1
+    if (st + kWgNBuf - 1 < n_stage) issue(st + kWgNBuf - 1);   // into the buffer of stage st - 1
     // operands of k-step ks + 1 are requested before the products of k-step ks are issued
     bf16x8_t fa[2][2], fb[2][4];
     auto frags = [&](int ks, bf16x8_t (&a)[2], bf16x8_t (&b)[4]) {
 #pragma unroll
       for (int i = 0; i < 2; ++i)
-        if ((uint32_t)i < ni) a[i] = read_tr8(buf + a_off + ks * 16 * kPitchA + i * 64, kPitchA);
+        if ((uint32_t)i < ni) a[i] = read_tr8(buf + a_off[i] + ks * 16 * kRowB);
 #pragma unroll
       for (int j = 0; j < 4; ++j)
-        if ((uint32_t)j < nj) b[j] = read_tr8(buf + b_off + ks * 16 * kPitchB + j * 64, kPitchB);
+        if ((uint32_t)j < nj) b[j] = read_tr8(buf + b_off[j] + ks * 16 * kRowB);
     };
     frags(0, fa[0], fb[0]);
 #pragma unroll
@@ -148,9 +179,13 @@ __global__ __launch_bounds__(kWgThreads) void linear_wgrad_kernel(
         for (int j = 0; j < 4; ++j)
           if ((uint32_t)i < ni && (uint32_t)j < nj)
             acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[ks & 1][i], fb[ks & 1][j], acc[i][j], 0, 0, 0);
+      if (with_bias) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+          if ((uint32_t)i < ni)
+            accb[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[ks & 1][i], ones, accb[i], 0, 0, 0);
+      }
     }
-    if (more) stash(lds_wg + ((st + 1) & 1u) * kWgBuf);
-    __syncthreads();
   }
 
   // ---- this slab's partial tile: accumulator slot e of a lane is row 8 (e / 4) + 4 half + e % 4, column lane % 32 ----
@@ -159,27 +194,15 @@ __global__ __launch_bounds__(kWgThreads) void linear_wgrad_kernel(
   for (int i = 0; i < 2; ++i) {
 #pragma unroll
     for (int e = 0; e < 16; ++e) {
-      const uint32_t n = n0 + nw * 64u + 32u * i + 8u * (e / 4) + 4u * half + (e % 4);
+      const uint32_t n = n_w + 32u * i + 8u * (e / 4) + 4u * half + (e % 4);
       if (n >= N) continue;
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        const uint32_t k = k0 + kw * 128u + 32u * j + (lane & 31u);
+        const uint32_t k = k_w + 32u * j + (lane & 31u);
         if (k < K) pw[(size_t)n * K + k] = acc[i][j][e];
       }
-    }
-  }
-  // ---- bias gradient: the 16 threads that staged the same 8 columns meet in LDS (the stage buffers are dead) ----
-  if (with_bias) {
-    constexpr int kGroups = kWgThreads / (kWgNT / 8);
-    float* s_cs = reinterpret_cast<float*>(lds_wg);
-    const uint32_t pc = tid % (kWgNT / 8), grp = tid / (kWgNT / 8);
-#pragma unroll
-    for (int e = 0; e < 8; ++e) s_cs[grp * kWgNT + pc * 8 + e] = colsum[e];
-    __syncthreads();
-    if (tid < (uint32_t)kWgNT && n0 + tid < N) {
-      float t = 0.f;
-      for (int g = 0; g < kGroups; ++g) t += s_cs[g * kWgNT + tid];
-      part_b[(size_t)slab * N + n0 + tid] = t;
+      // every column of the product with the matrix of ones holds the row sum
+      if (with_bias && (lane & 31u) == 0) part_b[(size_t)slab * N + n] = accb[i][e];
     }
   }
 }
