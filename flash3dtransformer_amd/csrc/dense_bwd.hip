@@ -137,18 +137,18 @@ __global__ __launch_bounds__(kWgThreads) void linear_wgrad_kernel(
   for (int e = 0; e < 8; ++e) ones[e] = (__bf16)1.0f;
 
   const uint32_t n_stage = m_end > m_begin ? (m_end - m_begin + kWgMT - 1) / kWgMT : 0u;
-#pragma unroll
-  for (int st = 0; st < kWgNBuf - 1; ++st)
-    if ((uint32_t)st < n_stage) issue(st);
-  for (uint32_t st = 0; st < n_stage; ++st) {
-    char* buf = lds_wg + (st % kWgNBuf) * kWgBuf;
-    // this wave's loads of stage st have landed once at most the loads of the later stages are outstanding
-    const uint32_t later = min(n_stage - 1u - st, (uint32_t)kWgNBuf - 2u);
+  static_assert(kWgMT == 32, "two k-steps per stage");
+  // waits until this wave's loads of stage st have landed (at most the loads of the later stages, two of them at
+  // that point, stay outstanding), zeroes the rows past the slab, and meets the other waves: after the barrier the
+  // whole stage is in LDS and every wave has its operands of the stages before it in registers
+  auto stage_ready = [&](uint32_t st) {
+    const uint32_t later = min(n_stage - 1u - st, 2u);
     if (later == 2u) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(4 * kDmaPerTile) : "memory");
     else if (later == 1u) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * kDmaPerTile) : "memory");
     else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     const uint32_t rows_left = m_end - (m_begin + st * kWgMT);
-    if (rows_left < (uint32_t)kWgMT) {   // rows past the slab: zeros
+    if (rows_left < (uint32_t)kWgMT) {
+      char* buf = lds_wg + (st % kWgNBuf) * kWgBuf;
 #pragma unroll
       for (int i = 0; i < kDmaPerTile; ++i)
         if (d_row[i] >= rows_left) {
@@ -157,35 +157,50 @@ __global__ __launch_bounds__(kWgThreads) void linear_wgrad_kernel(
           *reinterpret_cast<u32x4_t*>(buf + kTileB + pos) = u32x4_t{0u, 0u, 0u, 0u};
         }
     }
-    wg_barrier_lds();   // every wave's part of stage st is in LDS; every wave is done with stage st - 1
-    if (st + kWgNBuf - 1 < n_stage) issue(st + kWgNBuf - 1);   // into the buffer of stage st - 1
-    // operands of k-step ks + 1 are requested before the products of k-step ks are issued
-    bf16x8_t fa[2][2], fb[2][4];
-    auto frags = [&](int ks, bf16x8_t (&a)[2], bf16x8_t (&b)[4]) {
+    wg_barrier_lds();
+  };
+  bf16x8_t fa[2][2], fb[2][4];
+  auto frags = [&](uint32_t st, int ks, bf16x8_t (&a)[2], bf16x8_t (&b)[4]) {
+    const char* buf = lds_wg + (st % kWgNBuf) * kWgBuf;
 #pragma unroll
-      for (int i = 0; i < 2; ++i)
-        if ((uint32_t)i < ni) a[i] = read_tr8(buf + a_off[i] + ks * 16 * kRowB);
+    for (int i = 0; i < 2; ++i)
+      if ((uint32_t)i < ni) a[i] = read_tr8(buf + a_off[i] + ks * 16 * kRowB);
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      if ((uint32_t)j < nj) b[j] = read_tr8(buf + b_off[j] + ks * 16 * kRowB);
+  };
+  auto products = [&](const bf16x8_t (&a)[2], const bf16x8_t (&b)[4]) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
 #pragma unroll
       for (int j = 0; j < 4; ++j)
-        if ((uint32_t)j < nj) b[j] = read_tr8(buf + b_off[j] + ks * 16 * kRowB);
-    };
-    frags(0, fa[0], fb[0]);
-#pragma unroll
-    for (int ks = 0; ks < kWgMT / 16; ++ks) {
-      if (ks + 1 < kWgMT / 16) frags(ks + 1, fa[(ks + 1) & 1], fb[(ks + 1) & 1]);
+        if ((uint32_t)i < ni && (uint32_t)j < nj)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
+    if (with_bias) {
 #pragma unroll
       for (int i = 0; i < 2; ++i)
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-          if ((uint32_t)i < ni && (uint32_t)j < nj)
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[ks & 1][i], fb[ks & 1][j], acc[i][j], 0, 0, 0);
-      if (with_bias) {
-#pragma unroll
-        for (int i = 0; i < 2; ++i)
-          if ((uint32_t)i < ni)
-            accb[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[ks & 1][i], ones, accb[i], 0, 0, 0);
-      }
+        if ((uint32_t)i < ni) accb[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], ones, accb[i], 0, 0, 0);
     }
+  };
+  // Three stages are requested ahead.  The hand-over to the next stage (wait, barrier, first operand reads) sits
+  // between the two k-steps of a stage, so the products of the second k-step run over it.
+#pragma unroll
+  for (int st = 0; st < kWgNBuf - 1; ++st)
+    if ((uint32_t)st < n_stage) issue(st);
+  if (n_stage) {
+    stage_ready(0);
+    frags(0, 0, fa[0], fb[0]);
+  }
+  for (uint32_t st = 0; st < n_stage; ++st) {
+    // the buffer of stage st - 1 is free: every wave read the last of it before the barrier that made stage st ready
+    if (st + kWgNBuf - 1 < n_stage) issue(st + kWgNBuf - 1);
+    frags(st, 1, fa[1], fb[1]);
+    products(fa[0], fb[0]);
+    if (st + 1 < n_stage) {
+      stage_ready(st + 1);   // stages st + 2 and st + 3 are the ones still in flight
+      frags(st + 1, 0, fa[0], fb[0]);
+    }
+    products(fa[1], fb[1]);
   }
 
   // ---- this slab's partial tile: accumulator slot e of a lane is row 8 (e / 4) + 4 half + e % 4, column lane % 32 ----
