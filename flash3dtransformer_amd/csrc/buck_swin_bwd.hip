@@ -130,7 +130,8 @@ __global__ __launch_bounds__(2 * T) void buck_swin_bwd_dkdv_kernel(
     const uint16_t* __restrict__ o, const uint16_t* __restrict__ d_o, const float* __restrict__ lse,
     float* __restrict__ delta, uint16_t* __restrict__ dk, uint16_t* __restrict__ dv,
     const uint32_t* __restrict__ scope_buckets, uint32_t num_scope, uint32_t scope_size, uint32_t bs,
-    uint32_t seq_len, uint32_t num_head, float scale, float scale_log2, uint32_t n_items, uint32_t items_per_xcd) {
+    uint32_t seq_len, uint32_t num_head, float scale, float scale_log2, uint32_t n_items, uint32_t items_per_xcd,
+    uint32_t ldg) {
   using G = BwdGeom<D>;
   constexpr int KSTEPS = G::KSTEPS, ROWB = G::ROWB, OPB = T * ROWB;
   extern __shared__ __attribute__((aligned(16))) char lds_bwd[];
@@ -251,8 +252,10 @@ __global__ __launch_bounds__(2 * T) void buck_swin_bwd_dkdv_kernel(
   }
 
   // acc[g4*4 + r] = d?t[feature g4*8 + 4 half + r][key lq]: 4 consecutive features of the lane's key per group
-  uint16_t* dkrow = dk + base_o + (size_t)grow * ldo;
-  uint16_t* dvrow = dv + base_o + (size_t)grow * ldo;
+  // the gradients' rows are ldg elements apart (dense: ldg = ldo; thirds of one [B, L, 3 H D] tensor: ldg = 3 ldo)
+  const size_t base_g = (size_t)it.batch * seq_len * ldg + (size_t)it.head * D;
+  uint16_t* dkrow = dk + base_g + (size_t)grow * ldg;
+  uint16_t* dvrow = dv + base_g + (size_t)grow * ldg;
 #pragma unroll
   for (int g4 = 0; g4 < 4; ++g4) {
     const uint32_t d0 = g4 * 8 + half * 4;
@@ -275,7 +278,7 @@ __global__ __launch_bounds__(2 * T) void buck_swin_bwd_dq_kernel(
     const uint16_t* __restrict__ d_o, const float* __restrict__ lse, const float* __restrict__ delta,
     uint16_t* __restrict__ dq, const uint32_t* __restrict__ scope_buckets, uint32_t num_scope, uint32_t scope_size,
     uint32_t bs, uint32_t seq_len, uint32_t num_head, float scale, float scale_log2, uint32_t n_items,
-    uint32_t items_per_xcd) {
+    uint32_t items_per_xcd, uint32_t ldg) {
   using G = BwdGeom<D>;
   constexpr int KSTEPS = G::KSTEPS, ROWB = G::ROWB, OPB = T * ROWB;
   extern __shared__ __attribute__((aligned(16))) char lds_bwd[];
@@ -355,7 +358,8 @@ __global__ __launch_bounds__(2 * T) void buck_swin_bwd_dq_kernel(
       acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ktr[kk], __builtin_bit_cast(bf16x8_t, sraw), acc, 0, 0, 0);
     }
   }
-  uint16_t* dqrow = dq + base_o + (size_t)grow * ldo;
+  const size_t base_g = (size_t)it.batch * seq_len * ldg + (size_t)it.head * D;
+  uint16_t* dqrow = dq + base_g + (size_t)grow * ldg;
 #pragma unroll
   for (int g4 = 0; g4 < 4; ++g4) {
     const uint32_t d0 = g4 * 8 + half * 4;
@@ -372,7 +376,7 @@ template <int D, int T>
 static int launch_attn_bwd(const uint16_t* q, const uint16_t* k, const uint16_t* v, uint32_t ld, const uint16_t* o,
                            const uint16_t* d_o, const float* lse, float* delta, uint16_t* dq, uint16_t* dk,
                            uint16_t* dv, const uint32_t* scope_buckets, uint32_t num_scope, uint32_t scope_size,
-                           uint32_t bs, uint32_t batch, uint32_t seq_len, uint32_t num_head, int device,
+                           uint32_t bs, uint32_t batch, uint32_t seq_len, uint32_t num_head, uint32_t ldg, int device,
                            hipStream_t s) {
   static bool attr_set[64] = {};
   auto kern_a = buck_swin_bwd_dkdv_kernel<D, T>;
@@ -387,9 +391,9 @@ static int launch_attn_bwd(const uint16_t* q, const uint16_t* k, const uint16_t*
   const uint32_t per_xcd = (n_items + kBwdXcd - 1) / kBwdXcd;
   const float scale = 1.0f / sqrtf((float)D), scale_log2 = 1.4426950408889634f * scale;
   hipLaunchKernelGGL(kern_a, dim3(per_xcd * kBwdXcd), dim3(2 * T), lds_a, s, q, k, v, ld, o, d_o, lse, delta, dk, dv,
-                     scope_buckets, num_scope, scope_size, bs, seq_len, num_head, scale, scale_log2, n_items, per_xcd);
+                     scope_buckets, num_scope, scope_size, bs, seq_len, num_head, scale, scale_log2, n_items, per_xcd, ldg);
   hipLaunchKernelGGL(kern_b, dim3(per_xcd * kBwdXcd), dim3(2 * T), lds_b, s, q, k, v, ld, d_o, lse, delta, dq,
-                     scope_buckets, num_scope, scope_size, bs, seq_len, num_head, scale, scale_log2, n_items, per_xcd);
+                     scope_buckets, num_scope, scope_size, bs, seq_len, num_head, scale, scale_log2, n_items, per_xcd, ldg);
   return F3D_OK;
 }
 
@@ -401,8 +405,23 @@ extern "C" int f3d_buck_swin_bwd(const f3d_bf16_t* q, const f3d_bf16_t* k, const
                                  const uint32_t* scope_buckets, uint32_t num_scope, uint32_t scope_size,
                                  uint32_t bucket_size, uint32_t batch, uint32_t seq_len, uint32_t num_head,
                                  uint32_t head_dim, const int32_t* kv_len, int device, void* stream) {
+  return f3d_buck_swin_bwd_strided(q, k, v, qkv_row_stride, o, d_o, lse, delta, dq, dk, dv, num_head * head_dim,
+                                   scope_buckets, num_scope, scope_size, bucket_size, batch, seq_len, num_head, head_dim,
+                                   kv_len, device, stream);
+}
+
+extern "C" int f3d_buck_swin_bwd_strided(const f3d_bf16_t* q, const f3d_bf16_t* k, const f3d_bf16_t* v,
+                                         uint32_t qkv_row_stride, const f3d_bf16_t* o, const f3d_bf16_t* d_o,
+                                         const float* lse, float* delta, f3d_bf16_t* dq, f3d_bf16_t* dk, f3d_bf16_t* dv,
+                                         uint32_t grad_row_stride, const uint32_t* scope_buckets, uint32_t num_scope,
+                                         uint32_t scope_size, uint32_t bucket_size, uint32_t batch, uint32_t seq_len,
+                                         uint32_t num_head, uint32_t head_dim, const int32_t* kv_len, int device,
+                                         void* stream) {
   using namespace f3d;
   F3D_CHECK_ARG(q && k && v && o && d_o && lse && delta && dq && dk && dv && scope_buckets, "null tensor pointer");
+  F3D_CHECK_ARG(grad_row_stride >= num_head * head_dim && grad_row_stride % 8 == 0,
+                "dq/dk/dv row stride %u must be a multiple of 8 and at least num_head*head_dim=%u", grad_row_stride,
+                num_head * head_dim);
   F3D_CHECK_ARG(bucket_size >= 128 && bucket_size % 128 == 0, "bucket_size=%u must be a multiple of 128",
                 bucket_size);
   F3D_CHECK_ARG(seq_len % bucket_size == 0, "sequence length %u is not a multiple of bucket_size=%u", seq_len,
@@ -435,10 +454,11 @@ extern "C" int f3d_buck_swin_bwd(const f3d_bf16_t* q, const f3d_bf16_t* k, const
   int rc;
 #define F3D_BWD(DD, TT)                                                                                          \
   rc = launch_attn_bwd<DD, TT>(q, k, v, qkv_row_stride, o, d_o, lse, delta, dq, dk, dv, scope_buckets, num_scope, \
-                               scope_size, bucket_size, batch, seq_len, num_head, device, s)
+                               scope_size, bucket_size, batch, seq_len, num_head, grad_row_stride, device, s)
   if (!resident) {
     rc = launch_attn_bwd_stream(q, k, v, qkv_row_stride, o, d_o, lse, delta, dq, dk, dv, scope_buckets, num_scope,
-                                scope_size, bucket_size, batch, seq_len, num_head, head_dim, kv_len, device, s);
+                                scope_size, bucket_size, batch, seq_len, num_head, head_dim, kv_len, grad_row_stride,
+                                device, s);
   } else if (head_dim == 16) {
     if (scope_tokens == 256) F3D_BWD(16, 256); else F3D_BWD(16, 512);
   } else {

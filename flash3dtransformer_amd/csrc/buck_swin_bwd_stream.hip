@@ -176,7 +176,7 @@ __global__ __launch_bounds__(64 * kStreamWaves) void bwd_dkdv_stream_kernel(
     const uint16_t* __restrict__ d_o, const float* __restrict__ lse, const float* __restrict__ delta,
     uint16_t* __restrict__ dk, uint16_t* __restrict__ dv, const uint32_t* __restrict__ scope_buckets,
     uint32_t num_scope, uint32_t scope_size, uint32_t bs, uint32_t seq_len, uint32_t num_head,
-    const int32_t* __restrict__ kv_len, float scale, float scale_log2) {
+    const int32_t* __restrict__ kv_len, float scale, float scale_log2, uint32_t ldg) {
   using G = SGeom<D>;
   constexpr int KSTEPS = G::KSTEPS, ROWB = G::ROWB, DT = G::DT, TILEB = G::TILEB;
   extern __shared__ __attribute__((aligned(16))) char lds_s[];
@@ -312,8 +312,10 @@ __global__ __launch_bounds__(64 * kStreamWaves) void bwd_dkdv_stream_kernel(
   }
 
   // acc[dt][g4*4 + r] = d?t[feature 32 dt + g4*8 + 4 half + r][key lq]: 4 consecutive features of the lane's key per group
-  uint16_t* dkrow = dk + base_o + (size_t)krow * ldo;
-  uint16_t* dvrow = dv + base_o + (size_t)krow * ldo;
+  // the gradients' rows are ldg elements apart (dense: ldg = ldo; thirds of one [B, L, 3 H D] tensor: ldg = 3 ldo)
+  const size_t base_g = (size_t)it.batch * seq_len * ldg + (size_t)it.head * D;
+  uint16_t* dkrow = dk + base_g + (size_t)krow * ldg;
+  uint16_t* dvrow = dv + base_g + (size_t)krow * ldg;
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
@@ -338,7 +340,7 @@ __global__ __launch_bounds__(64 * kStreamWaves) void bwd_dq_stream_kernel(
     const uint16_t* __restrict__ d_o, const float* __restrict__ lse, const float* __restrict__ delta,
     uint16_t* __restrict__ dq, const uint32_t* __restrict__ scope_buckets, uint32_t num_scope, uint32_t scope_size,
     uint32_t bs, uint32_t seq_len, uint32_t num_head, const int32_t* __restrict__ kv_len, float scale,
-    float scale_log2) {
+    float scale_log2, uint32_t ldg) {
   using G = SGeom<D>;
   constexpr int KSTEPS = G::KSTEPS, ROWB = G::ROWB, DT = G::DT, TILEB = G::TILEB;
   extern __shared__ __attribute__((aligned(16))) char lds_s[];
@@ -456,7 +458,8 @@ __global__ __launch_bounds__(64 * kStreamWaves) void bwd_dq_stream_kernel(
     t = tn;
     b ^= 1u;
   }
-  uint16_t* dqrow = dq + base_o + (size_t)qrow * ldo;
+  const size_t base_g = (size_t)it.batch * seq_len * ldg + (size_t)it.head * D;
+  uint16_t* dqrow = dq + base_g + (size_t)qrow * ldg;
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
@@ -475,8 +478,8 @@ template <int D>
 static int launch_stream(const uint16_t* q, const uint16_t* k, const uint16_t* v, uint32_t ld, const uint16_t* o,
                          const uint16_t* d_o, const float* lse, float* delta, uint16_t* dq, uint16_t* dk, uint16_t* dv,
                          const uint32_t* scope_buckets, uint32_t num_scope, uint32_t scope_size, uint32_t bs,
-                         uint32_t batch, uint32_t seq_len, uint32_t num_head, const int32_t* kv_len, int device,
-                         hipStream_t s) {
+                         uint32_t batch, uint32_t seq_len, uint32_t num_head, const int32_t* kv_len, uint32_t ldg,
+                         int device, hipStream_t s) {
   const size_t lds = stream_lds_bytes<D>(scope_size);
   if (lds > 64 * 1024) {
     // the scope table is the only part that grows: 8 bytes per bucket of the scope
@@ -492,9 +495,9 @@ static int launch_stream(const uint16_t* q, const uint16_t* k, const uint16_t* v
                      num_scope, scope_size, bs, seq_len, num_head);
   const dim3 grid(scope_tokens / kStreamBlock, items), block(64 * kStreamWaves);
   hipLaunchKernelGGL(bwd_dkdv_stream_kernel<D>, grid, block, lds, s, q, k, v, ld, d_o, lse, delta, dk, dv, scope_buckets,
-                     num_scope, scope_size, bs, seq_len, num_head, kv_len, scale, scale_log2);
+                     num_scope, scope_size, bs, seq_len, num_head, kv_len, scale, scale_log2, ldg);
   hipLaunchKernelGGL(bwd_dq_stream_kernel<D>, grid, block, lds, s, q, k, v, ld, d_o, lse, delta, dq, scope_buckets, num_scope,
-                     scope_size, bs, seq_len, num_head, kv_len, scale, scale_log2);
+                     scope_size, bs, seq_len, num_head, kv_len, scale, scale_log2, ldg);
   return F3D_OK;
 }
 
@@ -503,7 +506,7 @@ int launch_attn_bwd_stream(const uint16_t* q, const uint16_t* k, const uint16_t*
                            const uint16_t* d_o, const float* lse, float* delta, uint16_t* dq, uint16_t* dk, uint16_t* dv,
                            const uint32_t* scope_buckets, uint32_t num_scope, uint32_t scope_size, uint32_t bs,
                            uint32_t batch, uint32_t seq_len, uint32_t num_head, uint32_t head_dim, const int32_t* kv_len,
-                           int device, hipStream_t s) {
+                           uint32_t ldg, int device, hipStream_t s) {
   if ((uint64_t)batch * num_scope * num_head > 65535u) {
     set_error("attention backward: %llu (batch, scope, head) items exceed one launch's 65535",
               (unsigned long long)batch * num_scope * num_head);
@@ -511,7 +514,7 @@ int launch_attn_bwd_stream(const uint16_t* q, const uint16_t* k, const uint16_t*
   }
 #define F3D_STREAM(DD)                                                                                                 \
   return launch_stream<DD>(q, k, v, ld, o, d_o, lse, delta, dq, dk, dv, scope_buckets, num_scope, scope_size, bs, batch, \
-                           seq_len, num_head, kv_len, device, s)
+                           seq_len, num_head, kv_len, ldg, device, s)
   switch (head_dim) {
     case 16: F3D_STREAM(16);
     case 32: F3D_STREAM(32);

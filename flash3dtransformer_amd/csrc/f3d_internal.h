@@ -24,12 +24,13 @@ void* workspace(int device, size_t bytes);
 uint32_t* psh_noalloc_scratch(int device);
 
 // Streaming attention backward (buck_swin_bwd_stream.hip): any scope size, head_dim 16 / 32 / 64 / 128, optional
-// valid lengths per bucket.  Launches on `s`; F3D_ERR_UNSUPPORTED (+ message) for other head sizes.
+// valid lengths per bucket; dq / dk / dv rows are `ldg` elements apart.  Launches on `s`; F3D_ERR_UNSUPPORTED (+ message)
+// for other head sizes.
 int launch_attn_bwd_stream(const uint16_t* q, const uint16_t* k, const uint16_t* v, uint32_t ld, const uint16_t* o,
                            const uint16_t* d_o, const float* lse, float* delta, uint16_t* dq, uint16_t* dk, uint16_t* dv,
                            const uint32_t* scope_buckets, uint32_t num_scope, uint32_t scope_size, uint32_t bs,
                            uint32_t batch, uint32_t seq_len, uint32_t num_head, uint32_t head_dim, const int32_t* kv_len,
-                           int device, hipStream_t s);
+                           uint32_t ldg, int device, hipStream_t s);
 
 bool sync_stream_enabled();
 uint32_t global_seed();

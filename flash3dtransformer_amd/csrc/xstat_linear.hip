@@ -46,7 +46,6 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
   using G = XsGeom<K>;
   constexpr int KS = K / 16;             // MFMA k-steps
   constexpr int ROWB = G::ROWB;
-  constexpr int NT = 64 * WAVES;
   constexpr int ROWS_WG = 32 * MT * WAVES;
   extern __shared__ __attribute__((aligned(1024))) char lds_xs[];
   constexpr size_t kFront = (size_t)NBUF * G::CHUNK_BYTES > (size_t)WAVES * 32 * (G::KP + 8) * 2
@@ -239,7 +238,6 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
   // stage 3: epilogue of chunk ci: the wave's 32 x 32 result tiles go through a wave-private LDS patch so
   // that the global stores are row-contiguous 16-byte pieces (4 lanes = 64 bytes of one row)
   auto stage_epilogue = [&](uint32_t ci) {
-    const uint32_t slot = ci % NBUF;
     const uint32_t col0 = actual(ci) * COLS;   // first output column of the chunk
     // Residual pieces of the whole chunk are requested up front (one memory latency for all of them, hidden
     // behind the packing below) instead of one by one where they are added.  Rows past M read row M - 1.

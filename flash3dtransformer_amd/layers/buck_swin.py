@@ -34,6 +34,36 @@ class BuckSwinFwdFunction(Function):
         return bwd.dQ, bwd.dK, bwd.dV, None, None
 
 
+class BuckSwinQKVFunction(Function):
+    """The same attention over the three thirds of one projection output qkv [B, L, 3 H D] (the kernel reads Q, K, V
+    as column slices).  The backward writes dQ, dK, dV straight into the thirds of one [B, L, 3 H D] gradient, so
+    autograd neither splits the projection output nor concatenates three gradients."""
+
+    @staticmethod
+    def forward(ctx, qkv, scope_buckets, buck_size: int, num_heads: int) -> torch.Tensor:
+        B, L, C3 = qkv.shape
+        D = C3 // 3 // num_heads
+        Q, K, V = (t.view(B, L, num_heads, D) for t in torch.chunk(qkv, 3, dim=-1))
+        buff = sa.BuckSwinFwdBuffers.create_buckswin_fwd_buff(Q)
+        pshattn.buck_swin_fwd(Q, K, V, buff.O, buff.LSE, scope_buckets, buck_size)
+        ctx.save_for_backward(qkv, buff.O, buff.LSE)
+        ctx.scope_buckets, ctx.buck_size, ctx.num_heads = scope_buckets, buck_size, num_heads
+        return buff.O
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        qkv, O, lse = ctx.saved_tensors
+        B, L, H, D = O.shape
+        Q, K, V = (t.view(B, L, H, D) for t in torch.chunk(qkv, 3, dim=-1))
+        dO = grad_output if grad_output.dtype == torch.bfloat16 else grad_output.to(torch.bfloat16)
+        # zero-filled: rows that no scope covers are not written
+        dqkv = torch.zeros_like(qkv)
+        dQ, dK, dV = (t.view(B, L, H, D) for t in torch.chunk(dqkv, 3, dim=-1))
+        delta = torch.zeros(B, L, H, dtype=torch.float32, device=O.device)
+        pshattn.buck_swin_bwd(Q, K, V, O, dO.contiguous(), lse, delta, dQ, dK, dV, ctx.scope_buckets, ctx.buck_size)
+        return dqkv, None, None, None
+
+
 class BucketSwinAttention(nn.Module):
     def __init__(self, buck_size: int) -> None:
         super().__init__()
@@ -67,8 +97,11 @@ class BucketSwinAttentionModule(nn.Module):
         if f3ddev.get_nvtx():
             nvtx.range_push(self.NVTX_SCOPE)
         qkv = self.qkv(x, pre_norm=pre_norm)   # pre_norm: LayerNorm applied inside the projection kernel
-        q, k, v = (t.view(B, L, self.num_heads, self.head_dim) for t in torch.chunk(qkv, 3, dim=-1))
-        attn_out = self.attn(q, k, v, scope_buckets)
+        if qkv.dtype == torch.bfloat16 and qkv.is_contiguous():
+            attn_out = BuckSwinQKVFunction.apply(qkv, scope_buckets, self.attn.buck_size, self.num_heads)
+        else:
+            q, k, v = (t.view(B, L, self.num_heads, self.head_dim) for t in torch.chunk(qkv, 3, dim=-1))
+            attn_out = self.attn(q, k, v, scope_buckets)
         out = self.proj(attn_out.view(B, L, C), residual=residual)
         if f3ddev.get_nvtx():
             nvtx.range_pop()

@@ -52,6 +52,30 @@ class PSHScatterLayer(nn.Module):
         return pm.batch_bucket_scatter(coords, seps, self.bucket_size, pad_to, hash_op)
 
 
+class _CoordEmbedGrad(torch.autograd.Function):
+    """emb = bf16(coord) @ w.T + b computed by the HIP forward; the coordinates carry no gradient, the weights take
+    theirs from the weight-gradient kernel over the coordinates padded to 8 columns (its inner sizes are multiples of 8)"""
+
+    @staticmethod
+    def forward(ctx, emb, weight, bias, coord):
+        ctx.save_for_backward(weight, bias, coord)
+        return emb.view_as(emb)
+
+    @staticmethod
+    def backward(ctx, dy):
+        weight, bias, coord = ctx.saved_tensors
+        dy2 = dy if dy.dtype == torch.bfloat16 else dy.to(torch.bfloat16)
+        if dy2.stride(-1) != 1:
+            dy2 = dy2.contiguous()
+        c8 = torch.zeros(coord.shape[0], 8, dtype=torch.bfloat16, device=coord.device)
+        c8[:, :3] = coord
+        dw8 = torch.empty(weight.shape[0], 8, dtype=torch.float32, device=coord.device)
+        db = torch.empty(weight.shape[0], dtype=torch.float32, device=coord.device) if bias is not None else None
+        pshattn.linear_wgrad_bf16(dy2, c8, dw8, db)
+        return (None, dw8[:, :3].to(weight.dtype) if ctx.needs_input_grad[1] else None,
+                db.to(bias.dtype) if bias is not None and ctx.needs_input_grad[2] else None, None)
+
+
 class PSH3DCoordEmbedding(nn.Module):
     """PSH-scatter the coordinates (padded to `alignment` rows) and embed them with a 3 -> emb_dim
     linear layer.  Returns the embedding; the scattered coordinates of the last call are kept in
@@ -75,6 +99,10 @@ class PSH3DCoordEmbedding(nn.Module):
         lin = self.lin
         pshattn.coord_embed_bf16(scattered, lin._w.get(lin.weight, lin.training), lin._b.get(lin.bias, lin.training), emb)
         # the coordinates carry no gradient; the embedding's weights do (bf16 view of the fp16 coordinates, as the kernel reads them)
+        if not (torch.is_grad_enabled() and (lin.weight.requires_grad or (lin.bias is not None and lin.bias.requires_grad))):
+            return emb
+        if lin.out_features % 8 == 0:
+            return _CoordEmbedGrad.apply(emb, lin.weight, lin.bias, scattered)
         coord_f = scattered
         ref = lambda w, b: torch.nn.functional.linear(coord_f.to(torch.bfloat16).float(), w, b)
         return torch_backward(emb, ref, lin.weight, lin.bias)

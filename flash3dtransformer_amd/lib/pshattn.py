@@ -406,8 +406,9 @@ def buck_swin_fwd(Q, K, V, O, L, Scope_buckets, bucket_size, kv_len=None):
 
 def buck_swin_bwd(Q, K, V, O, dO, LSE, Delta, dQ, dK, dV, Scope_buckets, bucket_size, kv_len=None):
     """declared src/f3d_frontend.cu:94-97, called at flash3dxfmr/layers/buck_swin.py:90-92.
-    Q, K, V [B,L,H,D] bf16 (may be column slices of one projection output, equal strides); O, dO, dQ, dK, dV dense
-    [B,L,H,D] bf16; LSE (from the forward), Delta (written here: rowsum(dO * O)) [B,L,H] fp32.  Rows that no scope
+    Q, K, V [B,L,H,D] bf16 (may be column slices of one projection output, equal strides); O, dO dense [B,L,H,D]
+    bf16; dQ, dK, dV [B,L,H,D] bf16, dense or (extension) column slices of one [B,L,3HD] gradient tensor with equal
+    strides; LSE (from the forward), Delta (written here: rowsum(dO * O)) [B,L,H] fp32.  Rows that no scope
     covers are not written (pass zero-filled dQ / dK / dV).  head_dim 16, 32, 64 or 128; scopes of any number of
     buckets.  kv_len (extension, as in the forward): int32 [L / bucket_size] valid rows per bucket."""
     dev = assert_same_device([Q, K, V, O, dO, LSE, Delta, dQ, dK, dV, Scope_buckets] +
@@ -420,7 +421,7 @@ def buck_swin_bwd(Q, K, V, O, dO, LSE, Delta, dQ, dK, dV, Scope_buckets, bucket_
     assert_dtype([Q, K, V, O, dO, dQ, dK, dV], torch.bfloat16)
     assert_dtype([LSE, Delta], torch.float32)
     assert_dtype([Scope_buckets], torch.uint32)
-    assert_contiguous([O, dO, dQ, dK, dV, LSE, Delta, Scope_buckets])
+    assert_contiguous([O, dO, LSE, Delta, Scope_buckets])
     if Q.dim() != 4 or any(t.shape != Q.shape for t in (K, V, O, dO, dQ, dK, dV)):
         raise RuntimeError("Q/K/V/O/dO/dQ/dK/dV must share one [B,L,H,D] shape")
     B, Ls, H, D = Q.shape
@@ -431,9 +432,12 @@ def buck_swin_bwd(Q, K, V, O, dO, LSE, Delta, dQ, dK, dV, Scope_buckets, bucket_
     for t in (Q, K, V):
         if t.stride(3) != 1 or t.stride(2) != D or t.stride(0) != t.stride(1) * Ls or t.stride() != Q.stride():
             raise RuntimeError("Q/K/V must be dense over (H, D) with identical strides")
-    rc = _load().f3d_buck_swin_bwd(
+    for t in (dQ, dK, dV):
+        if t.stride(3) != 1 or t.stride(2) != D or t.stride(0) != t.stride(1) * Ls or t.stride() != dQ.stride():
+            raise RuntimeError("dQ/dK/dV must be dense over (H, D) with identical strides")
+    rc = _load().f3d_buck_swin_bwd_strided(
         _ptr(Q), _ptr(K), _ptr(V), _u32(Q.stride(1)), _ptr(O), _ptr(dO), _ptr(LSE), _ptr(Delta), _ptr(dQ), _ptr(dK),
-        _ptr(dV), _ptr(Scope_buckets), _u32(Scope_buckets.shape[0]), _u32(Scope_buckets.shape[1]), _u32(bucket_size),
+        _ptr(dV), _u32(dQ.stride(1)), _ptr(Scope_buckets), _u32(Scope_buckets.shape[0]), _u32(Scope_buckets.shape[1]), _u32(bucket_size),
         _u32(B), _u32(Ls), _u32(H), _u32(D), _ptr(kv_len), _i32(dev), _stream(dev))
     if rc == 2:   # F3D_ERR_UNSUPPORTED: a shape outside the backward kernels
         raise NotImplementedError(_load().f3d_last_error().decode("utf-8", "replace"))

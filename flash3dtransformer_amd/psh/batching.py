@@ -66,7 +66,7 @@ def host_facts(seps: torch.Tensor) -> dict:
     if hit is not None and hit[0]() is seps and hit[1] == seps._version:
         return hit[2]
     facts = {}
-    _HOST_FACTS[key] = (weakref.ref(seps, lambda _r, k=key: _HOST_FACTS.pop(k, None)), seps._version, facts)
+    _HOST_FACTS[key] = (weakref.ref(seps, lambda _r, k=key, d=_HOST_FACTS: d.pop(k, None)), seps._version, facts)
     return facts
 
 

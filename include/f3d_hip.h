@@ -206,6 +206,16 @@ int f3d_buck_swin_bwd(const f3d_bf16_t* q, const f3d_bf16_t* k, const f3d_bf16_t
                       uint32_t scope_size, uint32_t bucket_size, uint32_t batch, uint32_t seq_len, uint32_t num_head,
                       uint32_t head_dim, const int32_t* kv_len, int device, void* stream);
 
+/* The same with dq, dk, dv rows `grad_row_stride` elements apart (each still dense over num_head * head_dim), e.g. the
+ * three thirds of one [batch, seq_len, 3 * num_head * head_dim] gradient of the qkv projection output, which spares
+ * the concatenation that torch's autograd would otherwise make of three dense tensors. */
+int f3d_buck_swin_bwd_strided(const f3d_bf16_t* q, const f3d_bf16_t* k, const f3d_bf16_t* v, uint32_t qkv_row_stride,
+                              const f3d_bf16_t* o, const f3d_bf16_t* d_o, const float* lse, float* delta,
+                              f3d_bf16_t* dq, f3d_bf16_t* dk, f3d_bf16_t* dv, uint32_t grad_row_stride,
+                              const uint32_t* scope_buckets, uint32_t num_scope, uint32_t scope_size,
+                              uint32_t bucket_size, uint32_t batch, uint32_t seq_len, uint32_t num_head,
+                              uint32_t head_dim, const int32_t* kv_len, int device, void* stream);
+
 /* ---- bucketed attention forward: buck_swin_fwd, declared src/f3d_frontend.cu:90-92, called from
  *      flash3dxfmr/layers/buck_swin.py:57 (kernel source absent from the reference) --------------
  * q,k,v,o [batch,seq_len,num_head,head_dim] bf16 contiguous; lse [batch,seq_len,num_head] fp32;

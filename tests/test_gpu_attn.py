@@ -207,7 +207,8 @@ def test_attention_argument_errors():
 # ---------------------------------------------------------------------------------------------
 
 def _run_bwd(Q, K, V, dO, scopes, bs, fused_buffer=False, kv_len=None):
-    """forward then backward through the C ABI; Q/K/V optionally as column slices of one [B,L,3HD] buffer"""
+    """forward then backward through the C ABI; Q/K/V optionally as column slices of one [B,L,3HD] buffer, and then
+    dQ/dK/dV as the column slices of one [B,L,3HD] gradient buffer"""
     from flash3dtransformer_amd.lib import pshattn
     B, L, H, D = Q.shape
     if fused_buffer:
@@ -220,7 +221,11 @@ def _run_bwd(Q, K, V, dO, scopes, bs, fused_buffer=False, kv_len=None):
     sc = torch.from_numpy(np.ascontiguousarray(scopes, dtype=np.uint32).view(np.int32)).to(DEV).view(torch.uint32)
     kl = None if kv_len is None else torch.from_numpy(np.asarray(kv_len, dtype=np.int32)).to(DEV)
     pshattn.buck_swin_fwd(q, k, v, O, LSE, sc, bs, kv_len=kl)
-    dq, dk, dv = [torch.zeros(B, L, H, D, dtype=torch.bfloat16, device=DEV) for _ in range(3)]
+    if fused_buffer:
+        dqkv = torch.zeros(B, L, 3 * H * D, dtype=torch.bfloat16, device=DEV)
+        dq, dk, dv = [t.view(B, L, H, D) for t in dqkv.chunk(3, dim=-1)]
+    else:
+        dq, dk, dv = [torch.zeros(B, L, H, D, dtype=torch.bfloat16, device=DEV) for _ in range(3)]
     delta = torch.zeros(B, L, H, dtype=torch.float32, device=DEV)
     pshattn.buck_swin_bwd(q, k, v, O, dO.to(DEV), LSE, delta, dq, dk, dv, sc, bs, kv_len=kl)
     torch.cuda.synchronize()
@@ -326,6 +331,25 @@ def test_backward_leaves_uncovered_rows_untouched(oracle):
         assert not t[:, 512:1024].any() and not t[:, 1536:].any()
     wq, wk, wv, _ = oracle.buck_swin_bwd(Q, K, V, dO, scopes, bs)
     _check_grads((dq, dk, dv), (wq, wk, wv), "partial cover")
+
+
+def test_attention_over_one_projection_output_matches_three_tensors():
+    """BuckSwinQKVFunction (one [B,L,3C] tensor in, one gradient tensor out) gives the bits of the three-tensor function"""
+    from flash3dtransformer_amd.layers.buck_swin import BucketSwinAttention, BuckSwinQKVFunction
+    B, L, H, D, bs = 2, 2048, 4, 32, 512
+    g = torch.Generator().manual_seed(17)
+    qkv = torch.randn(B, L, 3 * H * D, generator=g).to(torch.bfloat16).to(DEV)
+    w = torch.randn(B, L, H, D, generator=g).to(torch.bfloat16).to(DEV)
+    sc = torch.from_numpy(np.arange(L // bs, dtype=np.uint32).reshape(-1, 1).view(np.int32)).to(DEV).view(torch.uint32)
+    a = qkv.clone().requires_grad_(True)
+    O1 = BuckSwinQKVFunction.apply(a, sc, bs, H)
+    (O1.float() * w.float()).sum().backward()
+    b = qkv.clone().requires_grad_(True)
+    q, k, v = (t.view(B, L, H, D) for t in torch.chunk(b, 3, dim=-1))
+    O2 = BucketSwinAttention(bs)(q, k, v, sc)
+    (O2.float() * w.float()).sum().backward()
+    assert torch.equal(O1, O2) and torch.equal(a.grad, b.grad)
+    assert a.grad.abs().max().item() > 0
 
 
 def test_attention_module_backpropagates(oracle):
