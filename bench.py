@@ -318,6 +318,28 @@ def sub_backward(dev, out):
                 f(xin)
         out[f"layer_fwd_bwd_{name}"] = {"fwd_ms": round(ev_time(fwd, 5), 4), "fwd_bwd_ms": round(ev_time(step, 5), 4)}
         del xin, gy
+    del qkv, proj, mlp, ln
+    torch.cuda.empty_cache()
+    # forward + backward of the whole 5-level hourglass (config 5: 4 sweeps x 250,000 points), training mode, fp32
+    # master weights (their bf16 copies are made anew every step), loss = mean of squares; wall time per step
+    from flash3dtransformer_amd import configs
+    model = configs.hourglass(1005).to(dev).train()
+    coords_np, seps_np, _ = configs.lidar_batch(4, 250_000, 1005)
+    coords, seps = configs.to_device(coords_np, seps_np, dev)
+
+    def train_step():
+        for p_ in model.parameters():
+            p_.grad = None
+        (model(coords, None, seps).float() ** 2).mean().backward()
+    for _ in range(2):
+        train_step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(3):
+        train_step()
+    torch.cuda.synchronize()
+    out["hourglass_c5_fwd_bwd"] = {"ms": round((time.perf_counter() - t0) / 3 * 1e3, 2), "points": 1_000_000}
+    del model, coords, seps
     torch.cuda.empty_cache()
 
 

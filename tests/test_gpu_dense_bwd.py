@@ -4,6 +4,7 @@ autograd supply them: flash3dxfmr/layers/buck_swin.py:159-163, elem_wise.py:22-2
 fp64 / fp32 torch on the same bf16-rounded inputs.  Tolerances: the weight gradient is an fp32 sum of exact bf16
 products, so it matches the fp64 result to fp32 accumulation noise (1e-5 of the largest entry); bf16 outputs carry one
 bf16 rounding (2^-8 relative) on top of fp32 arithmetic."""
+import numpy as np
 import pytest
 import torch
 
@@ -43,6 +44,23 @@ def test_linear_wgrad_matches_fp64(M, N, K):
     pshattn.linear_wgrad_bf16(dy, x, dw2, db, accumulate=True)
     assert (dw2.double() - 2 * ref_w).abs().max().item() <= 2e-5 * ref_w.abs().max().item() + 1e-6
     assert (db.double() - 2 * ref_b).abs().max().item() <= 2e-5 * ref_b.abs().max().item() + 1e-6
+
+
+def test_linear_wgrad_random_shapes():
+    """shapes drawn at random (multiples of 8 in n and k, any row count), one of the operands a column slice"""
+    from flash3dtransformer_amd.lib import pshattn
+    rng = np.random.default_rng(2024)
+    for it in range(16):
+        M = int(rng.integers(1, 40000))
+        N, K = int(rng.integers(1, 80)) * 8, int(rng.integers(1, 80)) * 8
+        dy = _rand((M, N + 8), it, 0.5).to(DEV)[:, 8:]
+        x = _rand((M, K), 100 + it).to(DEV)
+        dw = torch.full((N, K), float("nan"), dtype=torch.float32, device=DEV)
+        db = torch.full((N,), float("nan"), dtype=torch.float32, device=DEV)
+        pshattn.linear_wgrad_bf16(dy, x, dw, db)
+        ref_w, ref_b = dy.double().t() @ x.double(), dy.double().sum(0)
+        assert (dw.double() - ref_w).abs().max().item() <= 1e-5 * ref_w.abs().max().item() + 1e-6, (M, N, K)
+        assert (db.double() - ref_b).abs().max().item() <= 1e-5 * ref_b.abs().max().item() + 1e-6, (M, N, K)
 
 
 def test_linear_wgrad_strided_operands_and_empty_input():

@@ -119,10 +119,12 @@ def test_unsupported_attention_backward_says_so():
                               f(B, Ls, H), z(B, Ls, H, D), z(B, Ls, H, D), z(B, Ls, H, D), sc, 512)
 
 
-@pytest.mark.parametrize("act,use_ln,use_res", [(None, False, True), ("gelu", True, False), ("swiglu", True, True)])
+@pytest.mark.parametrize("act,use_ln,use_res", [(None, False, True), (None, True, True), (None, True, False),
+                                                ("gelu", True, False), ("swiglu", True, True)])
 def test_dense_layer_gradients_vs_torch(act, use_ln, use_res):
-    """Linear (+ LayerNorm in front, activation, residual): forward from the HIP kernels, gradients through the
-    torch restatement; both against plain torch autograd in fp32 on the same bf16 inputs"""
+    """Linear (+ LayerNorm in front, activation, residual): forward from the HIP kernels, gradients from the HIP
+    backward kernels (no activation) or through the torch restatement (with one); both against plain torch autograd in
+    fp32 on the same bf16 inputs"""
     from flash3dtransformer_amd import layers as L
     torch.manual_seed(5)
     M, K, N = 300, 64, 128
@@ -153,9 +155,12 @@ def test_dense_layer_gradients_vs_torch(act, use_ln, use_res):
     assert (y.float().cpu() - yr).abs().max().item() <= 2e-2 * max(1.0, yr.abs().max().item())
     close = lambda a, b, tol: (a.float().cpu() - b).abs().max().item() <= tol * max(1.0, b.abs().max().item())
     assert close(x.grad, xr.grad, 1e-2)            # bf16 gradient tensor
-    assert close(lin.weight.grad, wr.grad, 1e-3) and close(lin.bias.grad, br.grad, 1e-3)
+    # the HIP backward behind a LayerNorm multiplies bf16 operands (LayerNorm(x) and dh rounded to bf16, 2^-9 relative
+    # each, as TransformerEngine's backward GEMMs do); the restatement and the LayerNorm-free case have exact operands
+    wtol = 1e-2 if (use_ln and act is None) else 1e-3
+    assert close(lin.weight.grad, wr.grad, wtol) and close(lin.bias.grad, br.grad, 1e-3)
     if use_ln:
-        assert close(ln.weight.grad, gr.grad, 1e-3) and close(ln.bias.grad, ber.grad, 1e-3)
+        assert close(ln.weight.grad, gr.grad, wtol) and close(ln.bias.grad, ber.grad, wtol)
     if use_res:
         assert close(res.grad, rr.grad, 1e-2)
 
