@@ -222,14 +222,22 @@ __global__ __launch_bounds__(kWgThreads) void linear_wgrad_kernel(
   }
 }
 
-// out[i] = (accumulate ? out[i] : 0) + sum over p of part[p][i].  A workgroup owns 256 consecutive elements (64 lanes x
-// 4 floats, len % 4 == 0); its 16 partial groups each sum every 16th partial (independent 16-byte loads), then the
-// first group adds the 16 group sums in ascending order: a fixed summation tree.
-__global__ __launch_bounds__(1024) void sum_partials_kernel(const float* __restrict__ part, uint32_t n_part, size_t len,
-                                                            float* __restrict__ out, uint32_t accumulate) {
+// out[i] = (accumulate ? out[i] : 0) + sum over p of part[p][i], for two arrays in one launch (the weight gradient and,
+// in the workgroups past blocks_a, the bias gradient; len_b may be 0).  A workgroup owns 256 consecutive elements (64
+// lanes x 4 floats, lengths are multiples of 4); its 16 partial groups each sum every 16th partial (independent 16-byte
+// loads), then the first group adds the 16 group sums in ascending order: a fixed summation tree.
+__global__ __launch_bounds__(1024) void sum_partials_kernel(const float* __restrict__ part_a, size_t len_a,
+                                                            float* __restrict__ out_a, uint32_t blocks_a,
+                                                            const float* __restrict__ part_b, size_t len_b,
+                                                            float* __restrict__ out_b, uint32_t n_part,
+                                                            uint32_t accumulate) {
   __shared__ float4 s_sum[16][64];
+  const bool second = blockIdx.x >= blocks_a;
+  const float* part = second ? part_b : part_a;
+  float* out = second ? out_b : out_a;
+  const size_t len = second ? len_b : len_a;
   const uint32_t tid = threadIdx.x, l = tid & 63u, g = tid >> 6;
-  const size_t i = ((size_t)blockIdx.x * 64u + l) * 4u;
+  const size_t i = ((size_t)(blockIdx.x - (second ? blocks_a : 0u)) * 64u + l) * 4u;
   float4 s = {0.f, 0.f, 0.f, 0.f};
   if (i < len)
     for (uint32_t p = g; p < n_part; p += 16u) {
@@ -442,11 +450,9 @@ int f3d_linear_wgrad_bf16(const f3d_bf16_t* dy, uint32_t lddy, const f3d_bf16_t*
   const uint32_t n_items = tiles * slabs, items_per_xcd = cdiv_u32(n_items, kXcd);
   hipLaunchKernelGGL(linear_wgrad_kernel, dim3(items_per_xcd * kXcd), dim3(kWgThreads), kWgLds, s, dy, lddy, x, ldx,
                      part_w, part_b, m, n, k, n_tiles, k_tiles, slabs, slab_rows, items_per_xcd);
-  hipLaunchKernelGGL(sum_partials_kernel, dim3((uint32_t)((nk + 255) / 256)), dim3(1024), 0, s, part_w, slabs, nk, dw,
-                     accumulate);
-  if (db)
-    hipLaunchKernelGGL(sum_partials_kernel, dim3(cdiv_u32(n, 256)), dim3(1024), 0, s, part_b, slabs, (size_t)n, db,
-                       accumulate);
+  const uint32_t blocks_w = (uint32_t)((nk + 255) / 256), blocks_b = db ? cdiv_u32(n, 256) : 0u;
+  hipLaunchKernelGGL(sum_partials_kernel, dim3(blocks_w + blocks_b), dim3(1024), 0, s, part_w, nk, dw, blocks_w, part_b,
+                     db ? (size_t)n : (size_t)0, db, slabs, accumulate);
   F3D_CHECK_HIP(hipGetLastError());
   return F3D_OK;
 }
