@@ -56,8 +56,9 @@ class BuckSwinQKVFunction(Function):
         B, L, H, D = O.shape
         Q, K, V = (t.view(B, L, H, D) for t in torch.chunk(qkv, 3, dim=-1))
         dO = grad_output if grad_output.dtype == torch.bfloat16 else grad_output.to(torch.bfloat16)
-        # zero-filled: rows that no scope covers are not written
-        dqkv = torch.zeros_like(qkv)
+        # rows that no scope covers are not written: zero-filled unless the planner vouches that its table covers all
+        covered = getattr(ctx.scope_buckets, "covers_all_rows", False)
+        dqkv = torch.empty_like(qkv) if covered else torch.zeros_like(qkv)
         dQ, dK, dV = (t.view(B, L, H, D) for t in torch.chunk(dqkv, 3, dim=-1))
         delta = torch.zeros(B, L, H, dtype=torch.float32, device=O.device)
         pshattn.buck_swin_bwd(Q, K, V, O, dO.contiguous(), lse, delta, dQ, dK, dV, ctx.scope_buckets, ctx.buck_size)

@@ -83,5 +83,7 @@ class SwinPlan:
                     f"(bucket {self.buck_size} x scope {self.scope_size_in_buck}): falling back to ONE global "
                     f"attention scope of {sz} buckets (quadratic cost)")
             hit = torch.arange(ns * sz, dtype=torch.int32).view(ns, sz).to(device).view(torch.uint32)
+            # every bucket of the buffer sits in exactly one scope: ops that write only covered rows write all rows
+            hit.covers_all_rows = True
             _SCOPE_CACHE[key] = hit
         return hit

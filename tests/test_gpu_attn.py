@@ -350,6 +350,21 @@ def test_attention_over_one_projection_output_matches_three_tensors():
     (O2.float() * w.float()).sum().backward()
     assert torch.equal(O1, O2) and torch.equal(a.grad, b.grad)
     assert a.grad.abs().max().item() > 0
+    # a table from the planner covers every row, so the gradient buffer is not zero-filled first: poison the block the
+    # allocator will hand out and check that every element was written
+    from flash3dtransformer_amd.psh.bucket_scope import SwinPlan
+    sc2 = SwinPlan("swin", bs, 1, 0).gen_scopes_from_plan(B * L, DEV)
+    assert getattr(sc2, "covers_all_rows", False) and tuple(sc2.shape) == (B * L // bs, 1)
+    c = qkv.clone().requires_grad_(True)
+    O3 = BuckSwinQKVFunction.apply(c.view(1, B * L, -1), sc2, bs, H)
+    poison = torch.full((B * L * 3 * H * D,), float("nan"), dtype=torch.bfloat16, device=DEV)
+    del poison
+    (O3.view(B, L, H, D).float() * w.float()).sum().backward()
+    a2 = qkv.clone().requires_grad_(True)
+    sc1 = torch.from_numpy(np.arange(B * L // bs, dtype=np.uint32).reshape(-1, 1).view(np.int32)).to(DEV).view(torch.uint32)
+    O4 = BuckSwinQKVFunction.apply(a2.view(1, B * L, -1), sc1, bs, H)
+    (O4.view(B, L, H, D).float() * w.float()).sum().backward()
+    assert torch.isfinite(c.grad).all() and torch.equal(c.grad, a2.grad)
 
 
 def test_attention_module_backpropagates(oracle):
