@@ -241,7 +241,8 @@ class _LinearGrad(torch.autograd.Function):
 class _GatedMLPGrad(torch.autograd.Function):
     """y = fc2(silu(z1) * z2) + b2 (+ residual), [z1 | z2] = LayerNorm(x) @ w1.T + b1, computed by the HIP forward.
     The backward recomputes LayerNorm(x) and z (the forward keeps neither), then runs
-    da = dy @ w2, (dz, a) = gate backward in place, dw2 = dy.T a, dw1 = dz.T h, dh = dz @ w1, LayerNorm backward.
+    da = dy @ w2, (dz, a) = gate backward (these three in one kernel at widths 128 and 256), dw2 = dy.T a, dw1 = dz.T h,
+    dh = dz @ w1, LayerNorm backward.
     When the residual is the layer's own input, its gradient dy is added to dx inside the LayerNorm backward."""
 
     @staticmethod
@@ -263,12 +264,14 @@ class _GatedMLPGrad(torch.autograd.Function):
         f32 = dict(dtype=torch.float32, device=dev)
         h = torch.empty(m, c, **bf)
         pshattn.layernorm_bf16(x2, g16, be16, h, ctx.eps)
-        z = torch.empty(m, 2 * hid, **bf)
-        pshattn.linear_bf16(h, w1_16, b1_16, None, z, None)
-        da = torch.empty(m, hid, **bf)
-        pshattn.linear_bf16(dy2, _transposed_bf16(w2_16), None, None, da, None)
-        pshattn.swiglu_bwd_bf16(z, da, z, da)          # z <- dz, da <- a
-        dz, a = z, da
+        dz, a = torch.empty(m, 2 * hid, **bf), torch.empty(m, hid, **bf)
+        w2t = _transposed_bf16(w2_16)
+        # one kernel where it exists (fc1 recomputed, da = dy @ w2 and the gate backward; neither z nor da is stored) ...
+        if not pshattn.mlp_gate_bwd_bf16(h, dy2, w1_16, b1_16, w2t, dz, a):
+            # ... otherwise fc1, da, then the gate backward in place (dz over z, a over da)
+            pshattn.linear_bf16(h, w1_16, b1_16, None, dz, None)
+            pshattn.linear_bf16(dy2, w2t, None, None, a, None)
+            pshattn.swiglu_bwd_bf16(dz, a, dz, a)
         dw2, db2 = torch.empty(c, hid, **f32), torch.empty(c, **f32)
         pshattn.linear_wgrad_bf16(dy2, a, dw2, db2)
         dw1, db1 = torch.empty(2 * hid, c, **f32), torch.empty(2 * hid, **f32)

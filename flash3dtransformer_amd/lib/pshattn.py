@@ -628,6 +628,29 @@ def swiglu_bwd_bf16(z, da, dz, a=None):
                                        _u32(m), _u32(h), _i32(dev), _stream(dev)))
 
 
+def mlp_gate_bwd_bf16(h, dy, w1, b1, w2t, dz, a):
+    """extension: (dz, a) of the gated MLP's backward from h = LayerNorm(x), dy, w1 [2 hidden, c], b1, w2t = w2.T
+    [hidden, c]: fc1 recomputed, da = dy @ w2 and the gate backward in one kernel.  Returns False (nothing written)
+    when that kernel does not cover the shape."""
+    dev = assert_same_device([h, dy, w1, w2t, dz, a])
+    _rows2d([h, dy, dz, a])
+    assert_dtype([w1, w2t], torch.bfloat16)
+    assert_contiguous([w1, w2t])
+    _check_vectors(h, [b1])
+    m, c = h.shape
+    hid = w2t.shape[0]
+    if tuple(dy.shape) != (m, c) or tuple(w1.shape) != (2 * hid, c) or tuple(w2t.shape) != (hid, c) \
+            or tuple(dz.shape) != (m, 2 * hid) or tuple(a.shape) != (m, hid) or (b1 is not None and tuple(b1.shape) != (2 * hid,)):
+        raise RuntimeError("mlp_gate_bwd shape mismatch")
+    rc = _load().f3d_mlp_gate_bwd_bf16(_ptr(h), _u32(h.stride(0)), _ptr(dy), _u32(dy.stride(0)), _ptr(w1), _ptr(b1),
+                                       _ptr(w2t), _ptr(dz), _u32(dz.stride(0)), _ptr(a), _u32(a.stride(0)), _u32(m),
+                                       _u32(c), _u32(hid), _i32(dev), _stream(dev))
+    if rc == 2:
+        return False
+    _check(rc)
+    return True
+
+
 def coord_embed_bf16(coord, w, bias, y):
     """extension: y = bf16(coord) @ w.T + bias for w [C,3] (PSH3DCoordEmbedding, psh_ops.py:64-67)"""
     assert_contiguous([coord, w, y])

@@ -135,6 +135,35 @@ def test_swiglu_backward_matches_autograd(M, H):
     assert torch.equal(z2, dz) and torch.equal(da2, a)
 
 
+@pytest.mark.parametrize("M,C,H", [(3001, 256, 1024), (70000, 256, 512), (777, 128, 96), (20000, 128, 512), (256, 256, 32)])
+def test_fused_gate_backward_matches_autograd(M, C, H):
+    """fc1 recomputed + da = dy w2 + gate backward in one kernel, against fp32 autograd of a = silu(z1) * z2 with
+    z = h w1^T + b1 and the upstream gradient da = dy w2 (bf16 outputs: one rounding on top of fp32 arithmetic)"""
+    from flash3dtransformer_amd.lib import pshattn
+    h, dy = _rand((M, C), M + C).to(DEV), _rand((M, C), 2 * M + C, 0.5).to(DEV)
+    w1, w2 = _rand((2 * H, C), C + H, C ** -0.5).to(DEV), _rand((C, H), C + 2 * H, H ** -0.5).to(DEV)
+    b1 = _rand((2 * H,), 7, 0.5).to(DEV)
+    dz = torch.full((M, 2 * H), float("nan"), dtype=torch.bfloat16, device=DEV)
+    a = torch.full((M, H), float("nan"), dtype=torch.bfloat16, device=DEV)
+    assert pshattn.mlp_gate_bwd_bf16(h, dy, w1, b1, w2.t().contiguous(), dz, a)
+    zr = (h.float() @ w1.float().t() + b1.float()).requires_grad_(True)
+    ar = torch.nn.functional.silu(zr[:, :H]) * zr[:, H:]
+    ar.backward(dy.float() @ w2.float())
+    for got, want in ((a, ar.detach()), (dz, zr.grad)):
+        err = (got.float() - want).abs()
+        assert (err <= 2e-2 * want.abs().clamp(min=1.0)).all(), err.max().item()
+    # no bias; widths outside the kernel are refused without touching the outputs
+    assert pshattn.mlp_gate_bwd_bf16(h, dy, w1, None, w2.t().contiguous(), dz, a)
+    zr = (h.float() @ w1.float().t()).requires_grad_(True)
+    (torch.nn.functional.silu(zr[:, :H]) * zr[:, H:]).backward(dy.float() @ w2.float())
+    err = (dz.float() - zr.grad).abs()
+    assert (err <= 2e-2 * zr.grad.abs().clamp(min=1.0)).all(), err.max().item()
+    a.fill_(5.0)
+    assert not pshattn.mlp_gate_bwd_bf16(h[:, :64].contiguous(), dy[:, :64].contiguous(), w1[:, :64].contiguous(), b1,
+                                         w2[:64].t().contiguous(), dz, a)
+    assert (a == 5.0).all()
+
+
 def test_gated_mlp_layer_gradients_vs_autograd():
     """LayerNormMLP with the residual taken from its own input (the way a block calls it): every gradient against
     fp32 torch autograd of the same formula.  The gradient tensors handed from kernel to kernel (da, dz, dh) are bf16 as
