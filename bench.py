@@ -297,6 +297,15 @@ def sub_backward(dev, out):
     gbs = M * C * 6.0 / ms / 1e6
     out["layernorm_bwd_256"] = {"ms": round(ms, 4), "gbs": round(gbs, 1), "frac_of_hbm_peak": round(gbs / HBM_PEAK_GBS, 4)}
     del x, dh, dx
+    # fc1 recomputation + da = dy w2 + gate backward in one kernel: 2 M C 3 H flops, reads h and dy, writes dz and a
+    hh, dyy = rnd(M, C), rnd(M, C)
+    w1, w2t, b1 = rnd(2 * HID, C) / 16, rnd(HID, C) / 16, rnd(2 * HID)
+    dz, aa = torch.empty(M, 2 * HID, dtype=torch.bfloat16, device=dev), torch.empty(M, HID, dtype=torch.bfloat16, device=dev)
+    ms = ev_time(lambda: pshattn.mlp_gate_bwd_bf16(hh, dyy, w1, b1, w2t, dz, aa), 10)
+    tf, gbs = 6.0 * M * C * HID / ms / 1e9, (2.0 * M * C * 2 + 3.0 * M * HID * 2) / ms / 1e6
+    out["mlp_gate_bwd_256x1024"] = {"ms": round(ms, 4), "tflops": round(tf, 1), "frac_of_bf16_mfma_peak": round(tf / MFMA_BF16_PEAK_TFLOPS, 4),
+                                    "gbs": round(gbs, 1), "frac_of_hbm_peak": round(gbs / HBM_PEAK_GBS, 4)}
+    del hh, dyy, dz, aa
     z, da = rnd(M, 2 * HID), rnd(M, HID)
     ms = ev_time(lambda: pshattn.swiglu_bwd_bf16(z, da, z, da), 10)
     gbs = M * HID * 12.0 / ms / 1e6
