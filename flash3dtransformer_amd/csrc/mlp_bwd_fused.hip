@@ -26,7 +26,7 @@ constexpr int kGbWaves = 8;
 template <int K>
 struct GbGeom {
   static constexpr int ROWB = K * 2;                  // bytes per weight row
-  static constexpr int CPR = K / 8;                   // 16-byte pieces per weight row (16 or 32)
+  static constexpr int CPR = K / 8;                   // 16-byte pieces per weight row (4, 8, 16 or 32)
   static constexpr int RPI = 1024 / ROWB;             // weight rows one direct load fills
   static constexpr int CHUNK = 96 * ROWB;             // value + gate + w2^T rows of 32 hidden features
   static constexpr int N_DMA = CHUNK / 1024;
@@ -36,7 +36,13 @@ struct GbGeom {
   static constexpr size_t loop_bytes() { return (size_t)2 * SLOT + (size_t)kGbWaves * 32 * kPatchRow * 2; }
   static constexpr size_t prologue_bytes() { return (size_t)kGbWaves * 32 * PROW * 2; }
   static constexpr size_t lds_bytes() { return loop_bytes() > prologue_bytes() ? loop_bytes() : prologue_bytes(); }
-  static_assert(N_DMA % kGbWaves == 0 && 32 % RPI == 0, "every wave issues the same number of direct loads");
+  static constexpr int MY_DMA_MAX = (N_DMA + kGbWaves - 1) / kGbWaves;
+  // 16 consecutive rows read at one piece index must fall into 16 different 16-byte slots of the 256 bank bytes: rows
+  // that share their offset modulo 256 get different swizzle values
+  static constexpr int RP = CPR >= 16 ? 1 : 16 / CPR;     // rows sharing one swizzle value
+  static constexpr int SWZ_MASK = (CPR < 16 ? CPR : 16) - 1;
+  __host__ __device__ static constexpr uint32_t swz(uint32_t row) { return (row / RP) & SWZ_MASK; }
+  static_assert(32 % RPI == 0 && 1024 % ROWB == 0, "a direct load fills whole rows of one weight block");
 };
 
 // 32 rows [row0, row0 + 32) of a row-major [M, K] tensor -> the wave's registers in B-operand layout: f[ks] of lane
@@ -73,12 +79,12 @@ __device__ __forceinline__ void load_rows_b(const uint16_t* __restrict__ src, ui
 // h [M, K] (LayerNorm output), dy [M, K], w1 [2 H, K] (value rows, then gate rows), b1 [2 H] or null, w2t [H, K] (w2
 // transposed); a [M, H], dz [M, 2 H].  H a multiple of 32.
 template <int K>
-__global__ __launch_bounds__(64 * kGbWaves) __attribute__((amdgpu_waves_per_eu(2, 2))) void mlp_gate_bwd_kernel(
+__global__ __launch_bounds__(64 * kGbWaves) __attribute__((amdgpu_waves_per_eu(2))) void mlp_gate_bwd_kernel(
     const uint16_t* __restrict__ h, uint32_t ldh, const uint16_t* __restrict__ dy, uint32_t lddy,
     const uint16_t* __restrict__ w1, const uint16_t* __restrict__ b1, const uint16_t* __restrict__ w2t,
     uint16_t* __restrict__ dz, uint32_t lddz, uint16_t* __restrict__ a, uint32_t lda, uint32_t M, uint32_t H) {
   using G = GbGeom<K>;
-  constexpr int KS = K / 16, ROWB = G::ROWB, WAVES = kGbWaves, ROWS_WG = 32 * WAVES, MY_DMA = G::N_DMA / WAVES;
+  constexpr int KS = K / 16, ROWB = G::ROWB, WAVES = kGbWaves, ROWS_WG = 32 * WAVES;
   extern __shared__ __attribute__((aligned(1024))) char lds_gb[];
   char* wbuf = lds_gb;                                                       // two chunk buffers (+ bias slots)
   uint16_t* patch = reinterpret_cast<uint16_t*>(lds_gb + 2 * G::SLOT);       // epilogue patches, one per wave
@@ -104,10 +110,11 @@ __global__ __launch_bounds__(64 * kGbWaves) __attribute__((amdgpu_waves_per_eu(2
   const uint32_t nchunk = H / 32;
   auto dma_chunk = [&](uint32_t c, uint32_t slot) {
 #pragma unroll
-    for (int i = 0; i < MY_DMA; ++i) {
+    for (int i = 0; i < G::MY_DMA_MAX; ++i) {
       const uint32_t q = wave + i * WAVES;
+      if (q >= (uint32_t)G::N_DMA) break;                       // wave-uniform
       const uint32_t lr = q * G::RPI + lane / G::CPR;           // row of the chunk: 0-31 value, 32-63 gate, 64-95 w2^T
-      const uint32_t piece = (lane % G::CPR) ^ (lr & 15u);      // the piece that belongs at this lane's LDS position
+      const uint32_t piece = (lane % G::CPR) ^ G::swz(lr);      // the piece that belongs at this lane's LDS position
       const uint32_t blk = __builtin_amdgcn_readfirstlane(q * G::RPI / 32u);
       const uint16_t* base = blk == 2 ? w2t : w1;
       const uint32_t grow = (blk == 1 ? H : 0u) + c * 32u + (lr & 31u);
@@ -118,7 +125,7 @@ __global__ __launch_bounds__(64 * kGbWaves) __attribute__((amdgpu_waves_per_eu(2
     if (wave == 0 && b1) xs_lds_dma2(b1, ((lane < 32u ? 0u : H - 32u) + c * 32u + lane) * 2u, wbuf + slot * G::SLOT + G::CHUNK);
   };
   // A operand of tile block t (0 value, 1 gate, 2 w2^T), k-step ks: row lq of the block, 16-byte piece 2 ks + half
-  const uint32_t a_row = lq * ROWB, a_swz = lq & 15u;
+  const uint32_t a_row = lq * ROWB, a_swz = G::swz(lq);   // block offsets (32 rows) leave the swizzle value unchanged
   auto a_frag = [&](const char* buf, int t, int ks) -> bf16x8_t {
     return *reinterpret_cast<const bf16x8_t*>(buf + t * 32 * ROWB + a_row + (((uint32_t)(2 * ks) + half) ^ a_swz) * 16u);
   };
@@ -126,8 +133,8 @@ __global__ __launch_bounds__(64 * kGbWaves) __attribute__((amdgpu_waves_per_eu(2
   dma_chunk(0, 0);
   for (uint32_t c = 0; c < nchunk; ++c) {
     const uint32_t slot = c & 1u;
-    // chunk c has landed when at most the stores of the previous epilogue (6 per wave, issued after its requests) are
-    // outstanding; where some stores may be skipped (rows past M) everything is waited for
+    // chunk c has landed when at most the stores of the previous epilogue (6 per wave, issued after its requests, however
+    // many of those the wave has) are outstanding; where some stores may be skipped (rows past M) everything is waited for
     if (wg_full && c > 0) xs_wait_vm(6); else __builtin_amdgcn_s_waitcnt(0x0F70);
     wg_barrier_lds();   // every wave's part of chunk c is in LDS; every wave is done reading chunk c - 1
     if (c + 1 < nchunk) dma_chunk(c + 1, slot ^ 1u);
@@ -232,9 +239,10 @@ extern "C" int f3d_mlp_gate_bwd_bf16(const f3d_bf16_t* h, uint32_t ldh, const f3
                                      uint32_t hidden, int device, void* stream) {
   using namespace f3d;
   F3D_CHECK_ARG(h && dy && w1 && w2t && dz && a, "null tensor pointer");
-  if (!(c == 128 || c == 256) || hidden == 0 || hidden % 32 != 0 || (uint64_t)hidden * c * 4 >= (1ull << 32)) {
-    set_error("No kernel found for the fused gate backward at width %u, hidden %u (widths 128 and 256, hidden a multiple "
-              "of 32)", c, hidden);
+  if (!(c == 32 || c == 64 || c == 128 || c == 256) || hidden == 0 || hidden % 32 != 0 ||
+      (uint64_t)hidden * c * 4 >= (1ull << 32)) {
+    set_error("No kernel found for the fused gate backward at width %u, hidden %u (widths 32, 64, 128 and 256, hidden a "
+              "multiple of 32)", c, hidden);
     return F3D_ERR_UNSUPPORTED;
   }
   F3D_CHECK_ARG(ldh >= c && ldh % 8 == 0 && lddy >= c && lddy % 8 == 0 && lddz >= 2 * hidden && lddz % 8 == 0 &&
@@ -248,8 +256,13 @@ extern "C" int f3d_mlp_gate_bwd_bf16(const f3d_bf16_t* h, uint32_t ldh, const f3
   F3D_CHECK_ARG(guard.ok, "cannot select device %d", device);
   hipStream_t s = (hipStream_t)stream;
   SyncBracket sync(s);
-  const int rc = c == 128 ? launch_gate_bwd<128>(h, ldh, dy, lddy, w1, b1, w2t, dz, lddz, a, lda, m, hidden, device, s)
-                          : launch_gate_bwd<256>(h, ldh, dy, lddy, w1, b1, w2t, dz, lddz, a, lda, m, hidden, device, s);
+  int rc;
+  switch (c) {
+    case 32: rc = launch_gate_bwd<32>(h, ldh, dy, lddy, w1, b1, w2t, dz, lddz, a, lda, m, hidden, device, s); break;
+    case 64: rc = launch_gate_bwd<64>(h, ldh, dy, lddy, w1, b1, w2t, dz, lddz, a, lda, m, hidden, device, s); break;
+    case 128: rc = launch_gate_bwd<128>(h, ldh, dy, lddy, w1, b1, w2t, dz, lddz, a, lda, m, hidden, device, s); break;
+    default: rc = launch_gate_bwd<256>(h, ldh, dy, lddy, w1, b1, w2t, dz, lddz, a, lda, m, hidden, device, s); break;
+  }
   if (rc != F3D_OK) return rc;
   F3D_CHECK_HIP(hipGetLastError());
   return F3D_OK;

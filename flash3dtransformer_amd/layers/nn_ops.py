@@ -241,7 +241,7 @@ class _LinearGrad(torch.autograd.Function):
 class _GatedMLPGrad(torch.autograd.Function):
     """y = fc2(silu(z1) * z2) + b2 (+ residual), [z1 | z2] = LayerNorm(x) @ w1.T + b1, computed by the HIP forward.
     The backward recomputes LayerNorm(x) and z (the forward keeps neither), then runs
-    da = dy @ w2, (dz, a) = gate backward (these three in one kernel at widths 128 and 256), dw2 = dy.T a, dw1 = dz.T h,
+    da = dy @ w2, (dz, a) = gate backward (these three in one kernel at widths 32 to 256), dw2 = dy.T a, dw1 = dz.T h,
     dh = dz @ w1, LayerNorm backward.
     When the residual is the layer's own input, its gradient dy is added to dx inside the LayerNorm backward."""
 

@@ -335,7 +335,7 @@ int f3d_swiglu_bwd_bf16(const f3d_bf16_t* z, uint32_t ldz, const f3d_bf16_t* da,
 /* The middle of the gated MLP's backward in one kernel: with h = LayerNorm(x) [m,c], dy [m,c], w1 [2 hidden, c] (value
  * rows, then gate rows), b1 [2 hidden] or NULL and w2t = w2 transposed [hidden, c], it recomputes [z1 | z2] = h · w1ᵀ + b1,
  * forms da = dy · w2 and writes a = silu(z1) * z2 [m,hidden] and dz [m, 2 hidden] (as f3d_swiglu_bwd_bf16 defines them);
- * neither z nor da is stored.  c in {128, 256}, hidden a multiple of 32, else F3D_ERR_UNSUPPORTED (then: f3d_linear_bf16
+ * neither z nor da is stored.  c in {32, 64, 128, 256}, hidden a multiple of 32, else F3D_ERR_UNSUPPORTED (then: f3d_linear_bf16
  * twice and f3d_swiglu_bwd_bf16). */
 int f3d_mlp_gate_bwd_bf16(const f3d_bf16_t* h, uint32_t ldh, const f3d_bf16_t* dy, uint32_t lddy, const f3d_bf16_t* w1,
                           const f3d_bf16_t* b1, const f3d_bf16_t* w2t, f3d_bf16_t* dz, uint32_t lddz, f3d_bf16_t* a,
