@@ -52,3 +52,18 @@ def test_load_state_dict_drops_copies_and_accepts_extra_state():
     sd["_extra_state"] = None
     lin.load_state_dict(sd, strict=True)
     assert isinstance(lin, nn_ops._CachedParamModule)
+
+
+def test_planner_tables_cover_every_bucket_and_say_so():
+    """every plan of bucket_scope.py puts each bucket of the buffer into exactly one scope (reference:
+    flash3dxfmr/psh/bucket_scope.py:58-82); the cached table carries that fact for ops that write only covered rows"""
+    from flash3dtransformer_amd.psh.bucket_scope import SwinPlan
+    for plan, total, bs, sc in (("swin", 8192, 512, 1), ("swin", 16384, 512, 8), ("swin", 5 * 512, 512, 2),
+                                ("stride", 12 * 256, 256, 2)):
+        import warnings
+        with warnings.catch_warnings():
+            warnings.simplefilter("ignore")
+            t = SwinPlan(plan, bs, sc, 0 if plan == "swin" else 1).gen_scopes_from_plan(total, torch.device("cpu"))
+        assert getattr(t, "covers_all_rows", False)
+        ids = t.view(torch.int32).flatten().tolist()
+        assert sorted(ids) == list(range(total // bs))
