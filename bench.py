@@ -49,7 +49,7 @@ def cpu_baseline(clouds, emb, blk, C, H, bs, scope, hash_op, activation):
     """the oracle pipeline on the whole batch (the same 4 sweeps), repeated for about ten seconds of CPU work,
     all host cores for the torch part"""
     from oracle import f3d_oracle as orc
-    from flash3dtransformer_amd import synth
+    import bench_workloads as synth
     cores = os.cpu_count() or 1
     torch.set_num_threads(cores)
     coords, seps = synth.batch_of(clouds)
@@ -96,7 +96,7 @@ def main():
               file=sys.stderr)
         sys.exit(2)
 
-    from flash3dtransformer_amd import synth
+    import bench_workloads as synth
     from flash3dtransformer_amd.lib import pshattn
     from flash3dtransformer_amd.psh import psh_main
     dev = "cuda:0"
@@ -109,7 +109,7 @@ def main():
     coords = torch.from_numpy(coords_np).to(dev)
     seps = torch.from_numpy(seps_np.view(np.int32)).to(dev).view(torch.uint32)
     n_pts = coords.shape[0]
-    from flash3dtransformer_amd import configs
+    import bench_workloads as configs
     emb, blk = configs.encoder_stage(args.mlp, 1004)
     emb, blk = emb.to(dev), blk.to(dev)
 
@@ -258,18 +258,61 @@ def sub_metrics(dev, only=None):
     return out
 
 
+def _bench_probe():
+    """bench_probe.so beside this file (built by __graft_entry__.build() from bench_probe.hip): measurement aids that
+    are not part of the library"""
+    import ctypes
+    path = os.path.join(ROOT, "bench_probe.so")
+    if not os.path.exists(path):
+        raise RuntimeError(f"{path} is missing: run `python __graft_entry__.py` first")
+    return ctypes.CDLL(path)
+
+
 def sub_mfma_rate(dev, out):
-    """what the matrix cores of this GPU sustain on dense bf16 products with nothing else running (register operands,
-    4 waves per SIMD): with random operands the power budget sets the clock, with a zero operand the data-sheet rate
-    is reached.  Context for the `frac` figures, which are priced against the data-sheet 2.5 PFLOP/s."""
+    """What the matrix cores of this GPU sustain on dense bf16 products with nothing else running (register operands,
+    4 waves per SIMD) and the shader clock they run at meanwhile (in-kernel shader-clock counter against the 100 MHz
+    constant-rate counter): with random operands the power budget sets the clock, with a zero operand the data-sheet
+    rate is reached.  Then the same question for the step's dominant kernel: the one-kernel gated MLP at the bench
+    shape with N(0,1) operands and with all-zero operands (same instruction stream and addresses, nothing toggling in
+    the multipliers).  Context for the `frac` figures, which are priced against the data-sheet 2.5 PFLOP/s."""
+    import ctypes
     from flash3dtransformer_amd.lib import pshattn
+    lib = _bench_probe()
     sink = torch.zeros(1, dtype=torch.float32, device=dev)
     wgs, iters = 1024, 100000
+    clocks = torch.zeros(wgs, 2, dtype=torch.int64, device=dev)
     flop = wgs * 4 * iters * 8 * 32768.0
-    for name, ra, rb in (("random_operands", True, True), ("one_zero_operand", False, True)):
-        ms = ev_time(lambda: pshattn.probe_mfma_bf16(wgs, iters, ra, rb, sink), 3, warmup=1)
+    u32, vp = ctypes.c_uint32, ctypes.c_void_p
+
+    def probe(ra, rb):
+        rc = lib.bench_probe_mfma_bf16(u32(wgs), u32(iters), u32(ra), u32(rb), vp(sink.data_ptr()),
+                                       vp(clocks.data_ptr()), vp(torch.cuda.current_stream(0).cuda_stream))
+        if rc != 0:
+            raise RuntimeError(f"bench_probe_mfma_bf16 failed with {rc}")
+    for name, ra, rb in (("random_operands", 1, 1), ("one_zero_operand", 0, 1)):
+        ms = ev_time(lambda: probe(ra, rb), 3, warmup=1)
+        ck = clocks.double().cpu()
+        ghz = (ck[:, 0] / (ck[:, 1] / 100e6) / 1e9)
         out["mfma_bf16_dense_rate_" + name] = {"ms": round(ms, 3), "tflops": round(flop / ms / 1e9, 1),
-                                               "frac_of_bf16_mfma_peak": round(flop / ms / 1e9 / MFMA_BF16_PEAK_TFLOPS, 4)}
+                                               "frac_of_bf16_mfma_peak": round(flop / ms / 1e9 / MFMA_BF16_PEAK_TFLOPS, 4),
+                                               "shader_clock_ghz_median": round(ghz.median().item(), 3),
+                                               "shader_clock_ghz_min": round(ghz.min().item(), 3)}
+    M, C, HID = 482_304, 256, 1024
+    gg = torch.Generator().manual_seed(1004)
+    rnd = lambda *shape, scale=1.0: (torch.randn(*shape, generator=gg) * scale).to(torch.bfloat16).to(dev)
+    y = torch.empty(M, C, dtype=torch.bfloat16, device=dev)
+    fl = 6.0 * M * C * HID
+    for name, zero in (("random_operands", False), ("zero_operands", True)):
+        x = torch.zeros(M, C, dtype=torch.bfloat16, device=dev) if zero else rnd(M, C)
+        w1 = torch.zeros(2 * HID, C, dtype=torch.bfloat16, device=dev) if zero else rnd(2 * HID, C, scale=1 / 16)
+        w2 = torch.zeros(C, HID, dtype=torch.bfloat16, device=dev) if zero else rnd(C, HID, scale=1 / 32)
+        b1 = torch.zeros(2 * HID, dtype=torch.bfloat16, device=dev) if zero else rnd(2 * HID)
+        b2 = torch.zeros(C, dtype=torch.bfloat16, device=dev) if zero else rnd(C)
+        g = torch.zeros(C, dtype=torch.bfloat16, device=dev) if zero else torch.ones(C, dtype=torch.bfloat16, device=dev)
+        ms = ev_time(lambda: pshattn.ln_mlp_swiglu_bf16(x, g, b2, 1e-5, w1, b1, w2, b2, x, y), 20)
+        out["ln_mlp_swiglu_256x1024_" + name] = {"ms": round(ms, 4), "tflops": round(fl / ms / 1e9, 1),
+                                                 "frac_of_bf16_mfma_peak": round(fl / ms / 1e9 / MFMA_BF16_PEAK_TFLOPS, 4)}
+        del x, w1, w2
 
 
 def sub_backward(dev, out):
@@ -331,7 +374,7 @@ def sub_backward(dev, out):
     torch.cuda.empty_cache()
     # forward + backward of the whole 5-level hourglass (config 5: 4 sweeps x 250,000 points), training mode, fp32
     # master weights (their bf16 copies are made anew every step), loss = mean of squares; wall time per step
-    from flash3dtransformer_amd import configs
+    import bench_workloads as configs
     model = configs.hourglass(1005).to(dev).train()
     coords_np, seps_np, _ = configs.lidar_batch(4, 250_000, 1005)
     coords, seps = configs.to_device(coords_np, seps_np, dev)
@@ -529,7 +572,7 @@ def hourglass_c5(dev):
     is not what the GPU waits for.  `gpu_busy_ms`: the sum of the kernel durations of one forward, from the
     profiler's kernel records (None when the profiler is not usable, e.g. under an outer tracer); `ms` minus it is
     the idle time between consecutive kernels."""
-    from flash3dtransformer_amd import configs
+    import bench_workloads as configs
     model = configs.hourglass(1005).to(dev).eval()
     coords_np, seps_np, _ = configs.lidar_batch(4, 250_000, 1005)
     coords, seps = configs.to_device(coords_np, seps_np, dev)

@@ -1,0 +1,65 @@
+// Measurement aids of bench.py (built into bench_probe.so beside it; not part of libf3d_hip.so and of no use to a
+// caller of the library).
+//
+// bench_probe_mfma_bf16: the rate at which the matrix cores of this GPU retire dense v_mfma_f32_32x32x16_bf16 products
+// when nothing else runs (operands in registers, eight independent accumulators per wave, four waves per SIMD), and the
+// shader clock they run at meanwhile.  With random operands the chip's power budget, not the issue rate, sets the
+// clock; with a zero operand the multipliers do not toggle and the rate is the 2.5 PFLOP/s of the data sheet.  Every
+// workgroup's first lane reads the shader-clock counter and the 100 MHz constant-rate counter at its start and end:
+// their ratio is the clock the products ran at.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16_t;
+
+__global__ __launch_bounds__(256) void probe_mfma_kernel(float* __restrict__ sink, uint64_t* __restrict__ clocks,
+                                                         uint32_t iters, uint32_t random_a, uint32_t random_b) {
+  uint32_t h = (blockIdx.x * 256u + threadIdx.x) * 2654435761u;
+  bf16x8_t a[4], b[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      h = h * 1664525u + 1013904223u;
+      a[i][e] = (__bf16)(random_a ? ((int)((h >> 8) & 0xFFFFu) - 32768) / 32768.0f : 0.f);
+      h = h * 1664525u + 1013904223u;
+      b[i][e] = (__bf16)(random_b ? ((int)((h >> 8) & 0xFFFFu) - 32768) / 32768.0f : 0.f);
+    }
+  f32x16_t acc[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[j][i] = 0.f;
+  const uint64_t c0 = clock64(), w0 = wall_clock64();
+  for (uint32_t it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[j & 3], b[(j + 1) & 3], acc[j], 0, 0, 0);
+  }
+  float s = 0.f;
+#pragma unroll
+  for (int j = 0; j < 8; ++j)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) s += acc[j][i];
+  const uint64_t c1 = clock64(), w1 = wall_clock64();
+  if (s == 123.456f) sink[0] = s;   // keeps the products alive; never true for these operands
+  if (clocks && threadIdx.x == 0) {
+    clocks[2 * blockIdx.x] = c1 - c0;
+    clocks[2 * blockIdx.x + 1] = w1 - w0;
+  }
+}
+
+extern "C" {
+
+// workgroups x 4 waves x iters x 8 products of 32,768 flops.  sink: one float of device memory (never written);
+// clocks: 2 x workgroups uint64 of device memory (shader-clock ticks, 100 MHz ticks per workgroup) or NULL.
+// Returns 0, or the HIP error code of the launch.
+int bench_probe_mfma_bf16(uint32_t workgroups, uint32_t iters, uint32_t random_a, uint32_t random_b, float* sink,
+                          uint64_t* clocks, void* stream) {
+  if (!sink || workgroups == 0 || workgroups > 65536u || iters > (1u << 24)) return -1;
+  hipLaunchKernelGGL(probe_mfma_kernel, dim3(workgroups), dim3(256), 0, (hipStream_t)stream, sink, clocks, iters,
+                     random_a, random_b);
+  return (int)hipGetLastError();
+}
+
+}  // extern "C"

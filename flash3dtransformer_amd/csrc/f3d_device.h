@@ -48,34 +48,39 @@ __device__ __forceinline__ float bf16_lo(uint32_t w) { return __builtin_bit_cast
 __device__ __forceinline__ float bf16_hi(uint32_t w) { return __builtin_bit_cast(float, w & 0xFFFF0000u); }
 
 // ---- voxel quantiser (reference: src/psh/hash_fns.cuh:23-33) ----------------------------------
-// q = ((c - min) * num_vox) * inv with inv = 1 / (max - min) rounded once; floor; clamp to
-// [0, num_vox - 1] with NaN -> num_vox - 1.  All steps are separate IEEE fp32 operations: the
-// translation units that use this are built with -ffp-contract=off.
+// floor(q), clamped to [0, num_vox - 1] with NaN -> num_vox - 1, where q is one of two roundings of
+// (c - min) * num_vox / (max - min):
+//   mode 0 (default): q = ((c - min) * num_vox) * inv with inv = 1 / (max - min) rounded once: what a build of
+//           the reference with nvcc --use_fast_math (its CMakeLists.txt:49-52) evaluates, given an exact reciprocal;
+//   mode 1: q = ((c - min) * num_vox) / (max - min), the IEEE division the source text spells out.
+// All steps are separate IEEE fp32 operations: the translation units that use this are built with
+// -ffp-contract=off.  Kernels receive the mode in bit 31 of their num_vox argument (num_vox <= 65536).
+constexpr uint32_t kVoxDivideBit = 0x80000000u;
+
 struct VoxAxis {
-  float mn, inv, nv, hi;
+  float mn, inv, nv, hi, den;
+  bool divide;
 };
 
-__device__ __forceinline__ VoxAxis make_vox_axis(uint16_t min_h, uint16_t max_h, uint32_t num_vox) {
+__device__ __forceinline__ VoxAxis make_vox_axis_f(float mn, float mx, uint32_t num_vox_mode) {
+  const uint32_t num_vox = num_vox_mode & ~kVoxDivideBit;
   VoxAxis a;
-  a.mn = half_bits_to_float(min_h);
-  float den = half_bits_to_float(max_h) - a.mn;
-  a.inv = __fdiv_rn(1.0f, den);
+  a.mn = mn;
+  a.den = __fsub_rn(mx, mn);
+  a.inv = __fdiv_rn(1.0f, a.den);
   a.nv = (float)num_vox;
   a.hi = (float)(num_vox - 1u);
+  a.divide = (num_vox_mode & kVoxDivideBit) != 0;
   return a;
 }
 
-__device__ __forceinline__ VoxAxis make_vox_axis_f(float mn, float mx, uint32_t num_vox) {
-  VoxAxis a;
-  a.mn = mn;
-  a.inv = __fdiv_rn(1.0f, mx - mn);
-  a.nv = (float)num_vox;
-  a.hi = (float)(num_vox - 1u);
-  return a;
+__device__ __forceinline__ VoxAxis make_vox_axis(uint16_t min_h, uint16_t max_h, uint32_t num_vox_mode) {
+  return make_vox_axis_f(half_bits_to_float(min_h), half_bits_to_float(max_h), num_vox_mode);
 }
 
 __device__ __forceinline__ uint32_t vox1(float c, const VoxAxis& a) {
-  float q = __fmul_rn(__fmul_rn(__fsub_rn(c, a.mn), a.nv), a.inv);
+  const float t = __fmul_rn(__fsub_rn(c, a.mn), a.nv);
+  const float q = a.divide ? __fdiv_rn(t, a.den) : __fmul_rn(t, a.inv);
   float v = floorf(q);
   float m = (v < a.hi) ? v : a.hi;  // NaN -> hi
   float r = (m > 0.f) ? m : 0.f;

@@ -35,6 +35,8 @@ int launch_attn_bwd_stream(const uint16_t* q, const uint16_t* k, const uint16_t*
 bool sync_stream_enabled();
 uint32_t global_seed();
 int rebalance_mode();
+// 0x80000000 when the voxel quantiser divides (f3d_set_quantiser(1)), else 0: OR-ed into a kernel's num_vox argument
+uint32_t quantiser_bit();
 
 #define F3D_CHECK_ARG(cond, ...)            \
   do {                                      \

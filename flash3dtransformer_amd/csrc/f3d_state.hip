@@ -20,6 +20,7 @@ static std::unordered_map<int, Ws> g_ws;
 static bool g_sync = false;
 static uint32_t g_seed = 3407u;
 static int g_rebalance = 1;
+static int g_quantiser = 0;
 
 void set_error(const char* fmt, ...) {
   va_list ap;
@@ -61,6 +62,7 @@ void* workspace(int device, size_t bytes) {
 bool sync_stream_enabled() { return g_sync; }
 uint32_t global_seed() { return g_seed; }
 int rebalance_mode() { return g_rebalance; }
+uint32_t quantiser_bit() { return g_quantiser ? 0x80000000u : 0u; }
 
 }  // namespace f3d
 
@@ -101,5 +103,16 @@ int f3d_set_psh_rebalance(int mode) {
 }
 
 int f3d_get_psh_rebalance(void) { return f3d::g_rebalance; }
+
+int f3d_set_quantiser(int mode) {
+  if (mode != 0 && mode != 1) {
+    f3d::set_error("quantiser mode must be 0 (multiply by the reciprocal) or 1 (IEEE division), got %d", mode);
+    return F3D_ERR_INVALID;
+  }
+  f3d::g_quantiser = mode;
+  return F3D_OK;
+}
+
+int f3d_get_quantiser(void) { return f3d::g_quantiser; }
 
 }  // extern "C"

@@ -506,7 +506,7 @@ static void launch_psh(const uint16_t* coord, uint16_t* bucket_id, uint32_t* buc
     auto k1 = zorder ? (mod ? psh_hash_hist_kernel<THREADS, ITEMS, true, true> : psh_hash_hist_kernel<THREADS, ITEMS, true, false>)
                      : (mod ? psh_hash_hist_kernel<THREADS, ITEMS, false, true> : psh_hash_hist_kernel<THREADS, ITEMS, false, false>);
     hipLaunchKernelGGL(k1, dim3(max_tiles, batch_size), dim3(THREADS), lds1, stream, coord, bucket_id, batch_sep,
-                       bbox_min, bbox_max, num_vox, dv, num_bucket, total_n, tile_hist, max_tiles);
+                       bbox_min, bbox_max, num_vox | quantiser_bit(), dv, num_bucket, total_n, tile_hist, max_tiles);
     hipLaunchKernelGGL(psh_tile_scan_kernel, dim3(cdiv_u32(num_bucket, kWave), batch_size), dim3(kScanWaves * kWave), 0,
                        stream, tile_hist, bucket_counter, cnt_ws, batch_sep, num_bucket, tile_pts, max_tiles);
     hipLaunchKernelGGL(psh_bucket_plan_kernel<REBAL>, dim3(batch_size), dim3(kPshThreads),

@@ -303,7 +303,7 @@ int f3d_subbuck_build(const f3d_half_t* coord, const uint32_t* batch_sep, uint32
   if (gx == 0 || (batch_size == 0 && pad_tiles == 0)) return F3D_OK;
   SyncBracket sync(s);
   hipLaunchKernelGGL(subbuck_build_kernel, dim3(gx, batch_size + (pad_tiles ? 1 : 0)), dim3(kSubThreads), 0, s, coord,
-                     batch_sep, reduced_batch_sep, batch_size, subbuck_size, tile_pts, num_vox, global_seed(),
+                     batch_sep, reduced_batch_sep, batch_size, subbuck_size, tile_pts, num_vox | quantiser_bit(), global_seed(),
                      subbuck_id, subbuck_off, unpool_ind, reduced_coord, reduced_n, reduced_aligned_n);
   F3D_CHECK_HIP(hipGetLastError());
   return F3D_OK;

@@ -119,6 +119,14 @@ class DeviceManagerSingleton:
     def get_psh_rebalance(self) -> int:
         return int(_load().f3d_get_psh_rebalance())
 
+    def set_quantiser(self, mode: int):
+        """0: quotient of the voxel quantiser as a multiply by the rounded reciprocal (a fast-math build of the
+        reference, default); 1: IEEE division (src/psh/hash_fns.cuh:23-33 as written)"""
+        _check(_load().f3d_set_quantiser(_i32(mode)))
+
+    def get_quantiser(self) -> int:
+        return int(_load().f3d_get_quantiser())
+
 
 # ---------------------------------------------------------------------------------------------
 # PSH bucketing
@@ -544,15 +552,6 @@ def ln_mlp_swiglu_bf16(x, gamma, beta, eps, w1, b1, w2, b2, residual, y) -> bool
         return False
     _check(rc)
     return True
-
-
-def probe_mfma_bf16(workgroups: int, iters: int, random_a: bool, random_b: bool, sink: torch.Tensor):
-    """measurement aid: workgroups x 4 waves x iters x 8 dense bf16 MFMA products (32,768 flops each) on register
-    operands, pseudo-random or zero; the caller times it (see bench.py)"""
-    assert_dtype([sink], torch.float32)
-    dev = assert_same_device([sink])
-    _check(_load().f3d_probe_mfma_bf16(_u32(workgroups), _u32(iters), _u32(1 if random_a else 0),
-                                       _u32(1 if random_b else 0), _ptr(sink), _i32(dev), _stream(dev)))
 
 
 def layernorm_bf16(x, gamma, beta, y, eps=1e-5):

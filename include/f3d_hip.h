@@ -109,6 +109,15 @@ int f3d_batch_psh_scatter_pad_hash_noalloc(const f3d_half_t* coord, uint16_t* bu
 int f3d_set_psh_rebalance(int mode);
 int f3d_get_psh_rebalance(void);
 
+/* Rounding of the voxel quantiser's quotient (src/psh/hash_fns.cuh:23-33: (c - min) * num_vox / (max - min) in fp32),
+ * for the bucketing op and the sub-bucket builder alike.
+ * 0 = multiply by the correctly rounded reciprocal of (max - min): the form a build of the reference with
+ *     nvcc --use_fast_math (its CMakeLists.txt:49-52) evaluates (default);
+ * 1 = IEEE fp32 division, as the source text reads (a reference build without fast-math).
+ * The two differ by at most one cell, for under 1 % of all fp16 inputs. */
+int f3d_set_quantiser(int mode);
+int f3d_get_quantiser(void);
+
 /* Whole-batch bounding box of fp16 coordinates (replaces the two torch.min/max passes of
  * flash3dxfmr/psh/psh_main.py:117-118).  bbox_min/max [3] fp16, written in place. */
 int f3d_coord_bbox(const f3d_half_t* coord, uint32_t total_n, f3d_half_t* bbox_min, f3d_half_t* bbox_max,
@@ -235,14 +244,6 @@ int f3d_buck_swin_fwd_strided(const f3d_bf16_t* q, const f3d_bf16_t* k, const f3
                               const uint32_t* scope_buckets, uint32_t num_scope, uint32_t scope_size,
                               uint32_t bucket_size, uint32_t batch, uint32_t seq_len, uint32_t num_head,
                               uint32_t head_dim, const int32_t* kv_len, int device, void* stream);
-
-/* ---- measurement aid (no counterpart in the reference, not on the hot path) -------------------
- * Runs `workgroups` x 4 waves x `iters` x 8 back-to-back v_mfma_f32_32x32x16_bf16 products (32,768 flops each) on
- * register operands that are pseudo-random (random_a / random_b != 0) or zero, so that a caller timing it sees the rate
- * the matrix cores sustain under the power budget (random operands) and at the data-sheet clock (a zero operand).
- * sink: one float of device memory (never written). */
-int f3d_probe_mfma_bf16(uint32_t workgroups, uint32_t iters, uint32_t random_a, uint32_t random_b, float* sink,
-                        int device, void* stream);
 
 /* ---- dense layers --------------------------------------------------------------------------
  * gemm_sm_bf16(A[M,K], B[K,N], O[M,N]) — src/f3d_frontend.cu:87-88, src/psh/gemm_dispatcher.cu;

@@ -101,17 +101,27 @@ uint16_t f3d_or_float_to_bf16(float f) {
 /* A1: voxel quantiser  — src/psh/hash_fns.cuh:23-33, clamp at src/common/arithmetic.cuh:26-28 */
 /* ------------------------------------------------------------------------------------------ */
 
-/* v = clamp(floor((c - min) * num_vox / (max - min)), 0, num_vox - 1).  The reference is built with
- * nvcc --use_fast_math (CMakeLists.txt:49-52), which turns the fp32 division into a multiplication
- * by the reciprocal of the divisor; the restatement pins that form with a correctly rounded
- * reciprocal: q = fl(fl((c - min) * num_vox) * fl(1 / (max - min))), every step IEEE fp32.
+/* v = clamp(floor((c - min) * num_vox / (max - min)), 0, num_vox - 1).  Two roundings of the quotient:
+ * mode 0 (default): the reference is built with nvcc --use_fast_math (CMakeLists.txt:49-52), which turns the fp32
+ *   division into a multiplication by the reciprocal of the divisor; pinned with a correctly rounded
+ *   reciprocal: q = fl(fl((c - min) * num_vox) * fl(1 / (max - min))), every step IEEE fp32;
+ * mode 1: q = fl(fl((c - min) * num_vox) / fl(max - min)), the IEEE division the source text spells out
+ *   (a build without fast-math).
  * clamp(x, lo, hi) = max(lo, min(x, hi)) with NaN-ignoring min (arithmetic.cuh:26-28), so a
- * degenerate axis (max == min: 0 * inf = NaN) lands on num_vox - 1. */
+ * degenerate axis (max == min: 0 * inf = 0 / 0 = NaN) lands on num_vox - 1. */
+static int g_quantiser_mode = 0;
+
+int f3d_or_set_quantiser(int mode) {
+  if (mode != 0 && mode != 1) return -1;
+  g_quantiser_mode = mode;
+  return 0;
+}
+
 uint16_t f3d_or_vox1(float c, float mn, float mx, uint32_t num_vox) {
   volatile float den = mx - mn;
   volatile float inv = 1.0f / den;
   volatile float num = (c - mn) * (float)num_vox;
-  volatile float q = num * inv;
+  volatile float q = g_quantiser_mode ? num / den : num * inv;
   float v = floorf(q);
   float hi = (float)(num_vox - 1u);
   float m = (v < hi) ? v : hi; /* NaN -> hi */

@@ -124,6 +124,13 @@ def gen_scopes(total_n: int, buck_size: int, scope_size: int, plan: str = "swin"
 # A1 / A2
 # ---------------------------------------------------------------------------------------------
 
+def set_quantiser(mode: int):
+    """0: the quantiser's quotient as a multiply by the rounded reciprocal (a fast-math build of the reference, default);
+    1: IEEE division (src/psh/hash_fns.cuh:23-33 as written).  Applies to every later call of this module."""
+    if lib().f3d_or_set_quantiser(ctypes.c_int(mode)) != 0:
+        raise ValueError(f"quantiser mode must be 0 or 1, got {mode}")
+
+
 def vox_coord(coord_h, bbox_min_h, bbox_max_h, num_vox: int = 0xFFFF):
     c = _u16(coord_h).reshape(-1, 3)
     out = np.empty_like(c)

@@ -43,6 +43,10 @@ def test_module_state_roundtrip(lib):
     lib.f3d_set_seed(ctypes.c_uint32(3407))
     assert lib.f3d_set_psh_rebalance(7) != 0 and b"rebalance" in lib.f3d_last_error()
     assert lib.f3d_set_psh_rebalance(1) == 0
+    assert lib.f3d_get_quantiser() == 0
+    assert lib.f3d_set_quantiser(1) == 0 and lib.f3d_get_quantiser() == 1
+    assert lib.f3d_set_quantiser(2) != 0 and b"quantiser mode" in lib.f3d_last_error()
+    assert lib.f3d_set_quantiser(0) == 0 and lib.f3d_get_quantiser() == 0
 
 
 def _psh_call(lib, *, num_bucket=64, divisor=1024, pad_to=512, total_n=512, hash_type=1, num_vox=0xFFFF):

@@ -28,19 +28,23 @@ def _state_dict_cpu(*modules_with_prefix):
     return sd
 
 
-def _bands(got, want, mean_tol=0.02, bulk_tol=0.05, max_tol=0.25):
+def _bands(got, want, mean_tol, bulk_tol, max_tol):
+    """mean error <= mean_tol * scale, 99 % of the entries within bulk_tol * scale, largest error <= max_tol * max|ref|
+    (scale = mean |ref|, at least 1).  The callers' values leave 3 to 4 times the measured error as headroom."""
     err = (got - want).abs()
     scale = want.abs().mean().item()
     assert scale > 0.05, "degenerate case: output too small to mean anything"
     assert torch.isfinite(got).all()
     assert err.mean().item() <= mean_tol * max(1.0, scale), f"mean err {err.mean().item()} at scale {scale}"
     assert err.max().item() <= max_tol * max(1.0, want.abs().max().item()), f"max err {err.max().item()}"
+    print(f"bands: mean err {err.mean().item():.5f} max err {err.max().item():.4f} scale {scale:.4f} "
+          f"ref max {want.abs().max().item():.3f} p99 {err.flatten().kthvalue(int(err.numel() * 0.99)).values.item():.4f}")
     assert (err <= bulk_tol * max(1.0, scale)).float().mean().item() >= 0.99
     return err.mean().item(), err.max().item(), scale
 
 
 def test_encoder_stage_4x120k_full_size_vs_oracle(oracle):
-    from flash3dtransformer_amd import configs
+    import bench_workloads as configs
     cfg = configs.ENCODER_STAGE
     C, H, bs, scope, hash_op = cfg["channels"], cfg["heads"], cfg["bucket_size"], cfg["scope_size"], cfg["hash_type"]
     coords, seps, _ = configs.lidar_batch(4, 120_000, 1004)
@@ -64,7 +68,8 @@ def test_encoder_stage_4x120k_full_size_vs_oracle(oracle):
     assert (feat.float().cpu() - x).abs().max().item() <= 2e-2 * max(1.0, x.abs().max().item())
     w = {k: sd["blk." + v] for k, v in oracle.XFMR_KEYS.items()}
     want = oracle.xfmr_block(x, w, oracle.gen_scopes(pad_to, bs, scope), bs, H, "swiglu")
-    _bands(out.float().cpu(), want)
+    # measured: mean 0.0009 at scale 0.73, 99th percentile 0.008, max 0.094 at max|ref| 15.6
+    _bands(out.float().cpu(), want, mean_tol=0.004, bulk_tol=0.03, max_tol=0.03)
 
 
 def _hook_pooling_buffers(model):
@@ -76,7 +81,7 @@ def _hook_pooling_buffers(model):
 
 
 def test_hourglass_five_levels_vs_oracle_pipeline(oracle):
-    from flash3dtransformer_amd import configs
+    import bench_workloads as configs
     cfg = configs.HOURGLASS
     bs, scope, S, hash_op = cfg["bucket_size"], cfg["scope_size"], cfg["subbuck_size"], cfg["hash_type"]
     model = configs.hourglass(1005)
@@ -108,14 +113,15 @@ def test_hourglass_five_levels_vs_oracle_pipeline(oracle):
         assert np.array_equal(got_u, unpool), f"level {level}: pooling map differs"
         assert np.array_equal(buf.reduced_coord.cpu().numpy().view(np.uint16), red_coord.view(np.uint16)), level
     assert out.shape == want.shape
-    # ten transformer blocks, four poolings and four unpoolings deep: the bands are those of the two-level case
-    _bands(out.float().cpu(), want)
+    # ten transformer blocks, four poolings and four unpoolings deep; measured: mean 0.009 at scale 1.5, 99th
+    # percentile 0.031, max 0.094 at max|ref| 6.3
+    _bands(out.float().cpu(), want, mean_tol=0.025, bulk_tol=0.08, max_tol=0.06)
 
 
 def test_hourglass_4x250k_full_size_properties():
     """config 5 at full size: finite output of the right shape; every level's pooling map is a bijection between the
     level's rows and the filled slots; restoring the input order inverts the PSH permutation"""
-    from flash3dtransformer_amd import configs
+    import bench_workloads as configs
     model = configs.hourglass(1005).to(DEV).eval()
     coords, seps, _ = configs.lidar_batch(4, 250_000, 1005)
     c, s = configs.to_device(coords, seps, DEV)
@@ -157,7 +163,7 @@ def test_encoder_stage_4x120k_backward_full_size_properties():
     """config 4 at full size through loss.backward(): every gradient is finite and not identically zero; a second run
     gives the same bits (no atomics anywhere in the backward); and the backward is linear in the upstream gradient:
     doubling it doubles every gradient exactly (a power of two commutes with every bf16 / fp32 rounding on the way)"""
-    from flash3dtransformer_amd import configs
+    import bench_workloads as configs
     cfg = configs.ENCODER_STAGE
     hash_op = cfg["hash_type"]
     coords, seps, _ = configs.lidar_batch(4, 120_000, 1004)
@@ -189,7 +195,7 @@ def test_hourglass_4x250k_backward_full_size_properties():
     """config 5 at full size through loss.backward(): PSH embedding, five levels of blocks, pooling and unpooling.  Every
     parameter receives a finite, not identically zero gradient; a second run gives the same bits; doubling the upstream
     gradient doubles every gradient exactly"""
-    from flash3dtransformer_amd import configs
+    import bench_workloads as configs
     model = configs.hourglass(1005).to(DEV).train()
     coords, seps, _ = configs.lidar_batch(4, 250_000, 1005)
     c, s = configs.to_device(coords, seps, DEV)

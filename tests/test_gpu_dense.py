@@ -265,7 +265,7 @@ def test_layernorm_mlp_layer_one_kernel_and_two_kernel_paths():
     assert b.fc2_weight.grad.abs().max().item() > 0
 
 
-def test_fused_mlp_and_output_panel_kernel_at_bench_size():
+def test_fused_mlp_and_output_panel_kernel_at_bench_size(oracle):
     """482,304 rows x 256 channels, hidden 1024 (the bench's MLP): the one-kernel MLP against LayerNorm+fc1+gate
     followed by fc2+residual (which at this size runs the output-panel kernel), and the output-panel kernel against
     the tiled GEMM on a row slice small enough to fall back to it."""
@@ -285,21 +285,25 @@ def test_fused_mlp_and_output_panel_kernel_at_bench_size():
     # one bf16 step of the fc2 output before the residual add, whose magnitude is at most |y| + |residual|
     d = (y.float() - y2.float()).abs() / (y2.float().abs() + x.float().abs()).clamp(min=1.0)
     assert d.max().item() <= 2 ** -6 and (d > 0).float().mean().item() < 0.02
+    # against the fp32 oracle on 4,096 rows spread over the launch (first panel, interior, the short panels of the
+    # last turn of the chip, the very last rows): as close to the unrounded mathematics as the reference's own
+    # sequence of bf16 roundings
+    rows = torch.cat([torch.arange(0, 1024), torch.arange(200_000, 201_024), torch.arange(481_000, 482_024),
+                      torch.arange(M - 1024, M)]).to(DEV)
+    xc, gc, bc, w1c, w2c, b1c, b2c = [t.cpu() for t in (x[rows], g, b, w1, w2, b1, b2)]
+    rb = lambda t: t.to(torch.bfloat16).float()
+    exact = oracle.linear(oracle.swiglu(oracle.linear(oracle.layernorm(xc, gc, bc, 1e-5), w1c, b1c)), w2c, b2c) + xc.float()
+    ref = rb(rb(oracle.linear(rb(oracle.swiglu(rb(oracle.linear(rb(oracle.layernorm(xc, gc, bc, 1e-5)), w1c, b1c)))),
+                              w2c, b2c)) + xc.float())
+    scale = exact.abs().clamp(min=1.0)
+    for got in (y[rows], y2[rows]):
+        err_us, err_ref = (got.float().cpu() - exact).abs() / scale, (ref - exact).abs() / scale
+        assert err_us.max() <= 1.5 * err_ref.max() + 4e-3, (err_us.max(), err_ref.max())
+        assert err_us.mean() <= 1.25 * err_ref.mean() + 1e-4, (err_us.mean(), err_ref.mean())
+        assert (got.float().cpu() - exact).abs().max() <= 2e-2 * exact.abs().max().clamp(min=1.0)
     n_small = 20000                                                   # fewer rows than the output-panel kernel takes
     y3 = torch.empty(n_small, C, dtype=torch.bfloat16, device=DEV)
     pshattn.linear_bf16(hid[-n_small:], w2, b2, x[-n_small:], y3, None)   # tiled GEMM
     torch.cuda.synchronize()
     d = (y2[-n_small:].float() - y3.float()).abs() / (y3.float().abs() + x[-n_small:].float().abs()).clamp(min=1.0)
     assert d.max().item() <= 2 ** -6 and (d > 0).float().mean().item() < 0.02
-
-
-def test_mfma_rate_probe_runs():
-    """the measurement aid behind bench.py's `mfma_bf16_dense_rate_*`: launches, finishes, leaves its sink alone"""
-    from flash3dtransformer_amd.lib import pshattn
-    sink = torch.full((1,), 5.0, dtype=torch.float32, device=DEV)
-    for ra, rb in ((True, True), (False, True)):
-        pshattn.probe_mfma_bf16(64, 100, ra, rb, sink)
-    torch.cuda.synchronize()
-    assert sink.item() == 5.0
-    with pytest.raises(RuntimeError, match="out of range"):
-        pshattn.probe_mfma_bf16(0, 100, True, True, sink)

@@ -32,7 +32,8 @@ def _bn(sd, prefix):
 
 
 def test_two_level_hourglass_matches_oracle_pipeline(oracle):
-    from flash3dtransformer_amd import layers as L, synth
+    from flash3dtransformer_amd import layers as L
+    import bench_workloads as synth
     from flash3dtransformer_amd.psh.bucket_scope import SwinPlan
     bs, scope, S, hash_op, align1 = 128, 2, 2, 1, 256
     torch.manual_seed(0)
@@ -101,10 +102,13 @@ def test_two_level_hourglass_matches_oracle_pipeline(oracle):
     err = (got - want).abs()
     scale = want.abs().mean().item()
     assert scale > 0.05, "degenerate test: output too small to be meaningful"
-    assert err.mean().item() <= 0.02 * max(1.0, scale), f"mean err {err.mean().item()} at scale {scale}"
-    assert err.max().item() <= 0.25 * max(1.0, want.abs().max().item()), f"max err {err.max().item()}"
+    print(f"bands: mean err {err.mean().item():.5f} max err {err.max().item():.4f} scale {scale:.4f} "
+          f"ref max {want.abs().max().item():.3f}")
+    # measured: mean 0.097 at scale 36, max 4.0 at max|ref| 556 (one bf16 step at that magnitude): 3 to 4 times headroom
+    assert err.mean().item() <= 0.01 * max(1.0, scale), f"mean err {err.mean().item()} at scale {scale}"
+    assert err.max().item() <= 0.03 * max(1.0, want.abs().max().item()), f"max err {err.max().item()}"
     # the bulk of the entries agree to bf16 precision
-    assert (err <= 0.05 * max(1.0, scale)).float().mean().item() >= 0.99
+    assert (err <= 0.02 * max(1.0, scale)).float().mean().item() >= 0.99
 
 
 def test_unsupported_attention_backward_says_so():
@@ -204,7 +208,8 @@ def test_transformer_block_trains(oracle):
 def test_two_level_model_backward_reaches_every_parameter():
     """loss.backward() through the whole hourglass: PSH embedding, transformer blocks, pooling, unpooling.  Every
     parameter receives a finite, not identically zero gradient, and an SGD step lowers the loss."""
-    from flash3dtransformer_amd import layers as L, synth
+    from flash3dtransformer_amd import layers as L
+    import bench_workloads as synth
     from flash3dtransformer_amd.psh.bucket_scope import SwinPlan
     bs, scope, S, hash_op, align1 = 256, 1, 2, 1, 256
     torch.manual_seed(1)
@@ -242,7 +247,8 @@ def test_model_consumes_point_features_and_restores_input_order():
     through the PSH permutation, `input_proj` trains, and `to_input_order` returns rows in the order the points
     came in: permuting the input points permutes that output the same way (bucket slots follow input order, so the
     comparison is through the point's coordinates: same multiset of (coord, output) rows per cloud)."""
-    from flash3dtransformer_amd import layers as L, synth
+    from flash3dtransformer_amd import layers as L
+    import bench_workloads as synth
     from flash3dtransformer_amd.psh.bucket_scope import SwinPlan
     bs, scope = 256, 1
     torch.manual_seed(2)
@@ -277,7 +283,8 @@ def test_model_consumes_point_features_and_restores_input_order():
 def test_restore_input_order_without_point_features():
     """Default model (input_feat ignored, as in the reference): to_input_order builds the permutation index on demand;
     row i of its result is the output row of input point i (checked through the scattered coordinates)."""
-    from flash3dtransformer_amd import layers as L, synth
+    from flash3dtransformer_amd import layers as L
+    import bench_workloads as synth
     from flash3dtransformer_amd.psh.bucket_scope import SwinPlan
     bs = 256
     torch.manual_seed(3)

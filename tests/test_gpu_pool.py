@@ -48,7 +48,7 @@ def test_builder_and_reduce_bit_exact(oracle, S, op, sizes, C):
 
 def test_c3_pool_unpool_full_size(oracle):
     """BASELINE config 3: 262,144 points x 128 channels, S=8 (2x2x2), mean and max, then unpool"""
-    from flash3dtransformer_amd import synth
+    import bench_workloads as synth
     from flash3dtransformer_amd.lib import pshattn
     n, C, S = 262144, 128, 8
     coords, seps = synth.batch_of([synth.uniform_cube(n // 4, 51.2, 1003 + i) for i in range(4)])

@@ -52,7 +52,7 @@ def _check_against_oracle(coords, seps, out, hash_op, oracle, rebalance=0, bucke
 @pytest.mark.parametrize("hash_op", [1, 2, 3, 4])
 def test_c1_uniform_cube_bit_exact(oracle, hash_op):
     """BASELINE config 1: 1 x 32,768 points uniform in a 51.2 m cube, bucket 512 -> 64 buckets"""
-    from flash3dtransformer_amd import synth
+    import bench_workloads as synth
     coords, seps = synth.batch_of([synth.uniform_cube(32768, 51.2, 1001)])
     out = _run_psh(coords, seps, 512, hash_op, 512, oracle)
     assert out["nb"] == 64 and out["div"] == 1024
@@ -60,6 +60,53 @@ def test_c1_uniform_cube_bit_exact(oracle, hash_op):
     assert not np.isnan(out["scat"]).any()
     rc, _ = oracle.scoreboard(out["ids"], out["cnt"], out["off"], seps)
     assert rc == 0
+
+
+def test_quantiser_division_mode_bit_exact(oracle):
+    """f3d_set_quantiser(1): IEEE division in the voxel quantiser (src/psh/hash_fns.cuh:23-33 as written), for a user
+    whose CUDA build of the reference was not a fast-math one.  Every fp16 pattern as a coordinate (so every rounding
+    case of the quotient is in the batch) plus config 1's cloud; ids, counts, slots and scattered rows against the
+    oracle in the same mode; the two modes differ on this input, so the switch is seen to act; the sub-bucket
+    builder follows the same switch."""
+    import bench_workloads as synth
+    from flash3dtransformer_amd.lib import pshattn
+    from flash3dtransformer_amd.psh import subbuck
+    mgr = pshattn.DeviceManagerSingleton.instance()
+    bits = np.arange(65536, dtype=np.uint16).view(np.float16)
+    bits = bits[np.isfinite(bits) & (np.abs(bits.astype(np.float32)) <= 80.0)]
+    rng = np.random.default_rng(11)
+    every = np.stack([bits, rng.permutation(bits), rng.permutation(bits)], axis=1)
+    cube, _ = synth.batch_of([synth.uniform_cube(32768, 51.2, 1001)])
+    coords = np.concatenate([every, cube]).astype(np.float16)
+    seps = np.array([every.shape[0], coords.shape[0]], dtype=np.uint32)
+    assert mgr.get_quantiser() == 0
+    base = _run_psh(coords, seps, 512, 1, 512, oracle)
+    try:
+        mgr.set_quantiser(1)
+        oracle.set_quantiser(1)
+        assert mgr.get_quantiser() == 1
+        for hash_op in (1, 2, 3, 4):
+            out = _run_psh(coords, seps, 512, hash_op, 512, oracle, rebalance=hash_op % 2)
+            _check_against_oracle(coords, seps, out, hash_op, oracle, rebalance=hash_op % 2)
+            if hash_op == 1:
+                assert (out["ids"] != base["ids"]).any() or (out["off"] != base["off"]).any()
+        # sub-bucket builder in the same mode
+        S = 4
+        c, s = t_f16(coords), t_u32(seps)
+        f = torch.zeros(coords.shape[0], 8, dtype=torch.bfloat16, device=DEV)
+        sb = subbuck.SubbuckBuffers.create_subbuck_buff(c, f, s, S, out_alignment=1)
+        max_n = int(np.diff(np.concatenate([[0], seps.astype(np.int64)])).max())
+        pshattn.batch_subbuck_reduce(c, f, s, max_n, S, 0xFFFF, sb.bbox_min, sb.bbox_max, sb.subbuck_id, sb.subbuck_off,
+                                     sb.reduced_sep, sb.reduced_coord, sb.reduced_feat, sb.unpool_ind, 1, 0)
+        torch.cuda.synchronize()
+        sid, soff, unpool, red_coord, _ = oracle.subbuck_build(coords, seps, S)
+        assert np.array_equal(n_u32(sb.unpool_ind), unpool) and np.array_equal(n_u32(sb.subbuck_id), sid)
+        assert np.array_equal(n_f16(sb.reduced_coord).view(np.uint16), red_coord.view(np.uint16))
+    finally:
+        mgr.set_quantiser(0)
+        oracle.set_quantiser(0)
+    with pytest.raises(RuntimeError, match="quantiser mode"):
+        mgr.set_quantiser(3)
 
 
 @pytest.mark.parametrize("sizes,bucket_size", [
@@ -107,7 +154,7 @@ def test_small_clouds_bit_exact(oracle, sizes, bucket_size, rebalance):
 def test_lidar_batch_reference_invariants(oracle):
     """4 synthetic sweeps (heavily clustered): the reference's three checks, through its own
     sanitizer entry point"""
-    from flash3dtransformer_amd import synth
+    import bench_workloads as synth
     from flash3dtransformer_amd.lib import pshattn
     clouds = [synth.lidar_sweep(30000, 1004 + i, oversample=2) for i in range(4)]
     coords, seps = synth.batch_of(clouds)
@@ -178,7 +225,7 @@ def test_python_wrapper_and_saturating_size_properties(oracle):
 def test_large_tile_configuration_bit_exact(oracle, rebalance):
     """Batches big enough for the 8192-point tiles (LDS-staged scatter): 72 ragged clouds, 4.5 M points, half of
     them clustered so that buckets overflow; ids, counts, slots and scattered rows bit-exact vs the oracle"""
-    from flash3dtransformer_amd import synth
+    import bench_workloads as synth
     rng = np.random.default_rng(77)
     clouds = []
     for i in range(72):
@@ -202,7 +249,7 @@ def test_large_tile_configuration_bit_exact(oracle, rebalance):
 def test_rebalance_bit_exact_and_reference_invariants(oracle, case):
     """A4 (deterministic overflow rebalance + recycle): final ids, counts, slots and scattered rows
     bit-exact vs the oracle, and the reference's three checks on the result"""
-    from flash3dtransformer_amd import synth
+    import bench_workloads as synth
     from flash3dtransformer_amd.lib import pshattn
     if case == "lidar":
         clouds = [synth.lidar_sweep(40000, 1004 + i, oversample=2) for i in range(3)]
@@ -295,7 +342,7 @@ def test_scatter_index_misaligned_rows_and_errors():
 def test_layer_permutation_is_differentiable_and_model_takes_features():
     """to_psh_order / to_input_order are each other's gradient; Flash3D with in_feat_dim consumes input_feat
     and to_input_order returns per-point rows in the order the points came in."""
-    from flash3dtransformer_amd import synth
+    import bench_workloads as synth
     from flash3dtransformer_amd.layers import psh_ops
     from flash3dtransformer_amd.psh import psh_main as pm
     coords, seps = synth.batch_of([synth.uniform_cube(9000, 40.0, 5), synth.uniform_cube(8200, 40.0, 6)])

@@ -371,3 +371,29 @@ def test_norm_act_layernorm_vs_torch(oracle):
     assert torch.equal(oracle.norm_act(x, p, None), want)
     assert torch.equal(oracle.norm_act(x, p, "gelu"), torch.nn.functional.gelu(want).to(torch.bfloat16).float())
     assert torch.equal(oracle.norm_act(x, None, None), x)
+
+
+def test_swiglu_half_order_closed_forms(oracle):
+    """The gate of te.LayerNormMLP(activation="swiglu") as the reference calls it (layers/elem_wise.py:22-26):
+    the activation acts on the FIRST half of the fc1 output and the second half multiplies it.  Closed
+    forms that a swapped-halves restatement fails: a unit multiplier leaves silu of the first half, a zero
+    first half gives zero whatever the multiplier (silu(0) = 0, while silu(g)*0 would too, so the converse
+    case is checked as well: a zero second half gives zero), silu of the second half never appears, and
+    swapping the halves changes the result."""
+    g = torch.Generator().manual_seed(5)
+    a = torch.randn(37, 48, generator=g) * 3
+    m = torch.randn(37, 48, generator=g) * 3
+    silu = a / (1 + torch.exp(-a))                       # written out, not the library call the oracle uses
+    assert torch.allclose(oracle.swiglu(torch.cat([a, torch.ones_like(a)], -1)), silu, atol=1e-6, rtol=1e-6)
+    assert (oracle.swiglu(torch.cat([torch.zeros_like(m), m], -1)) == 0).all()
+    assert (oracle.swiglu(torch.cat([a, torch.zeros_like(a)], -1)) == 0).all()
+    # first half = 1 gives silu(1) * m = 0.731058... * m, not silu(m)
+    got = oracle.swiglu(torch.cat([torch.ones_like(m), m], -1))
+    assert torch.allclose(got, m * (1 / (1 + math.exp(-1.0))), atol=1e-6, rtol=1e-6)
+    both = oracle.swiglu(torch.cat([a, m], -1))
+    assert torch.allclose(both, silu * m, atol=1e-5, rtol=1e-5)
+    assert not torch.allclose(both, oracle.swiglu(torch.cat([m, a], -1)), atol=1e-3)
+    # bf16 input is computed in fp32 and the output has half the width
+    hb = torch.cat([a, m], -1).to(torch.bfloat16)
+    out = oracle.swiglu(hb)
+    assert out.dtype == torch.float32 and out.shape == (37, 48)

@@ -81,6 +81,40 @@ def test_vox_bruteforce_all_fp16(oracle):
     assert np.array_equal(got[:, 2], want)
 
 
+def test_vox_division_mode_bruteforce_all_fp16(oracle):
+    """mode 1 of the quantiser (IEEE division, hash_fns.cuh:23-33 as written): every finite fp16 pattern against the
+    quotient computed in float64 and rounded once to float32 (for two float32 operands that is the correctly rounded
+    float32 quotient: 53 >= 2 * 24 + 2 bits), in two boxes; known answers keep their values; mode 0 comes back"""
+    bits = np.arange(65536, dtype=np.uint16)
+    c = bits.view(np.float16)
+    c = c[np.isfinite(c)]
+    coords = np.stack([c, c, c], axis=1)
+    try:
+        oracle.set_quantiser(1)
+        for mn, mx in ((np.float16(-40.5), np.float16(51.19)), (np.float16(-79.9), np.float16(80.0))):
+            got = oracle.vox_coord(coords, np.array([mn] * 3, np.float16), np.array([mx] * 3, np.float16))
+            num = ((c.astype(np.float32) - np.float32(mn)) * np.float32(65535.0)).astype(np.float64)
+            den = np.float64(np.float32(mx) - np.float32(mn))
+            with np.errstate(all="ignore"):
+                q = (num / den).astype(np.float32)
+            want = np.clip(np.floor(q), 0, 65534).astype(np.uint16)
+            assert np.array_equal(got[:, 0], want) and np.array_equal(got[:, 1], want)
+        L = oracle.lib()
+        assert L.f3d_or_vox1(25.6, 0.0, 51.2, 0xFFFF) == 32767 and L.f3d_or_vox1(3.0, 3.0, 3.0, 0xFFFF) == 0xFFFE
+        assert L.f3d_or_vox1(1.0, 0.0, 4.0, 16) == 4
+        # a case on which the two modes differ: 19.546875 in the box [-40.5, 51.1875]: the rounded reciprocal
+        # puts the quotient on the other side of an integer than the division does
+        got1 = oracle.vox_coord(coords, np.array([-40.5] * 3, np.float16), np.array([51.19] * 3, np.float16))
+        oracle.set_quantiser(0)
+        got0 = oracle.vox_coord(coords, np.array([-40.5] * 3, np.float16), np.array([51.19] * 3, np.float16))
+        assert 0 < (got0 != got1).mean() < 0.01
+        assert np.abs(got0.astype(np.int32) - got1.astype(np.int32)).max() == 1
+    finally:
+        oracle.set_quantiser(0)
+    with pytest.raises(ValueError):
+        oracle.set_quantiser(2)
+
+
 def test_morton_spread_bit_loop(oracle):
     L = oracle.lib()
     for k in range(16):
@@ -239,7 +273,7 @@ def test_rebalance_invariants(oracle, case):
     """A4: the invariants the reference's own checks rest on (tests/test_psh.py:117-129) plus the
     properties that define a rebalance: conservation, dense unique slots, bounded occupancy wherever
     capacity exists, untouched buckets stay put, leftovers go to bucket 0 only."""
-    from flash3dtransformer_amd import synth
+    import bench_workloads as synth
     bs = 512
     if case == "lidar":
         clouds = [synth.lidar_sweep(30000, 7 + i, oversample=2) for i in range(2)]

@@ -36,7 +36,8 @@ def _same(a, b):
 
 
 def test_no_alloc_entry_point_matches_the_allocating_one_on_calls_in_a_row():
-    from flash3dtransformer_amd import configs, synth
+    import bench_workloads as configs
+    synth = configs
     from flash3dtransformer_amd.lib import pshattn
     pshattn.DeviceManagerSingleton.instance().init_dev_info(0)
     pshattn.DeviceManagerSingleton.instance().set_psh_rebalance(1)
@@ -82,7 +83,8 @@ def test_no_alloc_entry_point_in_a_captured_graph_replays_to_the_eager_result():
     """A caller that captures its stream (the kind of caller the entry point is for): the call sits in a HIP graph next
     to the fill kernel that clears the counters; every replay, with eager work and synchronisations of the program in
     between, leaves exactly what the eager call leaves."""
-    from flash3dtransformer_amd import configs, synth
+    import bench_workloads as configs
+    synth = configs
     from flash3dtransformer_amd.lib import pshattn
     from flash3dtransformer_amd.psh import psh_main
     pshattn.DeviceManagerSingleton.instance().init_dev_info(0)
