@@ -74,6 +74,19 @@ __device__ __forceinline__ VoxAxis make_vox_axis_f(float mn, float mx, uint32_t 
   return a;
 }
 
+// the same with the reciprocal of the extent, fl(1 / fl(max - min)), computed by the caller
+__device__ __forceinline__ VoxAxis make_vox_axis_inv(float mn, float mx, float inv, uint32_t num_vox_mode) {
+  const uint32_t num_vox = num_vox_mode & ~kVoxDivideBit;
+  VoxAxis a;
+  a.mn = mn;
+  a.den = __fsub_rn(mx, mn);
+  a.inv = inv;
+  a.nv = (float)num_vox;
+  a.hi = (float)(num_vox - 1u);
+  a.divide = (num_vox_mode & kVoxDivideBit) != 0;
+  return a;
+}
+
 __device__ __forceinline__ VoxAxis make_vox_axis(uint16_t min_h, uint16_t max_h, uint32_t num_vox_mode) {
   return make_vox_axis_f(half_bits_to_float(min_h), half_bits_to_float(max_h), num_vox_mode);
 }

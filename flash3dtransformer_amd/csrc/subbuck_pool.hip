@@ -5,9 +5,11 @@
 //
 // Builder design: one 1024-thread workgroup per tile of tile_pts = (1024 / S) * S consecutive points
 // of one cloud.  The tile is rotated by a per-tile unit quaternion (stateless RNG), quantised inside
-// its own bounding box, keyed by the 13-bit z-order cell, and sorted by (cell, position) with a
-// register/LDS bitonic network — a deterministic stand-in for the reference's LDS counting sort,
-// whose tie order depends on atomic arbitration.  Consecutive runs of S sorted points form a
+// its own bounding box, keyed by the 13-bit z-order cell, and sorted by (cell, position) with an LDS
+// counting sort over the 8192 cells, as the reference does (shmem_cumsum_counter.cuh:25-167), made
+// deterministic: the atomic claim only yields a point's place inside its cell's run in arbitration
+// order; a second look at the run (almost always one or two points long) replaces it by the number of
+// run members that come earlier in the input.  Consecutive runs of S sorted points form a
 // sub-bucket.  Tile t owns output rows [t * tile_pts / S, ...) of its cloud, so no global counter
 // is needed.  Every output is a pure function of (coords, seps, S, seed).
 #include "f3d_device.h"
@@ -17,49 +19,73 @@ namespace f3d {
 
 constexpr int kSubThreads = 1024;
 
-__device__ __forceinline__ void tile_quat(uint32_t seed, uint32_t cloud, uint32_t tile, float q[4]) {
-  float acc = 0.f;
-#pragma unroll
-  for (uint32_t i = 0; i < 4; ++i) {
-    q[i] = __fadd_rn(0.1f, __fmul_rn(rng_u01(seed, cloud, tile, i), 0.9f));
-    acc = __fadd_rn(acc, __fmul_rn(q[i], q[i]));
-  }
-  const float nrm = __fsqrt_rn(acc);
-#pragma unroll
-  for (int i = 0; i < 4; ++i) q[i] = __fdiv_rn(q[i], nrm);
-}
-
-// rotation by unit quaternion (w, x, y, z); every product and sum rounded separately
-__device__ __forceinline__ void quat_rotate(const float q[4], const float p[3], float out[3]) {
+// rotation by unit quaternion (w, x, y, z), every product and sum rounded separately: the nine coefficients ...
+__device__ __forceinline__ void quat_matrix(const float q[4], float m[9]) {
   const float w = q[0], x = q[1], y = q[2], z = q[3];
   const float n1 = __fmul_rn(x, 2.0f), n2 = __fmul_rn(y, 2.0f), n3 = __fmul_rn(z, 2.0f);
   const float n4 = __fmul_rn(x, n1), n5 = __fmul_rn(y, n2), n6 = __fmul_rn(z, n3);
   const float n7 = __fmul_rn(x, n2), n8 = __fmul_rn(x, n3), n9 = __fmul_rn(y, n3);
   const float n10 = __fmul_rn(w, n1), n11 = __fmul_rn(w, n2), n12 = __fmul_rn(w, n3);
-  const float a0 = __fmul_rn(__fsub_rn(1.0f, __fadd_rn(n5, n6)), p[0]);
-  const float a1 = __fmul_rn(__fsub_rn(n7, n12), p[1]);
-  const float a2 = __fmul_rn(__fadd_rn(n8, n11), p[2]);
-  const float b0 = __fmul_rn(__fadd_rn(n7, n12), p[0]);
-  const float b1 = __fmul_rn(__fsub_rn(1.0f, __fadd_rn(n4, n6)), p[1]);
-  const float b2 = __fmul_rn(__fsub_rn(n9, n10), p[2]);
-  const float c0 = __fmul_rn(__fsub_rn(n8, n11), p[0]);
-  const float c1 = __fmul_rn(__fadd_rn(n9, n10), p[1]);
-  const float c2 = __fmul_rn(__fsub_rn(1.0f, __fadd_rn(n4, n5)), p[2]);
-  out[0] = __fadd_rn(__fadd_rn(a0, a1), a2);
-  out[1] = __fadd_rn(__fadd_rn(b0, b1), b2);
-  out[2] = __fadd_rn(__fadd_rn(c0, c1), c2);
+  m[0] = __fsub_rn(1.0f, __fadd_rn(n5, n6));
+  m[1] = __fsub_rn(n7, n12);
+  m[2] = __fadd_rn(n8, n11);
+  m[3] = __fadd_rn(n7, n12);
+  m[4] = __fsub_rn(1.0f, __fadd_rn(n4, n6));
+  m[5] = __fsub_rn(n9, n10);
+  m[6] = __fsub_rn(n8, n11);
+  m[7] = __fadd_rn(n9, n10);
+  m[8] = __fsub_rn(1.0f, __fadd_rn(n4, n5));
+}
+
+// ... and their application to a point
+__device__ __forceinline__ void matrix_rotate(const float m[9], const float p[3], float out[3]) {
+#pragma unroll
+  for (int d = 0; d < 3; ++d)
+    out[d] = __fadd_rn(__fadd_rn(__fmul_rn(m[3 * d], p[0]), __fmul_rn(m[3 * d + 1], p[1])), __fmul_rn(m[3 * d + 2], p[2]));
+}
+
+// Monotone 16-bit key of an fp16 bit pattern (a < b as numbers <=> key(a) < key(b) as unsigned) and its inverse
+__device__ __forceinline__ uint32_t half_order_key(uint32_t h) { return (h & 0x8000u) ? (~h & 0xFFFFu) : (h | 0x8000u); }
+__device__ __forceinline__ uint32_t half_from_key(uint32_t k) { return (k & 0x8000u) ? (k & 0x7FFFu) : (~k & 0xFFFFu); }
+
+typedef unsigned short u16x2_t __attribute__((ext_vector_type(2)));
+// minimum of both 16-bit halves at once
+__device__ __forceinline__ uint32_t pk_min_u16(uint32_t a, uint32_t b) {
+  return __builtin_bit_cast(uint32_t, __builtin_elementwise_min(__builtin_bit_cast(u16x2_t, a), __builtin_bit_cast(u16x2_t, b)));
+}
+
+// Per-tile unit quaternion, one component per lane (lane % 4), so that the four draws, squares and divisions of the
+// rotation cost a wave one pass instead of four; every lane ends up with all four components.
+__device__ __forceinline__ void tile_quat_lanes(uint32_t seed, uint32_t cloud, uint32_t tile, uint32_t lane, float q[4]) {
+  const float mine = __fadd_rn(0.1f, __fmul_rn(rng_u01(seed, cloud, tile, lane & 3u), 0.9f));
+  float c[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) c[i] = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, mine), i));
+  float acc = 0.f;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) acc = __fadd_rn(acc, __fmul_rn(c[i], c[i]));
+  const float unit = __fdiv_rn(mine, __fsqrt_rn(acc));
+#pragma unroll
+  for (int i = 0; i < 4; ++i) q[i] = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, unit), i));
 }
 
 __global__ __launch_bounds__(kSubThreads) void subbuck_build_kernel(
     const uint16_t* __restrict__ coord, const uint32_t* __restrict__ batch_sep,
-    const uint32_t* __restrict__ reduced_batch_sep, uint32_t batch_size, uint32_t subbuck_size, uint32_t tile_pts,
-    uint32_t num_vox, uint32_t seed, uint32_t* __restrict__ subbuck_id, uint16_t* __restrict__ subbuck_off,
-    uint32_t* __restrict__ unpool_ind, uint16_t* __restrict__ reduced_coord, uint32_t reduced_n,
-    uint32_t reduced_aligned_n) {
-  __shared__ uint32_t s_key[kSubThreads];
-  __shared__ uint16_t s_xyz[kSubThreads][3];
-  __shared__ float s_red[6][kSubThreads / kWave];
-  __shared__ float s_bb[6];
+    const uint32_t* __restrict__ reduced_batch_sep, uint32_t batch_size, uint32_t total_n, uint32_t subbuck_size,
+    uint32_t tile_pts, uint32_t num_vox, uint32_t seed, uint32_t* __restrict__ subbuck_id,
+    uint16_t* __restrict__ subbuck_off, uint32_t* __restrict__ unpool_ind, uint16_t* __restrict__ reduced_coord,
+    uint32_t reduced_n, uint32_t reduced_aligned_n) {
+  // cell counters, then cell bases: two 16-bit fields per word (a tile has at most 1024 points), plus the end marker
+  constexpr uint32_t kCells = 8192u, kCellWords = kCells / 2u, kWaves = kSubThreads / kWave;
+  constexpr uint32_t kRunBytes = kWave * 6u, kArea = wave_run_area_bytes<kRunBytes>();
+  __shared__ __attribute__((aligned(16))) uint32_t s_cell[kCellWords + 4];
+  __shared__ __attribute__((aligned(16))) char s_rows[kWaves * kArea];   // the tile's 6-byte rows, a wave's 64 per area
+  __shared__ uint16_t s_claim[kSubThreads];   // run position (arbitration order) -> point
+  __shared__ uint16_t s_key[kSubThreads];     // rank (input order inside a run) -> point
+  __shared__ uint32_t s_red[kWaves][3];       // per wave: packed keys of the minima and (complemented) maxima
+  __shared__ uint32_t s_wsum[kWaves];
+  __shared__ float s_mat[9];                  // the tile's rotation
+  __shared__ float s_bb[9];                   // min, max, 1 / (max - min) per axis
   const uint32_t tid = threadIdx.x, cloud = blockIdx.y, tile = blockIdx.x;
 
   if (cloud == batch_size) {  // zero the alignment rows [reduced_n, reduced_aligned_n)
@@ -79,99 +105,206 @@ __global__ __launch_bounds__(kSubThreads) void subbuck_build_kernel(
   const uint32_t m = min(tile_pts, n - t0);
   const bool valid = tid < m;
   const size_t g = (size_t)start + t0 + tid;
+  const uint32_t w = __builtin_amdgcn_readfirstlane(tid / kWave), l = tid % kWave;
 
+  // The wave's 64 rows arrive as aligned 16-byte pieces in its LDS area (rows are 6 bytes apart: per-lane loads would
+  // be 2-byte accesses).  64 rows are a multiple of 16 bytes, so every wave's run starts at the same offset of its area.
+  const uint32_t wave0 = w * kWave;
+  const uint32_t rows = wave0 < m ? min((uint32_t)kWave, m - wave0) : 0u;
+  uint32_t shift = (uint32_t)((uintptr_t)(coord + 3 * ((size_t)start + t0)) & 15u);
+  if (rows) shift = wave_fetch_run<kRunBytes>(coord + 3 * ((size_t)start + t0 + wave0), rows * 6u, coord + 3 * (size_t)total_n,
+                                              s_rows + w * kArea, l);
+  auto row_of = [&](uint32_t j) {              // point j of the tile
+    return reinterpret_cast<const uint16_t*>(s_rows + (j / kWave) * kArea + shift + 6u * (j % kWave));
+  };
+  // thread t owns the counters of cells 8 t .. 8 t + 7 (four words) in the zero-fill and in the scan
+  uint4* const my_cells = reinterpret_cast<uint4*>(s_cell) + tid;
+  *my_cells = make_uint4(0u, 0u, 0u, 0u);
+  if (w == 0) {
+    // the tile's rotation, once per workgroup
+    float q[4], mat[9];
+    tile_quat_lanes(seed, cloud, tile, l, q);
+    quat_matrix(q, mat);
+    if (l < 9u) {
+      float mine = mat[0];
+#pragma unroll
+      for (int i = 1; i < 9; ++i) mine = l == (uint32_t)i ? mat[i] : mine;
+      s_mat[l] = mine;
+    }
+  }
+  __syncthreads();
   float p[3] = {0.f, 0.f, 0.f};
   if (valid) {
+    const uint16_t* h = row_of(tid);
 #pragma unroll
-    for (int d = 0; d < 3; ++d) {
-      const uint16_t h = coord[3 * g + d];
-      s_xyz[tid][d] = h;
-      p[d] = half_bits_to_float(h);
-    }
+    for (int d = 0; d < 3; ++d) p[d] = half_bits_to_float(h[d]);
   }
-  float q[4], r[3], rh[3];
-  tile_quat(seed, cloud, tile, q);
-  quat_rotate(q, p, r);
-  float mn[3], mx[3];
+  float mat[9], r[3], rh[3];
+#pragma unroll
+  for (int i = 0; i < 9; ++i) mat[i] = s_mat[i];
+  matrix_rotate(mat, p, r);
+  // Bounding box of the rotated tile.  The rotated coordinates are fp16 values: as monotone 16-bit keys, two to a
+  // register, with the maxima complemented, all six extremes are minima of three registers.
+  uint32_t k[3];
 #pragma unroll
   for (int d = 0; d < 3; ++d) {
-    rh[d] = half_bits_to_float(float_to_half_bits(r[d]));  // the rotated coordinate is an fp16 value
-    mn[d] = valid ? rh[d] : INFINITY;
-    mx[d] = valid ? rh[d] : -INFINITY;
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) {
-      mn[d] = fminf(mn[d], __shfl_xor(mn[d], off, kWave));
-      mx[d] = fmaxf(mx[d], __shfl_xor(mx[d], off, kWave));
-    }
+    const uint32_t hb = float_to_half_bits(r[d]);
+    rh[d] = half_bits_to_float((uint16_t)hb);
+    k[d] = half_order_key(hb);
   }
-  const uint32_t w = tid / kWave, l = tid % kWave;
+  uint32_t red[3] = {k[0] | (k[1] << 16), k[2] | ((~k[0]) << 16), (~k[1] & 0xFFFFu) | ((~k[2]) << 16)};
+#pragma unroll
+  for (int i = 0; i < 3; ++i) {
+    red[i] = valid ? red[i] : 0xFFFFFFFFu;
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) red[i] = pk_min_u16(red[i], __shfl_xor(red[i], off, kWave));
+  }
   if (l == 0) {
 #pragma unroll
-    for (int d = 0; d < 3; ++d) { s_red[d][w] = mn[d]; s_red[3 + d][w] = mx[d]; }
+    for (int i = 0; i < 3; ++i) s_red[w][i] = red[i];
   }
   __syncthreads();
-  if (tid < 6) {
-    float a = s_red[tid][0];
-    for (int i = 1; i < kSubThreads / kWave; ++i) a = tid < 3 ? fminf(a, s_red[tid][i]) : fmaxf(a, s_red[tid][i]);
-    s_bb[tid] = a;
+  if (w == 0) {
+    // the waves' extremes (16 lanes), then per axis the reciprocal of the extent, once per tile
+    uint32_t fin[3];
+#pragma unroll
+    for (int i = 0; i < 3; ++i) {
+      fin[i] = s_red[l & 15u][i];
+#pragma unroll
+      for (int off = 8; off > 0; off >>= 1) fin[i] = pk_min_u16(fin[i], __shfl_xor(fin[i], off, kWave));
+    }
+    if (l < 3u) {
+      const uint32_t kmin = l == 0u ? fin[0] & 0xFFFFu : l == 1u ? fin[0] >> 16 : fin[1] & 0xFFFFu;
+      const uint32_t kmax = ~(l == 0u ? fin[1] >> 16 : l == 1u ? fin[2] : fin[2] >> 16) & 0xFFFFu;
+      const float a = half_bits_to_float((uint16_t)half_from_key(kmin)), b = half_bits_to_float((uint16_t)half_from_key(kmax));
+      s_bb[l] = a;
+      s_bb[3u + l] = b;
+      s_bb[6u + l] = __fdiv_rn(1.0f, __fsub_rn(b, a));
+    }
   }
   __syncthreads();
 
-  uint32_t key = 0xFFFFFFFFu;
+  // ---- counting sort by cell ----
+  uint32_t cell = 0, claim = 0;
   if (valid) {
     uint32_t v[3];
 #pragma unroll
-    for (int d = 0; d < 3; ++d) v[d] = vox1(rh[d], make_vox_axis_f(s_bb[d], s_bb[3 + d], num_vox));
-    const uint32_t cell = zorder16(v[0], v[1], v[2]) >> 3;  // H_ZORDER_DIV with divisor 65536 / 8192
-    key = (cell << 10) | tid;
+    for (int d = 0; d < 3; ++d) v[d] = vox1(rh[d], make_vox_axis_inv(s_bb[d], s_bb[3 + d], s_bb[6 + d], num_vox));
+    cell = zorder16(v[0], v[1], v[2]) >> 3;  // H_ZORDER_DIV with divisor 65536 / 8192
+    const uint32_t sh = 16u * (cell & 1u);
+    claim = (atomicAdd(&s_cell[cell >> 1], 1u << sh) >> sh) & 0xFFFFu;
   }
-
-  // bitonic sort of one key per thread, ascending over the workgroup: partner distances below a
-  // wave go through lane exchange, larger ones through LDS
-  for (uint32_t k = 2; k <= kSubThreads; k <<= 1) {
-    for (uint32_t j = k >> 1; j > 0; j >>= 1) {
-      uint32_t other;
-      if (j >= kWave) {
-        s_key[tid] = key;
-        __syncthreads();
-        other = s_key[tid ^ j];
-        __syncthreads();
-      } else {
-        other = __shfl_xor(key, j, kWave);
-      }
-      const bool up = (tid & k) == 0;
-      const bool lower = (tid & j) == 0;
-      key = (lower == up) ? min(key, other) : max(key, other);
-    }
-  }
-  s_key[tid] = key;
   __syncthreads();
-
-  // thread `tid` now owns rank `tid`
+  {
+    // exclusive prefix over the 8192 counts: 8 per thread, then over the threads of a wave, then over the waves
+    const uint4 c = *my_cells;
+    const uint32_t cw[4] = {c.x, c.y, c.z, c.w};
+    uint32_t pre[8], run = 0;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      pre[2 * i] = run;
+      run += cw[i] & 0xFFFFu;
+      pre[2 * i + 1] = run;
+      run += cw[i] >> 16;
+    }
+    uint32_t incl = run;
+#pragma unroll
+    for (int off = 1; off < kWave; off <<= 1) {
+      const uint32_t up = __shfl_up(incl, off, kWave);
+      if (l >= (uint32_t)off) incl += up;
+    }
+    if (l == kWave - 1) s_wsum[w] = incl;
+    __syncthreads();
+    uint32_t base = incl - run;
+    {
+      const uint32_t part = l < w ? s_wsum[l] : 0u;        // sum over the waves before this one
+      uint32_t tot = part;
+#pragma unroll
+      for (int off = 8; off > 0; off >>= 1) tot += __shfl_xor(tot, off, kWave);
+      base += __builtin_amdgcn_readfirstlane(tot);
+    }
+    *my_cells = make_uint4((base + pre[0]) | ((base + pre[1]) << 16), (base + pre[2]) | ((base + pre[3]) << 16),
+                           (base + pre[4]) | ((base + pre[5]) << 16), (base + pre[6]) | ((base + pre[7]) << 16));
+    if (tid == kSubThreads - 1) s_cell[kCellWords] = m;   // "base" of the cell after the last one
+  }
+  __syncthreads();
+  uint32_t run0 = 0, run1 = 0;
+  if (valid) {
+    run0 = (s_cell[cell >> 1] >> (16u * (cell & 1u))) & 0xFFFFu;
+    run1 = (s_cell[(cell + 1u) >> 1] >> (16u * ((cell + 1u) & 1u))) & 0xFFFFu;
+    s_claim[run0 + claim] = (uint16_t)tid;
+  }
+  __syncthreads();
   const uint32_t S = subbuck_size;
   const uint32_t rows_per_tile = tile_pts / S;
   const uint32_t row_base = rstart + tile * rows_per_tile;
+  const bool pow2 = (S & (S - 1u)) == 0u;
+  const uint32_t s_log = 31u - (uint32_t)__builtin_clz(S);
   if (valid) {
-    const uint32_t j = key & 1023u;
-    const size_t gp = (size_t)start + t0 + j;
-    const uint32_t sub = tid / S, off = tid - sub * S;
-    subbuck_id[gp] = tile * rows_per_tile + sub;
-    subbuck_off[gp] = (uint16_t)off;
-    unpool_ind[(size_t)row_base * S + tid] = (uint32_t)gp;
+    // place inside the run = number of its members that come earlier in the input
+    uint32_t before = 0;
+    if (run1 - run0 > 1u)
+      for (uint32_t j = run0; j < run1; ++j) before += (uint32_t)s_claim[j] < tid ? 1u : 0u;
+    const uint32_t rank = run0 + before;
+    s_key[rank] = (uint16_t)tid;
+    // the point's own outputs, written by the point's thread: consecutive addresses
+    const uint32_t sub = pow2 ? rank >> s_log : rank / S;
+    subbuck_id[g] = tile * rows_per_tile + sub;
+    subbuck_off[g] = (uint16_t)(rank - sub * S);
   }
+  __syncthreads();
+
+  // thread `tid` now stands for rank `tid`
+  const uint32_t key = valid ? s_key[tid] : 0u;
+  if (valid) unpool_ind[(size_t)row_base * S + tid] = (uint32_t)((size_t)start + t0 + key);
   // mean coordinate of every sub-bucket, members summed in rank order
-  const uint32_t nrow = (m + S - 1) / S;
-  if (tid < nrow) {
-    const uint32_t cnt = min(S, m - tid * S);
-    float acc[3] = {0.f, 0.f, 0.f};
-    for (uint32_t s = 0; s < cnt; ++s) {
-      const uint32_t j = s_key[tid * S + s] & 1023u;
+  if (pow2 && S <= (uint32_t)kWave) {
+    // a sub-bucket's ranks are neighbouring lanes of one wave: its first lane adds the others' coordinates one by one
+    float x[3] = {0.f, 0.f, 0.f}, acc[3];
+    if (valid) {
+      const uint16_t* h = row_of(key);
 #pragma unroll
-      for (int d = 0; d < 3; ++d) acc[d] = __fadd_rn(acc[d], half_bits_to_float(s_xyz[j][d]));
+      for (int d = 0; d < 3; ++d) x[d] = half_bits_to_float(h[d]);
     }
-    uint16_t* out = reduced_coord + 3 * (size_t)(row_base + tid);
 #pragma unroll
-    for (int d = 0; d < 3; ++d) out[d] = float_to_half_bits(__fdiv_rn(acc[d], (float)cnt));
+    for (int d = 0; d < 3; ++d) acc[d] = __fadd_rn(0.f, x[d]);
+    for (uint32_t s = 1; s < S; ++s) {
+      const bool take = tid + s < m;
+#pragma unroll
+      for (int d = 0; d < 3; ++d) {
+        const float v = __shfl_down(x[d], s, kWave);
+        if (take) acc[d] = __fadd_rn(acc[d], v);
+      }
+    }
+    if (valid && (tid & (S - 1u)) == 0u) {
+      const uint32_t sub = tid >> s_log;
+      const uint32_t cnt = min(S, m - tid);
+      uint16_t* out = reduced_coord + 3 * (size_t)(row_base + sub);
+      if (cnt == S) {
+        // a full group: S is a power of two, so the division is an exact scaling (sums of fp16 values are far from
+        // the subnormal range of fp32)
+        const float inv_s = __builtin_bit_cast(float, (127u - s_log) << 23);
+#pragma unroll
+        for (int d = 0; d < 3; ++d) out[d] = float_to_half_bits(__fmul_rn(acc[d], inv_s));
+      } else {
+#pragma unroll
+        for (int d = 0; d < 3; ++d) out[d] = float_to_half_bits(__fdiv_rn(acc[d], (float)cnt));
+      }
+    }
+  } else {
+    const uint32_t nrow = (m + S - 1) / S;
+    if (tid < nrow) {
+      const uint32_t cnt = min(S, m - tid * S);
+      float acc[3] = {0.f, 0.f, 0.f};
+      for (uint32_t s = 0; s < cnt; ++s) {
+        const uint16_t* h = row_of(s_key[tid * S + s]);
+#pragma unroll
+        for (int d = 0; d < 3; ++d) acc[d] = __fadd_rn(acc[d], half_bits_to_float(h[d]));
+      }
+      uint16_t* out = reduced_coord + 3 * (size_t)(row_base + tid);
+#pragma unroll
+      for (int d = 0; d < 3; ++d) out[d] = float_to_half_bits(__fdiv_rn(acc[d], (float)cnt));
+    }
   }
 }
 
@@ -286,7 +419,6 @@ int f3d_subbuck_build(const f3d_half_t* coord, const uint32_t* batch_sep, uint32
                       uint32_t reduced_aligned_n, uint32_t* unpool_ind, uint32_t reduced_n, int device,
                       void* stream) {
   using namespace f3d;
-  (void)total_n;
   F3D_CHECK_ARG(subbuck_size >= 1 && subbuck_size <= 1024, "subbuck_size=%u outside [1, 1024]", subbuck_size);
   F3D_CHECK_ARG(num_vox >= 2 && num_vox <= 0x10000u, "num_vox=%u does not fit the 16-bit voxel type", num_vox);
   F3D_CHECK_ARG(reduced_aligned_n >= reduced_n, "reduced buffer length(%u) is smaller than the reduced row count(%u)",
@@ -303,7 +435,8 @@ int f3d_subbuck_build(const f3d_half_t* coord, const uint32_t* batch_sep, uint32
   if (gx == 0 || (batch_size == 0 && pad_tiles == 0)) return F3D_OK;
   SyncBracket sync(s);
   hipLaunchKernelGGL(subbuck_build_kernel, dim3(gx, batch_size + (pad_tiles ? 1 : 0)), dim3(kSubThreads), 0, s, coord,
-                     batch_sep, reduced_batch_sep, batch_size, subbuck_size, tile_pts, num_vox | quantiser_bit(), global_seed(),
+                     batch_sep, reduced_batch_sep, batch_size, total_n, subbuck_size, tile_pts, num_vox | quantiser_bit(),
+                     global_seed(),
                      subbuck_id, subbuck_off, unpool_ind, reduced_coord, reduced_n, reduced_aligned_n);
   F3D_CHECK_HIP(hipGetLastError());
   return F3D_OK;

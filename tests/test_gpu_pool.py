@@ -46,6 +46,27 @@ def test_builder_and_reduce_bit_exact(oracle, S, op, sizes, C):
     assert np.array_equal(n_bf16_bits(sb.reduced_feat), want), "reduced features differ"
 
 
+def test_builder_long_runs_of_one_cell_bit_exact(oracle):
+    """Clouds whose points share few distinct positions (one position only; three; a 2000-point cloud of 40 positions):
+    whole tiles fall into one or a few cells of the counting sort, so the order inside a cell's run (input order) is
+    what decides every output."""
+    rng = np.random.default_rng(77)
+    same = np.tile(np.array([[1.5, -2.25, 0.75]]), (1500, 1))
+    three = np.array([[0.0, 0.0, 0.0], [10.0, -3.0, 2.0], [-7.0, 4.0, 1.0]])[rng.integers(0, 3, 1100)]
+    forty = rng.uniform(-20, 20, (40, 3))[rng.integers(0, 40, 2000)]
+    coords = np.concatenate([same, three, forty]).astype(np.float16)
+    seps = np.cumsum([1500, 1100, 2000]).astype(np.uint32)
+    feat = bf16_bits(rng.normal(0, 1, (coords.shape[0], 16)))
+    for S in (2, 8):
+        sb = _pool(coords, seps, feat, S, 0, 1, oracle)
+        sub_id, sub_off, unpool, red_coord, _ = oracle.subbuck_build(coords, seps, S)
+        assert np.array_equal(n_u32(sb.unpool_ind), unpool), "inverse map differs"
+        assert np.array_equal(n_u32(sb.subbuck_id), sub_id) and np.array_equal(n_u16(sb.subbuck_off), sub_off)
+        assert np.array_equal(n_f16(sb.reduced_coord).view(np.uint16), red_coord.view(np.uint16))
+        # one position only: the cloud's rows come out in input order
+        assert np.array_equal(unpool[:1500 // S].reshape(-1), np.arange(1500 // S * S))
+
+
 def test_c3_pool_unpool_full_size(oracle):
     """BASELINE config 3: 262,144 points x 128 channels, S=8 (2x2x2), mean and max, then unpool"""
     import bench_workloads as synth
