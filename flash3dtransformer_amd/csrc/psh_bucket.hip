@@ -235,8 +235,11 @@ __host__ __device__ constexpr size_t psh_scatter_lds_bytes(uint32_t num_bucket) 
   return (head + tables + tail) * sizeof(uint32_t);
 }
 
+// The large-tile configuration must fit eight waves per SIMD (at most 64 registers): its 1024-thread workgroups
+// then run two to a CU.  With a few registers more a CU holds a single workgroup and the launch takes a third longer
+// (measured: 173 against 127 us on 64 x 262,144 points).
 template <int THREADS, int ITEMS, bool REBAL, bool STAGE>
-__global__ __launch_bounds__(THREADS) void psh_rank_scatter_kernel(
+__global__ __launch_bounds__(THREADS, (STAGE ? 8 : 1)) void psh_rank_scatter_kernel(
     const uint16_t* __restrict__ coord, uint16_t* __restrict__ bucket_id,
     uint32_t* __restrict__ bucket_offset, const uint32_t* __restrict__ batch_sep, uint32_t batch_size,
     const uint32_t* __restrict__ tile_base, const uint32_t* __restrict__ bucket_counter,
