@@ -250,7 +250,7 @@ def sub_metrics(dev, only=None):
     unpooling GB/s on config 3 — each against its roofline.  `only`: a set of group names, or None for all"""
     out = {}
     groups = {"attention": sub_attention, "psh": sub_psh, "permute": sub_permute, "pool": sub_pool,
-              "hourglass": lambda d, o: o.__setitem__("hourglass_c5", hourglass_c5(d)), "mfma": sub_mfma_rate,
+              "hourglass": sub_hourglass, "mfma": sub_mfma_rate,
               "backward": sub_backward}
     for name, fn in groups.items():
         if only is None or name in only:
@@ -266,6 +266,11 @@ def _bench_probe():
     if not os.path.exists(path):
         raise RuntimeError(f"{path} is missing: run `python __graft_entry__.py` first")
     return ctypes.CDLL(path)
+
+
+def sub_hourglass(dev, out):
+    out["hourglass_c5"] = hourglass_c5(dev)
+    out["hourglass_c5_ref_shape"] = hourglass_c5(dev, ref_shape=True)
 
 
 def sub_mfma_rate(dev, out):
@@ -564,16 +569,19 @@ def _pool_case(dev, out, n, tag, iters):
     del coords, feat, res, up, sb
 
 
-def hourglass_c5(dev):
+def hourglass_c5(dev, ref_shape=False):
     """whole-model forward, config 5: 4 sweeps x 250,000 points, 5 levels C = 32/64/128/256/512, heads = C/32,
     bucket 512, scope of 1 bucket, pooling S = 2 (mean), swiglu MLP with hidden = 4C, hash 2.
+    `ref_shape`: the shape of the reference's own model test instead (scopes of 8 buckets, two encoder + two decoder
+    blocks per level, eval-mode BatchNorm1d + GELU around pooling / unpooling, pooled lengths aligned to bucket x scope).
     `ms`: wall time per forward, forwards queued back to back.  `host_enqueue_ms`: the time the host needs to queue
     one forward (the call returns before the GPU is done): below `ms`, the host runs ahead and per-call marshalling
     is not what the GPU waits for.  `gpu_busy_ms`: the sum of the kernel durations of one forward, from the
     profiler's kernel records (None when the profiler is not usable, e.g. under an outer tracer); `ms` minus it is
     the idle time between consecutive kernels."""
     import bench_workloads as configs
-    model = configs.hourglass(1005).to(dev).eval()
+    model = (configs.hourglass_ref_shape(1005) if ref_shape else configs.hourglass(1005)).to(dev).eval()
+    cfg = configs.HOURGLASS_REF_SHAPE if ref_shape else configs.HOURGLASS
     coords_np, seps_np, _ = configs.lidar_batch(4, 250_000, 1005)
     coords, seps = configs.to_device(coords_np, seps_np, dev)
     with torch.no_grad():
@@ -607,7 +615,8 @@ def hourglass_c5(dev):
     return {"ms": round(ms, 3), "host_enqueue_ms": round(enqueue_ms, 3),
             "gpu_busy_ms": None if busy is None else round(busy, 3),
             "launches_per_forward": n_kernels, "mpts_per_s": round(coords.shape[0] / ms / 1e3, 1), "points": int(coords.shape[0]),
-            "levels": list(configs.HOURGLASS["channels"]), "subbuck_size": configs.HOURGLASS["subbuck_size"],
+            "levels": list(cfg["channels"]), "subbuck_size": cfg["subbuck_size"], "scope_size": cfg["scope_size"],
+            "blocks_per_level": "2 + 2" if ref_shape else "1 + 1",
             "finite": bool(torch.isfinite(out.float()).all().item())}
 
 

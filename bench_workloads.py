@@ -124,6 +124,49 @@ def hourglass(seed=1005, channels=None, bucket_size=None, subbuck_size=None):
     return model.eval()
 
 
+HOURGLASS_REF_SHAPE = dict(channels=(32, 64, 128, 256, 512), bucket_size=512, scope_size=8, hash_type=2, subbuck_size=2)
+
+
+def hourglass_ref_shape(seed=1005, channels=None):
+    """Flash3D in the shape of the reference's own model test (tests/test_psh_hourglass.py:55-150 of the reference),
+    extended to five levels: scopes of 8 buckets of 512, two encoder and two decoder blocks per level (the first
+    encoder block of the first level on the "stride" plan, the others on "swin"), BatchNorm1d(eps=1e-3, momentum=0.01) +
+    GELU around pooling and unpooling, pooled lengths aligned to bucket x scope, mean pooling over 2 points, gated MLP
+    with 4 C hidden features.  Heads = C / 32 (the benchmark's head width; the reference's test uses 16-wide heads)."""
+    from functools import partial
+    from flash3dtransformer_amd import layers as L
+    from flash3dtransformer_amd.psh.bucket_scope import SwinPlan, swinable_alignment
+    c = HOURGLASS_REF_SHAPE
+    chans = list(channels or c["channels"])
+    bs, scope, S = c["bucket_size"], c["scope_size"], c["subbuck_size"]
+    torch.manual_seed(seed)
+    ln = lambda ch: L.LayerNorm(ch)
+    bn = partial(torch.nn.BatchNorm1d, eps=1e-3, momentum=0.01)
+    spec = lambda ch, plan, k: L.XFMRSpecs(ch, 4 * ch, ch // 32, True, SwinPlan(plan, bs, scope, k), ln)
+    levels = []
+    for i, ch in enumerate(chans):
+        last = i + 1 == len(chans)
+        levels.append(L.F3DLevelSpecs([spec(ch, "stride" if i == 0 else "swin", 1), spec(ch, "swin", 2)],
+                                      [spec(ch, "swin", 3), spec(ch, "swin", 4)], "mean", swinable_alignment(bs, scope),
+                                      None if last else bn, None if last else torch.nn.GELU,
+                                      None if last else bn, None if last else torch.nn.GELU))
+    model = L.Flash3D(levels, bs, scope, c["hash_type"], subbuck_size=S)
+    g = torch.Generator().manual_seed(seed)
+    for m in model.modules():                      # running statistics and affine parameters that matter
+        if isinstance(m, torch.nn.BatchNorm1d):
+            m.running_mean.copy_(torch.randn(m.num_features, generator=g) * 0.1)
+            m.running_var.copy_(torch.rand(m.num_features, generator=g) + 0.5)
+            m.weight.data.copy_(torch.rand(m.num_features, generator=g) + 0.5)
+            m.bias.data.copy_(torch.randn(m.num_features, generator=g) * 0.1)
+    for p in model.parameters():
+        p.data = p.data.to(torch.bfloat16).float()
+    return model.eval()
+
+
+def _act_name(act):
+    return {None: None, torch.nn.GELU: "gelu", torch.nn.ReLU: "relu"}[act]
+
+
 def hourglass_oracle_levels(model):
     """the per-level description oracle-side restatements of the model take (heads, block counts, pooling)"""
     out = []
@@ -131,7 +174,7 @@ def hourglass_oracle_levels(model):
         out.append(dict(heads=spec.encoder_specs[0].num_heads, n_enc=len(spec.encoder_specs),
                         n_dec=len(spec.decoder_specs), red_op={"mean": 0, "sum": 1, "min": 2, "max": 3}.get(
                             spec.reduction_op, spec.reduction_op), pool_align=spec.pool_align,
-                        pool_act=None, unpool_act=None))
+                        pool_act=_act_name(spec.pool_act), unpool_act=_act_name(spec.unpool_act)))
     return out
 
 

@@ -384,6 +384,7 @@ int f3d_linear_bf16(const f3d_bf16_t* x, uint32_t ldx, const f3d_bf16_t* w, cons
                     const f3d_bf16_t* residual, uint32_t ldr, f3d_bf16_t* y, uint32_t ldy, uint32_t m, uint32_t n,
                     uint32_t k, uint32_t act, int device, void* stream) {
   using namespace f3d;
+  StagedWeightsScope staged;
   F3D_CHECK_ARG(x && w && y, "null tensor pointer");
   F3D_CHECK_ARG(act <= F3D_ACT_RELU, "unknown activation id %u", act);
   const uint32_t n_out = act == F3D_ACT_SWIGLU ? n / 2 : n;
@@ -414,6 +415,7 @@ int f3d_ln_linear_bf16(const f3d_bf16_t* x, uint32_t ldx, const f3d_bf16_t* gamm
                        f3d_bf16_t* y, uint32_t ldy, uint32_t m, uint32_t n, uint32_t k, uint32_t act, int device,
                        void* stream) {
   using namespace f3d;
+  StagedWeightsScope staged;
   F3D_CHECK_ARG(x && gamma && w && y, "null tensor pointer");
   F3D_CHECK_ARG(act <= F3D_ACT_RELU, "unknown activation id %u", act);
   const uint32_t n_out = act == F3D_ACT_SWIGLU ? n / 2 : n;

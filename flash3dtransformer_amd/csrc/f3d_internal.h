@@ -19,6 +19,16 @@ void set_error(const char* fmt, ...) __attribute__((format(printf, 1, 2)));
 // Returns nullptr (and sets the error) on allocation failure.
 void* workspace(int device, size_t bytes);
 
+// Device memory for the weights a dense op prepares per call (LayerNorm folded into the weight, fragment-major
+// copies): the buffer the caller staged with f3d_stage_weights for this call, else the per-device workspace.
+// *ready: the staged buffer already holds this call's prepared weights, the preparation launch is skipped.
+// nullptr + error message when the staged buffer is too small or the workspace cannot grow.
+void* weight_area(int device, size_t bytes, bool* ready);
+// Declared at the top of every dense entry point: whatever the call does, the staging ends with it.
+struct StagedWeightsScope {
+  ~StagedWeightsScope();
+};
+
 // This device's copy of the fixed scratch array behind f3d_batch_psh_scatter_pad_hash_noalloc (resolved on the first
 // call per device; f3d_init_dev_info does it ahead of time).  nullptr + error message on failure.
 uint32_t* psh_noalloc_scratch(int device);

@@ -59,6 +59,28 @@ void* workspace(int device, size_t bytes) {
   return p;
 }
 
+// weights staged by the caller for the next dense call on this thread (f3d_stage_weights)
+static thread_local struct {
+  void* buf = nullptr;
+  size_t bytes = 0;
+  bool ready = false, armed = false;
+} g_staged;
+
+void* weight_area(int device, size_t bytes, bool* ready) {
+  *ready = false;
+  if (g_staged.armed) {
+    if (g_staged.bytes < bytes) {
+      set_error("the buffer given to f3d_stage_weights holds %zu bytes, this call prepares %zu", g_staged.bytes, bytes);
+      return nullptr;
+    }
+    *ready = g_staged.ready;
+    return g_staged.buf;
+  }
+  return workspace(device, bytes);
+}
+
+StagedWeightsScope::~StagedWeightsScope() { g_staged.armed = false; }
+
 bool sync_stream_enabled() { return g_sync; }
 uint32_t global_seed() { return g_seed; }
 int rebalance_mode() { return g_rebalance; }
@@ -114,5 +136,17 @@ int f3d_set_quantiser(int mode) {
 }
 
 int f3d_get_quantiser(void) { return f3d::g_quantiser; }
+
+int f3d_stage_weights(void* buf, size_t bytes, int ready) {
+  if (!buf || ((uintptr_t)buf & 255u) != 0) {
+    f3d::set_error("f3d_stage_weights needs a 256-byte aligned device buffer");
+    return F3D_ERR_INVALID;
+  }
+  f3d::g_staged.buf = buf;
+  f3d::g_staged.bytes = bytes;
+  f3d::g_staged.ready = ready != 0;
+  f3d::g_staged.armed = true;
+  return F3D_OK;
+}
 
 }  // extern "C"

@@ -601,6 +601,7 @@ int f3d_ln_mlp_swiglu_bf16(const f3d_bf16_t* x, uint32_t ldx, const f3d_bf16_t* 
                            const f3d_bf16_t* residual, uint32_t ldr, f3d_bf16_t* y, uint32_t ldy, uint32_t m,
                            uint32_t c, uint32_t hidden, int device, void* stream) {
   using namespace f3d;
+  StagedWeightsScope staged;
   F3D_CHECK_ARG(x && gamma && w1 && w2 && y, "null tensor pointer");
   const bool narrow = c == 32 || c == 64;
   if (!(narrow || c == 128 || c == 256) || hidden == 0 || hidden % 32 != 0 || (uint64_t)hidden * c * 4 >= (1ull << 32) ||
@@ -623,7 +624,8 @@ int f3d_ln_mlp_swiglu_bf16(const f3d_bf16_t* x, uint32_t ldx, const f3d_bf16_t* 
   // bias [C]
   const size_t w1_bytes = (size_t)2 * hidden * c * 2, b32_bytes = (((size_t)2 * hidden * 4) + 255) & ~(size_t)255;
   const size_t w2_bytes = (size_t)hidden * c * 2;
-  char* ws = (char*)workspace(device, w1_bytes + b32_bytes + w2_bytes + (size_t)c * 2);
+  bool ready = false;
+  char* ws = (char*)weight_area(device, w1_bytes + b32_bytes + w2_bytes + (size_t)c * 2, &ready);
   if (!ws) return F3D_ERR_RUNTIME;
   uint16_t* w1p = (uint16_t*)ws;
   float* b32 = (float*)(ws + w1_bytes);
@@ -631,8 +633,9 @@ int f3d_ln_mlp_swiglu_bf16(const f3d_bf16_t* x, uint32_t ldx, const f3d_bf16_t* 
   uint16_t* zero_bias = (uint16_t*)(ws + w1_bytes + b32_bytes + w2_bytes);
   if (!b2) b2 = zero_bias;
   const uint32_t fold_blocks = cdiv_u32(2 * hidden, 4);
-  hipLaunchKernelGGL(mlp_prep_kernel, dim3(fold_blocks + cdiv_u32(c * hidden / 8, 256)), dim3(256), 0, s, w1, gamma, beta, b1,
-                     w1p, b32, fold_blocks, w2, w2p, zero_bias, c, hidden);
+  if (!ready)
+    hipLaunchKernelGGL(mlp_prep_kernel, dim3(fold_blocks + cdiv_u32(c * hidden / 8, 256)), dim3(256), 0, s, w1, gamma, beta, b1,
+                       w1p, b32, fold_blocks, w2, w2p, zero_bias, c, hidden);
   int rc;
   if (c == 256) rc = launch_mlp<256>(x, ldx, eps, w1p, b32, w2p, b2, residual, ldr, y, ldy, m, hidden, device, s);
   else if (c == 32) rc = launch_mlp_small<32>(x, ldx, eps, w1p, b32, w2p, b2, residual, ldr, y, ldy, m, hidden, device, s);

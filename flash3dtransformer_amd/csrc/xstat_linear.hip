@@ -422,13 +422,14 @@ int launch_xstat_linear(const uint16_t* x, uint32_t ldx, const uint16_t* gamma, 
   if ((uint64_t)N * K * 2 >= (1ull << 32)) return F3D_ERR_UNSUPPORTED;   // 32-bit byte offsets into w
   const uint16_t* lnx = nullptr;
   if (ln) {
-    // per call: w' (bf16 [N][K]) and b' (fp32 [N]) in the per-device workspace
+    // w' (bf16 [N][K]) and b' (fp32 [N]): per call in the per-device workspace, or kept in the caller's staged buffer
     const size_t wp_bytes = ((size_t)N * K * 2 + 255) & ~(size_t)255;
-    char* ws = (char*)workspace(device, wp_bytes + (size_t)N * 4);
+    bool ready = false;
+    char* ws = (char*)weight_area(device, wp_bytes + (size_t)N * 4, &ready);
     if (!ws) return F3D_ERR_RUNTIME;
     uint16_t* wp = (uint16_t*)ws;
     float* b32 = (float*)(ws + wp_bytes);
-    launch_ln_fold(w, gamma, beta, bias, wp, b32, N, K, s);
+    if (!ready) launch_ln_fold(w, gamma, beta, bias, wp, b32, N, K, s);
     w = wp;
     lnx = (const uint16_t*)b32;   // the kernel reads b' from here
   }

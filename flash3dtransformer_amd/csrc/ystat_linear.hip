@@ -219,11 +219,12 @@ int launch_ystat_linear(const uint16_t* x, uint32_t ldx, const uint16_t* w, cons
     return F3D_ERR_UNSUPPORTED;
   if ((uint64_t)N * K * 2 >= (1ull << 32) || (uint64_t)256 * ldx * 2 >= (1ull << 31)) return F3D_ERR_UNSUPPORTED;
   const size_t wp_bytes = (size_t)N * K * 2;
-  char* ws = (char*)workspace(device, wp_bytes + (size_t)N * 2);
+  bool ready = false;
+  char* ws = (char*)weight_area(device, wp_bytes + (size_t)N * 2, &ready);
   if (!ws) return F3D_ERR_RUNTIME;
   uint16_t* wp = (uint16_t*)ws;
   uint16_t* zero_bias = (uint16_t*)(ws + wp_bytes);
-  hipLaunchKernelGGL(ys_w_prep_kernel, dim3(cdiv_u32(N * (K / 8), 256)), dim3(256), 0, s, w, wp, zero_bias, N, K);
+  if (!ready) hipLaunchKernelGGL(ys_w_prep_kernel, dim3(cdiv_u32(N * (K / 8), 256)), dim3(256), 0, s, w, wp, zero_bias, N, K);
   if (!bias) bias = zero_bias;
   if (N == 256) return launch_ys<256>(x, ldx, wp, bias, residual, ldr, y, ldy, M, K, device, s);
   return launch_ys<128>(x, ldx, wp, bias, residual, ldr, y, ldy, M, K, device, s);

@@ -114,16 +114,48 @@ class _Bf16Cache:
         return self._val
 
 
+class _StagedWeights:
+    """Device buffer in which a dense kernel keeps the weights it prepares per call (LayerNorm folded into the weight
+    and bias, fragment-major copies) between eval-mode forwards under no_grad.  The buffer is current while the bf16
+    tensors it was made from are the same storage at the same version (the entry holds them, so their memory cannot
+    be handed out again meanwhile); dropped together with the bf16 copies (train() / eval(), load_state_dict,
+    refresh_weights())."""
+
+    def __init__(self):
+        self._key = None
+        self._src = None
+        self._buf = None
+
+    def clear(self):
+        self._key = self._src = None
+
+    def arm(self, training: bool, rows: int, cols: int, *tensors, tag=None):
+        """call right before the dense op: stages the buffer for it (no-op while weights may change)"""
+        if training or torch.is_grad_enabled():
+            self.clear()
+            return
+        live = [t for t in tensors if t is not None]
+        key = (tag, rows, cols) + tuple((t.data_ptr(), t._version, tuple(t.shape)) for t in live)
+        need = 3 * rows * cols + 4 * rows + 2 * cols + 512
+        dev = live[0].device
+        if self._buf is None or self._buf.numel() < need or self._buf.device != dev:
+            self._buf = torch.empty(need, dtype=torch.uint8, device=dev)
+            self._key = None
+        ready = key == self._key
+        pshattn.stage_weights(self._buf, ready)
+        self._key, self._src = key, live
+
+
 class _CachedParamModule(nn.Module):
     """nn.Module whose kernels read bf16 copies of its parameters (`_Bf16Cache` attributes or lists of them)"""
 
     def _bf16_caches(self):
         for v in self.__dict__.values():
-            if isinstance(v, _Bf16Cache):
+            if isinstance(v, (_Bf16Cache, _StagedWeights)):
                 yield v
             elif isinstance(v, (list, tuple)):
                 for c in v:
-                    if isinstance(c, _Bf16Cache):
+                    if isinstance(c, (_Bf16Cache, _StagedWeights)):
                         yield c
 
     def refresh_weights(self):
@@ -309,6 +341,7 @@ class Linear(_CachedParamModule):
         self.weight = nn.Parameter(torch.empty(out_features, in_features))
         self.bias = nn.Parameter(torch.empty(out_features)) if bias else None
         self._w, self._b = _Bf16Cache(), _Bf16Cache()
+        self._staged = _StagedWeights()
         self.reset_parameters()
 
     def reset_parameters(self):
@@ -329,8 +362,13 @@ class Linear(_CachedParamModule):
         g = b = None
         if pre_norm is not None:
             g, b = norm_params_bf16(pre_norm)
+            if isinstance(pre_norm, LayerNorm):     # its bf16 copies are kept between calls, a torch norm's are not
+                self._staged.arm(self.training or pre_norm.training, self.out_features, self.in_features, w16, b16, g, b,
+                                 tag=("ln", float(pre_norm.eps)))
             pshattn.ln_linear_bf16(x2, g, b, pre_norm.eps, w16, b16, r2, y, act)
         else:
+            if self.in_features > 512:     # long inner dimension: the output-panel kernel re-lays the weight
+                self._staged.arm(self.training, self.out_features, self.in_features, w16, b16, tag="ys")
             pshattn.linear_bf16(x2, w16, b16, r2, y, act)
         ln_w = None if pre_norm is None else pre_norm.weight
         ln_b = None if pre_norm is None else pre_norm.bias
@@ -481,6 +519,7 @@ class LayerNormMLP(_CachedParamModule):
         nn.init.normal_(self.fc1_weight, std=0.023)
         nn.init.normal_(self.fc2_weight, std=0.023)
         self._c = [_Bf16Cache() for _ in range(6)]
+        self._staged = [_StagedWeights(), _StagedWeights()]      # fused kernel / fc1 of the two-kernel path; fc2
 
     def forward(self, x: torch.Tensor, residual: torch.Tensor = None):
         x2 = as_bf16_2d(x.reshape(-1, self.hidden_size)).contiguous()
@@ -491,17 +530,24 @@ class LayerNormMLP(_CachedParamModule):
         # on request, the whole gated MLP in one kernel where one exists (hidden activations stay in registers) ...
         want_fused = self.fused if self.fused is not None else (self.hidden_size <= 128 or x2.shape[0] >= 30000)
         fused = (want_fused and self.activation == "swiglu" and self.hidden_size in FUSED_MLP_WIDTHS
-                 and self.ffn_hidden_size % 32 == 0
-                 and pshattn.ln_mlp_swiglu_bf16(x2, g16, be16, self.eps, w1_16, b1_16, w2_16, b2_16, r2, y))
+                 and self.ffn_hidden_size % 32 == 0)
+        if fused:
+            self._staged[0].arm(self.training, w1_16.shape[0], self.hidden_size, g16, be16, w1_16, b1_16, w2_16, b2_16,
+                                tag=("mlp", float(self.eps)))
+            fused = pshattn.ln_mlp_swiglu_bf16(x2, g16, be16, self.eps, w1_16, b1_16, w2_16, b2_16, r2, y)
         if not fused:
             # ... otherwise LayerNorm + fc1 + activation, then fc2 + residual
             h = torch.empty(x2.shape[0], self.ffn_hidden_size, dtype=torch.bfloat16, device=x.device)
             if self.hidden_size in FUSABLE_LN_WIDTHS:
+                self._staged[0].arm(self.training, w1_16.shape[0], self.hidden_size, g16, be16, w1_16, b1_16,
+                                    tag=("fc1", float(self.eps)))
                 pshattn.ln_linear_bf16(x2, g16, be16, self.eps, w1_16, b1_16, None, h, self.activation)
             else:
                 ln = torch.empty_like(x2)
                 pshattn.layernorm_bf16(x2, g16, be16, ln, self.eps)
                 pshattn.linear_bf16(ln, w1_16, b1_16, None, h, self.activation)
+            if self.ffn_hidden_size > 512:
+                self._staged[1].arm(self.training, self.hidden_size, self.ffn_hidden_size, w2_16, b2_16, tag="ys")
             pshattn.linear_bf16(h, w2_16, b2_16, r2, y, None)
         x_in = x.reshape(-1, self.hidden_size)
         res_in = None if residual is None else residual.reshape(-1, self.hidden_size)

@@ -554,6 +554,14 @@ def ln_mlp_swiglu_bf16(x, gamma, beta, eps, w1, b1, w2, b2, residual, y) -> bool
     return True
 
 
+def stage_weights(buf: torch.Tensor, ready: bool):
+    """extension: the next dense call on this thread keeps the weights it prepares (LayerNorm fold, fragment-major
+    copies) in `buf` (uint8 device tensor, 256-byte aligned), or with `ready` reuses what an earlier call with the same
+    weights left there and skips the preparation launch"""
+    assert_dtype([buf], torch.uint8)
+    _check(_load().f3d_stage_weights(_ptr(buf), ctypes.c_size_t(buf.numel()), _i32(1 if ready else 0)))
+
+
 def layernorm_bf16(x, gamma, beta, y, eps=1e-5):
     """extension: LayerNorm over the last axis, fp32 statistics"""
     assert_contiguous([x, gamma, y])

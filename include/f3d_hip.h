@@ -19,6 +19,7 @@
 #ifndef F3D_HIP_H
 #define F3D_HIP_H
 
+#include <stddef.h>
 #include <stdint.h>
 
 #ifdef __cplusplus
@@ -244,6 +245,17 @@ int f3d_buck_swin_fwd_strided(const f3d_bf16_t* q, const f3d_bf16_t* k, const f3
                               const uint32_t* scope_buckets, uint32_t num_scope, uint32_t scope_size,
                               uint32_t bucket_size, uint32_t batch, uint32_t seq_len, uint32_t num_head,
                               uint32_t head_dim, const int32_t* kv_len, int device, void* stream);
+
+/* ---- frozen weights (extension; the reference leaves its dense layers to torch / TransformerEngine) -----------
+ * f3d_ln_linear_bf16, f3d_ln_mlp_swiglu_bf16 and f3d_linear_bf16 (long inner dimension) first prepare their weights
+ * (LayerNorm folded into the weight and bias, fragment-major copies): one small launch per call, into the library's
+ * workspace.  A caller whose weights do not change between calls (inference) stages a buffer of its own instead:
+ * the NEXT dense call on this thread prepares into `buf` (device memory, 256-byte aligned, `bytes` long; for a
+ * weight of n rows and k columns 3 n k + 4 n + 2 k + 512 bytes cover every case, with n = the fc1 rows for the
+ * gated MLP), or, with ready != 0, takes what an earlier call with the same weights and shapes left there and skips
+ * the preparation launch.  The staging ends with that call whatever its outcome.  A buffer that is too small makes
+ * the call fail with a message. */
+int f3d_stage_weights(void* buf, size_t bytes, int ready);
 
 /* ---- dense layers --------------------------------------------------------------------------
  * gemm_sm_bf16(A[M,K], B[K,N], O[M,N]) — src/f3d_frontend.cu:87-88, src/psh/gemm_dispatcher.cu;

@@ -118,6 +118,75 @@ def test_hourglass_five_levels_vs_oracle_pipeline(oracle):
     _bands(out.float().cpu(), want, mean_tol=0.025, bulk_tol=0.08, max_tol=0.06)
 
 
+def test_hourglass_reference_shape_vs_oracle_pipeline(oracle):
+    """The reference's own model shape (tests/test_psh_hourglass.py:55-150 of the reference: scopes of 8 buckets, two
+    encoder + two decoder blocks per level, eval-mode BatchNorm1d(eps=1e-3) + GELU around pooling / unpooling, pooled
+    lengths aligned to bucket x scope) on three levels 32 / 64 / 128 at 4 x 20,000 points against the oracle pipeline:
+    scattered coordinates, every pooling map and pooled coordinates bit for bit; the output inside bands."""
+    import bench_workloads as configs
+    cfg = configs.HOURGLASS_REF_SHAPE
+    bs, scope, S, hash_op = cfg["bucket_size"], cfg["scope_size"], cfg["subbuck_size"], cfg["hash_type"]
+    model = configs.hourglass_ref_shape(1005, channels=(32, 64, 128))
+    for name, p in model.named_parameters():
+        if p.dim() == 2:                     # make attention logits and MLP outputs matter
+            p.data = (p.data * 2.0).to(torch.bfloat16).float()
+    model = model.to(DEV).eval()
+    coords, seps, _ = configs.lidar_batch(4, 20_000, 1005)
+    c, s = configs.to_device(coords, seps, DEV)
+    seen, hooks = _hook_pooling_buffers(model)
+    with torch.no_grad():
+        out = model(c, None, s)
+        again = model(c, None, s)            # second forward: prepared weights are reused
+    torch.cuda.synchronize()
+    for h in hooks:
+        h.remove()
+    assert torch.equal(out, again)
+    sd = _state_dict_cpu(("", model))
+    trace = []
+    want, scat = oracle.flash3d_forward(sd, coords, seps, configs.hourglass_oracle_levels(model), bs, scope, hash_op, S,
+                                        trace)
+    assert np.array_equal(model.psh_scatter.last_scattered_coord.cpu().numpy().view(np.uint16), scat.view(np.uint16))
+    pools = [t for t in trace if t[0] == "pool"]
+    assert len(pools) == 2 and len(seen) == 4          # two poolings per forward, two forwards
+    for (_, level, unpool, red_coord), (_, _, buf) in zip(pools, seen):
+        assert buf.reduced_coord.shape[0] % (bs * scope) == 0
+        assert np.array_equal(buf.unpool_ind.cpu().view(torch.int32).numpy().view(np.uint32), unpool), level
+        assert np.array_equal(buf.reduced_coord.cpu().numpy().view(np.uint16), red_coord.view(np.uint16)), level
+    assert out.shape == want.shape
+    # measured: mean 0.029 at scale 5.9, 99th percentile 0.25, max 1.0 at max|ref| 247
+    _bands(out.float().cpu(), want, mean_tol=0.02, bulk_tol=0.15, max_tol=0.02)
+
+
+def test_hourglass_reference_shape_4x250k_properties():
+    """the same shape on five levels 32 ... 512 at 4 x 250,000 points: finite, bit-reproducible, every level's length a
+    multiple of bucket x scope (so that no level falls back to one global scope), pooling maps bijective"""
+    import bench_workloads as configs
+    import warnings
+    model = configs.hourglass_ref_shape(1005).to(DEV).eval()
+    coords, seps, _ = configs.lidar_batch(4, 250_000, 1005)
+    c, s = configs.to_device(coords, seps, DEV)
+    seen, hooks = _hook_pooling_buffers(model)
+    with torch.no_grad(), warnings.catch_warnings():
+        warnings.simplefilter("error")       # the planner warns when a length falls back to one global scope
+        out = model(c, None, s)
+        again = model(c, None, s)
+    torch.cuda.synchronize()
+    for h in hooks:
+        h.remove()
+    bs, scope = configs.HOURGLASS_REF_SHAPE["bucket_size"], configs.HOURGLASS_REF_SHAPE["scope_size"]
+    n = coords.shape[0]
+    pad_to = -(-n // (bs * scope * 6)) * (bs * scope * 6)
+    assert out.shape == (pad_to, 32) and torch.isfinite(out.float()).all() and torch.equal(out, again)
+    assert out.float().abs().mean().item() > 1e-3
+    rows = pad_to
+    for _, _, buf in seen[:4]:
+        u = buf.unpool_ind.cpu().view(torch.int32).numpy().view(np.uint32)
+        filled = u[u < rows]
+        assert filled.size == rows and np.array_equal(np.sort(filled), np.arange(rows, dtype=np.uint32))
+        rows = buf.reduced_coord.shape[0]
+        assert rows % (bs * scope) == 0
+
+
 def test_hourglass_4x250k_full_size_properties():
     """config 5 at full size: finite output of the right shape; every level's pooling map is a bijection between the
     level's rows and the filled slots; restoring the input order inverts the PSH permutation"""

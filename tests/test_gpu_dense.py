@@ -307,3 +307,56 @@ def test_fused_mlp_and_output_panel_kernel_at_bench_size(oracle):
     torch.cuda.synchronize()
     d = (y2[-n_small:].float() - y3.float()).abs() / (y3.float().abs() + x[-n_small:].float().abs()).clamp(min=1.0)
     assert d.max().item() <= 2 ** -6 and (d > 0).float().mean().item() < 0.02
+
+
+def test_staged_weights_are_reused_and_refreshed():
+    """Eval-mode forwards under no_grad keep the prepared weights (LayerNorm fold, fragment-major copies) between calls:
+    the second call must give the first call's bits, a changed parameter must show in the next output, and a buffer
+    that is too small is refused with a message."""
+    from flash3dtransformer_amd import layers as L
+    from flash3dtransformer_amd.lib import pshattn
+    torch.manual_seed(3)
+    ln = L.LayerNorm(256).to(DEV).eval()
+    lin = L.Linear(256, 768).to(DEV).eval()
+    mlp = L.LayerNormMLP(256, 1024).to(DEV).eval()
+    wide = L.LayerNormMLP(512, 2048).to(DEV).eval()          # two-kernel path: fc1 fold and the re-laid fc2 weight
+    x = torch.randn(40000, 256, device=DEV).to(torch.bfloat16)
+    xw = torch.randn(40000, 512, device=DEV).to(torch.bfloat16)
+    with torch.no_grad():
+        ln.weight.add_(torch.randn_like(ln.weight) * 0.1)
+        first = [lin(x, pre_norm=ln), mlp(x, residual=x), wide(xw)]
+        assert lin._staged._key is not None and mlp._staged[0]._key is not None and wide._staged[1]._key is not None
+        second = [lin(x, pre_norm=ln), mlp(x, residual=x), wide(xw)]
+        for a, b in zip(first, second):
+            assert torch.equal(a, b)
+        # the same layers without staging (training mode prepares per call): identical bits
+        for m in (ln, lin, mlp, wide):
+            m.train()
+        third = [lin(x, pre_norm=ln), mlp(x, residual=x), wide(xw)]
+        for a, b in zip(first, third):
+            assert torch.equal(a, b)
+        for m in (ln, lin, mlp, wide):
+            m.eval()
+        fourth = [lin(x, pre_norm=ln), mlp(x, residual=x), wide(xw)]       # staged again after train() / eval()
+        for a, b in zip(first, fourth):
+            assert torch.equal(a, b)
+        # a parameter update (version bump) is seen
+        ln.bias.add_(0.5)
+        mlp.fc2_bias.add_(1.0)
+        wide.fc2_weight.mul_(2.0)
+        fifth = [lin(x, pre_norm=ln), mlp(x, residual=x), wide(xw)]
+        for a, b in zip(first, fifth):
+            assert not torch.equal(a, b)
+        for m in (ln, lin, mlp, wide):
+            m.train()
+        sixth = [lin(x, pre_norm=ln), mlp(x, residual=x), wide(xw)]
+        for a, b in zip(fifth, sixth):
+            assert torch.equal(a, b)
+    small = torch.empty(1024, dtype=torch.uint8, device=DEV)
+    pshattn.stage_weights(small, False)
+    y = torch.empty(64, 768, dtype=torch.bfloat16, device=DEV)
+    w = torch.zeros(768, 256, dtype=torch.bfloat16, device=DEV)
+    g = torch.ones(256, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(RuntimeError, match="f3d_stage_weights"):
+        pshattn.ln_linear_bf16(x[:64], g, g, 1e-5, w, None, None, y, None)
+    pshattn.ln_linear_bf16(x[:64], g, g, 1e-5, w, None, None, y, None)     # the staging ended with the failed call
