@@ -14,6 +14,7 @@ is where the reference gets all of it (torch / TransformerEngine autograd).  The
 restatement.
 """
 import math
+import weakref
 
 import torch
 from torch import nn
@@ -180,6 +181,7 @@ def refresh_weights(module: nn.Module) -> None:
     for m in module.modules():
         if isinstance(m, _CachedParamModule):
             m.refresh_weights()
+        _BN_AFFINE.pop(m, None)
 
 
 def as_bf16_2d(x: torch.Tensor) -> torch.Tensor:
@@ -454,11 +456,23 @@ def apply_norm(norm: nn.Module, x: torch.Tensor) -> torch.Tensor:
     return norm(x)
 
 
+_BN_AFFINE = weakref.WeakKeyDictionary()      # eval-mode BatchNorm1d -> (key, scale, shift)
+
+
 def _bn_affine(bn: nn.BatchNorm1d):
+    """scale and shift of an eval-mode BatchNorm1d (running statistics folded with the affine parameters), fp32; kept per
+    module while its statistics and parameters stay at the same address and version"""
+    src = [bn.running_mean, bn.running_var] + ([bn.weight, bn.bias] if bn.affine else [])
+    key = (bn.eps,) + tuple((t.data_ptr(), t._version) for t in src)
+    hit = _BN_AFFINE.get(bn)
+    if hit is not None and hit[0] == key and not torch.is_grad_enabled():
+        return hit[1], hit[2]
     rstd = torch.rsqrt(bn.running_var.float() + bn.eps)
     g = bn.weight.detach().float() if bn.affine else torch.ones_like(rstd)
     b = bn.bias.detach().float() if bn.affine else torch.zeros_like(rstd)
-    return (g * rstd).contiguous(), (b - bn.running_mean.float() * g * rstd).contiguous()
+    scale, shift = (g * rstd).contiguous(), (b - bn.running_mean.float() * g * rstd).contiguous()
+    _BN_AFFINE[bn] = (key, scale, shift)
+    return scale, shift
 
 
 _ACT_NAMES = {nn.GELU: "gelu", nn.ReLU: "relu", nn.SiLU: "silu"}
