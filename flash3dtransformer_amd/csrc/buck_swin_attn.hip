@@ -846,7 +846,7 @@ int f3d_buck_swin_fwd_strided(const f3d_bf16_t* q, const f3d_bf16_t* k, const f3
                 "No kernel found for head_dim=%u (supported: 16, 32, 64, 128)", head_dim);
   F3D_CHECK_ARG(bucket_size >= 128 && bucket_size % 128 == 0, "bucket_size=%u must be a multiple of 128",
                 bucket_size);
-  F3D_CHECK_ARG(scope_size >= 1 && scope_size <= 8192, "scope_size=%u outside [1, 8192]", scope_size);
+  F3D_CHECK_ARG(scope_size >= 1 && scope_size <= 4096, "scope_size=%u outside [1, 4096]", scope_size);
   F3D_CHECK_ARG(seq_len % bucket_size == 0, "sequence length %u is not a multiple of bucket_size=%u", seq_len,
                 bucket_size);
   F3D_CHECK_ARG(qkv_row_stride >= num_head * head_dim && qkv_row_stride % 8 == 0,

@@ -20,6 +20,7 @@
 // Valid lengths (kv_len, may be null): keys at in-bucket position >= kv_len[bucket] have P = 0, and so have query rows
 // there (the forward gave them O = 0, LSE = 0): their gradients are zero and they add nothing to dK / dV.
 #include <type_traits>
+#include <algorithm>
 #include "f3d_device.h"
 #include "f3d_internal.h"
 
@@ -108,9 +109,10 @@ __device__ __forceinline__ void stream_load_tr(const char* tile, uint32_t tr_lo,
 struct StreamItem {
   uint32_t batch, scope, head, blk;
 };
-__device__ __forceinline__ StreamItem stream_item(uint32_t num_scope, uint32_t num_head) {
+// grid.y holds at most 65535 (batch, scope, head) items: a launch covers items [item0, item0 + gridDim.y)
+__device__ __forceinline__ StreamItem stream_item(uint32_t num_scope, uint32_t num_head, uint32_t item0) {
   StreamItem it;
-  const uint32_t item = blockIdx.y;
+  const uint32_t item = item0 + blockIdx.y;
   it.blk = blockIdx.x;
   it.head = item % num_head;
   it.scope = (item / num_head) % num_scope;
@@ -139,9 +141,9 @@ __global__ __launch_bounds__(256) void bwd_delta_kernel(const uint16_t* __restri
                                                         float* __restrict__ delta,
                                                         const uint32_t* __restrict__ scope_buckets, uint32_t num_scope,
                                                         uint32_t scope_size, uint32_t bs, uint32_t seq_len,
-                                                        uint32_t num_head) {
-  // thread -> (scope row, head); grid.y -> (batch, scope)
-  const uint32_t scope = blockIdx.y % num_scope, batch = blockIdx.y / num_scope;
+                                                        uint32_t num_head, uint32_t y0) {
+  // thread -> (scope row, head); y0 + grid.y -> (batch, scope)
+  const uint32_t scope = (y0 + blockIdx.y) % num_scope, batch = (y0 + blockIdx.y) / num_scope;
   const uint32_t idx = blockIdx.x * blockDim.x + threadIdx.x;
   const uint32_t head = idx % num_head, loc = idx / num_head;
   if (loc >= scope_size * bs) return;
@@ -176,7 +178,7 @@ __global__ __launch_bounds__(64 * kStreamWaves) void bwd_dkdv_stream_kernel(
     const uint16_t* __restrict__ d_o, const float* __restrict__ lse, const float* __restrict__ delta,
     uint16_t* __restrict__ dk, uint16_t* __restrict__ dv, const uint32_t* __restrict__ scope_buckets,
     uint32_t num_scope, uint32_t scope_size, uint32_t bs, uint32_t seq_len, uint32_t num_head,
-    const int32_t* __restrict__ kv_len, float scale, float scale_log2, uint32_t ldg) {
+    const int32_t* __restrict__ kv_len, float scale, float scale_log2, uint32_t ldg, uint32_t item0) {
   using G = SGeom<D>;
   constexpr int KSTEPS = G::KSTEPS, ROWB = G::ROWB, DT = G::DT, TILEB = G::TILEB;
   extern __shared__ __attribute__((aligned(16))) char lds_s[];
@@ -187,7 +189,7 @@ __global__ __launch_bounds__(64 * kStreamWaves) void bwd_dkdv_stream_kernel(
   int32_t* s_len = reinterpret_cast<int32_t*>(s_bucket + scope_size);
   const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)lds_s;
 
-  const StreamItem it = stream_item(num_scope, num_head);
+  const StreamItem it = stream_item(num_scope, num_head, item0);
   const uint32_t tid = threadIdx.x, lane = tid % kWave;
   const uint32_t wave = __builtin_amdgcn_readfirstlane(tid / kWave);
   const uint32_t lq = lane & 31u, half = lane >> 5;
@@ -340,7 +342,7 @@ __global__ __launch_bounds__(64 * kStreamWaves) void bwd_dq_stream_kernel(
     const uint16_t* __restrict__ d_o, const float* __restrict__ lse, const float* __restrict__ delta,
     uint16_t* __restrict__ dq, const uint32_t* __restrict__ scope_buckets, uint32_t num_scope, uint32_t scope_size,
     uint32_t bs, uint32_t seq_len, uint32_t num_head, const int32_t* __restrict__ kv_len, float scale,
-    float scale_log2, uint32_t ldg) {
+    float scale_log2, uint32_t ldg, uint32_t item0) {
   using G = SGeom<D>;
   constexpr int KSTEPS = G::KSTEPS, ROWB = G::ROWB, DT = G::DT, TILEB = G::TILEB;
   extern __shared__ __attribute__((aligned(16))) char lds_s[];
@@ -349,7 +351,7 @@ __global__ __launch_bounds__(64 * kStreamWaves) void bwd_dq_stream_kernel(
   int32_t* s_len = reinterpret_cast<int32_t*>(s_bucket + scope_size);
   const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)lds_s;
 
-  const StreamItem it = stream_item(num_scope, num_head);
+  const StreamItem it = stream_item(num_scope, num_head, item0);
   const uint32_t tid = threadIdx.x, lane = tid % kWave;
   const uint32_t wave = __builtin_amdgcn_readfirstlane(tid / kWave);
   const uint32_t lq = lane & 31u, half = lane >> 5;
@@ -491,13 +493,18 @@ static int launch_stream(const uint16_t* q, const uint16_t* k, const uint16_t* v
   const uint32_t items = batch * num_scope * num_head;
   const float scale = 1.0f / sqrtf((float)D), scale_log2 = 1.4426950408889634f * scale;
   const uint32_t dthreads = 256, dgrid = cdiv_u32(scope_tokens * num_head, dthreads);
-  hipLaunchKernelGGL(bwd_delta_kernel<D>, dim3(dgrid, batch * num_scope), dim3(dthreads), 0, s, o, d_o, delta, scope_buckets,
-                     num_scope, scope_size, bs, seq_len, num_head);
-  const dim3 grid(scope_tokens / kStreamBlock, items), block(64 * kStreamWaves);
-  hipLaunchKernelGGL(bwd_dkdv_stream_kernel<D>, grid, block, lds, s, q, k, v, ld, d_o, lse, delta, dk, dv, scope_buckets,
-                     num_scope, scope_size, bs, seq_len, num_head, kv_len, scale, scale_log2, ldg);
-  hipLaunchKernelGGL(bwd_dq_stream_kernel<D>, grid, block, lds, s, q, k, v, ld, d_o, lse, delta, dq, scope_buckets, num_scope,
-                     scope_size, bs, seq_len, num_head, kv_len, scale, scale_log2, ldg);
+  constexpr uint32_t kMaxY = 65535u;      // grid.y limit: longer lists of items go out in several launches
+  for (uint32_t y0 = 0; y0 < batch * num_scope; y0 += kMaxY)
+    hipLaunchKernelGGL(bwd_delta_kernel<D>, dim3(dgrid, std::min(kMaxY, batch * num_scope - y0)), dim3(dthreads), 0, s, o, d_o,
+                       delta, scope_buckets, num_scope, scope_size, bs, seq_len, num_head, y0);
+  const dim3 block(64 * kStreamWaves);
+  for (uint32_t item0 = 0; item0 < items; item0 += kMaxY) {
+    const dim3 grid(scope_tokens / kStreamBlock, std::min(kMaxY, items - item0));
+    hipLaunchKernelGGL(bwd_dkdv_stream_kernel<D>, grid, block, lds, s, q, k, v, ld, d_o, lse, delta, dk, dv, scope_buckets,
+                       num_scope, scope_size, bs, seq_len, num_head, kv_len, scale, scale_log2, ldg, item0);
+    hipLaunchKernelGGL(bwd_dq_stream_kernel<D>, grid, block, lds, s, q, k, v, ld, d_o, lse, delta, dq, scope_buckets,
+                       num_scope, scope_size, bs, seq_len, num_head, kv_len, scale, scale_log2, ldg, item0);
+  }
   return F3D_OK;
 }
 
@@ -507,10 +514,9 @@ int launch_attn_bwd_stream(const uint16_t* q, const uint16_t* k, const uint16_t*
                            const uint32_t* scope_buckets, uint32_t num_scope, uint32_t scope_size, uint32_t bs,
                            uint32_t batch, uint32_t seq_len, uint32_t num_head, uint32_t head_dim, const int32_t* kv_len,
                            uint32_t ldg, int device, hipStream_t s) {
-  if ((uint64_t)batch * num_scope * num_head > 65535u) {
-    set_error("attention backward: %llu (batch, scope, head) items exceed one launch's 65535",
-              (unsigned long long)batch * num_scope * num_head);
-    return F3D_ERR_UNSUPPORTED;
+  if ((uint64_t)batch * num_scope * num_head > 0x7FFFFFF0ull) {
+    set_error("attention problem too large for one launch (%llu items)", (unsigned long long)batch * num_scope * num_head);
+    return F3D_ERR_INVALID;
   }
 #define F3D_STREAM(DD)                                                                                                 \
   return launch_stream<DD>(q, k, v, ld, o, d_o, lse, delta, dq, dk, dv, scope_buckets, num_scope, scope_size, bs, batch, \

@@ -434,7 +434,7 @@ int f3d_ln_linear_bf16(const f3d_bf16_t* x, uint32_t ldx, const f3d_bf16_t* gamm
   int rc = launch_xstat_linear(x, ldx, gamma, beta, eps, w, bias, residual, ldr, y, ldy, m, n, k, act, device, s);
   if (rc == F3D_ERR_UNSUPPORTED) {
     // shape outside the fused kernel: normalise into the per-device workspace, then the tiled GEMM
-    uint16_t* tmp = (uint16_t*)workspace(device, (size_t)m * k * sizeof(uint16_t));
+    uint16_t* tmp = (uint16_t*)workspace(device, (size_t)m * k * sizeof(uint16_t), s);
     if (!tmp) return F3D_ERR_RUNTIME;
     F3D_CHECK_ARG(ldx == k, "LayerNorm+Linear on a strided input needs an output width that is a multiple of 64");
     launch_layernorm(x, gamma, beta, tmp, m, k, eps, s);

@@ -438,7 +438,7 @@ int f3d_linear_wgrad_bf16(const f3d_bf16_t* dy, uint32_t lddy, const f3d_bf16_t*
   if (m) slabs = cdiv_u32(m, slab_rows);
   const size_t nk = (size_t)n * k;
   const size_t part_w_bytes = (size_t)slabs * nk * 4, part_b_bytes = db ? (size_t)slabs * n * 4 : 0;
-  char* ws = (char*)workspace(device, part_w_bytes + part_b_bytes);
+  char* ws = (char*)workspace(device, part_w_bytes + part_b_bytes, s);
   if (!ws) return F3D_ERR_RUNTIME;
   float* part_w = (float*)ws;
   float* part_b = db ? (float*)(ws + part_w_bytes) : nullptr;
@@ -482,7 +482,7 @@ int f3d_layernorm_bwd_bf16(const f3d_bf16_t* x, uint32_t ldx, const f3d_bf16_t* 
   uint32_t wgs = cdiv_u32(m, rpb);
   if (wgs > n_cu * 8u) wgs = n_cu * 8u;
   if (wgs == 0) wgs = 1;
-  float* part = (float*)workspace(device, (size_t)wgs * 2u * c * 4u);
+  float* part = (float*)workspace(device, (size_t)wgs * 2u * c * 4u, s);
   if (!part) return F3D_ERR_RUNTIME;
 #define F3D_LNB(LPR)                                                                                                \
   hipLaunchKernelGGL((layernorm_bwd_kernel<LPR>), dim3(wgs), dim3(256), 0, s, x, ldx, dh, lddh, gamma, dres, lddr, \

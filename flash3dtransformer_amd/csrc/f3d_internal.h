@@ -16,14 +16,16 @@ void set_error(const char* fmt, ...) __attribute__((format(printf, 1, 2)));
 // Grow-only scratch buffer owned by the library, one per device.  Work that uses it is ordered on
 // the caller's stream; calls that overlap on different streams of one device must not share it, so
 // every entry point that needs scratch documents that it is not re-entrant per device.
-// Returns nullptr (and sets the error) on allocation failure.
-void* workspace(int device, size_t bytes);
+// `stream`: the caller's stream; when the buffer has to grow while that stream is being captured the call fails with a
+// message (warm the shapes up outside capture) and does not touch the device.
+// Returns nullptr (and sets the error) on failure.
+void* workspace(int device, size_t bytes, hipStream_t stream);
 
 // Device memory for the weights a dense op prepares per call (LayerNorm folded into the weight, fragment-major
 // copies): the buffer the caller staged with f3d_stage_weights for this call, else the per-device workspace.
 // *ready: the staged buffer already holds this call's prepared weights, the preparation launch is skipped.
 // nullptr + error message when the staged buffer is too small or the workspace cannot grow.
-void* weight_area(int device, size_t bytes, bool* ready);
+void* weight_area(int device, size_t bytes, bool* ready, hipStream_t stream);
 // Declared at the top of every dense entry point: whatever the call does, the staging ends with it.
 struct StagedWeightsScope {
   ~StagedWeightsScope();

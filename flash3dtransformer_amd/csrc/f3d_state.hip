@@ -29,15 +29,21 @@ void set_error(const char* fmt, ...) {
   va_end(ap);
 }
 
-void* workspace(int device, size_t bytes) {
+void* workspace(int device, size_t bytes, hipStream_t stream) {
   std::lock_guard<std::mutex> lk(g_mu);
   Ws& w = g_ws[device];
   if (w.bytes >= bytes && w.ptr) return w.ptr;
   DeviceGuard guard(device);
   // Work queued on the old buffer must finish before it is released.
   if (w.ptr) {
-    // (refused while a stream of this thread is being captured: the caller gets an error instead of a broken graph)
-    const hipError_t es = hipDeviceSynchronize();
+    // Refused while the caller's stream is being captured: the device cannot be synchronised then (the attempt itself
+    // would invalidate the capture), so the capture state is asked first and the device is left alone.
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    hipError_t es = hipSuccess;
+    if (hipStreamIsCapturing(stream, &cap) == hipSuccess && cap != hipStreamCaptureStatusNone)
+      es = hipErrorStreamCaptureUnsupported;
+    else
+      es = hipDeviceSynchronize();
     if (es != hipSuccess) {
       set_error("the workspace of device %d must grow from %zu to %zu bytes, but the device cannot be synchronised (%s): "
                 "warm the shapes up outside stream capture", device, w.bytes, bytes, hipGetErrorString(es));
@@ -66,7 +72,7 @@ static thread_local struct {
   bool ready = false, armed = false;
 } g_staged;
 
-void* weight_area(int device, size_t bytes, bool* ready) {
+void* weight_area(int device, size_t bytes, bool* ready, hipStream_t stream) {
   *ready = false;
   if (g_staged.armed) {
     if (g_staged.bytes < bytes) {
@@ -76,7 +82,7 @@ void* weight_area(int device, size_t bytes, bool* ready) {
     *ready = g_staged.ready;
     return g_staged.buf;
   }
-  return workspace(device, bytes);
+  return workspace(device, bytes, stream);
 }
 
 StagedWeightsScope::~StagedWeightsScope() { g_staged.armed = false; }
@@ -98,7 +104,7 @@ int f3d_init_dev_info(int device) {
   // The reference silently ignores a device that does not exist (device_manager.cu:59-60).
   if (device < 0 || device >= n) return F3D_OK;
   if (!f3d::psh_noalloc_scratch(device)) return F3D_ERR_RUNTIME;
-  return f3d::workspace(device, 1) ? F3D_OK : F3D_ERR_RUNTIME;
+  return f3d::workspace(device, 1, nullptr) ? F3D_OK : F3D_ERR_RUNTIME;
 }
 
 int f3d_set_sync_stream(int enable) {

@@ -625,7 +625,7 @@ int f3d_ln_mlp_swiglu_bf16(const f3d_bf16_t* x, uint32_t ldx, const f3d_bf16_t* 
   const size_t w1_bytes = (size_t)2 * hidden * c * 2, b32_bytes = (((size_t)2 * hidden * 4) + 255) & ~(size_t)255;
   const size_t w2_bytes = (size_t)hidden * c * 2;
   bool ready = false;
-  char* ws = (char*)weight_area(device, w1_bytes + b32_bytes + w2_bytes + (size_t)c * 2, &ready);
+  char* ws = (char*)weight_area(device, w1_bytes + b32_bytes + w2_bytes + (size_t)c * 2, &ready, s);
   if (!ws) return F3D_ERR_RUNTIME;
   uint16_t* w1p = (uint16_t*)ws;
   float* b32 = (float*)(ws + w1_bytes);

@@ -620,7 +620,7 @@ static int psh_run(const f3d_half_t* coord, uint16_t* bucket_id, uint32_t* bucke
   }
   DeviceGuard guard(device);
   F3D_CHECK_ARG(guard.ok, "cannot select device %d", device);
-  uint32_t* tile_hist = no_alloc ? psh_noalloc_scratch(device) : (uint32_t*)workspace(device, ws_words * sizeof(uint32_t));
+  uint32_t* tile_hist = no_alloc ? psh_noalloc_scratch(device) : (uint32_t*)workspace(device, ws_words * sizeof(uint32_t), s);
   if (!tile_hist) return F3D_ERR_RUNTIME;
   uint32_t* cnt_ws = tile_hist + hist_words;
   uint32_t* plan_ws = cnt_ws + cnt_words;
@@ -700,7 +700,7 @@ int f3d_coord_bbox(const f3d_half_t* coord, uint32_t total_n, f3d_half_t* bbox_m
   if (nblock > 1024) nblock = 1024;
   // partials live after the PSH histogram area would; a private slice at the workspace start is
   // enough because the op is ordered on the same stream as its consumers
-  float* partial = (float*)workspace(device, (size_t)1024 * 6 * sizeof(float));
+  float* partial = (float*)workspace(device, (size_t)1024 * 6 * sizeof(float), s);
   if (!partial) return F3D_ERR_RUNTIME;
   SyncBracket sync(s);
   hipLaunchKernelGGL(bbox_partial_kernel, dim3(nblock), dim3(256), 0, s, coord, total_n, partial);

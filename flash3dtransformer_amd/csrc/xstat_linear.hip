@@ -425,7 +425,7 @@ int launch_xstat_linear(const uint16_t* x, uint32_t ldx, const uint16_t* gamma, 
     // w' (bf16 [N][K]) and b' (fp32 [N]): per call in the per-device workspace, or kept in the caller's staged buffer
     const size_t wp_bytes = ((size_t)N * K * 2 + 255) & ~(size_t)255;
     bool ready = false;
-    char* ws = (char*)weight_area(device, wp_bytes + (size_t)N * 4, &ready);
+    char* ws = (char*)weight_area(device, wp_bytes + (size_t)N * 4, &ready, s);
     if (!ws) return F3D_ERR_RUNTIME;
     uint16_t* wp = (uint16_t*)ws;
     float* b32 = (float*)(ws + wp_bytes);

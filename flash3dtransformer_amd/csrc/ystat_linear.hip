@@ -220,7 +220,7 @@ int launch_ystat_linear(const uint16_t* x, uint32_t ldx, const uint16_t* w, cons
   if ((uint64_t)N * K * 2 >= (1ull << 32) || (uint64_t)256 * ldx * 2 >= (1ull << 31)) return F3D_ERR_UNSUPPORTED;
   const size_t wp_bytes = (size_t)N * K * 2;
   bool ready = false;
-  char* ws = (char*)weight_area(device, wp_bytes + (size_t)N * 2, &ready);
+  char* ws = (char*)weight_area(device, wp_bytes + (size_t)N * 2, &ready, s);
   if (!ws) return F3D_ERR_RUNTIME;
   uint16_t* wp = (uint16_t*)ws;
   uint16_t* zero_bias = (uint16_t*)(ws + wp_bytes);

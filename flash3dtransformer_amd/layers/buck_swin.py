@@ -57,7 +57,9 @@ class BuckSwinQKVFunction(Function):
         Q, K, V = (t.view(B, L, H, D) for t in torch.chunk(qkv, 3, dim=-1))
         dO = grad_output if grad_output.dtype == torch.bfloat16 else grad_output.to(torch.bfloat16)
         # rows that no scope covers are not written: zero-filled unless the planner vouches that its table covers all
-        covered = getattr(ctx.scope_buckets, "covers_all_rows", False)
+        # ... for THIS tensor: a table made for another length leaves rows out
+        covered = (getattr(ctx.scope_buckets, "covers_all_rows", False)
+                   and ctx.scope_buckets.numel() * ctx.buck_size == L)
         dqkv = torch.empty_like(qkv) if covered else torch.zeros_like(qkv)
         dQ, dK, dV = (t.view(B, L, H, D) for t in torch.chunk(dqkv, 3, dim=-1))
         delta = torch.zeros(B, L, H, dtype=torch.float32, device=O.device)

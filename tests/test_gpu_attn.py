@@ -358,6 +358,25 @@ def test_backward_with_valid_lengths(oracle):
                 assert not t[:, b * bs + n:(b + 1) * bs].any(), f"bucket {b}: gradient on a masked row"
 
 
+def test_streaming_backward_more_than_65535_items(oracle):
+    """8,192 one-bucket scopes of 128 tokens x 8 heads = 65,536 (batch, scope, head) items, one more than a launch's
+    grid.y holds: the forward takes them in one launch, the backward in two.  Gradients of scopes at both ends of the
+    list (the last item is the one the second launch covers) against the oracle."""
+    B, H, D, bs = 1, 8, 16, 128
+    n_scope = 8192
+    L = n_scope * bs
+    g = torch.Generator().manual_seed(65536)
+    Q, K, V, dO = [(torch.randn(B, L, H, D, generator=g)).to(torch.bfloat16) for _ in range(4)]
+    scopes = np.arange(n_scope, dtype=np.uint32)[:, None]
+    dq, dk, dv, delta, _ = _run_bwd(Q, K, V, dO, scopes, bs)
+    pick = [0, 1, 4095, 8190, 8191]
+    rows = np.concatenate([np.arange(b * bs, (b + 1) * bs) for b in pick])
+    ref = oracle.buck_swin_bwd(Q[:, rows], K[:, rows], V[:, rows], dO[:, rows], np.arange(len(pick), dtype=np.uint32)[:, None], bs)
+    for got, want, name in zip((dq, dk, dv), ref[:3], ("dq", "dk", "dv")):
+        assert (got[:, rows] - want).abs().max() <= TOL * max(1.0, want.abs().max().item()), name
+    assert (dq[:, -bs:].abs().sum() > 0) and (dk[:, -bs:].abs().sum() > 0)
+
+
 def test_backward_leaves_uncovered_rows_untouched(oracle):
     B, L, H, D, bs = 1, 2048, 2, 32, 512
     Q, K, V = _qkv(21, B, L, H, D)

@@ -169,7 +169,8 @@ def test_dense_layer_gradients_vs_torch(act, use_ln, use_res):
         assert close(res.grad, rr.grad, 1e-2)
 
 
-def test_transformer_block_trains(oracle):
+@pytest.mark.parametrize("n,C,H,bs", [(1024, 64, 2, 256), (4096, 64, 2, 512), (4096, 256, 8, 512)])
+def test_transformer_block_trains(oracle, n, C, H, bs):
     """one XFMR block (LayerNorm -> QKV -> bucketed attention -> proj + residual -> LayerNormMLP + residual):
     loss.backward() reaches every parameter; gradients against torch autograd through the oracle's restatement of
     the block (bf16 roundings are identities for the gradient)"""
@@ -177,7 +178,6 @@ def test_transformer_block_trains(oracle):
     from flash3dtransformer_amd.layers.stage import XFMR
     from flash3dtransformer_amd.psh.bucket_scope import SwinPlan
     torch.manual_seed(9)
-    n, C, H, bs = 1024, 64, 2, 256
     blk = XFMR(C, 2 * C, H, bs, True, SwinPlan("swin", bs, 1, 0), lambda ch: L.LayerNorm(ch)).to(DEV)
     for p in blk.parameters():
         if p.dim() == 2:
@@ -199,10 +199,16 @@ def test_transformer_block_trains(oracle):
     assert (out.float().cpu() - want.detach()).abs().mean().item() <= 0.02 * max(1.0, want.abs().mean().item())
     def rel(a, b):
         return (a.float().cpu() - b).abs().max().item() / max(1e-6, b.abs().max().item())
-    assert rel(x.grad, xr.grad) <= 0.06
+    def mean_rel(a, b):
+        return (a.float().cpu() - b).abs().mean().item() / max(1e-9, b.abs().mean().item())
+    # the wiring of the block's autograd functions (LayerNorm folded into QKV, attention over the projection output,
+    # projection + residual, gated MLP with a shared residual): largest deviation within 6 % of the largest gradient
+    # entry, average deviation within 1.5 % of the average entry (bf16 activations and gradients)
+    assert rel(x.grad, xr.grad) <= 0.06 and mean_rel(x.grad, xr.grad) <= 0.015, (rel(x.grad, xr.grad), mean_rel(x.grad, xr.grad))
     for k, v in XFMR_KEYS.items():
         g = dict(blk.named_parameters())[v].grad
         assert rel(g, sd[v].grad) <= 0.06, (k, rel(g, sd[v].grad))
+        assert mean_rel(g, sd[v].grad) <= 0.015, (k, mean_rel(g, sd[v].grad))
 
 
 def test_two_level_model_backward_reaches_every_parameter():
