@@ -12,7 +12,9 @@
 // max / sum run inside the lane plus one exchange with lane^32, and the bf16 P values are already in
 // the B-operand layout of the second MFMA, Ot += Vt Pt (keys are consumed in the permuted order the
 // accumulator layout yields; V is staged in that same order).  Softmax runs in the exp2 domain with
-// fp32 accumulation.  Workgroup ids are remapped so that the workgroups of one scope (which share
+// fp32 accumulation: first with the reference fixed at zero and pre-scaled Q (no running maximum, no
+// rescaling, row sums from the matrix core), and again with a running maximum for a workgroup whose row
+// sums left the safe range.  Workgroup ids are remapped so that the workgroups of one scope (which share
 // K/V and the 512-byte token rows) land on the same XCD and its L2.
 #include <type_traits>
 #include "f3d_device.h"
@@ -22,6 +24,7 @@ namespace f3d {
 
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16_t;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
 
 constexpr int kAttnThreads = 256;
 constexpr int kQBlock = 128;  // query rows per workgroup
@@ -147,95 +150,197 @@ __global__ __launch_bounds__(kAttnThreads) void buck_swin_fwd_kernel(
     }
   };
 
-  bool have = settle();
-  if (have) fetch(jb, kt);
-  while (have) {
-    const uint32_t cur_kt = kt;
-    const int32_t cur_len = bucket_len(jb);
-    __syncthreads();  // every wave is done reading the previous tile
-    stage();
-    __syncthreads();
-    // prefetch the next tile while this one is consumed
-    ++kt;
-    if (kt == tiles_per_bucket) { ++jb; kt = 0; }
-    have = settle();
+  // ---- fast pass: softmax with the reference fixed at zero.  Q is pre-multiplied by log2(e) / sqrt(D) (one bf16
+  //      rounding), so the score product emits exponents and the vector unit only exponentiates and packs; the row
+  //      sums come from the matrix core (a 16x16x32 product of P with a 0 / 1 selector, see the scope-resident
+  //      kernel below).  Exact as long as the numbers stay in range (softmax is shift-invariant, fp32 and bf16 share
+  //      the exponent range); a workgroup with a row sum outside [2^-24, 2^24) (or not a number) redoes its scope
+  //      with the running-maximum pass after it. ----
+  bool redo = false, any_tile = false;
+  {
+    bf16x8_t qs[C::KSTEPS];
+#pragma unroll
+    for (int ks = 0; ks < C::KSTEPS; ++ks) {
+      const u32x4_t raw = __builtin_bit_cast(u32x4_t, qf[ks]);
+      u32x4_t sc;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) sc[e] = pack_bf16x2(bf16_lo(raw[e]) * scale_log2, bf16_hi(raw[e]) * scale_log2);
+      qs[ks] = __builtin_bit_cast(bf16x8_t, sc);
+    }
+    bf16x8_t ones_sel;
+    {
+      const uint32_t m = lane & 15u, kb = lane >> 4;
+      const __bf16 val = ((m < 8u) == ((kb & 1u) == 0u)) ? (__bf16)1.0f : (__bf16)0.0f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) ones_sel[e] = val;
+    }
+    f32x4_t lacc = {0.f, 0.f, 0.f, 0.f};
+    bool have = settle();
     if (have) fetch(jb, kt);
-
-    // ---- St = K Qt for the whole tile ----
-    float s[C::NSUB * 16];
+    while (have) {
+      any_tile = true;
+      const uint32_t cur_kt = kt;
+      const int32_t cur_len = bucket_len(jb);
+      __syncthreads();  // every wave is done reading the previous tile
+      stage();
+      __syncthreads();
+      ++kt;
+      if (kt == tiles_per_bucket) { ++jb; kt = 0; }
+      have = settle();
+      if (have) fetch(jb, kt);
+      const bool boundary = (int32_t)((cur_kt + 1) * KT) > cur_len;   // uniform
 #pragma unroll
-    for (int j = 0; j < C::NSUB; ++j) {
-      f32x16_t sacc;
+      for (int j = 0; j < C::NSUB; ++j) {
+        f32x16_t sacc;
 #pragma unroll
-      for (int i = 0; i < 16; ++i) sacc[i] = 0.f;
+        for (int i = 0; i < 16; ++i) sacc[i] = 0.f;
 #pragma unroll
-      for (int ks = 0; ks < C::KSTEPS; ++ks) {
-        const bf16x8_t kf = *reinterpret_cast<const bf16x8_t*>(sK + (j * 32 + lq) * C::KROW + ks * 16 + half * 8);
-        sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[ks], sacc, 0, 0, 0);
-      }
-#pragma unroll
-      for (int i = 0; i < 16; ++i) s[j * 16 + i] = sacc[i];
-    }
-    // ---- mask keys beyond the bucket's valid length (only a boundary tile pays for this) ----
-    if ((int32_t)((cur_kt + 1) * KT) > cur_len) {
-#pragma unroll
-      for (int j = 0; j < C::NSUB; ++j)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          const int32_t key = cur_kt * KT + j * 32 + (i / 4) * 8 + half * 4 + (i % 4);
-          if (key >= cur_len) s[j * 16 + i] = -INFINITY;
+        for (int ks = 0; ks < C::KSTEPS; ++ks) {
+          const bf16x8_t kf = *reinterpret_cast<const bf16x8_t*>(sK + (j * 32 + lq) * C::KROW + ks * 16 + half * 8);
+          sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qs[ks], sacc, 0, 0, 0);
         }
-    }
-    // ---- online softmax (exp2 domain) ----
-    float mx = s[0];
+        if (boundary) {
 #pragma unroll
-    for (int i = 1; i < C::NSUB * 16; ++i) mx = fmaxf(mx, s[i]);
-    mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
-    const float m_new = fmaxf(m_run, mx * scale_log2);
-    const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-    const float alpha = __builtin_amdgcn_exp2f(m_run - m_use);  // m_run = -inf -> 0
-    m_run = m_new;
-    float psum = 0.f;
-    uint32_t pb[C::NSUB * 8];
-#pragma unroll
-    for (int i = 0; i < C::NSUB * 16; i += 2) {
-      const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[i], scale_log2, -m_use));
-      const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[i + 1], scale_log2, -m_use));
-      pb[i / 2] = pack_bf16x2(p0, p1);
-      // row sum of the bf16-rounded probabilities (what the PV product sees): one dot2 per pair
-      psum = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, pb[i / 2]),
-                                             __builtin_bit_cast(bf16x2_t, 0x3F803F80u), psum, false);
-    }
-    l_run = l_run * alpha + psum;
-    // the running maximum settles after the first tiles: rescale the accumulators only when some
-    // query of this wave actually moved (wave-uniform branch)
-    if (__ballot(alpha != 1.0f)) {
-#pragma unroll
-      for (int dt = 0; dt < C::DT; ++dt)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) acc[dt][i] *= alpha;
-    }
-    // ---- Ot += Vt Pt ----
-#pragma unroll
-    for (int j = 0; j < C::NSUB; ++j)
-#pragma unroll
-      for (int kk = 0; kk < 2; ++kk) {
-        u32x4_t praw = {pb[j * 8 + kk * 4 + 0], pb[j * 8 + kk * 4 + 1], pb[j * 8 + kk * 4 + 2], pb[j * 8 + kk * 4 + 3]};
-        const bf16x8_t pf = __builtin_bit_cast(bf16x8_t, praw);
-#pragma unroll
-        for (int dt = 0; dt < C::DT; ++dt) {
-          bf16x8_t vf;
-          if (D >= 32 || lq < (uint32_t)D) {
-            vf = *reinterpret_cast<const bf16x8_t*>(sVt + (dt * 32 + lq) * C::VROW + j * 32 + kk * 16 + half * 8);
-          } else {
-#pragma unroll
-            for (int e = 0; e < 8; ++e) vf[e] = (__bf16)0.f;
+          for (int i = 0; i < 16; ++i) {
+            const int32_t key = cur_kt * KT + j * 32 + (i / 4) * 8 + half * 4 + (i % 4);
+            if (key >= cur_len) sacc[i] = -INFINITY;
           }
-          acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf, acc[dt], 0, 0, 0);
+        }
+        uint32_t pb[8];
+#pragma unroll
+        for (int i = 0; i < 16; i += 2)
+          pb[i / 2] = pack_bf16x2(__builtin_amdgcn_exp2f(sacc[i]), __builtin_amdgcn_exp2f(sacc[i + 1]));
+#pragma unroll
+        for (int kk = 0; kk < 2; ++kk) {
+          const u32x4_t praw = {pb[kk * 4 + 0], pb[kk * 4 + 1], pb[kk * 4 + 2], pb[kk * 4 + 3]};
+          const bf16x8_t pf = __builtin_bit_cast(bf16x8_t, praw);
+#pragma unroll
+          for (int dt = 0; dt < C::DT; ++dt) {
+            bf16x8_t vf;
+            if (D >= 32 || lq < (uint32_t)D) {
+              vf = *reinterpret_cast<const bf16x8_t*>(sVt + (dt * 32 + lq) * C::VROW + j * 32 + kk * 16 + half * 8);
+            } else {
+#pragma unroll
+              for (int e = 0; e < 8; ++e) vf[e] = (__bf16)0.f;
+            }
+            acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf, acc[dt], 0, 0, 0);
+          }
+          lacc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones_sel, pf, lacc, 0, 0, 0);
         }
       }
+    }
+    // lanes 0-31 of the selector product hold the row sums of queries 0-15 (lane % 16), lanes 32-63 those of 16-31
+    const float l_fast = __shfl(lacc[0], (lq < 16u ? 0u : 32u) + (lq & 15u), kWave);
+    redo = any_tile && __syncthreads_or((!(l_fast > 0x1p-24f) || !(l_fast < 0x1p24f)) ? 1 : 0) != 0;
+    // the epilogue's formula: O = acc / l, LSE = (m + log2 l) ln 2 with m = 0; l_run is halved because the epilogue
+    // adds the two half-waves' partial sums of the running-maximum pass
+    m_run = any_tile ? 0.f : -INFINITY;
+    l_run = 0.5f * l_fast;
   }
-
+  if (redo) {
+    // ---- general pass: running-maximum softmax with the scale applied in fp32, from the start of the scope ----
+    jb = 0; kt = 0;
+#pragma unroll
+    for (int dt = 0; dt < C::DT; ++dt)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[dt][i] = 0.f;
+    m_run = -INFINITY; l_run = 0.f;
+    {
+      // unscaled Q, read again: the fast pass kept only its pre-scaled copy
+      const uint16_t* qp = q + (tok0 + q_row) * ld + head * D + half * 8;
+#pragma unroll
+      for (int ks = 0; ks < C::KSTEPS; ++ks) qf[ks] = *reinterpret_cast<const bf16x8_t*>(qp + ks * 16);
+    }
+    bool have = settle();
+    if (have) fetch(jb, kt);
+    while (have) {
+      const uint32_t cur_kt = kt;
+      const int32_t cur_len = bucket_len(jb);
+      __syncthreads();  // every wave is done reading the previous tile
+      stage();
+      __syncthreads();
+      // prefetch the next tile while this one is consumed
+      ++kt;
+      if (kt == tiles_per_bucket) { ++jb; kt = 0; }
+      have = settle();
+      if (have) fetch(jb, kt);
+  
+      // ---- St = K Qt for the whole tile ----
+      float s[C::NSUB * 16];
+  #pragma unroll
+      for (int j = 0; j < C::NSUB; ++j) {
+        f32x16_t sacc;
+  #pragma unroll
+        for (int i = 0; i < 16; ++i) sacc[i] = 0.f;
+  #pragma unroll
+        for (int ks = 0; ks < C::KSTEPS; ++ks) {
+          const bf16x8_t kf = *reinterpret_cast<const bf16x8_t*>(sK + (j * 32 + lq) * C::KROW + ks * 16 + half * 8);
+          sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[ks], sacc, 0, 0, 0);
+        }
+  #pragma unroll
+        for (int i = 0; i < 16; ++i) s[j * 16 + i] = sacc[i];
+      }
+      // ---- mask keys beyond the bucket's valid length (only a boundary tile pays for this) ----
+      if ((int32_t)((cur_kt + 1) * KT) > cur_len) {
+  #pragma unroll
+        for (int j = 0; j < C::NSUB; ++j)
+  #pragma unroll
+          for (int i = 0; i < 16; ++i) {
+            const int32_t key = cur_kt * KT + j * 32 + (i / 4) * 8 + half * 4 + (i % 4);
+            if (key >= cur_len) s[j * 16 + i] = -INFINITY;
+          }
+      }
+      // ---- online softmax (exp2 domain) ----
+      float mx = s[0];
+  #pragma unroll
+      for (int i = 1; i < C::NSUB * 16; ++i) mx = fmaxf(mx, s[i]);
+      mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
+      const float m_new = fmaxf(m_run, mx * scale_log2);
+      const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+      const float alpha = __builtin_amdgcn_exp2f(m_run - m_use);  // m_run = -inf -> 0
+      m_run = m_new;
+      float psum = 0.f;
+      uint32_t pb[C::NSUB * 8];
+  #pragma unroll
+      for (int i = 0; i < C::NSUB * 16; i += 2) {
+        const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[i], scale_log2, -m_use));
+        const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[i + 1], scale_log2, -m_use));
+        pb[i / 2] = pack_bf16x2(p0, p1);
+        // row sum of the bf16-rounded probabilities (what the PV product sees): one dot2 per pair
+        psum = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, pb[i / 2]),
+                                               __builtin_bit_cast(bf16x2_t, 0x3F803F80u), psum, false);
+      }
+      l_run = l_run * alpha + psum;
+      // the running maximum settles after the first tiles: rescale the accumulators only when some
+      // query of this wave actually moved (wave-uniform branch)
+      if (__ballot(alpha != 1.0f)) {
+  #pragma unroll
+        for (int dt = 0; dt < C::DT; ++dt)
+  #pragma unroll
+          for (int i = 0; i < 16; ++i) acc[dt][i] *= alpha;
+      }
+      // ---- Ot += Vt Pt ----
+  #pragma unroll
+      for (int j = 0; j < C::NSUB; ++j)
+  #pragma unroll
+        for (int kk = 0; kk < 2; ++kk) {
+          u32x4_t praw = {pb[j * 8 + kk * 4 + 0], pb[j * 8 + kk * 4 + 1], pb[j * 8 + kk * 4 + 2], pb[j * 8 + kk * 4 + 3]};
+          const bf16x8_t pf = __builtin_bit_cast(bf16x8_t, praw);
+  #pragma unroll
+          for (int dt = 0; dt < C::DT; ++dt) {
+            bf16x8_t vf;
+            if (D >= 32 || lq < (uint32_t)D) {
+              vf = *reinterpret_cast<const bf16x8_t*>(sVt + (dt * 32 + lq) * C::VROW + j * 32 + kk * 16 + half * 8);
+            } else {
+  #pragma unroll
+              for (int e = 0; e < 8; ++e) vf[e] = (__bf16)0.f;
+            }
+            acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf, acc[dt], 0, 0, 0);
+          }
+        }
+    }
+  
+}
   // ---- epilogue: normalise, store O (bf16) and LSE ----
   const float l_tot = l_run + __shfl_xor(l_run, 32, kWave);
   const bool row_ok = (int32_t)q_in_bucket < q_valid_len && l_tot > 0.f;
@@ -271,7 +376,6 @@ __device__ __forceinline__ void static_for(F&& f) {
 
 constexpr int kResMaxScope = 4;  // buckets per scope: at most 512 tokens in buckets of at least 128
 typedef short i16x4_t __attribute__((ext_vector_type(4)));
-typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
 typedef __attribute__((address_space(3))) void lds_void_t;
 typedef __attribute__((address_space(3))) i16x4_t lds_i16x4_t;
 
