@@ -14,6 +14,7 @@ constexpr int kXsChunk = 64;   // w rows per chunk (two 32-wide MFMA tiles)
 constexpr int kXsBufs = 3;     // w chunk buffers in LDS
 constexpr int kXsBiasSlots = 3;  // per-chunk bias slots in LDS (256 bytes each)
 constexpr int kPatchRow = 40;  // epilogue patch: 32 output columns + 8 pad (80-byte pitch keeps 16-byte alignment)
+constexpr int kPatchRow2 = 72;  // the same for 64 output columns (144-byte pitch)
 
 __device__ __forceinline__ float fast_silu(float a) {
   // a * sigmoid(a) with the hardware exp2 / rcp
@@ -67,10 +68,14 @@ __device__ __forceinline__ void xs_lds_dma2(const void* gbase, uint32_t voff, co
 __device__ __forceinline__ void xs_wait_vm(uint32_t n) {
   // vmcnt is split over bits 3:0 and 15:14 of the immediate; expcnt and lgkmcnt stay at "no wait"
 #define F3D_VM(N) case N: __builtin_amdgcn_s_waitcnt(0x0F70 | ((N) & 15) | (((N) >> 4) << 14)); break;
-  switch (n) {
+  switch (__builtin_amdgcn_readfirstlane(n)) {     // n is the same in every lane: branch on the scalar unit
     F3D_VM(0) F3D_VM(1) F3D_VM(2) F3D_VM(3) F3D_VM(4) F3D_VM(5) F3D_VM(6) F3D_VM(7) F3D_VM(8) F3D_VM(9) F3D_VM(10)
     F3D_VM(11) F3D_VM(12) F3D_VM(13) F3D_VM(14) F3D_VM(15) F3D_VM(16) F3D_VM(17) F3D_VM(18) F3D_VM(19) F3D_VM(20)
-    F3D_VM(21) F3D_VM(22) F3D_VM(23) F3D_VM(24)
+    F3D_VM(21) F3D_VM(22) F3D_VM(23) F3D_VM(24) F3D_VM(25) F3D_VM(26) F3D_VM(27) F3D_VM(28) F3D_VM(29) F3D_VM(30)
+    F3D_VM(31) F3D_VM(32) F3D_VM(33) F3D_VM(34) F3D_VM(35) F3D_VM(36) F3D_VM(37) F3D_VM(38) F3D_VM(39) F3D_VM(40)
+    F3D_VM(41) F3D_VM(42) F3D_VM(43) F3D_VM(44) F3D_VM(45) F3D_VM(46) F3D_VM(47) F3D_VM(48) F3D_VM(49) F3D_VM(50)
+    F3D_VM(51) F3D_VM(52) F3D_VM(53) F3D_VM(54) F3D_VM(55) F3D_VM(56) F3D_VM(57) F3D_VM(58) F3D_VM(59) F3D_VM(60)
+    F3D_VM(61) F3D_VM(62) F3D_VM(63)
     default: __builtin_amdgcn_s_waitcnt(0x0F70); break;
   }
 #undef F3D_VM

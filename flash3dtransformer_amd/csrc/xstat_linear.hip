@@ -28,10 +28,8 @@ namespace f3d {
 template <int K, int WAVES, int NBUF>
 constexpr size_t xs_lds_bytes() {
   using G = XsGeom<K>;
-  const size_t wbuf = (size_t)NBUF * G::CHUNK_BYTES;
-  const size_t xpatch = (size_t)WAVES * 32 * (G::KP + 8) * 2;
-  const size_t front = wbuf > xpatch ? wbuf : xpatch;
-  return front + (size_t)WAVES * 32 * kPatchRow * 2 + (size_t)kXsBiasSlots * 256;
+  const size_t front = (size_t)NBUF * G::CHUNK_BYTES;
+  return front + (size_t)WAVES * 32 * (K <= 256 ? kPatchRow2 : kPatchRow) * 2 + (size_t)kXsBiasSlots * 256;
 }
 
 // EPI: 0 = bias only, 1 = runtime activation and / or residual, 2 = residual only (its pieces are prefetched).
@@ -48,83 +46,17 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
   constexpr int ROWB = G::ROWB;
   constexpr int ROWS_WG = 32 * MT * WAVES;
   extern __shared__ __attribute__((aligned(1024))) char lds_xs[];
-  constexpr size_t kFront = (size_t)NBUF * G::CHUNK_BYTES > (size_t)WAVES * 32 * (G::KP + 8) * 2
-                                ? (size_t)NBUF * G::CHUNK_BYTES
-                                : (size_t)WAVES * 32 * (G::KP + 8) * 2;
+  constexpr size_t kFront = (size_t)NBUF * G::CHUNK_BYTES;
   constexpr uint32_t kAheadChunks = NBUF - 1;
   uint16_t* lds_patch = reinterpret_cast<uint16_t*>(lds_xs + kFront);
   // the bias of a chunk as fp32 (64 values), three slots: chunk c + 2 is parked while chunk c is being read
-  char* s_side = lds_xs + kFront + (size_t)WAVES * 32 * kPatchRow * 2;
+  constexpr int kPatchPitch = K <= 256 ? kPatchRow2 : kPatchRow;   // the 64-column patch where LDS has the room
+  char* s_side = lds_xs + kFront + (size_t)WAVES * 32 * kPatchPitch * 2;
   auto s_bias = [&](uint32_t c) -> float* { return reinterpret_cast<float*>(s_side + (c % kXsBiasSlots) * 256); };
 
   const uint32_t tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid / kWave), lane = tid % kWave;
   const uint32_t lq = lane & 31u, half = lane >> 5;
   const uint32_t row0 = blockIdx.x * ROWS_WG + wave * (32 * MT);
-
-  // ---- this wave's x rows -> registers in the B-operand layout.  Loaded row-contiguously and
-  //      transposed through a wave-private LDS patch, KP columns at a time ----
-  bf16x8_t xf[MT][KS];
-  {
-    constexpr int KP = G::KP, PROW = KP + 8, PCPR = KP / 8;
-    uint16_t* patch = reinterpret_cast<uint16_t*>(lds_xs) + wave * (32 * PROW);
-    constexpr int XLOADS = (32 * PCPR) / kWave;
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-      for (int kp = 0; kp < K / KP; ++kp) {
-        u32x4_t v[XLOADS];
-#pragma unroll
-        for (int i = 0; i < XLOADS; ++i) {
-          const uint32_t id = lane + i * kWave;
-          const uint32_t rr = id / PCPR, kc = (id % PCPR) * 8;
-          const uint32_t r = min(row0 + mt * 32 + rr, M - 1);
-          v[i] = *reinterpret_cast<const u32x4_t*>(x + (size_t)r * ldx + kp * KP + kc);
-        }
-#pragma unroll
-        for (int i = 0; i < XLOADS; ++i) {
-          const uint32_t id = lane + i * kWave;
-          const uint32_t rr = id / PCPR, kc = (id % PCPR) * 8;
-          *reinterpret_cast<u32x4_t*>(patch + rr * PROW + kc) = v[i];
-        }
-#pragma unroll
-        for (int ks = 0; ks < KP / 16; ++ks)
-          xf[mt][kp * (KP / 16) + ks] = *reinterpret_cast<const bf16x8_t*>(patch + lq * PROW + ks * 16 + half * 8);
-      }
-  }
-  // LayerNorm of this lane's rows in place: one sweep for the sums of d = x - x0 and d^2 (shifted by the row's first
-  // element so that the variance does not cancel), one that writes bf16((x - mean) * rstd) back
-  if (LN) {
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-      const float x0 = __shfl((float)xf[mt][0][0], lq, kWave);   // lane lq (half 0) holds element 0 of row lq
-      float s = 0.f, q = 0.f;
-#pragma unroll
-      for (int ks = 0; ks < KS; ++ks)
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          const float d = (float)xf[mt][ks][e] - x0;
-          s += d;
-          q = __builtin_fmaf(d, d, q);
-        }
-      const float sm = pair_sum(s) * (1.0f / K);
-      const float var = fmaxf(pair_sum(q) * (1.0f / K) - sm * sm, 0.f);
-      const float rstd = rsqrtf(var + eps), shift = -(x0 + sm) * rstd;
-      // one fragment at a time (kept opaque: otherwise the compiler holds every row element as a float from the first
-      // sweep to the second, 8 registers per fragment, and spills)
-#pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        u32x4_t raw = __builtin_bit_cast(u32x4_t, xf[mt][ks]);
-        asm volatile("" : "+v"(raw));
-        u32x4_t pk;
-#pragma unroll
-        for (int e = 0; e < 4; ++e)
-          pk[e] = pack_bf16x2(__builtin_fmaf(bf16_lo(raw[e]), rstd, shift), __builtin_fmaf(bf16_hi(raw[e]), rstd, shift));
-        asm volatile("" : "+v"(pk));
-        xf[mt][ks] = __builtin_bit_cast(bf16x8_t, pk);
-      }
-    }
-  }
-  __syncthreads();  // the transposition patches are dead; the space now holds w chunks
 
   // ---- w chunk streaming ----
   const uint32_t n_out = SWIGLU ? N / 2 : N;
@@ -170,14 +102,60 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
   auto actual = [&](uint32_t i) -> uint32_t { const uint32_t t = i + c_start; return t >= nchunk ? t - nchunk : t; };
 
   if (!bias_dma && tid < 64 * kXsBiasSlots) reinterpret_cast<float*>(s_side)[tid] = 0.f;   // no bias: zeros, once
+  // the first chunk(s) of w are requested before anything else, so that they travel while the rows are fetched
   dma_chunk(actual(0), 0, 0);
   if (kAheadChunks > 1 && nchunk > 1) dma_chunk(actual(1), 1, 1);
+
+  // ---- this wave's x rows -> registers in the B-operand layout: fragment ks of row tile mt is 16 bytes of row lq
+  //      at columns ks * 16 + half * 8, loaded straight into its register, all of them in flight at once (the four
+  //      fragments that share a 128-byte line are requested back to back).  Rows past M read row M - 1. ----
+  bf16x8_t xf[MT][KS];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    const uint32_t r = min(row0 + mt * 32 + lq, M - 1);
+    const uint16_t* xp = x + (size_t)r * ldx + half * 8;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) xf[mt][ks] = *reinterpret_cast<const bf16x8_t*>(xp + ks * 16);
+  }
+  // LayerNorm of this lane's rows in place: one sweep for the sums of d = x - x0 and d^2 (shifted by the row's first
+  // element so that the variance does not cancel), one that writes bf16((x - mean) * rstd) back
+  if (LN) {
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      const float x0 = __shfl((float)xf[mt][0][0], lq, kWave);   // lane lq (half 0) holds element 0 of row lq
+      float s = 0.f, q = 0.f;
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const float d = (float)xf[mt][ks][e] - x0;
+          s += d;
+          q = __builtin_fmaf(d, d, q);
+        }
+      const float sm = pair_sum(s) * (1.0f / K);
+      const float var = fmaxf(pair_sum(q) * (1.0f / K) - sm * sm, 0.f);
+      const float rstd = rsqrtf(var + eps), shift = -(x0 + sm) * rstd;
+      // one fragment at a time (kept opaque: otherwise the compiler holds every row element as a float from the first
+      // sweep to the second, 8 registers per fragment, and spills)
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        u32x4_t raw = __builtin_bit_cast(u32x4_t, xf[mt][ks]);
+        asm volatile("" : "+v"(raw));
+        u32x4_t pk;
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          pk[e] = pack_bf16x2(__builtin_fmaf(bf16_lo(raw[e]), rstd, shift), __builtin_fmaf(bf16_hi(raw[e]), rstd, shift));
+        asm volatile("" : "+v"(pk));
+        xf[mt][ks] = __builtin_bit_cast(bf16x8_t, pk);
+      }
+    }
+  }
   __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): the first chunk(s) have landed
   __syncthreads();
 
   // per-lane byte offset of its fragment inside a chunk buffer; k-step ks is reached by ^ (32 ks)
   const uint32_t frag_off = lq * ROWB + (((half ^ G::swz(lq)) & (uint32_t)(G::CPR - 1)) << 4);
-  uint16_t* patch = lds_patch + wave * (32 * kPatchRow);
+  uint16_t* patch = lds_patch + wave * (32 * kPatchPitch);
 
   // accumulators: acc[nt][mt][g*4+r] <-> column nt*32 + g*8 + half*4 + r
   f32x16_t acc[2][MT];
@@ -235,38 +213,62 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
       if (ks + kAhead < KS) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
     }
   };
-  // stage 3: epilogue of chunk ci: the wave's 32 x 32 result tiles go through a wave-private LDS patch so
-  // that the global stores are row-contiguous 16-byte pieces (4 lanes = 64 bytes of one row)
+  // stage 3: epilogue of chunk ci: a row tile's results (32 rows x 64 columns, 32 after swiglu) go through a
+  // wave-private LDS patch so that the global stores are row-contiguous: 8 lanes write the 128 bytes of one row (a
+  // whole line; measured against 64-byte pieces at this layer's pace: 5.2 against 4.2 TB/s), 4 lanes the 64 bytes
+  // of a gated row
+  constexpr bool WIDE = !SWIGLU && K <= 256 && EPI == 2;      // a row tile's 64 columns in one flush
+  constexpr int PW = WIDE ? 64 : 32;                          // output columns per flush
+  constexpr int NF = (SWIGLU || WIDE) ? 1 : 2;                // flushes per row tile
+  constexpr int PPITCH = WIDE ? kPatchRow2 : kPatchRow;       // patch pitch in elements
+  constexpr int LPR = PW / 8, RPI = kWave / LPR, NI = 32 / RPI;   // lanes per row, rows per instruction, instructions
+  // byte offsets of this lane's piece inside a block of RPI rows: kernel-lifetime constants, so that a store or a
+  // residual load needs one vector register of address (the rest of the address is uniform)
+  const uint32_t ch = (lane % LPR) * 8;      // this lane's 8 columns of a flush
+  const uint32_t y_lane = ((lane / LPR) * ldy + ch) * 2u, r_lane = ((lane / LPR) * ldr + ch) * 2u;
   auto stage_epilogue = [&](uint32_t ci) {
     const uint32_t col0 = actual(ci) * COLS;   // first output column of the chunk
+    // a plain last chunk may hold 32 columns only: the lanes of the missing ones read 32 columns further left (a valid
+    // address, the value is not used) and store nothing
+    auto col_ok = [&](int f) -> bool { return col0 + f * PW + ch < n_out; };
+    // uniform base of row block i of row tile mt (rows wave * 32 MT + mt * 32 + i * RPI ...), columns of flush f
+    auto y_base = [&](int mt, int f, int i) -> char* {
+      return reinterpret_cast<char*>(y_wg) + ((size_t)(wave * (32 * MT) + mt * 32 + i * RPI) * ldy + col0 + f * PW) * 2u;
+    };
+    auto r_base = [&](int mt, int f, int i) -> const char* {
+      return reinterpret_cast<const char*>(res_wg) + ((size_t)(wave * (32 * MT) + mt * 32 + i * RPI) * ldr + col0 + f * PW) * 2u;
+    };
     // Residual pieces of the whole chunk are requested up front (one memory latency for all of them, hidden
     // behind the packing below) instead of one by one where they are added.  Rows past M read row M - 1.
-    constexpr int NT_OUT = SWIGLU ? 1 : 2;
-    u32x4_t rres[EPI == 2 ? MT : 1][NT_OUT][2];
+    u32x4_t rres[EPI == 2 ? MT : 1][NF][NI];
     if (EPI == 2) {
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-        for (int nt = 0; nt < NT_OUT; ++nt)
+        for (int f = 0; f < NF; ++f)
 #pragma unroll
-          for (int h2 = 0; h2 < 2; ++h2) {
-            const uint32_t rr = (lane >> 2) + h2 * 16, ch = (lane & 3u) * 8;
-            const uint32_t row = min(row0 + mt * 32 + rr, M - 1);
-            const uint32_t lrow = row - blockIdx.x * ROWS_WG;
-            if (col0 + nt * 32 < n_out)
-              rres[mt][nt][h2] = *reinterpret_cast<const u32x4_t*>(res_wg + (lrow * ldr + col0 + nt * 32 + ch));
+          for (int i = 0; i < NI; ++i) {
+            if (wg_full) {
+              rres[mt][f][i] = *reinterpret_cast<const u32x4_t*>(r_base(mt, f, i) + (col_ok(f) ? r_lane : r_lane - 64u));
+            } else {
+              const uint32_t rr = lane / LPR + i * RPI;
+              const uint32_t lrow = min(row0 + mt * 32 + rr, M - 1) - blockIdx.x * ROWS_WG;
+              const uint32_t col = col_ok(f) ? col0 + f * PW + ch : n_out - 8;
+              rres[mt][f][i] = *reinterpret_cast<const u32x4_t*>(res_wg + (lrow * ldr + col));
+            }
           }
     }
-    auto flush_tile = [&](auto full_tag, int mt, int nt_out, uint32_t colbase) {
-      // patch holds rows [mt*32, mt*32+32) x 32 columns starting at output column colbase
+    auto flush_tile = [&](auto full_tag, int mt, int f) {
+      // patch holds rows [mt*32, mt*32+32) x PW columns starting at output column col0 + f * PW
       constexpr bool kFull = decltype(full_tag)::value;
+      const bool ok = col_ok(f);
 #pragma unroll
-      for (int h2 = 0; h2 < 2; ++h2) {
-        const uint32_t rr = (lane >> 2) + h2 * 16, ch = (lane & 3u) * 8;
+      for (int i = 0; i < NI; ++i) {
+        // two row blocks at a time: their patch reads are in flight together, and no more registers are held than that
+        if (i > 0 && i % 2 == 0) __builtin_amdgcn_sched_barrier(0);
+        const uint32_t rr = lane / LPR + i * RPI;
         const uint32_t row = row0 + mt * 32 + rr;
-        // element offsets from the workgroup's first row fit 32 bits (512 rows at most)
-        const uint32_t lrow = wave * (32 * MT) + mt * 32 + rr;
-        u32x4_t t = *reinterpret_cast<const u32x4_t*>(patch + rr * kPatchRow + ch);
+        u32x4_t t = *reinterpret_cast<const u32x4_t*>(patch + rr * PPITCH + ch);
         if (!kFull && row >= M) continue;
         if (EPI == 1) {
           if (!SWIGLU && act != F3D_ACT_NONE) {
@@ -274,19 +276,19 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
             for (int e = 0; e < 4; ++e) t[e] = pack_bf16x2(xs_act(bf16_lo(t[e]), act), xs_act(bf16_hi(t[e]), act));
           }
           if (residual) {
-            const u32x4_t rv = *reinterpret_cast<const u32x4_t*>(res_wg + (lrow * ldr + colbase + ch));
+            const u32x4_t rv = *reinterpret_cast<const u32x4_t*>(r_base(mt, f, i) + (ok ? r_lane : r_lane - 64u));
 #pragma unroll
             for (int e = 0; e < 4; ++e)
               t[e] = pack_bf16x2(bf16_lo(t[e]) + bf16_lo(rv[e]), bf16_hi(t[e]) + bf16_hi(rv[e]));
           }
         }
         if (EPI == 2) {
-          const u32x4_t rv = rres[EPI == 2 ? mt : 0][nt_out][h2];
+          const u32x4_t rv = rres[EPI == 2 ? mt : 0][f][i];
 #pragma unroll
           for (int e = 0; e < 4; ++e)
             t[e] = pack_bf16x2(bf16_lo(t[e]) + bf16_lo(rv[e]), bf16_hi(t[e]) + bf16_hi(rv[e]));
         }
-        *reinterpret_cast<u32x4_t*>(y_wg + (lrow * ldy + colbase + ch)) = t;
+        if (ok) *reinterpret_cast<u32x4_t*>(y_base(mt, f, i) + y_lane) = t;
       }
     };
     auto epilogue = [&](auto full_tag) {
@@ -300,10 +302,11 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
               uint2 pk;   // Linear output is bf16
               pk.x = pack_bf16x2(acc[nt][mt][g * 4 + 0], acc[nt][mt][g * 4 + 1]);
               pk.y = pack_bf16x2(acc[nt][mt][g * 4 + 2], acc[nt][mt][g * 4 + 3]);
-              *reinterpret_cast<uint2*>(patch + lq * kPatchRow + g * 8 + half * 4) = pk;
+              *reinterpret_cast<uint2*>(patch + lq * PPITCH + (WIDE ? nt * 32 : 0) + g * 8 + half * 4) = pk;
             }
-            if (col0 + nt * 32 < N) flush_tile(full_tag, mt, nt, col0 + nt * 32);
+            if (!WIDE) flush_tile(full_tag, mt, nt);
           }
+          if (WIDE) flush_tile(full_tag, mt, 0);
         } else {
 #pragma unroll
           for (int g = 0; g < 4; ++g) {
@@ -317,9 +320,9 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
             uint2 pk;
             pk.x = pack_bf16x2(hv[0], hv[1]);
             pk.y = pack_bf16x2(hv[2], hv[3]);
-            *reinterpret_cast<uint2*>(patch + lq * kPatchRow + g * 8 + half * 4) = pk;
+            *reinterpret_cast<uint2*>(patch + lq * PPITCH + g * 8 + half * 4) = pk;
           }
-          flush_tile(full_tag, mt, 0, col0);
+          flush_tile(full_tag, mt, 0);
         }
       }
     };
@@ -327,14 +330,16 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
   };
   // Chunk ci + 1 must have landed when the interval ends.  Its requests were issued one interval ago; since then this
   // wave has issued the memory operations of one epilogue (stores, and the residual loads of EPI 2: kEpiOps of them
-  // when every row of the workgroup is stored) and the requests of chunk ci + 2 (my_dma).  Memory operations complete
-  // in order, so "at most that many outstanding" is the weakest wait that covers chunk ci + 1, and it does not wait
-  // for the stores.  Where the epilogue's count is not fixed (partial workgroup, run-time residual) the stores are
-  // not allowed for: the wait is then early, never late.
-  constexpr uint32_t kEpiOps = EPI == 1 ? 0u : (uint32_t)(MT * (SWIGLU ? 1 : 2) * 2 * (EPI == 2 ? 2 : 1));
-  const uint32_t wait_n = my_dma + (wg_full ? kEpiOps : 0u);
+  // when every row of the workgroup is stored; none before the first epilogue) and the requests of chunk ci + 2
+  // (my_dma).  Memory operations complete in order, so "at most that many outstanding" is the weakest wait that covers
+  // chunk ci + 1, and it does not wait for the stores.  Allowing MORE than were issued would let the wait return before
+  // the chunk has landed; where the epilogue's count is not fixed (partial workgroup, run-time residual) the stores
+  // are therefore not allowed for: the wait is then early, never late.
+  // (two flushes of 32 columns per row tile: a last chunk may issue half of them, so none are allowed for)
+  const uint32_t kEpiOps = (EPI == 1 || !wg_full || NF > 1) ? 0u : (uint32_t)(MT * NI * (EPI == 2 ? 2 : 1));
   auto wait_next_chunk = [&](uint32_t ci) {
-    if (kAheadChunks > 1 && ci + kAheadChunks < nchunk) xs_wait_vm(wait_n); else __builtin_amdgcn_s_waitcnt(0x0F70);
+    if (kAheadChunks > 1 && ci + kAheadChunks < nchunk) xs_wait_vm(my_dma + (ci > 0 ? kEpiOps : 0u));
+    else __builtin_amdgcn_s_waitcnt(0x0F70);
   };
 
   // The two waves that share a SIMD (wave v and v + WAVES/2) run the stages of a barrier interval in
