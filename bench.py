@@ -273,7 +273,7 @@ def sub_metrics(dev, only=None):
     unpooling GB/s on config 3 — each against its roofline.  `only`: a set of group names, or None for all"""
     out = {}
     groups = {"attention": sub_attention, "psh": sub_psh, "permute": sub_permute, "pool": sub_pool,
-              "hourglass": sub_hourglass, "mfma": sub_mfma_rate,
+              "hourglass": sub_hourglass, "mfma": sub_mfma_rate, "stores": sub_store_rows,
               "backward": sub_backward}
     for name, fn in groups.items():
         if only is None or name in only:
@@ -341,6 +341,30 @@ def sub_mfma_rate(dev, out):
         out["ln_mlp_swiglu_256x1024_" + name] = {"ms": round(ms, 4), "tflops": round(fl / ms / 1e9, 1),
                                                  "frac_of_bf16_mfma_peak": round(fl / ms / 1e9 / MFMA_BF16_PEAK_TFLOPS, 4)}
         del x, w1, w2
+
+
+def sub_store_rows(dev, out):
+    """the write roof of the row-panel linear layers: their output (482,304 rows x 768 and x 256 bf16) written with
+    their own workgroup / chunk / wave geometry and nothing else, in row pieces of 64 and of 128 bytes, back to back and
+    with a pause per chunk (40 s_sleep, about the length of a chunk's products)"""
+    import ctypes
+    lib = _bench_probe()
+    u32, vp = ctypes.c_uint32, ctypes.c_void_p
+    M = 482_304
+    for n in (768, 256):
+        y = torch.empty(M, n, dtype=torch.bfloat16, device=dev)
+        for piece in (64, 128):
+            for pause in (0, 40):
+                def run():
+                    rc = lib.bench_probe_store_rows(vp(y.data_ptr()), u32(n), u32(M), u32(n), u32(piece), u32(pause),
+                                                    vp(torch.cuda.current_stream(0).cuda_stream))
+                    if rc != 0:
+                        raise RuntimeError(f"bench_probe_store_rows failed with {rc}")
+                ms = ev_time(run, 20)
+                out[f"store_rows_{M}x{n}_piece{piece}" + ("_paced" if pause else "")] = {
+                    "ms": round(ms, 4), "gbs": round(M * n * 2 / ms / 1e6, 1),
+                    "frac_of_hbm_peak": round(M * n * 2 / ms / 1e6 / HBM_PEAK_GBS, 4)}
+        del y
 
 
 def sub_backward(dev, out):

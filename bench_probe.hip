@@ -7,6 +7,12 @@
 // clock; with a zero operand the multipliers do not toggle and the rate is the 2.5 PFLOP/s of the data sheet.  Every
 // workgroup's first lane reads the shader-clock counter and the 100 MHz constant-rate counter at its start and end:
 // their ratio is the clock the products ran at.
+//
+// bench_probe_store_rows: what HBM takes when a [m][n] bf16 output is written the way the row-panel linear layers write
+// it: workgroups of eight waves own 512 rows, walk the 64-column chunks in rotated order, and a wave stores its 64 rows
+// of a chunk in row-contiguous pieces of 64 bytes (4 lanes per row, 16 rows per instruction) or 128 bytes (8 lanes per
+// row, 8 rows per instruction), with or without a pause per chunk that stands for the products between two
+// epilogues.  The write roof those layers sit under.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -49,7 +55,41 @@ __global__ __launch_bounds__(256) void probe_mfma_kernel(float* __restrict__ sin
   }
 }
 
+typedef uint32_t probe_u32x4 __attribute__((ext_vector_type(4)));
+
+template <int PIECE>
+__global__ __launch_bounds__(512) void probe_store_rows_kernel(uint16_t* __restrict__ y, uint32_t ldy, uint32_t m, uint32_t n,
+                                                              uint32_t pause) {
+  const uint32_t wave = threadIdx.x / 64, lane = threadIdx.x % 64;
+  const uint32_t nchunk = n / 64, c0 = (blockIdx.x * 5u) % nchunk;
+  const uint32_t row_w = blockIdx.x * 512 + wave * 64;
+  const probe_u32x4 v = {lane, wave, blockIdx.x, 7u};
+  constexpr uint32_t LPR = PIECE / 16, RPI = 64 / LPR;   // lanes per row, rows per instruction
+  for (uint32_t i = 0; i < nchunk; ++i) {
+    const uint32_t c = (i + c0) % nchunk;
+    for (uint32_t p = 0; p < pause; ++p) __builtin_amdgcn_s_sleep(1);
+#pragma unroll
+    for (uint32_t piece = 0; piece < 128 / PIECE; ++piece)
+#pragma unroll
+      for (uint32_t r0 = 0; r0 < 64; r0 += RPI) {
+        const uint32_t row = row_w + r0 + lane / LPR, col = c * 64 + piece * (PIECE / 2) + (lane % LPR) * 8;
+        if (row < m) *reinterpret_cast<probe_u32x4*>(y + ((size_t)row * ldy + col)) = v;
+      }
+  }
+}
+
 extern "C" {
+
+// Writes all of y[m][n] (bf16, row stride ldy elements, n a multiple of 64) in pieces of piece_bytes (64 or 128) per
+// row and instruction, `pause` s_sleep instructions per chunk.  Returns 0, -1 for bad arguments, or the HIP error code.
+int bench_probe_store_rows(uint16_t* y, uint32_t ldy, uint32_t m, uint32_t n, uint32_t piece_bytes, uint32_t pause,
+                           void* stream) {
+  if (!y || m == 0 || n == 0 || n % 64 != 0 || ldy < n || ldy % 8 != 0 || (piece_bytes != 64 && piece_bytes != 128)) return -1;
+  const dim3 grid((m + 511) / 512), block(512);
+  if (piece_bytes == 64) hipLaunchKernelGGL(probe_store_rows_kernel<64>, grid, block, 0, (hipStream_t)stream, y, ldy, m, n, pause);
+  else hipLaunchKernelGGL(probe_store_rows_kernel<128>, grid, block, 0, (hipStream_t)stream, y, ldy, m, n, pause);
+  return (int)hipGetLastError();
+}
 
 // workgroups x 4 waves x iters x 8 products of 32,768 flops.  sink: one float of device memory (never written);
 // clocks: 2 x workgroups uint64 of device memory (shader-clock ticks, 100 MHz ticks per workgroup) or NULL.

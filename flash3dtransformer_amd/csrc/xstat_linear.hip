@@ -213,10 +213,12 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
       if (ks + kAhead < KS) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
     }
   };
-  // stage 3: epilogue of chunk ci: a row tile's results (32 rows x 64 columns, 32 after swiglu) go through a
-  // wave-private LDS patch so that the global stores are row-contiguous: 8 lanes write the 128 bytes of one row (a
-  // whole line; measured against 64-byte pieces at this layer's pace: 5.2 against 4.2 TB/s), 4 lanes the 64 bytes
-  // of a gated row
+  // stage 3: epilogue of chunk ci: the results go through a wave-private LDS patch so that the global stores are
+  // row-contiguous.  Residual layers flush a row tile's 64 columns at once: 8 lanes read and write the 128 bytes (a
+  // whole line) of one row; measured at 482,304 rows, 256 -> 256: 0.150 against 0.171 ms with 64-byte pieces.  The
+  // bias-only epilogue keeps 32-column flushes (4 lanes per row): whole lines measured 3 % slower there (256 -> 768:
+  // 0.276 against 0.268 ms, same GPU), although a store-only loop of the same geometry takes them faster (5.1 against
+  // 3.7 TB/s): the layer is bound by the chain of stages of a wave, which the longer flush lengthens.
   constexpr bool WIDE = !SWIGLU && K <= 256 && EPI == 2;      // a row tile's 64 columns in one flush
   constexpr int PW = WIDE ? 64 : 32;                          // output columns per flush
   constexpr int NF = (SWIGLU || WIDE) ? 1 : 2;                // flushes per row tile
