@@ -233,6 +233,8 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
     // a plain last chunk may hold 32 columns only: the lanes of the missing ones read 32 columns further left (a valid
     // address, the value is not used) and store nothing
     auto col_ok = [&](int f) -> bool { return col0 + f * PW + ch < n_out; };
+    // (a SIGNED offset: 64 bytes to the left of the flush's first column, which lies at least 32 columns into the row)
+    auto r_off = [&](int f) -> ptrdiff_t { return col_ok(f) ? (ptrdiff_t)r_lane : (ptrdiff_t)r_lane - 64; };
     // uniform base of row block i of row tile mt (rows wave * 32 MT + mt * 32 + i * RPI ...), columns of flush f
     auto y_base = [&](int mt, int f, int i) -> char* {
       return reinterpret_cast<char*>(y_wg) + ((size_t)(wave * (32 * MT) + mt * 32 + i * RPI) * ldy + col0 + f * PW) * 2u;
@@ -251,7 +253,7 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
 #pragma unroll
           for (int i = 0; i < NI; ++i) {
             if (wg_full) {
-              rres[mt][f][i] = *reinterpret_cast<const u32x4_t*>(r_base(mt, f, i) + (col_ok(f) ? r_lane : r_lane - 64u));
+              rres[mt][f][i] = *reinterpret_cast<const u32x4_t*>(r_base(mt, f, i) + r_off(f));
             } else {
               const uint32_t rr = lane / LPR + i * RPI;
               const uint32_t lrow = min(row0 + mt * 32 + rr, M - 1) - blockIdx.x * ROWS_WG;
@@ -278,7 +280,7 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
             for (int e = 0; e < 4; ++e) t[e] = pack_bf16x2(xs_act(bf16_lo(t[e]), act), xs_act(bf16_hi(t[e]), act));
           }
           if (residual) {
-            const u32x4_t rv = *reinterpret_cast<const u32x4_t*>(r_base(mt, f, i) + (ok ? r_lane : r_lane - 64u));
+            const u32x4_t rv = *reinterpret_cast<const u32x4_t*>(r_base(mt, f, i) + r_off(f));
 #pragma unroll
             for (int e = 0; e < 4; ++e)
               t[e] = pack_bf16x2(bf16_lo(t[e]) + bf16_lo(rv[e]), bf16_hi(t[e]) + bf16_hi(rv[e]));
