@@ -54,6 +54,8 @@ def test_gemm_sm_bf16_reference_case():
     (140000, 32, 32, "gelu", True, True),
     (3001, 1536, 512, None, True, False),      # qkv of a C=512 level: 512 inner features in the row-panel kernel, ragged M
     (2500, 512, 512, None, True, True),        # out-projection + residual of that level
+    (2100, 96, 512, None, True, True),         # 512 inner features, residual, 32 columns in the last chunk
+    (120000, 32, 256, "silu", True, True),     # activation + residual on a single 32-column chunk, 512-row configuration
     (2100, 2048, 512, "swiglu", True, False),  # its fc1
     (700, 256, 512, "gelu", False, True),      # fc2 of a C=256 level
     (40000, 256, 1024, None, True, True),      # fc2 + residual of the C=256 block at a size the output-panel kernel takes
