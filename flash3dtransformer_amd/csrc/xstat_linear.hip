@@ -25,11 +25,15 @@
 
 namespace f3d {
 
+// the 64-column epilogue patch (residual layers with K <= 256) or the 32-column one
+template <int K, bool SWIGLU, int EPI>
+constexpr bool xs_wide_flush() { return !SWIGLU && K <= 256 && EPI == 2; }
+
 template <int K, int WAVES, int NBUF>
-constexpr size_t xs_lds_bytes() {
+constexpr size_t xs_lds_bytes(bool wide) {
   using G = XsGeom<K>;
   const size_t front = (size_t)NBUF * G::CHUNK_BYTES;
-  return front + (size_t)WAVES * 32 * (K <= 256 ? kPatchRow2 : kPatchRow) * 2 + (size_t)kXsBiasSlots * 256;
+  return front + (size_t)WAVES * 32 * (wide ? kPatchRow2 : kPatchRow) * 2 + (size_t)kXsBiasSlots * 256;
 }
 
 // EPI: 0 = bias only, 1 = runtime activation and / or residual, 2 = residual only (its pieces are prefetched).
@@ -50,7 +54,8 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
   constexpr uint32_t kAheadChunks = NBUF - 1;
   uint16_t* lds_patch = reinterpret_cast<uint16_t*>(lds_xs + kFront);
   // the bias of a chunk as fp32 (64 values), three slots: chunk c + 2 is parked while chunk c is being read
-  constexpr int kPatchPitch = K <= 256 ? kPatchRow2 : kPatchRow;   // the 64-column patch where LDS has the room
+  constexpr bool WIDE = xs_wide_flush<K, SWIGLU, EPI>();   // a row tile's 64 columns in one flush
+  constexpr int kPatchPitch = WIDE ? kPatchRow2 : kPatchRow;
   char* s_side = lds_xs + kFront + (size_t)WAVES * 32 * kPatchPitch * 2;
   auto s_bias = [&](uint32_t c) -> float* { return reinterpret_cast<float*>(s_side + (c % kXsBiasSlots) * 256); };
 
@@ -219,7 +224,6 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
   // bias-only epilogue keeps 32-column flushes (4 lanes per row): whole lines measured 3 % slower there (256 -> 768:
   // 0.276 against 0.268 ms, same GPU), although a store-only loop of the same geometry takes them faster (5.1 against
   // 3.7 TB/s): the layer is bound by the chain of stages of a wave, which the longer flush lengthens.
-  constexpr bool WIDE = !SWIGLU && K <= 256 && EPI == 2;      // a row tile's 64 columns in one flush
   constexpr int PW = WIDE ? 64 : 32;                          // output columns per flush
   constexpr int NF = (SWIGLU || WIDE) ? 1 : 2;                // flushes per row tile
   constexpr int PPITCH = WIDE ? kPatchRow2 : kPatchRow;       // patch pitch in elements
@@ -396,11 +400,11 @@ static int launch_k(bool ln, bool swiglu, hipStream_t s, const uint16_t* x, uint
   const bool general = act != F3D_ACT_NONE || residual != nullptr;
   const bool res_only = act == F3D_ACT_NONE && residual != nullptr;
   const dim3 grid(cdiv_u32(M, 32 * MT * WAVES)), block(64 * WAVES);
-  constexpr size_t lds = xs_lds_bytes<K, WAVES, NBUF>();
 #define F3D_XS(L, S, E)                                                                                            \
   do {                                                                                                             \
     static bool attr_set[64] = {};                                                                                 \
     auto kern = xstat_linear_kernel<K, MT, WAVES, NBUF, L, S, E>;                                                       \
+    constexpr size_t lds = xs_lds_bytes<K, WAVES, NBUF>(xs_wide_flush<K, S, E>());                                 \
     if (device < 0 || device >= 64 || !attr_set[device]) {                                                         \
       F3D_CHECK_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds)); \
       if (device >= 0 && device < 64) attr_set[device] = true;                                                     \
