@@ -69,6 +69,36 @@ __device__ __forceinline__ void tile_quat_lanes(uint32_t seed, uint32_t cloud, u
   for (int i = 0; i < 4; ++i) q[i] = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, unit), i));
 }
 
+// acc[d] += x[d] of the lane s above, s = 1 .. S - 1 in this order (a sequential sum, as the members are summed one by
+// one), for power-of-two groups of at most 16 lanes, which never straddle a row of 16 lanes.  Lane i reads lane i + s of
+// its row through a row shift of the operand (DPP); a member past the tile's last point (tid + s >= m) is not added.
+template <int SH>
+__device__ __forceinline__ float row_up(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x100 + SH, 0xF, 0xF, true));
+}
+template <int SH, int SMAX>
+__device__ __forceinline__ void seq_sum_steps(const float (&x)[3], float (&acc)[3], uint32_t tid, uint32_t m) {
+  if constexpr (SH < SMAX) {
+    const bool take = tid + SH < m;
+#pragma unroll
+    for (int d = 0; d < 3; ++d) {
+      const float v = row_up<SH>(x[d]);
+      if (take) acc[d] = __fadd_rn(acc[d], v);
+    }
+    seq_sum_steps<SH + 1, SMAX>(x, acc, tid, m);
+  }
+}
+__device__ __forceinline__ void seq_sum_row16(const float (&x)[3], float (&acc)[3], uint32_t S, uint32_t tid, uint32_t m) {
+  switch (S) {
+    case 2: seq_sum_steps<1, 2>(x, acc, tid, m); break;
+    case 4: seq_sum_steps<1, 4>(x, acc, tid, m); break;
+    case 8: seq_sum_steps<1, 8>(x, acc, tid, m); break;
+    case 16: seq_sum_steps<1, 16>(x, acc, tid, m); break;
+    default: break;   // S = 1: nothing to add
+  }
+}
+
+
 __global__ __launch_bounds__(kSubThreads) void subbuck_build_kernel(
     const uint16_t* __restrict__ coord, const uint32_t* __restrict__ batch_sep,
     const uint32_t* __restrict__ reduced_batch_sep, uint32_t batch_size, uint32_t total_n, uint32_t subbuck_size,
@@ -268,12 +298,18 @@ __global__ __launch_bounds__(kSubThreads) void subbuck_build_kernel(
     }
 #pragma unroll
     for (int d = 0; d < 3; ++d) acc[d] = __fadd_rn(0.f, x[d]);
-    for (uint32_t s = 1; s < S; ++s) {
-      const bool take = tid + s < m;
+    if (S <= 16u) {
+      // the group lies inside one row of 16 lanes: the neighbour s lanes up arrives through the data-parallel
+      // primitive of the adder's operand (one instruction per member and coordinate, no LDS permute)
+      seq_sum_row16(x, acc, S, tid, m);
+    } else {
+      for (uint32_t s = 1; s < S; ++s) {
+        const bool take = tid + s < m;
 #pragma unroll
-      for (int d = 0; d < 3; ++d) {
-        const float v = __shfl_down(x[d], s, kWave);
-        if (take) acc[d] = __fadd_rn(acc[d], v);
+        for (int d = 0; d < 3; ++d) {
+          const float v = __shfl_down(x[d], s, kWave);
+          if (take) acc[d] = __fadd_rn(acc[d], v);
+        }
       }
     }
     if (valid && (tid & (S - 1u)) == 0u) {

@@ -28,6 +28,8 @@ def _pool(coords, seps, feat_bits, S, op, out_align, oracle):
     (3, 0, [1300, 1400, 1023], 256),       # S does not divide 1024: 1023-point tiles
     (4, 3, [5000, 1], 64),
     (8, 2, [4096], 128),
+    (16, 0, [3000, 1029], 64),             # the widest group that is summed through row shifts
+    (32, 0, [2100, 33], 64),               # groups of two lane rows
     (2, 1, [3000, 2999], 40),              # 40 channels: 5 chunks per row
     (2, 0, [2000], 20),                    # channel count not a multiple of 8: scalar path
 ])
