@@ -34,6 +34,11 @@ class BuckSwinFwdFunction(Function):
         return bwd.dQ, bwd.dK, bwd.dV, None, None
 
 
+def _covers(scope_buckets, buck_size: int, L: int) -> bool:
+    """the planner vouches that its table covers all rows, and the table was made for a tensor of this length"""
+    return bool(getattr(scope_buckets, "covers_all_rows", False)) and scope_buckets.numel() * buck_size == L
+
+
 class BuckSwinQKVFunction(Function):
     """The same attention over the three thirds of one projection output qkv [B, L, 3 H D] (the kernel reads Q, K, V
     as column slices).  The backward writes dQ, dK, dV straight into the thirds of one [B, L, 3 H D] gradient, so
@@ -44,7 +49,7 @@ class BuckSwinQKVFunction(Function):
         B, L, C3 = qkv.shape
         D = C3 // 3 // num_heads
         Q, K, V = (t.view(B, L, num_heads, D) for t in torch.chunk(qkv, 3, dim=-1))
-        buff = sa.BuckSwinFwdBuffers.create_buckswin_fwd_buff(Q)
+        buff = sa.BuckSwinFwdBuffers.create_buckswin_fwd_buff(Q, _covers(scope_buckets, buck_size, L))
         pshattn.buck_swin_fwd(Q, K, V, buff.O, buff.LSE, scope_buckets, buck_size)
         ctx.save_for_backward(qkv, buff.O, buff.LSE)
         ctx.scope_buckets, ctx.buck_size, ctx.num_heads = scope_buckets, buck_size, num_heads
@@ -58,9 +63,7 @@ class BuckSwinQKVFunction(Function):
         dO = grad_output if grad_output.dtype == torch.bfloat16 else grad_output.to(torch.bfloat16)
         # rows that no scope covers are not written: zero-filled unless the planner vouches that its table covers all
         # ... for THIS tensor: a table made for another length leaves rows out
-        covered = (getattr(ctx.scope_buckets, "covers_all_rows", False)
-                   and ctx.scope_buckets.numel() * ctx.buck_size == L)
-        dqkv = torch.empty_like(qkv) if covered else torch.zeros_like(qkv)
+        dqkv = torch.empty_like(qkv) if _covers(ctx.scope_buckets, ctx.buck_size, L) else torch.zeros_like(qkv)
         dQ, dK, dV = (t.view(B, L, H, D) for t in torch.chunk(dqkv, 3, dim=-1))
         delta = torch.zeros(B, L, H, dtype=torch.float32, device=O.device)
         pshattn.buck_swin_bwd(Q, K, V, O, dO.contiguous(), lse, delta, dQ, dK, dV, ctx.scope_buckets, ctx.buck_size)

@@ -10,12 +10,13 @@ class BuckSwinFwdBuffers:
     LSE: torch.Tensor
 
     @staticmethod
-    def create_buckswin_fwd_buff(Q: torch.Tensor):
+    def create_buckswin_fwd_buff(Q: torch.Tensor, all_rows_covered: bool = False):
         B, L, H, D = Q.shape
-        # rows outside every scope keep these values (LSE 0, O uninitialised), as in the reference;
-        # every plan of bucket_scope.py covers all rows, so the model path never reads such a row
-        return BuckSwinFwdBuffers(torch.empty(B, L, H, D, dtype=Q.dtype, device=Q.device),
-                                  torch.zeros(B, L, H, dtype=torch.float32, device=Q.device))
+        # rows outside every scope keep these values (LSE 0, O uninitialised), as in the reference.
+        # `all_rows_covered`: the caller vouches that the scope table covers every row of THIS tensor (every plan of
+        # bucket_scope.py does); the kernel then writes every LSE value and the zero fill is left out
+        lse = (torch.empty if all_rows_covered else torch.zeros)(B, L, H, dtype=torch.float32, device=Q.device)
+        return BuckSwinFwdBuffers(torch.empty(B, L, H, D, dtype=Q.dtype, device=Q.device), lse)
 
 
 @dataclass(slots=True)
