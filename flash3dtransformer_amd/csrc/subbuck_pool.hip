@@ -14,6 +14,7 @@
 // is needed.  Every output is a pure function of (coords, seps, S, seed).
 #include "f3d_device.h"
 #include "f3d_internal.h"
+#include "row_norm.h"
 
 namespace f3d {
 
@@ -365,10 +366,12 @@ __device__ __forceinline__ float red_step(float acc, float v) {
   return __fadd_rn(acc, v);
 }
 
-template <int OP>
+// NORM: the reduced row (alignment rows included, as a norm layer applied to the whole tensor would) is normalised by
+// the lanes that hold it before it is stored (row_norm.h).
+template <int OP, bool NORM>
 __global__ __launch_bounds__(256) void reduce_feat_vec8_kernel(
     const uint16_t* __restrict__ feat, const uint32_t* __restrict__ unpool_ind, uint16_t* __restrict__ reduced,
-    uint32_t total_n, uint32_t reduced_n, uint32_t reduced_aligned_n, uint32_t chunks_per_row, uint32_t S) {
+    uint32_t total_n, uint32_t reduced_n, uint32_t reduced_aligned_n, uint32_t chunks_per_row, uint32_t S, RowNorm norm) {
   const size_t gid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   const uint32_t row = (uint32_t)(gid / chunks_per_row);
   const uint32_t chunk = (uint32_t)(gid - (size_t)row * chunks_per_row);
@@ -401,7 +404,12 @@ __global__ __launch_bounds__(256) void reduce_feat_vec8_kernel(
       out.v[i] = float_to_bf16_bits(a);
     }
   }
-  *reinterpret_cast<Bf16x8*>(reduced + (size_t)row * C + chunk * 8) = out;
+  if (NORM) {
+    const u32x4_t v = row_norm_chunk(__builtin_bit_cast(u32x4_t, out), norm, chunk, chunks_per_row);
+    *reinterpret_cast<u32x4_t*>(reduced + (size_t)row * C + chunk * 8) = v;
+  } else {
+    *reinterpret_cast<Bf16x8*>(reduced + (size_t)row * C + chunk * 8) = out;
+  }
 }
 
 // any channel count: one thread per (row, channel)
@@ -432,12 +440,17 @@ __global__ __launch_bounds__(256) void reduce_feat_scalar_kernel(
 
 template <int OP>
 static void launch_reduce(const uint16_t* feat, const uint32_t* unpool_ind, uint16_t* reduced, uint32_t total_n,
-                          uint32_t reduced_n, uint32_t reduced_aligned_n, uint32_t C, uint32_t S, hipStream_t s) {
+                          uint32_t reduced_n, uint32_t reduced_aligned_n, uint32_t C, uint32_t S, const RowNorm* norm,
+                          hipStream_t s) {
   const bool vec = (C % 8 == 0) && (((uintptr_t)feat | (uintptr_t)reduced) % 16 == 0);
   if (vec) {
     const size_t total = (size_t)reduced_aligned_n * (C / 8);
-    hipLaunchKernelGGL(reduce_feat_vec8_kernel<OP>, dim3((uint32_t)((total + 255) / 256)), dim3(256), 0, s, feat,
-                       unpool_ind, reduced, total_n, reduced_n, reduced_aligned_n, C / 8, S);
+    if (norm)
+      hipLaunchKernelGGL((reduce_feat_vec8_kernel<OP, true>), dim3((uint32_t)((total + 255) / 256)), dim3(256), 0, s, feat,
+                         unpool_ind, reduced, total_n, reduced_n, reduced_aligned_n, C / 8, S, *norm);
+    else
+      hipLaunchKernelGGL((reduce_feat_vec8_kernel<OP, false>), dim3((uint32_t)((total + 255) / 256)), dim3(256), 0, s, feat,
+                         unpool_ind, reduced, total_n, reduced_n, reduced_aligned_n, C / 8, S, RowNorm{});
   } else {
     const size_t total = (size_t)reduced_aligned_n * C;
     hipLaunchKernelGGL(reduce_feat_scalar_kernel<OP>, dim3((uint32_t)((total + 255) / 256)), dim3(256), 0, s, feat,
@@ -478,9 +491,9 @@ int f3d_subbuck_build(const f3d_half_t* coord, const uint32_t* batch_sep, uint32
   return F3D_OK;
 }
 
-int f3d_reduce_feat(const f3d_bf16_t* feat, uint32_t total_n, uint32_t feat_dim, const uint32_t* unpool_ind,
-                    uint32_t reduced_n, uint32_t subbuck_size, uint32_t red_op, f3d_bf16_t* reduced_feat,
-                    uint32_t reduced_aligned_n, int device, void* stream) {
+static int reduce_feat_impl(const f3d_bf16_t* feat, uint32_t total_n, uint32_t feat_dim, const uint32_t* unpool_ind,
+                            uint32_t reduced_n, uint32_t subbuck_size, uint32_t red_op, f3d_bf16_t* reduced_feat,
+                            uint32_t reduced_aligned_n, const f3d::RowNorm* norm, int device, void* stream) {
   using namespace f3d;
   F3D_CHECK_ARG(red_op <= 3, "Unsupported reduction operation id-%u", red_op);
   F3D_CHECK_ARG(reduced_aligned_n >= reduced_n, "reduced buffer length(%u) is smaller than the reduced row count(%u)",
@@ -492,13 +505,41 @@ int f3d_reduce_feat(const f3d_bf16_t* feat, uint32_t total_n, uint32_t feat_dim,
   hipStream_t s = (hipStream_t)stream;
   SyncBracket sync(s);
   switch (red_op) {
-    case F3D_O_MEAN: launch_reduce<F3D_O_MEAN>(feat, unpool_ind, reduced_feat, total_n, reduced_n, reduced_aligned_n, feat_dim, subbuck_size, s); break;
-    case F3D_O_SUM: launch_reduce<F3D_O_SUM>(feat, unpool_ind, reduced_feat, total_n, reduced_n, reduced_aligned_n, feat_dim, subbuck_size, s); break;
-    case F3D_O_MIN: launch_reduce<F3D_O_MIN>(feat, unpool_ind, reduced_feat, total_n, reduced_n, reduced_aligned_n, feat_dim, subbuck_size, s); break;
-    default: launch_reduce<F3D_O_MAX>(feat, unpool_ind, reduced_feat, total_n, reduced_n, reduced_aligned_n, feat_dim, subbuck_size, s); break;
+    case F3D_O_MEAN: launch_reduce<F3D_O_MEAN>(feat, unpool_ind, reduced_feat, total_n, reduced_n, reduced_aligned_n, feat_dim, subbuck_size, norm, s); break;
+    case F3D_O_SUM: launch_reduce<F3D_O_SUM>(feat, unpool_ind, reduced_feat, total_n, reduced_n, reduced_aligned_n, feat_dim, subbuck_size, norm, s); break;
+    case F3D_O_MIN: launch_reduce<F3D_O_MIN>(feat, unpool_ind, reduced_feat, total_n, reduced_n, reduced_aligned_n, feat_dim, subbuck_size, norm, s); break;
+    default: launch_reduce<F3D_O_MAX>(feat, unpool_ind, reduced_feat, total_n, reduced_n, reduced_aligned_n, feat_dim, subbuck_size, norm, s); break;
   }
   F3D_CHECK_HIP(hipGetLastError());
   return F3D_OK;
+}
+
+int f3d_reduce_feat(const f3d_bf16_t* feat, uint32_t total_n, uint32_t feat_dim, const uint32_t* unpool_ind,
+                    uint32_t reduced_n, uint32_t subbuck_size, uint32_t red_op, f3d_bf16_t* reduced_feat,
+                    uint32_t reduced_aligned_n, int device, void* stream) {
+  return reduce_feat_impl(feat, total_n, feat_dim, unpool_ind, reduced_n, subbuck_size, red_op, reduced_feat,
+                          reduced_aligned_n, nullptr, device, stream);
+}
+
+int f3d_reduce_feat_norm(const f3d_bf16_t* feat, uint32_t total_n, uint32_t feat_dim, const uint32_t* unpool_ind,
+                         uint32_t reduced_n, uint32_t subbuck_size, uint32_t red_op, f3d_bf16_t* reduced_feat,
+                         uint32_t reduced_aligned_n, uint32_t norm_mode, const f3d_bf16_t* gamma, const f3d_bf16_t* beta,
+                         const float* scale, const float* shift, float eps, uint32_t act, int device, void* stream) {
+  using namespace f3d;
+  F3D_CHECK_ARG(norm_mode == kRowNormLayer || norm_mode == kRowNormAffine, "unknown row normalisation %u", norm_mode);
+  F3D_CHECK_ARG(norm_mode == kRowNormLayer ? gamma != nullptr : (scale != nullptr && shift != nullptr),
+                "null normalisation parameter");
+  F3D_CHECK_ARG(act <= F3D_ACT_RELU && act != F3D_ACT_SWIGLU && (norm_mode == kRowNormAffine || act == F3D_ACT_NONE),
+                "unsupported activation id %u for normalisation %u", act, norm_mode);
+  if (!row_norm_supported(norm_mode, feat_dim) ||
+      (((uintptr_t)feat | (uintptr_t)reduced_feat | (uintptr_t)gamma | (uintptr_t)beta | (uintptr_t)scale | (uintptr_t)shift) & 15u)) {
+    set_error("No fused normalisation for %u channels (a multiple of 8; LayerNorm: 8 x a power of two up to 512; "
+              "16-byte aligned tensors)", feat_dim);
+    return F3D_ERR_UNSUPPORTED;
+  }
+  const RowNorm norm{norm_mode, gamma, beta, scale, shift, eps, act};
+  return reduce_feat_impl(feat, total_n, feat_dim, unpool_ind, reduced_n, subbuck_size, red_op, reduced_feat,
+                          reduced_aligned_n, &norm, device, stream);
 }
 
 int f3d_batch_subbuck_reduce(const f3d_half_t* scattered_coord, const f3d_bf16_t* scattered_feat,

@@ -10,7 +10,7 @@ from ..psh import batching as f3dbatch
 from ..psh import dev_context as f3ddev
 from ..psh import subbuck as f3dsubbuck
 from . import pooling, unpool
-from .nn_ops import Linear, apply_norm_act
+from .nn_ops import Linear, apply_norm_act, fused_row_norm
 
 
 class PoolingWrapper(nn.Module):
@@ -30,8 +30,12 @@ class PoolingWrapper(nn.Module):
         if f3ddev.get_nvtx():
             nvtx.range_push(self.NVTX_SCOPE)
         projected = self.proj(input_feat)
-        reduced_feat, subbuffers = self.pooling(coords, projected, seps)
-        reduced_feat = apply_norm_act(self.norm, self.act, reduced_feat)
+        post = fused_row_norm(self.norm, self.act, projected)
+        if post is not None:     # inference: the norm (and activation) runs inside the reduce kernel
+            reduced_feat, subbuffers = self.pooling(coords, projected, seps, post=post)
+        else:
+            reduced_feat, subbuffers = self.pooling(coords, projected, seps)
+            reduced_feat = apply_norm_act(self.norm, self.act, reduced_feat)
         if f3ddev.get_nvtx():
             nvtx.range_pop()
         return reduced_feat, projected, subbuffers
@@ -62,9 +66,16 @@ class AdditiveUnpoolingWrapper(nn.Module):
     def forward(self, residual, down, buffers: f3dsubbuck.SubbuckBuffers) -> torch.Tensor:
         if f3ddev.get_nvtx():
             nvtx.range_push(self.NVTX_SCOPE)
-        proj_down = self._branch(self.proj, down)
-        proj_skip = self._branch(self.proj_skip, residual)
-        output = self.unpool(proj_skip, proj_down, buffers)
+        raw_down, raw_skip = self.proj[0](down), self.proj_skip[0](residual)
+        nd = fused_row_norm(getattr(self.proj, "norm", None), getattr(self.proj, "act", None), raw_down)
+        ns = fused_row_norm(getattr(self.proj_skip, "norm", None), getattr(self.proj_skip, "act", None), raw_skip)
+        if nd is not None and ns is not None and nd[0][0] == ns[0][0] and nd[1] == ns[1]:
+            # inference: both branches' norm (and activation) run inside the unpooling kernel
+            output = self.unpool(raw_skip, raw_down, buffers, norms=(ns[0], nd[0], nd[1]))
+        else:
+            proj_down = apply_norm_act(getattr(self.proj, "norm", None), getattr(self.proj, "act", None), raw_down)
+            proj_skip = apply_norm_act(getattr(self.proj_skip, "norm", None), getattr(self.proj_skip, "act", None), raw_skip)
+            output = self.unpool(proj_skip, proj_down, buffers)
         if f3ddev.get_nvtx():
             nvtx.range_pop()
         return output

@@ -505,6 +505,28 @@ def apply_norm_act(norm, act, x: torch.Tensor) -> torch.Tensor:
     return x
 
 
+def fused_row_norm(norm, act, x: torch.Tensor):
+    """What the pooling / unpooling kernels can apply to their rows in place of `apply_norm_act(norm, act, .)` on the
+    tensor afterwards: (descriptor, activation name) or None.  Inference only (no autograd graph), bf16 rows on the
+    GPU: a LayerNorm over the channels without activation at the widths 32 .. 512, or an eval-mode BatchNorm1d with
+    no activation / GELU / ReLU / SiLU at a multiple of 8 channels."""
+    if torch.is_grad_enabled() or norm is None or not x.is_cuda or x.dtype != torch.bfloat16:
+        return None
+    c = x.shape[-1]
+    if act is None and is_fusable_layernorm(norm, c):
+        g, b = norm_params_bf16(norm)
+        return ("layer", g, b, norm.eps), None
+    if isinstance(norm, nn.BatchNorm1d) and not norm.training and norm.track_running_stats and c % 8 == 0:
+        act_name = None
+        if act is not None:
+            act_name = _ACT_NAMES.get(type(act))
+            if act_name is None or (isinstance(act, nn.GELU) and act.approximate != "none"):
+                return None
+        scale, shift = _bn_affine(norm)
+        return ("affine", scale, shift), act_name
+    return None
+
+
 class LayerNormMLP(_CachedParamModule):
     """LayerNorm -> fc1 -> activation -> fc2, the role te.LayerNormMLP plays in the reference
     (flash3dxfmr/layers/elem_wise.py:22-26).  Parameter names follow TransformerEngine

@@ -55,7 +55,20 @@ class InbucketPoolingLayer(nn.Module):
         self.out_align = out_alignment
         self.subbuck_size = subbuck_size
 
-    def forward(self, coords, input_feat, seps):
+    def forward(self, coords, input_feat, seps, post=None):
+        """post: (descriptor, activation name) from nn_ops.fused_row_norm: the norm / activation that follows the
+        pooling is then applied by the reduce kernel itself (inference only: no autograd graph is recorded)"""
         feat = input_feat if input_feat.dtype == torch.bfloat16 else input_feat.to(torch.bfloat16)
-        return SubbuckReduceFunction.apply(coords, feat.contiguous(), seps, self.subbuck_size, self.reduction_op,
-                                           self.out_align)
+        if post is None:
+            return SubbuckReduceFunction.apply(coords, feat.contiguous(), seps, self.subbuck_size, self.reduction_op,
+                                               self.out_align)
+        feat = feat.contiguous()
+        max_n = f3dbatch.max_inslen_from_seps(seps)
+        sb = f3dsubbuck.SubbuckBuffers.create_subbuck_buff(coords, feat, seps, self.subbuck_size,
+                                                           out_alignment=self.out_align)
+        pshattn.subbuck_build(coords, seps, max_n, self.subbuck_size, NUM_VOX, sb.subbuck_id, sb.subbuck_off,
+                              sb.reduced_sep, sb.reduced_coord, sb.unpool_ind)
+        pshattn.reduce_feat_norm(feat, coords.shape[0], sb.unpool_ind, sb.reduced_feat, self.subbuck_size,
+                                 self.reduction_op, post[0], post[1])
+        sb.remove_unused_buffers()
+        return sb.reduced_feat, sb

@@ -36,6 +36,15 @@ class AdditiveUnpoolLayer(nn.Module):
         assert 1 <= subbuck_size <= 1024, f"subbuck_size must be in [1, 1024], input is {subbuck_size}"
         self.subbuck_size = subbuck_size
 
-    def forward(self, residual_feat, down_feat, buffers: SubbuckBuffers) -> torch.Tensor:
+    def forward(self, residual_feat, down_feat, buffers: SubbuckBuffers, norms=None) -> torch.Tensor:
+        """norms: (descriptor of the residual branch, descriptor of the down branch, activation name), descriptors from
+        nn_ops.fused_row_norm: the two tensors are then normalised by the unpooling kernel as it reads them (inference
+        only: no autograd graph is recorded)"""
         to = lambda t: (t if t.dtype == torch.bfloat16 else t.to(torch.bfloat16)).contiguous()
-        return AdditiveUnpoolFunction.apply(to(residual_feat), to(down_feat), buffers, self.subbuck_size)
+        if norms is None:
+            return AdditiveUnpoolFunction.apply(to(residual_feat), to(down_feat), buffers, self.subbuck_size)
+        res = to(residual_feat)
+        buf = UnpoolBuffers.create_unpool_buff(res)
+        pshattn.additive_unpool_norm_fwd(res, to(down_feat), buf.up_add_feat, buffers.unpool_ind, self.subbuck_size,
+                                         norms[0], norms[1], norms[2])
+        return buf.up_add_feat

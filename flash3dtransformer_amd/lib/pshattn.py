@@ -358,6 +358,98 @@ def additive_unpool_fwd(res_feat, down_feat, up_add_feat, unpool_ind, subbuck_si
         _u32(unpool_ind.shape[0]), _u32(res_feat.shape[1]), _u32(subbuck_size), _i32(dev), _stream(dev)))
 
 
+ROW_NORM_LAYER, ROW_NORM_AFFINE = 1, 2
+
+
+def _row_norm_args(norm, c):
+    """(mode, gamma, beta, scale, shift, eps) of one branch -> ctypes arguments; norm = ("layer", gamma16, beta16 | None,
+    eps) or ("affine", scale32, shift32)"""
+    if norm[0] == "layer":
+        _, g, b, eps = norm
+        assert_dtype([g] + ([b] if b is not None else []), torch.bfloat16)
+        if g.numel() != c or (b is not None and b.numel() != c):
+            raise RuntimeError(f"LayerNorm parameters must hold {c} values")
+        return ROW_NORM_LAYER, [_ptr(g), _ptr(b), _vp(0), _vp(0), _f32(eps)]
+    _, sc, sh = norm
+    assert_dtype([sc, sh], torch.float32)
+    if sc.numel() != c or sh.numel() != c:
+        raise RuntimeError(f"scale / shift must hold {c} values")
+    return ROW_NORM_AFFINE, [_vp(0), _vp(0), _ptr(sc), _ptr(sh), _f32(0.0)]
+
+
+def subbuck_build(scattered_coord, batch_sep, instance_max_N, subbuck_size, num_vox, subbuck_id, subbuck_off,
+                  reduced_batch_sep, reduced_coord, unpool_ind):
+    """the first half of batch_subbuck_reduce alone (local_subbuck_ker, src/psh/batch_psh_subbuck_reduce.cuh:104-298):
+    sub-bucket ids / offsets, the inverse map and the reduced coordinates"""
+    ts = [scattered_coord, batch_sep, subbuck_id, subbuck_off, reduced_batch_sep, reduced_coord, unpool_ind]
+    assert_contiguous(ts)
+    dev = assert_same_device(ts)
+    assert_dtype([scattered_coord, reduced_coord], torch.float16)
+    assert_dtype([batch_sep, subbuck_id, reduced_batch_sep, unpool_ind], torch.uint32)
+    assert_dtype([subbuck_off], torch.uint16)
+    if scattered_coord.shape[1] != 3 or reduced_coord.shape[1] != 3:
+        raise RuntimeError(f"Input coordinates dim({scattered_coord.shape[1]}) or reduced coordinates "
+                           f"dim({reduced_coord.shape[1]}) are NOT 3D.")
+    if unpool_ind.shape[1] != subbuck_size:
+        raise RuntimeError(f"Unpool_ind last dimension({unpool_ind.shape[1]}) != subbucket_size({subbuck_size})")
+    _check(_load().f3d_subbuck_build(
+        _ptr(scattered_coord), _ptr(batch_sep), _u32(batch_sep.shape[0]), _u32(scattered_coord.shape[0]),
+        _u32(instance_max_N), _u32(subbuck_size), _u32(num_vox), _ptr(subbuck_id), _ptr(subbuck_off),
+        _ptr(reduced_batch_sep), _ptr(reduced_coord), _u32(reduced_coord.shape[0]), _ptr(unpool_ind),
+        _u32(unpool_ind.shape[0]), _i32(dev), _stream(dev)))
+
+
+def reduce_feat_norm(feat, total_n, unpool_ind, reduced_feat, subbuck_size, red_op, norm, act=None):
+    """extension: the feature reduce of batch_subbuck_reduce (reduce_feat_ker, src/psh/batch_psh_subbuck_reduce.cuh:300-359)
+    with the pooling wrapper's norm (and activation) applied to every reduced row before it is stored; total_n = number of
+    points (rows of feat beyond it are ignored).  norm = ("layer", gamma bf16, beta bf16 | None, eps) or
+    ("affine", scale fp32, shift fp32)"""
+    if total_n > feat.shape[0]:
+        raise RuntimeError(f"feat has {feat.shape[0]} rows, total_n is {total_n}")
+    assert_contiguous([feat, unpool_ind, reduced_feat])
+    dev = assert_same_device([feat, unpool_ind, reduced_feat])
+    assert_dtype([feat, reduced_feat], torch.bfloat16)
+    assert_dtype([unpool_ind], torch.uint32)
+    if feat.shape[1] != reduced_feat.shape[1]:
+        raise RuntimeError(f"Input feature dim({feat.shape[1]}) != output feature dim({reduced_feat.shape[1]}).")
+    if unpool_ind.shape[1] != subbuck_size:
+        raise RuntimeError(f"Unpool_ind last dimension({unpool_ind.shape[1]}) != subbucket_size({subbuck_size})")
+    mode, nargs = _row_norm_args(norm, feat.shape[1])
+    a = ACT[act] if not isinstance(act, int) else act
+    _check(_load().f3d_reduce_feat_norm(
+        _ptr(feat), _u32(total_n), _u32(feat.shape[1]), _ptr(unpool_ind), _u32(unpool_ind.shape[0]), _u32(subbuck_size),
+        _u32(red_op), _ptr(reduced_feat), _u32(reduced_feat.shape[0]), _u32(mode), *nargs, _u32(a), _i32(dev),
+        _stream(dev)))
+
+
+def additive_unpool_norm_fwd(res_feat, down_feat, up_add_feat, unpool_ind, subbuck_size, norm_res, norm_down, act=None):
+    """extension: additive_unpool_fwd with both operands normalised on the way in (the unpooling wrapper's
+    Linear -> norm -> activation branches, flash3dxfmr/layers/hourglass.py:152-159); norm_* as in reduce_feat_norm,
+    both of the same kind"""
+    ts = [res_feat, down_feat, up_add_feat, unpool_ind]
+    assert_contiguous(ts)
+    dev = assert_same_device(ts)
+    assert_dtype([res_feat, down_feat, up_add_feat], torch.bfloat16)
+    assert_dtype([unpool_ind], torch.uint32)
+    if res_feat.shape != up_add_feat.shape:
+        raise RuntimeError(f"res_feat shape {tuple(res_feat.shape)} != up_add_feat shape {tuple(up_add_feat.shape)}")
+    if res_feat.shape[1] != down_feat.shape[1]:
+        raise RuntimeError(f"Feature dim mismatch: res({res_feat.shape[1]}) vs down({down_feat.shape[1]})")
+    if unpool_ind.shape[1] != subbuck_size:
+        raise RuntimeError(f"Unpool_ind last dimension({unpool_ind.shape[1]}) != subbucket_size({subbuck_size})")
+    if down_feat.shape[0] < unpool_ind.shape[0]:
+        raise RuntimeError(f"down_feat has {down_feat.shape[0]} rows, unpool_ind needs {unpool_ind.shape[0]}")
+    if norm_res[0] != norm_down[0]:
+        raise RuntimeError("both branches must use the same kind of normalisation")
+    mode, ra = _row_norm_args(norm_res, res_feat.shape[1])
+    _, da = _row_norm_args(norm_down, res_feat.shape[1])
+    a = ACT[act] if not isinstance(act, int) else act
+    _check(_load().f3d_additive_unpool_norm_fwd(
+        _ptr(res_feat), _ptr(down_feat), _ptr(up_add_feat), _ptr(unpool_ind), _u32(res_feat.shape[0]),
+        _u32(unpool_ind.shape[0]), _u32(res_feat.shape[1]), _u32(subbuck_size), _u32(mode), *ra, *da, _u32(a), _i32(dev),
+        _stream(dev)))
+
+
 def additive_unpool_bwd(grad_res, grad_down, grad_up_added, unpool_ind, subbuck_size):
     """src/f3d_frontend.cu:103-105 -> src/psh/additive_unpool_dispatcher.cu:81-134: grad_res[r] = grad_up_added[r]
     for every pooled point r, grad_down[i] = sum over the points pooled into row i.  Rows of grad_res that no slot

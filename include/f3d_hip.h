@@ -152,12 +152,34 @@ int f3d_reduce_feat(const f3d_bf16_t* feat, uint32_t total_n, uint32_t feat_dim,
                     uint32_t reduced_n, uint32_t subbuck_size, uint32_t red_op, f3d_bf16_t* reduced_feat,
                     uint32_t reduced_aligned_n, int device, void* stream);
 
+/* The feature reduce with the layer that follows it in the reference's pooling wrapper applied to every reduced row
+ * before it is stored (flash3dxfmr/layers/hourglass.py:104-109: pooling -> norm -> activation), alignment rows
+ * included, as the layer applied to the whole tensor would.  norm_mode 1: LayerNorm (gamma, beta bf16 [feat_dim], beta
+ * may be NULL; eps; act must be F3D_ACT_NONE); norm_mode 2: act(x * scale + shift) with fp32 scale / shift [feat_dim] (an
+ * eval-mode BatchNorm1d folded) and act in {NONE, GELU, SILU, RELU}.  feat_dim a multiple of 8 (LayerNorm: 8 times a
+ * power of two, at most 512), all tensors 16-byte aligned; F3D_ERR_UNSUPPORTED otherwise. */
+int f3d_reduce_feat_norm(const f3d_bf16_t* feat, uint32_t total_n, uint32_t feat_dim, const uint32_t* unpool_ind,
+                         uint32_t reduced_n, uint32_t subbuck_size, uint32_t red_op, f3d_bf16_t* reduced_feat,
+                         uint32_t reduced_aligned_n, uint32_t norm_mode, const f3d_bf16_t* gamma, const f3d_bf16_t* beta,
+                         const float* scale, const float* shift, float eps, uint32_t act, int device, void* stream);
+
 /* ---- additive unpool: additive_unpool_fwd, src/f3d_frontend.cu:99-101,
  *      src/psh/additive_unpool_dispatcher.cu:26-79 ----------------------------------------------
  * up[r,:] = bf16(float(down[i,:]) + float(res[r,:])) for r = unpool_ind[i,s] < up_n. */
 int f3d_additive_unpool_fwd(const f3d_bf16_t* res_feat, const f3d_bf16_t* down_feat, f3d_bf16_t* up_add_feat,
                             const uint32_t* unpool_ind, uint32_t up_n, uint32_t down_n, uint32_t feat_dim,
                             uint32_t subbuck_size, int device, void* stream);
+
+/* The same with both operands normalised on the way in: up[r,:] = bf16(norm_down(down[i,:]) + norm_res(res[r,:])), where
+ * the reference's unpooling wrapper runs Linear -> norm -> activation on each branch before the op
+ * (flash3dxfmr/layers/hourglass.py:152-159).  Modes, parameters and limits as for f3d_reduce_feat_norm; one mode and one
+ * activation for both branches, parameters per branch. */
+int f3d_additive_unpool_norm_fwd(const f3d_bf16_t* res_feat, const f3d_bf16_t* down_feat, f3d_bf16_t* up_add_feat,
+                                 const uint32_t* unpool_ind, uint32_t up_n, uint32_t down_n, uint32_t feat_dim,
+                                 uint32_t subbuck_size, uint32_t norm_mode, const f3d_bf16_t* res_gamma,
+                                 const f3d_bf16_t* res_beta, const float* res_scale, const float* res_shift, float res_eps,
+                                 const f3d_bf16_t* down_gamma, const f3d_bf16_t* down_beta, const float* down_scale,
+                                 const float* down_shift, float down_eps, uint32_t act, int device, void* stream);
 
 /* ---- PSH permutation index and feature scatter: completes batch_psh_cumsum_scatter_feat_index_postpad_ker,
  *      src/psh/batch_psh_bucket.cuh:617-753 (unfinished in the reference: it writes the index, :735, and the pad

@@ -235,3 +235,137 @@ def test_pool_unpool_layers_backpropagate(oracle):
     g_feat = oracle.reduce_feat_bwd(g_down, n_bf16_bits(feat.detach()), unpool, 0)
     assert np.array_equal(n_bf16_bits(res.grad), g_res)
     assert np.array_equal(n_bf16_bits(feat.grad), g_feat)
+
+
+def _bf16_to_f32(bits):
+    return (bits.astype(np.uint32) << 16).view(np.float32)
+
+
+def _norm_reference(x_bits, kind, params, act):
+    """fp64 restatement of the two layers: LayerNorm over the channels, or act(bf16(x * scale + shift))"""
+    x = _bf16_to_f32(x_bits).astype(np.float64)
+    if kind == "layer":
+        g, b, eps = params
+        mu = x.mean(1, keepdims=True)
+        var = ((x - mu) ** 2).mean(1, keepdims=True)
+        return (x - mu) / np.sqrt(var + eps) * g + b
+    scale, shift = params
+    y = x * scale + shift
+    y = _bf16_to_f32(bf16_bits(y.astype(np.float32))).astype(np.float64)     # the norm's output is a bf16 tensor
+    if act == "gelu":
+        from math import erf
+        y = 0.5 * y * (1.0 + np.vectorize(erf)(y / np.sqrt(2.0)))
+    elif act == "relu":
+        y = np.maximum(y, 0.0)
+    elif act == "silu":
+        y = y / (1.0 + np.exp(-y))
+    return y
+
+
+def _norm_case(kind, C, rng):
+    """(descriptor for pshattn, parameters for _norm_reference)"""
+    if kind == "layer":
+        g = _bf16_to_f32(bf16_bits(rng.uniform(0.5, 1.5, C).astype(np.float32)))
+        b = _bf16_to_f32(bf16_bits(rng.normal(0, 0.3, C).astype(np.float32)))
+        desc = ("layer", t_bf16_bits(bf16_bits(g)), t_bf16_bits(bf16_bits(b)), 1e-5)
+        return desc, (g.astype(np.float64), b.astype(np.float64), 1e-5)
+    scale = rng.uniform(0.5, 1.5, C).astype(np.float32)
+    shift = rng.normal(0, 0.3, C).astype(np.float32)
+    desc = ("affine", torch.from_numpy(scale).to(DEV), torch.from_numpy(shift).to(DEV))
+    return desc, (scale.astype(np.float64), shift.astype(np.float64))
+
+
+@pytest.mark.parametrize("S,op,sizes,C,kind,act", [
+    (2, 0, [1300, 1024, 2051, 7], 32, "layer", None),
+    (2, 0, [3000, 2999], 64, "layer", None),
+    (8, 3, [4096, 100], 128, "layer", None),
+    (2, 0, [2500], 256, "layer", None),
+    (4, 0, [1500, 3], 512, "layer", None),
+    (2, 0, [1300, 1024], 64, "affine", "gelu"),
+    (2, 1, [2000, 7], 40, "affine", None),          # 40 channels: 5 lanes per row
+    (8, 2, [4100], 256, "affine", "relu"),
+    (2, 0, [999], 32, "affine", "silu"),
+])
+def test_reduce_with_fused_norm(oracle, S, op, sizes, C, kind, act):
+    """subbuck_build + reduce_feat_norm against the oracle's reduce followed by the norm in fp64 (a bf16 rounding of
+    slack), and against the library's own two kernels (reduce, then LayerNorm / affine + activation): at most one bf16
+    step apart"""
+    from flash3dtransformer_amd.lib import pshattn
+    from flash3dtransformer_amd.psh import subbuck
+    rng = np.random.default_rng(S * 100 + op + C)
+    coords = rng.uniform(-30, 30, (sum(sizes), 3)).astype(np.float16)
+    seps = np.cumsum(sizes).astype(np.uint32)
+    feat = bf16_bits(rng.normal(0.3, 1.0, (sum(sizes), C)))
+    desc, ref_params = _norm_case(kind, C, rng)
+    plain = _pool(coords, seps, feat, S, op, 16, oracle)          # builder + plain reduce
+    c, s, f = t_f16(coords), t_u32(seps), t_bf16_bits(feat)
+    sb = subbuck.SubbuckBuffers.create_subbuck_buff(c, f, s, S, out_alignment=16)
+    max_n = int(np.diff(np.concatenate([[0], seps.astype(np.int64)])).max())
+    pshattn.subbuck_build(c, s, max_n, S, 0xFFFF, sb.subbuck_id, sb.subbuck_off, sb.reduced_sep, sb.reduced_coord, sb.unpool_ind)
+    pshattn.reduce_feat_norm(f, coords.shape[0], sb.unpool_ind, sb.reduced_feat, S, op, desc, act)
+    torch.cuda.synchronize()
+    assert np.array_equal(n_u32(sb.unpool_ind), n_u32(plain.unpool_ind))
+    assert np.array_equal(n_f16(sb.reduced_coord).view(np.uint16), n_f16(plain.reduced_coord).view(np.uint16))
+    got = _bf16_to_f32(n_bf16_bits(sb.reduced_feat)).astype(np.float64)
+    want = _norm_reference(n_bf16_bits(plain.reduced_feat), kind, ref_params, act)       # alignment rows included
+    assert got.shape == want.shape
+    assert np.all(np.abs(got - want) <= 2.0 ** -8 * np.abs(want) + 1e-6), np.abs(got - want).max()
+    # the two-kernel path of the library
+    two = torch.empty_like(plain.reduced_feat)
+    if kind == "layer":
+        pshattn.layernorm_bf16(plain.reduced_feat, desc[1], desc[2], two, 1e-5)
+    else:
+        pshattn.affine_act_bf16(plain.reduced_feat, desc[1], desc[2], two, act)
+    torch.cuda.synchronize()
+    two = _bf16_to_f32(n_bf16_bits(two)).astype(np.float64)
+    assert np.all(np.abs(got - two) <= 2.0 ** -7 * np.abs(two) + 1e-6), np.abs(got - two).max()
+
+
+@pytest.mark.parametrize("S,C,kind,act", [(2, 64, "layer", None), (2, 32, "layer", None), (8, 256, "layer", None),
+                                          (3, 128, "layer", None), (2, 64, "affine", "gelu"), (3, 24, "affine", None),
+                                          (2, 512, "affine", "relu")])
+def test_unpool_with_fused_norm(oracle, S, C, kind, act):
+    """up[r] = norm_down(down[i]) + norm_res(res[r]) for r = unpool_ind[i, s]; rows that no slot references keep the
+    caller's prefill"""
+    from flash3dtransformer_amd.lib import pshattn
+    rng = np.random.default_rng(S + C + len(kind))
+    n = 1501
+    r = -(-n // S)
+    unpool = np.full((r, S), n + 3, dtype=np.uint32)
+    keep = rng.permutation(n)[: n - 20]                        # 20 rows are referred to by no slot
+    unpool.reshape(-1)[: keep.size] = keep
+    res, down = bf16_bits(rng.normal(0.2, 1, (n, C))), bf16_bits(rng.normal(-0.1, 1, (r + 2, C)))
+    dr, pr = _norm_case(kind, C, rng)
+    dd, pd = _norm_case(kind, C, rng)
+    up = torch.full((n, C), 7.0, dtype=torch.bfloat16, device=DEV)
+    pshattn.additive_unpool_norm_fwd(t_bf16_bits(res), t_bf16_bits(down), up, t_u32(unpool), S, dr, dd, act)
+    torch.cuda.synchronize()
+    got = _bf16_to_f32(n_bf16_bits(up)).astype(np.float64)
+    nres = _bf16_to_f32(bf16_bits(_norm_reference(res, kind, pr, act).astype(np.float32))).astype(np.float64)
+    ndown = _bf16_to_f32(bf16_bits(_norm_reference(down, kind, pd, act).astype(np.float32))).astype(np.float64)
+    want = np.full((n, C), 7.0)
+    for i in range(r):
+        for s in range(S):
+            t = unpool[i, s]
+            if t < n:
+                want[t] = nres[t] + ndown[i]
+    # each operand may be one bf16 step off its fp64 value, and the sum is rounded once more
+    tol = 2.0 ** -7 * (np.abs(nres) + np.abs(ndown[0:1]).max() + np.abs(want)) + 1e-6
+    assert np.all(np.abs(got - want) <= tol), np.abs(got - want).max()
+    untouched = np.setdiff1d(np.arange(n), keep)
+    assert np.all(got[untouched] == 7.0)
+
+
+def test_fused_norm_argument_errors():
+    from flash3dtransformer_amd.lib import pshattn
+    C = 24          # LayerNorm over 3 lanes per row is not covered
+    feat = torch.zeros(64, C, dtype=torch.bfloat16, device=DEV)
+    ind = torch.zeros(32, 2, dtype=torch.int32, device=DEV).view(torch.uint32)
+    out = torch.zeros(32, C, dtype=torch.bfloat16, device=DEV)
+    g = torch.ones(C, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(RuntimeError, match="No fused normalisation"):
+        pshattn.reduce_feat_norm(feat, 64, ind, out, 2, 0, ("layer", g, None, 1e-5))
+    with pytest.raises(RuntimeError, match="unsupported activation"):
+        pshattn.reduce_feat_norm(torch.zeros(64, 32, dtype=torch.bfloat16, device=DEV), 64, ind,
+                                 torch.zeros(32, 32, dtype=torch.bfloat16, device=DEV), 2, 0,
+                                 ("layer", torch.ones(32, dtype=torch.bfloat16, device=DEV), None, 1e-5), "gelu")
