@@ -273,7 +273,7 @@ def sub_metrics(dev, only=None):
     unpooling GB/s on config 3 — each against its roofline.  `only`: a set of group names, or None for all"""
     out = {}
     groups = {"attention": sub_attention, "psh": sub_psh, "permute": sub_permute, "pool": sub_pool,
-              "hourglass": sub_hourglass, "mfma": sub_mfma_rate, "stores": sub_store_rows,
+              "hourglass": sub_hourglass, "mfma": sub_mfma_rate, "issue": sub_issue, "stores": sub_store_rows,
               "backward": sub_backward}
     for name, fn in groups.items():
         if only is None or name in only:
@@ -289,6 +289,46 @@ def _bench_probe():
     if not os.path.exists(path):
         raise RuntimeError(f"{path} is missing: run `python __graft_entry__.py` first")
     return ctypes.CDLL(path)
+
+
+def issue_probe(dev, mode, iters=20000):
+    """shader clocks a SIMD spends per loop trip of bench_probe_issue's mode with four waves on it, and the shader clock
+    it ran at.  The SIMD's arbiter serves its oldest wave first, so the four waves of a SIMD finish one after the other:
+    the last one's elapsed clocks are the time of all four (4 x trips)."""
+    import ctypes
+    lib = _bench_probe()
+    n_cu = torch.cuda.get_device_properties(0).multi_processor_count
+    sink = torch.zeros(1, dtype=torch.float32, device=dev)
+    clocks = torch.zeros(n_cu * 16, 2, dtype=torch.int64, device=dev)
+    for _ in range(2):
+        rc = lib.bench_probe_issue(ctypes.c_uint32(mode), ctypes.c_uint32(n_cu), ctypes.c_uint32(iters),
+                                   ctypes.c_void_p(sink.data_ptr()), ctypes.c_void_p(clocks.data_ptr()),
+                                   ctypes.c_void_p(torch.cuda.current_stream(0).cuda_stream))
+        if rc != 0:
+            raise RuntimeError(f"bench_probe_issue failed with {rc}")
+    torch.cuda.synchronize()
+    ck = clocks.double().cpu().view(n_cu, 4, 4, 2)          # workgroup, wave / 4, SIMD (wave % 4), counter
+    last = ck[..., 0].max(dim=1).values                     # the last wave of each SIMD
+    ghz = (ck[..., 0] / (ck[..., 1] / 100e6) / 1e9).median().item()
+    return last.median().item() / (4.0 * iters), ghz
+
+
+def sub_issue(dev, out):
+    """What the vector issue port of a SIMD takes for the instructions of the attention forward's inner step (one
+    32 x 32 block of scores at 32-wide heads: 16 v_exp_f32, 8 v_cvt_pk_bf16_f32, four 32x32x16 and two 16x16x32 bf16
+    MFMAs), each kind alone and all together with the step's dependencies, on register operands with four waves per
+    SIMD and no memory instruction: the floor the attention kernels are priced against (`valu_issue_bound_ms`)."""
+    exp_clk, ghz0 = issue_probe(dev, 0)
+    cvt_clk, ghz1 = issue_probe(dev, 1)
+    mm_clk, ghz2 = issue_probe(dev, 2)
+    mix_clk, ghz3 = issue_probe(dev, 3)
+    out["issue_port_probe"] = {"v_exp_f32_clocks": round(exp_clk / 16, 2),
+                               "v_cvt_pk_bf16_f32_clocks": round(cvt_clk / 8, 2),
+                               "six_mfma_of_a_block_clocks": round(mm_clk, 1),
+                               "attention_block_mix_clocks": round(mix_clk, 1),
+                               "matrix_core_clocks_per_block": 4 * 32 + 2 * 16,
+                               "shader_clock_ghz": {"exp": round(ghz0, 3), "cvt": round(ghz1, 3), "mfma": round(ghz2, 3),
+                                                    "mix": round(ghz3, 3)}}
 
 
 def sub_hourglass(dev, out):
@@ -459,16 +499,19 @@ def sub_attention(dev, out):
     sc = torch.arange(L // BS, dtype=torch.int32, device=dev).view(-1, 1).view(torch.uint32)
     med, mn, mean = ev_stats(lambda: pshattn.buck_swin_fwd(q, k, v, o, lse, sc, BS))
     fl = 4.0 * L * BS * H * D
-    # What the vector issue port allows: per 32 x 32 block of scores a wave issues 16 v_exp_f32 (8 clocks each at full
-    # occupancy), 8 v_cvt_pk_bf16_f32 (4.3) and 6 MFMAs (about 10 clocks of the port each): 222 clocks per block, on
-    # 1024 SIMDs at 2.4 GHz; next to it the matrix-core and HBM minimum times
+    # What the vector issue port allows: per 32 x 32 block of scores a wave issues 16 v_exp_f32, 8 v_cvt_pk_bf16_f32 and
+    # 6 MFMAs; bench_probe_issue runs exactly that mix with the step's dependencies on register operands (no LDS, no
+    # memory) with four waves per SIMD, and its clocks per block at its own shader clock are the floor, next to the
+    # matrix-core and HBM minimum times
     blocks = (L / 32) * (BS / 32) * H
-    port_clk = 16 * 8.0 + 8 * 4.3 + 6 * 10.0
+    port_clk, port_ghz = issue_probe(dev, 3)
     out["attention_c2_unmasked"] = {"ms": round(med, 4), "ms_min": round(mn, 4), "ms_mean": round(mean, 4), "launches_timed": 200,
                                     "tflops": round(fl / med / 1e9, 2),
                                     "frac_of_bf16_mfma_peak": round(fl / med / 1e9 / MFMA_BF16_PEAK_TFLOPS, 4),
                                     "algorithmic_gflop": round(fl / 1e9, 2),
-                                    "valu_issue_bound_ms": round(blocks * port_clk / 1024 / 2.4e9 * 1e3, 4),
+                                    "valu_issue_bound_ms": round(blocks * port_clk / 1024 / (port_ghz * 1e9) * 1e3, 4),
+                                    "issue_probe_clocks_per_block": round(port_clk, 1),
+                                    "issue_probe_shader_clock_ghz": round(port_ghz, 3),
                                     "mfma_bound_ms": round(fl / (MFMA_BF16_PEAK_TFLOPS * 1e12) * 1e3, 4),
                                     "hbm_bound_ms": round((2.0 * L * 4 * H * D + 4.0 * L * H) / (HBM_PEAK_GBS * 1e9) * 1e3, 4)}
     kl = torch.from_numpy(np.random.default_rng(1002).integers(384, 513, L // BS).astype(np.int32)).to(dev)

@@ -427,8 +427,8 @@ __device__ __forceinline__ void lds_dma16_at(const void* gbase, uint32_t voff, u
 // which some are partly valid take the general pass.
 //
 // What bounds the pass is the vector unit's issue port: per 32 x 32 scores a wave issues 16 v_exp_f32 (two slots
-// each), 8 v_cvt_pk_bf16_f32 and six MFMAs (each holds the port for about ten clocks), some 240 clocks against
-// 160 clocks of matrix-core time.  Hence: the scores of the next (step, block) are issued before the
+// each), 8 v_cvt_pk_bf16_f32 and six MFMAs (each holds the port for about nine clocks): 228 clocks measured for
+// that mix alone against 160 clocks of matrix-core time.  Hence: the scores of the next (step, block) are issued before the
 // exponentials of the current one, so that the matrix core works under them; the row sums come from the matrix
 // core too (one 16x16x32 product of P with a 0 / 1 selector per 16 keys, a quarter of a score product, instead
 // of eight dot instructions on the vector unit); the steps are fully unrolled (LDS offsets are immediates, no
