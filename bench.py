@@ -29,7 +29,7 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 # size, see profiles/encoder_stage_4x120k_hbm_traffic.md) at this bench's shapes
 TRAFFIC_FROM = "profiles/encoder_stage_4x120k_hbm_traffic.md (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this bench's step; re-measure when a kernel changes)"
 TRAFFIC_BYTES_PER_LAUNCH = {"ln_fc1_act": 1.613e9, "ln_qkv": 1.022e9, "attention": 1.019e9,
-                            "proj_residual": 0.763e9, "fc2_residual": 1.847e9, "ln_mlp_residual": 0.849e9}
+                            "proj_residual": 0.767e9, "fc2_residual": 1.851e9, "ln_mlp_residual": 0.849e9}
 
 
 def ev_time(fn, iters, warmup=3):
@@ -180,33 +180,42 @@ def main():
             "coord_embed": lambda: pshattn.coord_embed_bf16(scat, We, Be, emb_out),
             "ln_qkv": lambda: pshattn.ln_linear_bf16(feat, Wn, Bn, 1e-5, Wq, Bq, None, qkv, None),
             "attention": lambda: pshattn.buck_swin_fwd(q, k, v, o, lse, scopes, BS),
-            "proj_residual": lambda: pshattn.linear_bf16(o.view(n_pad, C), Wp, Bp, feat, mid, None),
         }
-        # the gated MLP runs as one kernel at this size (the layer's choice); with gelu, LayerNorm+fc1+act then fc2
+        # the out-projection with its residual and the gated MLP with its residual run as one kernel at this size (the
+        # block's choice at inference); with gelu: the projection, LayerNorm+fc1+act, then fc2
+        separate = {"proj_residual": lambda: pshattn.linear_bf16(o.view(n_pad, C), Wp, Bp, feat, mid, None),
+                    "ln_mlp_residual": lambda: pshattn.ln_mlp_swiglu_bf16(mid, Wm, Bm, 1e-5, W1, B1, W2, B2, mid, y)}
         two_kernel = {"ln_fc1_act": lambda: pshattn.ln_linear_bf16(mid, Wm, Bm, 1e-5, W1, B1, None, hid, args.mlp),
                       "fc2_residual": lambda: pshattn.linear_bf16(hid, W2, B2, mid, y, None)}
         if args.mlp == "swiglu":
-            ops["ln_mlp_residual"] = lambda: pshattn.ln_mlp_swiglu_bf16(mid, Wm, Bm, 1e-5, W1, B1, W2, B2, mid, y)
+            ops["proj_ln_mlp_residual"] = lambda: pshattn.proj_ln_mlp_swiglu_bf16(o.view(n_pad, C), Wp, Bp, feat, Wm, Bm, 1e-5,
+                                                                                  W1, B1, W2, B2, y)
         else:
+            ops["proj_residual"] = separate["proj_residual"]
             ops.update(two_kernel)
         breakdown = {name: ev_time(fn, 20) for name, fn in ops.items()}
         two_kernel_ms = {name: ev_time(fn, 20) for name, fn in two_kernel.items()}
+        separate_ms = {name: ev_time(fn, 20) for name, fn in separate.items()} if args.mlp == "swiglu" else {}
     fc1_n = 2 * HID if args.mlp == "swiglu" else HID
     flops = {"ln_qkv": 2.0 * n_pad * C * 3 * C, "proj_residual": 2.0 * n_pad * C * C,
              "ln_fc1_act": 2.0 * n_pad * C * fc1_n, "fc2_residual": 2.0 * n_pad * HID * C,
              "ln_mlp_residual": 2.0 * n_pad * C * fc1_n + 2.0 * n_pad * HID * C,
+             "proj_ln_mlp_residual": 2.0 * n_pad * C * C + 2.0 * n_pad * C * fc1_n + 2.0 * n_pad * HID * C,
              "attention": 4.0 * n_pad * BS * SCOPE * C}
     # algorithmic HBM bytes per launch (bf16 activations in and out, weights negligible)
     hbm_bytes = {"ln_qkv": 2.0 * n_pad * (C + 3 * C), "proj_residual": 2.0 * n_pad * 3 * C,
                  "ln_fc1_act": 2.0 * n_pad * (C + HID), "fc2_residual": 2.0 * n_pad * (HID + 2 * C),
                  "ln_mlp_residual": 2.0 * n_pad * 2 * C,      # x (also the residual) in, y out
+                 "proj_ln_mlp_residual": 2.0 * n_pad * 3 * C,  # attention output and block input in, y out
                  "attention": 2.0 * n_pad * 4 * C + 4.0 * n_pad * H}
     kernels = {"attention": "buck_swin_fwd_scope_kernel<32,512,16>",
                "ln_qkv": "xstat_linear_kernel<256,2,8,3,LN> + ln_fold_kernel",
                "ln_fc1_act": "xstat_linear_kernel<256,2,8,3,LN,swiglu> + ln_fold_kernel",
                "proj_residual": "xstat_linear_kernel<256,2,8,3,residual>",
                "fc2_residual": "ystat_linear_kernel<256> + ys_w_prep_kernel",
-               "ln_mlp_residual": "ln_mlp_swiglu_kernel<256> + mlp_prep_kernel"}
+               "ln_mlp_residual": "ln_mlp_swiglu_kernel<256, false> + mlp_prep_kernel",
+               "proj_ln_mlp_residual": "ln_mlp_swiglu_kernel<256, true> + mlp_prep_kernel"}
+    all_flops = dict(flops)
     flops = {kname: vv for kname, vv in flops.items() if kname in breakdown}
     # the two-kernel form of the MLP (what the layer runs below 60 k rows, or with fused=False), same tensors
     two_kernel_mlp = None
@@ -214,9 +223,16 @@ def main():
         ms_2 = two_kernel_ms["ln_fc1_act"] + two_kernel_ms["fc2_residual"]
         two_kernel_mlp = {"kernels": kernels["ln_fc1_act"] + " ; " + kernels["fc2_residual"],
                           "ms": {kname: round(vv, 4) for kname, vv in two_kernel_ms.items()},
-                          "tflops": round(flops["ln_mlp_residual"] / ms_2 / 1e9, 1),
+                          "tflops": round(all_flops["ln_mlp_residual"] / ms_2 / 1e9, 1),
                           "traffic": TRAFFIC_BYTES_PER_LAUNCH["ln_fc1_act"] + TRAFFIC_BYTES_PER_LAUNCH["fc2_residual"],
                           "hidden_activation_bytes": int(n_pad) * HID * 2}
+    # the out-projection and the one-kernel MLP as two launches (what the block runs under autograd), same tensors
+    separate_proj_mlp = None
+    if separate_ms:
+        separate_proj_mlp = {"kernels": kernels["proj_residual"] + " ; " + kernels["ln_mlp_residual"],
+                             "ms": {kname: round(vv, 4) for kname, vv in separate_ms.items()},
+                             "ln_mlp_tflops": round(all_flops["ln_mlp_residual"] / separate_ms["ln_mlp_residual"] / 1e9, 1),
+                             "x1_bytes_written_and_read_again": int(n_pad) * C * 2 * 3}
     dominant = max(flops, key=lambda kname: breakdown[kname])
     t_dom = breakdown[dominant] * 1e-3
     ach = flops[dominant] / t_dom / 1e12
@@ -253,6 +269,7 @@ def main():
         "roofline": roofline,
         "breakdown_ms": {kname: round(vv, 4) for kname, vv in breakdown.items()},
         "per_op": per_op,
+        "separate_proj_and_mlp_under_autograd": separate_proj_mlp,
         "two_kernel_mlp_on_request": two_kernel_mlp,
         "sub_metrics": sub,
     }

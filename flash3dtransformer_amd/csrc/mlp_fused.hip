@@ -38,6 +38,16 @@
 
 namespace f3d {
 
+// f(std::integral_constant<uint32_t, 0>) ... f(std::integral_constant<uint32_t, N - 1>): a loop whose counter is a
+// constant expression inside the body (statically indexed register arrays)
+template <uint32_t N, uint32_t I = 0, class F>
+__device__ __forceinline__ void mlp_static_for(F&& f) {
+  if constexpr (I < N) {
+    f(std::integral_constant<uint32_t, I>{});
+    mlp_static_for<N, I + 1>(f);
+  }
+}
+
 constexpr int kMlpWaves = 8, kMlpBufs = 2;   // chunk c + 1 is requested when chunk c starts
 constexpr int kMlpFragsAhead = 2;            // LDS fragment reads in flight ahead of their products
 
@@ -48,23 +58,39 @@ struct MlpGeom {
   static constexpr int CH1 = G::CHUNK_BYTES;                // w1 chunk: 64 rows
   static constexpr int CH2 = K * 32 * 2;                    // w2 chunk: K outputs x 32 hidden
   static constexpr int N_DMA2 = CH2 / 1024;
-  // weight buffers and the b' slots of the w1 buffers; at least the prologue's transposition patches
-  static constexpr size_t lds_bytes() {
-    const size_t loop = (size_t)kMlpBufs * (CH1 + 1024 + CH2);
+  static constexpr int NPC = K / kXsChunk;                  // 64-row chunks of the out-projection weight
+  static constexpr size_t loop_bytes() { return (size_t)kMlpBufs * (CH1 + 1024 + CH2); }
+  static constexpr size_t row_patch_bytes() { return (size_t)kMlpWaves * 32 * kPatchRow * 2; }
+  // weight buffers and the b' slots of the w1 buffers; at least the prologue's transposition patches; with the
+  // out-projection in front, the wave-private patches its result is re-laid through come after the weight buffers
+  static constexpr size_t lds_bytes(bool proj = false) {
+    const size_t loop = loop_bytes();
     const size_t patches = (size_t)kMlpWaves * 32 * (G::KP + 8) * 2;
-    return loop > patches ? loop : patches;
+    return proj ? loop + row_patch_bytes() : (loop > patches ? loop : patches);
   }
+};
+
+// The out-projection in front of the MLP (PROJ kernels): a [M][K] are the attention output rows, w [K][K] / b [K] the
+// projection's weight and bias; the kernel's x is then the block input that the projection's result is added to.
+struct MlpProj {
+  const uint16_t* a;
+  uint32_t lda;
+  const uint16_t* w;
+  const uint16_t* b;
 };
 
 // w1p: LayerNorm-folded fc1 weight [2 H][K] (value rows then gate rows), b32: b' = b1 + w1 beta as fp32 [2 H] (mlp_prep_kernel);
 // w2p: fc2 weight, fragment-major per chunk (mlp_prep_kernel); bias2 [K] (zeros when the layer has none);
 // H: hidden width, multiple of 32.
-template <int K>
+// PROJ: x1 = bf16(bf16(a wpT + bp) + x) is formed first (the block's out-projection with its residual, held in
+// registers only), and the kernel returns bf16(x1 + MLP(x1)): `residual` must be null, the fc2 accumulators start from
+// x1 + b2.
+template <int K, bool PROJ>
 __global__ __launch_bounds__(64 * kMlpWaves) __attribute__((amdgpu_waves_per_eu(2, 2))) void ln_mlp_swiglu_kernel(
     const uint16_t* __restrict__ x, uint32_t ldx, float eps, const uint16_t* __restrict__ w1p,
     const float* __restrict__ b32, const uint16_t* __restrict__ w2p, const uint16_t* __restrict__ bias2,
     const uint16_t* __restrict__ residual, uint32_t ldr, uint16_t* __restrict__ y, uint32_t ldy, uint32_t M,
-    uint32_t H, uint32_t main_wgs, uint32_t tail_rows) {
+    uint32_t H, uint32_t main_wgs, uint32_t tail_rows, MlpProj pj) {
   using G = XsGeom<K>;
   using MG = MlpGeom<K>;
   constexpr int KS = K / 16, ROWB = G::ROWB, WAVES = kMlpWaves, NB1 = kMlpBufs, NB2 = kMlpBufs, OT = MG::OT;
@@ -85,34 +111,179 @@ __global__ __launch_bounds__(64 * kMlpWaves) __attribute__((amdgpu_waves_per_eu(
   const uint32_t row0 = wg_row0 + wave * 32;
   const bool has_rows = (wave * 32 < (in_tail ? tail_rows : (uint32_t)ROWS_WG)) && row0 < M;
 
-  // ---- this wave's 32 rows of x -> registers (B-operand layout), through a wave-private transposition patch ----
+  // ---- weight streaming: per chunk 64 rows of w1 (N_DMA kilobytes), K x 32 of w2 (N_DMA2), the 64 values of b' (wave 0) ----
+  const uint32_t nchunk = H / 32;
+  static_assert(G::N_DMA % WAVES == 0 && MG::N_DMA2 % WAVES == 0, "direct loads split evenly over the waves");
+  constexpr uint32_t kDma1 = G::N_DMA / WAVES, kDma2 = MG::N_DMA2 / WAVES;
+  // One direct load moves 64 pieces = RPD w1 rows. The lane's byte offset inside such a group (its row of the group,
+  // its piece of the row under the row's swizzle) is the same for every group the wave loads, because the groups of
+  // one wave lie a multiple of 16 rows apart and the swizzle has period 16; everything else about an address is
+  // uniform and goes into the scalar base. (Addresses recomputed per load in vector registers cost the issuing wave
+  // about 60 cycles of dependent arithmetic each, with the matrix pipeline idle.)
+  constexpr uint32_t RPD = 64 / G::CPR;
+  static_assert((WAVES * RPD) % 16 == 0 && G::RP == 1 && 32 % RPD == 0, "one lane offset serves all groups of a wave");
+  const uint32_t w1_lane_off = ((lane / G::CPR) * K + (((lane % G::CPR) ^ G::swz(wave * RPD + lane / G::CPR)) * 8u)) * 2u;
+  const uint32_t tab_lane_off = (lane < 32 ? lane : H + lane - 32) * 4u;
+  auto dma_chunk = [&](uint32_t c) __attribute__((always_inline)) {
+    const char* b1 = w1buf + (c % NB1) * MG::CH1;
+#pragma unroll
+    for (uint32_t i = 0; i < kDma1; ++i) {
+      const uint32_t qi = wave + i * WAVES, r0 = qi * RPD;                       // first chunk row of the group
+      const uint32_t wrow0 = r0 < 32 ? c * 32u + r0 : H + c * 32u + (r0 - 32u);   // value rows, then gate rows
+      xs_lds_dma16(reinterpret_cast<const char*>(w1p) + (size_t)wrow0 * (K * 2), w1_lane_off, b1 + qi * 1024);
+    }
+    const char* b2 = w2buf + (c % NB2) * MG::CH2;
+#pragma unroll
+    for (uint32_t i = 0; i < kDma2; ++i)
+      xs_lds_dma16(reinterpret_cast<const char*>(w2p) + (size_t)c * MG::CH2 + (wave + i * WAVES) * 1024u, lane * 16u,
+                   b2 + (wave + i * WAVES) * 1024);
+    if (wave == 0) xs_lds_dma4(reinterpret_cast<const char*>(b32) + (size_t)c * 128, tab_lane_off, s_side + (c % NB1) * 1024);
+  };
+  // chunk c of the out-projection weight (rows 64 c .. 64 c + 63 of w, row-major) into w1 buffer c % NB1, laid out
+  // like a w1 chunk
+  auto dma_proj = [&](uint32_t c) __attribute__((always_inline)) {
+    const char* b1 = w1buf + (c % NB1) * MG::CH1;
+#pragma unroll
+    for (uint32_t i = 0; i < kDma1; ++i) {
+      const uint32_t qi = wave + i * WAVES;
+      xs_lds_dma16(reinterpret_cast<const char*>(pj.w) + (size_t)(c * kXsChunk + qi * RPD) * (K * 2), w1_lane_off, b1 + qi * 1024);
+    }
+  };
+
   bf16x8_t xf[KS];
-  {
-    constexpr int KP = G::KP, PROW = KP + 8, PCPR = KP / 8;
-    static_assert((size_t)WAVES * 32 * PROW * 2 <= MG::lds_bytes(), "the transposition patches alias everything else");
-    uint16_t* patch = reinterpret_cast<uint16_t*>(lds_mlp) + wave * (32 * PROW);
-    constexpr int XLOADS = (32 * PCPR) / kWave;
-    u32x4_t v[K / KP][XLOADS];
+  f32x16_t acc2[OT];
+  // acc2[ot][g*4+r] <-> output column ot*32 + g*8 + half*4 + r of row lq; they start from a bias
+  auto acc2_from_bias = [&](const uint16_t* bias) __attribute__((always_inline)) {
 #pragma unroll
-    for (int kp = 0; kp < K / KP; ++kp)
+    for (int ot = 0; ot < OT; ++ot)
 #pragma unroll
-      for (int i = 0; i < XLOADS; ++i) {
-        const uint32_t id = lane + i * kWave;
-        const uint32_t rr = id / PCPR, kc = (id % PCPR) * 8;
-        const uint32_t r = min(row0 + rr, M - 1);
-        v[kp][i] = *reinterpret_cast<const u32x4_t*>(x + (size_t)r * ldx + kp * KP + kc);
+      for (int g = 0; g < 4; ++g) {
+        const uint2 bb = *reinterpret_cast<const uint2*>(bias + ot * 32 + g * 8 + half * 4);
+        acc2[ot][g * 4 + 0] = bf16_lo(bb.x); acc2[ot][g * 4 + 1] = bf16_hi(bb.x);
+        acc2[ot][g * 4 + 2] = bf16_lo(bb.y); acc2[ot][g * 4 + 3] = bf16_hi(bb.y);
       }
+  };
+  if constexpr (PROJ) {
+    // ---- out-projection first: the projection's first weight chunk is requested before anything else; the wave's 32
+    //      rows of the attention output go straight into operand registers (16 bytes of a row per lane and k-step) ----
+    dma_proj(0);
+    {
+      const uint32_t r = min(row0 + lq, M - 1);
+      const uint16_t* ap = pj.a + (size_t)r * pj.lda + half * 8;
 #pragma unroll
-    for (int kp = 0; kp < K / KP; ++kp) {
+      for (int ks = 0; ks < KS; ++ks) xf[ks] = *reinterpret_cast<const bf16x8_t*>(ap + ks * 16);
+    }
+    acc2_from_bias(pj.b);
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+    __syncthreads();
+    // a wpT: output tile 2 c + t (32 columns) from rows 32 t .. 32 t + 31 of chunk c; the MLP's first chunk is
+    // requested under the projection's last one
+    const uint32_t poff = lq * ROWB + (((half ^ G::swz(lq)) & (uint32_t)(G::CPR - 1)) << 4);
+    const uint16_t* x_wg = x + (size_t)wg_row0 * ldx;
+    u32x4_t rin[OT][2];      // the block input's pieces of the wave's rows, row-contiguous (as the epilogue reads a residual)
+    auto load_rin = [&](int ot0, int ot1) __attribute__((always_inline)) {
 #pragma unroll
-      for (int i = 0; i < XLOADS; ++i) {
-        const uint32_t id = lane + i * kWave;
-        const uint32_t rr = id / PCPR, kc = (id % PCPR) * 8;
-        *reinterpret_cast<u32x4_t*>(patch + rr * PROW + kc) = v[kp][i];
+      for (int ot = ot0; ot < ot1; ++ot)
+#pragma unroll
+        for (int h2 = 0; h2 < 2; ++h2) {
+          const uint32_t rr = (lane >> 2) + h2 * 16, ch = (lane & 3u) * 8;
+          const uint32_t row = min(row0 + rr, M - 1);            // rows past M read row M - 1
+          rin[ot][h2] = *reinterpret_cast<const u32x4_t*>(x_wg + ((size_t)(row - wg_row0) * ldx + ot * 32 + ch));
+        }
+    };
+    mlp_static_for<MG::NPC>([&](auto c_c) {
+      constexpr uint32_t c = decltype(c_c)::value;
+      if constexpr (c + 1 < (uint32_t)MG::NPC) dma_proj(c + 1);
+      else dma_chunk(0);
+      if (has_rows) {
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+          const char* sw = w1buf + (c % NB1) * MG::CH1 + t * 32 * ROWB;
+          constexpr int kAhead = kMlpFragsAhead;
+          bf16x8_t wf[KS];
+#pragma unroll
+          for (int ks = 0; ks < kAhead; ++ks) wf[ks] = *reinterpret_cast<const bf16x8_t*>(sw + (poff ^ (uint32_t)(ks * 32)));
+#pragma unroll
+          for (int ks = 0; ks < KS; ++ks) {
+            if (ks + kAhead < KS) wf[ks + kAhead] = *reinterpret_cast<const bf16x8_t*>(sw + (poff ^ (uint32_t)((ks + kAhead) * 32)));
+            acc2[2 * c + t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[ks], xf[ks], acc2[2 * c + t], 0, 0, 0);
+          }
+        }
+        if constexpr (c + 1 == (uint32_t)MG::NPC) {
+          // the attention rows are dead: their registers take the block input's pieces, requested under the last wait
+          __builtin_amdgcn_sched_barrier(0);
+          load_rin(0, OT / 2);
+        }
       }
+      __builtin_amdgcn_s_waitcnt(0x0F70);
+      wg_barrier_lds();
+    });
+    // x1 = bf16(bf16(projection) + x), 32 columns at a time through the wave's patch: written in the accumulator
+    // layout, read and rewritten row-contiguous (where the block input's pieces are added), then read twice more:
+    // in operand layout (the k-steps 2 ot, 2 ot + 1 of the LayerNorm / fc1 panel) and in the accumulator layout
+    // (x1 + b2, what the fc2 products add to)
+    if (has_rows) {
+      uint16_t* xp1 = reinterpret_cast<uint16_t*>(lds_mlp + MG::loop_bytes()) + wave * (32 * kPatchRow);
+      load_rin(OT / 2, OT);
 #pragma unroll
-      for (int ks = 0; ks < KP / 16; ++ks)
-        xf[kp * (KP / 16) + ks] = *reinterpret_cast<const bf16x8_t*>(patch + lq * PROW + ks * 16 + half * 8);
+      for (int ot = 0; ot < OT; ++ot) {
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          uint2 pk;
+          pk.x = pack_bf16x2(acc2[ot][g * 4 + 0], acc2[ot][g * 4 + 1]);
+          pk.y = pack_bf16x2(acc2[ot][g * 4 + 2], acc2[ot][g * 4 + 3]);
+          *reinterpret_cast<uint2*>(xp1 + lq * kPatchRow + g * 8 + half * 4) = pk;
+        }
+#pragma unroll
+        for (int h2 = 0; h2 < 2; ++h2) {
+          const uint32_t rr = (lane >> 2) + h2 * 16, ch = (lane & 3u) * 8;
+          u32x4_t t = *reinterpret_cast<const u32x4_t*>(xp1 + rr * kPatchRow + ch);
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            t[e] = pack_bf16x2(bf16_lo(t[e]) + bf16_lo(rin[ot][h2][e]), bf16_hi(t[e]) + bf16_hi(rin[ot][h2][e]));
+          *reinterpret_cast<u32x4_t*>(xp1 + rr * kPatchRow + ch) = t;
+        }
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+          xf[2 * ot + j] = *reinterpret_cast<const bf16x8_t*>(xp1 + lq * kPatchRow + j * 16 + half * 8);
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const uint2 v = *reinterpret_cast<const uint2*>(xp1 + lq * kPatchRow + g * 8 + half * 4);
+          const uint2 bb = *reinterpret_cast<const uint2*>(bias2 + ot * 32 + g * 8 + half * 4);
+          acc2[ot][g * 4 + 0] = bf16_lo(v.x) + bf16_lo(bb.x); acc2[ot][g * 4 + 1] = bf16_hi(v.x) + bf16_hi(bb.x);
+          acc2[ot][g * 4 + 2] = bf16_lo(v.y) + bf16_lo(bb.y); acc2[ot][g * 4 + 3] = bf16_hi(v.y) + bf16_hi(bb.y);
+        }
+      }
+    }
+  } else {
+    // ---- this wave's 32 rows of x -> registers (B-operand layout), through a wave-private transposition patch ----
+    {
+      constexpr int KP = G::KP, PROW = KP + 8, PCPR = KP / 8;
+      static_assert((size_t)WAVES * 32 * PROW * 2 <= MG::lds_bytes(), "the transposition patches alias everything else");
+      uint16_t* patch = reinterpret_cast<uint16_t*>(lds_mlp) + wave * (32 * PROW);
+      constexpr int XLOADS = (32 * PCPR) / kWave;
+      u32x4_t v[K / KP][XLOADS];
+  #pragma unroll
+      for (int kp = 0; kp < K / KP; ++kp)
+  #pragma unroll
+        for (int i = 0; i < XLOADS; ++i) {
+          const uint32_t id = lane + i * kWave;
+          const uint32_t rr = id / PCPR, kc = (id % PCPR) * 8;
+          const uint32_t r = min(row0 + rr, M - 1);
+          v[kp][i] = *reinterpret_cast<const u32x4_t*>(x + (size_t)r * ldx + kp * KP + kc);
+        }
+  #pragma unroll
+      for (int kp = 0; kp < K / KP; ++kp) {
+  #pragma unroll
+        for (int i = 0; i < XLOADS; ++i) {
+          const uint32_t id = lane + i * kWave;
+          const uint32_t rr = id / PCPR, kc = (id % PCPR) * 8;
+          *reinterpret_cast<u32x4_t*>(patch + rr * PROW + kc) = v[kp][i];
+        }
+  #pragma unroll
+        for (int ks = 0; ks < KP / 16; ++ks)
+          xf[kp * (KP / 16) + ks] = *reinterpret_cast<const bf16x8_t*>(patch + lq * PROW + ks * 16 + half * 8);
+      }
     }
   }
   // LayerNorm in place (statistics shifted by the row's first element; x <- bf16((x - mean) * rstd), one fragment at a
@@ -143,50 +314,14 @@ __global__ __launch_bounds__(64 * kMlpWaves) __attribute__((amdgpu_waves_per_eu(
       xf[ks] = __builtin_bit_cast(bf16x8_t, pk);
     }
   }
-  // fc2 accumulators start from the bias: acc2[ot][g*4+r] <-> output column ot*32 + g*8 + half*4 + r of row lq
-  f32x16_t acc2[OT];
-#pragma unroll
-  for (int ot = 0; ot < OT; ++ot)
-#pragma unroll
-    for (int g = 0; g < 4; ++g) {
-      const uint2 bb = *reinterpret_cast<const uint2*>(bias2 + ot * 32 + g * 8 + half * 4);
-      acc2[ot][g * 4 + 0] = bf16_lo(bb.x); acc2[ot][g * 4 + 1] = bf16_hi(bb.x);
-      acc2[ot][g * 4 + 2] = bf16_lo(bb.y); acc2[ot][g * 4 + 3] = bf16_hi(bb.y);
-    }
-  __builtin_amdgcn_s_waitcnt(0x0F70);
-  __syncthreads();   // the transposition patches are dead; the space now holds weight chunks
-
-  // ---- weight streaming: per chunk 64 rows of w1 (N_DMA kilobytes), K x 32 of w2 (N_DMA2), the 64 values of b' (wave 0) ----
-  const uint32_t nchunk = H / 32;
-  static_assert(G::N_DMA % WAVES == 0 && MG::N_DMA2 % WAVES == 0, "direct loads split evenly over the waves");
-  constexpr uint32_t kDma1 = G::N_DMA / WAVES, kDma2 = MG::N_DMA2 / WAVES;
-  // One direct load moves 64 pieces = RPD w1 rows. The lane's byte offset inside such a group (its row of the group,
-  // its piece of the row under the row's swizzle) is the same for every group the wave loads, because the groups of
-  // one wave lie a multiple of 16 rows apart and the swizzle has period 16; everything else about an address is
-  // uniform and goes into the scalar base. (Addresses recomputed per load in vector registers cost the issuing wave
-  // about 60 cycles of dependent arithmetic each, with the matrix pipeline idle.)
-  constexpr uint32_t RPD = 64 / G::CPR;
-  static_assert((WAVES * RPD) % 16 == 0 && G::RP == 1 && 32 % RPD == 0, "one lane offset serves all groups of a wave");
-  const uint32_t w1_lane_off = ((lane / G::CPR) * K + (((lane % G::CPR) ^ G::swz(wave * RPD + lane / G::CPR)) * 8u)) * 2u;
-  const uint32_t tab_lane_off = (lane < 32 ? lane : H + lane - 32) * 4u;
-  auto dma_chunk = [&](uint32_t c) __attribute__((always_inline)) {
-    const char* b1 = w1buf + (c % NB1) * MG::CH1;
-#pragma unroll
-    for (uint32_t i = 0; i < kDma1; ++i) {
-      const uint32_t qi = wave + i * WAVES, r0 = qi * RPD;                       // first chunk row of the group
-      const uint32_t wrow0 = r0 < 32 ? c * 32u + r0 : H + c * 32u + (r0 - 32u);   // value rows, then gate rows
-      xs_lds_dma16(reinterpret_cast<const char*>(w1p) + (size_t)wrow0 * (K * 2), w1_lane_off, b1 + qi * 1024);
-    }
-    const char* b2 = w2buf + (c % NB2) * MG::CH2;
-#pragma unroll
-    for (uint32_t i = 0; i < kDma2; ++i)
-      xs_lds_dma16(reinterpret_cast<const char*>(w2p) + (size_t)c * MG::CH2 + (wave + i * WAVES) * 1024u, lane * 16u,
-                   b2 + (wave + i * WAVES) * 1024);
-    if (wave == 0) xs_lds_dma4(reinterpret_cast<const char*>(b32) + (size_t)c * 128, tab_lane_off, s_side + (c % NB1) * 1024);
-  };
-  dma_chunk(0);
-  __builtin_amdgcn_s_waitcnt(0x0F70);
-  __syncthreads();
+  if constexpr (!PROJ) {
+    acc2_from_bias(bias2);
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+    __syncthreads();   // the transposition patches are dead; the space now holds weight chunks
+    dma_chunk(0);
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+    __syncthreads();
+  }
 
   // the lane's row of a half's fc1 tile inside the chunk buffer (half h adds 16 rows): value rows 0-15, gate rows 32-47
   const uint32_t trow = lq < 16 ? lq : lq + 16;
@@ -532,14 +667,14 @@ __global__ __launch_bounds__(256) void mlp_prep_kernel(const uint16_t* __restric
 }
 
 
-template <int K>
+template <int K, bool PROJ = false>
 static int launch_mlp(const uint16_t* x, uint32_t ldx, float eps, const uint16_t* w1p, const float* b32,
                            const uint16_t* w2p, const uint16_t* bias2, const uint16_t* residual, uint32_t ldr, uint16_t* y,
-                           uint32_t ldy, uint32_t M, uint32_t H, int device, hipStream_t s) {
-  constexpr size_t lds = MlpGeom<K>::lds_bytes();
+                           uint32_t ldy, uint32_t M, uint32_t H, int device, hipStream_t s, MlpProj pj = MlpProj{}) {
+  constexpr size_t lds = MlpGeom<K>::lds_bytes(PROJ);
   static_assert(lds <= 160 * 1024, "chunk buffers exceed the LDS of a compute unit");
   static bool attr_set[64] = {};
-  auto kern = ln_mlp_swiglu_kernel<K>;
+  auto kern = ln_mlp_swiglu_kernel<K, PROJ>;
   if (device < 0 || device >= 64 || !attr_set[device]) {
     F3D_CHECK_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     if (device >= 0 && device < 64) attr_set[device] = true;
@@ -562,7 +697,7 @@ static int launch_mlp(const uint16_t* x, uint32_t ldx, float eps, const uint16_t
     tail_wgs = cdiv_u32(left, tail_rows);
   }
   hipLaunchKernelGGL(kern, dim3(main_wgs + tail_wgs), dim3(64 * kMlpWaves), lds, s, x, ldx, eps, w1p, b32, w2p, bias2, residual,
-                     ldr, y, ldy, M, H, main_wgs, tail_rows);
+                     ldr, y, ldy, M, H, main_wgs, tail_rows, pj);
   return F3D_OK;
 }
 
@@ -641,6 +776,53 @@ int f3d_ln_mlp_swiglu_bf16(const f3d_bf16_t* x, uint32_t ldx, const f3d_bf16_t* 
   else if (c == 32) rc = launch_mlp_small<32>(x, ldx, eps, w1p, b32, w2p, b2, residual, ldr, y, ldy, m, hidden, device, s);
   else if (c == 64) rc = launch_mlp_small<64>(x, ldx, eps, w1p, b32, w2p, b2, residual, ldr, y, ldy, m, hidden, device, s);
   else rc = launch_mlp<128>(x, ldx, eps, w1p, b32, w2p, b2, residual, ldr, y, ldy, m, hidden, device, s);
+  if (rc != F3D_OK) return rc;
+  F3D_CHECK_HIP(hipGetLastError());
+  return F3D_OK;
+}
+
+int f3d_proj_ln_mlp_swiglu_bf16(const f3d_bf16_t* a, uint32_t lda, const f3d_bf16_t* w_proj, const f3d_bf16_t* b_proj,
+                                const f3d_bf16_t* x, uint32_t ldx, const f3d_bf16_t* gamma, const f3d_bf16_t* beta, float eps,
+                                const f3d_bf16_t* w1, const f3d_bf16_t* b1, const f3d_bf16_t* w2, const f3d_bf16_t* b2,
+                                f3d_bf16_t* y, uint32_t ldy, uint32_t m, uint32_t c, uint32_t hidden, int device,
+                                void* stream) {
+  using namespace f3d;
+  StagedWeightsScope staged;
+  F3D_CHECK_ARG(a && w_proj && x && gamma && w1 && w2 && y, "null tensor pointer");
+  if (!(c == 128 || c == 256) || hidden == 0 || hidden % 32 != 0 || (uint64_t)hidden * c * 4 >= (1ull << 32)) {
+    set_error("No out-projection + MLP kernel for width %u with hidden width %u (widths 128 and 256, hidden a multiple of 32)",
+              c, hidden);
+    return F3D_ERR_UNSUPPORTED;
+  }
+  F3D_CHECK_ARG(lda >= c && lda % 8 == 0 && ldx >= c && ldx % 8 == 0 && ldy >= c && ldy % 8 == 0,
+                "row strides must be aligned and cover a row (lda=%u ldx=%u ldy=%u)", lda, ldx, ldy);
+  F3D_CHECK_ARG((((uintptr_t)a | (uintptr_t)w_proj | (uintptr_t)b_proj | (uintptr_t)x | (uintptr_t)w1 | (uintptr_t)w2 |
+                  (uintptr_t)y | (uintptr_t)gamma | (uintptr_t)beta | (uintptr_t)b2) & 15u) == 0,
+                "a/w_proj/b_proj/x/w1/w2/b2/y/gamma/beta must be 16-byte aligned");
+  if (m == 0) return F3D_OK;
+  DeviceGuard guard(device);
+  F3D_CHECK_ARG(guard.ok, "cannot select device %d", device);
+  hipStream_t s = (hipStream_t)stream;
+  SyncBracket sync(s);
+  // the MLP's prepared weights exactly as in f3d_ln_mlp_swiglu_bf16 (the same staged buffer serves both entry points)
+  const size_t w1_bytes = (size_t)2 * hidden * c * 2, b32_bytes = (((size_t)2 * hidden * 4) + 255) & ~(size_t)255;
+  const size_t w2_bytes = (size_t)hidden * c * 2;
+  bool ready = false;
+  char* ws = (char*)weight_area(device, w1_bytes + b32_bytes + w2_bytes + (size_t)c * 2, &ready, s);
+  if (!ws) return F3D_ERR_RUNTIME;
+  uint16_t* w1p = (uint16_t*)ws;
+  float* b32 = (float*)(ws + w1_bytes);
+  uint16_t* w2p = (uint16_t*)(ws + w1_bytes + b32_bytes);
+  uint16_t* zero_bias = (uint16_t*)(ws + w1_bytes + b32_bytes + w2_bytes);
+  if (!b2) b2 = zero_bias;
+  const uint32_t fold_blocks = cdiv_u32(2 * hidden, 4);
+  if (!ready)
+    hipLaunchKernelGGL(mlp_prep_kernel, dim3(fold_blocks + cdiv_u32(c * hidden / 8, 256)), dim3(256), 0, s, w1, gamma, beta, b1,
+                       w1p, b32, fold_blocks, w2, w2p, zero_bias, c, hidden);
+  const MlpProj pj{a, lda, w_proj, b_proj ? b_proj : zero_bias};
+  int rc;
+  if (c == 256) rc = launch_mlp<256, true>(x, ldx, eps, w1p, b32, w2p, b2, nullptr, 0, y, ldy, m, hidden, device, s, pj);
+  else rc = launch_mlp<128, true>(x, ldx, eps, w1p, b32, w2p, b2, nullptr, 0, y, ldy, m, hidden, device, s, pj);
   if (rc != F3D_OK) return rc;
   F3D_CHECK_HIP(hipGetLastError());
   return F3D_OK;

@@ -93,10 +93,11 @@ class BucketSwinAttentionModule(nn.Module):
         self.proj = Linear(channels, channels)
 
     def forward(self, x: torch.Tensor, scope_buckets: torch.Tensor, residual: torch.Tensor = None,
-                pre_norm=None) -> torch.Tensor:
+                pre_norm=None, skip_proj: bool = False) -> torch.Tensor:
         """x [B, L, C] -> [B, L, C].  Q, K and V are read by the attention kernel straight out of the
         [B, L, 3C] projection output (the reference makes three contiguous copies, :187-190); the
-        residual, when given, is added in the out-projection's epilogue."""
+        residual, when given, is added in the out-projection's epilogue.  skip_proj: return the attention output
+        itself (the caller applies `self.proj`, e.g. inside the kernel of the MLP that follows)."""
         assert x.dim() == 3, f"Expect input features with three axes [B, L, C], but got shape={x.shape}"
         B, L, C = x.shape
         assert C == self.num_heads * self.head_dim, f"Expect input channels are {self.num_heads * self.head_dim}, but got {C}"
@@ -108,7 +109,7 @@ class BucketSwinAttentionModule(nn.Module):
         else:
             q, k, v = (t.view(B, L, self.num_heads, self.head_dim) for t in torch.chunk(qkv, 3, dim=-1))
             attn_out = self.attn(q, k, v, scope_buckets)
-        out = self.proj(attn_out.view(B, L, C), residual=residual)
+        out = attn_out.view(B, L, C) if skip_proj else self.proj(attn_out.view(B, L, C), residual=residual)
         if f3ddev.get_nvtx():
             nvtx.range_pop()
         return out

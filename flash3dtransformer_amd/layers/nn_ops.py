@@ -416,6 +416,7 @@ class LayerNorm(_CachedParamModule):
 
 FUSABLE_LN_WIDTHS = (32, 64, 128, 256, 512)
 FUSED_MLP_WIDTHS = (32, 64, 128, 256)      # widths the one-kernel gated MLP covers (32 / 64: while the weights fit into LDS)
+PROJ_MLP_WIDTHS = (128, 256)               # widths at which it also takes the out-projection and its residual in front
 
 
 def is_fusable_layernorm(norm, width: int) -> bool:
@@ -556,6 +557,29 @@ class LayerNormMLP(_CachedParamModule):
         nn.init.normal_(self.fc2_weight, std=0.023)
         self._c = [_Bf16Cache() for _ in range(6)]
         self._staged = [_StagedWeights(), _StagedWeights()]      # fused kernel / fc1 of the two-kernel path; fc2
+
+    def after_projection(self, a: torch.Tensor, proj: "Linear", x: torch.Tensor):
+        """x1 = proj(a) + x;  x1 + MLP(x1) in one kernel (x1 is never stored): the second half of a transformer block
+        (flash3dxfmr/layers/stage.py:92-102) at inference.  a, x [rows, hidden_size] bf16.  Returns None where that
+        kernel does not apply (autograd on, other widths or activation, few rows): the caller then runs `proj` with its
+        residual and this module."""
+        if (torch.is_grad_enabled() or self.activation != "swiglu" or self.hidden_size not in PROJ_MLP_WIDTHS
+                or self.ffn_hidden_size % 32 != 0 or self.fused is False or proj.in_features != self.hidden_size
+                or proj.out_features != self.hidden_size or not a.is_cuda or a.dtype != torch.bfloat16
+                or x.dtype != torch.bfloat16 or a.shape[0] < 30000):
+            return None
+        a2, x2 = a.reshape(-1, self.hidden_size), x.reshape(-1, self.hidden_size)
+        if a2.stride(1) != 1 or x2.stride(1) != 1:
+            return None
+        params = (self.layer_norm_weight, self.layer_norm_bias, self.fc1_weight, self.fc1_bias, self.fc2_weight, self.fc2_bias)
+        g16, be16, w1_16, b1_16, w2_16, b2_16 = (c.get(p, self.training) for c, p in zip(self._c, params))
+        wp16, bp16 = proj._w.get(proj.weight, proj.training), proj._b.get(proj.bias, proj.training)
+        y = torch.empty(a2.shape[0], self.hidden_size, dtype=torch.bfloat16, device=a.device)
+        self._staged[0].arm(self.training, w1_16.shape[0], self.hidden_size, g16, be16, w1_16, b1_16, w2_16, b2_16,
+                            tag=("mlp", float(self.eps)))
+        if not pshattn.proj_ln_mlp_swiglu_bf16(a2, wp16, bp16, x2, g16, be16, self.eps, w1_16, b1_16, w2_16, b2_16, y):
+            return None
+        return y.view(x.shape)
 
     def forward(self, x: torch.Tensor, residual: torch.Tensor = None):
         x2 = as_bf16_2d(x.reshape(-1, self.hidden_size)).contiguous()

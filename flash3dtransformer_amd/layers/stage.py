@@ -43,13 +43,20 @@ class XFMR(nn.Module):
         scope_bucks = self.swin_plan.gen_scopes_from_plan(N, reduced_feat.device)
         if f3ddev.get_nvtx():
             nvtx.range_push(self.NVTX_SCOPE)
-        if is_fusable_layernorm(self.norm, C):   # norm -> qkv in one kernel
-            mid = self.bwa(reduced_feat.view(1, N, C), scope_bucks, residual=reduced_feat.view(1, N, C),
-                           pre_norm=self.norm).view(N, C)
+        fused_ln = is_fusable_layernorm(self.norm, C)   # norm -> qkv in one kernel
+        x = reduced_feat if fused_ln else apply_norm(self.norm, reduced_feat)
+        pre = self.norm if fused_ln else None
+        out = None
+        if not torch.is_grad_enabled() and reduced_feat.dtype == torch.bfloat16:
+            # inference: out-projection + residual + MLP + residual in one kernel where it applies
+            attn = self.bwa(x.view(1, N, C), scope_bucks, pre_norm=pre, skip_proj=True).view(N, C)
+            out = self.mlp.mlp.after_projection(attn, self.bwa.proj, reduced_feat)
+            if out is None:
+                mid = self.bwa.proj(attn, residual=reduced_feat)
+                out = self.mlp(mid, residual=mid)
         else:
-            x = apply_norm(self.norm, reduced_feat)
-            mid = self.bwa(x.view(1, N, C), scope_bucks, residual=reduced_feat.view(1, N, C)).view(N, C)
-        out = self.mlp(mid, residual=mid)
+            mid = self.bwa(x.view(1, N, C), scope_bucks, residual=reduced_feat.view(1, N, C), pre_norm=pre).view(N, C)
+            out = self.mlp(mid, residual=mid)
         if f3ddev.get_nvtx():
             nvtx.range_pop()
         return out

@@ -646,6 +646,32 @@ def ln_mlp_swiglu_bf16(x, gamma, beta, eps, w1, b1, w2, b2, residual, y) -> bool
     return True
 
 
+def proj_ln_mlp_swiglu_bf16(a, w_proj, b_proj, x, gamma, beta, eps, w1, b1, w2, b2, y) -> bool:
+    """extension: the second half of a block in one kernel (stage.py:92-102): x1 = a w_proj.T + b_proj + x, then
+    y = x1 + MLP(LayerNorm(x1)) with the gated MLP of ln_mlp_swiglu_bf16; x1 never reaches memory.  Returns False,
+    leaving y untouched, when no kernel covers the widths (the caller then runs linear_bf16 + ln_mlp_swiglu_bf16)."""
+    dev = assert_same_device([a, w_proj, x, gamma, w1, w2, y])
+    assert_dtype([a, w_proj, x, gamma, w1, w2, y], torch.bfloat16)
+    assert_contiguous([w_proj, w1, w2, gamma])
+    _check_vectors(x, [b_proj, beta, b1, b2])
+    if any(t.dim() != 2 or t.stride(1) != 1 for t in (a, x, y)):
+        raise RuntimeError("proj_ln_mlp_swiglu_bf16 expects 2-D row-major a, x and y")
+    m, c = x.shape
+    hidden = w2.shape[1]
+    if (tuple(a.shape) != (m, c) or tuple(w_proj.shape) != (c, c) or tuple(w1.shape) != (2 * hidden, c) or w2.shape[0] != c
+            or tuple(y.shape) != (m, c) or gamma.shape[0] != c):
+        raise RuntimeError(f"proj_ln_mlp shape mismatch: a{tuple(a.shape)} x{tuple(x.shape)} w_proj{tuple(w_proj.shape)} "
+                           f"w1{tuple(w1.shape)} w2{tuple(w2.shape)} y{tuple(y.shape)}")
+    rc = _load().f3d_proj_ln_mlp_swiglu_bf16(_ptr(a), _u32(a.stride(0)), _ptr(w_proj), _ptr(b_proj), _ptr(x),
+                                             _u32(x.stride(0)), _ptr(gamma), _ptr(beta), _f32(eps), _ptr(w1), _ptr(b1),
+                                             _ptr(w2), _ptr(b2), _ptr(y), _u32(y.stride(0)), _u32(m), _u32(c),
+                                             _u32(hidden), _i32(dev), _stream(dev))
+    if rc == 2:
+        return False
+    _check(rc)
+    return True
+
+
 def stage_weights(buf: torch.Tensor, ready: bool):
     """extension: the next dense call on this thread keeps the weights it prepares (LayerNorm fold, fragment-major
     copies) in `buf` (uint8 device tensor, 256-byte aligned), or with `ready` reuses what an earlier call with the same

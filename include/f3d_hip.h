@@ -320,6 +320,20 @@ int f3d_ln_mlp_swiglu_bf16(const f3d_bf16_t* x, uint32_t ldx, const f3d_bf16_t* 
                            const f3d_bf16_t* residual, uint32_t ldr, f3d_bf16_t* y, uint32_t ldy, uint32_t m,
                            uint32_t c, uint32_t hidden, int device, void* stream);
 
+/* The second half of a transformer block in one kernel (flash3dxfmr/layers/stage.py:92-102: `proj`, the residual
+ * add, then the MLP with its residual):
+ *   x1 = a w_projT + b_proj + x,   y = x1 + MLP(LayerNorm(x1))   with the MLP of f3d_ln_mlp_swiglu_bf16.
+ * a [m,c] (row stride lda) is the attention output, x [m,c] (row stride ldx) the block input, w_proj [c,c], b_proj [c]
+ * or NULL; the other arguments as in f3d_ln_mlp_swiglu_bf16 (no residual argument: x1 is the residual).  x1 is rounded
+ * to bf16 as a separate projection kernel would store it and is held in registers only.  c in {128, 256}, hidden a
+ * multiple of 32; anything else returns F3D_ERR_UNSUPPORTED without touching y (use f3d_linear_bf16 with the residual,
+ * then f3d_ln_mlp_swiglu_bf16).  Inference only: no backward consumes its result. */
+int f3d_proj_ln_mlp_swiglu_bf16(const f3d_bf16_t* a, uint32_t lda, const f3d_bf16_t* w_proj, const f3d_bf16_t* b_proj,
+                                const f3d_bf16_t* x, uint32_t ldx, const f3d_bf16_t* gamma, const f3d_bf16_t* beta, float eps,
+                                const f3d_bf16_t* w1, const f3d_bf16_t* b1, const f3d_bf16_t* w2, const f3d_bf16_t* b2,
+                                f3d_bf16_t* y, uint32_t ldy, uint32_t m, uint32_t c, uint32_t hidden, int device,
+                                void* stream);
+
 /* LayerNorm over the last axis, fp32 statistics (norm callables of flash3dxfmr/layers/stage.py:67).
  * x,y [m,c] bf16; gamma,beta [c] bf16 (beta may be NULL). */
 int f3d_layernorm_bf16(const f3d_bf16_t* x, const f3d_bf16_t* gamma, const f3d_bf16_t* beta, f3d_bf16_t* y,

@@ -234,6 +234,62 @@ def test_fused_mlp_matches_two_kernel_path(oracle, M, C, H, use_res, use_bias):
     assert err_us.mean() <= 1.25 * err_ref.mean() + 1e-4, (err_us.mean(), err_ref.mean())
 
 
+@pytest.mark.parametrize("M,C,H,use_bias", [
+    (4096, 256, 1024, True),       # the C = 256 block
+    (1000, 256, 512, True),        # ragged M
+    (777, 128, 512, False),        # C = 128 (two projection chunks), no biases
+    (300, 256, 32, True),          # a single hidden chunk behind the projection
+    (70000, 128, 256, True),       # many workgroups
+    (66000, 256, 64, True),        # more panels than CUs: shorter panels in the last turn
+])
+def test_proj_residual_mlp_in_one_kernel(oracle, M, C, H, use_bias):
+    """out-projection + residual + gated MLP + residual in one kernel against (a) the projection kernel followed by the
+    one-kernel MLP, whose roundings it reproduces up to the last one (the MLP's output is added to x1 in fp32 and rounded
+    once instead of twice), and (b) the unrounded mathematics next to the reference's rounding sequence."""
+    from flash3dtransformer_amd.lib import pshattn
+    a = _rand((M, C), 11, scale=1.5).to(DEV)
+    x = (_rand((M, C), 1, scale=2.0) + 0.3).to(DEV)
+    wp = _rand((C, C), 12, scale=1 / math.sqrt(C)).to(DEV)
+    bp = _rand((C,), 13).to(DEV) if use_bias else None
+    g, b = (_rand((C,), 3) + 1.0).to(DEV), _rand((C,), 4, scale=0.2).to(DEV)
+    w1, w2 = _rand((2 * H, C), 2, scale=1 / math.sqrt(C)).to(DEV), _rand((C, H), 5, scale=1 / math.sqrt(H)).to(DEV)
+    b1 = _rand((2 * H,), 6).to(DEV) if use_bias else None
+    b2 = _rand((C,), 7).to(DEV) if use_bias else None
+    y = torch.full((M, C), 9.0, dtype=torch.bfloat16, device=DEV)
+    assert pshattn.proj_ln_mlp_swiglu_bf16(a, wp, bp, x, g, b, 1e-5, w1, b1, w2, b2, y)
+    x1 = torch.empty_like(x)
+    y2 = torch.empty_like(y)
+    pshattn.linear_bf16(a, wp, bp, x, x1, None)
+    assert pshattn.ln_mlp_swiglu_bf16(x1, g, b, 1e-5, w1, b1, w2, b2, x1, y2)
+    torch.cuda.synchronize()
+    d = (y.float() - y2.float()).abs()
+    scale = y2.float().abs().clamp(min=1.0)
+    assert (d / scale).max().item() <= 2 ** -5, (d / scale).max().item()
+    assert (d > 0).float().mean().item() < 0.35          # one rounding instead of two moves the last bit now and then
+    ac, xc, wpc, gc, bc, w1c, w2c = a.cpu(), x.cpu(), wp.cpu(), g.cpu(), b.cpu(), w1.cpu(), w2.cpu()
+    cpu = lambda t: None if t is None else t.cpu()
+    rb = lambda t: t.to(torch.bfloat16).float()
+    mlp = lambda t, r: oracle.linear(r(oracle.swiglu(r(oracle.linear(r(oracle.layernorm(t, gc, bc, 1e-5)), w1c, cpu(b1))))), w2c, cpu(b2))
+    same = lambda t: t
+    x1e = oracle.linear(ac, wpc, cpu(bp)) + xc.float()
+    exact = x1e + mlp(x1e, same)
+    x1r = rb(rb(oracle.linear(ac, wpc, cpu(bp))) + xc.float())
+    ref = rb(x1r + rb(mlp(x1r, rb)))
+    scale = exact.abs().clamp(min=1.0)
+    err_us, err_ref = (y.float().cpu() - exact).abs() / scale, (ref - exact).abs() / scale
+    assert err_us.max() <= 1.5 * err_ref.max() + 4e-3, (err_us.max(), err_ref.max())
+    assert err_us.mean() <= 1.25 * err_ref.mean() + 1e-4, (err_us.mean(), err_ref.mean())
+
+
+def test_proj_residual_mlp_unsupported_width_is_reported():
+    from flash3dtransformer_amd.lib import pshattn
+    mk = lambda *s: torch.zeros(*s, dtype=torch.bfloat16, device=DEV)
+    y = torch.full((64, 64), 3.0, dtype=torch.bfloat16, device=DEV)
+    assert not pshattn.proj_ln_mlp_swiglu_bf16(mk(64, 64), mk(64, 64), None, mk(64, 64), mk(64), mk(64), 1e-5, mk(256, 64),
+                                               None, mk(64, 128), None, y)
+    assert (y == 3.0).all()
+
+
 def test_fused_mlp_unsupported_width_is_reported():
     from flash3dtransformer_amd.lib import pshattn
     mk = lambda *s: torch.zeros(*s, dtype=torch.bfloat16, device=DEV)
