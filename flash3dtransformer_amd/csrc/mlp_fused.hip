@@ -32,6 +32,11 @@
 // C = 128, H = 512: 0.138 ms against 0.224 ms.  (A first form with 64 rows per wave and one wave per SIMD, whose
 // register file the x rows (128) and the fc2 accumulators (256) fill, took 0.87 ms: with a single wave per SIMD
 // nothing overlaps the issue of the roughly 1000 instructions that go with the 100 products of a chunk.)
+//
+// With the block's out-projection in front (PROJ kernels, f3d_proj_ln_mlp_swiglu_bf16; flash3dxfmr/layers/stage.py:92-102:
+// proj, residual add, MLP, residual add): x1 = a wpT + bp + x is formed in the fc2 accumulators before the LayerNorm
+// and never reaches memory; the kernel then returns x1 + MLP(LayerNorm(x1)).  482,304 rows, C = 256: 0.775 ms against
+// 0.155 + 0.70 ms for the projection kernel followed by this kernel without it.
 #include <algorithm>
 
 #include "xstat_common.h"
@@ -60,7 +65,7 @@ struct MlpGeom {
   static constexpr int N_DMA2 = CH2 / 1024;
   static constexpr int NPC = K / kXsChunk;                  // 64-row chunks of the out-projection weight
   static constexpr size_t loop_bytes() { return (size_t)kMlpBufs * (CH1 + 1024 + CH2); }
-  static constexpr size_t row_patch_bytes() { return (size_t)kMlpWaves * 32 * kPatchRow * 2; }
+  static constexpr size_t row_patch_bytes() { return (size_t)2 * kMlpWaves * 32 * kPatchRow * 2; }   // two patches per wave
   // weight buffers and the b' slots of the w1 buffers; at least the prologue's transposition patches; with the
   // out-projection in front, the wave-private patches its result is re-laid through come after the weight buffers
   static constexpr size_t lds_bytes(bool proj = false) {
@@ -196,6 +201,7 @@ __global__ __launch_bounds__(64 * kMlpWaves) __attribute__((amdgpu_waves_per_eu(
       if constexpr (c + 1 < (uint32_t)MG::NPC) dma_proj(c + 1);
       else dma_chunk(0);
       if (has_rows) {
+        if constexpr (c == 0) load_rin(0, OT / 2);    // spare registers take the first half right away
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
           const char* sw = w1buf + (c % NB1) * MG::CH1 + t * 32 * ROWB;
@@ -209,50 +215,51 @@ __global__ __launch_bounds__(64 * kMlpWaves) __attribute__((amdgpu_waves_per_eu(
             acc2[2 * c + t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[ks], xf[ks], acc2[2 * c + t], 0, 0, 0);
           }
         }
-        if constexpr (c + 1 == (uint32_t)MG::NPC) {
-          // the attention rows are dead: their registers take the block input's pieces, requested under the last wait
-          __builtin_amdgcn_sched_barrier(0);
-          load_rin(0, OT / 2);
-        }
       }
-      __builtin_amdgcn_s_waitcnt(0x0F70);
+      // the next chunk has landed.  In the first round the block input's pieces were requested AFTER the chunk's direct
+      // loads and may stay in flight: OT younger loads (a wave without rows has none)
+      static_assert(OT < 16, "the count fits the low bits of the wait's immediate");
+      if (c == 0 && has_rows) __builtin_amdgcn_s_waitcnt(0x0F70 | OT);
+      else __builtin_amdgcn_s_waitcnt(0x0F70);
       wg_barrier_lds();
     });
-    // x1 = bf16(bf16(projection) + x), 32 columns at a time through the wave's patch: written in the accumulator
-    // layout, read and rewritten row-contiguous (where the block input's pieces are added), then read twice more:
-    // in operand layout (the k-steps 2 ot, 2 ot + 1 of the LayerNorm / fc1 panel) and in the accumulator layout
-    // (x1 + b2, what the fc2 products add to)
+    // x1 = bf16(bf16(projection) + x).  The block input's pieces arrive row-contiguous; they go through the wave's first
+    // patch into the accumulator layout (all eight tiles back to back: LDS serves a wave in order, so the next tile's
+    // writes need not wait for this tile's reads), x1 is formed in registers (also x1 + b2, what the fc2 products add
+    // to), written to the second patch in the accumulator layout and read back in operand layout (the k-steps 2 ot,
+    // 2 ot + 1 of the LayerNorm / fc1 panel), again without a wait between tiles.
     if (has_rows) {
-      uint16_t* xp1 = reinterpret_cast<uint16_t*>(lds_mlp + MG::loop_bytes()) + wave * (32 * kPatchRow);
-      load_rin(OT / 2, OT);
+      uint16_t* pa = reinterpret_cast<uint16_t*>(lds_mlp + MG::loop_bytes()) + wave * (32 * kPatchRow);
+      uint16_t* pb = pa + WAVES * (32 * kPatchRow);
+      load_rin(OT / 2, OT);     // the attention rows are dead: their registers take the second half
+      uint2 rc[OT][4];
+#pragma unroll
+      for (int ot = 0; ot < OT; ++ot) {
+#pragma unroll
+        for (int h2 = 0; h2 < 2; ++h2) {
+          const uint32_t rr = (lane >> 2) + h2 * 16, ch = (lane & 3u) * 8;
+          *reinterpret_cast<u32x4_t*>(pa + rr * kPatchRow + ch) = rin[ot][h2];
+        }
+#pragma unroll
+        for (int g = 0; g < 4; ++g) rc[ot][g] = *reinterpret_cast<const uint2*>(pa + lq * kPatchRow + g * 8 + half * 4);
+      }
 #pragma unroll
       for (int ot = 0; ot < OT; ++ot) {
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
-          uint2 pk;
-          pk.x = pack_bf16x2(acc2[ot][g * 4 + 0], acc2[ot][g * 4 + 1]);
-          pk.y = pack_bf16x2(acc2[ot][g * 4 + 2], acc2[ot][g * 4 + 3]);
-          *reinterpret_cast<uint2*>(xp1 + lq * kPatchRow + g * 8 + half * 4) = pk;
-        }
-#pragma unroll
-        for (int h2 = 0; h2 < 2; ++h2) {
-          const uint32_t rr = (lane >> 2) + h2 * 16, ch = (lane & 3u) * 8;
-          u32x4_t t = *reinterpret_cast<const u32x4_t*>(xp1 + rr * kPatchRow + ch);
-#pragma unroll
-          for (int e = 0; e < 4; ++e)
-            t[e] = pack_bf16x2(bf16_lo(t[e]) + bf16_lo(rin[ot][h2][e]), bf16_hi(t[e]) + bf16_hi(rin[ot][h2][e]));
-          *reinterpret_cast<u32x4_t*>(xp1 + rr * kPatchRow + ch) = t;
+          const uint2 bb = *reinterpret_cast<const uint2*>(bias2 + ot * 32 + g * 8 + half * 4);
+          const uint32_t p0 = pack_bf16x2(acc2[ot][g * 4 + 0], acc2[ot][g * 4 + 1]);      // the projection as a kernel of its own would store it
+          const uint32_t p1 = pack_bf16x2(acc2[ot][g * 4 + 2], acc2[ot][g * 4 + 3]);
+          uint2 x1;
+          x1.x = pack_bf16x2(bf16_lo(p0) + bf16_lo(rc[ot][g].x), bf16_hi(p0) + bf16_hi(rc[ot][g].x));
+          x1.y = pack_bf16x2(bf16_lo(p1) + bf16_lo(rc[ot][g].y), bf16_hi(p1) + bf16_hi(rc[ot][g].y));
+          *reinterpret_cast<uint2*>(pb + lq * kPatchRow + g * 8 + half * 4) = x1;
+          acc2[ot][g * 4 + 0] = bf16_lo(x1.x) + bf16_lo(bb.x); acc2[ot][g * 4 + 1] = bf16_hi(x1.x) + bf16_hi(bb.x);
+          acc2[ot][g * 4 + 2] = bf16_lo(x1.y) + bf16_lo(bb.y); acc2[ot][g * 4 + 3] = bf16_hi(x1.y) + bf16_hi(bb.y);
         }
 #pragma unroll
         for (int j = 0; j < 2; ++j)
-          xf[2 * ot + j] = *reinterpret_cast<const bf16x8_t*>(xp1 + lq * kPatchRow + j * 16 + half * 8);
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          const uint2 v = *reinterpret_cast<const uint2*>(xp1 + lq * kPatchRow + g * 8 + half * 4);
-          const uint2 bb = *reinterpret_cast<const uint2*>(bias2 + ot * 32 + g * 8 + half * 4);
-          acc2[ot][g * 4 + 0] = bf16_lo(v.x) + bf16_lo(bb.x); acc2[ot][g * 4 + 1] = bf16_hi(v.x) + bf16_hi(bb.x);
-          acc2[ot][g * 4 + 2] = bf16_lo(v.y) + bf16_lo(bb.y); acc2[ot][g * 4 + 3] = bf16_hi(v.y) + bf16_hi(bb.y);
-        }
+          xf[2 * ot + j] = *reinterpret_cast<const bf16x8_t*>(pb + lq * kPatchRow + j * 16 + half * 8);
       }
     }
   } else {
