@@ -35,8 +35,9 @@
 //
 // With the block's out-projection in front (PROJ kernels, f3d_proj_ln_mlp_swiglu_bf16; flash3dxfmr/layers/stage.py:92-102:
 // proj, residual add, MLP, residual add): x1 = a wpT + bp + x is formed in the fc2 accumulators before the LayerNorm
-// and never reaches memory; the kernel then returns x1 + MLP(LayerNorm(x1)).  482,304 rows, C = 256: 0.775 ms against
-// 0.155 + 0.70 ms for the projection kernel followed by this kernel without it.
+// (the block input enters through products with an identity) and never reaches memory; the kernel then returns
+// x1 + MLP(LayerNorm(x1)).  482,304 rows, C = 256: 0.78 ms against 0.155 + 0.70 ms for the projection kernel followed
+// by this kernel without it.
 #include <algorithm>
 
 #include "xstat_common.h"
@@ -65,7 +66,7 @@ struct MlpGeom {
   static constexpr int N_DMA2 = CH2 / 1024;
   static constexpr int NPC = K / kXsChunk;                  // 64-row chunks of the out-projection weight
   static constexpr size_t loop_bytes() { return (size_t)kMlpBufs * (CH1 + 1024 + CH2); }
-  static constexpr size_t row_patch_bytes() { return (size_t)2 * kMlpWaves * 32 * kPatchRow * 2; }   // two patches per wave
+  static constexpr size_t row_patch_bytes() { return (size_t)kMlpWaves * 32 * kPatchRow * 2; }
   // weight buffers and the b' slots of the w1 buffers; at least the prologue's transposition patches; with the
   // out-projection in front, the wave-private patches its result is re-laid through come after the weight buffers
   static constexpr size_t lds_bytes(bool proj = false) {
@@ -87,9 +88,8 @@ struct MlpProj {
 // w1p: LayerNorm-folded fc1 weight [2 H][K] (value rows then gate rows), b32: b' = b1 + w1 beta as fp32 [2 H] (mlp_prep_kernel);
 // w2p: fc2 weight, fragment-major per chunk (mlp_prep_kernel); bias2 [K] (zeros when the layer has none);
 // H: hidden width, multiple of 32.
-// PROJ: x1 = bf16(bf16(a wpT + bp) + x) is formed first (the block's out-projection with its residual, held in
-// registers only), and the kernel returns bf16(x1 + MLP(x1)): `residual` must be null, the fc2 accumulators start from
-// x1 + b2.
+// PROJ: x1 = bf16(a wpT + bp + x) is formed first (the block's out-projection with its residual, held in registers
+// only), and the kernel returns bf16(x1 + MLP(x1)): `residual` must be null, the fc2 accumulators start from x1 + b2.
 template <int K, bool PROJ>
 __global__ __launch_bounds__(64 * kMlpWaves) __attribute__((amdgpu_waves_per_eu(2, 2))) void ln_mlp_swiglu_kernel(
     const uint16_t* __restrict__ x, uint32_t ldx, float eps, const uint16_t* __restrict__ w1p,
@@ -179,29 +179,37 @@ __global__ __launch_bounds__(64 * kMlpWaves) __attribute__((amdgpu_waves_per_eu(
       for (int ks = 0; ks < KS; ++ks) xf[ks] = *reinterpret_cast<const bf16x8_t*>(ap + ks * 16);
     }
     acc2_from_bias(pj.b);
+    // a wpT: output tile 2 c + t (32 columns) from rows 32 t .. 32 t + 31 of chunk c; the MLP's first chunk is
+    // requested under the projection's last one.  The block input is added ON THE MATRIX CORE: its 32 columns of a
+    // tile, loaded straight into operand layout while the tile's products run, times a 32 x 32 identity (two
+    // k-steps; exact: one bf16 value times one, summed in fp32) land in the same accumulators, so the residual needs
+    // no re-laying and no vector arithmetic.
+    const uint32_t poff = lq * ROWB + (((half ^ G::swz(lq)) & (uint32_t)(G::CPR - 1)) << 4);
+    // identity fragments: k-step j of a tile holds its columns 16 j .. 16 j + 15; lane (lq, half) carries elements
+    // 8 half .. 8 half + 7 of output column lq's row of the identity
+    bf16x8_t idf[2];
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) idf[j][e] = (lq == (uint32_t)(16 * j + e) + 8u * half) ? (__bf16)1.0f : (__bf16)0.0f;
+    const uint16_t* xrow = x + (size_t)min(row0 + lq, M - 1) * ldx + half * 8;      // rows past M read row M - 1
+    // the block input's columns of chunk c's two tiles, requested one chunk ahead (chunk 0's before the first wait)
+    bf16x8_t xt[2][2][2];
+    auto load_xt = [&](uint32_t c) __attribute__((always_inline)) {
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) xt[c & 1u][t][j] = *reinterpret_cast<const bf16x8_t*>(xrow + (2 * c + t) * 32 + j * 16);
+    };
+    load_xt(0);
     __builtin_amdgcn_s_waitcnt(0x0F70);
     __syncthreads();
-    // a wpT: output tile 2 c + t (32 columns) from rows 32 t .. 32 t + 31 of chunk c; the MLP's first chunk is
-    // requested under the projection's last one
-    const uint32_t poff = lq * ROWB + (((half ^ G::swz(lq)) & (uint32_t)(G::CPR - 1)) << 4);
-    const uint16_t* x_wg = x + (size_t)wg_row0 * ldx;
-    u32x4_t rin[OT][2];      // the block input's pieces of the wave's rows, row-contiguous (as the epilogue reads a residual)
-    auto load_rin = [&](int ot0, int ot1) __attribute__((always_inline)) {
-#pragma unroll
-      for (int ot = ot0; ot < ot1; ++ot)
-#pragma unroll
-        for (int h2 = 0; h2 < 2; ++h2) {
-          const uint32_t rr = (lane >> 2) + h2 * 16, ch = (lane & 3u) * 8;
-          const uint32_t row = min(row0 + rr, M - 1);            // rows past M read row M - 1
-          rin[ot][h2] = *reinterpret_cast<const u32x4_t*>(x_wg + ((size_t)(row - wg_row0) * ldx + ot * 32 + ch));
-        }
-    };
     mlp_static_for<MG::NPC>([&](auto c_c) {
       constexpr uint32_t c = decltype(c_c)::value;
       if constexpr (c + 1 < (uint32_t)MG::NPC) dma_proj(c + 1);
       else dma_chunk(0);
       if (has_rows) {
-        if constexpr (c == 0) load_rin(0, OT / 2);    // spare registers take the first half right away
+        if constexpr (c + 1 < (uint32_t)MG::NPC) load_xt(c + 1);
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
           const char* sw = w1buf + (c % NB1) * MG::CH1 + t * 32 * ROWB;
@@ -215,44 +223,31 @@ __global__ __launch_bounds__(64 * kMlpWaves) __attribute__((amdgpu_waves_per_eu(
             acc2[2 * c + t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[ks], xf[ks], acc2[2 * c + t], 0, 0, 0);
           }
         }
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+          for (int j = 0; j < 2; ++j)
+            acc2[2 * c + t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(idf[j], xt[c & 1u][t][j], acc2[2 * c + t], 0, 0, 0);
       }
-      // the next chunk has landed.  In the first round the block input's pieces were requested AFTER the chunk's direct
-      // loads and may stay in flight: OT younger loads (a wave without rows has none)
-      static_assert(OT < 16, "the count fits the low bits of the wait's immediate");
-      if (c == 0 && has_rows) __builtin_amdgcn_s_waitcnt(0x0F70 | OT);
+      // the next chunk has landed; the block input's pieces requested above (4 loads, younger than the chunk's direct
+      // loads) may stay in flight
+      if (c + 1 < (uint32_t)MG::NPC && has_rows) __builtin_amdgcn_s_waitcnt(0x0F70 | 4);
       else __builtin_amdgcn_s_waitcnt(0x0F70);
       wg_barrier_lds();
     });
-    // x1 = bf16(bf16(projection) + x).  The block input's pieces arrive row-contiguous; they go through the wave's first
-    // patch into the accumulator layout (all eight tiles back to back: LDS serves a wave in order, so the next tile's
-    // writes need not wait for this tile's reads), x1 is formed in registers (also x1 + b2, what the fc2 products add
-    // to), written to the second patch in the accumulator layout and read back in operand layout (the k-steps 2 ot,
-    // 2 ot + 1 of the LayerNorm / fc1 panel), again without a wait between tiles.
+    // x1 = bf16(projection + bias + x), 32 columns at a time: written to the wave's patch in the accumulator layout
+    // and read back in operand layout (the k-steps 2 ot, 2 ot + 1 of the LayerNorm / fc1 panel), without a wait between
+    // tiles (LDS serves a wave in order); the accumulators go on as x1 + b2, what the fc2 products add to
     if (has_rows) {
-      uint16_t* pa = reinterpret_cast<uint16_t*>(lds_mlp + MG::loop_bytes()) + wave * (32 * kPatchRow);
-      uint16_t* pb = pa + WAVES * (32 * kPatchRow);
-      load_rin(OT / 2, OT);     // the attention rows are dead: their registers take the second half
-      uint2 rc[OT][4];
-#pragma unroll
-      for (int ot = 0; ot < OT; ++ot) {
-#pragma unroll
-        for (int h2 = 0; h2 < 2; ++h2) {
-          const uint32_t rr = (lane >> 2) + h2 * 16, ch = (lane & 3u) * 8;
-          *reinterpret_cast<u32x4_t*>(pa + rr * kPatchRow + ch) = rin[ot][h2];
-        }
-#pragma unroll
-        for (int g = 0; g < 4; ++g) rc[ot][g] = *reinterpret_cast<const uint2*>(pa + lq * kPatchRow + g * 8 + half * 4);
-      }
+      uint16_t* pb = reinterpret_cast<uint16_t*>(lds_mlp + MG::loop_bytes()) + wave * (32 * kPatchRow);
 #pragma unroll
       for (int ot = 0; ot < OT; ++ot) {
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
           const uint2 bb = *reinterpret_cast<const uint2*>(bias2 + ot * 32 + g * 8 + half * 4);
-          const uint32_t p0 = pack_bf16x2(acc2[ot][g * 4 + 0], acc2[ot][g * 4 + 1]);      // the projection as a kernel of its own would store it
-          const uint32_t p1 = pack_bf16x2(acc2[ot][g * 4 + 2], acc2[ot][g * 4 + 3]);
           uint2 x1;
-          x1.x = pack_bf16x2(bf16_lo(p0) + bf16_lo(rc[ot][g].x), bf16_hi(p0) + bf16_hi(rc[ot][g].x));
-          x1.y = pack_bf16x2(bf16_lo(p1) + bf16_lo(rc[ot][g].y), bf16_hi(p1) + bf16_hi(rc[ot][g].y));
+          x1.x = pack_bf16x2(acc2[ot][g * 4 + 0], acc2[ot][g * 4 + 1]);
+          x1.y = pack_bf16x2(acc2[ot][g * 4 + 2], acc2[ot][g * 4 + 3]);
           *reinterpret_cast<uint2*>(pb + lq * kPatchRow + g * 8 + half * 4) = x1;
           acc2[ot][g * 4 + 0] = bf16_lo(x1.x) + bf16_lo(bb.x); acc2[ot][g * 4 + 1] = bf16_hi(x1.x) + bf16_hi(bb.x);
           acc2[ot][g * 4 + 2] = bf16_lo(x1.y) + bf16_lo(bb.y); acc2[ot][g * 4 + 3] = bf16_hi(x1.y) + bf16_hi(bb.y);
