@@ -465,16 +465,19 @@ __global__ __launch_bounds__(64 * kMlpWaves) __attribute__((amdgpu_waves_per_eu(
 constexpr int kMlpSmallWaves = 8;
 
 template <int K>
-__host__ __device__ constexpr size_t mlp_small_lds_bytes(uint32_t H) {
-  return (size_t)(H / 32) * (64 * K * 2 + K * 64 + 1024) + (size_t)kMlpSmallWaves * 32 * (K + 8) * 2;
+__host__ __device__ constexpr size_t mlp_small_lds_bytes(uint32_t H, bool proj = false) {
+  return (size_t)(H / 32) * (64 * K * 2 + K * 64 + 1024) + (size_t)kMlpSmallWaves * 32 * (K + 8) * 2 + (proj ? (size_t)K * K * 2 : 0);
 }
 
-template <int K>
+// PROJ: as in the streaming kernel, x1 = bf16(a wpT + bp + x) is formed per tile in front of the LayerNorm (the
+// projection weight sits in LDS with the others, the block input enters through products with an identity) and the
+// kernel returns bf16(x1 + MLP(x1)); `residual` must be null.
+template <int K, bool PROJ>
 __global__ __launch_bounds__(64 * kMlpSmallWaves) void ln_mlp_swiglu_small_kernel(
     const uint16_t* __restrict__ x, uint32_t ldx, float eps, const uint16_t* __restrict__ w1p,
     const float* __restrict__ b32, const uint16_t* __restrict__ w2p, const uint16_t* __restrict__ bias2,
     const uint16_t* __restrict__ residual, uint32_t ldr, uint16_t* __restrict__ y, uint32_t ldy, uint32_t M,
-    uint32_t H) {
+    uint32_t H, MlpProj pj) {
   using G = XsGeom<K>;
   constexpr int KS = K / 16, ROWB = G::ROWB, WAVES = kMlpSmallWaves, OT = K / 32;
   constexpr int CH1 = 64 * ROWB, CH2 = K * 64, N2 = CH2 / 1024, PROW = K + 8, PCPR = K / 8;
@@ -488,9 +491,17 @@ __global__ __launch_bounds__(64 * kMlpSmallWaves) void ln_mlp_swiglu_small_kerne
   const uint32_t tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid / kWave), lane = tid % kWave;
   const uint32_t lq = lane & 31u, half = lane >> 5;
   uint16_t* patch = reinterpret_cast<uint16_t*>(s_side + (size_t)nchunk * 1024) + wave * (32 * PROW);
+  char* wpbuf = s_side + (size_t)nchunk * 1024 + (size_t)WAVES * 32 * PROW * 2;    // PROJ: the projection weight, laid out like a w1 chunk
 
   // ---- every weight of the layer -> LDS, the direct loads dealt out over the waves ----
   {
+    if constexpr (PROJ) {
+      constexpr uint32_t NP = (uint32_t)K * K * 2 / 1024;
+      for (uint32_t j = wave; j < NP; j += WAVES) {
+        const uint32_t r = (j * 64u + lane) / G::CPR, pc = lane % G::CPR;
+        xs_lds_dma16(pj.w, (r * K + (pc ^ G::swz(r)) * 8u) * 2u, wpbuf + j * 1024);
+      }
+    }
     constexpr uint32_t per = G::N_DMA + N2 + 1;
     for (uint32_t pi = wave; pi < nchunk * per; pi += WAVES) {
       const uint32_t c = pi / per, j = pi % per;
@@ -516,15 +527,25 @@ __global__ __launch_bounds__(64 * kMlpSmallWaves) void ln_mlp_swiglu_small_kerne
   // current one is computed
   constexpr int XLOADS = (32 * PCPR) / kWave;
   u32x4_t xv[XLOADS];
+  const uint16_t* const panel = PROJ ? pj.a : x;         // what the tile's operand rows are read from
+  const uint32_t ld_panel = PROJ ? pj.lda : ldx;
   auto request_x = [&](uint32_t tile) __attribute__((always_inline)) {
 #pragma unroll
     for (int i = 0; i < XLOADS; ++i) {
       const uint32_t id = lane + i * kWave;
       const uint32_t rr = id / PCPR, kc = (id % PCPR) * 8;
       const uint32_t r = min(tile * 32 + rr, M - 1);
-      xv[i] = *reinterpret_cast<const u32x4_t*>(x + (size_t)r * ldx + kc);
+      xv[i] = *reinterpret_cast<const u32x4_t*>(panel + (size_t)r * ld_panel + kc);
     }
   };
+  // PROJ: identity fragments (k-step j of a 32-column tile holds its columns 16 j .. 16 j + 15) and the lane's offset
+  // into a 32-row block of the projection weight
+  bf16x8_t idf[2];
+#pragma unroll
+  for (int j = 0; j < 2; ++j)
+#pragma unroll
+    for (int e = 0; e < 8; ++e) idf[j][e] = (lq == (uint32_t)(16 * j + e) + 8u * half) ? (__bf16)1.0f : (__bf16)0.0f;
+  const uint32_t poff = lq * ROWB + (((half ^ G::swz(lq)) & (uint32_t)(G::CPR - 1)) << 4);
   const uint32_t tile_step = gridDim.x * WAVES;
   if (blockIdx.x * WAVES + wave < ntiles) request_x(blockIdx.x * WAVES + wave);
   for (uint32_t tile = blockIdx.x * WAVES + wave; tile < ntiles; tile += tile_step) {
@@ -541,6 +562,50 @@ __global__ __launch_bounds__(64 * kMlpSmallWaves) void ln_mlp_swiglu_small_kerne
     for (int ks = 0; ks < KS; ++ks)
       xf[ks] = *reinterpret_cast<const bf16x8_t*>(patch + lq * PROW + ks * 16 + half * 8);
     if (tile + tile_step < ntiles) request_x(tile + tile_step);
+    f32x16_t acc2[OT];
+    if constexpr (PROJ) {
+      // the block input's columns in operand layout, requested now; a wpT + bp; + x through the identity; x1 through
+      // the wave's patch into operand layout; the accumulators go on as x1 + b2
+      bf16x8_t xt[OT][2];
+      const uint16_t* xrow = x + (size_t)min(row0 + lq, M - 1) * ldx + half * 8;
+#pragma unroll
+      for (int ot = 0; ot < OT; ++ot)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) xt[ot][j] = *reinterpret_cast<const bf16x8_t*>(xrow + ot * 32 + j * 16);
+#pragma unroll
+      for (int ot = 0; ot < OT; ++ot) {
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const uint2 bb = *reinterpret_cast<const uint2*>(pj.b + ot * 32 + g * 8 + half * 4);
+          acc2[ot][g * 4 + 0] = bf16_lo(bb.x); acc2[ot][g * 4 + 1] = bf16_hi(bb.x);
+          acc2[ot][g * 4 + 2] = bf16_lo(bb.y); acc2[ot][g * 4 + 3] = bf16_hi(bb.y);
+        }
+        const char* sw = wpbuf + ot * 32 * ROWB;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+          const bf16x8_t wf = *reinterpret_cast<const bf16x8_t*>(sw + (poff ^ (uint32_t)(ks * 32)));
+          acc2[ot] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf, xf[ks], acc2[ot], 0, 0, 0);
+        }
+      }
+#pragma unroll
+      for (int ot = 0; ot < OT; ++ot) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) acc2[ot] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(idf[j], xt[ot][j], acc2[ot], 0, 0, 0);
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const uint2 bb = *reinterpret_cast<const uint2*>(bias2 + ot * 32 + g * 8 + half * 4);
+          uint2 x1;
+          x1.x = pack_bf16x2(acc2[ot][g * 4 + 0], acc2[ot][g * 4 + 1]);
+          x1.y = pack_bf16x2(acc2[ot][g * 4 + 2], acc2[ot][g * 4 + 3]);
+          *reinterpret_cast<uint2*>(patch + lq * kPatchRow + g * 8 + half * 4) = x1;
+          acc2[ot][g * 4 + 0] = bf16_lo(x1.x) + bf16_lo(bb.x); acc2[ot][g * 4 + 1] = bf16_hi(x1.x) + bf16_hi(bb.x);
+          acc2[ot][g * 4 + 2] = bf16_lo(x1.y) + bf16_lo(bb.y); acc2[ot][g * 4 + 3] = bf16_hi(x1.y) + bf16_hi(bb.y);
+        }
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+          xf[2 * ot + j] = *reinterpret_cast<const bf16x8_t*>(patch + lq * kPatchRow + j * 16 + half * 8);
+      }
+    }
     // the residual rows of the tile, requested now, used at the end
     u32x4_t rres[OT][2];
     if (residual) {
@@ -579,15 +644,16 @@ __global__ __launch_bounds__(64 * kMlpSmallWaves) void ln_mlp_swiglu_small_kerne
       }
     }
     // fc2 accumulators start from the bias: acc2[ot][g*4+r] <-> output column ot*32 + g*8 + half*4 + r of row lq
-    f32x16_t acc2[OT];
+    if constexpr (!PROJ) {
 #pragma unroll
-    for (int ot = 0; ot < OT; ++ot)
+      for (int ot = 0; ot < OT; ++ot)
 #pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        const uint2 bb = *reinterpret_cast<const uint2*>(bias2 + ot * 32 + g * 8 + half * 4);
-        acc2[ot][g * 4 + 0] = bf16_lo(bb.x); acc2[ot][g * 4 + 1] = bf16_hi(bb.x);
-        acc2[ot][g * 4 + 2] = bf16_lo(bb.y); acc2[ot][g * 4 + 3] = bf16_hi(bb.y);
-      }
+        for (int g = 0; g < 4; ++g) {
+          const uint2 bb = *reinterpret_cast<const uint2*>(bias2 + ot * 32 + g * 8 + half * 4);
+          acc2[ot][g * 4 + 0] = bf16_lo(bb.x); acc2[ot][g * 4 + 1] = bf16_hi(bb.x);
+          acc2[ot][g * 4 + 2] = bf16_lo(bb.y); acc2[ot][g * 4 + 3] = bf16_hi(bb.y);
+        }
+    }
     for (uint32_t c = 0; c < nchunk; ++c) {
 #pragma unroll
       for (int h = 0; h < 2; ++h) {
@@ -704,11 +770,12 @@ static int launch_mlp(const uint16_t* x, uint32_t ldx, float eps, const uint16_t
 }
 
 
-template <int K>
+template <int K, bool PROJ = false>
 static int launch_mlp_small(const uint16_t* x, uint32_t ldx, float eps, const uint16_t* w1p, const float* b32,
                             const uint16_t* w2p, const uint16_t* bias2, const uint16_t* residual, uint32_t ldr,
-                            uint16_t* y, uint32_t ldy, uint32_t M, uint32_t H, int device, hipStream_t s) {
-  const size_t lds = mlp_small_lds_bytes<K>(H);
+                            uint16_t* y, uint32_t ldy, uint32_t M, uint32_t H, int device, hipStream_t s,
+                            MlpProj pj = MlpProj{}) {
+  const size_t lds = mlp_small_lds_bytes<K>(H, PROJ);
   static int cus[64] = {};
   static size_t attr_lds[64] = {};
   int n_cu = 256;
@@ -716,7 +783,7 @@ static int launch_mlp_small(const uint16_t* x, uint32_t ldx, float eps, const ui
     if (!cus[device]) F3D_CHECK_HIP(hipDeviceGetAttribute(&cus[device], hipDeviceAttributeMultiprocessorCount, device));
     n_cu = cus[device];
   }
-  auto kern = ln_mlp_swiglu_small_kernel<K>;
+  auto kern = ln_mlp_swiglu_small_kernel<K, PROJ>;
   if (device < 0 || device >= 64 || attr_lds[device] < lds) {
     F3D_CHECK_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     if (device >= 0 && device < 64) attr_lds[device] = lds;
@@ -725,7 +792,7 @@ static int launch_mlp_small(const uint16_t* x, uint32_t ldx, float eps, const ui
   const uint32_t per_cu = (uint32_t)std::max<size_t>(1, std::min<size_t>(4, (160 * 1024) / lds));
   const uint32_t wgs = std::min<uint32_t>(cdiv_u32(cdiv_u32(M, 32), kMlpSmallWaves), (uint32_t)n_cu * per_cu);
   hipLaunchKernelGGL(kern, dim3(wgs), dim3(64 * kMlpSmallWaves), lds, s, x, ldx, eps, w1p, b32, w2p, bias2, residual, ldr,
-                     y, ldy, M, H);
+                     y, ldy, M, H, pj);
   return F3D_OK;
 }
 
@@ -791,9 +858,12 @@ int f3d_proj_ln_mlp_swiglu_bf16(const f3d_bf16_t* a, uint32_t lda, const f3d_bf1
   using namespace f3d;
   StagedWeightsScope staged;
   F3D_CHECK_ARG(a && w_proj && x && gamma && w1 && w2 && y, "null tensor pointer");
-  if (!(c == 128 || c == 256) || hidden == 0 || hidden % 32 != 0 || (uint64_t)hidden * c * 4 >= (1ull << 32)) {
-    set_error("No out-projection + MLP kernel for width %u with hidden width %u (widths 128 and 256, hidden a multiple of 32)",
-              c, hidden);
+  const bool narrow = c == 32 || c == 64;
+  if (!(narrow || c == 128 || c == 256) || hidden == 0 || hidden % 32 != 0 || (uint64_t)hidden * c * 4 >= (1ull << 32) ||
+      (c == 32 && mlp_small_lds_bytes<32>(hidden, true) > 160 * 1024) ||
+      (c == 64 && mlp_small_lds_bytes<64>(hidden, true) > 160 * 1024)) {
+    set_error("No out-projection + MLP kernel for width %u with hidden width %u (widths 128 and 256 with hidden a multiple "
+              "of 32; widths 32 and 64 while all weights fit into LDS)", c, hidden);
     return F3D_ERR_UNSUPPORTED;
   }
   F3D_CHECK_ARG(lda >= c && lda % 8 == 0 && ldx >= c && ldx % 8 == 0 && ldy >= c && ldy % 8 == 0,
@@ -824,6 +894,8 @@ int f3d_proj_ln_mlp_swiglu_bf16(const f3d_bf16_t* a, uint32_t lda, const f3d_bf1
   const MlpProj pj{a, lda, w_proj, b_proj ? b_proj : zero_bias};
   int rc;
   if (c == 256) rc = launch_mlp<256, true>(x, ldx, eps, w1p, b32, w2p, b2, nullptr, 0, y, ldy, m, hidden, device, s, pj);
+  else if (c == 32) rc = launch_mlp_small<32, true>(x, ldx, eps, w1p, b32, w2p, b2, nullptr, 0, y, ldy, m, hidden, device, s, pj);
+  else if (c == 64) rc = launch_mlp_small<64, true>(x, ldx, eps, w1p, b32, w2p, b2, nullptr, 0, y, ldy, m, hidden, device, s, pj);
   else rc = launch_mlp<128, true>(x, ldx, eps, w1p, b32, w2p, b2, nullptr, 0, y, ldy, m, hidden, device, s, pj);
   if (rc != F3D_OK) return rc;
   F3D_CHECK_HIP(hipGetLastError());

@@ -416,7 +416,7 @@ class LayerNorm(_CachedParamModule):
 
 FUSABLE_LN_WIDTHS = (32, 64, 128, 256, 512)
 FUSED_MLP_WIDTHS = (32, 64, 128, 256)      # widths the one-kernel gated MLP covers (32 / 64: while the weights fit into LDS)
-PROJ_MLP_WIDTHS = (128, 256)               # widths at which it also takes the out-projection and its residual in front
+PROJ_MLP_WIDTHS = (32, 64, 128, 256)       # widths at which it also takes the out-projection and its residual in front
 
 
 def is_fusable_layernorm(norm, width: int) -> bool:
@@ -566,7 +566,7 @@ class LayerNormMLP(_CachedParamModule):
         if (torch.is_grad_enabled() or self.activation != "swiglu" or self.hidden_size not in PROJ_MLP_WIDTHS
                 or self.ffn_hidden_size % 32 != 0 or self.fused is False or proj.in_features != self.hidden_size
                 or proj.out_features != self.hidden_size or not a.is_cuda or a.dtype != torch.bfloat16
-                or x.dtype != torch.bfloat16 or a.shape[0] < 30000):
+                or x.dtype != torch.bfloat16 or (self.hidden_size == 256 and a.shape[0] < 30000)):
             return None
         a2, x2 = a.reshape(-1, self.hidden_size), x.reshape(-1, self.hidden_size)
         if a2.stride(1) != 1 or x2.stride(1) != 1:

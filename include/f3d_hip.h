@@ -325,8 +325,9 @@ int f3d_ln_mlp_swiglu_bf16(const f3d_bf16_t* x, uint32_t ldx, const f3d_bf16_t* 
  *   x1 = a w_projT + b_proj + x,   y = x1 + MLP(LayerNorm(x1))   with the MLP of f3d_ln_mlp_swiglu_bf16.
  * a [m,c] (row stride lda) is the attention output, x [m,c] (row stride ldx) the block input, w_proj [c,c], b_proj [c]
  * or NULL; the other arguments as in f3d_ln_mlp_swiglu_bf16 (no residual argument: x1 is the residual).  x1 is rounded
- * to bf16 once, from the fp32 sum, and is held in registers only.  c in {128, 256}, hidden a
- * multiple of 32; anything else returns F3D_ERR_UNSUPPORTED without touching y (use f3d_linear_bf16 with the residual,
+ * to bf16 once, from the fp32 sum, and is held in registers only.  c in {128, 256} with hidden a multiple of 32, or
+ * c in {32, 64} while all weights fit into LDS (as for f3d_ln_mlp_swiglu_bf16, with c * c * 2 bytes more); anything else
+ * returns F3D_ERR_UNSUPPORTED without touching y (use f3d_linear_bf16 with the residual,
  * then f3d_ln_mlp_swiglu_bf16).  Inference only: no backward consumes its result. */
 int f3d_proj_ln_mlp_swiglu_bf16(const f3d_bf16_t* a, uint32_t lda, const f3d_bf16_t* w_proj, const f3d_bf16_t* b_proj,
                                 const f3d_bf16_t* x, uint32_t ldx, const f3d_bf16_t* gamma, const f3d_bf16_t* beta, float eps,

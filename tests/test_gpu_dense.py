@@ -241,6 +241,10 @@ def test_fused_mlp_matches_two_kernel_path(oracle, M, C, H, use_res, use_bias):
     (300, 256, 32, True),          # a single hidden chunk behind the projection
     (70000, 128, 256, True),       # many workgroups
     (66000, 256, 64, True),        # more panels than CUs: shorter panels in the last turn
+    (5000, 32, 128, True),         # narrow layers: the projection weight resident in LDS with the others
+    (100000, 64, 256, True),       # ... more tiles than resident waves
+    (333, 64, 64, False),          # ... ragged M, no biases
+    (40, 32, 512, True),           # ... fewer rows than one workgroup's waves
 ])
 def test_proj_residual_mlp_in_one_kernel(oracle, M, C, H, use_bias):
     """out-projection + residual + gated MLP + residual in one kernel against (a) the projection kernel followed by the
@@ -289,9 +293,14 @@ def test_proj_residual_mlp_unsupported_width_is_reported():
     from flash3dtransformer_amd.lib import pshattn
     mk = lambda *s: torch.zeros(*s, dtype=torch.bfloat16, device=DEV)
     y = torch.full((64, 64), 3.0, dtype=torch.bfloat16, device=DEV)
-    assert not pshattn.proj_ln_mlp_swiglu_bf16(mk(64, 64), mk(64, 64), None, mk(64, 64), mk(64), mk(64), 1e-5, mk(256, 64),
-                                               None, mk(64, 128), None, y)
+    # C = 64 with a hidden width whose weights do not fit into LDS; C = 512
+    assert not pshattn.proj_ln_mlp_swiglu_bf16(mk(64, 64), mk(64, 64), None, mk(64, 64), mk(64), mk(64), 1e-5, mk(640, 64),
+                                               None, mk(64, 320), None, y)
     assert (y == 3.0).all()
+    y5 = torch.full((64, 512), 3.0, dtype=torch.bfloat16, device=DEV)
+    assert not pshattn.proj_ln_mlp_swiglu_bf16(mk(64, 512), mk(512, 512), None, mk(64, 512), mk(512), mk(512), 1e-5,
+                                               mk(128, 512), None, mk(512, 64), None, y5)
+    assert (y5 == 3.0).all()
 
 
 def test_fused_mlp_unsupported_width_is_reported():
