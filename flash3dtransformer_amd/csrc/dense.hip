@@ -347,7 +347,8 @@ __global__ __launch_bounds__(256) void affine_act_kernel(const uint16_t* __restr
 
 int launch_xstat_linear(const uint16_t* x, uint32_t ldx, const uint16_t* gamma, const uint16_t* beta, float eps,
                         const uint16_t* w, const uint16_t* bias, const uint16_t* residual, uint32_t ldr, uint16_t* y,
-                        uint32_t ldy, uint32_t M, uint32_t N, uint32_t K, uint32_t act, int device, hipStream_t s);
+                        uint32_t ldy, uint32_t M, uint32_t N, uint32_t K, uint32_t act, int device, hipStream_t s,
+                        const uint16_t* coord = nullptr, const uint16_t* etab = nullptr);
 // output-panel kernel for long inner dimensions and 128 / 256 outputs (ystat_linear.hip); F3D_ERR_UNSUPPORTED otherwise
 int launch_ystat_linear(const uint16_t* x, uint32_t ldx, const uint16_t* w, const uint16_t* bias,
                         const uint16_t* residual, uint32_t ldr, uint16_t* y, uint32_t ldy, uint32_t M, uint32_t N,
@@ -440,6 +441,33 @@ int f3d_ln_linear_bf16(const f3d_bf16_t* x, uint32_t ldx, const f3d_bf16_t* gamm
     launch_layernorm(x, gamma, beta, tmp, m, k, eps, s);
     rc = launch_gemm(false, tmp, k, w, k, bias, residual, ldr, y, ldy, m, n, k, act, s);
   }
+  if (rc != F3D_OK) return rc;
+  F3D_CHECK_HIP(hipGetLastError());
+  return F3D_OK;
+}
+
+int f3d_embed_ln_linear_bf16(const f3d_half_t* coord, const f3d_bf16_t* embed_table, const f3d_bf16_t* gamma,
+                             const f3d_bf16_t* beta, float eps, const f3d_bf16_t* w, const f3d_bf16_t* bias, f3d_bf16_t* y,
+                             uint32_t ldy, uint32_t m, uint32_t n, uint32_t k, int device, void* stream) {
+  using namespace f3d;
+  StagedWeightsScope staged;
+  F3D_CHECK_ARG(coord && embed_table && gamma && w && y, "null tensor pointer");
+  if (!(k == 32 || k == 64 || k == 128 || k == 256) || n % 32 != 0) {
+    set_error("No embedding + LayerNorm + Linear kernel for width %u with %u outputs (widths 32, 64, 128, 256; outputs a "
+              "multiple of 32)", k, n);
+    return F3D_ERR_UNSUPPORTED;
+  }
+  F3D_CHECK_ARG(ldy >= n && ldy % 8 == 0, "row stride must be aligned and cover a row (ldy=%u)", ldy);
+  F3D_CHECK_ARG((((uintptr_t)embed_table | (uintptr_t)w | (uintptr_t)y | (uintptr_t)gamma | (uintptr_t)beta) & 15u) == 0 &&
+                    ((uintptr_t)coord & 1u) == 0,
+                "embed_table/w/y/gamma/beta must be 16-byte aligned");
+  if (m == 0) return F3D_OK;
+  DeviceGuard guard(device);
+  F3D_CHECK_ARG(guard.ok, "cannot select device %d", device);
+  hipStream_t s = (hipStream_t)stream;
+  SyncBracket sync(s);
+  const int rc = launch_xstat_linear(nullptr, 0, gamma, beta, eps, w, bias, nullptr, 0, y, ldy, m, n, k, F3D_ACT_NONE, device,
+                                     s, coord, embed_table);
   if (rc != F3D_OK) return rc;
   F3D_CHECK_HIP(hipGetLastError());
   return F3D_OK;

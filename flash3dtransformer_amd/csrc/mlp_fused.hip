@@ -78,19 +78,40 @@ struct MlpGeom {
 
 // The out-projection in front of the MLP (PROJ kernels): a [M][K] are the attention output rows, w [K][K] / b [K] the
 // projection's weight and bias; the kernel's x is then the block input that the projection's result is added to.
+// EMBED kernels: the block input is not read but formed: it is the coordinate embedding of the rows' points (coord fp16
+// [M][3]; etab bf16 [K][8] = (wx, wy, wz, b, 0, 0, 0, 0) per channel), one product per 32 channels into the accumulators.
 struct MlpProj {
   const uint16_t* a;
   uint32_t lda;
   const uint16_t* w;
   const uint16_t* b;
+  const uint16_t* coord;
+  const uint16_t* etab;
 };
+
+// the rows' (x, y, z, 1) as the B operand of the embedding product: lane (lq, half = 0) carries row lq's four values
+__device__ __forceinline__ bf16x8_t embed_rows_operand(const uint16_t* coord, uint32_t row, uint32_t half) {
+  u32x4_t cb = {0u, 0u, 0u, 0u};
+  if (half == 0) {
+    const uint16_t* cp = coord + (size_t)row * 3;
+    cb[0] = pack_bf16x2(half_bits_to_float(cp[0]), half_bits_to_float(cp[1]));
+    cb[1] = pack_bf16x2(half_bits_to_float(cp[2]), 1.0f);
+  }
+  return __builtin_bit_cast(bf16x8_t, cb);
+}
+// the (wx, wy, wz, b) of channels 32 tile + lq as the A operand
+__device__ __forceinline__ bf16x8_t embed_channels_operand(const uint16_t* etab, uint32_t tile, uint32_t lq, uint32_t half) {
+  u32x4_t ea = {0u, 0u, 0u, 0u};
+  if (half == 0) ea = *reinterpret_cast<const u32x4_t*>(etab + (size_t)(tile * 32 + lq) * 8);
+  return __builtin_bit_cast(bf16x8_t, ea);
+}
 
 // w1p: LayerNorm-folded fc1 weight [2 H][K] (value rows then gate rows), b32: b' = b1 + w1 beta as fp32 [2 H] (mlp_prep_kernel);
 // w2p: fc2 weight, fragment-major per chunk (mlp_prep_kernel); bias2 [K] (zeros when the layer has none);
 // H: hidden width, multiple of 32.
 // PROJ: x1 = bf16(a wpT + bp + x) is formed first (the block's out-projection with its residual, held in registers
 // only), and the kernel returns bf16(x1 + MLP(x1)): `residual` must be null, the fc2 accumulators start from x1 + b2.
-template <int K, bool PROJ>
+template <int K, bool PROJ, bool EMBED = false>
 __global__ __launch_bounds__(64 * kMlpWaves) __attribute__((amdgpu_waves_per_eu(2, 2))) void ln_mlp_swiglu_kernel(
     const uint16_t* __restrict__ x, uint32_t ldx, float eps, const uint16_t* __restrict__ w1p,
     const float* __restrict__ b32, const uint16_t* __restrict__ w2p, const uint16_t* __restrict__ bias2,
@@ -192,15 +213,21 @@ __global__ __launch_bounds__(64 * kMlpWaves) __attribute__((amdgpu_waves_per_eu(
     for (int j = 0; j < 2; ++j)
 #pragma unroll
       for (int e = 0; e < 8; ++e) idf[j][e] = (lq == (uint32_t)(16 * j + e) + 8u * half) ? (__bf16)1.0f : (__bf16)0.0f;
-    const uint16_t* xrow = x + (size_t)min(row0 + lq, M - 1) * ldx + half * 8;      // rows past M read row M - 1
+    const uint16_t* xrow = EMBED ? nullptr : x + (size_t)min(row0 + lq, M - 1) * ldx + half * 8;      // rows past M read row M - 1
     // the block input's columns of chunk c's two tiles, requested one chunk ahead (chunk 0's before the first wait)
     bf16x8_t xt[2][2][2];
     auto load_xt = [&](uint32_t c) __attribute__((always_inline)) {
+      if constexpr (!EMBED) {
 #pragma unroll
-      for (int t = 0; t < 2; ++t)
+        for (int t = 0; t < 2; ++t)
 #pragma unroll
-        for (int j = 0; j < 2; ++j) xt[c & 1u][t][j] = *reinterpret_cast<const bf16x8_t*>(xrow + (2 * c + t) * 32 + j * 16);
+          for (int j = 0; j < 2; ++j) xt[c & 1u][t][j] = *reinterpret_cast<const bf16x8_t*>(xrow + (2 * c + t) * 32 + j * 16);
+      }
     };
+    // EMBED: the block input is the embedding of the rows' coordinates: one product of a tile's channel parameters
+    // with the rows' (x, y, z, 1) per tile instead of the two identity products (fp32, not rounded to bf16 in between)
+    bf16x8_t cbe;
+    if constexpr (EMBED) cbe = embed_rows_operand(pj.coord, min(row0 + lq, M - 1), half);
     load_xt(0);
     __builtin_amdgcn_s_waitcnt(0x0F70);
     __syncthreads();
@@ -210,6 +237,11 @@ __global__ __launch_bounds__(64 * kMlpWaves) __attribute__((amdgpu_waves_per_eu(
       else dma_chunk(0);
       if (has_rows) {
         if constexpr (c + 1 < (uint32_t)MG::NPC) load_xt(c + 1);
+        bf16x8_t eat[2];
+        if constexpr (EMBED) {
+#pragma unroll
+          for (int t = 0; t < 2; ++t) eat[t] = embed_channels_operand(pj.etab, 2 * c + t, lq, half);
+        }
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
           const char* sw = w1buf + (c % NB1) * MG::CH1 + t * 32 * ROWB;
@@ -224,14 +256,19 @@ __global__ __launch_bounds__(64 * kMlpWaves) __attribute__((amdgpu_waves_per_eu(
           }
         }
 #pragma unroll
-        for (int t = 0; t < 2; ++t)
+        for (int t = 0; t < 2; ++t) {
+          if constexpr (EMBED) {
+            acc2[2 * c + t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(eat[t], cbe, acc2[2 * c + t], 0, 0, 0);
+          } else {
 #pragma unroll
-          for (int j = 0; j < 2; ++j)
-            acc2[2 * c + t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(idf[j], xt[c & 1u][t][j], acc2[2 * c + t], 0, 0, 0);
+            for (int j = 0; j < 2; ++j)
+              acc2[2 * c + t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(idf[j], xt[c & 1u][t][j], acc2[2 * c + t], 0, 0, 0);
+          }
+        }
       }
       // the next chunk has landed; the block input's pieces requested above (4 loads, younger than the chunk's direct
       // loads) may stay in flight
-      if (c + 1 < (uint32_t)MG::NPC && has_rows) __builtin_amdgcn_s_waitcnt(0x0F70 | 4);
+      if (!EMBED && c + 1 < (uint32_t)MG::NPC && has_rows) __builtin_amdgcn_s_waitcnt(0x0F70 | 4);
       else __builtin_amdgcn_s_waitcnt(0x0F70);
       wg_barrier_lds();
     });
@@ -472,7 +509,7 @@ __host__ __device__ constexpr size_t mlp_small_lds_bytes(uint32_t H, bool proj =
 // PROJ: as in the streaming kernel, x1 = bf16(a wpT + bp + x) is formed per tile in front of the LayerNorm (the
 // projection weight sits in LDS with the others, the block input enters through products with an identity) and the
 // kernel returns bf16(x1 + MLP(x1)); `residual` must be null.
-template <int K, bool PROJ>
+template <int K, bool PROJ, bool EMBED = false>
 __global__ __launch_bounds__(64 * kMlpSmallWaves) void ln_mlp_swiglu_small_kernel(
     const uint16_t* __restrict__ x, uint32_t ldx, float eps, const uint16_t* __restrict__ w1p,
     const float* __restrict__ b32, const uint16_t* __restrict__ w2p, const uint16_t* __restrict__ bias2,
@@ -566,12 +603,18 @@ __global__ __launch_bounds__(64 * kMlpSmallWaves) void ln_mlp_swiglu_small_kerne
     if constexpr (PROJ) {
       // the block input's columns in operand layout, requested now; a wpT + bp; + x through the identity; x1 through
       // the wave's patch into operand layout; the accumulators go on as x1 + b2
-      bf16x8_t xt[OT][2];
-      const uint16_t* xrow = x + (size_t)min(row0 + lq, M - 1) * ldx + half * 8;
+      bf16x8_t xt[OT][2], eat[OT], cbe;
+      if constexpr (EMBED) {
+        cbe = embed_rows_operand(pj.coord, min(row0 + lq, M - 1), half);
 #pragma unroll
-      for (int ot = 0; ot < OT; ++ot)
+        for (int ot = 0; ot < OT; ++ot) eat[ot] = embed_channels_operand(pj.etab, ot, lq, half);
+      } else {
+        const uint16_t* xrow = x + (size_t)min(row0 + lq, M - 1) * ldx + half * 8;
 #pragma unroll
-        for (int j = 0; j < 2; ++j) xt[ot][j] = *reinterpret_cast<const bf16x8_t*>(xrow + ot * 32 + j * 16);
+        for (int ot = 0; ot < OT; ++ot)
+#pragma unroll
+          for (int j = 0; j < 2; ++j) xt[ot][j] = *reinterpret_cast<const bf16x8_t*>(xrow + ot * 32 + j * 16);
+      }
 #pragma unroll
       for (int ot = 0; ot < OT; ++ot) {
 #pragma unroll
@@ -589,8 +632,12 @@ __global__ __launch_bounds__(64 * kMlpSmallWaves) void ln_mlp_swiglu_small_kerne
       }
 #pragma unroll
       for (int ot = 0; ot < OT; ++ot) {
+        if constexpr (EMBED) {
+          acc2[ot] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(eat[ot], cbe, acc2[ot], 0, 0, 0);
+        } else {
 #pragma unroll
-        for (int j = 0; j < 2; ++j) acc2[ot] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(idf[j], xt[ot][j], acc2[ot], 0, 0, 0);
+          for (int j = 0; j < 2; ++j) acc2[ot] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(idf[j], xt[ot][j], acc2[ot], 0, 0, 0);
+        }
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
           const uint2 bb = *reinterpret_cast<const uint2*>(bias2 + ot * 32 + g * 8 + half * 4);
@@ -735,14 +782,14 @@ __global__ __launch_bounds__(256) void mlp_prep_kernel(const uint16_t* __restric
 }
 
 
-template <int K, bool PROJ = false>
+template <int K, bool PROJ = false, bool EMBED = false>
 static int launch_mlp(const uint16_t* x, uint32_t ldx, float eps, const uint16_t* w1p, const float* b32,
                            const uint16_t* w2p, const uint16_t* bias2, const uint16_t* residual, uint32_t ldr, uint16_t* y,
                            uint32_t ldy, uint32_t M, uint32_t H, int device, hipStream_t s, MlpProj pj = MlpProj{}) {
   constexpr size_t lds = MlpGeom<K>::lds_bytes(PROJ);
   static_assert(lds <= 160 * 1024, "chunk buffers exceed the LDS of a compute unit");
   static bool attr_set[64] = {};
-  auto kern = ln_mlp_swiglu_kernel<K, PROJ>;
+  auto kern = ln_mlp_swiglu_kernel<K, PROJ, EMBED>;
   if (device < 0 || device >= 64 || !attr_set[device]) {
     F3D_CHECK_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     if (device >= 0 && device < 64) attr_set[device] = true;
@@ -770,7 +817,7 @@ static int launch_mlp(const uint16_t* x, uint32_t ldx, float eps, const uint16_t
 }
 
 
-template <int K, bool PROJ = false>
+template <int K, bool PROJ = false, bool EMBED = false>
 static int launch_mlp_small(const uint16_t* x, uint32_t ldx, float eps, const uint16_t* w1p, const float* b32,
                             const uint16_t* w2p, const uint16_t* bias2, const uint16_t* residual, uint32_t ldr,
                             uint16_t* y, uint32_t ldy, uint32_t M, uint32_t H, int device, hipStream_t s,
@@ -783,7 +830,7 @@ static int launch_mlp_small(const uint16_t* x, uint32_t ldx, float eps, const ui
     if (!cus[device]) F3D_CHECK_HIP(hipDeviceGetAttribute(&cus[device], hipDeviceAttributeMultiprocessorCount, device));
     n_cu = cus[device];
   }
-  auto kern = ln_mlp_swiglu_small_kernel<K, PROJ>;
+  auto kern = ln_mlp_swiglu_small_kernel<K, PROJ, EMBED>;
   if (device < 0 || device >= 64 || attr_lds[device] < lds) {
     F3D_CHECK_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     if (device >= 0 && device < 64) attr_lds[device] = lds;
@@ -850,14 +897,16 @@ int f3d_ln_mlp_swiglu_bf16(const f3d_bf16_t* x, uint32_t ldx, const f3d_bf16_t* 
   return F3D_OK;
 }
 
-int f3d_proj_ln_mlp_swiglu_bf16(const f3d_bf16_t* a, uint32_t lda, const f3d_bf16_t* w_proj, const f3d_bf16_t* b_proj,
-                                const f3d_bf16_t* x, uint32_t ldx, const f3d_bf16_t* gamma, const f3d_bf16_t* beta, float eps,
-                                const f3d_bf16_t* w1, const f3d_bf16_t* b1, const f3d_bf16_t* w2, const f3d_bf16_t* b2,
-                                f3d_bf16_t* y, uint32_t ldy, uint32_t m, uint32_t c, uint32_t hidden, int device,
-                                void* stream) {
+// x != NULL: the block input is read; else coord / embed_table say how it is formed
+static int proj_ln_mlp_impl(const f3d_bf16_t* a, uint32_t lda, const f3d_bf16_t* w_proj, const f3d_bf16_t* b_proj,
+                            const f3d_bf16_t* x, uint32_t ldx, const f3d_half_t* coord, const f3d_bf16_t* embed_table,
+                            const f3d_bf16_t* gamma, const f3d_bf16_t* beta, float eps, const f3d_bf16_t* w1,
+                            const f3d_bf16_t* b1, const f3d_bf16_t* w2, const f3d_bf16_t* b2, f3d_bf16_t* y, uint32_t ldy,
+                            uint32_t m, uint32_t c, uint32_t hidden, int device, void* stream) {
   using namespace f3d;
   StagedWeightsScope staged;
-  F3D_CHECK_ARG(a && w_proj && x && gamma && w1 && w2 && y, "null tensor pointer");
+  const bool embed = x == nullptr;
+  F3D_CHECK_ARG(a && w_proj && (x || (coord && embed_table)) && gamma && w1 && w2 && y, "null tensor pointer");
   const bool narrow = c == 32 || c == 64;
   if (!(narrow || c == 128 || c == 256) || hidden == 0 || hidden % 32 != 0 || (uint64_t)hidden * c * 4 >= (1ull << 32) ||
       (c == 32 && mlp_small_lds_bytes<32>(hidden, true) > 160 * 1024) ||
@@ -866,11 +915,12 @@ int f3d_proj_ln_mlp_swiglu_bf16(const f3d_bf16_t* a, uint32_t lda, const f3d_bf1
               "of 32; widths 32 and 64 while all weights fit into LDS)", c, hidden);
     return F3D_ERR_UNSUPPORTED;
   }
-  F3D_CHECK_ARG(lda >= c && lda % 8 == 0 && ldx >= c && ldx % 8 == 0 && ldy >= c && ldy % 8 == 0,
+  F3D_CHECK_ARG(lda >= c && lda % 8 == 0 && (embed || (ldx >= c && ldx % 8 == 0)) && ldy >= c && ldy % 8 == 0,
                 "row strides must be aligned and cover a row (lda=%u ldx=%u ldy=%u)", lda, ldx, ldy);
-  F3D_CHECK_ARG((((uintptr_t)a | (uintptr_t)w_proj | (uintptr_t)b_proj | (uintptr_t)x | (uintptr_t)w1 | (uintptr_t)w2 |
-                  (uintptr_t)y | (uintptr_t)gamma | (uintptr_t)beta | (uintptr_t)b2) & 15u) == 0,
-                "a/w_proj/b_proj/x/w1/w2/b2/y/gamma/beta must be 16-byte aligned");
+  F3D_CHECK_ARG((((uintptr_t)a | (uintptr_t)w_proj | (uintptr_t)b_proj | (uintptr_t)x | (uintptr_t)embed_table | (uintptr_t)w1 |
+                  (uintptr_t)w2 | (uintptr_t)y | (uintptr_t)gamma | (uintptr_t)beta | (uintptr_t)b2) & 15u) == 0 &&
+                    ((uintptr_t)coord & 1u) == 0,
+                "a/w_proj/b_proj/x/embed_table/w1/w2/b2/y/gamma/beta must be 16-byte aligned");
   if (m == 0) return F3D_OK;
   DeviceGuard guard(device);
   F3D_CHECK_ARG(guard.ok, "cannot select device %d", device);
@@ -891,15 +941,45 @@ int f3d_proj_ln_mlp_swiglu_bf16(const f3d_bf16_t* a, uint32_t lda, const f3d_bf1
   if (!ready)
     hipLaunchKernelGGL(mlp_prep_kernel, dim3(fold_blocks + cdiv_u32(c * hidden / 8, 256)), dim3(256), 0, s, w1, gamma, beta, b1,
                        w1p, b32, fold_blocks, w2, w2p, zero_bias, c, hidden);
-  const MlpProj pj{a, lda, w_proj, b_proj ? b_proj : zero_bias};
+  const MlpProj pj{a, lda, w_proj, b_proj ? b_proj : zero_bias, coord, embed_table};
   int rc;
-  if (c == 256) rc = launch_mlp<256, true>(x, ldx, eps, w1p, b32, w2p, b2, nullptr, 0, y, ldy, m, hidden, device, s, pj);
-  else if (c == 32) rc = launch_mlp_small<32, true>(x, ldx, eps, w1p, b32, w2p, b2, nullptr, 0, y, ldy, m, hidden, device, s, pj);
-  else if (c == 64) rc = launch_mlp_small<64, true>(x, ldx, eps, w1p, b32, w2p, b2, nullptr, 0, y, ldy, m, hidden, device, s, pj);
-  else rc = launch_mlp<128, true>(x, ldx, eps, w1p, b32, w2p, b2, nullptr, 0, y, ldy, m, hidden, device, s, pj);
+#define F3D_PM(LAUNCH, KK)                                                                                                 \
+  rc = embed ? LAUNCH<KK, true, true>(x, ldx, eps, w1p, b32, w2p, b2, nullptr, 0, y, ldy, m, hidden, device, s, pj)        \
+             : LAUNCH<KK, true, false>(x, ldx, eps, w1p, b32, w2p, b2, nullptr, 0, y, ldy, m, hidden, device, s, pj)
+  if (c == 256) F3D_PM(launch_mlp, 256);
+  else if (c == 32) F3D_PM(launch_mlp_small, 32);
+  else if (c == 64) F3D_PM(launch_mlp_small, 64);
+  else F3D_PM(launch_mlp, 128);
+#undef F3D_PM
   if (rc != F3D_OK) return rc;
   F3D_CHECK_HIP(hipGetLastError());
   return F3D_OK;
+}
+
+int f3d_proj_ln_mlp_swiglu_bf16(const f3d_bf16_t* a, uint32_t lda, const f3d_bf16_t* w_proj, const f3d_bf16_t* b_proj,
+                                const f3d_bf16_t* x, uint32_t ldx, const f3d_bf16_t* gamma, const f3d_bf16_t* beta, float eps,
+                                const f3d_bf16_t* w1, const f3d_bf16_t* b1, const f3d_bf16_t* w2, const f3d_bf16_t* b2,
+                                f3d_bf16_t* y, uint32_t ldy, uint32_t m, uint32_t c, uint32_t hidden, int device,
+                                void* stream) {
+  if (!x) {
+    f3d::set_error("null tensor pointer");
+    return F3D_ERR_INVALID;
+  }
+  return proj_ln_mlp_impl(a, lda, w_proj, b_proj, x, ldx, nullptr, nullptr, gamma, beta, eps, w1, b1, w2, b2, y, ldy, m, c,
+                          hidden, device, stream);
+}
+
+int f3d_embed_proj_ln_mlp_swiglu_bf16(const f3d_bf16_t* a, uint32_t lda, const f3d_bf16_t* w_proj, const f3d_bf16_t* b_proj,
+                                      const f3d_half_t* coord, const f3d_bf16_t* embed_table, const f3d_bf16_t* gamma,
+                                      const f3d_bf16_t* beta, float eps, const f3d_bf16_t* w1, const f3d_bf16_t* b1,
+                                      const f3d_bf16_t* w2, const f3d_bf16_t* b2, f3d_bf16_t* y, uint32_t ldy, uint32_t m,
+                                      uint32_t c, uint32_t hidden, int device, void* stream) {
+  if (!coord || !embed_table) {
+    f3d::set_error("null tensor pointer");
+    return F3D_ERR_INVALID;
+  }
+  return proj_ln_mlp_impl(a, lda, w_proj, b_proj, nullptr, 0, coord, embed_table, gamma, beta, eps, w1, b1, w2, b2, y, ldy, m,
+                          c, hidden, device, stream);
 }
 
 }  // extern "C"

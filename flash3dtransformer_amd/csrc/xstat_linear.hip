@@ -39,12 +39,14 @@ constexpr size_t xs_lds_bytes(bool wide) {
 // EPI: 0 = bias only, 1 = runtime activation and / or residual, 2 = residual only (its pieces are prefetched).
 // With LN the kernel expects w = w' and lnx = b' as fp32 [N], both prepared by ln_fold_kernel.
 // NBUF: w chunk buffers in LDS (chunk c + NBUF - 1 is requested when chunk c starts).
-template <int K, int MT, int WAVES, int NBUF, bool LN, bool SWIGLU, int EPI>
+// EMBED: the rows are not read but formed: row r is the coordinate embedding bf16(coord[r] . etab[c][0:3] + etab[c][3])
+// of its point (coord fp16 [M][3]; etab bf16 [K][8] = (wx, wy, wz, b, 0, 0, 0, 0) per channel), one MFMA per 32 channels.
+template <int K, int MT, int WAVES, int NBUF, bool LN, bool SWIGLU, int EPI, bool EMBED = false>
 __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2))) void xstat_linear_kernel(
     const uint16_t* __restrict__ x, uint32_t ldx, float eps, const uint16_t* __restrict__ w,
     const uint16_t* __restrict__ bias, const uint16_t* __restrict__ lnx,
     const uint16_t* __restrict__ residual, uint32_t ldr, uint16_t* __restrict__ y, uint32_t ldy, uint32_t M,
-    uint32_t N, uint32_t act) {
+    uint32_t N, uint32_t act, const uint16_t* __restrict__ coord, const uint16_t* __restrict__ etab) {
   using G = XsGeom<K>;
   constexpr int KS = K / 16;             // MFMA k-steps
   constexpr int ROWB = G::ROWB;
@@ -115,12 +117,50 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
   //      at columns ks * 16 + half * 8, loaded straight into its register, all of them in flight at once (the four
   //      fragments that share a 128-byte line are requested back to back).  Rows past M read row M - 1. ----
   bf16x8_t xf[MT][KS];
+  if constexpr (EMBED) {
+    // The rows are the coordinate embedding of their points (flash3dxfmr/layers/psh_ops.py:67-68: Linear(3, K) of the
+    // coordinates cast to bf16), formed here instead of being read: per row tile and 32 channels one product of the
+    // channels' (wx, wy, wz, b) with the rows' (x, y, z, 1), rounded to bf16 as the embedding layer stores it and
+    // re-laid from the accumulator layout into operand layout through the wave's (still unused) epilogue patch.
+    static_assert(K % 32 == 0 && EPI == 0 && !SWIGLU, "embedding in front of a plain bias epilogue");
+    uint16_t* ep = lds_patch + wave * (32 * kPatchPitch);
 #pragma unroll
-  for (int mt = 0; mt < MT; ++mt) {
-    const uint32_t r = min(row0 + mt * 32 + lq, M - 1);
-    const uint16_t* xp = x + (size_t)r * ldx + half * 8;
+    for (int mt = 0; mt < MT; ++mt) {
+      const uint32_t r = min(row0 + mt * 32 + lq, M - 1);
+      u32x4_t cb = {0u, 0u, 0u, 0u};
+      if (half == 0) {
+        const uint16_t* cp = coord + (size_t)r * 3;
+        cb[0] = pack_bf16x2(half_bits_to_float(cp[0]), half_bits_to_float(cp[1]));
+        cb[1] = pack_bf16x2(half_bits_to_float(cp[2]), 1.0f);
+      }
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) xf[mt][ks] = *reinterpret_cast<const bf16x8_t*>(xp + ks * 16);
+      for (int t = 0; t < K / 32; ++t) {
+        u32x4_t ea = {0u, 0u, 0u, 0u};
+        if (half == 0) ea = *reinterpret_cast<const u32x4_t*>(etab + (size_t)(t * 32 + lq) * 8);
+        f32x16_t e;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) e[i] = 0.f;
+        e = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, ea), __builtin_bit_cast(bf16x8_t, cb), e, 0, 0, 0);
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          uint2 pk;
+          pk.x = pack_bf16x2(e[g * 4 + 0], e[g * 4 + 1]);
+          pk.y = pack_bf16x2(e[g * 4 + 2], e[g * 4 + 3]);
+          *reinterpret_cast<uint2*>(ep + lq * kPatchPitch + g * 8 + half * 4) = pk;
+        }
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+          xf[mt][2 * t + j] = *reinterpret_cast<const bf16x8_t*>(ep + lq * kPatchPitch + j * 16 + half * 8);
+      }
+    }
+  } else {
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      const uint32_t r = min(row0 + mt * 32 + lq, M - 1);
+      const uint16_t* xp = x + (size_t)r * ldx + half * 8;
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) xf[mt][ks] = *reinterpret_cast<const bf16x8_t*>(xp + ks * 16);
+    }
   }
   // LayerNorm of this lane's rows in place: one sweep for the sums of d = x - x0 and d^2 (shifted by the row's first
   // element so that the variance does not cancel), one that writes bf16((x - mean) * rstd) back
@@ -396,22 +436,31 @@ template <int K, int MT, int WAVES, int NBUF>
 static int launch_k(bool ln, bool swiglu, hipStream_t s, const uint16_t* x, uint32_t ldx, float eps,
                     const uint16_t* w, const uint16_t* bias, const uint16_t* lnx,
                     const uint16_t* residual, uint32_t ldr, uint16_t* y, uint32_t ldy, uint32_t M, uint32_t N,
-                    uint32_t act, int device) {
+                    uint32_t act, int device, const uint16_t* coord = nullptr, const uint16_t* etab = nullptr) {
   const bool general = act != F3D_ACT_NONE || residual != nullptr;
   const bool res_only = act == F3D_ACT_NONE && residual != nullptr;
   const dim3 grid(cdiv_u32(M, 32 * MT * WAVES)), block(64 * WAVES);
-#define F3D_XS(L, S, E)                                                                                            \
+#define F3D_XS(L, S, E, ...)                                                                                       \
   do {                                                                                                             \
     static bool attr_set[64] = {};                                                                                 \
-    auto kern = xstat_linear_kernel<K, MT, WAVES, NBUF, L, S, E>;                                                       \
+    auto kern = xstat_linear_kernel<K, MT, WAVES, NBUF, L, S, E, ##__VA_ARGS__>;                                        \
     constexpr size_t lds = xs_lds_bytes<K, WAVES, NBUF>(xs_wide_flush<K, S, E>());                                 \
     if (device < 0 || device >= 64 || !attr_set[device]) {                                                         \
       F3D_CHECK_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds)); \
       if (device >= 0 && device < 64) attr_set[device] = true;                                                     \
     }                                                                                                              \
     hipLaunchKernelGGL(kern, grid, block, lds, s, x, ldx, eps, w, bias, lnx, residual, ldr, y, ldy, M, N,          \
-                       act);                                                                                       \
+                       act, coord, etab);                                                                          \
   } while (0)
+  if constexpr (K <= 256) {
+    if (coord) {       // the rows are the coordinate embedding, formed in the kernel (LayerNorm + bias epilogue only)
+      if (!ln || swiglu || general) return F3D_ERR_UNSUPPORTED;
+      F3D_XS(true, false, 0, true);
+      return F3D_OK;
+    }
+  } else if (coord) {
+    return F3D_ERR_UNSUPPORTED;
+  }
   if (ln && swiglu) { if (res_only) F3D_XS(true, true, 2); else if (general) F3D_XS(true, true, 1); else F3D_XS(true, true, 0); }
   else if (ln) { if (res_only) F3D_XS(true, false, 2); else if (general) F3D_XS(true, false, 1); else F3D_XS(true, false, 0); }
   else if (swiglu) { if (res_only) F3D_XS(false, true, 2); else if (general) F3D_XS(false, true, 1); else F3D_XS(false, true, 0); }
@@ -424,7 +473,8 @@ static int launch_k(bool ln, bool swiglu, hipStream_t s, const uint16_t* x, uint
 // the tiled GEMM), another code on failure.
 int launch_xstat_linear(const uint16_t* x, uint32_t ldx, const uint16_t* gamma, const uint16_t* beta, float eps,
                         const uint16_t* w, const uint16_t* bias, const uint16_t* residual, uint32_t ldr, uint16_t* y,
-                        uint32_t ldy, uint32_t M, uint32_t N, uint32_t K, uint32_t act, int device, hipStream_t s) {
+                        uint32_t ldy, uint32_t M, uint32_t N, uint32_t K, uint32_t act, int device, hipStream_t s,
+                        const uint16_t* coord, const uint16_t* etab) {
   const bool ln = gamma != nullptr;
   const bool swiglu = act == F3D_ACT_SWIGLU;
   const uint32_t run_act = swiglu ? (uint32_t)F3D_ACT_NONE : act;
@@ -454,9 +504,9 @@ int launch_xstat_linear(const uint16_t* x, uint32_t ldx, const uint16_t* gamma, 
 #define F3D_XS_CASE(KK)                                                                                                  \
   case KK:                                                                                                               \
     return big ? launch_k<KK, 2, 8, 3>(ln, swiglu, s, x, ldx, eps, w, bias, lnx, residual, ldr, y, ldy, M, N,   \
-                                       run_act, device)                                                                  \
+                                       run_act, device, coord, etab)                                                     \
                : launch_k<KK, 1, 4, 2>(ln, swiglu, s, x, ldx, eps, w, bias, lnx, residual, ldr, y, ldy, M, N,   \
-                                       run_act, device);
+                                       run_act, device, coord, etab);
   switch (K) {
     F3D_XS_CASE(32)
     F3D_XS_CASE(64)
@@ -465,7 +515,7 @@ int launch_xstat_linear(const uint16_t* x, uint32_t ldx, const uint16_t* gamma, 
     case 512:
       // 512 inner features fill the register budget with 32 rows per wave; two 64 KB chunk buffers
       return launch_k<512, 1, 8, 2>(ln, swiglu, s, x, ldx, eps, w, bias, lnx, residual, ldr, y, ldy, M, N,
-                                    run_act, device);
+                                    run_act, device, coord, etab);
     default: return F3D_ERR_UNSUPPORTED;
   }
 #undef F3D_XS_CASE

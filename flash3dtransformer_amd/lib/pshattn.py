@@ -646,6 +646,40 @@ def ln_mlp_swiglu_bf16(x, gamma, beta, eps, w1, b1, w2, b2, residual, y) -> bool
     return True
 
 
+def embed_table(w: torch.Tensor, bias) -> torch.Tensor:
+    """[c, 8] bf16 rows (w[c,0], w[c,1], w[c,2], bias[c], 0, 0, 0, 0): the coordinate embedding's parameters as the
+    kernels that form the embedding themselves read them"""
+    c = w.shape[0]
+    t = torch.zeros(c, 8, dtype=torch.bfloat16, device=w.device)
+    t[:, :3] = w.detach().to(torch.bfloat16)
+    if bias is not None:
+        t[:, 3] = bias.detach().to(torch.bfloat16)
+    return t
+
+
+def embed_ln_linear_bf16(coord, table, gamma, beta, eps, w, bias, y) -> bool:
+    """extension: y = LayerNorm(embed(coord)) w.T + bias with the coordinate embedding (psh_ops.py:64-68) formed inside
+    the kernel instead of read from memory; `table` from embed_table().  Returns False, leaving y untouched, when no
+    kernel covers the widths (the caller then runs coord_embed_bf16 + ln_linear_bf16)."""
+    dev = assert_same_device([coord, table, gamma, w, y])
+    assert_dtype([coord], torch.float16)
+    assert_dtype([table, gamma, w, y], torch.bfloat16)
+    assert_contiguous([coord, table, gamma, w])
+    _check_vectors(y, [beta, bias])
+    m = coord.shape[0]
+    n, k = w.shape
+    if (coord.dim() != 2 or coord.shape[1] != 3 or tuple(table.shape) != (k, 8) or gamma.shape[0] != k
+            or tuple(y.shape) != (m, n) or y.stride(1) != 1):
+        raise RuntimeError(f"embed_ln_linear shape mismatch: coord{tuple(coord.shape)} table{tuple(table.shape)} "
+                           f"w{tuple(w.shape)} y{tuple(y.shape)}")
+    rc = _load().f3d_embed_ln_linear_bf16(_ptr(coord), _ptr(table), _ptr(gamma), _ptr(beta), _f32(eps), _ptr(w), _ptr(bias),
+                                          _ptr(y), _u32(y.stride(0)), _u32(m), _u32(n), _u32(k), _i32(dev), _stream(dev))
+    if rc == 2:
+        return False
+    _check(rc)
+    return True
+
+
 def proj_ln_mlp_swiglu_bf16(a, w_proj, b_proj, x, gamma, beta, eps, w1, b1, w2, b2, y) -> bool:
     """extension: the second half of a block in one kernel (stage.py:92-102): x1 = a w_proj.T + b_proj + x, then
     y = x1 + MLP(LayerNorm(x1)) with the gated MLP of ln_mlp_swiglu_bf16; x1 never reaches memory.  Returns False,
@@ -666,6 +700,34 @@ def proj_ln_mlp_swiglu_bf16(a, w_proj, b_proj, x, gamma, beta, eps, w1, b1, w2, 
                                              _u32(x.stride(0)), _ptr(gamma), _ptr(beta), _f32(eps), _ptr(w1), _ptr(b1),
                                              _ptr(w2), _ptr(b2), _ptr(y), _u32(y.stride(0)), _u32(m), _u32(c),
                                              _u32(hidden), _i32(dev), _stream(dev))
+    if rc == 2:
+        return False
+    _check(rc)
+    return True
+
+
+def embed_proj_ln_mlp_swiglu_bf16(a, w_proj, b_proj, coord, table, gamma, beta, eps, w1, b1, w2, b2, y) -> bool:
+    """extension: proj_ln_mlp_swiglu_bf16 with the block input x = embed(coord) formed inside the kernel (the first block
+    behind PSH3DCoordEmbedding, psh_ops.py:64-68); `table` from embed_table().  Returns False, leaving y untouched, when
+    no kernel covers the widths."""
+    dev = assert_same_device([a, w_proj, coord, table, gamma, w1, w2, y])
+    assert_dtype([coord], torch.float16)
+    assert_dtype([a, w_proj, table, gamma, w1, w2, y], torch.bfloat16)
+    assert_contiguous([w_proj, w1, w2, gamma, coord, table])
+    _check_vectors(y, [b_proj, beta, b1, b2])
+    if any(t.dim() != 2 or t.stride(1) != 1 for t in (a, y)):
+        raise RuntimeError("embed_proj_ln_mlp_swiglu_bf16 expects 2-D row-major a and y")
+    m, c = a.shape
+    hidden = w2.shape[1]
+    if (tuple(coord.shape) != (m, 3) or tuple(table.shape) != (c, 8) or tuple(w_proj.shape) != (c, c)
+            or tuple(w1.shape) != (2 * hidden, c) or w2.shape[0] != c or tuple(y.shape) != (m, c) or gamma.shape[0] != c):
+        raise RuntimeError(f"embed_proj_ln_mlp shape mismatch: a{tuple(a.shape)} coord{tuple(coord.shape)} "
+                           f"table{tuple(table.shape)} w_proj{tuple(w_proj.shape)} w1{tuple(w1.shape)} w2{tuple(w2.shape)} "
+                           f"y{tuple(y.shape)}")
+    rc = _load().f3d_embed_proj_ln_mlp_swiglu_bf16(_ptr(a), _u32(a.stride(0)), _ptr(w_proj), _ptr(b_proj), _ptr(coord),
+                                                   _ptr(table), _ptr(gamma), _ptr(beta), _f32(eps), _ptr(w1), _ptr(b1),
+                                                   _ptr(w2), _ptr(b2), _ptr(y), _u32(y.stride(0)), _u32(m), _u32(c),
+                                                   _u32(hidden), _i32(dev), _stream(dev))
     if rc == 2:
         return False
     _check(rc)

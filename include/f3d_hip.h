@@ -335,6 +335,17 @@ int f3d_proj_ln_mlp_swiglu_bf16(const f3d_bf16_t* a, uint32_t lda, const f3d_bf1
                                 f3d_bf16_t* y, uint32_t ldy, uint32_t m, uint32_t c, uint32_t hidden, int device,
                                 void* stream);
 
+/* The same with the block input formed inside the kernel from the points' coordinates: x = embed(coord), the
+ * `PSH3DCoordEmbedding` output that feeds the FIRST block (flash3dxfmr/layers/psh_ops.py:64-68), never stored.  coord [m,3]
+ * fp16 and embed_table [c,8] bf16 as in f3d_embed_ln_linear_bf16; the embedding enters the sum in fp32 (one product per 32
+ * channels on the matrix core), x1 is rounded to bf16 once.  Same widths and return codes as
+ * f3d_proj_ln_mlp_swiglu_bf16. */
+int f3d_embed_proj_ln_mlp_swiglu_bf16(const f3d_bf16_t* a, uint32_t lda, const f3d_bf16_t* w_proj, const f3d_bf16_t* b_proj,
+                                      const f3d_half_t* coord, const f3d_bf16_t* embed_table, const f3d_bf16_t* gamma,
+                                      const f3d_bf16_t* beta, float eps, const f3d_bf16_t* w1, const f3d_bf16_t* b1,
+                                      const f3d_bf16_t* w2, const f3d_bf16_t* b2, f3d_bf16_t* y, uint32_t ldy, uint32_t m,
+                                      uint32_t c, uint32_t hidden, int device, void* stream);
+
 /* LayerNorm over the last axis, fp32 statistics (norm callables of flash3dxfmr/layers/stage.py:67).
  * x,y [m,c] bf16; gamma,beta [c] bf16 (beta may be NULL). */
 int f3d_layernorm_bf16(const f3d_bf16_t* x, const f3d_bf16_t* gamma, const f3d_bf16_t* beta, f3d_bf16_t* y,
@@ -344,6 +355,18 @@ int f3d_layernorm_bf16(const f3d_bf16_t* x, const f3d_bf16_t* gamma, const f3d_b
  * (flash3dxfmr/layers/psh_ops.py:64-67): y[r,:] = bf16(coord[r,:]) · wᵀ + bias; w [c,3] bf16. */
 int f3d_coord_embed_bf16(const f3d_half_t* coord, const f3d_bf16_t* w, const f3d_bf16_t* bias, f3d_bf16_t* y,
                          uint32_t m, uint32_t c, int device, void* stream);
+
+/* The coordinate embedding fused into its first consumer (extension): y = LayerNorm(embed(coord)) wT + bias without
+ * the embedding ever being stored, the `PSH3DCoordEmbedding` output feeding `norm -> qkv` of the first block
+ * (flash3dxfmr/layers/psh_ops.py:64-68, stage.py:94-96).  coord [m,3] fp16 (the scattered coordinates); embed_table
+ * [k,8] bf16 holds (w[c,0], w[c,1], w[c,2], bias[c], 0, 0, 0, 0) per embedding channel c; gamma, beta, eps, w [n,k],
+ * bias [n] or NULL, y [m,n] (row stride ldy) as in f3d_ln_linear_bf16.  The kernel forms each row's embedding on the
+ * matrix core (fp32 sum of the three products and the bias, rounded to bf16 as the embedding layer stores it) and goes
+ * on as f3d_ln_linear_bf16.  k in {32, 64, 128, 256}, n a multiple of 32; anything else returns F3D_ERR_UNSUPPORTED
+ * without touching y (use f3d_coord_embed_bf16, then f3d_ln_linear_bf16). */
+int f3d_embed_ln_linear_bf16(const f3d_half_t* coord, const f3d_bf16_t* embed_table, const f3d_bf16_t* gamma,
+                             const f3d_bf16_t* beta, float eps, const f3d_bf16_t* w, const f3d_bf16_t* bias, f3d_bf16_t* y,
+                             uint32_t ldy, uint32_t m, uint32_t n, uint32_t k, int device, void* stream);
 
 /* Per-channel affine + optional activation: eval-mode BatchNorm1d folded to scale/shift followed
  * by GELU/ReLU (pool / unpool norm+act callables, tests/test_psh_hourglass.py:103-106).

@@ -303,6 +303,73 @@ def test_proj_residual_mlp_unsupported_width_is_reported():
     assert (y5 == 3.0).all()
 
 
+@pytest.mark.parametrize("M,K,N", [(70000, 256, 768), (5000, 32, 96), (333, 64, 192), (200000, 128, 384), (1, 256, 32)])
+def test_embedding_inside_layernorm_linear(oracle, M, K, N):
+    """LayerNorm + Linear on the coordinate embedding formed inside the kernel against the embedding kernel followed by
+    the LayerNorm + Linear kernel (the embedding is summed in another order on the matrix core: a bf16 step apart in
+    a few places), and against fp32 mathematics."""
+    from flash3dtransformer_amd.lib import pshattn
+    g = torch.Generator().manual_seed(21)
+    coord = ((torch.rand(M, 3, generator=g) - 0.5) * 80.0).to(torch.float16).to(DEV)
+    we, be = _rand((K, 3), 22, scale=0.5).to(DEV), _rand((K,), 23).to(DEV)
+    gam, bet = (_rand((K,), 3) + 1.0).to(DEV), _rand((K,), 4, scale=0.2).to(DEV)
+    w, b = _rand((N, K), 2, scale=1 / math.sqrt(K)).to(DEV), _rand((N,), 6).to(DEV)
+    y = torch.full((M, N), 9.0, dtype=torch.bfloat16, device=DEV)
+    assert pshattn.embed_ln_linear_bf16(coord, pshattn.embed_table(we, be), gam, bet, 1e-5, w, b, y)
+    x = torch.empty(M, K, dtype=torch.bfloat16, device=DEV)
+    y2 = torch.empty_like(y)
+    pshattn.coord_embed_bf16(coord, we, be, x)
+    pshattn.ln_linear_bf16(x, gam, bet, 1e-5, w, b, None, y2, None)
+    torch.cuda.synchronize()
+    d = (y.float() - y2.float()).abs() / y2.float().abs().clamp(min=1.0)
+    assert d.max().item() <= 2 ** -4, d.max().item()
+    assert (d > 0).float().mean().item() < 0.05
+    xe = oracle.linear(coord.cpu().to(torch.bfloat16), we.cpu(), be.cpu()).to(torch.bfloat16)
+    ref = oracle.linear(oracle.layernorm(xe, gam.cpu(), bet.cpu(), 1e-5), w.cpu(), b.cpu())
+    _close(y.float().cpu(), ref)
+
+
+@pytest.mark.parametrize("M,C,H", [(70000, 256, 1024), (5000, 32, 128), (333, 64, 64), (66000, 128, 256)])
+def test_embedding_as_block_input_of_proj_residual_mlp(oracle, M, C, H):
+    """the one-kernel second half of a block with its block input formed from the coordinates against the same kernel
+    reading the stored embedding (the embedding enters unrounded: a bf16 step apart in places), and against the
+    unrounded mathematics"""
+    from flash3dtransformer_amd.lib import pshattn
+    g = torch.Generator().manual_seed(31)
+    coord = ((torch.rand(M, 3, generator=g) - 0.5) * 8.0).to(torch.float16).to(DEV)
+    we, be = _rand((C, 3), 22, scale=0.5).to(DEV), _rand((C,), 23).to(DEV)
+    a = _rand((M, C), 11, scale=1.5).to(DEV)
+    wp, bp = _rand((C, C), 12, scale=1 / math.sqrt(C)).to(DEV), _rand((C,), 13).to(DEV)
+    gam, bet = (_rand((C,), 3) + 1.0).to(DEV), _rand((C,), 4, scale=0.2).to(DEV)
+    w1, w2 = _rand((2 * H, C), 2, scale=1 / math.sqrt(C)).to(DEV), _rand((C, H), 5, scale=1 / math.sqrt(H)).to(DEV)
+    b1, b2 = _rand((2 * H,), 6).to(DEV), _rand((C,), 7).to(DEV)
+    y = torch.full((M, C), 9.0, dtype=torch.bfloat16, device=DEV)
+    assert pshattn.embed_proj_ln_mlp_swiglu_bf16(a, wp, bp, coord, pshattn.embed_table(we, be), gam, bet, 1e-5, w1, b1, w2, b2, y)
+    x = torch.empty(M, C, dtype=torch.bfloat16, device=DEV)
+    y2 = torch.empty_like(y)
+    pshattn.coord_embed_bf16(coord, we, be, x)
+    assert pshattn.proj_ln_mlp_swiglu_bf16(a, wp, bp, x, gam, bet, 1e-5, w1, b1, w2, b2, y2)
+    torch.cuda.synchronize()
+    d = (y.float() - y2.float()).abs() / y2.float().abs().clamp(min=1.0)
+    assert d.max().item() <= 0.25 and d.mean().item() <= 4e-3, (d.max().item(), d.mean().item())
+    c = lambda t: t.cpu()
+    xe = oracle.linear(c(coord).to(torch.bfloat16), c(we), c(be))
+    x1 = oracle.linear(c(a), c(wp), c(bp)) + xe
+    exact = x1 + oracle.linear(oracle.swiglu(oracle.linear(oracle.layernorm(x1, c(gam), c(bet), 1e-5), c(w1), c(b1))), c(w2), c(b2))
+    scale = exact.abs().clamp(min=1.0)
+    err_us, err_ref = (y.float().cpu() - exact).abs() / scale, (y2.float().cpu() - exact).abs() / scale
+    assert err_us.max() <= 1.5 * err_ref.max() + 4e-3 and err_us.mean() <= 1.25 * err_ref.mean() + 1e-4
+
+
+def test_embedding_inside_layernorm_linear_unsupported_width_is_reported():
+    from flash3dtransformer_amd.lib import pshattn
+    mk = lambda *s: torch.zeros(*s, dtype=torch.bfloat16, device=DEV)
+    y = torch.full((64, 64), 3.0, dtype=torch.bfloat16, device=DEV)
+    coord = torch.zeros(64, 3, dtype=torch.float16, device=DEV)
+    assert not pshattn.embed_ln_linear_bf16(coord, mk(512, 8), mk(512), mk(512), 1e-5, mk(64, 512), None, y)
+    assert (y == 3.0).all()
+
+
 def test_fused_mlp_unsupported_width_is_reported():
     from flash3dtransformer_amd.lib import pshattn
     mk = lambda *s: torch.zeros(*s, dtype=torch.bfloat16, device=DEV)
