@@ -133,7 +133,8 @@ def main():
 
     @torch.no_grad()
     def step():
-        feat = emb(coords, seps, HASH)
+        # lazy: the embedding is not stored; the block forms it inside its LayerNorm+QKV and out-projection+MLP kernels
+        feat = emb(coords, seps, HASH, lazy=True)
         return blk(None, feat, None)
 
     # Priming, before the W warm-up steps: the first process on a fresh box has been seen to stall the host once, for
@@ -176,41 +177,55 @@ def main():
         scat = emb.last_scattered_coord
         We, Be = bw(emb.lin.weight), bw(emb.lin.bias)
         emb_out = torch.empty_like(feat)
-        ops = {
-            "psh_scatter": lambda: psh_main.batch_bucket_scatter(coords, seps, BS, n_pad, HASH),
-            "coord_embed": lambda: pshattn.coord_embed_bf16(scat, We, Be, emb_out),
-            "ln_qkv": lambda: pshattn.ln_linear_bf16(feat, Wn, Bn, 1e-5, Wq, Bq, None, qkv, None),
-            "attention": lambda: pshattn.buck_swin_fwd(q, k, v, o, lse, scopes, BS),
-        }
+        etab = pshattn.embed_table(We, Be)
+        swiglu = args.mlp == "swiglu"
+        # with the gated MLP the embedding is formed inside its two consumers and never stored
+        stored = {"coord_embed": lambda: pshattn.coord_embed_bf16(scat, We, Be, emb_out),
+                  "ln_qkv": lambda: pshattn.ln_linear_bf16(feat, Wn, Bn, 1e-5, Wq, Bq, None, qkv, None)}
+        ops = {"psh_scatter": lambda: psh_main.batch_bucket_scatter(coords, seps, BS, n_pad, HASH)}
+        if swiglu:
+            ops["embed_ln_qkv"] = lambda: pshattn.embed_ln_linear_bf16(scat, etab, Wn, Bn, 1e-5, Wq, Bq, qkv)
+        else:
+            ops.update(stored)
+        ops["attention"] = lambda: pshattn.buck_swin_fwd(q, k, v, o, lse, scopes, BS)
         # the out-projection with its residual and the gated MLP with its residual run as one kernel at this size (the
         # block's choice at inference); with gelu: the projection, LayerNorm+fc1+act, then fc2
         separate = {"proj_residual": lambda: pshattn.linear_bf16(o.view(n_pad, C), Wp, Bp, feat, mid, None),
                     "ln_mlp_residual": lambda: pshattn.ln_mlp_swiglu_bf16(mid, Wm, Bm, 1e-5, W1, B1, W2, B2, mid, y)}
         two_kernel = {"ln_fc1_act": lambda: pshattn.ln_linear_bf16(mid, Wm, Bm, 1e-5, W1, B1, None, hid, args.mlp),
                       "fc2_residual": lambda: pshattn.linear_bf16(hid, W2, B2, mid, y, None)}
-        if args.mlp == "swiglu":
-            ops["proj_ln_mlp_residual"] = lambda: pshattn.proj_ln_mlp_swiglu_bf16(o.view(n_pad, C), Wp, Bp, feat, Wm, Bm, 1e-5,
-                                                                                  W1, B1, W2, B2, y)
+        if swiglu:
+            ops["embed_proj_ln_mlp_residual"] = lambda: pshattn.embed_proj_ln_mlp_swiglu_bf16(
+                o.view(n_pad, C), Wp, Bp, scat, etab, Wm, Bm, 1e-5, W1, B1, W2, B2, y)
+            stored["proj_ln_mlp_residual"] = lambda: pshattn.proj_ln_mlp_swiglu_bf16(o.view(n_pad, C), Wp, Bp, feat, Wm, Bm,
+                                                                                     1e-5, W1, B1, W2, B2, y)
         else:
             ops["proj_residual"] = separate["proj_residual"]
             ops.update(two_kernel)
         breakdown = {name: ev_time(fn, 20) for name, fn in ops.items()}
         two_kernel_ms = {name: ev_time(fn, 20) for name, fn in two_kernel.items()}
-        separate_ms = {name: ev_time(fn, 20) for name, fn in separate.items()} if args.mlp == "swiglu" else {}
+        separate_ms = {name: ev_time(fn, 20) for name, fn in separate.items()} if swiglu else {}
+        stored_ms = {name: ev_time(fn, 20) for name, fn in stored.items()} if swiglu else {}
     fc1_n = 2 * HID if args.mlp == "swiglu" else HID
-    flops = {"ln_qkv": 2.0 * n_pad * C * 3 * C, "proj_residual": 2.0 * n_pad * C * C,
+    flops = {"ln_qkv": 2.0 * n_pad * C * 3 * C, "embed_ln_qkv": 2.0 * n_pad * C * 3 * C + 2.0 * n_pad * 4 * C,
+             "proj_residual": 2.0 * n_pad * C * C,
              "ln_fc1_act": 2.0 * n_pad * C * fc1_n, "fc2_residual": 2.0 * n_pad * HID * C,
              "ln_mlp_residual": 2.0 * n_pad * C * fc1_n + 2.0 * n_pad * HID * C,
              "proj_ln_mlp_residual": 2.0 * n_pad * C * C + 2.0 * n_pad * C * fc1_n + 2.0 * n_pad * HID * C,
+             "embed_proj_ln_mlp_residual": 2.0 * n_pad * C * C + 2.0 * n_pad * C * fc1_n + 2.0 * n_pad * HID * C + 2.0 * n_pad * 4 * C,
              "attention": 4.0 * n_pad * BS * SCOPE * C}
     # algorithmic HBM bytes per launch (bf16 activations in and out, weights negligible)
-    hbm_bytes = {"ln_qkv": 2.0 * n_pad * (C + 3 * C), "proj_residual": 2.0 * n_pad * 3 * C,
+    hbm_bytes = {"ln_qkv": 2.0 * n_pad * (C + 3 * C), "embed_ln_qkv": 2.0 * n_pad * 3 * C + 6.0 * n_pad,   # coordinates in, qkv out
+                 "proj_residual": 2.0 * n_pad * 3 * C,
                  "ln_fc1_act": 2.0 * n_pad * (C + HID), "fc2_residual": 2.0 * n_pad * (HID + 2 * C),
                  "ln_mlp_residual": 2.0 * n_pad * 2 * C,      # x (also the residual) in, y out
                  "proj_ln_mlp_residual": 2.0 * n_pad * 3 * C,  # attention output and block input in, y out
+                 "embed_proj_ln_mlp_residual": 2.0 * n_pad * 2 * C + 6.0 * n_pad,  # attention output and coordinates in, y out
                  "attention": 2.0 * n_pad * 4 * C + 4.0 * n_pad * H}
     kernels = {"attention": "buck_swin_fwd_scope_kernel<32,512,16>",
                "ln_qkv": "xstat_linear_kernel<256,2,8,3,LN> + ln_fold_kernel",
+               "embed_ln_qkv": "xstat_linear_kernel<256,2,8,3,LN,embed> + ln_fold_kernel",
+               "embed_proj_ln_mlp_residual": "ln_mlp_swiglu_kernel<256, true, true> + mlp_prep_kernel",
                "ln_fc1_act": "xstat_linear_kernel<256,2,8,3,LN,swiglu> + ln_fold_kernel",
                "proj_residual": "xstat_linear_kernel<256,2,8,3,residual>",
                "fc2_residual": "ystat_linear_kernel<256> + ys_w_prep_kernel",
@@ -270,6 +285,7 @@ def main():
         "roofline": roofline,
         "breakdown_ms": {kname: round(vv, 4) for kname, vv in breakdown.items()},
         "per_op": per_op,
+        "stored_embedding_kernels": {kname: round(vv, 4) for kname, vv in stored_ms.items()} or None,
         "separate_proj_and_mlp_under_autograd": separate_proj_mlp,
         "two_kernel_mlp_on_request": two_kernel_mlp,
         "sub_metrics": sub,

@@ -9,7 +9,7 @@ from torch.autograd import Function
 from ..lib import pshattn
 from ..psh import dev_context as f3ddev
 from ..psh import swin_attn as sa
-from .nn_ops import Linear
+from .nn_ops import CoordEmbedding, Linear
 
 
 class BuckSwinFwdFunction(Function):
@@ -98,12 +98,16 @@ class BucketSwinAttentionModule(nn.Module):
         [B, L, 3C] projection output (the reference makes three contiguous copies, :187-190); the
         residual, when given, is added in the out-projection's epilogue.  skip_proj: return the attention output
         itself (the caller applies `self.proj`, e.g. inside the kernel of the MLP that follows)."""
-        assert x.dim() == 3, f"Expect input features with three axes [B, L, C], but got shape={x.shape}"
-        B, L, C = x.shape
+        if isinstance(x, CoordEmbedding):      # [L, C], not stored: one batch element
+            B, (L, C) = 1, x.shape
+        else:
+            assert x.dim() == 3, f"Expect input features with three axes [B, L, C], but got shape={x.shape}"
+            B, L, C = x.shape
         assert C == self.num_heads * self.head_dim, f"Expect input channels are {self.num_heads * self.head_dim}, but got {C}"
         if f3ddev.get_nvtx():
             nvtx.range_push(self.NVTX_SCOPE)
-        qkv = self.qkv(x, pre_norm=pre_norm)   # pre_norm: LayerNorm applied inside the projection kernel
+        # pre_norm: LayerNorm applied inside the projection kernel; a CoordEmbedding is formed there too
+        qkv = self.qkv.embedded(x, pre_norm).view(B, L, -1) if isinstance(x, CoordEmbedding) else self.qkv(x, pre_norm=pre_norm)
         if qkv.dtype == torch.bfloat16 and qkv.is_contiguous():
             attn_out = BuckSwinQKVFunction.apply(qkv, scope_buckets, self.attn.buck_size, self.num_heads)
         else:

@@ -106,7 +106,8 @@ class Flash3D(nn.Module):
     def forward(self, coords: torch.Tensor, input_feat: torch.Tensor, seps: torch.Tensor) -> torch.Tensor:
         if f3ddev.get_nvtx():
             nvtx.range_push(self.NVTX_SCOPE)
-        psh_feat = self.psh_scatter(coords, seps, self.first_hashtype)
+        # at inference without input features the embedding is not stored: the first block forms it inside its kernels
+        psh_feat = self.psh_scatter(coords, seps, self.first_hashtype, lazy=self.in_feat_dim is None)
         scattered = self.psh_scatter.last_scattered_coord
         self._last_index, self._last_n, self._last_seps = None, coords.shape[0], seps
         if self.in_feat_dim is not None:

@@ -386,8 +386,59 @@ class Linear(_CachedParamModule):
             out = torch_backward(y, _linear_ref(act, eps), x_in, self.weight, self.bias, res_in, ln_w, ln_b)
         return out.view(*lead, n_out)
 
+    def embedded(self, emb: "CoordEmbedding", pre_norm):
+        """forward(emb.materialize(), pre_norm=pre_norm) without storing the embedding: inference only"""
+        if isinstance(pre_norm, LayerNorm) and self.in_features in CoordEmbedding.EMBED_WIDTHS and self.out_features % 32 == 0:
+            w16, b16 = self._w.get(self.weight, self.training), self._b.get(self.bias, self.training)
+            g, b = norm_params_bf16(pre_norm)
+            y = torch.empty(emb.shape[0], self.out_features, dtype=torch.bfloat16, device=emb.device)
+            self._staged.arm(self.training or pre_norm.training, self.out_features, self.in_features, w16, b16, g, b,
+                             tag=("ln", float(pre_norm.eps)))
+            if pshattn.embed_ln_linear_bf16(emb.coord, emb.table(), g, b, pre_norm.eps, w16, b16, y):
+                return y
+        return self.forward(emb.materialize(), pre_norm=pre_norm)
+
     def extra_repr(self):
         return f"in_features={self.in_features}, out_features={self.out_features}, bias={self.bias is not None}"
+
+
+class CoordEmbedding:
+    """The coordinate embedding `lin(coord.bf16())` of PSH-scattered points that has NOT been stored: at inference the
+    first block forms it inside its own kernels (LayerNorm + QKV; out-projection + MLP) from the coordinates, and the
+    [rows, channels] tensor is neither written nor read.  Anything else calls materialize()."""
+    EMBED_WIDTHS = (32, 64, 128, 256)
+
+    def __init__(self, coord: torch.Tensor, lin: "Linear"):
+        self.coord, self.lin = coord, lin
+        self.shape = torch.Size((coord.shape[0], lin.out_features))
+        self.dtype, self.device = torch.bfloat16, coord.device
+        self._tensor = None
+
+    def dim(self):
+        return 2
+
+    def table(self) -> torch.Tensor:
+        """[channels, 8] bf16 rows (wx, wy, wz, b, 0, 0, 0, 0), rebuilt when the layer's parameters change"""
+        lin = self.lin
+        key = (lin.weight._version, lin.weight.data_ptr(), None if lin.bias is None else (lin.bias._version, lin.bias.data_ptr()))
+        cached = getattr(lin, "_embed_table", None)
+        if cached is None or cached[0] != key or cached[1].device != self.device:
+            cached = (key, pshattn.embed_table(lin.weight, lin.bias))
+            lin._embed_table = cached
+        return cached[1]
+
+    def materialize(self) -> torch.Tensor:
+        if self._tensor is None:
+            lin = self.lin
+            out = torch.empty(self.shape[0], lin.out_features, dtype=torch.bfloat16, device=self.device)
+            pshattn.coord_embed_bf16(self.coord, lin._w.get(lin.weight, lin.training), lin._b.get(lin.bias, lin.training), out)
+            self._tensor = out
+        return self._tensor
+
+
+def materialize(feat):
+    """a feature tensor as a tensor (a CoordEmbedding is stored first)"""
+    return feat.materialize() if isinstance(feat, CoordEmbedding) else feat
 
 
 class LayerNorm(_CachedParamModule):
@@ -560,16 +611,18 @@ class LayerNormMLP(_CachedParamModule):
 
     def after_projection(self, a: torch.Tensor, proj: "Linear", x: torch.Tensor):
         """x1 = proj(a) + x;  x1 + MLP(x1) in one kernel (x1 is never stored): the second half of a transformer block
-        (flash3dxfmr/layers/stage.py:92-102) at inference.  a, x [rows, hidden_size] bf16.  Returns None where that
+        (flash3dxfmr/layers/stage.py:92-102) at inference.  a, x [rows, hidden_size] bf16 (x may be a CoordEmbedding: the
+        kernel then forms the block input from the coordinates).  Returns None where that
         kernel does not apply (autograd on, other widths or activation, few rows): the caller then runs `proj` with its
         residual and this module."""
-        if (torch.is_grad_enabled() or self.activation != "swiglu" or self.hidden_size not in PROJ_MLP_WIDTHS
-                or self.ffn_hidden_size % 32 != 0 or self.fused is False or proj.in_features != self.hidden_size
-                or proj.out_features != self.hidden_size or not a.is_cuda or a.dtype != torch.bfloat16
-                or x.dtype != torch.bfloat16 or (self.hidden_size == 256 and a.shape[0] < 30000)):
+        if not self.takes_projection(a.shape[0]) or proj.in_features != self.hidden_size \
+                or proj.out_features != self.hidden_size or not a.is_cuda or a.dtype != torch.bfloat16 \
+                or x.dtype != torch.bfloat16:
             return None
-        a2, x2 = a.reshape(-1, self.hidden_size), x.reshape(-1, self.hidden_size)
-        if a2.stride(1) != 1 or x2.stride(1) != 1:
+        lazy = x if isinstance(x, CoordEmbedding) else None
+        a2 = a.reshape(-1, self.hidden_size)
+        x2 = None if lazy is not None else x.reshape(-1, self.hidden_size)
+        if a2.stride(1) != 1 or (x2 is not None and x2.stride(1) != 1):
             return None
         params = (self.layer_norm_weight, self.layer_norm_bias, self.fc1_weight, self.fc1_bias, self.fc2_weight, self.fc2_bias)
         g16, be16, w1_16, b1_16, w2_16, b2_16 = (c.get(p, self.training) for c, p in zip(self._c, params))
@@ -577,9 +630,17 @@ class LayerNormMLP(_CachedParamModule):
         y = torch.empty(a2.shape[0], self.hidden_size, dtype=torch.bfloat16, device=a.device)
         self._staged[0].arm(self.training, w1_16.shape[0], self.hidden_size, g16, be16, w1_16, b1_16, w2_16, b2_16,
                             tag=("mlp", float(self.eps)))
-        if not pshattn.proj_ln_mlp_swiglu_bf16(a2, wp16, bp16, x2, g16, be16, self.eps, w1_16, b1_16, w2_16, b2_16, y):
-            return None
-        return y.view(x.shape)
+        if lazy is not None:
+            ok = pshattn.embed_proj_ln_mlp_swiglu_bf16(a2, wp16, bp16, lazy.coord, lazy.table(), g16, be16, self.eps, w1_16,
+                                                       b1_16, w2_16, b2_16, y)
+        else:
+            ok = pshattn.proj_ln_mlp_swiglu_bf16(a2, wp16, bp16, x2, g16, be16, self.eps, w1_16, b1_16, w2_16, b2_16, y)
+        return y.view(x.shape) if ok else None
+
+    def takes_projection(self, rows: int) -> bool:
+        """whether after_projection() has a kernel for this layer at `rows` rows (inference only)"""
+        return not (torch.is_grad_enabled() or self.activation != "swiglu" or self.hidden_size not in PROJ_MLP_WIDTHS
+                    or self.ffn_hidden_size % 32 != 0 or self.fused is False or (self.hidden_size == 256 and rows < 30000))
 
     def forward(self, x: torch.Tensor, residual: torch.Tensor = None):
         x2 = as_bf16_2d(x.reshape(-1, self.hidden_size)).contiguous()

@@ -7,7 +7,7 @@ from torch import nn
 from ..lib import pshattn
 from ..psh import arithmatic as f3darith
 from ..psh import psh_main as pm
-from .nn_ops import Linear, torch_backward
+from .nn_ops import CoordEmbedding, Linear, torch_backward
 
 
 class _PermuteRows(torch.autograd.Function):
@@ -90,11 +90,15 @@ class PSH3DCoordEmbedding(nn.Module):
         self.last_scattered_coord = None
         self.last_buffers = None
 
-    def forward(self, coords, seps, hash_op):
+    def forward(self, coords, seps, hash_op, lazy: bool = False):
+        """lazy (inference only): return a CoordEmbedding, which the first block turns into its input inside its own
+        kernels, instead of storing the [rows, emb_dim] tensor"""
         pad_to = f3darith.cdiv(coords.shape[0], self.alignment) * self.alignment
         scattered, buffers = pm.batch_bucket_scatter(coords, seps, self.bucket_size, pad_to, hash_op)
         self.last_scattered_coord = scattered
         self.last_buffers = buffers
+        if lazy and not torch.is_grad_enabled() and self.lin.out_features in CoordEmbedding.EMBED_WIDTHS:
+            return CoordEmbedding(scattered, self.lin)
         emb = torch.empty(pad_to, self.lin.out_features, dtype=torch.bfloat16, device=coords.device)
         lin = self.lin
         pshattn.coord_embed_bf16(scattered, lin._w.get(lin.weight, lin.training), lin._b.get(lin.bias, lin.training), emb)

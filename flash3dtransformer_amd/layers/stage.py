@@ -9,7 +9,7 @@ from torch import nn
 from ..psh import bucket_scope
 from ..psh import dev_context as f3ddev
 from . import buck_swin, elem_wise
-from .nn_ops import apply_norm, is_fusable_layernorm
+from .nn_ops import CoordEmbedding, apply_norm, is_fusable_layernorm, materialize
 
 
 @dataclass(slots=True)
@@ -44,15 +44,18 @@ class XFMR(nn.Module):
         if f3ddev.get_nvtx():
             nvtx.range_push(self.NVTX_SCOPE)
         fused_ln = is_fusable_layernorm(self.norm, C)   # norm -> qkv in one kernel
+        if isinstance(reduced_feat, CoordEmbedding) and not (fused_ln and self.mlp.mlp.takes_projection(N)):
+            reduced_feat = reduced_feat.materialize()   # an unstored embedding needs both of the block's kernels that form it
         x = reduced_feat if fused_ln else apply_norm(self.norm, reduced_feat)
         pre = self.norm if fused_ln else None
         out = None
         if not torch.is_grad_enabled() and reduced_feat.dtype == torch.bfloat16:
             # inference: out-projection + residual + MLP + residual in one kernel where it applies
-            attn = self.bwa(x.view(1, N, C), scope_bucks, pre_norm=pre, skip_proj=True).view(N, C)
+            x_in = x if isinstance(x, CoordEmbedding) else x.view(1, N, C)
+            attn = self.bwa(x_in, scope_bucks, pre_norm=pre, skip_proj=True).view(N, C)
             out = self.mlp.mlp.after_projection(attn, self.bwa.proj, reduced_feat)
             if out is None:
-                mid = self.bwa.proj(attn, residual=reduced_feat)
+                mid = self.bwa.proj(attn, residual=materialize(reduced_feat))
                 out = self.mlp(mid, residual=mid)
         else:
             mid = self.bwa(x.view(1, N, C), scope_bucks, residual=reduced_feat.view(1, N, C), pre_norm=pre).view(N, C)
@@ -85,7 +88,7 @@ class Stage(nn.Module):
         x = reduced_feat
         for block in self.encoder_blocks:
             x = block(reduced_coord, x, reduced_sep)
-        x = self.middle(reduced_coord, x, reduced_sep)
+        x = self.middle(reduced_coord, materialize(x), reduced_sep)
         for block in self.decoder_blocks:
             x = block(reduced_coord, x, reduced_sep)
         if f3ddev.get_nvtx():
