@@ -133,9 +133,16 @@ def main():
 
     @torch.no_grad()
     def step():
-        # lazy: the embedding is not stored; the block forms it inside its LayerNorm+QKV and out-projection+MLP kernels
+        # lazy: the embedding is not stored; the block forms its rows inside the attention kernel (LayerNorm + QKV of the
+        # rank-4 embedding, folded) and inside the out-projection + MLP kernel
         feat = emb(coords, seps, HASH, lazy=True)
         return blk(None, feat, None)
+
+    @torch.no_grad()
+    def step_stored():
+        # the same stage with the embedding stored: the kernels a block runs on ANY input (LayerNorm+QKV, attention over
+        # the stored projection output, out-projection + MLP)
+        return blk(None, emb(coords, seps, HASH), None)
 
     # Priming, before the W warm-up steps: the first process on a fresh box has been seen to stall the host once, for
     # 30-40 ms, within its first dozen steps (the stall moves when unrelated host code before the loop changes, so it
@@ -157,6 +164,14 @@ def main():
     dt = time.perf_counter() - t0
     ms_per_step = dt / args.steps * 1e3
     value = n_pts / (dt / args.steps) / 1e6
+    for _ in range(max(3, args.warmup)):
+        step_stored()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step_stored()
+    torch.cuda.synchronize()
+    ms_per_step_stored = (time.perf_counter() - t0) / args.steps * 1e3
 
     # ---- per-op breakdown on the same tensors, events on the launch stream ----
     with torch.no_grad():
@@ -179,15 +194,20 @@ def main():
         emb_out = torch.empty_like(feat)
         etab = pshattn.embed_table(We, Be)
         swiglu = args.mlp == "swiglu"
-        # with the gated MLP the embedding is formed inside its two consumers and never stored
+        # with the gated MLP the embedding is formed inside its consumers and never stored, and Q, K, V neither: the
+        # attention kernel forms its rows from the coordinates
         stored = {"coord_embed": lambda: pshattn.coord_embed_bf16(scat, We, Be, emb_out),
                   "ln_qkv": lambda: pshattn.ln_linear_bf16(feat, Wn, Bn, 1e-5, Wq, Bq, None, qkv, None)}
+        attention = lambda: pshattn.buck_swin_fwd(q, k, v, o, lse, scopes, BS)
         ops = {"psh_scatter": lambda: psh_main.batch_bucket_scatter(coords, seps, BS, n_pad, HASH)}
         if swiglu:
-            ops["embed_ln_qkv"] = lambda: pshattn.embed_ln_linear_bf16(scat, etab, Wn, Bn, 1e-5, Wq, Bq, qkv)
+            fold = pshattn.embed_qkv_fold(We, Be, Wn, Bn, 1e-5, Wq, Bq, H)
+            ops["embed_attention"] = lambda: pshattn.embed_buck_swin_fwd(scat, fold[0], fold[1], o, lse, scopes, BS)
+            stored["embed_ln_qkv"] = lambda: pshattn.embed_ln_linear_bf16(scat, etab, Wn, Bn, 1e-5, Wq, Bq, qkv)
+            stored["attention"] = attention
         else:
             ops.update(stored)
-        ops["attention"] = lambda: pshattn.buck_swin_fwd(q, k, v, o, lse, scopes, BS)
+            ops["attention"] = attention
         # the out-projection with its residual and the gated MLP with its residual run as one kernel at this size (the
         # block's choice at inference); with gelu: the projection, LayerNorm+fc1+act, then fc2
         separate = {"proj_residual": lambda: pshattn.linear_bf16(o.view(n_pad, C), Wp, Bp, feat, mid, None),
@@ -213,7 +233,8 @@ def main():
              "ln_mlp_residual": 2.0 * n_pad * C * fc1_n + 2.0 * n_pad * HID * C,
              "proj_ln_mlp_residual": 2.0 * n_pad * C * C + 2.0 * n_pad * C * fc1_n + 2.0 * n_pad * HID * C,
              "embed_proj_ln_mlp_residual": 2.0 * n_pad * C * C + 2.0 * n_pad * C * fc1_n + 2.0 * n_pad * HID * C + 2.0 * n_pad * 4 * C,
-             "attention": 4.0 * n_pad * BS * SCOPE * C}
+             "attention": 4.0 * n_pad * BS * SCOPE * C,
+             "embed_attention": 4.0 * n_pad * BS * SCOPE * C + 2.0 * n_pad * 4 * 3 * C}
     # algorithmic HBM bytes per launch (bf16 activations in and out, weights negligible)
     hbm_bytes = {"ln_qkv": 2.0 * n_pad * (C + 3 * C), "embed_ln_qkv": 2.0 * n_pad * 3 * C + 6.0 * n_pad,   # coordinates in, qkv out
                  "proj_residual": 2.0 * n_pad * 3 * C,
@@ -221,8 +242,10 @@ def main():
                  "ln_mlp_residual": 2.0 * n_pad * 2 * C,      # x (also the residual) in, y out
                  "proj_ln_mlp_residual": 2.0 * n_pad * 3 * C,  # attention output and block input in, y out
                  "embed_proj_ln_mlp_residual": 2.0 * n_pad * 2 * C + 6.0 * n_pad,  # attention output and coordinates in, y out
-                 "attention": 2.0 * n_pad * 4 * C + 4.0 * n_pad * H}
+                 "attention": 2.0 * n_pad * 4 * C + 4.0 * n_pad * H,
+                 "embed_attention": 6.0 * n_pad + 2.0 * n_pad * C + 4.0 * n_pad * H}   # coordinates in, O and LSE out
     kernels = {"attention": "buck_swin_fwd_scope_kernel<32,512,16>",
+               "embed_attention": "buck_swin_fwd_scope_kernel<32,512,16,rows formed in the kernel>",
                "ln_qkv": "xstat_linear_kernel<256,2,8,3,LN> + ln_fold_kernel",
                "embed_ln_qkv": "xstat_linear_kernel<256,2,8,3,LN,embed> + ln_fold_kernel",
                "embed_proj_ln_mlp_residual": "ln_mlp_swiglu_kernel<256, true, true> + mlp_prep_kernel",
@@ -285,7 +308,11 @@ def main():
         "roofline": roofline,
         "breakdown_ms": {kname: round(vv, 4) for kname, vv in breakdown.items()},
         "per_op": per_op,
-        "stored_embedding_kernels": {kname: round(vv, 4) for kname, vv in stored_ms.items()} or None,
+        "stored_intermediates": {"ms_per_step": round(ms_per_step_stored, 4),
+                                 "what": "the same stage with the embedding and the QKV projection stored (the kernels a "
+                                         "block runs on any input); `value` is the first block as the reference's model "
+                                         "feeds it: its input is the coordinate embedding (flash3d.py:162-163)",
+                                 "kernels_ms": {kname: round(vv, 4) for kname, vv in stored_ms.items()} or None},
         "separate_proj_and_mlp_under_autograd": separate_proj_mlp,
         "two_kernel_mlp_on_request": two_kernel_mlp,
         "sub_metrics": sub,

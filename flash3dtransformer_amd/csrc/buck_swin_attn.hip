@@ -439,14 +439,26 @@ constexpr size_t scope_lds_bytes() {
   return (size_t)2 * 2 * T * D * 2;
 }
 
-template <int D, int T, int WAVES>
+// GEN: Q, K and V are not read but formed from the rows' coordinates (the first block of a model, whose input is the
+// coordinate embedding: LayerNorm and the QKV projection of a rank-4 input fold into one 4-column matrix per output
+// row plus a per-row scale).  `table` holds, per head and tile (0: Q in the exponent's units, 1: K, 2: V, 3: Q
+// unscaled, for the general pass), 32 rows of 16 bf16, the A operand of one 32x32x16 product; `chol` the
+// upper-triangular factor of the embedding's centred Gram matrix (10 numbers) and the LayerNorm epsilon.
+struct ScopeGen {
+  const uint16_t* coord;   // [batch * seq_len][3] fp16
+  const uint16_t* table;   // [num_head][4][32][16] bf16
+  const float* chol;       // L00 L01 L02 L03 L11 L12 L13 L22 L23 L33 eps
+};
+
+template <int D, int T, int WAVES, bool GEN = false>
 __global__ __launch_bounds__(64 * WAVES) void buck_swin_fwd_scope_kernel(
     const uint16_t* __restrict__ q, const uint16_t* __restrict__ k, const uint16_t* __restrict__ v, uint32_t ld,
     uint16_t* __restrict__ o, float* __restrict__ lse, const uint32_t* __restrict__ scope_buckets,
     uint32_t num_scope, uint32_t scope_size, uint32_t bs, uint32_t seq_len, uint32_t num_head,
     const int32_t* __restrict__ kv_len, float scale_log2, uint32_t n_items, uint32_t items_per_xcd,
-    uint32_t n_slots) {
+    uint32_t n_slots, ScopeGen gen) {
   constexpr int QB = T / (32 * WAVES);     // 32-query blocks per wave
+  static_assert(!GEN || (QB == 1 && D == 32), "rows formed in the kernel: one 32-row block per wave, 32-wide heads");
   constexpr int KSTEPS = D / 16;
   constexpr int CPK = D / 8;               // 16-byte chunks per row
   constexpr int ROWB = D * 2;              // bytes per K / V row in LDS
@@ -570,14 +582,85 @@ __global__ __launch_bounds__(64 * WAVES) void buck_swin_fwd_scope_kernel(
   cur.len = load_len(cur.ids);
   nxt.ids = my_items > 1 ? load_ids(p_nxt) : 0xFFFFFFFFu;
   nxt.len = load_len(nxt.ids);
-  static_for<QB>([&](auto b_c) { issue_q_one(p_cur, cur, b_c); });
-  if (kv_wanted(cur)) {
-    const size_t goff = kv_base(p_cur, cur);
+  // GEN: what an item's rows are formed from, requested one item ahead: the three coordinates of the lane's row
+  // (row lq of the wave's 32, which are its queries and its share of the keys) and the A operands of the head's
+  // Q / K / V tiles
+  uint16_t g_c[3] = {0, 0, 0};
+  u32x4_t g_a[3];
+  auto gen_row = [&](const Pos& p, const Scope& sc) { return (size_t)p.batch * seq_len + q_row_of(sc, 0); };
+  auto gen_tile_ptr = [&](const Pos& p, uint32_t tile) {
+    return reinterpret_cast<const u32x4_t*>(gen.table + (((size_t)p.head * 4 + tile) * 32 + lq) * 16 + half * 8);
+  };
+  auto issue_gen = [&](const Pos& p, const Scope& sc) {
+    const uint16_t* cp = gen.coord + gen_row(p, sc) * 3;
 #pragma unroll
-    for (uint32_t i = 0; i < 2u * BPW; ++i) issue_kv_one(goff, i, lds0);
+    for (int j = 0; j < 3; ++j) g_c[j] = cp[j];
+#pragma unroll
+    for (int tl = 0; tl < 3; ++tl) g_a[tl] = *gen_tile_ptr(p, tl);
+  };
+  float chol[11];
+  if constexpr (GEN) {
+#pragma unroll
+    for (int i = 0; i < 11; ++i) chol[i] = gen.chol[i];
   }
-  __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
-  __syncthreads();
+  // the rows' B operand: c~ = (x, y, z, 1) / sqrt(var + eps) as bf16 high and low parts; lanes < 32 carry the high
+  // parts twice (against the matrix's high and low parts), lanes >= 32 the low parts and two ones (the bias)
+  auto gen_rows_operand = [&](const uint16_t (&c)[3]) {
+    float cc[3];
+#pragma unroll
+    for (int j = 0; j < 3; ++j) cc[j] = bf16_bits_to_float(float_to_bf16_bits(half_bits_to_float(c[j])));
+    const float t0 = __builtin_fmaf(chol[0], cc[0], __builtin_fmaf(chol[1], cc[1], __builtin_fmaf(chol[2], cc[2], chol[3])));
+    const float t1 = __builtin_fmaf(chol[4], cc[1], __builtin_fmaf(chol[5], cc[2], chol[6]));
+    const float t2 = __builtin_fmaf(chol[7], cc[2], chol[8]);
+    const float var = __builtin_fmaf(t0, t0, __builtin_fmaf(t1, t1, __builtin_fmaf(t2, t2, chol[9] * chol[9])));
+    const float rstd = __builtin_amdgcn_rsqf(var + chol[10]);
+    const float s[4] = {cc[0] * rstd, cc[1] * rstd, cc[2] * rstd, rstd};
+    float hi[4], lo[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      hi[j] = bf16_bits_to_float(float_to_bf16_bits(s[j]));
+      lo[j] = s[j] - hi[j];
+    }
+    u32x4_t b;
+    if (half == 0) {
+      b[0] = pack_bf16x2(hi[0], hi[1]);
+      b[1] = pack_bf16x2(hi[2], hi[3]);
+      b[2] = b[0];
+      b[3] = b[1];
+    } else {
+      b[0] = pack_bf16x2(lo[0], lo[1]);
+      b[1] = pack_bf16x2(lo[2], lo[3]);
+      b[2] = 0x3F803F80u;     // (1, 1)
+      b[3] = 0u;
+    }
+    return __builtin_bit_cast(bf16x8_t, b);
+  };
+  // one tile of the rows' projection, transposed: register i of lane (lq, half) is feature 8 half + i (i < 8) or
+  // 16 + 8 half + i - 8 of row lq, the order of the score product's Q operand and of the 16-byte pieces of a K / V row
+  auto gen_tile = [&](const u32x4_t& a, const bf16x8_t& rows) {
+    f32x16_t z;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) z[i] = 0.f;
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), rows, z, 0, 0, 0);
+  };
+  auto pack_tile = [&](const f32x16_t& x, int ks) {
+    u32x4_t w;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) w[e] = pack_bf16x2(x[ks * 8 + 2 * e], x[ks * 8 + 2 * e + 1]);
+    return w;
+  };
+  if constexpr (GEN) {
+    issue_gen(p_cur, cur);
+  } else {
+    static_for<QB>([&](auto b_c) { issue_q_one(p_cur, cur, b_c); });
+    if (kv_wanted(cur)) {
+      const size_t goff = kv_base(p_cur, cur);
+#pragma unroll
+      for (uint32_t i = 0; i < 2u * BPW; ++i) issue_kv_one(goff, i, lds0);
+    }
+    __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
+    __syncthreads();
+  }
 
   for (uint32_t n = 0; n < my_items; ++n) {
     const bool has_next = n + 1 < my_items;
@@ -585,6 +668,22 @@ __global__ __launch_bounds__(64 * WAVES) void buck_swin_fwd_scope_kernel(
 
     // Q of this item arrived during the previous one: scale into the exponent's units and round once
     bf16x8_t qf[QB][KSTEPS];
+    if constexpr (GEN) {
+      // form the item's Q (kept in registers), K and V (the wave's 32 rows of this item's LDS buffer: the buffer's
+      // last readers, two items back, passed the previous barrier), then meet the other waves
+      const bf16x8_t rows = gen_rows_operand(g_c);
+      const f32x16_t tq = gen_tile(g_a[0], rows), tk = gen_tile(g_a[1], rows), tv = gen_tile(g_a[2], rows);
+#pragma unroll
+      for (int ks = 0; ks < KSTEPS; ++ks) qf[0][ks] = __builtin_bit_cast(bf16x8_t, pack_tile(tq, ks));
+      char* const wb = const_cast<char*>(sbuf) + wave * 32u * ROWB;
+#pragma unroll
+      for (int ks = 0; ks < KSTEPS; ++ks) {
+        *reinterpret_cast<u32x4_t*>(wb + (k_off ^ (ks * 32u))) = pack_tile(tk, ks);
+        *reinterpret_cast<u32x4_t*>(wb + OPB + lq * ROWB + (half + 2u * ks) * 16u) = pack_tile(tv, ks);
+      }
+      if (has_next) issue_gen(p_nxt, nxt);
+      wg_barrier_lds();
+    } else {
 #pragma unroll
     for (int b = 0; b < QB; ++b)
 #pragma unroll
@@ -595,11 +694,12 @@ __global__ __launch_bounds__(64 * WAVES) void buck_swin_fwd_scope_kernel(
           sc[e] = pack_bf16x2(bf16_lo(qraw[b][ks][e]) * scale_log2, bf16_hi(qraw[b][ks][e]) * scale_log2);
         qf[b][ks] = __builtin_bit_cast(bf16x8_t, sc);
       }
+    }
     // The next item's operands go in flight during the first half of this item's passes, a few vector-memory
     // instructions per step (issued all at once they would hold every wave of the workgroup at the memory pipeline's door for a
     // microsecond or two with the SIMDs idle): `vm_next` counts those already issued, 2 BPW direct loads of K / V
     // first, then the Q rows of the wave's QB blocks.
-    constexpr uint32_t VM_OPS = 2u * BPW + QB, VM_PER_STEP = (VM_OPS + NSTEP / 2 - 1) / (NSTEP / 2);   // all in the first half
+    constexpr uint32_t VM_OPS = GEN ? 0u : 2u * BPW + QB, VM_PER_STEP = (VM_OPS + NSTEP / 2 - 1) / (NSTEP / 2);   // all in the first half
     const bool nxt_kv = has_next && kv_wanted(nxt);
     const size_t nxt_goff = nxt_kv ? kv_base(p_nxt, nxt) : 0;
     const uint32_t nxt_buf = lds0 + ((n + 1) & 1u) * BUF;
@@ -769,7 +869,14 @@ __global__ __launch_bounds__(64 * WAVES) void buck_swin_fwd_scope_kernel(
       for (int b = 0; b < QB; ++b) {
         // unscaled Q, read again: the fast pass keeps only its pre-scaled copy
         bf16x8_t qr[KSTEPS];
-        {
+        if constexpr (GEN) {
+          // formed again from the row's coordinates with the head's unscaled tile
+          const uint16_t* cp = gen.coord + gen_row(p_cur, cur) * 3;
+          const uint16_t c3[3] = {cp[0], cp[1], cp[2]};
+          const f32x16_t tq = gen_tile(*gen_tile_ptr(p_cur, 3), gen_rows_operand(c3));
+#pragma unroll
+          for (int ks = 0; ks < KSTEPS; ++ks) qr[ks] = __builtin_bit_cast(bf16x8_t, pack_tile(tq, ks));
+        } else {
           const char* qp = reinterpret_cast<const char*>(q + in_base(p_cur)) + (q_row_of(cur, b) * ld + half * 8u) * 2u;
 #pragma unroll
           for (int ks = 0; ks < KSTEPS; ++ks) qr[ks] = *reinterpret_cast<const bf16x8_t*>(qp + ks * 32u);
@@ -874,16 +981,16 @@ __global__ __launch_bounds__(64 * WAVES) void buck_swin_fwd_scope_kernel(
     p_cur = p_nxt;
     p_nxt = p_nxt2;
     // the next buffer is complete; this buffer is free for the item after next.  Not __syncthreads(): that would wait
-    // for the output stores just issued
-    wg_barrier_lds();
+    // for the output stores just issued.  (GEN: the barrier after an item's rows are formed does both jobs.)
+    if constexpr (!GEN) wg_barrier_lds();
   }
 }
 
-template <int D, int T, int WAVES>
+template <int D, int T, int WAVES, bool GEN = false>
 static int launch_attn_scope(const uint16_t* q, const uint16_t* k, const uint16_t* v, uint32_t ld, uint16_t* o, float* lse,
                              const uint32_t* scope_buckets, uint32_t num_scope, uint32_t scope_size, uint32_t bs,
                              uint32_t batch, uint32_t seq_len, uint32_t num_head, const int32_t* kv_len, int device,
-                             hipStream_t s) {
+                             hipStream_t s, ScopeGen gen = ScopeGen{nullptr, nullptr, nullptr}) {
   const uint64_t n_items64 = (uint64_t)batch * num_scope * num_head;
   if (n_items64 == 0) return F3D_OK;
   if (n_items64 > 0x7FFFFFF0ull) {
@@ -896,9 +1003,9 @@ static int launch_attn_scope(const uint16_t* q, const uint16_t* k, const uint16_
   static int wg_per_cu[64] = {};
   int per_cu = (device >= 0 && device < 64) ? wg_per_cu[device] : 0;
   if (per_cu == 0) {
-    F3D_CHECK_HIP(hipFuncSetAttribute((const void*)buck_swin_fwd_scope_kernel<D, T, WAVES>,
+    F3D_CHECK_HIP(hipFuncSetAttribute((const void*)buck_swin_fwd_scope_kernel<D, T, WAVES, GEN>,
                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    F3D_CHECK_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, buck_swin_fwd_scope_kernel<D, T, WAVES>,
+    F3D_CHECK_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, buck_swin_fwd_scope_kernel<D, T, WAVES, GEN>,
                                                                64 * WAVES, lds));
     if (per_cu < 1) per_cu = 1;
     if (device >= 0 && device < 64) wg_per_cu[device] = per_cu;
@@ -909,10 +1016,94 @@ static int launch_attn_scope(const uint16_t* q, const uint16_t* k, const uint16_
   const uint32_t items_per_xcd = cdiv_u32(n_items, kNumXcd);
   const uint32_t n_slots = std::max(1u, std::min((uint32_t)n_cu * (uint32_t)per_cu / kNumXcd, items_per_xcd));
   const float scale_log2 = 1.4426950408889634f / sqrtf((float)D);
-  hipLaunchKernelGGL((buck_swin_fwd_scope_kernel<D, T, WAVES>), dim3(n_slots * kNumXcd), dim3(64 * WAVES), lds, s, q, k,
+  hipLaunchKernelGGL((buck_swin_fwd_scope_kernel<D, T, WAVES, GEN>), dim3(n_slots * kNumXcd), dim3(64 * WAVES), lds, s, q, k,
                      v, ld, o, lse, scope_buckets, num_scope, scope_size, bs, seq_len, num_head, kv_len, scale_log2,
-                     n_items, items_per_xcd, n_slots);
+                     n_items, items_per_xcd, n_slots, gen);
   return F3D_OK;
+}
+
+// ---- LayerNorm + QKV projection of the coordinate embedding, folded --------------------------------------------
+// The first block's input is x = E c, c = (x, y, z, 1), E = [w_embed | b_embed] (C x 4).  Over the channels,
+// x - mean(x) = E' c with E' = E minus its column means, var(x) = |E' c|^2 / C = |L c|^2 with L the upper-triangular
+// Cholesky factor of G = E'^T E' / C, and
+//   qkv = W (gamma * (x - mean) * rstd + beta) + b = rstd * (M c) + b',   M = W diag(gamma) E'  (3C x 4),  b' = W beta + b.
+// One thread per output row writes that row's 16 bf16 of the attention kernel's table: (M high parts, M low parts |
+// M high parts, b' high, b' low, 0, 0), to be multiplied with (c~ high, c~ high | c~ low, 1, 1, 0, 0), c~ = rstd c;
+// row position inside the head's 32-row tile = the row of the 32x32 accumulator layout that hands a lane the features
+// 8 half .. 8 half + 7 and 16 + 8 half .. 16 + 8 half + 7.  Thread 0 writes the Cholesky factor and eps.
+__global__ __launch_bounds__(64) void embed_qkv_fold_kernel(
+    const uint16_t* __restrict__ ew, const uint16_t* __restrict__ eb, const uint16_t* __restrict__ gamma,
+    const uint16_t* __restrict__ beta, float eps, const uint16_t* __restrict__ w, const uint16_t* __restrict__ b,
+    uint32_t C, uint32_t num_head, float scale_log2, uint16_t* __restrict__ table, float* __restrict__ chol) {
+  const uint32_t row = blockIdx.x * 64 + threadIdx.x;      // output feature of the projection, < 3 C
+  auto e_at = [&](uint32_t ch, uint32_t j) {
+    return j < 3 ? bf16_bits_to_float(ew[ch * 3 + j]) : (eb ? bf16_bits_to_float(eb[ch]) : 0.f);
+  };
+  double mean[4] = {0, 0, 0, 0};
+  for (uint32_t ch = 0; ch < C; ++ch)
+    for (uint32_t j = 0; j < 4; ++j) mean[j] += e_at(ch, j);
+  for (uint32_t j = 0; j < 4; ++j) mean[j] /= C;
+  if (row < 3 * C) {
+    double m[4] = {0, 0, 0, 0}, bp = b ? bf16_bits_to_float(b[row]) : 0.f;
+    for (uint32_t ch = 0; ch < C; ++ch) {
+      const double wv = bf16_bits_to_float(w[(size_t)row * C + ch]);
+      const double wg = wv * (gamma ? bf16_bits_to_float(gamma[ch]) : 1.f);
+      for (uint32_t j = 0; j < 4; ++j) m[j] += wg * (e_at(ch, j) - mean[j]);
+      if (beta) bp += wv * bf16_bits_to_float(beta[ch]);
+    }
+    const uint32_t part = row / C, within = row % C, head = within / 32, d = within % 32;
+    const uint32_t hf = (d % 16) / 8, i = d < 16 ? d % 8 : 8 + d % 8;
+    const uint32_t r = (i % 4) + 8 * (i / 4) + 4 * hf;
+    auto emit = [&](uint32_t tile, double sc) {
+      uint16_t* out = table + (((size_t)head * 4 + tile) * 32 + r) * 16;
+      for (uint32_t j = 0; j < 4; ++j) {
+        const float f = (float)(m[j] * sc);
+        const uint16_t hi = float_to_bf16_bits(f);
+        out[j] = hi;
+        out[4 + j] = float_to_bf16_bits(f - bf16_bits_to_float(hi));
+        out[8 + j] = hi;
+      }
+      const float fb = (float)(bp * sc);
+      const uint16_t bh = float_to_bf16_bits(fb);
+      out[12] = bh;
+      out[13] = float_to_bf16_bits(fb - bf16_bits_to_float(bh));
+      out[14] = 0;
+      out[15] = 0;
+    };
+    if (part == 0) {
+      emit(0, (double)scale_log2);
+      emit(3, 1.0);
+    } else {
+      emit(part, 1.0);
+    }
+  }
+  if (row == 0) {
+    double g[4][4];
+    for (int a = 0; a < 4; ++a)
+      for (int c = 0; c < 4; ++c) g[a][c] = 0;
+    for (uint32_t ch = 0; ch < C; ++ch)
+      for (int a = 0; a < 4; ++a)
+        for (int c = a; c < 4; ++c) g[a][c] += ((double)e_at(ch, a) - mean[a]) * ((double)e_at(ch, c) - mean[c]);
+    double l[4][4];
+    for (int a = 0; a < 4; ++a)
+      for (int c = 0; c < 4; ++c) l[a][c] = 0;
+    for (int a = 0; a < 4; ++a) {           // G = L^T L, row by row; a pivot that is not positive ends its row at zero
+      double piv = g[a][a] / C;
+      for (int k2 = 0; k2 < a; ++k2) piv -= l[k2][a] * l[k2][a];
+      if (!(piv > 0)) continue;
+      l[a][a] = sqrt(piv);
+      for (int c = a + 1; c < 4; ++c) {
+        double s = g[a][c] / C;
+        for (int k2 = 0; k2 < a; ++k2) s -= l[k2][a] * l[k2][c];
+        l[a][c] = s / l[a][a];
+      }
+    }
+    int n = 0;
+    for (int a = 0; a < 4; ++a)
+      for (int c = a; c < 4; ++c) chol[n++] = (float)l[a][c];
+    chol[10] = eps;
+    for (n = 11; n < 16; ++n) chol[n] = 0.f;
+  }
 }
 
 template <int D, int KT>
@@ -990,6 +1181,62 @@ int f3d_buck_swin_fwd_strided(const f3d_bf16_t* q, const f3d_bf16_t* k, const f3
     default: F3D_ATTN(128, 64); break;
   }
 #undef F3D_ATTN
+  if (rc != F3D_OK) return rc;
+  F3D_CHECK_HIP(hipGetLastError());
+  return F3D_OK;
+}
+
+int f3d_embed_qkv_fold_bf16(const f3d_bf16_t* embed_w, const f3d_bf16_t* embed_b, const f3d_bf16_t* gamma,
+                            const f3d_bf16_t* beta, float eps, const f3d_bf16_t* w_qkv, const f3d_bf16_t* b_qkv, uint32_t c,
+                            uint32_t num_head, uint32_t head_dim, f3d_bf16_t* table, float* chol, int device,
+                            void* stream) {
+  using namespace f3d;
+  F3D_CHECK_ARG(embed_w && w_qkv && table && chol, "null tensor pointer");
+  F3D_CHECK_ARG(c > 0 && num_head > 0 && c == num_head * head_dim, "channels %u != num_head %u * head_dim %u", c, num_head,
+                head_dim);
+  if (head_dim != 32) {
+    set_error("rows are formed inside the attention kernel for head_dim 32 only (got %u)", head_dim);
+    return F3D_ERR_UNSUPPORTED;
+  }
+  DeviceGuard guard(device);
+  F3D_CHECK_ARG(guard.ok, "cannot select device %d", device);
+  hipStream_t s = (hipStream_t)stream;
+  SyncBracket sync(s);
+  const float scale_log2 = 1.4426950408889634f / sqrtf((float)head_dim);
+  hipLaunchKernelGGL(embed_qkv_fold_kernel, dim3(cdiv_u32(3 * c, 64)), dim3(64), 0, s, embed_w, embed_b, gamma, beta, eps,
+                     w_qkv, b_qkv, c, num_head, scale_log2, table, chol);
+  F3D_CHECK_HIP(hipGetLastError());
+  return F3D_OK;
+}
+
+int f3d_embed_buck_swin_fwd(const f3d_half_t* coord, const f3d_bf16_t* table, const float* chol, f3d_bf16_t* o, float* lse,
+                            const uint32_t* scope_buckets, uint32_t num_scope, uint32_t scope_size, uint32_t bucket_size,
+                            uint32_t batch, uint32_t seq_len, uint32_t num_head, uint32_t head_dim, int device,
+                            void* stream) {
+  using namespace f3d;
+  F3D_CHECK_ARG(coord && table && chol && o && lse && scope_buckets, "null tensor pointer");
+  F3D_CHECK_ARG(bucket_size >= 128 && bucket_size % 128 == 0, "bucket_size=%u must be a multiple of 128", bucket_size);
+  F3D_CHECK_ARG(seq_len % bucket_size == 0, "sequence length %u is not a multiple of bucket_size=%u", seq_len, bucket_size);
+  F3D_CHECK_ARG((((uintptr_t)table | (uintptr_t)o) & 15u) == 0, "table / o must be 16-byte aligned");
+  const uint32_t scope_tokens = scope_size * bucket_size;
+  if (head_dim != 32 || scope_size < 1 || scope_size > (uint32_t)kResMaxScope || (scope_tokens != 256 && scope_tokens != 512) ||
+      (uint64_t)seq_len * num_head * head_dim * 2 >= (1ull << 32)) {
+    set_error("rows are formed inside the attention kernel for head_dim 32 and scopes of 256 or 512 tokens only "
+              "(head_dim %u, %u tokens)", head_dim, scope_tokens);
+    return F3D_ERR_UNSUPPORTED;
+  }
+  DeviceGuard guard(device);
+  F3D_CHECK_ARG(guard.ok, "cannot select device %d", device);
+  hipStream_t s = (hipStream_t)stream;
+  SyncBracket sync(s);
+  const ScopeGen gen = {coord, table, chol};
+  int rc;
+  if (scope_tokens == 256)
+    rc = launch_attn_scope<32, 256, 8, true>(nullptr, nullptr, nullptr, num_head * head_dim, o, lse, scope_buckets, num_scope,
+                                             scope_size, bucket_size, batch, seq_len, num_head, nullptr, device, s, gen);
+  else
+    rc = launch_attn_scope<32, 512, 16, true>(nullptr, nullptr, nullptr, num_head * head_dim, o, lse, scope_buckets, num_scope,
+                                              scope_size, bucket_size, batch, seq_len, num_head, nullptr, device, s, gen);
   if (rc != F3D_OK) return rc;
   F3D_CHECK_HIP(hipGetLastError());
   return F3D_OK;

@@ -9,7 +9,7 @@ from torch.autograd import Function
 from ..lib import pshattn
 from ..psh import dev_context as f3ddev
 from ..psh import swin_attn as sa
-from .nn_ops import CoordEmbedding, Linear
+from .nn_ops import CoordEmbedding, LayerNorm, Linear, _DerivedCache, norm_params_bf16
 
 
 class BuckSwinFwdFunction(Function):
@@ -91,6 +91,37 @@ class BucketSwinAttentionModule(nn.Module):
         self.qkv = Linear(channels, channels * 3, bias=qkv_bias)
         self.attn = BucketSwinAttention(buck_size)
         self.proj = Linear(channels, channels)
+        self.qkv._fold = _DerivedCache()      # (table, chol): LayerNorm + QKV of a coordinate embedding, folded
+
+    def _attention_of_embedding(self, emb: CoordEmbedding, pre_norm, scope_buckets):
+        """The attention output [1, L, H, D] of an unstored coordinate embedding with Q, K and V formed inside the
+        attention kernel: LayerNorm and the QKV projection of the rank-4 embedding fold into four numbers per output
+        feature (prepared once per set of weights).  None where no kernel covers the shape (32-wide heads, scopes of
+        256 or 512 tokens, LayerNorm in front): the caller then runs the projection kernel on the embedding."""
+        tokens = scope_buckets.shape[1] * self.attn.buck_size
+        if (torch.is_grad_enabled() or not isinstance(pre_norm, LayerNorm) or self.head_dim != 32 or tokens not in (256, 512)
+                or scope_buckets.shape[1] > 4):
+            return None
+        lin, qkv = emb.lin, self.qkv
+
+        def build():
+            training = self.training or pre_norm.training or lin.training
+            g, be = norm_params_bf16(pre_norm)
+            return pshattn.embed_qkv_fold(lin._w.get(lin.weight, training), lin._b.get(lin.bias, training), g, be, pre_norm.eps,
+                                          qkv._w.get(qkv.weight, training), qkv._b.get(qkv.bias, training), self.num_heads)
+
+        fold = qkv._fold.get_or_build((lin.weight, lin.bias, pre_norm.weight, pre_norm.bias, qkv.weight, qkv.bias),
+                                      (float(pre_norm.eps), self.num_heads), build)
+        if fold is None:
+            return None
+        table, chol = fold
+        L = emb.shape[0]
+        O = torch.empty(1, L, self.num_heads, self.head_dim, dtype=torch.bfloat16, device=emb.device)
+        lse = (torch.empty if _covers(scope_buckets, self.attn.buck_size, L) else torch.zeros)(
+            1, L, self.num_heads, dtype=torch.float32, device=emb.device)
+        if not pshattn.embed_buck_swin_fwd(emb.coord, table, chol, O, lse, scope_buckets, self.attn.buck_size):
+            return None
+        return O
 
     def forward(self, x: torch.Tensor, scope_buckets: torch.Tensor, residual: torch.Tensor = None,
                 pre_norm=None, skip_proj: bool = False) -> torch.Tensor:
@@ -106,13 +137,15 @@ class BucketSwinAttentionModule(nn.Module):
         assert C == self.num_heads * self.head_dim, f"Expect input channels are {self.num_heads * self.head_dim}, but got {C}"
         if f3ddev.get_nvtx():
             nvtx.range_push(self.NVTX_SCOPE)
-        # pre_norm: LayerNorm applied inside the projection kernel; a CoordEmbedding is formed there too
-        qkv = self.qkv.embedded(x, pre_norm).view(B, L, -1) if isinstance(x, CoordEmbedding) else self.qkv(x, pre_norm=pre_norm)
-        if qkv.dtype == torch.bfloat16 and qkv.is_contiguous():
-            attn_out = BuckSwinQKVFunction.apply(qkv, scope_buckets, self.attn.buck_size, self.num_heads)
-        else:
-            q, k, v = (t.view(B, L, self.num_heads, self.head_dim) for t in torch.chunk(qkv, 3, dim=-1))
-            attn_out = self.attn(q, k, v, scope_buckets)
+        attn_out = self._attention_of_embedding(x, pre_norm, scope_buckets) if isinstance(x, CoordEmbedding) else None
+        if attn_out is None:
+            # pre_norm: LayerNorm applied inside the projection kernel; a CoordEmbedding is formed there too
+            qkv = self.qkv.embedded(x, pre_norm).view(B, L, -1) if isinstance(x, CoordEmbedding) else self.qkv(x, pre_norm=pre_norm)
+            if qkv.dtype == torch.bfloat16 and qkv.is_contiguous():
+                attn_out = BuckSwinQKVFunction.apply(qkv, scope_buckets, self.attn.buck_size, self.num_heads)
+            else:
+                q, k, v = (t.view(B, L, self.num_heads, self.head_dim) for t in torch.chunk(qkv, 3, dim=-1))
+                attn_out = self.attn(q, k, v, scope_buckets)
         out = attn_out.view(B, L, C) if skip_proj else self.proj(attn_out.view(B, L, C), residual=residual)
         if f3ddev.get_nvtx():
             nvtx.range_pop()

@@ -147,6 +147,18 @@ class _StagedWeights:
         self._key, self._src = key, live
 
 
+class _DerivedCache(_Bf16Cache):
+    """something computed from several parameters (a folded table), kept while their addresses and versions stay;
+    dropped with the owning module's bf16 copies (train() / eval(), load_state_dict, refresh_weights())"""
+
+    def get_or_build(self, params, extra, build):
+        key = tuple(None if p is None else (p.data_ptr(), p._version, p.dtype, p.device) for p in params) + tuple(extra)
+        if key != self._key:
+            self._val = build()
+            self._key = key if self._val is not None else None
+        return self._val
+
+
 class _CachedParamModule(nn.Module):
     """nn.Module whose kernels read bf16 copies of its parameters (`_Bf16Cache` attributes or lists of them)"""
 

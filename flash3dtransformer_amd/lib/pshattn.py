@@ -680,6 +680,61 @@ def embed_ln_linear_bf16(coord, table, gamma, beta, eps, w, bias, y) -> bool:
     return True
 
 
+def embed_qkv_fold(embed_w, embed_b, gamma, beta, eps, w_qkv, b_qkv, num_heads: int):
+    """extension: LayerNorm + QKV projection of the coordinate embedding (psh_ops.py:64-68 -> stage.py:94-96) folded
+    into what embed_buck_swin_fwd reads: a table [num_heads, 4, 32, 16] bf16 (per head the Q tile in the exponent's
+    units, K, V, and Q unscaled) and 16 floats (Cholesky factor of the embedding's centred Gram matrix, eps).
+    Returns None when no kernel covers the head width."""
+    dev = assert_same_device([embed_w, gamma, w_qkv])
+    assert_dtype([embed_w, gamma, w_qkv], torch.bfloat16)
+    assert_contiguous([embed_w, gamma, w_qkv])
+    c = embed_w.shape[0]
+    if tuple(embed_w.shape) != (c, 3) or tuple(w_qkv.shape) != (3 * c, c) or gamma.shape[0] != c or c % num_heads:
+        raise RuntimeError(f"embed_qkv_fold shape mismatch: embed_w{tuple(embed_w.shape)} w_qkv{tuple(w_qkv.shape)}")
+    for v, n in ((embed_b, c), (beta, c), (b_qkv, 3 * c)):
+        if v is not None:
+            assert_dtype([v], torch.bfloat16)
+            assert_contiguous([v])
+            if v.numel() != n:
+                raise RuntimeError("embed_qkv_fold: bias / beta length mismatch")
+    table = torch.empty(num_heads, 4, 32, 16, dtype=torch.bfloat16, device=embed_w.device)
+    chol = torch.empty(16, dtype=torch.float32, device=embed_w.device)
+    rc = _load().f3d_embed_qkv_fold_bf16(_ptr(embed_w), _ptr(embed_b), _ptr(gamma), _ptr(beta), _f32(eps), _ptr(w_qkv),
+                                         _ptr(b_qkv), _u32(c), _u32(num_heads), _u32(c // num_heads), _ptr(table),
+                                         _ptr(chol), _i32(dev), _stream(dev))
+    if rc == 2:
+        return None
+    _check(rc)
+    return table, chol
+
+
+def embed_buck_swin_fwd(coord, table, chol, O, L, Scope_buckets, bucket_size) -> bool:
+    """extension: buck_swin_fwd of the first block with Q, K and V formed inside the kernel from the rows' coordinates
+    (coord [B * L, 3] fp16, table / chol from embed_qkv_fold) instead of read from a projection output.  O [B,L,H,32]
+    bf16, L (LSE) [B,L,H] fp32.  Returns False, leaving O untouched, when no kernel covers the shape (scopes of 256 or
+    512 tokens, 32-wide heads)."""
+    dev = assert_same_device([coord, table, chol, O, L, Scope_buckets])
+    assert_dtype([coord], torch.float16)
+    assert_dtype([table, O], torch.bfloat16)
+    assert_dtype([chol, L], torch.float32)
+    assert_dtype([Scope_buckets], torch.uint32)
+    assert_contiguous([coord, table, chol, O, L, Scope_buckets])
+    if O.dim() != 4:
+        raise RuntimeError(f"O must be [B,L,H,D], got {tuple(O.shape)}")
+    B, Ls, H, D = O.shape
+    if (coord.dim() != 2 or tuple(coord.shape) != (B * Ls, 3) or tuple(table.shape) != (H, 4, 32, 16) or chol.numel() != 16
+            or tuple(L.shape) != (B, Ls, H) or Scope_buckets.dim() != 2):
+        raise RuntimeError(f"embed_buck_swin_fwd shape mismatch: coord{tuple(coord.shape)} table{tuple(table.shape)} "
+                           f"O{tuple(O.shape)} L{tuple(L.shape)}")
+    rc = _load().f3d_embed_buck_swin_fwd(_ptr(coord), _ptr(table), _ptr(chol), _ptr(O), _ptr(L), _ptr(Scope_buckets),
+                                         _u32(Scope_buckets.shape[0]), _u32(Scope_buckets.shape[1]), _u32(bucket_size),
+                                         _u32(B), _u32(Ls), _u32(H), _u32(D), _i32(dev), _stream(dev))
+    if rc == 2:
+        return False
+    _check(rc)
+    return True
+
+
 def proj_ln_mlp_swiglu_bf16(a, w_proj, b_proj, x, gamma, beta, eps, w1, b1, w2, b2, y) -> bool:
     """extension: the second half of a block in one kernel (stage.py:92-102): x1 = a w_proj.T + b_proj + x, then
     y = x1 + MLP(LayerNorm(x1)) with the gated MLP of ln_mlp_swiglu_bf16; x1 never reaches memory.  Returns False,

@@ -346,6 +346,33 @@ int f3d_embed_proj_ln_mlp_swiglu_bf16(const f3d_bf16_t* a, uint32_t lda, const f
                                       const f3d_bf16_t* w2, const f3d_bf16_t* b2, f3d_bf16_t* y, uint32_t ldy, uint32_t m,
                                       uint32_t c, uint32_t hidden, int device, void* stream);
 
+/* The first block's `norm -> qkv -> attention` (flash3dxfmr/layers/stage.py:94-96, buck_swin.py:176-192) on the
+ * coordinate embedding (psh_ops.py:64-68) without embedding, LayerNorm output or projection output ever being stored
+ * (extension; inference only).  The embedding is x = E c with c = (x, y, z, 1) and E = [w_embed | b_embed]; over the
+ * channels x - mean(x) = E' c (E' = E minus its column means) and var(x) = |L c|^2 (L: upper Cholesky factor of
+ * E'^T E' / C), hence   qkv = rstd (M c) + b',  M = w_qkv diag(gamma) E',  b' = w_qkv beta + b_qkv,  rstd = 1 / sqrt(|L c|^2 + eps):
+ * four multiplications per output instead of C, exact in real arithmetic (the embedding and the LayerNorm output are
+ * not rounded to bf16 in between, so the result is closer to the unrounded mathematics than the three stored steps).
+ *
+ * f3d_embed_qkv_fold_bf16 prepares, from embed_w [c,3], embed_b [c] or NULL, gamma [c] or NULL, beta [c] or NULL, w_qkv [3c,c], b_qkv [3c]
+ * or NULL (all bf16): `table` [num_head][4][32][16] bf16 (per head: Q in units of log2(e)/sqrt(head_dim), K, V, Q unscaled;
+ * each number as a bf16 high and low part) and `chol` [16] fp32 (the ten entries of L row by row, eps, zeros).  Once per
+ * set of weights.  head_dim must be 32 (F3D_ERR_UNSUPPORTED otherwise).
+ *
+ * f3d_embed_buck_swin_fwd is f3d_buck_swin_fwd with Q, K, V formed inside the kernel: a wave builds its 32 rows of an
+ * item from their coordinates (coord [batch * seq_len, 3] fp16, the scattered coordinates) with three products on the
+ * matrix core and writes K and V straight into LDS.  o, lse, scope_buckets and the sizes as in f3d_buck_swin_fwd; no
+ * valid lengths.  head_dim 32 with scopes of 256 or 512 tokens; anything else returns F3D_ERR_UNSUPPORTED without
+ * touching o (use f3d_embed_ln_linear_bf16, then f3d_buck_swin_fwd_strided). */
+int f3d_embed_qkv_fold_bf16(const f3d_bf16_t* embed_w, const f3d_bf16_t* embed_b, const f3d_bf16_t* gamma,
+                            const f3d_bf16_t* beta, float eps, const f3d_bf16_t* w_qkv, const f3d_bf16_t* b_qkv, uint32_t c,
+                            uint32_t num_head, uint32_t head_dim, f3d_bf16_t* table, float* chol, int device,
+                            void* stream);
+int f3d_embed_buck_swin_fwd(const f3d_half_t* coord, const f3d_bf16_t* table, const float* chol, f3d_bf16_t* o, float* lse,
+                            const uint32_t* scope_buckets, uint32_t num_scope, uint32_t scope_size, uint32_t bucket_size,
+                            uint32_t batch, uint32_t seq_len, uint32_t num_head, uint32_t head_dim, int device,
+                            void* stream);
+
 /* LayerNorm over the last axis, fp32 statistics (norm callables of flash3dxfmr/layers/stage.py:67).
  * x,y [m,c] bf16; gamma,beta [c] bf16 (beta may be NULL). */
 int f3d_layernorm_bf16(const f3d_bf16_t* x, const f3d_bf16_t* gamma, const f3d_bf16_t* beta, f3d_bf16_t* y,

@@ -436,3 +436,112 @@ def test_attention_module_backpropagates(oracle):
     torch.cuda.synchronize()
     wq, wk, wv, _ = oracle.buck_swin_bwd(Q.detach().cpu(), K.detach().cpu(), V.detach().cpu(), w, scopes, bs)
     _check_grads([t.grad.float().cpu() for t in (Q, K, V)], (wq, wk, wv), "autograd")
+
+
+# ---- first block: Q, K, V formed inside the attention kernel from the coordinates ------------------------------
+
+def _first_block_weights(C, seed):
+    g = torch.Generator().manual_seed(seed)
+    r = lambda *s, scale=1.0: (torch.randn(*s, generator=g) * scale).to(torch.bfloat16)
+    return dict(ew=r(C, 3, scale=0.5), eb=r(C, scale=0.5), gamma=(r(C, scale=0.2).float() + 1.0).to(torch.bfloat16),
+                beta=r(C, scale=0.2), w=r(3 * C, C, scale=1.0 / math.sqrt(C)), b=r(3 * C, scale=0.3))
+
+
+def _exact_qkv(coord, p, eps):
+    """float64: embedding (of the bf16-cast coordinates), LayerNorm, projection, no rounding in between"""
+    c = coord.to(torch.bfloat16).double()
+    x = c @ p["ew"].double().T + p["eb"].double()
+    mu, var = x.mean(1, keepdim=True), x.var(1, unbiased=False, keepdim=True)
+    ln = (x - mu) / torch.sqrt(var + eps) * p["gamma"].double() + p["beta"].double()
+    return ln @ p["w"].double().T + p["b"].double()
+
+
+def test_embedding_layernorm_qkv_fold_table():
+    """the folded table against float64: M = W diag(gamma) E' and b' = W beta + b as bf16 high + low parts at the tile
+    positions the attention kernel expects; the Cholesky factor reproduces the LayerNorm variance of random rows"""
+    from flash3dtransformer_amd.lib import pshattn
+    C, H, eps = 128, 4, 1e-5
+    p = _first_block_weights(C, 5)
+    d = {k: v.to(DEV) for k, v in p.items()}
+    table, chol = pshattn.embed_qkv_fold(d["ew"], d["eb"], d["gamma"], d["beta"], eps, d["w"], d["b"], H)
+    torch.cuda.synchronize()
+    table, chol = table.float().cpu().double(), chol.cpu().double()
+    E = torch.cat([p["ew"].double(), p["eb"].double()[:, None]], 1)
+    Ep = E - E.mean(0, keepdim=True)
+    M = (p["w"].double() * p["gamma"].double()[None, :]) @ Ep
+    bp = p["w"].double() @ p["beta"].double() + p["b"].double()
+    scale = math.log2(math.e) / math.sqrt(32)
+    for part, tile, sc in ((0, 0, scale), (0, 3, 1.0), (1, 1, 1.0), (2, 2, 1.0)):
+        for h in range(H):
+            for dd in range(32):
+                half, i = (dd % 16) // 8, (dd % 8 if dd < 16 else 8 + dd % 8)
+                r = (i % 4) + 8 * (i // 4) + 4 * half
+                row = table[h, tile, r]
+                o = part * C + h * 32 + dd
+                got_m, got_b = row[0:4] + row[4:8], row[12] + row[13]
+                assert torch.equal(row[8:12], row[0:4]) and row[14] == 0 and row[15] == 0
+                assert (got_m - M[o] * sc).abs().max() <= 2e-5 * max(1.0, M[o].abs().max().item() * sc)
+                assert abs(got_b - bp[o] * sc) <= 2e-5 * max(1.0, abs(bp[o].item()) * sc)
+    L = torch.zeros(4, 4, dtype=torch.float64)
+    L[0, :], L[1, 1:], L[2, 2:], L[3, 3] = chol[0:4], chol[4:7], chol[7:9], chol[9]
+    assert abs(chol[10].item() - eps) < 1e-12
+    c = torch.cat([(torch.rand(1000, 3, dtype=torch.float64) - 0.5) * 100, torch.ones(1000, 1, dtype=torch.float64)], 1)
+    var = (c @ Ep.T).pow(2).mean(1)
+    assert ((c @ L.T).pow(2).sum(1) - var).abs().max() <= 1e-5 * var.max()
+
+
+@pytest.mark.parametrize("B,L,C,bs,scope_size,spread", [
+    (1, 4096, 256, 512, 1, 80.0),       # the encoder stage's shape
+    (2, 2048, 64, 256, 2, 8.0),         # two buckets per scope, two batch elements
+    (1, 1536, 32, 256, 1, 80.0),        # scopes of 256 tokens, one head
+    (1, 3072, 128, 128, 4, 40.0),       # four buckets per scope
+])
+def test_first_block_attention_rows_formed_in_kernel(oracle, B, L, C, bs, scope_size, spread):
+    """embed_buck_swin_fwd against (1) the stored pipeline of this library (embedding + LayerNorm + QKV kernel, then the
+    attention kernel over its output) and (2) attention over the float64 projection of the same rows"""
+    from flash3dtransformer_amd.lib import pshattn
+    H, eps = C // 32, 1e-5
+    g = torch.Generator().manual_seed(L + C)
+    coord = ((torch.rand(B * L, 3, generator=g) - 0.5) * spread).to(torch.float16)
+    p = _first_block_weights(C, C + 1)
+    d = {k: v.to(DEV) for k, v in p.items()}
+    scopes = oracle.gen_scopes(L, bs, scope_size)
+    if scope_size > 1:          # buckets of a scope in shuffled order
+        scopes = np.random.default_rng(3).permuted(scopes, axis=1)
+    sc = torch.from_numpy(np.ascontiguousarray(scopes, dtype=np.uint32).view(np.int32)).to(DEV).view(torch.uint32)
+    cd = coord.to(DEV)
+    fold = pshattn.embed_qkv_fold(d["ew"], d["eb"], d["gamma"], d["beta"], eps, d["w"], d["b"], H)
+    assert fold is not None
+    O = torch.full((B, L, H, 32), 7.0, dtype=torch.bfloat16, device=DEV)
+    LSE = torch.zeros(B, L, H, dtype=torch.float32, device=DEV)
+    assert pshattn.embed_buck_swin_fwd(cd, fold[0], fold[1], O, LSE, sc, bs)
+    # (1) the stored pipeline
+    qkv = torch.empty(B * L, 3 * C, dtype=torch.bfloat16, device=DEV)
+    assert pshattn.embed_ln_linear_bf16(cd, pshattn.embed_table(d["ew"], d["eb"]), d["gamma"], d["beta"], eps, d["w"], d["b"], qkv)
+    Q, K, V = (t.view(B, L, H, 32) for t in torch.chunk(qkv.view(B, L, 3 * C), 3, dim=-1))
+    O2, LSE2 = torch.zeros_like(O), torch.zeros_like(LSE)
+    pshattn.buck_swin_fwd(Q, K, V, O2, LSE2, sc, bs)
+    torch.cuda.synchronize()
+    d_o, d_l = (O.float() - O2.float()).abs().max().item(), (LSE - LSE2).abs().max().item()
+    assert d_o <= 2 * TOL and d_l <= 2 * TOL, (d_o, d_l)      # two bf16 pipelines, each within TOL of the mathematics
+    # (2) float64 rows, fp32 attention of the oracle
+    ex = _exact_qkv(coord, p, eps).float().view(B, L, 3 * C)
+    Qe, Ke, Ve = (t.reshape(B, L, H, 32) for t in torch.chunk(ex, 3, dim=-1))
+    o_ref, lse_ref = oracle.buck_swin_fwd(Qe, Ke, Ve, scopes, bs)
+    err_us, err_stored = (O.float().cpu() - o_ref).abs(), (O2.float().cpu() - o_ref).abs()
+    e_max, e_lse = err_us.max().item(), (LSE.cpu() - lse_ref).abs().max().item()
+    assert e_max <= TOL and e_lse <= TOL, (e_max, e_lse)
+    e_mean, s_mean = err_us.mean().item(), err_stored.mean().item()
+    assert e_mean <= 1.1 * s_mean + 1e-4, (e_mean, s_mean)    # no further from the mathematics than the stored pipeline
+
+
+def test_first_block_attention_unsupported_shapes_are_reported():
+    from flash3dtransformer_amd.lib import pshattn
+    z = lambda *s: torch.zeros(*s, dtype=torch.bfloat16, device=DEV)
+    assert pshattn.embed_qkv_fold(z(64, 3), None, z(64), None, 1e-5, z(192, 64), None, 1) is None        # 64-wide head
+    coord = torch.zeros(4096, 3, dtype=torch.float16, device=DEV)
+    O = torch.full((1, 4096, 2, 32), 3.0, dtype=torch.bfloat16, device=DEV)
+    LSE = torch.zeros(1, 4096, 2, dtype=torch.float32, device=DEV)
+    sc = torch.arange(4, dtype=torch.int32, device=DEV).view(torch.uint32).view(1, 4)     # one scope of 4096 tokens
+    assert not pshattn.embed_buck_swin_fwd(coord, z(2, 4, 32, 16), torch.zeros(16, device=DEV), O, LSE, sc, 1024)
+    assert (O == 3.0).all()

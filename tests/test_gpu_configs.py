@@ -79,6 +79,33 @@ def test_encoder_stage_4x120k_full_size_vs_oracle(oracle):
     assert d.mean().item() <= 0.004 and d.max().item() <= 0.5, (d.mean().item(), d.max().item())
 
 
+def test_first_block_follows_weight_changes_with_unstored_embedding():
+    """the folded LayerNorm + QKV table of the first block is rebuilt when a parameter it was made from changes"""
+    import bench_workloads as configs
+    cfg = configs.ENCODER_STAGE
+    coords, seps, _ = configs.lidar_batch(2, 20_000, 77)
+    emb, blk = configs.encoder_stage("swiglu", 77)
+    emb, blk = emb.to(DEV), blk.to(DEV)
+    c, s = configs.to_device(coords, seps, DEV)
+
+    def both():
+        with torch.no_grad():
+            stored = blk(None, emb(c, s, cfg["hash_type"]), None)
+            lazy = blk(None, emb(c, s, cfg["hash_type"], lazy=True), None)
+        return stored.float(), lazy.float()
+
+    s0, l0 = both()
+    assert blk.bwa.qkv._fold._val is not None, "the first block did not take the attention kernel that forms its own rows"
+    assert (s0 - l0).abs().mean().item() <= 0.004
+    with torch.no_grad():
+        blk.bwa.qkv.weight.mul_(-0.5)
+        blk.norm.bias.add_(0.3)
+        emb.lin.weight.mul_(1.5)
+    s1, l1 = both()
+    assert (s1 - s0).abs().mean().item() > 0.05          # the change matters ...
+    assert (s1 - l1).abs().mean().item() <= 0.004        # ... and the unstored path follows it
+
+
 def _hook_pooling_buffers(model):
     from flash3dtransformer_amd.layers.hourglass import PoolingWrapper
     seen = []
