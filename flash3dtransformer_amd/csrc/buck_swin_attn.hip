@@ -1027,30 +1027,39 @@ static int launch_attn_scope(const uint16_t* q, const uint16_t* k, const uint16_
 // x - mean(x) = E' c with E' = E minus its column means, var(x) = |E' c|^2 / C = |L c|^2 with L the upper-triangular
 // Cholesky factor of G = E'^T E' / C, and
 //   qkv = W (gamma * (x - mean) * rstd + beta) + b = rstd * (M c) + b',   M = W diag(gamma) E'  (3C x 4),  b' = W beta + b.
-// One thread per output row writes that row's 16 bf16 of the attention kernel's table: (M high parts, M low parts |
+// One wave per output row writes that row's 16 bf16 of the attention kernel's table: (M high parts, M low parts |
 // M high parts, b' high, b' low, 0, 0), to be multiplied with (c~ high, c~ high | c~ low, 1, 1, 0, 0), c~ = rstd c;
 // row position inside the head's 32-row tile = the row of the 32x32 accumulator layout that hands a lane the features
-// 8 half .. 8 half + 7 and 16 + 8 half .. 16 + 8 half + 7.  Thread 0 writes the Cholesky factor and eps.
+// 8 half .. 8 half + 7 and 16 + 8 half .. 16 + 8 half + 7.  One more wave writes the Cholesky factor and eps.
 __global__ __launch_bounds__(64) void embed_qkv_fold_kernel(
     const uint16_t* __restrict__ ew, const uint16_t* __restrict__ eb, const uint16_t* __restrict__ gamma,
     const uint16_t* __restrict__ beta, float eps, const uint16_t* __restrict__ w, const uint16_t* __restrict__ b,
     uint32_t C, uint32_t num_head, float scale_log2, uint16_t* __restrict__ table, float* __restrict__ chol) {
-  const uint32_t row = blockIdx.x * 64 + threadIdx.x;      // output feature of the projection, < 3 C
+  // one wave per output feature of the projection (block 3 C: the Cholesky factor); lanes stride over the channels
+  const uint32_t row = blockIdx.x, lane = threadIdx.x;
   auto e_at = [&](uint32_t ch, uint32_t j) {
     return j < 3 ? bf16_bits_to_float(ew[ch * 3 + j]) : (eb ? bf16_bits_to_float(eb[ch]) : 0.f);
   };
+  auto wave_sum = [&](double v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+    return v;
+  };
   double mean[4] = {0, 0, 0, 0};
-  for (uint32_t ch = 0; ch < C; ++ch)
+  for (uint32_t ch = lane; ch < C; ch += kWave)
     for (uint32_t j = 0; j < 4; ++j) mean[j] += e_at(ch, j);
-  for (uint32_t j = 0; j < 4; ++j) mean[j] /= C;
+  for (uint32_t j = 0; j < 4; ++j) mean[j] = wave_sum(mean[j]) / C;
   if (row < 3 * C) {
-    double m[4] = {0, 0, 0, 0}, bp = b ? bf16_bits_to_float(b[row]) : 0.f;
-    for (uint32_t ch = 0; ch < C; ++ch) {
+    double m[4] = {0, 0, 0, 0}, bp = 0;
+    for (uint32_t ch = lane; ch < C; ch += kWave) {
       const double wv = bf16_bits_to_float(w[(size_t)row * C + ch]);
       const double wg = wv * (gamma ? bf16_bits_to_float(gamma[ch]) : 1.f);
       for (uint32_t j = 0; j < 4; ++j) m[j] += wg * (e_at(ch, j) - mean[j]);
       if (beta) bp += wv * bf16_bits_to_float(beta[ch]);
     }
+    for (uint32_t j = 0; j < 4; ++j) m[j] = wave_sum(m[j]);
+    bp = wave_sum(bp) + (b ? bf16_bits_to_float(b[row]) : 0.f);
+    if (lane != 0) return;
     const uint32_t part = row / C, within = row % C, head = within / 32, d = within % 32;
     const uint32_t hf = (d % 16) / 8, i = d < 16 ? d % 8 : 8 + d % 8;
     const uint32_t r = (i % 4) + 8 * (i / 4) + 4 * hf;
@@ -1076,34 +1085,35 @@ __global__ __launch_bounds__(64) void embed_qkv_fold_kernel(
     } else {
       emit(part, 1.0);
     }
+    return;
   }
-  if (row == 0) {
-    double g[4][4];
-    for (int a = 0; a < 4; ++a)
-      for (int c = 0; c < 4; ++c) g[a][c] = 0;
-    for (uint32_t ch = 0; ch < C; ++ch)
-      for (int a = 0; a < 4; ++a)
-        for (int c = a; c < 4; ++c) g[a][c] += ((double)e_at(ch, a) - mean[a]) * ((double)e_at(ch, c) - mean[c]);
-    double l[4][4];
-    for (int a = 0; a < 4; ++a)
-      for (int c = 0; c < 4; ++c) l[a][c] = 0;
-    for (int a = 0; a < 4; ++a) {           // G = L^T L, row by row; a pivot that is not positive ends its row at zero
-      double piv = g[a][a] / C;
-      for (int k2 = 0; k2 < a; ++k2) piv -= l[k2][a] * l[k2][a];
-      if (!(piv > 0)) continue;
-      l[a][a] = sqrt(piv);
-      for (int c = a + 1; c < 4; ++c) {
-        double s = g[a][c] / C;
-        for (int k2 = 0; k2 < a; ++k2) s -= l[k2][a] * l[k2][c];
-        l[a][c] = s / l[a][a];
-      }
+  double g[4][4];
+  for (int a = 0; a < 4; ++a)
+    for (int c = a; c < 4; ++c) {
+      double s = 0;
+      for (uint32_t ch = lane; ch < C; ch += kWave) s += ((double)e_at(ch, a) - mean[a]) * ((double)e_at(ch, c) - mean[c]);
+      g[a][c] = wave_sum(s) / C;
     }
-    int n = 0;
-    for (int a = 0; a < 4; ++a)
-      for (int c = a; c < 4; ++c) chol[n++] = (float)l[a][c];
-    chol[10] = eps;
-    for (n = 11; n < 16; ++n) chol[n] = 0.f;
+  if (lane != 0) return;
+  double l[4][4];
+  for (int a = 0; a < 4; ++a)
+    for (int c = 0; c < 4; ++c) l[a][c] = 0;
+  for (int a = 0; a < 4; ++a) {           // G = L^T L, row by row; a pivot that is not positive ends its row at zero
+    double piv = g[a][a];
+    for (int k2 = 0; k2 < a; ++k2) piv -= l[k2][a] * l[k2][a];
+    if (!(piv > 0)) continue;
+    l[a][a] = sqrt(piv);
+    for (int c = a + 1; c < 4; ++c) {
+      double s = g[a][c];
+      for (int k2 = 0; k2 < a; ++k2) s -= l[k2][a] * l[k2][c];
+      l[a][c] = s / l[a][a];
+    }
   }
+  int n = 0;
+  for (int a = 0; a < 4; ++a)
+    for (int c = a; c < 4; ++c) chol[n++] = (float)l[a][c];
+  chol[10] = eps;
+  for (n = 11; n < 16; ++n) chol[n] = 0.f;
 }
 
 template <int D, int KT>
@@ -1203,7 +1213,7 @@ int f3d_embed_qkv_fold_bf16(const f3d_bf16_t* embed_w, const f3d_bf16_t* embed_b
   hipStream_t s = (hipStream_t)stream;
   SyncBracket sync(s);
   const float scale_log2 = 1.4426950408889634f / sqrtf((float)head_dim);
-  hipLaunchKernelGGL(embed_qkv_fold_kernel, dim3(cdiv_u32(3 * c, 64)), dim3(64), 0, s, embed_w, embed_b, gamma, beta, eps,
+  hipLaunchKernelGGL(embed_qkv_fold_kernel, dim3(3 * c + 1), dim3(64), 0, s, embed_w, embed_b, gamma, beta, eps,
                      w_qkv, b_qkv, c, num_head, scale_log2, table, chol);
   F3D_CHECK_HIP(hipGetLastError());
   return F3D_OK;
