@@ -30,7 +30,8 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 TRAFFIC_FROM = "profiles/encoder_stage_4x120k_hbm_traffic.md (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this bench's step; re-measure when a kernel changes)"
 TRAFFIC_BYTES_PER_LAUNCH = {"ln_fc1_act": 1.613e9, "ln_qkv": 1.022e9, "attention": 1.019e9,
                             "proj_residual": 0.767e9, "fc2_residual": 1.850e9, "ln_mlp_residual": 0.848e9,
-                            "proj_ln_mlp_residual": 0.876e9, "embed_ln_qkv": 0.779e9, "embed_proj_ln_mlp_residual": 0.629e9}
+                            "proj_ln_mlp_residual": 0.876e9, "embed_ln_qkv": 0.780e9, "embed_proj_ln_mlp_residual": 0.627e9,
+                            "embed_attention": 0.266e9}
 
 
 def ev_time(fn, iters, warmup=3):
