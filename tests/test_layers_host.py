@@ -67,3 +67,30 @@ def test_planner_tables_cover_every_bucket_and_say_so():
         assert getattr(t, "covers_all_rows", False)
         ids = t.view(torch.int32).flatten().tolist()
         assert sorted(ids) == list(range(total // bs))
+
+
+def test_layernorm_qkv_of_a_rank4_embedding_folds_to_four_numbers_per_feature():
+    """The identity behind the first block's attention kernel that forms Q, K, V from coordinates (float64, no GPU):
+    for x = E c with c = (x, y, z, 1),  W (gamma * (x - mean x) / sqrt(var x + eps) + beta) + b
+    = rstd (M c) + b'  with  M = W diag(gamma) E',  b' = W beta + b,  rstd = 1 / sqrt(|L c|^2 + eps),
+    E' = E minus its column means and L the upper Cholesky factor of E'^T E' / C -- checked against LayerNorm and the
+    two linear layers evaluated as the reference's module sequence writes them (psh_ops.py:64-68, stage.py:94-96)."""
+    import torch
+    g = torch.Generator().manual_seed(3)
+    C, N, eps = 96, 500, 1e-5
+    rnd = lambda *s: torch.randn(*s, generator=g, dtype=torch.float64)
+    ew, eb, gamma, beta, w, b = rnd(C, 3), rnd(C), 1 + 0.2 * rnd(C), 0.3 * rnd(C), rnd(3 * C, C) / C ** 0.5, rnd(3 * C)
+    c3 = rnd(N, 3) * torch.tensor([40.0, 40.0, 3.0], dtype=torch.float64)
+    x = torch.nn.functional.linear(c3, ew, eb)
+    want = torch.nn.functional.linear(torch.nn.functional.layer_norm(x, (C,), gamma, beta, eps), w, b)
+    E = torch.cat([ew, eb[:, None]], 1)
+    Ep = E - E.mean(0, keepdim=True)
+    L = torch.linalg.cholesky(Ep.T @ Ep / C).T
+    M, bp = (w * gamma[None, :]) @ Ep, w @ beta + b
+    c = torch.cat([c3, torch.ones(N, 1, dtype=torch.float64)], 1)
+    rstd = 1.0 / torch.sqrt((c @ L.T).pow(2).sum(1, keepdim=True) + eps)
+    got = rstd * (c @ M.T) + bp
+    assert (got - want).abs().max().item() <= 1e-9 * max(1.0, want.abs().max().item())
+    # a dropped mean, a missing gamma or the uncentred Gram matrix are not the same function
+    assert ((rstd * (c @ ((w * gamma[None, :]) @ E).T) + bp) - want).abs().max().item() > 1e-3
+    assert ((rstd * (c @ (w @ Ep).T) + bp) - want).abs().max().item() > 1e-3
