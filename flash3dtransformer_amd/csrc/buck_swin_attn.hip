@@ -6,8 +6,9 @@
 // rows of the scope's buckets, plus the natural-log LSE.
 //
 // Streaming kernel (any scope size, head_dim up to 128): one 256-thread workgroup (4 waves) per (batch, scope,
-// head, 128-query block); each wave owns 32 query rows.  K and V of the scope stream through LDS in tiles of KT keys (K row-major,
-// V transposed), prefetched into registers one tile ahead.  Scores are computed TRANSPOSED,
+// head, 128-query block); each wave owns 32 query rows.  K and V of the scope stream through LDS in tiles of KT keys (K row-major;
+// V row-major too for 32-wide heads, read with the transposing LDS load, and stored transposed for the other widths),
+// prefetched into registers one tile ahead.  Scores are computed TRANSPOSED,
 // St = K Qt with v_mfma_f32_32x32x16_bf16, so that a lane holds 16 keys of ONE query: the softmax
 // max / sum run inside the lane plus one exchange with lane^32, and the bf16 P values are already in
 // the B-operand layout of the second MFMA, Ot += Vt Pt (keys are consumed in the permuted order the
@@ -25,6 +26,10 @@ namespace f3d {
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16_t;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
+
+typedef short i16x4_t __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) void lds_void_t;
+typedef __attribute__((address_space(3))) i16x4_t lds_i16x4_t;
 
 constexpr int kAttnThreads = 256;
 constexpr int kQBlock = 128;  // query rows per workgroup
@@ -44,7 +49,11 @@ struct AttnCfg {
   static constexpr int VROW = KT + 8;                   // padded LDS row of Vt (elements)
   static constexpr int CHUNKS = KT * D / 8;             // 16-byte chunks per K (or V) tile
   static constexpr int NCH = (CHUNKS + kAttnThreads - 1) / kAttnThreads;
-  static constexpr int LDS_BYTES = (KT * KROW + D * VROW) * 2;   // plus 8 bytes per scope entry
+  // 32-wide heads keep V row-major [KT][D] (unpadded, as the global rows) and read it with the transposing LDS load;
+  // the other widths stage a transposed copy [D][VROW]
+  static constexpr bool V_ROW_MAJOR = D == 32;
+  static constexpr int V_ELEMS = V_ROW_MAJOR ? KT * D : D * VROW;
+  static constexpr int LDS_BYTES = (KT * KROW + V_ELEMS) * 2;   // plus 8 bytes per scope entry
 };
 
 template <int D, int KT>
@@ -59,7 +68,7 @@ __global__ __launch_bounds__(kAttnThreads) void buck_swin_fwd_kernel(
   uint16_t* sVt = lds_attn + KT * C::KROW;  // [D][VROW]
   // per scope entry: bucket id and number of valid keys (0 for an id outside the sequence), read once
   // from global memory so that the tile loop never waits on a scalar load
-  uint32_t* s_bucket = reinterpret_cast<uint32_t*>(lds_attn + KT * C::KROW + D * C::VROW);
+  uint32_t* s_bucket = reinterpret_cast<uint32_t*>(lds_attn + KT * C::KROW + C::V_ELEMS);
   int32_t* s_len = reinterpret_cast<int32_t*>(s_bucket + scope_size);
 
   // XCD-aware remap: hardware deals consecutive workgroup ids round-robin to the 8 XCDs
@@ -139,15 +148,30 @@ __global__ __launch_bounds__(kAttnThreads) void buck_swin_fwd_kernel(
       if (C::CHUNKS % kAttnThreads == 0 || c < (uint32_t)C::CHUNKS) {
         const uint32_t key = c / (D / 8), dc = c % (D / 8);
         *reinterpret_cast<u32x4_t*>(sK + key * C::KROW + dc * 8) = rk[i];
-        const uint32_t pos = (key & ~15u) | vperm16(key & 15u);
-        uint16_t* col = sVt + (dc * 8) * C::VROW + pos;
+        if constexpr (C::V_ROW_MAJOR) {
+          *reinterpret_cast<u32x4_t*>(sVt + key * D + dc * 8) = rv[i];
+        } else {
+          const uint32_t pos = (key & ~15u) | vperm16(key & 15u);
+          uint16_t* col = sVt + (dc * 8) * C::VROW + pos;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          col[(2 * e) * C::VROW] = (uint16_t)(rv[i][e] & 0xFFFFu);
-          col[(2 * e + 1) * C::VROW] = (uint16_t)(rv[i][e] >> 16);
+          for (int e = 0; e < 4; ++e) {
+            col[(2 * e) * C::VROW] = (uint16_t)(rv[i][e] & 0xFFFFu);
+            col[(2 * e + 1) * C::VROW] = (uint16_t)(rv[i][e] >> 16);
+          }
         }
       }
     }
+  };
+  // V^T operand of the 16 keys [key0, key0 + 16) of the staged tile (32-wide heads): the transposing load hands lane i
+  // of a 16-lane block column i % 4 of the four 8-byte pieces addressed by lanes i / 4 + {0, 4, 8, 12}; with lane r
+  // pointing at key r / 4, features 4 (r % 4) .., slots 0..3 of a lane are keys 4 half + 0..3, slots 4..7 the same + 8:
+  // the key order of the packed P values
+  const uint32_t v_tr_off = (4u * half + (lane & 15u) / 4u) * D + 16u * ((lane >> 4) & 1u) + 4u * (lane & 3u);   // elements
+  auto v_frag_tr = [&](uint32_t key0) {
+    const uint16_t* vt = sVt + key0 * D + v_tr_off;
+    const i16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_t*)vt);
+    const i16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_t*)(vt + 8 * D));
+    return __builtin_bit_cast(bf16x8_t, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
   };
 
   // ---- fast pass: softmax with the reference fixed at zero.  Q is pre-multiplied by log2(e) / sqrt(D) (one bf16
@@ -217,7 +241,9 @@ __global__ __launch_bounds__(kAttnThreads) void buck_swin_fwd_kernel(
 #pragma unroll
           for (int dt = 0; dt < C::DT; ++dt) {
             bf16x8_t vf;
-            if (D >= 32 || lq < (uint32_t)D) {
+            if constexpr (C::V_ROW_MAJOR) {
+              vf = v_frag_tr(j * 32 + kk * 16);
+            } else if (D >= 32 || lq < (uint32_t)D) {
               vf = *reinterpret_cast<const bf16x8_t*>(sVt + (dt * 32 + lq) * C::VROW + j * 32 + kk * 16 + half * 8);
             } else {
 #pragma unroll
@@ -329,7 +355,9 @@ __global__ __launch_bounds__(kAttnThreads) void buck_swin_fwd_kernel(
   #pragma unroll
           for (int dt = 0; dt < C::DT; ++dt) {
             bf16x8_t vf;
-            if (D >= 32 || lq < (uint32_t)D) {
+            if constexpr (C::V_ROW_MAJOR) {
+              vf = v_frag_tr(j * 32 + kk * 16);
+            } else if (D >= 32 || lq < (uint32_t)D) {
               vf = *reinterpret_cast<const bf16x8_t*>(sVt + (dt * 32 + lq) * C::VROW + j * 32 + kk * 16 + half * 8);
             } else {
   #pragma unroll
@@ -375,9 +403,6 @@ __device__ __forceinline__ void static_for(F&& f) {
 }
 
 constexpr int kResMaxScope = 4;  // buckets per scope: at most 512 tokens in buckets of at least 128
-typedef short i16x4_t __attribute__((ext_vector_type(4)));
-typedef __attribute__((address_space(3))) void lds_void_t;
-typedef __attribute__((address_space(3))) i16x4_t lds_i16x4_t;
 
 // 16 bytes per lane from global memory straight into LDS: lane l of the wave lands at lds + 16 l.
 // gbase and lds are wave-uniform, voff is the lane's byte offset from gbase.
