@@ -22,7 +22,6 @@
 namespace f3d {
 
 constexpr int kPshThreads = 256;
-constexpr int kPshWaves = kPshThreads / kWave;
 
 // Position inside a tile of the point handled by (wave w, round j, lane l): each wave owns a
 // contiguous run of 64*ITEMS points and walks it 64 at a time, so (j, l) order is input order.
