@@ -61,7 +61,8 @@ __global__ __launch_bounds__(kAttnThreads) void buck_swin_fwd_kernel(
     const uint16_t* __restrict__ q, const uint16_t* __restrict__ k, const uint16_t* __restrict__ v, uint32_t ld,
     uint16_t* __restrict__ o, float* __restrict__ lse, const uint32_t* __restrict__ scope_buckets,
     uint32_t num_scope, uint32_t scope_size, uint32_t bs, uint32_t seq_len, uint32_t num_head,
-    const int32_t* __restrict__ kv_len, float scale_log2, uint32_t n_work, uint32_t work_per_xcd) {
+    const int32_t* __restrict__ kv_len, float scale_log2, uint32_t n_work, uint32_t work_per_xcd,
+    uint32_t only_marked) {
   using C = AttnCfg<D, KT>;
   extern __shared__ __attribute__((aligned(16))) uint16_t lds_attn[];
   uint16_t* sK = lds_attn;                  // [KT][KROW]
@@ -100,6 +101,12 @@ __global__ __launch_bounds__(kAttnThreads) void buck_swin_fwd_kernel(
   const uint32_t q_row = q_bucket * bs + q_in_bucket;
   const size_t tok0 = (size_t)batch * seq_len;
   const int32_t q_valid_len = s_len[q_local / bs];
+  // only_marked: this launch follows the bucket-streaming scope kernel, which leaves a NaN in the LSE of the rows whose
+  // sums left the range of its fixed-reference softmax; only workgroups that own such a row go on (uniform decision)
+  if (only_marked) {
+    const float mark = lse[(tok0 + q_row) * num_head + head];
+    if (!__syncthreads_or(mark != mark ? 1 : 0)) return;
+  }
 
   bf16x8_t qf[C::KSTEPS];
   {
@@ -475,7 +482,12 @@ struct ScopeGen {
   const float* chol;       // L00 L01 L02 L03 L11 L12 L13 L22 L23 L33 eps
 };
 
-template <int D, int T, int WAVES, bool GEN = false>
+// STREAM: scopes of more than T tokens in buckets of exactly T rows.  An item is (batch, scope, head, query bucket); the
+// scope's key buckets pass through the two LDS buffers one after the other (the next one streams in while the current one
+// is consumed, exactly as the next item does otherwise) and the accumulators live across them.  Fixed-reference softmax
+// only: a wave whose row sums leave its range writes NaN into its rows' LSE instead of a result, and the launcher runs
+// the streaming kernel after this one for the workgroups that own such rows.
+template <int D, int T, int WAVES, bool GEN = false, bool STREAM = false>
 __global__ __launch_bounds__(64 * WAVES) void buck_swin_fwd_scope_kernel(
     const uint16_t* __restrict__ q, const uint16_t* __restrict__ k, const uint16_t* __restrict__ v, uint32_t ld,
     uint16_t* __restrict__ o, float* __restrict__ lse, const uint32_t* __restrict__ scope_buckets,
@@ -484,6 +496,8 @@ __global__ __launch_bounds__(64 * WAVES) void buck_swin_fwd_scope_kernel(
     uint32_t n_slots, ScopeGen gen) {
   constexpr int QB = T / (32 * WAVES);     // 32-query blocks per wave
   static_assert(!GEN || (QB == 1 && D == 32), "rows formed in the kernel: one 32-row block per wave, 32-wide heads");
+  static_assert(!(GEN && STREAM), "rows are formed in the kernel for resident scopes only");
+  const uint32_t n_kb = STREAM ? scope_size : 1u;       // key buckets an item walks
   constexpr int KSTEPS = D / 16;
   constexpr int CPK = D / 8;               // 16-byte chunks per row
   constexpr int ROWB = D * 2;              // bytes per K / V row in LDS
@@ -535,13 +549,22 @@ __global__ __launch_bounds__(64 * WAVES) void buck_swin_fwd_scope_kernel(
   // advances by a mixed-radix addition with carries, one division at the start and none per item (the scalar unit
   // is shared by all waves of a SIMD, and every wave does this bookkeeping).
   struct Pos {
-    uint32_t head, scope, batch;
+    uint32_t qb, head, scope, batch;      // qb: the item's query bucket inside its scope (STREAM; 0 otherwise)
   };
-  const uint32_t d_head = n_slots % num_head, d_scope = (n_slots / num_head) % num_scope,
-                 d_batch = n_slots / (num_head * num_scope);
+  // STREAM: the query bucket is the fastest index, so that the items that share a scope's K and V run at the same time
+  // on one XCD
+  const uint32_t slots_h = n_slots / n_kb;
+  const uint32_t d_qb = n_slots % n_kb, d_head = slots_h % num_head, d_scope = (slots_h / num_head) % num_scope,
+                 d_batch = slots_h / (num_head * num_scope);
   auto advance = [&](Pos p) {
-    p.head += d_head;
-    uint32_t carry = p.head >= num_head ? 1u : 0u;
+    uint32_t carry = 0;
+    if constexpr (STREAM) {
+      p.qb += d_qb;
+      carry = p.qb >= n_kb ? 1u : 0u;
+      p.qb -= carry ? n_kb : 0u;
+    }
+    p.head += d_head + carry;
+    carry = p.head >= num_head ? 1u : 0u;
     p.head -= carry ? num_head : 0u;
     p.scope += d_scope + carry;
     carry = p.scope >= num_scope ? 1u : 0u;
@@ -572,10 +595,12 @@ __global__ __launch_bounds__(64 * WAVES) void buck_swin_fwd_scope_kernel(
   // the wave's first row (valid when kv_wanted()).  Issued as inline assembly on purpose: the compiler then keeps no
   // record of LDS writes in flight and puts no full vmcnt wait in front of the fragment reads (they read the OTHER
   // buffer).  The wait that matters is the explicit one before the per-item barrier.
-  const uint32_t kv_row0 = wave * (T / WAVES), kv_j = kv_row0 / bs;     // a wave's rows never straddle buckets
-  auto kv_wanted = [&](const Scope& sc) { return len_of(sc, kv_j) > 0; };
-  auto kv_base = [&](const Pos& p, const Scope& sc) {
-    return in_base(p) * 2u + (size_t)(bucket_of(sc, kv_j) * bs + (kv_row0 - kv_j * bs)) * ld * 2u;
+  // (STREAM: the key bucket kb of the sub-item, whose T rows the waves share)
+  const uint32_t kv_row0 = wave * (T / WAVES), kv_j0 = STREAM ? 0u : kv_row0 / bs;     // a wave's rows never straddle buckets
+  auto kv_wanted = [&](const Scope& sc, uint32_t kb) { return len_of(sc, STREAM ? kb : kv_j0) > 0; };
+  auto kv_base = [&](const Pos& p, const Scope& sc, uint32_t kb) {
+    const uint32_t j = STREAM ? kb : kv_j0;
+    return in_base(p) * 2u + (size_t)(bucket_of(sc, j) * bs + (kv_row0 - kv_j0 * bs)) * ld * 2u;
   };
   // LDS addresses as plain 32-bit numbers (a generic pointer costs a null check per conversion)
   const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)lds_scope;
@@ -586,21 +611,23 @@ __global__ __launch_bounds__(64 * WAVES) void buck_swin_fwd_scope_kernel(
     else lds_dma16_at(reinterpret_cast<const char*>(v) + g, dma_v, buf_addr + OPB + blk * 1024);
   };
   // row inside the sequence of query lq of block b (0 when the scope entry names no bucket of the sequence)
-  auto q_row_of = [&](const Scope& sc, uint32_t b) {
-    const uint32_t q_local = (wave * QB + b) * 32u, qj = q_local / bs, id = bucket_of(sc, qj);
+  auto q_row_of = [&](const Pos& p, const Scope& sc, uint32_t b) {
+    const uint32_t q_local = (wave * QB + b) * 32u, qj = STREAM ? 0u : q_local / bs;
+    const uint32_t id = bucket_of(sc, STREAM ? p.qb : qj);
     return (id < n_bucket ? id : 0u) * bs + (q_local - qj * bs) + lq;
   };
   u32x4_t qraw[QB][KSTEPS];
   auto issue_q_one = [&](const Pos& p, const Scope& sc, auto b_c) {
     constexpr uint32_t b = decltype(b_c)::value;
     const char* qp = reinterpret_cast<const char*>(q + in_base(p));
-    const uint32_t off = (q_row_of(sc, b) * ld + half * 8u) * 2u;      // fits 32 bits (checked by the host)
+    const uint32_t off = (q_row_of(p, sc, b) * ld + half * 8u) * 2u;      // fits 32 bits (checked by the host)
 #pragma unroll
     for (int ks = 0; ks < KSTEPS; ++ks) qraw[b][ks] = *reinterpret_cast<const u32x4_t*>(qp + (off + ks * 32u));
   };
 
   // ---- prologue: the first item's scope, K / V / Q; the second item's bucket ids ----
-  Pos p_cur = {item_lo % num_head, (item_lo / num_head) % num_scope, item_lo / (num_head * num_scope)};
+  const uint32_t item_h = item_lo / n_kb;
+  Pos p_cur = {item_lo % n_kb, item_h % num_head, (item_h / num_head) % num_scope, item_h / (num_head * num_scope)};
   Pos p_nxt = advance(p_cur);
   Scope cur, nxt;
   cur.ids = load_ids(p_cur);
@@ -612,7 +639,7 @@ __global__ __launch_bounds__(64 * WAVES) void buck_swin_fwd_scope_kernel(
   // Q / K / V tiles
   uint16_t g_c[3] = {0, 0, 0};
   u32x4_t g_a[3];
-  auto gen_row = [&](const Pos& p, const Scope& sc) { return (size_t)p.batch * seq_len + q_row_of(sc, 0); };
+  auto gen_row = [&](const Pos& p, const Scope& sc) { return (size_t)p.batch * seq_len + q_row_of(p, sc, 0); };
   auto gen_tile_ptr = [&](const Pos& p, uint32_t tile) {
     return reinterpret_cast<const u32x4_t*>(gen.table + (((size_t)p.head * 4 + tile) * 32 + lq) * 16 + half * 8);
   };
@@ -678,8 +705,8 @@ __global__ __launch_bounds__(64 * WAVES) void buck_swin_fwd_scope_kernel(
     issue_gen(p_cur, cur);
   } else {
     static_for<QB>([&](auto b_c) { issue_q_one(p_cur, cur, b_c); });
-    if (kv_wanted(cur)) {
-      const size_t goff = kv_base(p_cur, cur);
+    if (kv_wanted(cur, 0)) {
+      const size_t goff = kv_base(p_cur, cur, 0);
 #pragma unroll
       for (uint32_t i = 0; i < 2u * BPW; ++i) issue_kv_one(goff, i, lds0);
     }
@@ -687,12 +714,24 @@ __global__ __launch_bounds__(64 * WAVES) void buck_swin_fwd_scope_kernel(
     __syncthreads();
   }
 
-  for (uint32_t n = 0; n < my_items; ++n) {
+  // One turn of the loop is a sub-item: an item, or (STREAM) one key bucket of an item.  What lives across an item's
+  // key buckets is declared out here.
+  uint32_t n = 0, kb = 0;           // item counter, key bucket inside the item
+  bf16x8_t qf[QB][KSTEPS];
+  uint32_t q_row[QB];
+  bool q_live[QB], q_exists[QB];
+  int32_t q_len[QB];
+  f32x16_t acc[QB];
+  f32x4_t lacc[QB];
+  float m_ref[QB], l_fin[QB];
+  bool any_keys = false;            // STREAM: some key bucket of the item so far held a valid key
+  const uint32_t n_sub = my_items * n_kb;
+  for (uint32_t sub = 0; sub < n_sub; ++sub) {
+    const bool first = !STREAM || kb == 0, last = !STREAM || kb + 1 == n_kb;
     const bool has_next = n + 1 < my_items;
-    const char* const sbuf = lds_scope + (n & 1u) * BUF;
+    const char* const sbuf = lds_scope + (sub & 1u) * BUF;
 
     // Q of this item arrived during the previous one: scale into the exponent's units and round once
-    bf16x8_t qf[QB][KSTEPS];
     if constexpr (GEN) {
       // form the item's Q (kept in registers), K and V (the wave's 32 rows of this item's LDS buffer: the buffer's
       // last readers, two items back, passed the previous barrier), then meet the other waves
@@ -708,7 +747,7 @@ __global__ __launch_bounds__(64 * WAVES) void buck_swin_fwd_scope_kernel(
       }
       if (has_next) issue_gen(p_nxt, nxt);
       wg_barrier_lds();
-    } else {
+    } else if (first) {
 #pragma unroll
     for (int b = 0; b < QB; ++b)
 #pragma unroll
@@ -725,15 +764,17 @@ __global__ __launch_bounds__(64 * WAVES) void buck_swin_fwd_scope_kernel(
     // microsecond or two with the SIMDs idle): `vm_next` counts those already issued, 2 BPW direct loads of K / V
     // first, then the Q rows of the wave's QB blocks.
     constexpr uint32_t VM_OPS = GEN ? 0u : 2u * BPW + QB, VM_PER_STEP = (VM_OPS + NSTEP / 2 - 1) / (NSTEP / 2);   // all in the first half
-    const bool nxt_kv = has_next && kv_wanted(nxt);
-    const size_t nxt_goff = nxt_kv ? kv_base(p_nxt, nxt) : 0;
-    const uint32_t nxt_buf = lds0 + ((n + 1) & 1u) * BUF;
+    // (STREAM: the next sub-item is the item's next key bucket, or the first one of the next item together with its Q)
+    const bool nx_same = STREAM && !last;
+    const bool nxt_kv = nx_same ? kv_wanted(cur, kb + 1) : (has_next && kv_wanted(nxt, 0));
+    const size_t nxt_goff = !nxt_kv ? 0 : (nx_same ? kv_base(p_cur, cur, kb + 1) : kv_base(p_nxt, nxt, 0));
+    const uint32_t nxt_buf = lds0 + ((sub + 1) & 1u) * BUF;
     auto issue_vm = [&](auto i_c) {
       constexpr uint32_t i = decltype(i_c)::value;
       if constexpr (i < 2u * BPW) {
         if (nxt_kv) issue_kv_one(nxt_goff, i, nxt_buf);
       } else if constexpr (i < VM_OPS) {
-        if (has_next) issue_q_one(p_nxt, nxt, std::integral_constant<uint32_t, i - 2u * BPW>{});
+        if (has_next && last) issue_q_one(p_nxt, nxt, std::integral_constant<uint32_t, i - 2u * BPW>{});
       }
     };
     uint32_t vm_next = 0;
@@ -742,30 +783,23 @@ __global__ __launch_bounds__(64 * WAVES) void buck_swin_fwd_scope_kernel(
     nxt2.ids = n + 2 < my_items ? load_ids(p_nxt2) : 0xFFFFFFFFu;
 
     // per block: do its rows exist / are they valid (uniform), how many of them, which rows
-    uint32_t q_row[QB];
-    bool q_live[QB], q_exists[QB];
-    int32_t q_len[QB];
+    if (first) {
+      any_keys = false;
 #pragma unroll
-    for (int b = 0; b < QB; ++b) {
-      const uint32_t q_local = (wave * QB + b) * 32u, qj = q_local / bs;
-      const int32_t in_b = (int32_t)(q_local - qj * bs);
-      q_exists[b] = bucket_of(cur, qj) < n_bucket;
-      q_len[b] = len_of(cur, qj) - in_b;               // valid rows of the block, counted from its first row
-      q_live[b] = q_exists[b] && q_len[b] > 0;
-      q_row[b] = q_row_of(cur, b);
-    }
-
-    f32x16_t acc[QB];
-    f32x4_t lacc[QB];
-    float m_ref[QB], l_fin[QB];
+      for (int b = 0; b < QB; ++b) {
+        const uint32_t q_local = (wave * QB + b) * 32u, qj = STREAM ? p_cur.qb : q_local / bs;
+        const int32_t in_b = (int32_t)(STREAM ? q_local : q_local - qj * bs);
+        q_exists[b] = bucket_of(cur, qj) < n_bucket;
+        q_len[b] = len_of(cur, qj) - in_b;               // valid rows of the block, counted from its first row
+        q_live[b] = q_exists[b] && q_len[b] > 0;
+        q_row[b] = q_row_of(p_cur, cur, b);
+        m_ref[b] = 0.f;
+        l_fin[b] = 0.f;
 #pragma unroll
-    for (int b = 0; b < QB; ++b) {
-      m_ref[b] = 0.f;
-      l_fin[b] = 0.f;
+        for (int i = 0; i < 4; ++i) lacc[b][i] = 0.f;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) lacc[b][i] = 0.f;
-#pragma unroll
-      for (int i = 0; i < 16; ++i) acc[b][i] = 0.f;
+        for (int i = 0; i < 16; ++i) acc[b][i] = 0.f;
+      }
     }
 
     auto load_k = [&](uint32_t st, bf16x8_t (&kf)[KSTEPS]) {
@@ -807,15 +841,17 @@ __global__ __launch_bounds__(64 * WAVES) void buck_swin_fwd_scope_kernel(
 
     // ---- fast pass: scopes whose keys are all valid, and one-bucket scopes with a valid prefix (steps past it are
     //      skipped, the boundary step gets -inf scores: 2^-inf = 0 exactly) ----
-    const bool any_valid = __ballot(cur.len > 0) != 0;
-    const bool all_full = __ballot(lane < scope_size && cur.len != (int32_t)bs) == 0;
-    const int32_t len0 = len_of(cur, 0);
+    // (STREAM: the sub-item's key bucket stands where a one-bucket scope stands otherwise)
+    const int32_t len0 = len_of(cur, STREAM ? kb : 0u);
+    const bool any_valid = STREAM ? len0 > 0 : __ballot(cur.len > 0) != 0;
+    const bool all_full = STREAM ? len0 == (int32_t)bs : __ballot(lane < scope_size && cur.len != (int32_t)bs) == 0;
     bool any_live = false;
 #pragma unroll
     for (int b = 0; b < QB; ++b) any_live = any_live || q_live[b];
-    bool redo = false;
+    bool redo = false, failed = false;
     if (any_valid && any_live) {
-      redo = !(all_full || scope_size == 1);
+      any_keys = true;
+      redo = !(all_full || scope_size == 1 || STREAM);
       if (!redo) {
         const uint32_t n_full = all_full ? NSTEP : (uint32_t)len0 / 32u;        // steps whose 32 keys are all valid
         const int32_t tail_keys = all_full ? 0 : len0 - (int32_t)n_full * 32;   // valid keys of the step after them
@@ -880,10 +916,22 @@ __global__ __launch_bounds__(64 * WAVES) void buck_swin_fwd_scope_kernel(
           });
         }
         // redo with a moving reference where a row sum left the safe range (also catches inf / nan)
+        if constexpr (!STREAM) {
+#pragma unroll
+          for (int b = 0; b < QB; ++b) {
+            l_fin[b] = __shfl(lacc[b][0], l_src, kWave);
+            redo = redo || (q_live[b] && __ballot(!(l_fin[b] > 0x1p-24f) || !(l_fin[b] < 0x1p24f)) != 0);
+          }
+        }
+      }
+    }
+    if constexpr (STREAM) {
+      // the item's sums are complete after its last key bucket: out of range -> the rows are marked for the other kernel
+      if (last && any_keys) {
 #pragma unroll
         for (int b = 0; b < QB; ++b) {
           l_fin[b] = __shfl(lacc[b][0], l_src, kWave);
-          redo = redo || (q_live[b] && __ballot(!(l_fin[b] > 0x1p-24f) || !(l_fin[b] < 0x1p24f)) != 0);
+          failed = failed || (q_live[b] && __ballot(!(l_fin[b] > 0x1p-24f) || !(l_fin[b] < 0x1p24f)) != 0);
         }
       }
     }
@@ -902,7 +950,7 @@ __global__ __launch_bounds__(64 * WAVES) void buck_swin_fwd_scope_kernel(
 #pragma unroll
           for (int ks = 0; ks < KSTEPS; ++ks) qr[ks] = __builtin_bit_cast(bf16x8_t, pack_tile(tq, ks));
         } else {
-          const char* qp = reinterpret_cast<const char*>(q + in_base(p_cur)) + (q_row_of(cur, b) * ld + half * 8u) * 2u;
+          const char* qp = reinterpret_cast<const char*>(q + in_base(p_cur)) + (q_row_of(p_cur, cur, b) * ld + half * 8u) * 2u;
 #pragma unroll
           for (int ks = 0; ks < KSTEPS; ++ks) qr[ks] = *reinterpret_cast<const bf16x8_t*>(qp + ks * 32u);
         }
@@ -980,7 +1028,13 @@ __global__ __launch_bounds__(64 * WAVES) void buck_swin_fwd_scope_kernel(
     char* const op = reinterpret_cast<char*>(o + obase * D);
 #pragma unroll
     for (int b = 0; b < QB; ++b) {
+      if (!last) continue;                 // STREAM: more key buckets to come
       if (!q_exists[b]) continue;          // a scope entry outside the sequence names no rows
+      if (STREAM && failed) {              // no result: the mark the streaming kernel looks for
+        if (half == 0)
+          *reinterpret_cast<float*>(reinterpret_cast<char*>(lse + obase) + q_row[b] * num_head * 4u) = __builtin_nanf("");
+        continue;
+      }
       const float l_tot = q_live[b] ? l_fin[b] : 0.f;
       const bool row_ok = (int32_t)lq < q_len[b] && l_tot > 0.f;
       const float inv = row_ok ? 1.0f / l_tot : 0.f;
@@ -1001,24 +1055,30 @@ __global__ __launch_bounds__(64 * WAVES) void buck_swin_fwd_scope_kernel(
             row_ok ? (m_ref[b] + __builtin_amdgcn_logf(l_tot)) * ln2 : 0.f;
       }
     }
-    cur = nxt;
-    nxt = nxt2;
-    p_cur = p_nxt;
-    p_nxt = p_nxt2;
+    if (last) {
+      cur = nxt;
+      nxt = nxt2;
+      p_cur = p_nxt;
+      p_nxt = p_nxt2;
+      ++n;
+      kb = 0;
+    } else {
+      ++kb;
+    }
     // the next buffer is complete; this buffer is free for the item after next.  Not __syncthreads(): that would wait
     // for the output stores just issued.  (GEN: the barrier after an item's rows are formed does both jobs.)
     if constexpr (!GEN) wg_barrier_lds();
   }
 }
 
-template <int D, int T, int WAVES, bool GEN = false>
+template <int D, int T, int WAVES, bool GEN = false, bool STREAM = false>
 static int launch_attn_scope(const uint16_t* q, const uint16_t* k, const uint16_t* v, uint32_t ld, uint16_t* o, float* lse,
                              const uint32_t* scope_buckets, uint32_t num_scope, uint32_t scope_size, uint32_t bs,
                              uint32_t batch, uint32_t seq_len, uint32_t num_head, const int32_t* kv_len, int device,
                              hipStream_t s, ScopeGen gen = ScopeGen{nullptr, nullptr, nullptr}) {
-  const uint64_t n_items64 = (uint64_t)batch * num_scope * num_head;
+  const uint64_t n_items64 = (uint64_t)batch * num_scope * num_head * (STREAM ? scope_size : 1u);
   if (n_items64 == 0) return F3D_OK;
-  if (n_items64 > 0x7FFFFFF0ull) {
+  if (n_items64 > 0x7FFFFFF0ull / (STREAM ? scope_size : 1u)) {
     set_error("attention problem too large for one launch (%llu items)", (unsigned long long)n_items64);
     return F3D_ERR_INVALID;
   }
@@ -1028,9 +1088,9 @@ static int launch_attn_scope(const uint16_t* q, const uint16_t* k, const uint16_
   static int wg_per_cu[64] = {};
   int per_cu = (device >= 0 && device < 64) ? wg_per_cu[device] : 0;
   if (per_cu == 0) {
-    F3D_CHECK_HIP(hipFuncSetAttribute((const void*)buck_swin_fwd_scope_kernel<D, T, WAVES, GEN>,
+    F3D_CHECK_HIP(hipFuncSetAttribute((const void*)buck_swin_fwd_scope_kernel<D, T, WAVES, GEN, STREAM>,
                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    F3D_CHECK_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, buck_swin_fwd_scope_kernel<D, T, WAVES, GEN>,
+    F3D_CHECK_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, buck_swin_fwd_scope_kernel<D, T, WAVES, GEN, STREAM>,
                                                                64 * WAVES, lds));
     if (per_cu < 1) per_cu = 1;
     if (device >= 0 && device < 64) wg_per_cu[device] = per_cu;
@@ -1041,7 +1101,7 @@ static int launch_attn_scope(const uint16_t* q, const uint16_t* k, const uint16_
   const uint32_t items_per_xcd = cdiv_u32(n_items, kNumXcd);
   const uint32_t n_slots = std::max(1u, std::min((uint32_t)n_cu * (uint32_t)per_cu / kNumXcd, items_per_xcd));
   const float scale_log2 = 1.4426950408889634f / sqrtf((float)D);
-  hipLaunchKernelGGL((buck_swin_fwd_scope_kernel<D, T, WAVES, GEN>), dim3(n_slots * kNumXcd), dim3(64 * WAVES), lds, s, q, k,
+  hipLaunchKernelGGL((buck_swin_fwd_scope_kernel<D, T, WAVES, GEN, STREAM>), dim3(n_slots * kNumXcd), dim3(64 * WAVES), lds, s, q, k,
                      v, ld, o, lse, scope_buckets, num_scope, scope_size, bs, seq_len, num_head, kv_len, scale_log2,
                      n_items, items_per_xcd, n_slots, gen);
   return F3D_OK;
@@ -1144,7 +1204,8 @@ __global__ __launch_bounds__(64) void embed_qkv_fold_kernel(
 template <int D, int KT>
 static int launch_attn(const uint16_t* q, const uint16_t* k, const uint16_t* v, uint32_t ld, uint16_t* o, float* lse,
                        const uint32_t* scope_buckets, uint32_t num_scope, uint32_t scope_size, uint32_t bs,
-                       uint32_t batch, uint32_t seq_len, uint32_t num_head, const int32_t* kv_len, hipStream_t s) {
+                       uint32_t batch, uint32_t seq_len, uint32_t num_head, const int32_t* kv_len, hipStream_t s,
+                       uint32_t only_marked = 0) {
   using C = AttnCfg<D, KT>;
   const uint64_t n_work64 = (uint64_t)batch * num_scope * num_head * (scope_size * bs / kQBlock);
   if (n_work64 == 0) return F3D_OK;
@@ -1158,7 +1219,7 @@ static int launch_attn(const uint16_t* q, const uint16_t* k, const uint16_t* v, 
   hipLaunchKernelGGL((buck_swin_fwd_kernel<D, KT>), dim3(per_xcd * kNumXcd), dim3(kAttnThreads),
                      C::LDS_BYTES + scope_size * 8, s, q, k,
                      v, ld, o, lse, scope_buckets, num_scope, scope_size, bs, seq_len, num_head, kv_len, scale_log2,
-                     n_work, per_xcd);
+                     n_work, per_xcd, only_marked);
   return F3D_OK;
 }
 
@@ -1202,6 +1263,25 @@ int f3d_buck_swin_fwd_strided(const f3d_bf16_t* q, const f3d_bf16_t* k, const f3
       if (scope_tokens == 256) F3D_RES(32, 256); else F3D_RES(32, 512);
     }
 #undef F3D_RES
+    if (rc != F3D_OK) return rc;
+    F3D_CHECK_HIP(hipGetLastError());
+    return F3D_OK;
+  }
+  // larger scopes in buckets of 256 / 512 rows with 32-wide heads (the reference model's scopes of 8 buckets of 512):
+  // the scope-resident kernel with the key buckets streaming through its two LDS buffers, then the streaming kernel for
+  // the rows it marked (sums outside the range of the fixed-reference softmax), which are rare
+  if (head_dim == 32 && (bucket_size == 256 || bucket_size == 512) && scope_tokens > 512 && scope_size <= 64 &&
+      (uint64_t)seq_len * qkv_row_stride * 2 < (1ull << 32)) {
+    if (bucket_size == 256)
+      rc = launch_attn_scope<32, 256, 8, false, true>(q, k, v, qkv_row_stride, o, lse, scope_buckets, num_scope, scope_size,
+                                                      bucket_size, batch, seq_len, num_head, kv_len, device, s);
+    else
+      rc = launch_attn_scope<32, 512, 16, false, true>(q, k, v, qkv_row_stride, o, lse, scope_buckets, num_scope, scope_size,
+                                                       bucket_size, batch, seq_len, num_head, kv_len, device, s);
+    if (rc != F3D_OK) return rc;
+    F3D_CHECK_HIP(hipGetLastError());
+    rc = launch_attn<32, 64>(q, k, v, qkv_row_stride, o, lse, scope_buckets, num_scope, scope_size, bucket_size, batch,
+                             seq_len, num_head, kv_len, s, 1u);
     if (rc != F3D_OK) return rc;
     F3D_CHECK_HIP(hipGetLastError());
     return F3D_OK;

@@ -119,7 +119,59 @@ def test_padding_masks_extension(oracle):
     assert (O - o_ref).abs().max() <= TOL and (LSE - lse_ref).abs().max() <= TOL
 
 
-@pytest.mark.parametrize("D,bs,scope_size", [(32, 512, 1), (16, 256, 2), (32, 128, 2)])
+@pytest.mark.parametrize("scope_size,bs,permute", [(8, 512, False), (3, 256, True), (5, 512, True), (64, 256, False)])
+def test_large_scopes_in_whole_buckets_vs_oracle(oracle, scope_size, bs, permute):
+    """32-wide heads, scopes of more than 512 tokens in buckets of 256 / 512 rows (the reference model's scopes of 8
+    buckets of 512): the scope kernel with the key buckets streaming through LDS.  Buckets of a scope in shuffled order;
+    a second batch element; a scope table with an entry outside the sequence."""
+    B, H, D = 2, 3, 32
+    n_scope = 2 if scope_size == 64 else 4
+    L = bs * scope_size * n_scope
+    Q, K, V = _qkv(scope_size * 7 + bs, B, L, H, D)
+    scopes = oracle.gen_scopes(L, bs, scope_size)
+    if permute:
+        scopes = np.random.default_rng(5).permuted(scopes, axis=1)
+    O, LSE = _run(Q, K, V, scopes, bs)
+    o_ref, lse_ref = oracle.buck_swin_fwd(Q, K, V, scopes, bs)
+    assert (O - o_ref).abs().max() <= TOL
+    assert (LSE - lse_ref).abs().max() <= TOL
+    if scope_size == 5:
+        # the last entry of the first scope names no bucket of the sequence: its rows stay as they were, its keys drop out
+        sc2 = scopes.copy()
+        lost = int(sc2[0, -1])
+        sc2[0, -1] = L // bs + 3
+        init = torch.full(Q.shape, 5.0, dtype=torch.bfloat16)
+        O2, LSE2 = _run(Q, K, V, sc2, bs, o_init=init)
+        kl = np.full(L // bs, bs)
+        kl[lost] = 0               # for the other rows of that scope the same as the bucket not being there
+        o_ref2, lse_ref2 = oracle.buck_swin_fwd(Q, K, V, scopes, bs, kv_len=kl)
+        rows = slice(lost * bs, (lost + 1) * bs)
+        assert (O2[:, rows] == 5.0).all()
+        keep = np.ones(L, dtype=bool)
+        keep[rows] = False
+        assert (O2[:, keep] - o_ref2[:, keep]).abs().max() <= TOL
+        assert (LSE2[:, keep] - lse_ref2[:, keep]).abs().max() <= TOL
+
+
+def test_large_scopes_with_padding_masks(oracle):
+    """valid lengths per key bucket in scopes of 4 buckets of 512 (an empty bucket, a one-key bucket, a full one)"""
+    B, L, H, D, bs, scope_size = 1, 8192, 4, 32, 512, 4
+    Q, K, V = _qkv(19, B, L, H, D, scale=1 / math.sqrt(32) * 4)
+    scopes = oracle.gen_scopes(L, bs, scope_size)
+    same = _run(Q, K, V, scopes, bs, kv_len=np.full(L // bs, bs))
+    full = _run(Q, K, V, scopes, bs)
+    assert torch.equal(full[0], same[0]) and torch.equal(full[1], same[1])
+    kl = np.random.default_rng(7).integers(300, 513, L // bs)
+    kl[0], kl[1], kl[2] = 1, 0, bs
+    kl[4:8] = 0                                   # a scope without a single valid key: zero rows, LSE 0
+    O, LSE = _run(Q, K, V, scopes, bs, kv_len=kl)
+    o_ref, lse_ref = oracle.buck_swin_fwd(Q, K, V, scopes, bs, kv_len=kl)
+    assert (O - o_ref).abs().max() <= TOL
+    assert (LSE - lse_ref).abs().max() <= TOL
+    assert (O[:, 4 * bs:8 * bs] == 0).all() and (LSE[:, 4 * bs:8 * bs] == 0).all()
+
+
+@pytest.mark.parametrize("D,bs,scope_size", [(32, 512, 1), (16, 256, 2), (32, 128, 2), (32, 512, 3), (32, 256, 4)])
 @pytest.mark.parametrize("kind", ["huge", "tiny", "ramp"])
 def test_softmax_range_extremes(oracle, kind, D, bs, scope_size):
     """Scores far from zero: exponent sums beyond 2^60 ("huge"), below 2^-60 for every key ("tiny"), and a
