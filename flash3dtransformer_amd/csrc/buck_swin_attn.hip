@@ -482,7 +482,7 @@ struct ScopeGen {
   const float* chol;       // L00 L01 L02 L03 L11 L12 L13 L22 L23 L33 eps
 };
 
-// STREAM: scopes of more than T tokens in buckets of exactly T rows.  An item is (batch, scope, head, query bucket); the
+// STREAM: scopes of more than 512 tokens in buckets of exactly T rows.  An item is (batch, scope, head, query bucket); the
 // scope's key buckets pass through the two LDS buffers one after the other (the next one streams in while the current one
 // is consumed, exactly as the next item does otherwise) and the accumulators live across them.  Fixed-reference softmax
 // only: a wave whose row sums leave its range writes NaN into its rows' LSE instead of a result, and the launcher runs
@@ -1267,21 +1267,27 @@ int f3d_buck_swin_fwd_strided(const f3d_bf16_t* q, const f3d_bf16_t* k, const f3
     F3D_CHECK_HIP(hipGetLastError());
     return F3D_OK;
   }
-  // larger scopes in buckets of 256 / 512 rows with 32-wide heads (the reference model's scopes of 8 buckets of 512):
-  // the scope-resident kernel with the key buckets streaming through its two LDS buffers, then the streaming kernel for
-  // the rows it marked (sums outside the range of the fixed-reference softmax), which are rare
-  if (head_dim == 32 && (bucket_size == 256 || bucket_size == 512) && scope_tokens > 512 && scope_size <= 64 &&
+  // larger scopes in buckets of 256 / 512 rows with 16- or 32-wide heads (the reference model's scopes of 8 buckets of
+  // 512): the scope-resident kernel with the key buckets streaming through its two LDS buffers, then the streaming
+  // kernel for the rows it marked (sums outside the range of the fixed-reference softmax), which are rare
+  if (head_dim <= 32 && (bucket_size == 256 || bucket_size == 512) && scope_tokens > 512 && scope_size <= 64 &&
       (uint64_t)seq_len * qkv_row_stride * 2 < (1ull << 32)) {
-    if (bucket_size == 256)
-      rc = launch_attn_scope<32, 256, 8, false, true>(q, k, v, qkv_row_stride, o, lse, scope_buckets, num_scope, scope_size,
-                                                      bucket_size, batch, seq_len, num_head, kv_len, device, s);
-    else
-      rc = launch_attn_scope<32, 512, 16, false, true>(q, k, v, qkv_row_stride, o, lse, scope_buckets, num_scope, scope_size,
-                                                       bucket_size, batch, seq_len, num_head, kv_len, device, s);
-    if (rc != F3D_OK) return rc;
-    F3D_CHECK_HIP(hipGetLastError());
-    rc = launch_attn<32, 64>(q, k, v, qkv_row_stride, o, lse, scope_buckets, num_scope, scope_size, bucket_size, batch,
-                             seq_len, num_head, kv_len, s, 1u);
+#define F3D_RES_STREAM(DD, TT, KK)                                                                                        \
+  do {                                                                                                                    \
+    rc = launch_attn_scope<DD, TT, TT / 32, false, true>(q, k, v, qkv_row_stride, o, lse, scope_buckets, num_scope,       \
+                                                         scope_size, bucket_size, batch, seq_len, num_head, kv_len, device, \
+                                                         s);                                                              \
+    if (rc != F3D_OK) return rc;                                                                                          \
+    F3D_CHECK_HIP(hipGetLastError());                                                                                     \
+    rc = launch_attn<DD, KK>(q, k, v, qkv_row_stride, o, lse, scope_buckets, num_scope, scope_size, bucket_size, batch,   \
+                             seq_len, num_head, kv_len, s, 1u);                                                           \
+  } while (0)
+    if (head_dim == 16) {
+      if (bucket_size == 256) F3D_RES_STREAM(16, 256, 128); else F3D_RES_STREAM(16, 512, 128);
+    } else {
+      if (bucket_size == 256) F3D_RES_STREAM(32, 256, 64); else F3D_RES_STREAM(32, 512, 64);
+    }
+#undef F3D_RES_STREAM
     if (rc != F3D_OK) return rc;
     F3D_CHECK_HIP(hipGetLastError());
     return F3D_OK;

@@ -119,12 +119,14 @@ def test_padding_masks_extension(oracle):
     assert (O - o_ref).abs().max() <= TOL and (LSE - lse_ref).abs().max() <= TOL
 
 
-@pytest.mark.parametrize("scope_size,bs,permute", [(8, 512, False), (3, 256, True), (5, 512, True), (64, 256, False)])
-def test_large_scopes_in_whole_buckets_vs_oracle(oracle, scope_size, bs, permute):
-    """32-wide heads, scopes of more than 512 tokens in buckets of 256 / 512 rows (the reference model's scopes of 8
-    buckets of 512): the scope kernel with the key buckets streaming through LDS.  Buckets of a scope in shuffled order;
-    a second batch element; a scope table with an entry outside the sequence."""
-    B, H, D = 2, 3, 32
+@pytest.mark.parametrize("scope_size,bs,permute,D", [(8, 512, False, 32), (3, 256, True, 32), (5, 512, True, 32), (64, 256, False, 32),
+                                                      (8, 512, True, 16), (4, 256, False, 16)])
+def test_large_scopes_in_whole_buckets_vs_oracle(oracle, scope_size, bs, permute, D):
+    """16- / 32-wide heads, scopes of more than 512 tokens in buckets of 256 / 512 rows (the reference model's scopes of 8
+    buckets of 512, 16-wide heads in its own test, tests/test_psh_hourglass.py:56-57, :66-70): the scope kernel with the key
+    buckets streaming through LDS.  Buckets of a scope in shuffled order; a second batch element; a scope table with an
+    entry outside the sequence."""
+    B, H = 2, 3
     n_scope = 2 if scope_size == 64 else 4
     L = bs * scope_size * n_scope
     Q, K, V = _qkv(scope_size * 7 + bs, B, L, H, D)
@@ -171,7 +173,7 @@ def test_large_scopes_with_padding_masks(oracle):
     assert (O[:, 4 * bs:8 * bs] == 0).all() and (LSE[:, 4 * bs:8 * bs] == 0).all()
 
 
-@pytest.mark.parametrize("D,bs,scope_size", [(32, 512, 1), (16, 256, 2), (32, 128, 2), (32, 512, 3), (32, 256, 4)])
+@pytest.mark.parametrize("D,bs,scope_size", [(32, 512, 1), (16, 256, 2), (32, 128, 2), (32, 512, 3), (32, 256, 4), (16, 512, 2)])
 @pytest.mark.parametrize("kind", ["huge", "tiny", "ramp"])
 def test_softmax_range_extremes(oracle, kind, D, bs, scope_size):
     """Scores far from zero: exponent sums beyond 2^60 ("huge"), below 2^-60 for every key ("tiny"), and a
