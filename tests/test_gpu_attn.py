@@ -599,3 +599,30 @@ def test_first_block_attention_unsupported_shapes_are_reported():
     sc = torch.arange(4, dtype=torch.int32, device=DEV).view(torch.uint32).view(1, 4)     # one scope of 4096 tokens
     assert not pshattn.embed_buck_swin_fwd(coord, z(2, 4, 32, 16), torch.zeros(16, device=DEV), O, LSE, sc, 1024)
     assert (O == 3.0).all()
+
+
+def test_first_block_attention_scope_entries_outside_the_sequence():
+    """rows formed in the kernel: a scope entry that names no bucket of the sequence contributes no keys and owns no
+    rows, rows of buckets no scope names stay as they were -- the same as the kernel that reads a stored projection"""
+    from flash3dtransformer_amd.lib import pshattn
+    L, C, bs, H, eps = 2048, 64, 256, 2, 1e-5
+    g = torch.Generator().manual_seed(17)
+    coord = ((torch.rand(L, 3, generator=g) - 0.5) * 20).to(torch.float16).to(DEV)
+    d = {k: v.to(DEV) for k, v in _first_block_weights(C, 3).items()}
+    table = np.array([[0, 99], [3, 2], [7, 5]], dtype=np.uint32)          # buckets 1, 4, 6 in no scope; 99 outside
+    sc = torch.from_numpy(table.view(np.int32)).to(DEV).view(torch.uint32)
+    fold = pshattn.embed_qkv_fold(d["ew"], d["eb"], d["gamma"], d["beta"], eps, d["w"], d["b"], H)
+    O = torch.full((1, L, H, 32), 7.0, dtype=torch.bfloat16, device=DEV)
+    LSE = torch.full((1, L, H), -3.0, dtype=torch.float32, device=DEV)
+    assert pshattn.embed_buck_swin_fwd(coord, fold[0], fold[1], O, LSE, sc, bs)
+    qkv = torch.empty(L, 3 * C, dtype=torch.bfloat16, device=DEV)
+    assert pshattn.embed_ln_linear_bf16(coord, pshattn.embed_table(d["ew"], d["eb"]), d["gamma"], d["beta"], eps, d["w"], d["b"], qkv)
+    Q, K, V = (t.view(1, L, H, 32) for t in torch.chunk(qkv.view(1, L, 3 * C), 3, dim=-1))
+    O2, LSE2 = torch.full_like(O, 7.0), torch.full_like(LSE, -3.0)
+    pshattn.buck_swin_fwd(Q, K, V, O2, LSE2, sc, bs)
+    torch.cuda.synchronize()
+    for b in (1, 4, 6):
+        assert (O[:, b * bs:(b + 1) * bs] == 7.0).all() and (LSE[:, b * bs:(b + 1) * bs] == -3.0).all()
+    assert (O.float() - O2.float()).abs().max().item() <= 2 * TOL
+    assert (LSE - LSE2).abs().max().item() <= 2 * TOL
+    assert torch.isfinite(O.float()).all()
