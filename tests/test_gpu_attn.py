@@ -626,3 +626,17 @@ def test_first_block_attention_scope_entries_outside_the_sequence():
     assert (O.float() - O2.float()).abs().max().item() <= 2 * TOL
     assert (LSE - LSE2).abs().max().item() <= 2 * TOL
     assert torch.isfinite(O.float()).all()
+
+
+@pytest.mark.parametrize("scope_size,bs,n_scope,H", [(5, 512, 9, 3), (3, 256, 30, 2), (7, 256, 11, 1)])
+def test_large_scopes_item_walk_with_carries(oracle, scope_size, bs, n_scope, H):
+    """more items than persistent workgroups, with a workgroup count that is no multiple of the scope size: a workgroup's
+    walk over (query bucket, head, scope, batch) carries from one index into the next"""
+    B, D = 2, 32
+    L = bs * scope_size * n_scope
+    Q, K, V = _qkv(n_scope + bs, B, L, H, D)
+    scopes = np.random.default_rng(11).permuted(oracle.gen_scopes(L, bs, scope_size), axis=1)
+    O, LSE = _run(Q, K, V, scopes, bs)
+    o_ref, lse_ref = oracle.buck_swin_fwd(Q, K, V, scopes, bs)
+    assert (O - o_ref).abs().max() <= TOL
+    assert (LSE - lse_ref).abs().max() <= TOL
